@@ -1,0 +1,176 @@
+/*
+ * C ABI of the MI355X (gfx950) matrix-fragment hot path: GEMM, DLRM dot interaction and
+ * GEMV kernels built on MFMA.  Plain pointers and sizes only; every device pointer is
+ * caller-owned HIP device memory; `stream` is a hipStream_t passed as void* (NULL = the
+ * null stream).  Calls are asynchronous on `stream`, re-entrant, and allocate nothing.
+ * Every entry point returns R355_OK or a negative r355_status; r355_last_error() gives
+ * the message of the calling thread's most recent failure.
+ *
+ * The reference is a header-only device library whose host boundary is the kernel
+ * launch itself; each entry point below names the reference launch it stands in for.
+ */
+#ifndef R355_WMMA_H
+#define R355_WMMA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum
+{
+    R355_OK                 = 0,
+    R355_ERR_BAD_ARG        = -1, /* null pointer, zero size, unknown enum value          */
+    R355_ERR_UNSUPPORTED    = -2, /* type / layout combination has no kernel              */
+    R355_ERR_BAD_SIZE       = -3, /* dimension not a multiple of the block the kernel needs
+                                     (the reference kernels leave D untouched in that case:
+                                     samples/perf_hgemm.cpp:549-553,757-762)               */
+    R355_ERR_MISALIGNED     = -4, /* pointer or leading dimension breaks vector alignment */
+    R355_ERR_LAUNCH         = -5, /* hipGetLastError() after the launch                   */
+    R355_ERR_NOT_24_SPARSE  = -6  /* r355_compress_24: a group of 4 holds > 2 non-zeros   */
+} r355_status;
+
+/* element types (storage) */
+typedef enum
+{
+    R355_F16  = 0, /* IEEE binary16                      */
+    R355_BF16 = 1, /* bfloat16                           */
+    R355_E4M3 = 2, /* OCP FP8 E4M3 (gfx950 native)       */
+    R355_I8   = 3, /* signed 8-bit integer               */
+    R355_F32  = 4,
+    R355_I32  = 5
+} r355_dtype;
+
+/* memory orientation; BLAS letters: row-major = "T", col-major = "N" for A (m x k) */
+typedef enum
+{
+    R355_ROW_MAJOR = 0,
+    R355_COL_MAJOR = 1
+} r355_layout;
+
+typedef enum
+{
+    R355_KERNEL_AUTO   = 0, /* macro-tile kernel when shapes allow, else block-per-wave      */
+    R355_KERNEL_SIMPLE = 1, /* one MFMA block per wave through the fragment API, no LDS
+                               (samples/simple_hgemm.cpp:81-139,
+                                test/gemm/gemm_PGR0_LB0_MP0_SB_NC/device/kernel_device_func.hpp:50-175) */
+    R355_KERNEL_TILED  = 2  /* LDS-staged double-buffered macro tile
+                               (samples/perf_hgemm.cpp:515-711,
+                                test/gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp:52-283) */
+} r355_gemm_kernel;
+
+/*
+ * D = alpha * A * B + beta * C.  A is m x k, B is k x n, C and D are m x n.
+ * Argument order and meaning follow the reference kernel signature
+ * (test/gemm/gemm_kernel_base.hpp:101-114): leading dimensions in elements.
+ * Supported (in -> out, accumulate): f16 -> f32|f16 (f32), bf16 -> f32|bf16 (f32),
+ * e4m3 -> f32 (f32), i8 -> i32 (i32, alpha/beta truncated to int32), f32 -> f32 (f32).
+ * beta == 0 means C is never read and may be NULL.
+ *
+ * sparse24 != 0: A is 2:4 structured-sparse along k, row-major, 1-byte elements:
+ * `a` holds the m x k/2 kept values, `a_meta` the m x k/8 index bytes (format of
+ * r355_compress_24); lda is then the leading dimension of the compressed values.
+ * The reference has no sparse path; this form has no counterpart there.
+ */
+typedef struct
+{
+    int32_t     in_type;  /* r355_dtype of A and B */
+    int32_t     out_type; /* r355_dtype of C and D */
+    int32_t     layout_a, layout_b, layout_c, layout_d; /* r355_layout */
+    uint32_t    m, n, k;
+    const void* a;
+    const void* b;
+    const void* c;
+    void*       d;
+    uint32_t    lda, ldb, ldc, ldd;
+    float       alpha, beta;
+    int32_t     sparse24;
+    const void* a_meta;
+    int32_t     kernel; /* r355_gemm_kernel */
+} r355_gemm_args;
+
+/* Replaces: hipExtLaunchKernelGGL(gemm_rocwmma_d, ...) in samples/perf_hgemm.cpp:820-842 and
+ * test/gemm/gemm_kernel_base_impl.hpp:622-645. */
+int r355_gemm(const r355_gemm_args* args, void* stream);
+
+/* Launch description the AUTO/TILED/SIMPLE choice resolves to, without launching
+ * (the values the reference computes on the host: samples/perf_hgemm.cpp:807-817). */
+typedef struct
+{
+    int32_t  kernel;                       /* r355_gemm_kernel actually selected */
+    uint32_t macro_tile_m, macro_tile_n, macro_tile_k;
+    uint32_t grid_x, grid_y, block_x, block_y;
+    uint32_t lds_bytes;
+} r355_gemm_plan;
+int r355_gemm_query(const r355_gemm_args* args, r355_gemm_plan* plan);
+
+/* Timing helper in the reference's protocol (test/gemm/gemm_kernel_base_impl.hpp:647-676):
+ * `warmup` untimed launches, then `iters` launches between two hipEvents on `stream`;
+ * *avg_ms = elapsed / iters.  Synchronises the stream. */
+int r355_gemm_timed(const r355_gemm_args* args, void* stream, int warmup, int iters, float* avg_ms);
+
+/*
+ * DLRM dot-interaction forward.  in: [batch][m][k], out: [batch][k + m(m-1)/2]:
+ * out[b][0:k] = in[b][0][:], then the strict lower triangle of X X^T in row-major (i, j<i)
+ * order, f32 accumulation, rounded to dtype (R355_F16, R355_BF16 or R355_F32).  Any m <= 32,
+ * k a multiple of 32 up to 256.  No scratch buffer (the reference's `acc` argument is gone).
+ * Replaces: dlrmDotFwd launch, test/dlrm/dlrm_kernel_base_impl.hpp:78-96,
+ * test/dlrm/device/dlrm_dot_fwd.hpp:35-138, samples/simple_dlrm.cpp:184-284.
+ */
+int r355_dlrm_fwd(int32_t dtype, const void* in, void* out, uint32_t m, uint32_t k, uint32_t batch, void* stream);
+int r355_dlrm_fwd_timed(int32_t dtype, const void* in, void* out, uint32_t m, uint32_t k, uint32_t batch,
+                        void* stream, int warmup, int iters, float* avg_ms);
+
+/*
+ * DLRM dot-interaction backward.  upstream: [batch][k + m(m-1)/2]; mlp_grad: [batch][k];
+ * in_grad: [batch][m][k].  Replaces: dlrmDotBwd + trilReconstruct launches,
+ * test/dlrm/device/dlrm_dot_bwd.hpp:35-176.
+ */
+int r355_dlrm_bwd(int32_t dtype, const void* in, const void* upstream, void* mlp_grad, void* in_grad,
+                  uint32_t m, uint32_t k, uint32_t batch, void* stream);
+
+/*
+ * y_out = alpha * A * x + beta * y_in.  A is m x k f32 (layout_a), x has k elements, y m.
+ * Replaces: sgemv_rocwmma_d launch, samples/simple_sgemv.cpp:103-150,240-262.
+ */
+int r355_gemv(int32_t layout_a, uint32_t m, uint32_t k, const float* a, uint32_t lda, const float* x,
+              const float* y_in, float* y_out, float alpha, float beta, void* stream);
+int r355_gemv_timed(int32_t layout_a, uint32_t m, uint32_t k, const float* a, uint32_t lda, const float* x,
+                    const float* y_in, float* y_out, float alpha, float beta, void* stream, int warmup,
+                    int iters, float* avg_ms);
+
+/*
+ * Host-side 2:4 compressor for a row-major m x k matrix of 1-byte elements (host pointers).
+ * values: m x k/2 kept elements (in position order); meta: m x k/8 bytes, one nibble per
+ * group of 4 = idx0 | idx1 << 2 with idx0 < idx1, even group in the low nibble.  k % 8 == 0.
+ * r355_decompress_24 is the inverse.  No counterpart in the reference.
+ */
+int r355_compress_24(const uint8_t* dense, uint32_t m, uint32_t k, uint8_t* values, uint8_t* meta);
+int r355_decompress_24(const uint8_t* values, const uint8_t* meta, uint32_t m, uint32_t k, uint8_t* dense);
+
+/* Device facts used by the roofline report (test/hip_device.hpp:101-119 in the reference). */
+typedef struct
+{
+    char     arch[64];
+    int32_t  compute_units;
+    int32_t  wave_size;
+    int32_t  clock_mhz;         /* peak engine clock reported by HIP */
+    int32_t  memory_clock_mhz;
+    int32_t  lds_bytes_per_block;
+    uint64_t hbm_bytes;
+} r355_device_info;
+int r355_get_device_info(r355_device_info* info);
+
+/* Message for the calling thread's last non-OK status ("" if none). */
+const char* r355_last_error(void);
+
+/* Library version string. */
+const char* r355_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* R355_WMMA_H */

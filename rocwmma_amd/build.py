@@ -1,0 +1,67 @@
+"""Builds the gfx950 shared library (csrc/*.hip, csrc/api.cpp -> lib/librocwmma_amd.so) with hipcc.
+
+Usage: python -m rocwmma_amd.build [--force]
+Objects are rebuilt when their source (or any header) is newer; translation units compile in parallel.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+INC = os.path.join(HERE, "include")
+LIBDIR = os.path.join(HERE, "lib")
+OBJDIR = os.path.join(HERE, "build")
+LIB = os.path.join(LIBDIR, "librocwmma_amd.so")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+SOURCES = ["api.cpp", "gemm_simple.hip", "gemm_tiled.hip", "dlrm.hip", "sparse.hip", "gemv.hip"]
+
+# packed-fp32 instructions are disabled on purpose (device pass only; the host pass warns that it
+# does not know the feature, which is harmless)
+FLAGS = [
+    "--offload-arch=gfx950", "-std=c++17", "-O3", "-fPIC", "-x", "hip",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument", "-I" + INC,
+]
+
+
+def _headers():
+    hs = []
+    for root in (CSRC, INC, os.path.join(os.path.dirname(HERE), "include")):
+        for d, _, files in os.walk(root):
+            hs += [os.path.join(d, f) for f in files if f.endswith((".hpp", ".h"))]
+    return hs
+
+
+def _compile(src, force):
+    obj = os.path.join(OBJDIR, os.path.splitext(src)[0] + ".o")
+    path = os.path.join(CSRC, src)
+    newest = max(os.path.getmtime(p) for p in [path] + _headers())
+    if not force and os.path.exists(obj) and os.path.getmtime(obj) >= newest:
+        return obj, False
+    r = subprocess.run([HIPCC] + FLAGS + ["-c", path, "-o", obj], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed for %s:\n%s" % (src, r.stderr))
+    return obj, True
+
+
+def build(force=False, verbose=True):
+    os.makedirs(LIBDIR, exist_ok=True)
+    os.makedirs(OBJDIR, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=min(6, os.cpu_count() or 1)) as ex:
+        results = list(ex.map(lambda s: _compile(s, force), SOURCES))
+    objs = [o for o, _ in results]
+    if force or any(c for _, c in results) or not os.path.exists(LIB):
+        r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs,
+                           capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("link failed:\n" + r.stderr)
+    if verbose:
+        print("built", LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    build(force="--force" in sys.argv)

@@ -1,0 +1,54 @@
+// Shared host-side plumbing of the C ABI: status codes, error text, dtype helpers.
+#ifndef R355_COMMON_HPP
+#define R355_COMMON_HPP
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include <hip/hip_runtime.h>
+
+#include "../../include/r355_wmma.h"
+
+namespace r355
+{
+    // Records a formatted message for r355_last_error() and returns `code`.
+    int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+    inline uint32_t dtypeBytes(int32_t t)
+    {
+        switch(t)
+        {
+        case R355_F16:
+        case R355_BF16: return 2;
+        case R355_E4M3:
+        case R355_I8: return 1;
+        case R355_F32:
+        case R355_I32: return 4;
+        default: return 0;
+        }
+    }
+
+    inline bool aligned(const void* p, size_t bytes)
+    {
+        return (reinterpret_cast<uintptr_t>(p) % bytes) == 0;
+    }
+
+    inline int checkLaunch(const char* what)
+    {
+        hipError_t e = hipGetLastError();
+        if(e != hipSuccess)
+            return fail(R355_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+        return R355_OK;
+    }
+
+    // Kernel families (defined in their own translation units)
+    int gemmSimpleCheck(const r355_gemm_args& g, r355_gemm_plan* plan);
+    int gemmSimpleLaunch(const r355_gemm_args& g, hipStream_t stream);
+    int gemmTiledCheck(const r355_gemm_args& g, r355_gemm_plan* plan);
+    int gemmTiledLaunch(const r355_gemm_args& g, hipStream_t stream);
+    int gemmSparseCheck(const r355_gemm_args& g, r355_gemm_plan* plan);
+    int gemmSparseLaunch(const r355_gemm_args& g, hipStream_t stream);
+} // namespace r355
+
+#endif // R355_COMMON_HPP

@@ -1,0 +1,316 @@
+// DLRM dot-interaction forward and backward for gfx950.
+//
+// Forward takes the place of test/dlrm/device/dlrm_dot_fwd.hpp:35-138 (and the LDS variant
+// dlrm_dot_fwd_lds.hpp:35-190, samples/simple_dlrm.cpp:184-284).  The reference gives each
+// wave one 16x16 tile of X X^T, stores f32 tiles to a global scratch `acc[b][m][m]` and
+// re-reads them to scatter the lower triangle.  This path is HBM-bound (about 24 flop per
+// byte), so the kernel is organised around memory traffic instead:
+//
+//   * one wave owns one sample at a time; a workgroup (4 waves) owns 8 consecutive samples,
+//     whose outputs form one contiguous, 16-byte aligned run of 8 * (k + m(m-1)/2) elements;
+//   * X (m x k, m <= 32) is read once with fully coalesced 128-bit loads, parked in LDS with
+//     a per-row XOR swizzle, and fed to v_mfma_f32_32x32x16 with the same register as both
+//     operands (X X^T): k / 16 matrix instructions, one 128-bit LDS read each; rows >= m are
+//     kept zero in LDS, which is the 27 -> 32 padding;
+//   * the strict lower triangle and the copied first row are assembled in an LDS image of
+//     the output and leave with coalesced 128-bit stores.  No global scratch.
+//
+// Backward takes the place of test/dlrm/device/dlrm_dot_bwd.hpp:35-176: the upstream
+// triangle is rebuilt symmetric in LDS (trilReconstruct) and multiplied into X with the
+// same matrix instruction, again without global scratch.
+#include <hip/hip_runtime.h>
+
+#include "common.hpp"
+
+namespace
+{
+    using f32x16 = float __attribute__((ext_vector_type(16)));
+    using i32x4  = int __attribute__((ext_vector_type(4)));
+    using f16x8  = _Float16 __attribute__((ext_vector_type(8)));
+    using bf16x8 = __bf16 __attribute__((ext_vector_type(8)));
+
+    constexpr uint32_t WAVES          = 4;
+    constexpr uint32_t THREADS        = WAVES * 64;
+    constexpr uint32_t SAMPLES_PER_WG = 8; // 8 * out_row_bytes is a multiple of 16 for every (m, k)
+    constexpr uint32_t MAX_M          = 32;
+    constexpr uint32_t MAX_K          = 256;
+
+    template <bool BF16>
+    __device__ inline f32x16 mfma16(f32x16 acc, i32x4 x, i32x4 y)
+    {
+        if constexpr(BF16)
+            return __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                __builtin_bit_cast(bf16x8, x), __builtin_bit_cast(bf16x8, y), acc, 0, 0, 0);
+        else
+            return __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                __builtin_bit_cast(f16x8, x), __builtin_bit_cast(f16x8, y), acc, 0, 0, 0);
+    }
+
+    template <bool BF16>
+    __device__ inline uint16_t roundOut(float v)
+    {
+        if constexpr(BF16)
+            return __builtin_bit_cast(uint16_t, static_cast<__bf16>(v));
+        else
+            return __builtin_bit_cast(uint16_t, static_cast<_Float16>(v));
+    }
+
+    // K is a template parameter (32, 64, 128, 256): rows of X are K * 2 bytes = K / 8 chunks.
+    template <bool BF16, uint32_t K>
+    __global__ void __launch_bounds__(THREADS)
+        dlrmFwdKernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out, uint32_t m, uint32_t batch)
+    {
+        constexpr uint32_t ROW_CHUNKS = K / 8; // 16-byte chunks per row
+        constexpr uint32_t X_BYTES    = MAX_M * K * 2; // LDS image of one padded sample
+        constexpr uint32_t MAX_OUT    = K + MAX_M * (MAX_M - 1) / 2;
+
+        __shared__ __attribute__((aligned(16))) char     xLds[WAVES][X_BYTES];
+        __shared__ __attribute__((aligned(16))) uint16_t outLds[SAMPLES_PER_WG * MAX_OUT + 8];
+
+        const uint32_t tid       = threadIdx.x;
+        const uint32_t lane      = tid & 63u;
+        const uint32_t wave      = tid >> 6;
+        const uint32_t outStride = K + m * (m - 1) / 2; // elements per sample
+        const uint32_t b0        = blockIdx.x * SAMPLES_PER_WG;
+        const uint32_t inChunks  = m * ROW_CHUNKS; // 16-byte chunks of one sample
+
+        char* xw = xLds[wave];
+        // rows m..31 stay zero for the whole kernel: the padding rows of the 32 x 32 product
+        for(uint32_t c = inChunks + lane; c < MAX_M * ROW_CHUNKS; c += 64)
+            *reinterpret_cast<i32x4*>(xw + c * 16u) = i32x4{0, 0, 0, 0};
+
+        for(uint32_t sIdx = wave; sIdx < SAMPLES_PER_WG; sIdx += WAVES)
+        {
+            const uint32_t b = b0 + sIdx;
+            if(b >= batch)
+                break;
+            // ---- X -> LDS: chunk c of the sample goes to row c / ROW_CHUNKS, slot (c % ROW_CHUNKS) ^ (row % ROW_CHUNKS')
+            const char* src = reinterpret_cast<const char*>(in) + (uint64_t)b * m * K * 2u;
+            for(uint32_t c = lane; c < inChunks; c += 64)
+            {
+                const i32x4    v    = *reinterpret_cast<const i32x4*>(src + c * 16u);
+                const uint32_t row  = c / ROW_CHUNKS, col = c % ROW_CHUNKS;
+                const uint32_t slot = col ^ (row & (ROW_CHUNKS - 1u) & 15u);
+                *reinterpret_cast<i32x4*>(xw + (row * ROW_CHUNKS + slot) * 16u) = v;
+            }
+            __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): this wave's LDS writes are done
+            __builtin_amdgcn_wave_barrier();
+
+            // ---- Gram matrix: acc(i, j) = sum_k X(i, k) X(j, k)
+            f32x16         acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            const uint32_t row = lane & 31u;
+#pragma unroll
+            for(uint32_t s = 0; s < K / 16; ++s)
+            {
+                const uint32_t col  = 2u * s + (lane >> 5);
+                const uint32_t slot = col ^ (row & (ROW_CHUNKS - 1u) & 15u);
+                const i32x4    x    = *reinterpret_cast<const i32x4*>(xw + (row * ROW_CHUNKS + slot) * 16u);
+                acc                 = mfma16<BF16>(acc, x, x);
+            }
+
+            // ---- output image: first row, then strict lower triangle (i, j < i) row-major
+            uint16_t* o = outLds + sIdx * outStride;
+            for(uint32_t e = lane; e < K; e += 64)
+                o[e] = reinterpret_cast<const uint16_t*>(xw)[e]; // row 0 is stored unswizzled
+            const uint32_t j = lane & 31u;
+#pragma unroll
+            for(uint32_t r = 0; r < 16; ++r)
+            {
+                const uint32_t i = 8u * (r >> 2) + 4u * (lane >> 5) + (r & 3u);
+                if(j < i && i < m)
+                    o[K + i * (i - 1u) / 2u + j] = roundOut<BF16>(acc[r]);
+            }
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_wave_barrier();
+        }
+        __syncthreads();
+
+        // ---- coalesced copy-out of the workgroup's samples
+        const uint32_t nSamples = (batch - b0) < SAMPLES_PER_WG ? (batch - b0) : SAMPLES_PER_WG;
+        const uint32_t total    = nSamples * outStride; // elements
+        uint16_t*      dst      = out + (uint64_t)b0 * outStride;
+        const uint32_t vecs     = total / 8u;
+        for(uint32_t v = tid; v < vecs; v += THREADS)
+            reinterpret_cast<i32x4*>(dst)[v] = reinterpret_cast<const i32x4*>(outLds)[v];
+        for(uint32_t e = vecs * 8u + tid; e < total; e += THREADS)
+            dst[e] = outLds[e];
+    }
+
+    // Backward: S = T + T^T (T = strict lower triangle from the upstream gradient),
+    // grad(m x k) = S X, computed as acc(i, c) = sum_j S(i, j) X(j, c) per 32-column slab of k.
+    template <bool BF16, uint32_t K>
+    __global__ void __launch_bounds__(THREADS) dlrmBwdKernel(const uint16_t* __restrict__ in,
+                                                            const uint16_t* __restrict__ upstream,
+                                                            uint16_t* __restrict__ mlpGrad,
+                                                            uint16_t* __restrict__ inGrad,
+                                                            uint32_t m,
+                                                            uint32_t batch)
+    {
+        // S: 32 x 32 elements, row i holds S(i, 0..31) -> K-contiguous operand X-role "A" (32 x 32, K = j)
+        // X^T is needed as the other operand: lane (c = lane % 32, j-run) -> X(j, c) for 8 consecutive j;
+        // X is stored (j, c) row-major in memory, i.e. contiguous along c: keep X in LDS as [j][c]
+        // and gather the 8 values of a lane's j-run with 16-bit LDS reads.
+        __shared__ uint16_t sLds[WAVES][32 * 32];
+        __shared__ uint16_t xLds[WAVES][32 * MAX_K];
+
+        const uint32_t tid      = threadIdx.x;
+        const uint32_t lane     = tid & 63u;
+        const uint32_t wave     = tid >> 6;
+        const uint32_t upStride = K + m * (m - 1) / 2;
+        uint16_t*      sw       = sLds[wave];
+        uint16_t*      xw       = xLds[wave];
+
+        for(uint32_t b = blockIdx.x * WAVES + wave; b < batch; b += gridDim.x * WAVES)
+        {
+            const uint16_t* up = upstream + (uint64_t)b * upStride;
+            const uint16_t* x  = in + (uint64_t)b * m * K;
+            for(uint32_t e = lane; e < K; e += 64)
+                mlpGrad[(uint64_t)b * K + e] = up[e];
+            // symmetric S with zero diagonal and zero padding
+            for(uint32_t e = lane; e < 32 * 32; e += 64)
+            {
+                const uint32_t i = e >> 5, j = e & 31u;
+                uint16_t       v = 0;
+                if(i < m && j < m && i != j)
+                {
+                    const uint32_t hi = i > j ? i : j, lo = i > j ? j : i;
+                    v                 = up[K + hi * (hi - 1u) / 2u + lo];
+                }
+                sw[e] = v;
+            }
+            for(uint32_t e = lane; e < 32 * K; e += 64)
+                xw[e] = e < m * K ? x[e] : (uint16_t)0;
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_wave_barrier();
+
+            const uint32_t idx = lane & 31u, run = 8u * (lane >> 5);
+            for(uint32_t c0 = 0; c0 < K; c0 += 32)
+            {
+                f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+                for(uint32_t s = 0; s < 2; ++s) // j = 16 s + run .. + 7
+                {
+                    // swapped operands: "rows" of the instruction = c, "cols" = i, so that a lane
+                    // ends up with 4 consecutive c of one output row i
+                    union
+                    {
+                        uint16_t h[8];
+                        i32x4    v;
+                    } xo, so;
+#pragma unroll
+                    for(uint32_t e = 0; e < 8; ++e)
+                    {
+                        const uint32_t j = 16u * s + run + e;
+                        xo.h[e]          = xw[j * K + c0 + idx]; // X(j, c0 + idx)
+                        so.h[e]          = sw[idx * 32u + j]; // S(idx, j)
+                    }
+                    acc = mfma16<BF16>(acc, xo.v, so.v);
+                }
+                // lane: i = idx, c = c0 + 8 (r / 4) + 4 (lane / 32) + r % 4
+                if(idx < m)
+                {
+#pragma unroll
+                    for(uint32_t q = 0; q < 4; ++q)
+                    {
+                        union
+                        {
+                            uint16_t h[4];
+                            uint64_t v;
+                        } o;
+#pragma unroll
+                        for(uint32_t e = 0; e < 4; ++e)
+                            o.h[e] = roundOut<BF16>(acc[4 * q + e]);
+                        const uint32_t c = c0 + 8u * q + 4u * (lane >> 5);
+                        *reinterpret_cast<uint64_t*>(inGrad + (uint64_t)b * m * K + idx * K + c) = o.v;
+                    }
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
+
+    int checkArgs(const char* what, int32_t dtype, const void* in, const void* out, uint32_t m, uint32_t k, uint32_t batch)
+    {
+        if(!in || !out)
+            return r355::fail(R355_ERR_BAD_ARG, "%s: null pointer", what);
+        if(dtype != R355_F16 && dtype != R355_BF16)
+            return r355::fail(R355_ERR_UNSUPPORTED, "%s: dtype must be R355_F16 or R355_BF16", what);
+        if(m < 2 || m > MAX_M)
+            return r355::fail(R355_ERR_BAD_SIZE, "%s: m=%u must be in [2, %u]", what, m, MAX_M);
+        if(k != 32 && k != 64 && k != 128 && k != 256)
+            return r355::fail(R355_ERR_BAD_SIZE, "%s: k=%u must be 32, 64, 128 or 256", what, k);
+        if(batch == 0)
+            return r355::fail(R355_ERR_BAD_ARG, "%s: batch is zero", what);
+        if(!r355::aligned(in, 16) || !r355::aligned(out, 16))
+            return r355::fail(R355_ERR_MISALIGNED, "%s: in / out must be 16-byte aligned", what);
+        return R355_OK;
+    }
+} // namespace
+
+extern "C" int r355_dlrm_fwd(int32_t dtype, const void* in, void* out, uint32_t m, uint32_t k, uint32_t batch, void* stream)
+{
+    int rc = checkArgs("dlrm_fwd", dtype, in, out, m, k, batch);
+    if(rc != R355_OK)
+        return rc;
+    const dim3  grid((batch + SAMPLES_PER_WG - 1) / SAMPLES_PER_WG), block(THREADS);
+    hipStream_t s  = static_cast<hipStream_t>(stream);
+    auto*       pi = static_cast<const uint16_t*>(in);
+    auto*       po = static_cast<uint16_t*>(out);
+#define R355_FWD(BF, KK) hipLaunchKernelGGL((dlrmFwdKernel<BF, KK>), grid, block, 0, s, pi, po, m, batch)
+#define R355_FWD_K(BF)   \
+    switch(k)            \
+    {                    \
+    case 32: R355_FWD(BF, 32); break;   \
+    case 64: R355_FWD(BF, 64); break;   \
+    case 128: R355_FWD(BF, 128); break; \
+    default: R355_FWD(BF, 256); break;  \
+    }
+    if(dtype == R355_BF16)
+    {
+        R355_FWD_K(true)
+    }
+    else
+    {
+        R355_FWD_K(false)
+    }
+#undef R355_FWD_K
+#undef R355_FWD
+    return r355::checkLaunch("dlrm_fwd");
+}
+
+extern "C" int r355_dlrm_bwd(int32_t dtype, const void* in, const void* upstream, void* mlp_grad, void* in_grad,
+                             uint32_t m, uint32_t k, uint32_t batch, void* stream)
+{
+    int rc = checkArgs("dlrm_bwd", dtype, in, in_grad, m, k, batch);
+    if(rc != R355_OK)
+        return rc;
+    if(!upstream || !mlp_grad)
+        return r355::fail(R355_ERR_BAD_ARG, "dlrm_bwd: null pointer");
+    const uint32_t wgs = (batch + WAVES - 1) / WAVES;
+    const dim3     grid(wgs < 4096 ? wgs : 4096), block(THREADS);
+    hipStream_t    s  = static_cast<hipStream_t>(stream);
+    auto*          pi = static_cast<const uint16_t*>(in);
+    auto*          pu = static_cast<const uint16_t*>(upstream);
+    auto*          pm = static_cast<uint16_t*>(mlp_grad);
+    auto*          pg = static_cast<uint16_t*>(in_grad);
+#define R355_BWD(BF, KK) hipLaunchKernelGGL((dlrmBwdKernel<BF, KK>), grid, block, 0, s, pi, pu, pm, pg, m, batch)
+#define R355_BWD_K(BF)   \
+    switch(k)            \
+    {                    \
+    case 32: R355_BWD(BF, 32); break;   \
+    case 64: R355_BWD(BF, 64); break;   \
+    case 128: R355_BWD(BF, 128); break; \
+    default: R355_BWD(BF, 256); break;  \
+    }
+    if(dtype == R355_BF16)
+    {
+        R355_BWD_K(true)
+    }
+    else
+    {
+        R355_BWD_K(false)
+    }
+#undef R355_BWD_K
+#undef R355_BWD
+    return r355::checkLaunch("dlrm_bwd");
+}

@@ -1,0 +1,616 @@
+// LDS-staged, double-buffered macro-tile GEMM for gfx950, written directly against the
+// hardware (no fragment-API composition).
+//
+// Takes the place of samples/perf_hgemm.cpp:515-711 and
+// test/gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp:52-283.  The reference
+// kernel moves 128x128x16 macro tiles through 16 KiB of LDS with element-wise LDS reads
+// and eight matrix instructions per wave between barriers; this one is shaped for
+// MI355X's 160 KB LDS and 256 CUs:
+//
+//   macro tile   256 x 256, K stage of 128 bytes (64 f16/bf16, 128 int8/fp8 elements)
+//   workgroup    256 threads = 4 waves in a 2 x 2 grid, wave tile 128 x 128
+//                = 4 x 4 v_mfma_*_32x32x{16,32} accumulators (256 accumulator registers)
+//   LDS          2 stages x (A 32 KiB + B 32 KiB) = 128 KiB, one workgroup per CU
+//   global->LDS  128-bit loads, either staged through registers or written straight
+//                into LDS by the memory pipeline (global_load_lds_dwordx4)
+//   LDS layout   16-byte chunks, XOR-swizzled inside each row so that both the
+//                row-contiguous writes and the MFMA-shaped reads are bank-conflict free
+//   LDS->regs    K-contiguous operands: one ds_read_b128 per 32x(16|32) operand block;
+//                M/N-contiguous 16-bit operands: two ds_read_b64_tr_b16 (transposing
+//                read) -- no element-wise reads anywhere
+//   grid         1-D, remapped so that each XCD (workgroup id mod 8) owns a compact
+//                rectangle of tiles and walks it in 4-row groups (L2 reuse of A and B)
+//
+// Operand orientation is a template parameter per operand ("K-contiguous" = A row-major /
+// B col-major).  The MFMA operands are swapped so that each lane holds four consecutive
+// columns of a row of D; a col-major D is computed as the row-major D^T = B^T A^T.
+#include <hip/hip_runtime.h>
+
+#include "common.hpp"
+
+namespace
+{
+    using f32x16 = float __attribute__((ext_vector_type(16)));
+    using i32x16 = int __attribute__((ext_vector_type(16)));
+    using i32x4  = int __attribute__((ext_vector_type(4)));
+    using i32x2  = int __attribute__((ext_vector_type(2)));
+    using f16x8  = _Float16 __attribute__((ext_vector_type(8)));
+    using f16x4  = _Float16 __attribute__((ext_vector_type(4)));
+    using bf16x8 = __bf16 __attribute__((ext_vector_type(8)));
+    typedef __fp16 trv4 __attribute__((__vector_size__(4 * sizeof(__fp16)))); // operand type of the transposing LDS read
+
+    enum class Elem
+    {
+        F16,
+        BF16,
+        E4M3,
+        I8
+    };
+
+    constexpr uint32_t TILE_M      = 256;
+    constexpr uint32_t TILE_N      = 256;
+    constexpr uint32_t STAGE_KB    = 128; // bytes of K per stage per row
+    constexpr uint32_t OPER_BYTES  = TILE_M * STAGE_KB; // 32 KiB per operand per stage
+    constexpr uint32_t STAGE_BYTES = 2 * OPER_BYTES;
+    constexpr uint32_t NUM_STAGES  = 2;
+    constexpr uint32_t THREADS     = 256;
+    constexpr uint32_t CHUNK       = 16; // bytes moved per lane per access
+    constexpr uint32_t LOADS_PER_OPER = OPER_BYTES / CHUNK / THREADS; // 8
+
+    template <Elem E>
+    struct ElemTraits;
+    template <>
+    struct ElemTraits<Elem::F16>
+    {
+        static constexpr uint32_t Bytes = 2;
+        using Acc                       = f32x16;
+    };
+    template <>
+    struct ElemTraits<Elem::BF16>
+    {
+        static constexpr uint32_t Bytes = 2;
+        using Acc                       = f32x16;
+    };
+    template <>
+    struct ElemTraits<Elem::E4M3>
+    {
+        static constexpr uint32_t Bytes = 1;
+        using Acc                       = f32x16;
+    };
+    template <>
+    struct ElemTraits<Elem::I8>
+    {
+        static constexpr uint32_t Bytes = 1;
+        using Acc                       = i32x16;
+    };
+
+    // acc += X(32 x k) * Y(k x 32) with 16 bytes of K per lane per operand
+    template <Elem E>
+    __device__ inline void mfma32(typename ElemTraits<E>::Acc& acc, i32x4 x, i32x4 y)
+    {
+        if constexpr(E == Elem::F16)
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                __builtin_bit_cast(f16x8, x), __builtin_bit_cast(f16x8, y), acc, 0, 0, 0);
+        else if constexpr(E == Elem::BF16)
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                __builtin_bit_cast(bf16x8, x), __builtin_bit_cast(bf16x8, y), acc, 0, 0, 0);
+        else if constexpr(E == Elem::I8)
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(x, y, acc, 0, 0, 0);
+        else
+        {
+            // fp8: two 32x32x16 steps on the low / high 8 bytes (a K permutation shared by X and Y)
+            using l2 = long __attribute__((ext_vector_type(2)));
+            l2 xl    = __builtin_bit_cast(l2, x);
+            l2 yl    = __builtin_bit_cast(l2, y);
+            acc      = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(xl[0], yl[0], acc, 0, 0, 0);
+            acc      = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(xl[1], yl[1], acc, 0, 0, 0);
+        }
+    }
+
+    // ---- LDS swizzles.  A tile is `rows` rows of `rowBytes`; chunk c of row r lives in
+    // chunk slot (c ^ swz(r)) of that row.
+    //   K-contiguous tile: 256 rows x 128 B (8 slots).   Readers: lane -> row, 8 (or 16)
+    //     lanes share a chunk index, so consecutive rows must land in different slots.
+    //   M/N-contiguous tile: 64 k-rows x 512 B (32 slots).  Readers: 16 lanes cover
+    //     4 k-rows x 32 B, so consecutive k-rows must land in different 32-byte pairs.
+    // BANKS64 selects the pattern for a 256-byte-per-clock LDS (64 banks) instead of 128.
+    struct Params
+    {
+        uint32_t    m, n, k;
+        const char* a;
+        const char* b;
+        const char* c;
+        char*       d;
+        uint32_t    lda, ldb, ldc, ldd; // elements
+        float       alpha, beta;
+        uint32_t    tilesM, tilesN;
+        uint32_t    banks64; // LDS swizzle tuned for 64 banks instead of 32
+    };
+
+    // Workgroup id -> (tile row, tile col).  Hardware deals workgroup ids round-robin to the
+    // 8 XCDs; ids with the same (id mod 8) share an L2.  Give each XCD a contiguous run of
+    // tile indices and walk the run in groups of GROUP_M tile rows, column by column, so that
+    // the 32 tiles resident on an XCD at one time cover about 4 x 8 tiles.
+    __device__ inline bool tileCoord(uint32_t bid, uint32_t tilesM, uint32_t tilesN, uint32_t& tm, uint32_t& tn)
+    {
+        constexpr uint32_t XCDS = 8, GROUP_M = 4;
+        const uint32_t     total  = tilesM * tilesN;
+        const uint32_t     perXcd = (total + XCDS - 1) / XCDS;
+        const uint32_t     id     = (bid % XCDS) * perXcd + bid / XCDS;
+        if(id >= total)
+            return false;
+        const uint32_t groupSize = GROUP_M * tilesN;
+        const uint32_t group     = id / groupSize;
+        const uint32_t first     = group * GROUP_M;
+        const uint32_t rowsHere  = (tilesM - first) < GROUP_M ? (tilesM - first) : GROUP_M;
+        const uint32_t inGroup   = id % groupSize;
+        tm                       = first + inGroup % rowsHere;
+        tn                       = inGroup / rowsHere;
+        return true;
+    }
+
+    // Scheduling hint for the current region: next come MFMAS matrix instructions, then DSREADS
+    // LDS reads, then VMEM global loads.
+    template <uint32_t MFMAS, uint32_t DSREADS, uint32_t VMEM>
+    __device__ inline void schedGroup()
+    {
+        __builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
+        if constexpr(DSREADS > 0)
+            __builtin_amdgcn_sched_group_barrier(0x100, DSREADS, 0);
+        if constexpr(VMEM > 0)
+            __builtin_amdgcn_sched_group_barrier(0x020, VMEM, 0);
+    }
+
+    template <Elem E, typename OutT, bool A_KCONTIG, bool B_KCONTIG, bool DIRECT>
+    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
+        gemmTiledKernel(Params p)
+    {
+        using Traits          = ElemTraits<E>;
+        using Acc             = typename Traits::Acc;
+        constexpr uint32_t ES = Traits::Bytes;
+        constexpr uint32_t TK = STAGE_KB / ES; // K elements per stage
+        static_assert(ES == 2 || (A_KCONTIG && B_KCONTIG), "8-bit operands must be K-contiguous");
+        // LDS reads per operand block: one 128-bit read, or two transposing 64-bit reads
+        constexpr uint32_t READS_PER_SUB = (A_KCONTIG ? 4u : 8u) + (B_KCONTIG ? 4u : 8u);
+
+        // One variable per stage: the compiler tracks outstanding direct-to-LDS loads per LDS
+        // variable, so reads of one stage need not wait for loads in flight to the other.
+        __shared__ __attribute__((aligned(1024))) char stage0[STAGE_BYTES];
+        __shared__ __attribute__((aligned(1024))) char stage1[STAGE_BYTES];
+
+        uint32_t tm, tn;
+        if(!tileCoord(blockIdx.x, p.tilesM, p.tilesN, tm, tn))
+            return;
+
+        const uint32_t tid   = threadIdx.x;
+        const uint32_t lane  = tid & 63u;
+        const uint32_t wave  = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const uint32_t wm    = wave >> 1; // wave row in the 2 x 2 wave grid
+        const uint32_t wn    = wave & 1u;
+        const bool     b64   = p.banks64 != 0;
+        auto           swzK  = [&](uint32_t row) { return b64 ? ((row >> 1) & 7u) : (row & 7u); };
+        auto           swzMN = [&](uint32_t krow) { return b64 ? ((krow & 3u) << 2) : ((krow & 3u) << 1); };
+
+        // ---------------- global -> LDS addressing (per thread, fixed for the whole K loop)
+        // chunk L = j * 256 + tid of an operand tile sits at LDS byte 16 L.  The swizzle terms
+        // depend on the row only through bits that j does not change (j * 32 rows for the
+        // K-contiguous tile, j * 8 k-rows for the other), so one lane offset serves all j.
+        uint32_t gOffA, gOffB; // byte offset of this thread's j = 0 chunk from the tile origin
+        uint32_t gStepA, gStepB; // bytes between consecutive j
+        uint64_t gStageA, gStageB; // bytes between consecutive K stages
+        if constexpr(A_KCONTIG)
+        {
+            const uint32_t r = tid >> 3, slot = tid & 7u;
+            gOffA   = r * p.lda * ES + ((slot ^ swzK(r)) * CHUNK);
+            gStepA  = 32u * p.lda * ES;
+            gStageA = STAGE_KB;
+        }
+        else
+        {
+            const uint32_t r = tid >> 5, slot = tid & 31u;
+            gOffA   = r * p.lda * ES + ((slot ^ swzMN(r)) * CHUNK);
+            gStepA  = 8u * p.lda * ES;
+            gStageA = (uint64_t)TK * p.lda * ES;
+        }
+        if constexpr(B_KCONTIG)
+        {
+            const uint32_t r = tid >> 3, slot = tid & 7u;
+            gOffB   = r * p.ldb * ES + ((slot ^ swzK(r)) * CHUNK);
+            gStepB  = 32u * p.ldb * ES;
+            gStageB = STAGE_KB;
+        }
+        else
+        {
+            const uint32_t r = tid >> 5, slot = tid & 31u;
+            gOffB   = r * p.ldb * ES + ((slot ^ swzMN(r)) * CHUNK);
+            gStepB  = 8u * p.ldb * ES;
+            gStageB = (uint64_t)TK * p.ldb * ES;
+        }
+        const char* gA = p.a + (A_KCONTIG ? (uint64_t)tm * TILE_M * p.lda * ES : (uint64_t)tm * TILE_M * ES);
+        const char* gB = p.b + (B_KCONTIG ? (uint64_t)tn * TILE_N * p.ldb * ES : (uint64_t)tn * TILE_N * ES);
+
+        // ---------------- LDS -> register addressing (per lane, fixed)
+        // K-contiguous: block i rows are (i * 32 + lane % 32); sub-step s reads chunk 2 s + lane / 32.
+        // M/N-contiguous: sub-step s, half h: k-row 16 s + 8 (lane / 32) + 4 h + (lane % 16) / 4,
+        //                 8-byte piece m / 4 with m = 32 i + 16 ((lane / 16) & 1) + 4 (lane % 4).
+        uint32_t rdA[4], rdB[4];
+        if constexpr(A_KCONTIG)
+        {
+            const uint32_t r = wm * 128u + (lane & 31u);
+#pragma unroll
+            for(uint32_t s = 0; s < 4; ++s)
+                rdA[s] = r * STAGE_KB + (((2u * s + (lane >> 5)) ^ swzK(r)) * CHUNK);
+        }
+        else
+        {
+            const uint32_t t = lane & 15u, kr = 8u * (lane >> 5) + (t >> 2);
+#pragma unroll
+            for(uint32_t i = 0; i < 4; ++i)
+            {
+                const uint32_t piece = wm * 32u + 8u * i + 4u * ((lane >> 4) & 1u) + (t & 3u);
+                rdA[i] = kr * 512u + (((piece >> 1) ^ swzMN(kr)) * CHUNK) + (piece & 1u) * 8u;
+            }
+        }
+        if constexpr(B_KCONTIG)
+        {
+            const uint32_t r = wn * 128u + (lane & 31u);
+#pragma unroll
+            for(uint32_t s = 0; s < 4; ++s)
+                rdB[s] = OPER_BYTES + r * STAGE_KB + (((2u * s + (lane >> 5)) ^ swzK(r)) * CHUNK);
+        }
+        else
+        {
+            const uint32_t t = lane & 15u, kr = 8u * (lane >> 5) + (t >> 2);
+#pragma unroll
+            for(uint32_t i = 0; i < 4; ++i)
+            {
+                const uint32_t piece = wn * 32u + 8u * i + 4u * ((lane >> 4) & 1u) + (t & 3u);
+                rdB[i] = OPER_BYTES + kr * 512u + (((piece >> 1) ^ swzMN(kr)) * CHUNK) + (piece & 1u) * 8u;
+            }
+        }
+
+        // operand block i of sub-step s from a stage buffer
+        auto readA = [&](const char* base, uint32_t i, uint32_t s) -> i32x4 {
+            if constexpr(A_KCONTIG)
+                return *reinterpret_cast<const i32x4*>(base + rdA[s] + i * 32u * STAGE_KB);
+            else
+            {
+                using lp        = __attribute__((address_space(3))) trv4*;
+                const char* q   = base + rdA[i] + s * 16u * 512u;
+                const i32x2 lo  = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lp)q));
+                const i32x2 hi  = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lp)(q + 4u * 512u)));
+                return i32x4{lo[0], lo[1], hi[0], hi[1]};
+            }
+        };
+        auto readB = [&](const char* base, uint32_t i, uint32_t s) -> i32x4 {
+            if constexpr(B_KCONTIG)
+                return *reinterpret_cast<const i32x4*>(base + rdB[s] + i * 32u * STAGE_KB);
+            else
+            {
+                using lp        = __attribute__((address_space(3))) trv4*;
+                const char* q   = base + rdB[i] + s * 16u * 512u;
+                const i32x2 lo  = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lp)q));
+                const i32x2 hi  = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lp)(q + 4u * 512u)));
+                return i32x4{lo[0], lo[1], hi[0], hi[1]};
+            }
+        };
+
+        // ---------------- stage movement
+        i32x4 stageRegs[DIRECT ? 1 : 2 * LOADS_PER_OPER];
+
+        auto issueGlobal = [&](uint32_t kt, char* stage) {
+            // uniform (scalar) base per load + one 32-bit lane offset per operand
+            const char* srcA = gA + kt * gStageA;
+            const char* srcB = gB + kt * gStageB;
+#pragma unroll
+            for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
+            {
+                const char* pa = srcA + gOffA;
+                const char* pb = srcB + gOffB;
+                srcA += gStepA;
+                srcB += gStepB;
+                if constexpr(DIRECT)
+                {
+                    // the memory pipeline writes lane l's 16 bytes at (uniform LDS base + 16 l)
+                    char* dstA = stage + (j * THREADS + wave * 64u) * CHUNK;
+                    char* dstB = dstA + OPER_BYTES;
+                    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)pa,
+                                                     (__attribute__((address_space(3))) void*)dstA, 16, 0, 0);
+                    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)pb,
+                                                     (__attribute__((address_space(3))) void*)dstB, 16, 0, 0);
+                }
+                else
+                {
+                    stageRegs[j]                  = *reinterpret_cast<const i32x4*>(pa);
+                    stageRegs[LOADS_PER_OPER + j] = *reinterpret_cast<const i32x4*>(pb);
+                }
+            }
+        };
+
+        auto commitLds = [&](char* stage) {
+            if constexpr(!DIRECT)
+            {
+#pragma unroll
+                for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
+                {
+                    char* dstA = stage + (j * THREADS + tid) * CHUNK;
+                    *reinterpret_cast<i32x4*>(dstA)              = stageRegs[j];
+                    *reinterpret_cast<i32x4*>(dstA + OPER_BYTES) = stageRegs[LOADS_PER_OPER + j];
+                }
+            }
+        };
+
+        Acc acc[4][4];
+#pragma unroll
+        for(uint32_t i = 0; i < 4; ++i)
+#pragma unroll
+            for(uint32_t j = 0; j < 4; ++j)
+#pragma unroll
+                for(uint32_t e = 0; e < 16; ++e)
+                    acc[i][j][e] = 0;
+
+        // operands swapped: each lane then holds 4 consecutive columns of a row of D
+        auto mfmaStep = [&](const i32x4 (&fa)[4], const i32x4 (&fb)[4]) {
+#pragma unroll
+            for(uint32_t i = 0; i < 4; ++i)
+#pragma unroll
+                for(uint32_t j = 0; j < 4; ++j)
+                    mfma32<E>(acc[i][j], fb[j], fa[i]);
+        };
+
+        const uint32_t numStages = p.k / TK;
+        i32x4          fa[2][4], fb[2][4];
+
+        // One K stage.  `cur` / `nxt` are the LDS buffers of stage kt / kt + 1.
+        // Sub-steps 0..2 run against `cur` while the reads for the following sub-step are in
+        // flight; before sub-step 3 every wave has all its operands of `cur` in registers, so
+        // after the barrier `cur` is refilled with stage kt + 2 and the first operands of
+        // stage kt + 1 are fetched from `nxt` underneath the last 16 matrix instructions.
+        auto stageBody = [&](uint32_t kt, char* cur, char* nxt, auto refill, auto hasNext) {
+            constexpr bool REFILL = decltype(refill)::value; // stage kt + 2 exists
+            constexpr bool NEXT   = decltype(hasNext)::value; // stage kt + 1 exists
+#pragma unroll
+            for(uint32_t s = 0; s < 3; ++s)
+            {
+#pragma unroll
+                for(uint32_t i = 0; i < 4; ++i)
+                {
+                    fa[(s + 1) & 1][i] = readA(cur, i, s + 1);
+                    fb[(s + 1) & 1][i] = readB(cur, i, s + 1);
+                }
+                mfmaStep(fa[s & 1], fb[s & 1]);
+                // LDS reads early in the sub-step, matrix instructions throughout
+#pragma unroll
+                for(uint32_t g = 0; g < 8; ++g)
+                    schedGroup<1, READS_PER_SUB / 8u, 0>();
+                schedGroup<8, 0, 0>();
+            }
+            if constexpr(!DIRECT && NEXT)
+                commitLds(nxt);
+            // Direct-to-LDS loads are tracked by vmcnt of the issuing wave only: every wave must
+            // see its own loads of stage kt + 1 land before the barrier publishes them to the others.
+            if constexpr(DIRECT)
+                __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+            __syncthreads(); // also waits for this wave's LDS reads of `cur`
+            if constexpr(REFILL)
+                issueGlobal(kt + 2, cur);
+            if constexpr(NEXT)
+            {
+#pragma unroll
+                for(uint32_t i = 0; i < 4; ++i)
+                {
+                    fa[0][i] = readA(nxt, i, 0);
+                    fb[0][i] = readB(nxt, i, 0);
+                }
+            }
+            mfmaStep(fa[1], fb[1]);
+#pragma unroll
+            for(uint32_t g = 0; g < 8; ++g)
+                schedGroup<1, NEXT ? READS_PER_SUB / 8u : 0u, REFILL ? 2u : 0u>();
+            schedGroup<8, 0, 0>();
+        };
+        constexpr std::true_type  yes{};
+        constexpr std::false_type no{};
+
+        // prologue: stage 0 resident, stage 1 in flight, first operands in registers
+        issueGlobal(0, stage0);
+        if constexpr(DIRECT)
+        {
+            issueGlobal(1, stage1);
+            __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+        }
+        else
+        {
+            commitLds(stage0);
+            issueGlobal(1, stage1);
+        }
+        __syncthreads();
+#pragma unroll
+        for(uint32_t i = 0; i < 4; ++i)
+        {
+            fa[0][i] = readA(stage0, i, 0);
+            fb[0][i] = readB(stage0, i, 0);
+        }
+
+        // numStages is even (checked on the host): steady state in pairs, last pair peeled
+        uint32_t kt = 0;
+        for(; kt + 2 < numStages; kt += 2)
+        {
+            stageBody(kt, stage0, stage1, yes, yes);
+            stageBody(kt + 1, stage1, stage0, yes, yes);
+        }
+        stageBody(kt, stage0, stage1, no, yes);
+        stageBody(kt + 1, stage1, stage0, no, no);
+
+        // ---------------- epilogue: D = alpha * acc + beta * C, row-major
+        // lane holds D(m = lane % 32, n = 8 (e / 4) + 4 (lane / 32) + e % 4) of each 32 x 32 block
+        using AccE = std::conditional_t<E == Elem::I8, int, float>;
+        using OutV = OutT __attribute__((ext_vector_type(4)));
+        const AccE     alpha = static_cast<AccE>(p.alpha), beta = static_cast<AccE>(p.beta);
+        const uint32_t m0 = tm * TILE_M + wm * 128u, n0 = tn * TILE_N + wn * 128u;
+#pragma unroll
+        for(uint32_t i = 0; i < 4; ++i)
+        {
+#pragma unroll
+            for(uint32_t j = 0; j < 4; ++j)
+            {
+#pragma unroll
+                for(uint32_t q = 0; q < 4; ++q)
+                {
+                    const uint32_t row  = m0 + 32u * i + (lane & 31u);
+                    const uint32_t col  = n0 + 32u * j + 8u * q + 4u * (lane >> 5);
+                    const uint64_t offD = (uint64_t)row * p.ldd + col;
+                    OutV           out;
+                    if(beta != static_cast<AccE>(0))
+                    {
+                        const uint64_t offC = (uint64_t)row * p.ldc + col;
+                        const OutV     cv   = *reinterpret_cast<const OutV*>(p.c + offC * sizeof(OutT));
+#pragma unroll
+                        for(uint32_t e = 0; e < 4; ++e)
+                            out[e] = static_cast<OutT>(alpha * static_cast<AccE>(acc[i][j][4 * q + e])
+                                                       + beta * static_cast<AccE>(cv[e]));
+                    }
+                    else
+                    {
+#pragma unroll
+                        for(uint32_t e = 0; e < 4; ++e)
+                            out[e] = static_cast<OutT>(alpha * static_cast<AccE>(acc[i][j][4 * q + e]));
+                    }
+                    *reinterpret_cast<OutV*>(p.d + offD * sizeof(OutT)) = out;
+                }
+            }
+        }
+    }
+
+    struct Variant
+    {
+        bool direct;
+        bool banks64;
+    };
+    // Defaults chosen from measurements on MI355X; R355_TILED_VARIANT=<bit0: direct-to-LDS loads,
+    // bit1: 64-bank swizzle> overrides them for experiments.
+    Variant chosenVariant()
+    {
+        static const Variant v = [] {
+            Variant     r{true, false};
+            const char* e = getenv("R355_TILED_VARIANT");
+            if(e)
+            {
+                int x     = atoi(e);
+                r.direct  = x & 1;
+                r.banks64 = x & 2;
+            }
+            return r;
+        }();
+        return v;
+    }
+
+    template <Elem E, typename OutT, bool AK, bool BK>
+    int launchVariant(Params p, hipStream_t stream)
+    {
+        const Variant  v    = chosenVariant();
+        const uint32_t grid = ((p.tilesM * p.tilesN + 7u) / 8u) * 8u;
+        p.banks64           = v.banks64;
+        if(v.direct)
+            hipLaunchKernelGGL((gemmTiledKernel<E, OutT, AK, BK, true>), dim3(grid), dim3(THREADS), 0, stream, p);
+        else
+            hipLaunchKernelGGL((gemmTiledKernel<E, OutT, AK, BK, false>), dim3(grid), dim3(THREADS), 0, stream, p);
+        return r355::checkLaunch("gemm (macro tile)");
+    }
+
+    template <Elem E, typename OutT>
+    int launchLayouts(bool aK, bool bK, const Params& p, hipStream_t stream)
+    {
+        if constexpr(ElemTraits<E>::Bytes == 1)
+            return launchVariant<E, OutT, true, true>(p, stream);
+        else
+        {
+            if(aK && bK)
+                return launchVariant<E, OutT, true, true>(p, stream);
+            if(aK && !bK)
+                return launchVariant<E, OutT, true, false>(p, stream);
+            if(!aK && bK)
+                return launchVariant<E, OutT, false, true>(p, stream);
+            return launchVariant<E, OutT, false, false>(p, stream);
+        }
+    }
+} // namespace
+
+namespace r355
+{
+    int gemmTiledCheck(const r355_gemm_args& g, r355_gemm_plan* plan)
+    {
+        const bool pairOk = (g.in_type == R355_F16 && (g.out_type == R355_F16 || g.out_type == R355_F32))
+                            || (g.in_type == R355_BF16 && (g.out_type == R355_BF16 || g.out_type == R355_F32))
+                            || (g.in_type == R355_E4M3 && g.out_type == R355_F32)
+                            || (g.in_type == R355_I8 && g.out_type == R355_I32);
+        if(!pairOk)
+            return fail(R355_ERR_UNSUPPORTED, "tiled gemm: no kernel for in_type %d -> out_type %d", g.in_type, g.out_type);
+        const uint32_t es = dtypeBytes(g.in_type), os = dtypeBytes(g.out_type);
+        if(es == 1 && !(g.layout_a == R355_ROW_MAJOR && g.layout_b == R355_COL_MAJOR))
+            return fail(R355_ERR_UNSUPPORTED, "tiled gemm: 8-bit operands must be K-contiguous (A row-major, B col-major)");
+        if(g.beta != 0.0f && g.layout_c != g.layout_d)
+            return fail(R355_ERR_UNSUPPORTED, "tiled gemm: C and D must share an orientation");
+        const uint32_t tk = STAGE_KB / es;
+        if(g.m % TILE_M || g.n % TILE_N || g.k % (2 * tk) || g.k == 0)
+            return fail(R355_ERR_BAD_SIZE, "tiled gemm: m=%u n=%u must be multiples of 256 and k=%u of %u", g.m, g.n, g.k, 2 * tk);
+        if(!aligned(g.a, 16) || !aligned(g.b, 16) || (g.lda * es) % 16 || (g.ldb * es) % 16 || !aligned(g.d, 4 * os)
+           || (g.ldd * os) % (4 * os) || (g.beta != 0.0f && (!aligned(g.c, 4 * os) || (g.ldc * os) % (4 * os))))
+            return fail(R355_ERR_MISALIGNED, "tiled gemm: A/B need 16-byte, C/D 4-element alignment of pointers and leading dimensions");
+        if(plan)
+        {
+            plan->kernel       = R355_KERNEL_TILED;
+            plan->macro_tile_m = TILE_M;
+            plan->macro_tile_n = TILE_N;
+            plan->macro_tile_k = tk;
+            plan->grid_x       = (((g.m / TILE_M) * (g.n / TILE_N) + 7u) / 8u) * 8u;
+            plan->grid_y       = 1;
+            plan->block_x      = THREADS;
+            plan->block_y      = 1;
+            plan->lds_bytes    = NUM_STAGES * STAGE_BYTES;
+        }
+        return R355_OK;
+    }
+
+    int gemmTiledLaunch(const r355_gemm_args& g, hipStream_t stream)
+    {
+        // The kernel writes D row-major.  A col-major D (and C) is the row-major transpose:
+        // D^T = B^T A^T, i.e. swap the operands and the roles of m and n; an operand's
+        // K-contiguity is unchanged by the swap.
+        const bool dRow = g.layout_d == R355_ROW_MAJOR;
+        Params     p;
+        p.k = g.k;
+        p.c = static_cast<const char*>(g.c), p.d = static_cast<char*>(g.d);
+        p.ldc = g.ldc, p.ldd = g.ldd;
+        p.alpha = g.alpha, p.beta = g.beta;
+        bool aK, bK;
+        if(dRow)
+        {
+            p.m = g.m, p.n = g.n;
+            p.a = static_cast<const char*>(g.a), p.b = static_cast<const char*>(g.b);
+            p.lda = g.lda, p.ldb = g.ldb;
+            aK = g.layout_a == R355_ROW_MAJOR, bK = g.layout_b == R355_COL_MAJOR;
+        }
+        else
+        {
+            p.m = g.n, p.n = g.m;
+            p.a = static_cast<const char*>(g.b), p.b = static_cast<const char*>(g.a);
+            p.lda = g.ldb, p.ldb = g.lda;
+            aK = g.layout_b == R355_COL_MAJOR, bK = g.layout_a == R355_ROW_MAJOR;
+        }
+        p.tilesM = p.m / TILE_M, p.tilesN = p.n / TILE_N;
+        p.banks64 = 0;
+        switch(g.in_type)
+        {
+        case R355_F16:
+            return g.out_type == R355_F16 ? launchLayouts<Elem::F16, _Float16>(aK, bK, p, stream)
+                                          : launchLayouts<Elem::F16, float>(aK, bK, p, stream);
+        case R355_BF16:
+            return g.out_type == R355_BF16 ? launchLayouts<Elem::BF16, __bf16>(aK, bK, p, stream)
+                                           : launchLayouts<Elem::BF16, float>(aK, bK, p, stream);
+        case R355_E4M3: return launchLayouts<Elem::E4M3, float>(aK, bK, p, stream);
+        case R355_I8: return launchLayouts<Elem::I8, int>(aK, bK, p, stream);
+        default: return fail(R355_ERR_UNSUPPORTED, "tiled gemm: unknown in_type %d", g.in_type);
+        }
+    }
+} // namespace r355

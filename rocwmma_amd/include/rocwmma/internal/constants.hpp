@@ -1,0 +1,37 @@
+// Hardware constants of the one supported target (gfx950 / MI355X).
+// Public names follow library/include/rocwmma/internal/constants.hpp:33-101.
+#ifndef ROCWMMA_CONSTANTS_HPP
+#define ROCWMMA_CONSTANTS_HPP
+
+#include "types.hpp"
+
+namespace rocwmma
+{
+    struct Constants
+    {
+        static constexpr uint32_t AMDGCN_ARCH_ID_GFX950 = 0x950;
+        static constexpr uint32_t AMDGCN_ARCH_ID_NONE   = 0x0;
+
+        static constexpr uint32_t AMDGCN_WAVE_SIZE_64   = 64u;
+        static constexpr uint32_t AMDGCN_WAVE_SIZE_32   = 32u;
+        static constexpr uint32_t AMDGCN_WAVE_SIZE_NONE = 0u;
+
+#if ROCWMMA_ARCH_GFX950
+        static constexpr uint32_t AMDGCN_CURRENT_ARCH_ID = AMDGCN_ARCH_ID_GFX950;
+#else
+        static constexpr uint32_t AMDGCN_CURRENT_ARCH_ID = AMDGCN_ARCH_ID_NONE;
+#endif
+        // Host code sees the device's wave size too: there is only one.
+        static constexpr uint32_t AMDGCN_WAVE_SIZE = AMDGCN_WAVE_SIZE_64;
+
+        static constexpr uint32_t AMDGCN_REGISTER_ELEMENT_SIZE_BYTES = 4u;
+        static constexpr uint32_t AMDGCN_REGISTER_SIZE_BYTES
+            = AMDGCN_REGISTER_ELEMENT_SIZE_BYTES * AMDGCN_WAVE_SIZE;
+
+        static constexpr uint32_t AMDGCN_LDS_MAX_SIZE_BYTES    = 163840u; // 160 KiB per CU
+        static constexpr uint32_t AMDGCN_CACHE_LINE_SIZE_BYTES = 128u;
+        static constexpr uint32_t AMDGCN_DWORD_SIZE_BYTES      = 4u;
+    };
+} // namespace rocwmma
+
+#endif // ROCWMMA_CONSTANTS_HPP

@@ -1,0 +1,106 @@
+"""CPU-side checks of the C-ABI boundary: the library loads, exports every symbol the header
+declares, and validates arguments before touching a GPU."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import rocwmma_amd as R
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "r355_wmma.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(r355_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_symbols()
+    assert len(names) >= 12
+    L = ctypes.CDLL(R.LIB_PATH)
+    for name in names:
+        assert hasattr(L, name), name
+    assert sorted(R.EXPORTS) == names
+
+
+def test_version_and_error_channel():
+    assert "gfx950" in R.version()
+    g = R.gemm_args(R.F16, R.F16, 0, 256, 256, 1, 1, None, 1, 1.0, 0.0, R.ROW_MAJOR, R.COL_MAJOR, R.ROW_MAJOR, R.ROW_MAJOR)
+    with pytest.raises(R.R355Error) as e:
+        R.gemm_query(g)
+    assert e.value.code == -1 and "non-zero" in str(e.value)
+
+
+def _args(**kw):
+    base = dict(in_type=R.F16, out_type=R.F16, m=256, n=256, k=256, a=0x1000, b=0x2000, c=None, d=0x3000, alpha=1.0,
+                beta=0.0, layout_a=R.COL_MAJOR, layout_b=R.ROW_MAJOR, layout_c=R.ROW_MAJOR, layout_d=R.ROW_MAJOR)
+    base.update(kw)
+    return R.gemm_args(**base)
+
+
+def test_query_selects_kernel_family_and_reports_launch_shape():
+    plan = R.gemm_query(_args(m=8192, n=8192, k=8192))
+    assert plan.kernel == R.KERNEL_TILED
+    assert (plan.macro_tile_m, plan.macro_tile_n, plan.macro_tile_k) == (256, 256, 64)
+    assert plan.grid_x == 1024 and plan.block_x == 256 and plan.lds_bytes == 131072
+    # int8: 128 elements of K per stage
+    plan = R.gemm_query(_args(in_type=R.I8, out_type=R.I32, m=512, n=256, k=1024, layout_a=R.ROW_MAJOR, layout_b=R.COL_MAJOR))
+    assert plan.kernel == R.KERNEL_TILED and plan.macro_tile_k == 128 and plan.grid_x == 8
+    # shapes that do not fill a macro tile fall back to one block per wave
+    plan = R.gemm_query(_args(m=64, n=48, k=80, a=0x1000))
+    assert plan.kernel == R.KERNEL_SIMPLE and plan.lds_bytes == 0 and plan.macro_tile_m == 32
+
+
+@pytest.mark.parametrize("kw,code", [
+    (dict(a=None), -1),
+    (dict(beta=1.0, c=None), -1),
+    (dict(layout_a=7), -1),
+    (dict(in_type=R.F16, out_type=R.I32), -2),
+    (dict(m=100, n=256), -3),
+    (dict(k=24), -3),
+    (dict(kernel=R.KERNEL_TILED, m=128), -3),
+    (dict(a=0x1002, layout_a=R.ROW_MAJOR), -4),
+    (dict(lda=8), -1),
+])
+def test_argument_validation(kw, code):
+    with pytest.raises(R.R355Error) as e:
+        R.gemm_query(_args(**kw))
+    assert e.value.code == code, str(e.value)
+    assert str(e.value)
+
+
+def test_dlrm_and_gemv_validation_without_gpu():
+    with pytest.raises(R.R355Error) as e:
+        R.dlrm_fwd(R.F16, 0x1000, 0x2000, 40, 128, 8)
+    assert e.value.code == -3
+    with pytest.raises(R.R355Error) as e:
+        R.dlrm_fwd(R.F16, 0x1000, 0x2000, 27, 100, 8)
+    assert e.value.code == -3
+    with pytest.raises(R.R355Error) as e:
+        R.dlrm_fwd(R.F32, 0x1000, 0x2000, 27, 128, 8)
+    assert e.value.code == -2
+    with pytest.raises(R.R355Error) as e:
+        R.gemv(R.COL_MAJOR, 10, 16, 0x1000, 0x2000, None, 0x3000)
+    assert e.value.code == -3
+
+
+def test_compress_24_host_roundtrip_and_rejection():
+    import oraclelib as O
+
+    m, k = 32, 128
+    mask = O.sparse24_mask(9, m, k)
+    dense = np.where(mask, np.maximum(O.uniform_int8(10, m * k).reshape(m, k), 1), 0).astype(np.int8)
+    vals, meta = R.compress_24(dense)
+    # same format as the oracle's compressor
+    ov, om = O.compress24(dense.view(np.uint8), m, k)
+    assert np.array_equal(vals.view(np.uint8), ov) and np.array_equal(meta, om)
+    assert np.array_equal(R.decompress_24(vals, meta), dense)
+    bad = dense.copy()
+    bad[3, 4:8] = 1
+    with pytest.raises(R.R355Error) as e:
+        R.compress_24(bad)
+    assert e.value.code == -6 and "row 3" in str(e.value)

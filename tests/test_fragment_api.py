@@ -1,0 +1,185 @@
+"""GPU checks of the header-only fragment API (rocwmma_amd/include/rocwmma) through small device
+kernels (tests/kernels/api_kernels.hip).  The invariants are the reference's unit-test invariants:
+load -> store returns the block and nothing else (test/unit/load_store_matrix_sync_test,
+contamination_test), fill stores a constant (fill_fragment_test), cooperative load/store over
+1..8 waves reproduces the block (load_store_matrix_coop_sync_test), MappingUtil arithmetic
+(map_util_test), and mma_sync on one tile equals the CPU oracle's gemm."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import oraclelib as O
+from gpuutil import api_lib, device_filled, to_device, to_host
+
+pytestmark = pytest.mark.gpu
+
+CASES = list(range(26))
+
+
+def _info(cid):
+    r, c, eb, rm, ne = (ctypes.c_uint32() for _ in range(5))
+    assert api_lib().api_case_info(cid, ctypes.byref(r), ctypes.byref(c), ctypes.byref(eb), ctypes.byref(rm), ctypes.byref(ne)) == 0
+    return r.value, c.value, eb.value, bool(rm.value), ne.value
+
+
+def _np_dtype(eb):
+    return {1: np.uint8, 2: np.uint16, 4: np.uint32}[eb]
+
+
+def _padded(rows, cols, eb, row_major, pad, seed):
+    """A (rows+2pad) x (cols+2pad) matrix of distinct-ish bytes; returns storage, ld, block offset."""
+    R_, C_ = rows + 2 * pad, cols + 2 * pad
+    dt = _np_dtype(eb)
+    vals = (np.arange(R_ * C_, dtype=np.uint64) * 2654435761 + seed) % (1 << (8 * eb) - 1)
+    if eb == 4:
+        vals = vals % (1 << 22)  # keep f32 patterns finite
+    mat = vals.astype(dt).reshape(R_, C_)
+    ld = C_ if row_major else R_
+    off = pad * ld + pad
+    flat = mat.ravel() if row_major else np.ascontiguousarray(mat.T).ravel()
+    return mat, flat, ld, off
+
+
+@pytest.mark.parametrize("cid", CASES)
+def test_load_store_round_trip_leaves_padding_untouched(cid):
+    rows, cols, eb, rm, _ = _info(cid)
+    # alignment: vector accesses need the block origin aligned to 16 bytes along the contiguous dim
+    pad = 16 // eb
+    mat, flat, ld, off = _padded(rows, cols, eb, rm, pad, cid)
+    d_in = to_device(flat)
+    d_out = device_filled(flat.size, flat.dtype, 0xEE)
+    rc = api_lib().api_round_trip(cid, ctypes.c_void_p(d_in.data_ptr() + off * eb), ctypes.c_void_p(d_out.data_ptr() + off * eb), ld, ld)
+    assert rc == 0
+    out = to_host(d_out, flat.dtype)
+    out2d = out.reshape(mat.shape) if rm else out.reshape(mat.shape[::-1]).T
+    assert np.array_equal(out2d[pad:pad + rows, pad:pad + cols], mat[pad:pad + rows, pad:pad + cols])
+    canary = np.frombuffer(bytes([0xEE] * eb), dtype=flat.dtype)[0]
+    mask = np.ones(mat.shape, dtype=bool)
+    mask[pad:pad + rows, pad:pad + cols] = False
+    assert np.all(out2d[mask] == canary)
+
+
+@pytest.mark.parametrize("cid", [0, 3, 8, 9, 10, 11, 12, 22])
+def test_runtime_layout_overloads(cid):
+    rows, cols, eb, rm, _ = _info(cid)
+    mat, flat, ld, _ = _padded(rows, cols, eb, rm, 0, 77 + cid)
+    d_in, d_out = to_device(flat), device_filled(flat.size, flat.dtype, 0xEE)
+    assert api_lib().api_round_trip_runtime(cid, ctypes.c_void_p(d_in.data_ptr()), ctypes.c_void_p(d_out.data_ptr()), ld) == 0
+    assert np.array_equal(to_host(d_out, flat.dtype), flat)
+
+
+@pytest.mark.parametrize("cid", [0, 5, 6, 8, 11, 13, 15, 17, 20, 22, 25])
+def test_fill_fragment(cid):
+    rows, cols, eb, rm, ne = _info(cid)
+    assert ne == rows * cols // 64
+    ld = cols if rm else rows
+    d_out = device_filled(rows * cols, _np_dtype(eb), 0xEE)
+    assert api_lib().api_fill(cid, ctypes.c_void_p(d_out.data_ptr()), ld, ctypes.c_float(-3.0)) == 0
+    out = to_host(d_out, _np_dtype(eb))
+    if cid in (13, 21):
+        want = np.int8(-3).view(np.uint8)
+    elif cid == 22:
+        want = np.int32(-3).view(np.uint32)
+    elif cid in (15, 16):
+        want = O.f32_to_storage(np.float32([-3.0]), O.E4M3)[0]
+    elif cid in (6, 7):
+        want = O.f32_to_storage(np.float32([-3.0]), O.BF16)[0]
+    elif eb == 2:
+        want = np.float16(-3.0).view(np.uint16)
+    else:
+        want = np.float32(-3.0).view(np.uint32)
+    assert np.all(out == want)
+
+
+@pytest.mark.parametrize("cid", [4, 7, 10, 17, 18, 19, 20, 21, 25])
+@pytest.mark.parametrize("waves", [(1, 1), (2, 1), (2, 2), (4, 2)])
+@pytest.mark.parametrize("use_lds", [0, 1])
+def test_cooperative_round_trip(cid, waves, use_lds):
+    rows, cols, eb, rm, _ = _info(cid)
+    mat, flat, ld, _ = _padded(rows, cols, eb, rm, 0, 5 * cid + 1)
+    d_in, d_out = to_device(flat), device_filled(flat.size, flat.dtype, 0xEE)
+    rc = api_lib().api_coop_round_trip(cid, ctypes.c_void_p(d_in.data_ptr()), ctypes.c_void_p(d_out.data_ptr()), ld, waves[0], waves[1], use_lds)
+    assert rc == 0
+    assert np.array_equal(to_host(d_out, flat.dtype), flat)
+
+
+@pytest.mark.parametrize("cid", [17, 18])
+def test_cooperative_static_wave_count(cid):
+    rows, cols, eb, rm, _ = _info(cid)
+    mat, flat, ld, _ = _padded(rows, cols, eb, rm, 0, 31)
+    d_in, d_out = to_device(flat), device_filled(flat.size, flat.dtype, 0xEE)
+    assert api_lib().api_coop_round_trip_static4(cid, ctypes.c_void_p(d_in.data_ptr()), ctypes.c_void_p(d_out.data_ptr()), ld) == 0
+    assert np.array_equal(to_host(d_out, flat.dtype), flat)
+
+
+def test_transpose_and_data_layout_relabels():
+    # matrix_b 16(k) x 64(n) row-major viewed as matrix_a 64 x 16 col-major: same memory image
+    k, n = 16, 64
+    src = (np.arange(k * n) % 1000).astype(np.uint16)
+    d_in, d_out = to_device(src), device_filled(src.size, np.uint16, 0xEE)
+    assert api_lib().api_transpose_store(ctypes.c_void_p(d_in.data_ptr()), ctypes.c_void_p(d_out.data_ptr()), n) == 0
+    assert np.array_equal(to_host(d_out, np.uint16), src)
+    # matrix_a 32 x 16 loaded row-major, stored through the col-major relabel: memory holds the transpose
+    m, kk = 32, 16
+    a = (np.arange(m * kk) * 7 % 1000).astype(np.uint16).reshape(m, kk)
+    d_in, d_out = to_device(a.ravel()), device_filled(a.size, np.uint16, 0xEE)
+    assert api_lib().api_relayout_store(ctypes.c_void_p(d_in.data_ptr()), ctypes.c_void_p(d_out.data_ptr()), kk, m) == 0
+    assert np.array_equal(to_host(d_out, np.uint16).reshape(kk, m), a.T)
+
+
+def test_mapping_util_coordinates():
+    gx, gy, wx, wy, ld = 3, 2, 2, 4, 640
+    waves = gx * gy * wx * wy
+    d_out = device_filled(waves * 8, np.uint32, 0xEE)
+    assert api_lib().api_mapping_probe(ctypes.c_void_p(d_out.data_ptr()), ld, gx, gy, wx, wy) == 0
+    out = to_host(d_out, np.uint32).reshape(waves, 8)
+    for by in range(gy):
+        for bx in range(gx):
+            for w0 in range(wx):
+                for w1 in range(wy):
+                    w = (by * gx + bx) * wx * wy + w0 * wy + w1
+                    blk = (bx * wx + w0, by * wy + w1)
+                    mat = (blk[0] * 32, blk[1] * 16)
+                    assert tuple(out[w, :6]) == (w0, w1, blk[0], blk[1], mat[0], mat[1])
+                    assert out[w, 6] == mat[0] * ld + mat[1] and out[w, 7] == out[w, 6]
+
+
+TYPES = {0: (O.F16, O.F32), 1: (O.BF16, O.F32), 2: (O.E4M3, O.F32), 3: (O.I8, O.I32), 4: (O.F32, O.F32), 5: (O.F16, O.F16)}
+SHAPES = {0: [(16, 16), (16, 32), (32, 8), (32, 16)], 1: [(16, 16), (16, 32), (32, 8), (32, 16)],
+          2: [(16, 32), (16, 64), (32, 16), (32, 32)], 3: [(16, 32), (16, 64), (32, 16), (32, 32)],
+          4: [(16, 4), (16, 16), (32, 2), (32, 8)], 5: [(16, 16), (32, 16)]}
+
+
+@pytest.mark.parametrize("type_id", sorted(TYPES))
+@pytest.mark.parametrize("a_row,b_row,c_row", [(1, 0, 1), (0, 1, 0), (1, 1, 1), (0, 0, 0)])
+def test_mma_sync_single_tile_matches_oracle(type_id, a_row, b_row, c_row):
+    in_t, out_t = TYPES[type_id]
+    for blk, bk in SHAPES[type_id]:
+        m = n = blk
+        if in_t == O.I8:
+            a, b = O.uniform_int8(1, m * bk), O.uniform_int8(2, bk * n)
+            c = (O.uniform_int8(3, m * n).astype(np.int32) * 100)
+        else:
+            src = O.normal if in_t == O.E4M3 else O.uniform_pm1
+            a = O.f32_to_storage(src(1, m * bk), in_t)
+            b = O.f32_to_storage(src(2, bk * n), in_t)
+            c = O.f32_to_storage(O.uniform_pm1(3, m * n), out_t)
+        la, lb, lc = (O.ROW if a_row else O.COL), (O.ROW if b_row else O.COL), (O.ROW if c_row else O.COL)
+        want = O.gemm(in_t, out_t, la, lb, lc, lc, m, n, bk, a, b, c, 1.0, 1.0)
+        da, db, dc = to_device(a), to_device(b), to_device(c)
+        dd = device_filled(m * n, O.NP_STORAGE[out_t], 0xFF)
+        lda = bk if a_row else m
+        ldb = n if b_row else bk
+        rc = api_lib().api_mma_tile(type_id, blk, bk, a_row, b_row, c_row, ctypes.c_void_p(da.data_ptr()),
+                                    ctypes.c_void_p(db.data_ptr()), ctypes.c_void_p(dc.data_ptr()),
+                                    ctypes.c_void_p(dd.data_ptr()), lda, ldb, n if c_row else m)
+        assert rc == 0, (blk, bk)
+        got = to_host(dd, O.NP_STORAGE[out_t])
+        if in_t == O.I8:
+            assert np.array_equal(got, want), (blk, bk)
+        else:
+            # same products, different summation order than the sequential oracle: 10 eps of the
+            # output type on the reference's metric (100 eps for the 16-bit accumulate type)
+            ok, mx = O.compare(out_t, got, want, 100.0 if type_id == 5 else 10.0)
+            assert ok, (blk, bk, mx)

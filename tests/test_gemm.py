@@ -1,0 +1,183 @@
+"""GPU parity of the GEMM kernels (through the C ABI) against the CPU oracle.
+
+Bars: int8 -> int32 bit-exact; f16 / bf16 within 1e-3 and fp8 within 1e-2 relative error against
+the f32-accumulating oracle (on the reference's metric |a-b| / (|a|+|b|+1), which is what its
+validator uses), plus exact equality on the reference's integer-valued test inputs, where every
+partial sum is exact in any order."""
+import itertools
+
+import numpy as np
+import pytest
+
+import oraclelib as O
+import rocwmma_amd as R
+from gpuutil import device_filled, to_device, to_host
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = {O.F16: 1e-3, O.BF16: 1e-3, O.E4M3: 1e-2}
+
+
+def _inputs(in_t, out_t, m, n, k, seed=1, pattern="random"):
+    if pattern == "reference":
+        return None
+    if in_t == O.I8:
+        a, b = O.uniform_int8(seed, m * k), O.uniform_int8(seed + 1, k * n)
+        c = O.uniform_int8(seed + 2, m * n).astype(np.int32) * 37
+    else:
+        src = O.normal if in_t == O.E4M3 else O.uniform_pm1
+        a = O.f32_to_storage(src(seed, m * k), in_t)
+        b = O.f32_to_storage(src(seed + 1, k * n), in_t)
+        c = O.f32_to_storage(O.uniform_pm1(seed + 2, m * n), out_t)
+    return a, b, c
+
+
+def _run(in_t, out_t, la, lb, lc, ld, m, n, k, a, b, c, alpha, beta, kernel):
+    da, db = to_device(a), to_device(b)
+    dc = to_device(c) if c is not None else None
+    dd = device_filled(m * n, O.NP_STORAGE[out_t], 0xFF)
+    R.gemm(in_t, out_t, m, n, k, da, db, dc, dd, alpha, beta, la, lb, lc, ld, kernel=kernel)
+    return to_host(dd, O.NP_STORAGE[out_t])
+
+
+def _max_rel(out_t, got, want):
+    g = O.storage_to_f32(got, out_t).astype(np.float64)
+    w = O.storage_to_f32(want, out_t).astype(np.float64)
+    assert np.all(np.isfinite(g))
+    return float(np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)))
+
+
+def _check(in_t, out_t, got, want):
+    if in_t == O.I8:
+        assert np.array_equal(got, want)
+    else:
+        assert _max_rel(out_t, got, want) <= REL_TOL.get(in_t, 1e-5)
+
+
+def test_config1_256_cubed_f16_tn_alpha_beta_2():
+    # BASELINE config 1: A row-major (T), B col-major (N), C/D f32 row-major, alpha = beta = 2
+    m = n = k = 256
+    a, b, c = _inputs(O.F16, O.F32, m, n, k, seed=1)
+    want = O.gemm(O.F16, O.F32, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, 2.0)
+    for kernel in (R.KERNEL_SIMPLE, R.KERNEL_TILED):
+        got = _run(O.F16, O.F32, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, 2.0, kernel)
+        assert _max_rel(O.F32, got, want) <= 1e-3
+        # and the reference's own pass criterion: 10 eps(f32)
+        ok, mx = O.compare(O.F32, got, want, 10.0)
+        assert ok, mx
+
+
+TYPE_PAIRS = [(O.F16, O.F32), (O.F16, O.F16), (O.BF16, O.F32), (O.BF16, O.BF16), (O.E4M3, O.F32), (O.I8, O.I32), (O.F32, O.F32)]
+
+
+@pytest.mark.parametrize("in_t,out_t", TYPE_PAIRS)
+@pytest.mark.parametrize("la,lb", list(itertools.product([O.ROW, O.COL], repeat=2)))
+def test_simple_kernel_all_layouts_reference_inputs_exact(in_t, out_t, la, lb):
+    # the reference's integer-valued inputs (test/device/common.hpp:203-220): GPU == CPU exactly
+    m, n, k = 64, 96, 128
+    a, b = O.fill_ref(in_t, m, k, la), O.fill_ref(in_t, k, n, lb)
+    for lc, ld in ((O.ROW, O.COL), (O.COL, O.ROW)):
+        c = O.fill_ref(out_t, m, n, lc)
+        want = O.gemm(in_t, out_t, la, lb, lc, ld, m, n, k, a, b, c, 2.0, 2.0)
+        got = _run(in_t, out_t, la, lb, lc, ld, m, n, k, a, b, c, 2.0, 2.0, R.KERNEL_SIMPLE)
+        assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("in_t,out_t", TYPE_PAIRS)
+def test_simple_kernel_random_inputs_and_block16(in_t, out_t):
+    # 48 x 80: only the 16 x 16 block fits; non-square, ragged against the workgroup tile
+    m, n, k = 48, 80, 96
+    a, b, c = _inputs(in_t, out_t, m, n, k, seed=5)
+    want = O.gemm(in_t, out_t, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, -1.0)
+    got = _run(in_t, out_t, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, -1.0, R.KERNEL_SIMPLE)
+    if in_t == O.F32:
+        assert _max_rel(out_t, got, want) <= 1e-5
+    else:
+        _check(in_t, out_t, got, want)
+
+
+TILED_LAYOUTS_16 = list(itertools.product([O.ROW, O.COL], repeat=2))
+
+
+@pytest.mark.parametrize("in_t,out_t", [(O.F16, O.F16), (O.F16, O.F32), (O.BF16, O.BF16), (O.BF16, O.F32)])
+@pytest.mark.parametrize("la,lb", TILED_LAYOUTS_16)
+@pytest.mark.parametrize("ldl", [O.ROW, O.COL])
+def test_tiled_kernel_16bit_layouts(in_t, out_t, la, lb, ldl):
+    m, n, k = 512, 256, 384
+    a, b, c = _inputs(in_t, out_t, m, n, k, seed=11)
+    want = O.gemm(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, c, 2.0, 2.0)
+    got = _run(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, c, 2.0, 2.0, R.KERNEL_TILED)
+    _check(in_t, out_t, got, want)
+    # reference-pattern inputs: exact
+    a, b = O.fill_ref(in_t, m, k, la), O.fill_ref(in_t, k, n, lb)
+    want = O.gemm(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, None, 1.0, 0.0)
+    got = _run(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, None, 1.0, 0.0, R.KERNEL_TILED)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32)])
+@pytest.mark.parametrize("ldl", [O.ROW, O.COL])
+def test_tiled_kernel_8bit(in_t, out_t, ldl):
+    m, n, k = 256, 512, 768
+    a, b, c = _inputs(in_t, out_t, m, n, k, seed=21)
+    want = O.gemm(in_t, out_t, O.ROW, O.COL, ldl, ldl, m, n, k, a, b, c, 1.0, 1.0)
+    got = _run(in_t, out_t, O.ROW, O.COL, ldl, ldl, m, n, k, a, b, c, 1.0, 1.0, R.KERNEL_TILED)
+    _check(in_t, out_t, got, want)
+
+
+def test_tiled_kernel_many_tiles_xcd_mapping():
+    # 5 x 3 tiles: a tile count that is not a multiple of 8 and a partial row group
+    m, n, k = 1280, 768, 128
+    a, b, _ = _inputs(O.I8, O.I32, m, n, k, seed=31)
+    want = O.gemm(O.I8, O.I32, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0)
+    got = _run(O.I8, O.I32, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0, R.KERNEL_TILED)
+    assert np.array_equal(got, want)
+
+
+def test_auto_falls_back_and_bad_sizes_error():
+    m, n, k = 96, 64, 64
+    a, b, _ = _inputs(O.F16, O.F16, m, n, k)
+    want = O.gemm(O.F16, O.F16, O.COL, O.ROW, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0)
+    got = _run(O.F16, O.F16, O.COL, O.ROW, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0, R.KERNEL_AUTO)
+    _check(O.F16, O.F16, got, want)
+    with pytest.raises(R.R355Error) as e:
+        _run(O.F16, O.F16, O.COL, O.ROW, O.ROW, O.ROW, 100, 64, 64, a, b, None, 1.0, 0.0, R.KERNEL_AUTO)
+    assert e.value.code == -3
+
+
+@pytest.mark.parametrize("in_t,out_t,la,lb", [(O.F16, O.F16, O.COL, O.ROW), (O.BF16, O.BF16, O.COL, O.ROW),
+                                               (O.I8, O.I32, O.ROW, O.COL), (O.E4M3, O.F32, O.ROW, O.COL)])
+def test_full_size_8192_sampled_rows(in_t, out_t, la, lb):
+    # BASELINE configs 2 / 3 at full size.  Each element of the oracle depends only on its own row
+    # of A and column of B, so complete rows computed by the oracle are exactly its values.
+    import torch
+
+    m = n = k = 8192
+    if in_t == O.I8:
+        a, b = O.uniform_int8(1, m * k), O.uniform_int8(2, k * n)
+    else:
+        src = O.normal if in_t == O.E4M3 else O.uniform_pm1
+        a, b = O.f32_to_storage(src(1, m * k), in_t), O.f32_to_storage(src(2, k * n), in_t)
+    da, db = to_device(a), to_device(b)
+    dd = device_filled(m * n, O.NP_STORAGE[out_t], 0xFF)
+    R.gemm(in_t, out_t, m, n, k, da, db, None, dd, 1.0, 0.0, la, lb, O.ROW, O.ROW, kernel=R.KERNEL_TILED)
+    got = to_host(dd, O.NP_STORAGE[out_t]).reshape(m, n)
+    rows = np.array([0, 1, 255, 256, 4095, 5000, 8191, 7777], dtype=np.uint32)
+    want = O.gemm_rows(in_t, out_t, la, lb, m, n, k, a, b, rows)
+    if in_t == O.I8:
+        assert np.array_equal(got[rows], want)
+        # checksum of checksums over the whole matrix: sum(D) = (1^T A)(B 1), exact in int64
+        A = O.as_matrix(a, m, k, la).astype(np.int64)
+        B = O.as_matrix(b, k, n, lb).astype(np.int64)
+        assert int(got.astype(np.int64).sum()) == int(A.sum(axis=0) @ B.sum(axis=1))
+    else:
+        assert _max_rel(out_t, got[rows], want) <= REL_TOL[in_t]
+        # size-independent property on the full matrix: column sums against a float64 matvec
+        A = O.storage_to_f32(O.as_matrix(a, m, k, la), in_t).astype(np.float64)
+        B = O.storage_to_f32(O.as_matrix(b, k, n, lb), in_t).astype(np.float64)
+        colsum = A.sum(axis=0) @ B
+        gs = O.storage_to_f32(got, out_t).astype(np.float64).sum(axis=0)
+        scale = np.abs(A).sum(axis=0) @ np.abs(B)
+        assert np.max(np.abs(gs - colsum) / scale) < (2e-3 if in_t != O.E4M3 else 1e-3)
+    del da, db, dd
+    torch.cuda.empty_cache()

@@ -1,0 +1,27 @@
+"""GPU parity of the f32 GEMV kernel against the oracle's GEMM with n = 1 (the reference validates
+its GEMV sample the same way: samples/simple_sgemv.cpp runs gemm_cpu_h with n = 1)."""
+import numpy as np
+import pytest
+
+import oraclelib as O
+import rocwmma_amd as R
+from gpuutil import device_filled, to_device, to_host
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("layout", [O.ROW, O.COL])
+@pytest.mark.parametrize("m,k", [(256, 256), (1024, 512), (8192, 8192), (4100, 260)])
+def test_gemv_vs_oracle(layout, m, k):
+    a, x, y = O.uniform_pm1(1, m * k), O.uniform_pm1(2, k), O.uniform_pm1(3, m)
+    want = O.gemm(O.F32, O.F32, layout, O.COL, O.COL, O.COL, m, 1, k, a, x, y, 2.0, 2.0)
+    da, dx, dy = to_device(a), to_device(x), to_device(y)
+    dout = device_filled(m, np.float32, 0xFF)
+    R.gemv(layout, m, k, da, dx, dy, dout, 2.0, 2.0)
+    got = to_host(dout, np.float32)
+    # f32 sums of k products in a different order: k * eps relative to sum |a||x|
+    A = O.as_matrix(a, m, k, layout).astype(np.float64)
+    bound = (np.abs(A) @ np.abs(x.astype(np.float64))) * 2.0 * k * 6e-8 + 1e-6
+    assert np.all(np.abs(got.astype(np.float64) - want.astype(np.float64)) <= bound)
+    ok, mx = O.compare(O.F32, got, want, 100.0)
+    assert ok, mx

@@ -1,0 +1,60 @@
+"""GPU parity of the 2:4 structured-sparse GEMM (v_smfmac) against the oracle's dense GEMM on the
+decompressed A.  The reference has no sparse path: parity is pinned by the oracle plus the format
+invariants checked in test_oracle.py / test_cabi.py."""
+import numpy as np
+import pytest
+
+import oraclelib as O
+import rocwmma_amd as R
+from gpuutil import device_filled, to_device, to_host
+
+pytestmark = pytest.mark.gpu
+
+
+def _sparse_inputs(in_t, m, n, k, seed):
+    mask = O.sparse24_mask(seed, m, k)
+    if in_t == O.I8:
+        vals = O.uniform_int8(seed + 1, m * k).reshape(m, k)
+        b = O.uniform_int8(seed + 2, k * n)
+    else:
+        vals = O.f32_to_storage(O.normal(seed + 1, m * k), O.E4M3).view(np.int8).reshape(m, k)
+        b = O.f32_to_storage(O.normal(seed + 2, k * n), O.E4M3)
+    dense = np.where(mask, vals, np.int8(0)).astype(np.int8)
+    return dense, b
+
+
+@pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32)])
+@pytest.mark.parametrize("m,n,k", [(32, 32, 64), (96, 64, 256), (256, 128, 1024)])
+@pytest.mark.parametrize("ldl", [O.ROW, O.COL])
+def test_sparse_gemm_vs_dense_oracle(in_t, out_t, m, n, k, ldl):
+    dense, b = _sparse_inputs(in_t, m, n, k, 40)
+    vals, meta = R.compress_24(dense)
+    assert np.array_equal(R.decompress_24(vals, meta), dense)
+    storage = dense.view(np.uint8) if in_t == O.E4M3 else dense
+    c = (O.uniform_int8(50, m * n).astype(np.int32) * 11) if in_t == O.I8 else O.uniform_pm1(50, m * n)
+    want = O.gemm(in_t, out_t, O.ROW, O.COL, ldl, ldl, m, n, k, storage.ravel(), b, c, 1.0, 1.0)
+    dv, dm, db, dc = to_device(vals), to_device(meta), to_device(b), to_device(c)
+    dd = device_filled(m * n, O.NP_STORAGE[out_t], 0xFF)
+    R.gemm(in_t, out_t, m, n, k, dv, db, dc, dd, 1.0, 1.0, O.ROW, O.COL, ldl, ldl, a_meta=dm)
+    got = to_host(dd, O.NP_STORAGE[out_t])
+    if in_t == O.I8:
+        assert np.array_equal(got, want)
+    else:
+        g, w = got.astype(np.float64), want.astype(np.float64)
+        assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= 1e-2
+
+
+def test_sparse_config4_sampled_rows():
+    # BASELINE config 4: M = N = 4096, dense-equivalent K = 8192, int8
+    m, n, k = 4096, 4096, 8192
+    dense, b = _sparse_inputs(O.I8, m, n, k, 60)
+    vals, meta = R.compress_24(dense)
+    dv, dm, db = to_device(vals), to_device(meta), to_device(b)
+    dd = device_filled(m * n, np.int32, 0xFF)
+    R.gemm(O.I8, O.I32, m, n, k, dv, db, None, dd, 1.0, 0.0, O.ROW, O.COL, O.ROW, O.ROW, a_meta=dm)
+    got = to_host(dd, np.int32).reshape(m, n)
+    rows = np.array([0, 31, 32, 2047, 4095, 1234], dtype=np.uint32)
+    want = O.gemm_rows(O.I8, O.I32, O.ROW, O.COL, m, n, k, dense.ravel(), b, rows)
+    assert np.array_equal(got[rows], want)
+    B = b.reshape(n, k).astype(np.int64)
+    assert int(got.astype(np.int64).sum()) == int(dense.astype(np.int64).sum(axis=0) @ B.sum(axis=0))
