@@ -63,5 +63,19 @@ def build(force=False, verbose=True):
     return LIB
 
 
+def build_host_bench(verbose=True):
+    """C++ host bench (csrc/host_bench.cpp -> lib/host_bench), linked against the C-ABI library."""
+    exe = os.path.join(LIBDIR, "host_bench")
+    r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-std=c++17", "-O2", "-x", "hip",
+                        "-Wno-unused-command-line-argument", os.path.join(CSRC, "host_bench.cpp"), "-o", exe,
+                        "-L" + LIBDIR, "-lrocwmma_amd", "-Wl,-rpath,$ORIGIN"], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("host_bench build failed:\n" + r.stderr)
+    if verbose:
+        print("built", exe)
+    return exe
+
+
 if __name__ == "__main__":
     build(force="--force" in sys.argv)
+    build_host_bench()

@@ -1,0 +1,254 @@
+// C++ host bench for the C ABI: allocates device buffers, fills them from a seeded generator,
+// times the kernel with the reference's protocol (warm-up launches, then N launches between two
+// hipEvents: test/gemm/gemm_kernel_base_impl.hpp:647-676) and reports throughput the way the
+// reference does (2 m n k flop, test/performance.hpp:424-442), plus the fraction of MI355X's
+// published peak.  Usage:
+//   host_bench gemm  [--type f16|bf16|i8|e4m3] [--out f16|bf16|f32|i32] [--layout nt|tn|nn|tt]
+//                    [--m M --n N --k K] [--kernel auto|simple|tiled] [--warmup W --iters I]
+//   host_bench dlrm  [--batch B --m M --k K] [--warmup W --iters I]
+//   host_bench gemv  [--m M --k K --layout n|t]
+//   host_bench copy  [--bytes N]      plain device copy of known size (counter calibration)
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include <hip/hip_runtime.h>
+
+#include "../../include/r355_wmma.h"
+
+#define HIP_OK(expr)                                                                       \
+    do                                                                                     \
+    {                                                                                      \
+        hipError_t e_ = (expr);                                                            \
+        if(e_ != hipSuccess)                                                               \
+        {                                                                                  \
+            fprintf(stderr, "hip error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); \
+            return 1;                                                                      \
+        }                                                                                  \
+    } while(0)
+
+namespace
+{
+    uint64_t splitmix(uint64_t seed, uint64_t i)
+    {
+        uint64_t z = (i + 1) * 0x9E3779B97F4A7C15ull + seed * 0xD1B54A32D192ED03ull;
+        z          = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z          = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        return z ^ (z >> 31);
+    }
+
+    // cheap bit patterns in a sane range for each type: small values, no NaN / inf
+    void fillBytes(std::vector<uint8_t>& buf, int dtype, uint64_t seed)
+    {
+        const size_t es = (dtype == R355_F16 || dtype == R355_BF16) ? 2 : (dtype == R355_F32 ? 4 : 1);
+        const size_t n  = buf.size() / es;
+        for(size_t i = 0; i < n; ++i)
+        {
+            const uint64_t r = splitmix(seed, i);
+            switch(dtype)
+            {
+            case R355_F16: // sign, exponent 2^-4..2^-1, random mantissa: |x| in [1/16, 1)
+                reinterpret_cast<uint16_t*>(buf.data())[i]
+                    = static_cast<uint16_t>(((r & 1) << 15) | ((11 + ((r >> 1) & 3)) << 10) | ((r >> 8) & 0x3FF));
+                break;
+            case R355_BF16:
+                reinterpret_cast<uint16_t*>(buf.data())[i]
+                    = static_cast<uint16_t>(((r & 1) << 15) | ((123 + ((r >> 1) & 3)) << 7) | ((r >> 8) & 0x7F));
+                break;
+            case R355_E4M3: // exponent 3..6: |x| in [1/16, 1)
+                buf[i] = static_cast<uint8_t>(((r & 1) << 7) | ((3 + ((r >> 1) & 3)) << 3) | ((r >> 8) & 7));
+                break;
+            case R355_I8: buf[i] = static_cast<uint8_t>(r >> 32); break;
+            default: reinterpret_cast<float*>(buf.data())[i] = static_cast<float>((r >> 40) & 0xFFFF) / 65536.0f - 0.5f;
+            }
+        }
+    }
+
+    int parseType(const std::string& s)
+    {
+        if(s == "f16") return R355_F16;
+        if(s == "bf16") return R355_BF16;
+        if(s == "e4m3" || s == "fp8") return R355_E4M3;
+        if(s == "i8") return R355_I8;
+        if(s == "f32") return R355_F32;
+        if(s == "i32") return R355_I32;
+        return -1;
+    }
+
+    size_t bytesOf(int t)
+    {
+        return (t == R355_F16 || t == R355_BF16) ? 2 : ((t == R355_F32 || t == R355_I32) ? 4 : 1);
+    }
+
+    __global__ void copyKernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n)
+    {
+        for(size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+            dst[i] = src[i];
+    }
+} // namespace
+
+int main(int argc, char** argv)
+{
+    if(argc < 2)
+    {
+        fprintf(stderr, "usage: host_bench gemm|dlrm|gemv|copy [options]\n");
+        return 2;
+    }
+    const std::string op = argv[1];
+    std::string       type = "f16", out = "", layout = "nt", kernel = "auto";
+    uint32_t          m = 8192, n = 8192, k = 8192, batch = 65536;
+    bool              mSet = false, kSet = false;
+    int               warmup = 2, iters = 10;
+    size_t            bytes = 1ull << 30;
+    for(int i = 2; i + 1 < argc; i += 2)
+    {
+        const std::string a = argv[i], v = argv[i + 1];
+        if(a == "--type") type = v;
+        else if(a == "--out") out = v;
+        else if(a == "--layout") layout = v;
+        else if(a == "--kernel") kernel = v;
+        else if(a == "--m") m = atoi(v.c_str()), mSet = true;
+        else if(a == "--n") n = atoi(v.c_str());
+        else if(a == "--k") k = atoi(v.c_str()), kSet = true;
+        else if(a == "--batch") batch = atoi(v.c_str());
+        else if(a == "--warmup") warmup = atoi(v.c_str());
+        else if(a == "--iters") iters = atoi(v.c_str());
+        else if(a == "--bytes") bytes = strtoull(v.c_str(), nullptr, 10);
+        else
+        {
+            fprintf(stderr, "unknown option %s\n", a.c_str());
+            return 2;
+        }
+    }
+    r355_device_info dev;
+    if(r355_get_device_info(&dev) != R355_OK)
+    {
+        fprintf(stderr, "%s\n", r355_last_error());
+        return 1;
+    }
+    float ms = 0.0f;
+
+    if(op == "gemm")
+    {
+        const int inT = parseType(type);
+        if(out.empty())
+            out = inT == R355_I8 ? "i32" : (inT == R355_E4M3 ? "f32" : type);
+        const int outT = parseType(out);
+        r355_gemm_args g;
+        memset(&g, 0, sizeof(g));
+        g.in_type = inT, g.out_type = outT;
+        g.layout_a = layout[0] == 't' ? R355_ROW_MAJOR : R355_COL_MAJOR; // BLAS letters: T = row-major A
+        g.layout_b = layout[1] == 't' ? R355_ROW_MAJOR : R355_COL_MAJOR;
+        g.layout_c = g.layout_d = R355_ROW_MAJOR;
+        g.m = m, g.n = n, g.k = k;
+        g.lda = g.layout_a == R355_ROW_MAJOR ? k : m;
+        g.ldb = g.layout_b == R355_ROW_MAJOR ? n : k;
+        g.ldc = g.ldd = n;
+        g.alpha = 1.0f, g.beta = 0.0f;
+        g.kernel = kernel == "simple" ? R355_KERNEL_SIMPLE : (kernel == "tiled" ? R355_KERNEL_TILED : R355_KERNEL_AUTO);
+        std::vector<uint8_t> ha((size_t)m * k * bytesOf(inT)), hb((size_t)k * n * bytesOf(inT));
+        fillBytes(ha, inT, 1);
+        fillBytes(hb, inT, 2);
+        void *da, *db, *dd;
+        HIP_OK(hipMalloc(&da, ha.size()));
+        HIP_OK(hipMalloc(&db, hb.size()));
+        HIP_OK(hipMalloc(&dd, (size_t)m * n * bytesOf(outT)));
+        HIP_OK(hipMemcpy(da, ha.data(), ha.size(), hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(db, hb.data(), hb.size(), hipMemcpyHostToDevice));
+        HIP_OK(hipMemset(dd, 0xFF, (size_t)m * n * bytesOf(outT))); // NaN-prefill as the reference does
+        g.a = da, g.b = db, g.d = dd;
+        r355_gemm_plan plan;
+        if(r355_gemm_query(&g, &plan) != R355_OK || r355_gemm_timed(&g, nullptr, warmup, iters, &ms) != R355_OK)
+        {
+            fprintf(stderr, "%s\n", r355_last_error());
+            return 1;
+        }
+        const double flop   = 2.0 * m * n * k;
+        const double tflops = flop / ms / 1e9;
+        const double vendor = (inT == R355_I8 || inT == R355_E4M3) ? 5000.0 : 2500.0; // dense TFLOP/s | TOP/s
+        const double perClk = (inT == R355_I8 || inT == R355_E4M3) ? 8192.0 : 4096.0; // flop / CU / clk
+        const double model  = perClk * dev.compute_units * dev.clock_mhz * 1e-6; // TFLOP/s at the reported clock
+        printf("{\"op\": \"gemm\", \"type\": \"%s\", \"out\": \"%s\", \"layout\": \"%s\", \"m\": %u, \"n\": %u, \"k\": %u, "
+               "\"kernel\": %d, \"macro_tile\": [%u, %u, %u], \"lds_bytes\": %u, \"ms\": %.4f, \"tflops\": %.1f, "
+               "\"frac_vendor_peak\": %.4f, \"frac_clock_model_peak\": %.4f, \"cus\": %d, \"clock_mhz\": %d}\n",
+               type.c_str(), out.c_str(), layout.c_str(), m, n, k, plan.kernel, plan.macro_tile_m, plan.macro_tile_n,
+               plan.macro_tile_k, plan.lds_bytes, ms, tflops, tflops / vendor, tflops / model, dev.compute_units,
+               dev.clock_mhz);
+    }
+    else if(op == "dlrm")
+    {
+        if(!mSet) m = 27;
+        if(!kSet) k = 128;
+        const size_t inElems = (size_t)batch * m * k, outElems = (size_t)batch * (k + m * (m - 1) / 2);
+        std::vector<uint8_t> hx(inElems * 2);
+        fillBytes(hx, R355_F16, 3);
+        void *dx, *dout;
+        HIP_OK(hipMalloc(&dx, hx.size()));
+        HIP_OK(hipMalloc(&dout, outElems * 2));
+        HIP_OK(hipMemcpy(dx, hx.data(), hx.size(), hipMemcpyHostToDevice));
+        if(r355_dlrm_fwd_timed(R355_F16, dx, dout, m, k, batch, nullptr, warmup, iters, &ms) != R355_OK)
+        {
+            fprintf(stderr, "%s\n", r355_last_error());
+            return 1;
+        }
+        const double byts = (double)(inElems + outElems) * 2.0;
+        printf("{\"op\": \"dlrm_fwd\", \"batch\": %u, \"m\": %u, \"k\": %u, \"ms\": %.4f, \"gbps\": %.1f, "
+               "\"frac_hbm_peak\": %.4f, \"gflops_ref_convention\": %.1f}\n",
+               batch, m, k, ms, byts / ms / 1e6, byts / ms / 1e6 / 8000.0, 2.0 * m * m * k * batch / ms / 1e6);
+    }
+    else if(op == "gemv")
+    {
+        if(!mSet) m = 8192;
+        if(!kSet) k = 8192;
+        std::vector<uint8_t> ha((size_t)m * k * 4), hx((size_t)k * 4);
+        fillBytes(ha, R355_F32, 4);
+        fillBytes(hx, R355_F32, 5);
+        void *da, *dx, *dy;
+        HIP_OK(hipMalloc(&da, ha.size()));
+        HIP_OK(hipMalloc(&dx, hx.size()));
+        HIP_OK(hipMalloc(&dy, (size_t)m * 4));
+        HIP_OK(hipMemcpy(da, ha.data(), ha.size(), hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(dx, hx.data(), hx.size(), hipMemcpyHostToDevice));
+        const int lay = layout[0] == 't' ? R355_ROW_MAJOR : R355_COL_MAJOR;
+        if(r355_gemv_timed(lay, m, k, (const float*)da, lay == R355_ROW_MAJOR ? k : m, (const float*)dx, nullptr,
+                           (float*)dy, 1.0f, 0.0f, nullptr, warmup, iters, &ms)
+           != R355_OK)
+        {
+            fprintf(stderr, "%s\n", r355_last_error());
+            return 1;
+        }
+        const double byts = (double)m * k * 4.0 + (double)(m + k) * 4.0;
+        printf("{\"op\": \"gemv\", \"m\": %u, \"k\": %u, \"ms\": %.4f, \"gbps\": %.1f, \"frac_hbm_peak\": %.4f}\n", m, k,
+               ms, byts / ms / 1e6, byts / ms / 1e6 / 8000.0);
+    }
+    else if(op == "copy")
+    {
+        void *src, *dst;
+        HIP_OK(hipMalloc(&src, bytes));
+        HIP_OK(hipMalloc(&dst, bytes));
+        HIP_OK(hipMemset(src, 1, bytes));
+        hipEvent_t e0, e1;
+        HIP_OK(hipEventCreate(&e0));
+        HIP_OK(hipEventCreate(&e1));
+        for(int i = 0; i < warmup; ++i)
+            hipLaunchKernelGGL(copyKernel, dim3(4096), dim3(256), 0, 0, (const uint4*)src, (uint4*)dst, bytes / 16);
+        HIP_OK(hipEventRecord(e0));
+        for(int i = 0; i < iters; ++i)
+            hipLaunchKernelGGL(copyKernel, dim3(4096), dim3(256), 0, 0, (const uint4*)src, (uint4*)dst, bytes / 16);
+        HIP_OK(hipEventRecord(e1));
+        HIP_OK(hipEventSynchronize(e1));
+        HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+        ms /= iters;
+        printf("{\"op\": \"copy\", \"bytes_read\": %zu, \"bytes_written\": %zu, \"ms\": %.4f, \"gbps\": %.1f}\n", bytes,
+               bytes, ms, 2.0 * bytes / ms / 1e6);
+    }
+    else
+    {
+        fprintf(stderr, "unknown op %s\n", op.c_str());
+        return 2;
+    }
+    return 0;
+}

@@ -9,8 +9,9 @@
 // B is dense, col-major (k contiguous); D row- or col-major.
 //
 // Kernel: one 32 x 32 block of D per wave, operands streamed from global memory
-// (lane = row / column, 16 kept bytes + 4 index bytes of A and 32 dense bytes of B per
-// 64-wide K step).
+// (lane = row / column, 16 kept bytes + 4 index bytes of A and 2 x 16 dense bytes of B per
+// 64-wide K step).  Operand formats of v_smfmac_*_32x32x64 as measured on MI355X: index
+// bits [2 p + 1 : 2 p] give the position within its group of 4 of kept byte p of the lane.
 #include <hip/hip_runtime.h>
 
 #include <cstring>
@@ -55,7 +56,11 @@ namespace
 
         const uint8_t* pa = aVals + (uint64_t)(row0 + idx) * lda + 16u * g;
         const uint8_t* pm = aMeta + (uint64_t)(row0 + idx) * (k / 8u) + 4u * g;
-        const uint8_t* pb = b + (uint64_t)(col0 + idx) * ldb + 32u * g;
+        // The instruction pairs A's lane group g, kept bytes [8 q, 8 q + 8) with B's lane group q,
+        // dense bytes [16 g, 16 g + 16).  With A's lane group g holding the kept values of dense
+        // k in [32 g, 32 g + 32), B's lane group h therefore holds dense k in [16 h, 16 h + 16)
+        // and [32 + 16 h, 48 + 16 h) of each 64-wide step.
+        const uint8_t* pb = b + (uint64_t)(col0 + idx) * ldb + 16u * g;
 
         Acc acc;
 #pragma unroll
@@ -67,7 +72,7 @@ namespace
             const i32x4 av   = *reinterpret_cast<const i32x4*>(pa + kd / 2u);
             const int   meta = *reinterpret_cast<const int*>(pm + kd / 8u);
             const i32x4 b0   = *reinterpret_cast<const i32x4*>(pb + kd);
-            const i32x4 b1   = *reinterpret_cast<const i32x4*>(pb + kd + 16u);
+            const i32x4 b1   = *reinterpret_cast<const i32x4*>(pb + kd + 32u);
             const i32x8 bv   = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
             if constexpr(FP8)
                 acc = __builtin_amdgcn_smfmac_f32_32x32x64_fp8_fp8(av, bv, acc, meta, 0, 0);

@@ -180,6 +180,12 @@ def test_mma_sync_single_tile_matches_oracle(type_id, a_row, b_row, c_row):
             assert np.array_equal(got, want), (blk, bk)
         else:
             # same products, different summation order than the sequential oracle: 10 eps of the
-            # output type on the reference's metric (100 eps for the 16-bit accumulate type)
-            ok, mx = O.compare(out_t, got, want, 100.0 if type_id == 5 else 10.0)
-            assert ok, (blk, bk, mx)
+            # output type on the reference's metric (100 eps for the 16-bit accumulate type).
+            # The fp8 matrix core does not keep full f32 precision inside one instruction
+            # (observed 1e-4): it gets the stated fp8 bar of 1e-2.
+            if in_t == O.E4M3:
+                g, w = got.astype(np.float64), want.astype(np.float64)
+                assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= 1e-2, (blk, bk)
+            else:
+                ok, mx = O.compare(out_t, got, want, 100.0 if type_id == 5 else 10.0)
+                assert ok, (blk, bk, mx)

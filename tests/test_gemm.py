@@ -1,9 +1,15 @@
 """GPU parity of the GEMM kernels (through the C ABI) against the CPU oracle.
 
-Bars: int8 -> int32 bit-exact; f16 / bf16 within 1e-3 and fp8 within 1e-2 relative error against
-the f32-accumulating oracle (on the reference's metric |a-b| / (|a|+|b|+1), which is what its
-validator uses), plus exact equality on the reference's integer-valued test inputs, where every
-partial sum is exact in any order."""
+Bars, on the reference's metric |a-b| / (|a|+|b|+1) (test/device/common.hpp:111-124):
+  int8 -> int32            bit-exact
+  f16, bf16 inputs         <= 1e-3 against the oracle's f32 result (f32 accumulation on both
+                           sides, different summation order)
+  fp8 e4m3 inputs          <= 1e-2
+  16-bit outputs           the bound above plus half an ulp of the output type (2^-11 for f16,
+                           2^-9 for bf16) against the oracle's f32 result, and never more than
+                           one ulp away from the oracle's own 16-bit result
+plus exact equality on the reference's integer-valued test inputs (test/device/common.hpp:203-220),
+where every partial sum is exact in any order."""
 import itertools
 
 import numpy as np
@@ -47,11 +53,27 @@ def _max_rel(out_t, got, want):
     return float(np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)))
 
 
-def _check(in_t, out_t, got, want):
+HALF_ULP = {O.F16: 2.0 ** -11, O.BF16: 2.0 ** -9, O.F32: 0.0}
+
+
+def _check(in_t, out_t, got, want, want_f32=None):
+    """got / want in out_t storage; want_f32 = the oracle's f32-output result when out_t is 16-bit."""
     if in_t == O.I8:
         assert np.array_equal(got, want)
-    else:
-        assert _max_rel(out_t, got, want) <= REL_TOL.get(in_t, 1e-5)
+        return
+    tol = REL_TOL.get(in_t, 1e-5)
+    if out_t == O.F32:
+        assert _max_rel(out_t, got, want) <= tol
+        return
+    g = O.storage_to_f32(got, out_t).astype(np.float64)
+    assert np.all(np.isfinite(g))
+    if want_f32 is not None:
+        w = want_f32.astype(np.float64)
+        assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= tol + HALF_ULP[out_t]
+    # at most one ulp of the output type from the oracle's rounded result
+    w16 = O.storage_to_f32(want, out_t).astype(np.float64)
+    ulp = np.maximum(np.abs(w16), 2.0 ** -14) * (4 * HALF_ULP[out_t])
+    assert np.all(np.abs(g - w16) <= ulp + tol * (np.abs(w16) + 1.0))
 
 
 def test_config1_256_cubed_f16_tn_alpha_beta_2():
@@ -62,9 +84,14 @@ def test_config1_256_cubed_f16_tn_alpha_beta_2():
     for kernel in (R.KERNEL_SIMPLE, R.KERNEL_TILED):
         got = _run(O.F16, O.F32, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, 2.0, kernel)
         assert _max_rel(O.F32, got, want) <= 1e-3
-        # and the reference's own pass criterion: 10 eps(f32)
+    # the reference's own pass criterion (10 eps of f32) applies to its integer-valued inputs,
+    # where GPU and CPU agree exactly
+    a, b, c = O.fill_ref(O.F16, m, k, O.ROW), O.fill_ref(O.F16, k, n, O.COL), O.fill_ref(O.F32, m, n, O.ROW)
+    want = O.gemm(O.F16, O.F32, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, 2.0)
+    for kernel in (R.KERNEL_SIMPLE, R.KERNEL_TILED):
+        got = _run(O.F16, O.F32, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, 2.0, kernel)
         ok, mx = O.compare(O.F32, got, want, 10.0)
-        assert ok, mx
+        assert ok and mx == 0.0, mx
 
 
 TYPE_PAIRS = [(O.F16, O.F32), (O.F16, O.F16), (O.BF16, O.F32), (O.BF16, O.BF16), (O.E4M3, O.F32), (O.I8, O.I32), (O.F32, O.F32)]
@@ -90,10 +117,11 @@ def test_simple_kernel_random_inputs_and_block16(in_t, out_t):
     a, b, c = _inputs(in_t, out_t, m, n, k, seed=5)
     want = O.gemm(in_t, out_t, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, -1.0)
     got = _run(in_t, out_t, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, -1.0, R.KERNEL_SIMPLE)
-    if in_t == O.F32:
-        assert _max_rel(out_t, got, want) <= 1e-5
-    else:
-        _check(in_t, out_t, got, want)
+    w32 = None
+    if out_t in (O.F16, O.BF16):
+        c32 = O.storage_to_f32(c, out_t)
+        w32 = O.gemm(in_t, O.F32, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c32, 2.0, -1.0)
+    _check(in_t, out_t, got, want, w32)
 
 
 TILED_LAYOUTS_16 = list(itertools.product([O.ROW, O.COL], repeat=2))
@@ -107,7 +135,10 @@ def test_tiled_kernel_16bit_layouts(in_t, out_t, la, lb, ldl):
     a, b, c = _inputs(in_t, out_t, m, n, k, seed=11)
     want = O.gemm(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, c, 2.0, 2.0)
     got = _run(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, c, 2.0, 2.0, R.KERNEL_TILED)
-    _check(in_t, out_t, got, want)
+    w32 = None
+    if out_t != O.F32:
+        w32 = O.gemm(in_t, O.F32, la, lb, ldl, ldl, m, n, k, a, b, O.storage_to_f32(c, out_t), 2.0, 2.0)
+    _check(in_t, out_t, got, want, w32)
     # reference-pattern inputs: exact
     a, b = O.fill_ref(in_t, m, k, la), O.fill_ref(in_t, k, n, lb)
     want = O.gemm(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, None, 1.0, 0.0)
@@ -127,7 +158,7 @@ def test_tiled_kernel_8bit(in_t, out_t, ldl):
 
 def test_tiled_kernel_many_tiles_xcd_mapping():
     # 5 x 3 tiles: a tile count that is not a multiple of 8 and a partial row group
-    m, n, k = 1280, 768, 128
+    m, n, k = 1280, 768, 256
     a, b, _ = _inputs(O.I8, O.I32, m, n, k, seed=31)
     want = O.gemm(O.I8, O.I32, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0)
     got = _run(O.I8, O.I32, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0, R.KERNEL_TILED)
@@ -171,7 +202,8 @@ def test_full_size_8192_sampled_rows(in_t, out_t, la, lb):
         B = O.as_matrix(b, k, n, lb).astype(np.int64)
         assert int(got.astype(np.int64).sum()) == int(A.sum(axis=0) @ B.sum(axis=1))
     else:
-        assert _max_rel(out_t, got[rows], want) <= REL_TOL[in_t]
+        w32 = O.gemm_rows(in_t, O.F32, la, lb, m, n, k, a, b, rows) if out_t != O.F32 else None
+        _check(in_t, out_t, got[rows].ravel(), want.ravel(), None if w32 is None else w32.ravel())
         # size-independent property on the full matrix: column sums against a float64 matvec
         A = O.storage_to_f32(O.as_matrix(a, m, k, la), in_t).astype(np.float64)
         B = O.storage_to_f32(O.as_matrix(b, k, n, lb), in_t).astype(np.float64)
