@@ -1,0 +1,191 @@
+#!/usr/bin/env python3
+"""Headline benchmark: dense GEMM M = N = K = 8192, f16 inputs (A col-major, B row-major = "NT"),
+f32 accumulation, f16 row-major output, alpha = 1, beta = 0 -- on one MI355X through the C ABI.
+
+One "step" is one GEMM launch on device-resident operands.  Prints ONE JSON line:
+  value        TFLOP/s over the timed region (2 m n k flop per step, wall clock between two
+               torch.cuda.synchronize() calls)
+  roofline     the same kernel timed with HIP events on its launch stream, against MI355X's
+               published dense f16 MFMA peak (2.5 PFLOP/s)
+  cpu_baseline the CPU oracle (port of the reference's OpenMP gemm_CPU) timed on a bounded sample
+               of complete output rows of the same workload; the same rows validate the GPU result
+  extra        the other BASELINE configurations (bf16, int8, fp8, 2:4 sparse, DLRM) with their
+               own roofline fractions (skipped with --quick)
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "e4m3": 5000.0, "i8": 5000.0}
+HBM_PEAK_GBPS = 8000.0
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--size", type=int, default=8192, help="M = N = K (default: the BASELINE size)")
+    ap.add_argument("--cpu-rows", type=int, default=48, help="output rows the CPU baseline computes")
+    ap.add_argument("--quick", action="store_true", help="skip the extra configurations")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (got --gpus %d); every kernel here is a "
+              "single-device kernel and nothing is sharded" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    import oraclelib as O  # CPU oracle: used only for cpu_baseline and for validating the result
+    import rocwmma_amd as R
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    if not os.path.exists(R.LIB_PATH):
+        from rocwmma_amd import build
+
+        build.build()
+    dev = R.device_info()
+    m = n = k = args.size
+    flop = 2.0 * m * n * k
+
+    # ---- workload: seeded U[-1, 1) rounded to f16 (seeds 1, 2), generated on the host so that the
+    # CPU baseline sees the same bits
+    a = O.f32_to_storage(O.uniform_pm1(1, m * k), O.F16)  # col-major m x k
+    b = O.f32_to_storage(O.uniform_pm1(2, k * n), O.F16)  # row-major k x n
+    da = torch.from_numpy(a.view(np.int16)).cuda()
+    db = torch.from_numpy(b.view(np.int16)).cuda()
+    dd = torch.full((m * n,), -1, dtype=torch.int16, device="cuda")  # 0xFFFF = NaN prefill
+    g = R.gemm_args(R.F16, R.F16, m, n, k, da, db, None, dd, 1.0, 0.0, R.COL_MAJOR, R.ROW_MAJOR, R.ROW_MAJOR,
+                    R.ROW_MAJOR, kernel=R.KERNEL_AUTO)
+    plan = R.gemm_query(g)
+
+    import ctypes
+
+    launch = R.lib().r355_gemm
+    gref = ctypes.byref(g)
+    for _ in range(args.warmup):
+        assert launch(gref, None) == 0, R.lib().r355_last_error()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        launch(gref, None)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = flop / wall_ms / 1e9
+
+    # kernel duration by HIP events on the launch stream
+    ev_ms = R.gemm_timed(g, 1, args.steps)
+    achieved = flop / ev_ms / 1e9
+
+    # ---- CPU baseline on a bounded sample (complete rows of D), doubling as validation
+    rows = np.linspace(0, m - 1, args.cpu_rows).astype(np.uint32)
+    t0 = time.perf_counter()
+    want = O.gemm_rows(O.F16, O.F16, O.COL, O.ROW, m, n, k, a, b, rows)
+    cpu_s = time.perf_counter() - t0
+    cpu_tflops = 2.0 * len(rows) * n * k / cpu_s / 1e12
+    got = dd.cpu().numpy().view(np.uint16).reshape(m, n)[rows]
+    gf, wf = got.view(np.float16).astype(np.float64), want.view(np.float16).astype(np.float64)
+    max_rel = float(np.max(np.abs(gf - wf) / (np.abs(gf) + np.abs(wf) + 1.0)))
+    validated = bool(np.all(np.isfinite(gf)) and max_rel <= 1e-3)
+
+    extra = {}
+    if not args.quick:
+        extra = run_extras(R, O, np, torch, args)
+
+    line = {
+        "metric": "TFLOPS at 8192^3 f16 GEMM (f32 accumulate, NT, f16 out); int8 / bf16 / fp8 / sparse / DLRM in extra",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "dense GEMM M=N=K=%d, f16 A (col-major) x f16 B (row-major) -> f16 row-major, "
+                               "f32 accumulate, alpha=1 beta=0 (BASELINE configs[1])" % m,
+                   "kernel": {1: "block-per-wave", 2: "macro-tile"}[plan.kernel],
+                   "macro_tile": [plan.macro_tile_m, plan.macro_tile_n, plan.macro_tile_k],
+                   "lds_bytes": plan.lds_bytes, "grid": plan.grid_x, "block": plan.block_x,
+                   "seeds": {"A": 1, "B": 2}},
+        "frac_of_peak": round(value / PEAK_TFLOPS["f16"], 4),
+        "validated": validated,
+        "max_rel_error_vs_oracle": max_rel,
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_TFLOPS["f16"], 4), "traffic": None,
+                     "kernel_ms": round(ev_ms, 4), "algorithmic_flop": flop,
+                     "algorithmic_bytes": (m * k + k * n) * 2 + m * n * 2},
+        "cpu_baseline": {"value": round(cpu_tflops, 6), "unit": "TFLOP/s", "cores": O.lib().orc_num_threads(),
+                         "kind": "port",
+                         "sample": "%d complete rows of D (all %d columns, full K=%d) of the same workload, %.1f s; "
+                                   "extrapolated full problem %.0f s" % (len(rows), n, k, cpu_s, cpu_s * m / len(rows))},
+        "device": {"arch": dev.arch.decode(), "cus": dev.compute_units, "clock_mhz": dev.clock_mhz},
+        "extra": extra,
+    }
+    print(json.dumps(line))
+
+
+def run_extras(R, O, np, torch, args):
+    """The remaining BASELINE configurations, each timed with HIP events over args.steps launches."""
+    out = {}
+    s = args.size
+
+    def rnd16(nel, bf):
+        t = (torch.rand(nel, device="cuda") * 2 - 1)
+        return t.to(torch.bfloat16 if bf else torch.float16)
+
+    def gemm_case(name, in_t, out_t, la, lb, a, b, peak, unit, sparse_meta=None, mm=s, nn=s, kk=s, peak_scale=1.0):
+        d = torch.empty(mm * nn * R.DTYPE_BYTES[out_t], dtype=torch.uint8, device="cuda")
+        g = R.gemm_args(in_t, out_t, mm, nn, kk, a, b, None, d, 1.0, 0.0, la, lb, R.ROW_MAJOR, R.ROW_MAJOR,
+                        a_meta=sparse_meta)
+        ms = R.gemm_timed(g, args.warmup, args.steps)
+        tf = 2.0 * mm * nn * kk / ms / 1e9
+        out[name] = {"ms": round(ms, 4), "value": round(tf, 2), "unit": unit, "peak": peak * peak_scale,
+                     "frac": round(tf / (peak * peak_scale), 4)}
+
+    gemm_case("gemm_bf16_nt_8192", R.BF16, R.BF16, R.COL_MAJOR, R.ROW_MAJOR, rnd16(s * s, True), rnd16(s * s, True),
+              PEAK_TFLOPS["bf16"], "TFLOP/s")
+    gemm_case("gemm_f16_tn_8192", R.F16, R.F16, R.ROW_MAJOR, R.COL_MAJOR, rnd16(s * s, False), rnd16(s * s, False),
+              PEAK_TFLOPS["f16"], "TFLOP/s")
+    i8 = lambda nel: torch.randint(-128, 128, (nel,), dtype=torch.int16, device="cuda").to(torch.int8)
+    gemm_case("gemm_i8_tn_8192", R.I8, R.I32, R.ROW_MAJOR, R.COL_MAJOR, i8(s * s), i8(s * s), PEAK_TFLOPS["i8"], "TOP/s")
+    # e4m3 codes with exponent 3..9: |x| in [1/16, 8), no NaN
+    f8 = lambda nel: ((torch.randint(0x18, 0x50, (nel,), dtype=torch.int16, device="cuda")
+                       | (torch.randint(0, 2, (nel,), dtype=torch.int16, device="cuda") << 7)).to(torch.uint8))
+    gemm_case("gemm_e4m3_tn_8192", R.E4M3, R.F32, R.ROW_MAJOR, R.COL_MAJOR, f8(s * s), f8(s * s), PEAK_TFLOPS["e4m3"],
+              "TFLOP/s")
+    # 2:4 sparse, BASELINE config 4: M = N = 4096, dense-equivalent K = 8192, int8; dense-equivalent ops
+    # against the sparse peak (2 x dense)
+    sm, sn, sk = 4096, 4096, 8192
+    vals = i8(sm * sk // 2)
+    # index nibbles 0x4 = positions (0, 1) and 0x8 = positions (0, 2): idx0 < idx1 in every group
+    meta = torch.full((sm * sk // 8,), 0x84, dtype=torch.uint8, device="cuda")
+    gemm_case("gemm_i8_sparse24_4096x4096x8192", R.I8, R.I32, R.ROW_MAJOR, R.COL_MAJOR, vals, i8(sk * sn),
+              PEAK_TFLOPS["i8"], "TOP/s (dense-equivalent)", sparse_meta=meta, mm=sm, nn=sn, kk=sk, peak_scale=2.0)
+    # DLRM dot interaction forward, BASELINE config 5
+    bsz, mm, kk = 65536, 27, 128
+    x = torch.randn(bsz * mm * kk, device="cuda").to(torch.float16)
+    o = torch.empty(bsz * (kk + mm * (mm - 1) // 2), dtype=torch.float16, device="cuda")
+    ms = R.dlrm_fwd_timed(R.F16, x, o, mm, kk, bsz, args.warmup, args.steps)
+    byts = bsz * (mm * kk + kk + mm * (mm - 1) // 2) * 2
+    out["dlrm_fwd_b65536_f27_d128"] = {"ms": round(ms, 4), "value": round(byts / ms / 1e6, 1), "unit": "GB/s",
+                                       "peak": HBM_PEAK_GBPS, "frac": round(byts / ms / 1e6 / HBM_PEAK_GBPS, 4),
+                                       "algorithmic_bytes": byts,
+                                       "gflops_ref_convention": round(2.0 * mm * mm * kk * bsz / ms / 1e6, 1)}
+    return out
+
+
+if __name__ == "__main__":
+    main()

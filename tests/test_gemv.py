@@ -23,7 +23,7 @@ def test_gemv_vs_oracle(layout, m, k):
     A = O.as_matrix(a, m, k, layout).astype(np.float64)
     bound = (np.abs(A) @ np.abs(x.astype(np.float64))) * 2.0 * k * 6e-8 + 1e-6
     assert np.all(np.abs(got.astype(np.float64) - want.astype(np.float64)) <= bound)
-    # and close to the exact (float64) result on the reference's metric
+    # and close to the exact (float64) result on the reference's metric: k f32 roundings
     exact = 2.0 * (A @ x.astype(np.float64)) + 2.0 * y.astype(np.float64)
     g = got.astype(np.float64)
-    assert np.max(np.abs(g - exact) / (np.abs(g) + np.abs(exact) + 1.0)) <= 1e-5
+    assert np.max(np.abs(g - exact) / (np.abs(g) + np.abs(exact) + 1.0)) <= 1e-7 * k
