@@ -79,19 +79,46 @@ namespace
         for(uint32_t c = inChunks + lane; c < MAX_M * ROW_CHUNKS; c += 64)
             *reinterpret_cast<i32x4*>(xw + c * 16u) = i32x4{0, 0, 0, 0};
 
-        for(uint32_t sIdx = wave; sIdx < SAMPLES_PER_WG; sIdx += WAVES)
+        // Both samples of this wave are requested from HBM before either is consumed: the kernel is
+        // bandwidth-bound, and bytes in flight per CU are what keeps HBM busy.
+        constexpr uint32_t PER_WAVE   = SAMPLES_PER_WG / WAVES; // 2
+        constexpr uint32_t MAX_CHUNKS = (MAX_M * ROW_CHUNKS + 63u) / 64u; // loads per lane per sample
+        i32x4              stash[PER_WAVE][MAX_CHUNKS];
+#pragma unroll
+        for(uint32_t q = 0; q < PER_WAVE; ++q)
         {
-            const uint32_t b = b0 + sIdx;
+            const uint32_t b = b0 + wave + q * WAVES;
+            if(b < batch)
+            {
+                const char* src = reinterpret_cast<const char*>(in) + (uint64_t)b * m * K * 2u;
+#pragma unroll
+                for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
+                {
+                    const uint32_t c = j * 64u + lane;
+                    if(c < inChunks)
+                        stash[q][j] = *reinterpret_cast<const i32x4*>(src + c * 16u);
+                }
+            }
+        }
+
+#pragma unroll
+        for(uint32_t q = 0; q < PER_WAVE; ++q)
+        {
+            const uint32_t sIdx = wave + q * WAVES;
+            const uint32_t b    = b0 + sIdx;
             if(b >= batch)
                 break;
-            // ---- X -> LDS: chunk c of the sample goes to row c / ROW_CHUNKS, slot (c % ROW_CHUNKS) ^ (row % ROW_CHUNKS')
-            const char* src = reinterpret_cast<const char*>(in) + (uint64_t)b * m * K * 2u;
-            for(uint32_t c = lane; c < inChunks; c += 64)
+            // ---- X -> LDS: chunk c of the sample goes to row c / ROW_CHUNKS, slot (c % ROW_CHUNKS) ^ (row % 16)
+#pragma unroll
+            for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
             {
-                const i32x4    v    = *reinterpret_cast<const i32x4*>(src + c * 16u);
-                const uint32_t row  = c / ROW_CHUNKS, col = c % ROW_CHUNKS;
-                const uint32_t slot = col ^ (row & (ROW_CHUNKS - 1u) & 15u);
-                *reinterpret_cast<i32x4*>(xw + (row * ROW_CHUNKS + slot) * 16u) = v;
+                const uint32_t c = j * 64u + lane;
+                if(c < inChunks)
+                {
+                    const uint32_t row  = c / ROW_CHUNKS, col = c % ROW_CHUNKS;
+                    const uint32_t slot = col ^ (row & (ROW_CHUNKS - 1u) & 15u);
+                    *reinterpret_cast<i32x4*>(xw + (row * ROW_CHUNKS + slot) * 16u) = stash[q][j];
+                }
             }
             __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): this wave's LDS writes are done
             __builtin_amdgcn_wave_barrier();

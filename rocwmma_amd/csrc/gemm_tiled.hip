@@ -27,6 +27,7 @@
 #include <hip/hip_runtime.h>
 
 #include "common.hpp"
+#include "tile_map.hpp"
 
 namespace
 {
@@ -107,6 +108,17 @@ namespace
         }
     }
 
+    // fp8 e4m3 at full rate: v_mfma_f32_32x32x64_f8f6f4 takes 32 bytes of K per lane per operand
+    // (two 16-byte pieces here: any K permutation shared by both operands is legal).  Formats
+    // cbsz = blgp = 0 select e4m3 for both operands; the E8M0 block scales are 127 = 2^0.
+    __device__ inline void mfma64Fp8(f32x16& acc, i32x4 x0, i32x4 x1, i32x4 y0, i32x4 y1)
+    {
+        using i32x8 = int __attribute__((ext_vector_type(8)));
+        const i32x8 x = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+        const i32x8 y = {y0[0], y0[1], y0[2], y0[3], y1[0], y1[1], y1[2], y1[3]};
+        acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, acc, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+    }
+
     // ---- LDS swizzles.  A tile is `rows` rows of `rowBytes`; chunk c of row r lives in
     // chunk slot (c ^ swz(r)) of that row.
     //   K-contiguous tile: 256 rows x 128 B (8 slots).   Readers: lane -> row, 8 (or 16)
@@ -126,28 +138,6 @@ namespace
         uint32_t    tilesM, tilesN;
         uint32_t    banks64; // LDS swizzle tuned for 64 banks instead of 32
     };
-
-    // Workgroup id -> (tile row, tile col).  Hardware deals workgroup ids round-robin to the
-    // 8 XCDs; ids with the same (id mod 8) share an L2.  Give each XCD a contiguous run of
-    // tile indices and walk the run in groups of GROUP_M tile rows, column by column, so that
-    // the 32 tiles resident on an XCD at one time cover about 4 x 8 tiles.
-    __device__ inline bool tileCoord(uint32_t bid, uint32_t tilesM, uint32_t tilesN, uint32_t& tm, uint32_t& tn)
-    {
-        constexpr uint32_t XCDS = 8, GROUP_M = 4;
-        const uint32_t     total  = tilesM * tilesN;
-        const uint32_t     perXcd = (total + XCDS - 1) / XCDS;
-        const uint32_t     id     = (bid % XCDS) * perXcd + bid / XCDS;
-        if(id >= total)
-            return false;
-        const uint32_t groupSize = GROUP_M * tilesN;
-        const uint32_t group     = id / groupSize;
-        const uint32_t first     = group * GROUP_M;
-        const uint32_t rowsHere  = (tilesM - first) < GROUP_M ? (tilesM - first) : GROUP_M;
-        const uint32_t inGroup   = id % groupSize;
-        tm                       = first + inGroup % rowsHere;
-        tn                       = inGroup / rowsHere;
-        return true;
-    }
 
     // Scheduling hint for the current region: next come MFMAS matrix instructions, then DSREADS
     // LDS reads, then VMEM global loads.
@@ -179,7 +169,7 @@ namespace
         __shared__ __attribute__((aligned(1024))) char stage1[STAGE_BYTES];
 
         uint32_t tm, tn;
-        if(!tileCoord(blockIdx.x, p.tilesM, p.tilesN, tm, tn))
+        if(!r355::tileCoord(blockIdx.x, p.tilesM, p.tilesN, tm, tn))
             return;
 
         const uint32_t tid   = threadIdx.x;
@@ -299,30 +289,41 @@ namespace
         i32x4 stageRegs[DIRECT ? 1 : 2 * LOADS_PER_OPER];
 
         auto issueGlobal = [&](uint32_t kt, char* stage) {
-            // uniform (scalar) base per load + one 32-bit lane offset per operand
+            // Buffer addressing keeps every per-load term scalar: resource = origin of this stage's
+            // panel (uniform), soffset = j * step (uniform), voffset = the lane's fixed offset.
             const char* srcA = gA + kt * gStageA;
             const char* srcB = gB + kt * gStageB;
-#pragma unroll
-            for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
+            if constexpr(DIRECT)
             {
-                const char* pa = srcA + gOffA;
-                const char* pb = srcB + gOffB;
-                srcA += gStepA;
-                srcB += gStepB;
-                if constexpr(DIRECT)
+                // the panel origins are wave-uniform; say so, or the resource ends up in VGPRs
+                auto uniform = [](const char* ptr) {
+                    const uint64_t v  = reinterpret_cast<uint64_t>(ptr);
+                    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+                    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+                    return reinterpret_cast<char*>((static_cast<uint64_t>(hi) << 32) | lo);
+                };
+                constexpr int RSRC_FLAGS = 0x00020000; // raw buffer, 32-bit data format, no swizzle
+                const __amdgpu_buffer_rsrc_t rsrcA
+                    = __builtin_amdgcn_make_buffer_rsrc(uniform(srcA), 0, 0x7FFFFFFF, RSRC_FLAGS);
+                const __amdgpu_buffer_rsrc_t rsrcB
+                    = __builtin_amdgcn_make_buffer_rsrc(uniform(srcB), 0, 0x7FFFFFFF, RSRC_FLAGS);
+                using lp = __attribute__((address_space(3))) void*;
+#pragma unroll
+                for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
                 {
                     // the memory pipeline writes lane l's 16 bytes at (uniform LDS base + 16 l)
                     char* dstA = stage + (j * THREADS + wave * 64u) * CHUNK;
-                    char* dstB = dstA + OPER_BYTES;
-                    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)pa,
-                                                     (__attribute__((address_space(3))) void*)dstA, 16, 0, 0);
-                    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)pb,
-                                                     (__attribute__((address_space(3))) void*)dstB, 16, 0, 0);
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lp)dstA, 16, gOffA, j * gStepA, 0, 0);
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lp)(dstA + OPER_BYTES), 16, gOffB, j * gStepB, 0, 0);
                 }
-                else
+            }
+            else
+            {
+#pragma unroll
+                for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
                 {
-                    stageRegs[j]                  = *reinterpret_cast<const i32x4*>(pa);
-                    stageRegs[LOADS_PER_OPER + j] = *reinterpret_cast<const i32x4*>(pb);
+                    stageRegs[j]                  = *reinterpret_cast<const i32x4*>(srcA + (uint64_t)j * gStepA + gOffA);
+                    stageRegs[LOADS_PER_OPER + j] = *reinterpret_cast<const i32x4*>(srcB + (uint64_t)j * gStepB + gOffB);
                 }
             }
         };
@@ -340,7 +341,8 @@ namespace
             }
         };
 
-        Acc acc[4][4];
+        Acc            acc[4][4];
+        const uint32_t numStages = p.k / TK;
 #pragma unroll
         for(uint32_t i = 0; i < 4; ++i)
 #pragma unroll
@@ -358,8 +360,21 @@ namespace
                     mfma32<E>(acc[i][j], fb[j], fa[i]);
         };
 
-        const uint32_t numStages = p.k / TK;
-        i32x4          fa[2][4], fb[2][4];
+        // fp8: one matrix instruction spans two 16-byte sub-steps of K
+        constexpr bool     PAIRED = (E == Elem::E4M3);
+        constexpr uint32_t NBUF   = PAIRED ? 4u : 2u;
+        auto mfmaPair = [&](const i32x4 (&fa0)[4], const i32x4 (&fa1)[4], const i32x4 (&fb0)[4], const i32x4 (&fb1)[4]) {
+            if constexpr(PAIRED)
+            {
+#pragma unroll
+                for(uint32_t i = 0; i < 4; ++i)
+#pragma unroll
+                    for(uint32_t j = 0; j < 4; ++j)
+                        mfma64Fp8(acc[i][j], fb0[j], fb1[j], fa0[i], fa1[i]);
+            }
+        };
+
+        i32x4 fa[NBUF][4], fb[NBUF][4];
 
         // One K stage.  `cur` / `nxt` are the LDS buffers of stage kt / kt + 1.
         // Sub-steps 0..2 run against `cur` while the reads for the following sub-step are in
@@ -369,6 +384,49 @@ namespace
         auto stageBody = [&](uint32_t kt, char* cur, char* nxt, auto refill, auto hasNext) {
             constexpr bool REFILL = decltype(refill)::value; // stage kt + 2 exists
             constexpr bool NEXT   = decltype(hasNext)::value; // stage kt + 1 exists
+            if constexpr(PAIRED)
+            {
+                // sub-steps (0, 1) are in registers; fetch (2, 3) under the first 16 instructions
+#pragma unroll
+                for(uint32_t s = 2; s < 4; ++s)
+#pragma unroll
+                    for(uint32_t i = 0; i < 4; ++i)
+                    {
+                        fa[s][i] = readA(cur, i, s);
+                        fb[s][i] = readB(cur, i, s);
+                    }
+                mfmaPair(fa[0], fa[1], fb[0], fb[1]);
+#pragma unroll
+                for(uint32_t g = 0; g < 8; ++g)
+                    schedGroup<1, 2, 0>();
+                schedGroup<8, 0, 0>();
+                if constexpr(DIRECT)
+                    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+                else if constexpr(NEXT)
+                    commitLds(nxt);
+                __syncthreads();
+                if constexpr(REFILL)
+                    issueGlobal(kt + 2, cur);
+                if constexpr(NEXT)
+                {
+#pragma unroll
+                    for(uint32_t s = 0; s < 2; ++s)
+#pragma unroll
+                        for(uint32_t i = 0; i < 4; ++i)
+                        {
+                            fa[s][i] = readA(nxt, i, s);
+                            fb[s][i] = readB(nxt, i, s);
+                        }
+                }
+                mfmaPair(fa[2], fa[3], fb[2], fb[3]);
+#pragma unroll
+                for(uint32_t g = 0; g < 8; ++g)
+                    schedGroup<1, NEXT ? 2u : 0u, REFILL ? 1u : 0u>();
+#pragma unroll
+                for(uint32_t g = 0; g < 8; ++g)
+                    schedGroup<1, 0, REFILL ? 1u : 0u>();
+                return;
+            }
 #pragma unroll
             for(uint32_t s = 0; s < 3; ++s)
             {
@@ -404,10 +462,13 @@ namespace
                 }
             }
             mfmaStep(fa[1], fb[1]);
+            // reads early (their data is needed first), one global load per matrix instruction
 #pragma unroll
             for(uint32_t g = 0; g < 8; ++g)
-                schedGroup<1, NEXT ? READS_PER_SUB / 8u : 0u, REFILL ? 2u : 0u>();
-            schedGroup<8, 0, 0>();
+                schedGroup<1, NEXT ? READS_PER_SUB / 8u : 0u, REFILL ? 1u : 0u>();
+#pragma unroll
+            for(uint32_t g = 0; g < 8; ++g)
+                schedGroup<1, 0, REFILL ? 1u : 0u>();
         };
         constexpr std::true_type  yes{};
         constexpr std::false_type no{};
@@ -426,11 +487,13 @@ namespace
         }
         __syncthreads();
 #pragma unroll
-        for(uint32_t i = 0; i < 4; ++i)
-        {
-            fa[0][i] = readA(stage0, i, 0);
-            fb[0][i] = readB(stage0, i, 0);
-        }
+        for(uint32_t s = 0; s < (PAIRED ? 2u : 1u); ++s)
+#pragma unroll
+            for(uint32_t i = 0; i < 4; ++i)
+            {
+                fa[s][i] = readA(stage0, i, s);
+                fb[s][i] = readB(stage0, i, s);
+            }
 
         // numStages is even (checked on the host): steady state in pairs, last pair peeled
         uint32_t kt = 0;
@@ -448,6 +511,74 @@ namespace
         using OutV = OutT __attribute__((ext_vector_type(4)));
         const AccE     alpha = static_cast<AccE>(p.alpha), beta = static_cast<AccE>(p.beta);
         const uint32_t m0 = tm * TILE_M + wm * 128u, n0 = tn * TILE_N + wn * 128u;
+
+        if(beta == static_cast<AccE>(0))
+        {
+            // The stage buffers are idle now: every wave transposes its 128 x 128 result through its
+            // own 32 KiB of LDS so that a store instruction covers whole 256- or 512-byte rows of D
+            // (128-bit per lane) instead of 8- / 16-byte pieces of 32 different rows.
+            constexpr uint32_t OS         = sizeof(OutT);
+            constexpr uint32_t ROW_BYTES  = 128u * OS; // one row of the wave tile
+            constexpr uint32_t ROW_CHUNKS = ROW_BYTES / CHUNK; // 16 (2-byte) or 32 (4-byte)
+            constexpr uint32_t ROWS_PASS  = 32768u / ROW_BYTES; // 128 or 64 rows per pass
+            constexpr uint32_t BLOCKS_I   = ROWS_PASS / 32u; // 32-row blocks per pass
+            char*              wl         = ((wave < 2u) ? stage0 : stage1) + (wave & 1u) * 32768u;
+            const uint32_t     r32 = lane & 31u, h = lane >> 5;
+#pragma unroll
+            for(uint32_t pass = 0; pass < 4u / BLOCKS_I; ++pass)
+            {
+#pragma unroll
+                for(uint32_t ii = 0; ii < BLOCKS_I; ++ii)
+                {
+                    const uint32_t i   = pass * BLOCKS_I + ii;
+                    const uint32_t row = 32u * ii + r32; // row inside the pass
+#pragma unroll
+                    for(uint32_t j = 0; j < 4; ++j)
+#pragma unroll
+                        for(uint32_t q = 0; q < 4; ++q)
+                        {
+                            OutV out;
+#pragma unroll
+                            for(uint32_t e = 0; e < 4; ++e)
+                                out[e] = static_cast<OutT>(alpha * static_cast<AccE>(acc[i][j][4 * q + e]));
+                            if constexpr(OS == 2)
+                            {
+                                // 8 bytes: chunk 4 j + q, half h; rows 16 apart share a chunk slot, so
+                                // they take opposite halves
+                                const uint32_t c = 4u * j + q;
+                                char* dst = wl + row * ROW_BYTES + ((c ^ (row & 15u)) * CHUNK) + ((h ^ ((row >> 4) & 1u)) * 8u);
+                                *reinterpret_cast<OutV*>(dst) = out;
+                            }
+                            else
+                            {
+                                const uint32_t c = 8u * j + 2u * q + h;
+                                char* dst = wl + row * ROW_BYTES + ((c ^ (row & 31u)) * CHUNK);
+                                *reinterpret_cast<OutV*>(dst) = out;
+                            }
+                        }
+                }
+                __builtin_amdgcn_wave_barrier(); // same wave reads back what it wrote (LDS is in order per wave)
+#pragma unroll
+                for(uint32_t it = 0; it < ROWS_PASS * ROW_CHUNKS / 64u; ++it)
+                {
+                    const uint32_t L = it * 64u + lane, row = L / ROW_CHUNKS, c = L % ROW_CHUNKS;
+                    i32x4          v;
+                    if constexpr(OS == 2)
+                    {
+                        v = *reinterpret_cast<const i32x4*>(wl + row * ROW_BYTES + ((c ^ (row & 15u)) * CHUNK));
+                        if((row >> 4) & 1u)
+                            v = i32x4{v[2], v[3], v[0], v[1]};
+                    }
+                    else
+                        v = *reinterpret_cast<const i32x4*>(wl + row * ROW_BYTES + ((c ^ (row & 31u)) * CHUNK));
+                    const uint64_t offD = (uint64_t)(m0 + pass * ROWS_PASS + row) * p.ldd + n0;
+                    *reinterpret_cast<i32x4*>(p.d + offD * OS + c * CHUNK) = v;
+                }
+                __builtin_amdgcn_wave_barrier();
+            }
+            return;
+        }
+
 #pragma unroll
         for(uint32_t i = 0; i < 4; ++i)
         {
@@ -460,22 +591,13 @@ namespace
                     const uint32_t row  = m0 + 32u * i + (lane & 31u);
                     const uint32_t col  = n0 + 32u * j + 8u * q + 4u * (lane >> 5);
                     const uint64_t offD = (uint64_t)row * p.ldd + col;
+                    const uint64_t offC = (uint64_t)row * p.ldc + col;
+                    const OutV     cv   = *reinterpret_cast<const OutV*>(p.c + offC * sizeof(OutT));
                     OutV           out;
-                    if(beta != static_cast<AccE>(0))
-                    {
-                        const uint64_t offC = (uint64_t)row * p.ldc + col;
-                        const OutV     cv   = *reinterpret_cast<const OutV*>(p.c + offC * sizeof(OutT));
 #pragma unroll
-                        for(uint32_t e = 0; e < 4; ++e)
-                            out[e] = static_cast<OutT>(alpha * static_cast<AccE>(acc[i][j][4 * q + e])
-                                                       + beta * static_cast<AccE>(cv[e]));
-                    }
-                    else
-                    {
-#pragma unroll
-                        for(uint32_t e = 0; e < 4; ++e)
-                            out[e] = static_cast<OutT>(alpha * static_cast<AccE>(acc[i][j][4 * q + e]));
-                    }
+                    for(uint32_t e = 0; e < 4; ++e)
+                        out[e] = static_cast<OutT>(alpha * static_cast<AccE>(acc[i][j][4 * q + e])
+                                                   + beta * static_cast<AccE>(cv[e]));
                     *reinterpret_cast<OutV*>(p.d + offD * sizeof(OutT)) = out;
                 }
             }
@@ -554,9 +676,9 @@ namespace r355
         const uint32_t tk = STAGE_KB / es;
         if(g.m % TILE_M || g.n % TILE_N || g.k % (2 * tk) || g.k == 0)
             return fail(R355_ERR_BAD_SIZE, "tiled gemm: m=%u n=%u must be multiples of 256 and k=%u of %u", g.m, g.n, g.k, 2 * tk);
-        if(!aligned(g.a, 16) || !aligned(g.b, 16) || (g.lda * es) % 16 || (g.ldb * es) % 16 || !aligned(g.d, 4 * os)
-           || (g.ldd * os) % (4 * os) || (g.beta != 0.0f && (!aligned(g.c, 4 * os) || (g.ldc * os) % (4 * os))))
-            return fail(R355_ERR_MISALIGNED, "tiled gemm: A/B need 16-byte, C/D 4-element alignment of pointers and leading dimensions");
+        if(!aligned(g.a, 16) || !aligned(g.b, 16) || (g.lda * es) % 16 || (g.ldb * es) % 16 || !aligned(g.d, 16)
+           || (g.ldd * os) % 16 || (g.beta != 0.0f && (!aligned(g.c, 16) || (g.ldc * os) % 16)))
+            return fail(R355_ERR_MISALIGNED, "tiled gemm: pointers and leading dimensions of A, B, C, D must keep 16-byte alignment");
         if(plan)
         {
             plan->kernel       = R355_KERNEL_TILED;

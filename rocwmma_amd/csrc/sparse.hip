@@ -8,15 +8,21 @@
 //                     register one lane feeds to v_smfmac_*_32x32x64 for its 16 kept values.
 // B is dense, col-major (k contiguous); D row- or col-major.
 //
-// Kernel: one 32 x 32 block of D per wave, operands streamed from global memory
-// (lane = row / column, 16 kept bytes + 4 index bytes of A and 2 x 16 dense bytes of B per
-// 64-wide K step).  Operand formats of v_smfmac_*_32x32x64 as measured on MI355X: index
+// Two kernels:
+//   sparseTiledKernel    256 x 256 macro tile, 128 dense K per stage, double-buffered LDS filled
+//                        by direct-to-LDS loads (kept values 16 KiB + indices 4 KiB + dense B
+//                        32 KiB per stage), 2 x 2 waves with 4 x 4 v_smfmac_*_32x32x64 accumulators
+//                        each; the result is transposed through LDS so that D leaves in whole rows.
+//   sparseBlockPerWave   one 32 x 32 block of D per wave straight from global memory; fallback
+//                        for shapes that do not fill a macro tile.
+// Per 64-wide K step a lane feeds 16 kept bytes + 4 index bytes of A and 2 x 16 dense bytes of B.  Operand formats of v_smfmac_*_32x32x64 as measured on MI355X: index
 // bits [2 p + 1 : 2 p] give the position within its group of 4 of kept byte p of the lane.
 #include <hip/hip_runtime.h>
 
 #include <cstring>
 
 #include "common.hpp"
+#include "tile_map.hpp"
 
 namespace
 {
@@ -93,6 +99,250 @@ namespace
             static_cast<AccE*>(d)[dRow ? (uint64_t)r * ldd + cc : (uint64_t)cc * ldd + r] = v;
         }
     }
+
+    // ------------------------------------------------------------------ macro-tile kernel
+    constexpr uint32_t T_M = 256, T_N = 256, T_K = 128; // dense K per stage
+    constexpr uint32_t T_THREADS   = 256;
+    constexpr uint32_t A_BYTES     = T_M * (T_K / 2); // 16 KiB kept values
+    constexpr uint32_t META_BYTES  = T_M * (T_K / 8); // 4 KiB indices
+    constexpr uint32_t B_BYTES     = T_N * T_K; // 32 KiB dense
+    constexpr uint32_t OFF_META    = A_BYTES;
+    constexpr uint32_t OFF_B       = A_BYTES + META_BYTES;
+    constexpr uint32_t STAGE_BYTES = A_BYTES + META_BYTES + B_BYTES; // 52 KiB
+
+    struct TiledParams
+    {
+        uint32_t       m, n, k;
+        const uint8_t* aVals;
+        const uint8_t* aMeta;
+        const uint8_t* b;
+        const char*    c;
+        char*          d;
+        uint32_t       lda, ldb, ldc, ldd;
+        float          alpha, beta;
+        uint32_t       tilesM, tilesN;
+        uint32_t       dRow; // D (and C) row-major
+    };
+
+    template <bool FP8>
+    __global__ void __launch_bounds__(T_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
+        sparseTiledKernel(TiledParams p)
+    {
+        using Acc  = std::conditional_t<FP8, f32x16, i32x16>;
+        using AccE = std::conditional_t<FP8, float, int>;
+
+        __shared__ __attribute__((aligned(1024))) char stage0[STAGE_BYTES];
+        __shared__ __attribute__((aligned(1024))) char stage1[STAGE_BYTES];
+
+        uint32_t tm, tn;
+        if(!r355::tileCoord(blockIdx.x, p.tilesM, p.tilesN, tm, tn))
+            return;
+
+        const uint32_t tid  = threadIdx.x;
+        const uint32_t lane = tid & 63u;
+        const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const uint32_t wm = wave >> 1, wn = wave & 1u;
+        const uint32_t r32 = lane & 31u, g = lane >> 5;
+
+        // ---- global -> LDS (per thread, fixed).  LDS chunk L = j * 256 + tid of each operand tile.
+        //   kept values: 4 chunks per row, chunk c of row r in slot c ^ ((r >> 2) & 3)
+        //   dense B:     8 chunks per row, chunk c of row r in slot c ^ ((r >> 1) & 7)
+        //   indices:     one 16-byte chunk per row, thread t <-> row t
+        const uint32_t rowA = tid >> 2, slotA = tid & 3u;
+        const uint32_t gOffA = rowA * p.lda + ((slotA ^ ((rowA >> 2) & 3u)) * 16u);
+        const uint32_t rowB = tid >> 3, slotB = tid & 7u;
+        const uint32_t gOffB = rowB * p.ldb + ((slotB ^ ((rowB >> 1) & 7u)) * 16u);
+        const uint32_t gOffM = tid * (p.k / 8u);
+        const uint8_t* gA = p.aVals + (uint64_t)tm * T_M * p.lda;
+        const uint8_t* gM = p.aMeta + (uint64_t)tm * T_M * (p.k / 8u);
+        const uint8_t* gB = p.b + (uint64_t)tn * T_N * p.ldb;
+
+        auto issueGlobal = [&](uint32_t kt, char* stage) {
+            using gp = const __attribute__((address_space(1))) void*;
+            using lp = __attribute__((address_space(3))) void*;
+            const uint8_t* srcA = gA + kt * (T_K / 2u);
+            const uint8_t* srcB = gB + kt * T_K;
+            char* dst = stage + wave * 1024u; // lane l lands at dst + 16 l
+#pragma unroll
+            for(uint32_t j = 0; j < 4; ++j) // 64 rows of kept values per j
+                __builtin_amdgcn_global_load_lds((gp)(srcA + (uint64_t)j * 64u * p.lda + gOffA), (lp)(dst + j * 4096u), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gp)(gM + kt * (T_K / 8u) + gOffM), (lp)(dst + OFF_META), 16, 0, 0);
+#pragma unroll
+            for(uint32_t j = 0; j < 8; ++j) // 32 rows of B per j
+                __builtin_amdgcn_global_load_lds((gp)(srcB + (uint64_t)j * 32u * p.ldb + gOffB), (lp)(dst + OFF_B + j * 4096u), 16, 0, 0);
+        };
+
+        // ---- LDS -> registers (per lane, fixed)
+        const uint32_t rA   = wm * 128u + r32, rB = wn * 128u + r32;
+        const uint32_t swA  = (r32 >> 2) & 3u, swB = (r32 >> 1) & 7u;
+        uint32_t       rdA[2], rdB[4];
+#pragma unroll
+        for(uint32_t q = 0; q < 2; ++q) // K group q: kept-value chunk 2 q + g
+            rdA[q] = rA * 64u + (((2u * q + g) ^ swA) * 16u);
+        const uint32_t rdM = OFF_META + rA * 16u + 4u * g; // + 8 q
+#pragma unroll
+        for(uint32_t s = 0; s < 4; ++s) // K group q uses dense chunks 4 q + g and 4 q + 2 + g
+            rdB[s] = OFF_B + rB * 128u + (((2u * s + g) ^ swB) * 16u);
+
+        struct Frags
+        {
+            i32x4 a[4];
+            int   idx[4];
+            i32x4 b0[4], b1[4];
+        };
+        auto readGroup = [&](Frags& f, const char* base, uint32_t q) {
+#pragma unroll
+            for(uint32_t i = 0; i < 4; ++i)
+            {
+                f.a[i]   = *reinterpret_cast<const i32x4*>(base + rdA[q] + i * 32u * 64u);
+                f.idx[i] = *reinterpret_cast<const int*>(base + rdM + 8u * q + i * 32u * 16u);
+                f.b0[i]  = *reinterpret_cast<const i32x4*>(base + rdB[2u * q] + i * 32u * 128u);
+                f.b1[i]  = *reinterpret_cast<const i32x4*>(base + rdB[2u * q + 1u] + i * 32u * 128u);
+            }
+        };
+
+        Acc acc[4][4];
+#pragma unroll
+        for(uint32_t i = 0; i < 4; ++i)
+#pragma unroll
+            for(uint32_t j = 0; j < 4; ++j)
+#pragma unroll
+                for(uint32_t e = 0; e < 16; ++e)
+                    acc[i][j][e] = 0;
+
+        auto mfmaGroup = [&](const Frags& f) {
+#pragma unroll
+            for(uint32_t i = 0; i < 4; ++i)
+#pragma unroll
+                for(uint32_t j = 0; j < 4; ++j)
+                {
+                    const i32x8 bv = {f.b0[j][0], f.b0[j][1], f.b0[j][2], f.b0[j][3],
+                                      f.b1[j][0], f.b1[j][1], f.b1[j][2], f.b1[j][3]};
+                    if constexpr(FP8)
+                        acc[i][j] = __builtin_amdgcn_smfmac_f32_32x32x64_fp8_fp8(f.a[i], bv, acc[i][j], f.idx[i], 0, 0);
+                    else
+                        acc[i][j] = __builtin_amdgcn_smfmac_i32_32x32x64_i8(f.a[i], bv, acc[i][j], f.idx[i], 0, 0);
+                }
+        };
+        auto hint = [&](bool reads, bool loads) {
+            // 16 LDS reads (4 values + 4 indices + 8 dense) and 13 global loads per 16 matrix instructions
+#pragma unroll
+            for(uint32_t x = 0; x < 8; ++x)
+            {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if(reads)
+                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                if(loads)
+                    __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+        };
+
+        Frags f0, f1;
+        auto  stageBody = [&](uint32_t kt, char* cur, char* nxt, auto refill, auto hasNext) {
+            constexpr bool REFILL = decltype(refill)::value, NEXT = decltype(hasNext)::value;
+            readGroup(f1, cur, 1);
+            mfmaGroup(f0);
+            hint(true, false);
+            __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): own direct loads of stage kt + 1 have landed
+            __syncthreads();
+            if constexpr(REFILL)
+                issueGlobal(kt + 2, cur);
+            if constexpr(NEXT)
+                readGroup(f0, nxt, 0);
+            mfmaGroup(f1);
+            hint(NEXT, REFILL);
+        };
+        constexpr std::true_type  yes{};
+        constexpr std::false_type no{};
+
+        const uint32_t numStages = p.k / T_K; // even, >= 2 (checked on the host)
+        issueGlobal(0, stage0);
+        issueGlobal(1, stage1);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+        readGroup(f0, stage0, 0);
+        uint32_t kt = 0;
+        for(; kt + 2 < numStages; kt += 2)
+        {
+            stageBody(kt, stage0, stage1, yes, yes);
+            stageBody(kt + 1, stage1, stage0, yes, yes);
+        }
+        stageBody(kt, stage0, stage1, no, yes);
+        stageBody(kt + 1, stage1, stage0, no, no);
+
+        // ---- epilogue.  lane holds D(m = 8 (e / 4) + 4 g + e % 4, n = lane % 32) of each block:
+        // four consecutive rows of one column.
+        const AccE     alpha = static_cast<AccE>(p.alpha), beta = static_cast<AccE>(p.beta);
+        const uint32_t m0 = tm * T_M + wm * 128u, n0 = tn * T_N + wn * 128u;
+        using V4 = AccE __attribute__((ext_vector_type(4)));
+        if(!p.dRow)
+        {
+            // col-major: a lane's four rows are contiguous
+#pragma unroll
+            for(uint32_t i = 0; i < 4; ++i)
+#pragma unroll
+                for(uint32_t j = 0; j < 4; ++j)
+#pragma unroll
+                    for(uint32_t q = 0; q < 4; ++q)
+                    {
+                        const uint32_t row = m0 + 32u * i + 8u * q + 4u * g, col = n0 + 32u * j + r32;
+                        V4             out;
+#pragma unroll
+                        for(uint32_t e = 0; e < 4; ++e)
+                            out[e] = alpha * acc[i][j][4 * q + e];
+                        if(beta != static_cast<AccE>(0))
+                        {
+                            const V4 cv = *reinterpret_cast<const V4*>(p.c + ((uint64_t)col * p.ldc + row) * 4u);
+#pragma unroll
+                            for(uint32_t e = 0; e < 4; ++e)
+                                out[e] += beta * cv[e];
+                        }
+                        *reinterpret_cast<V4*>(p.d + ((uint64_t)col * p.ldd + row) * 4u) = out;
+                    }
+            return;
+        }
+        // row-major: transpose through this wave's 26 KiB of the idle stage buffers, 32 rows (one
+        // block row i) at a time: rows of 128 x 4 bytes = 32 chunks, chunk c of row r in slot c ^ r.
+        char* wl = ((wave < 2u) ? stage0 : stage1) + (wave & 1u) * 26624u;
+#pragma unroll
+        for(uint32_t i = 0; i < 4; ++i)
+        {
+#pragma unroll
+            for(uint32_t j = 0; j < 4; ++j)
+#pragma unroll
+                for(uint32_t e = 0; e < 16; ++e)
+                {
+                    const uint32_t row = 8u * (e >> 2) + 4u * g + (e & 3u), col = 32u * j + r32;
+                    *reinterpret_cast<AccE*>(wl + row * 512u + (((col >> 2) ^ row) * 16u) + (col & 3u) * 4u)
+                        = alpha * acc[i][j][e];
+                }
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for(uint32_t it = 0; it < 16; ++it)
+            {
+                const uint32_t L = it * 64u + lane, row = L >> 5, c = L & 31u;
+                V4             v = *reinterpret_cast<const V4*>(wl + row * 512u + ((c ^ row) * 16u));
+                const uint64_t off = (uint64_t)(m0 + 32u * i + row);
+                if(beta != static_cast<AccE>(0))
+                {
+                    const V4 cv = *reinterpret_cast<const V4*>(p.c + (off * p.ldc + n0) * 4u + c * 16u);
+#pragma unroll
+                    for(uint32_t e = 0; e < 4; ++e)
+                        v[e] += beta * cv[e];
+                }
+                *reinterpret_cast<V4*>(p.d + (off * p.ldd + n0) * 4u + c * 16u) = v;
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
+
+    bool tiledOk(const r355_gemm_args& g)
+    {
+        return g.kernel != R355_KERNEL_SIMPLE && g.m % T_M == 0 && g.n % T_N == 0 && g.k % (2 * T_K) == 0
+               && g.layout_c == g.layout_d && (g.ldd % 4) == 0 && r355::aligned(g.d, 16)
+               && (g.beta == 0.0f || ((g.ldc % 4) == 0 && r355::aligned(g.c, 16))) && r355::aligned(g.a_meta, 16);
+    }
 } // namespace
 
 namespace r355
@@ -111,7 +361,21 @@ namespace r355
             return fail(R355_ERR_BAD_SIZE, "sparse gemm: m=%u n=%u must be multiples of 32 and k=%u of 64", g.m, g.n, g.k);
         if(!aligned(g.a, 16) || g.lda % 16 || !aligned(g.b, 16) || g.ldb % 16 || !aligned(g.a_meta, 4) || !aligned(g.d, 4))
             return fail(R355_ERR_MISALIGNED, "sparse gemm: values / B need 16-byte alignment, metadata 4-byte");
-        if(plan)
+        if(g.kernel == R355_KERNEL_TILED && !tiledOk(g))
+            return fail(R355_ERR_BAD_SIZE, "sparse gemm (macro tile): m=%u n=%u must be multiples of 256, k=%u of 256, C/D same orientation and 16-byte aligned", g.m, g.n, g.k);
+        if(plan && tiledOk(g))
+        {
+            plan->kernel       = R355_KERNEL_TILED;
+            plan->macro_tile_m = T_M;
+            plan->macro_tile_n = T_N;
+            plan->macro_tile_k = T_K;
+            plan->grid_x       = (((g.m / T_M) * (g.n / T_N) + 7u) / 8u) * 8u;
+            plan->grid_y       = 1;
+            plan->block_x      = T_THREADS;
+            plan->block_y      = 1;
+            plan->lds_bytes    = 2 * STAGE_BYTES;
+        }
+        else if(plan)
         {
             plan->kernel       = R355_KERNEL_SIMPLE;
             plan->macro_tile_m = 32 * WAVES_X;
@@ -128,6 +392,24 @@ namespace r355
 
     int gemmSparseLaunch(const r355_gemm_args& g, hipStream_t stream)
     {
+        if(tiledOk(g))
+        {
+            TiledParams p;
+            p.m = g.m, p.n = g.n, p.k = g.k;
+            p.aVals = static_cast<const uint8_t*>(g.a), p.aMeta = static_cast<const uint8_t*>(g.a_meta);
+            p.b = static_cast<const uint8_t*>(g.b);
+            p.c = static_cast<const char*>(g.c), p.d = static_cast<char*>(g.d);
+            p.lda = g.lda, p.ldb = g.ldb, p.ldc = g.ldc, p.ldd = g.ldd;
+            p.alpha = g.alpha, p.beta = g.beta;
+            p.tilesM = g.m / T_M, p.tilesN = g.n / T_N;
+            p.dRow = g.layout_d == R355_ROW_MAJOR;
+            const uint32_t grid = ((p.tilesM * p.tilesN + 7u) / 8u) * 8u;
+            if(g.in_type == R355_E4M3)
+                hipLaunchKernelGGL(sparseTiledKernel<true>, dim3(grid), dim3(T_THREADS), 0, stream, p);
+            else
+                hipLaunchKernelGGL(sparseTiledKernel<false>, dim3(grid), dim3(T_THREADS), 0, stream, p);
+            return checkLaunch("sparse gemm (macro tile)");
+        }
         dim3 block(WAVES_X * 64, WAVES_Y);
         dim3 grid((g.m + 32 * WAVES_X - 1) / (32 * WAVES_X), (g.n + 32 * WAVES_Y - 1) / (32 * WAVES_Y));
         auto* av = static_cast<const uint8_t*>(g.a);
