@@ -17,7 +17,8 @@
 //                row-contiguous writes and the MFMA-shaped reads are bank-conflict free
 //   LDS->regs    K-contiguous operands: one ds_read_b128 per 32x(16|32) operand block;
 //                M/N-contiguous 16-bit operands: two ds_read_b64_tr_b16 (transposing
-//                read) -- no element-wise reads anywhere
+//                read) -- no element-wise reads anywhere; operands are fetched two
+//                matrix-instruction K steps (32 instructions) ahead of their use
 //   grid         1-D, remapped so that each XCD (workgroup id mod 8) owns a compact
 //                rectangle of tiles and walks it in 4-row groups (L2 reuse of A and B)
 //
@@ -362,7 +363,7 @@ namespace
 
         // fp8: one matrix instruction spans two 16-byte sub-steps of K
         constexpr bool     PAIRED = (E == Elem::E4M3);
-        constexpr uint32_t NBUF   = PAIRED ? 4u : 2u;
+        constexpr uint32_t NBUF   = 4u;
         auto mfmaPair = [&](const i32x4 (&fa0)[4], const i32x4 (&fa1)[4], const i32x4 (&fb0)[4], const i32x4 (&fb1)[4]) {
             if constexpr(PAIRED)
             {
@@ -376,11 +377,12 @@ namespace
 
         i32x4 fa[NBUF][4], fb[NBUF][4];
 
-        // One K stage.  `cur` / `nxt` are the LDS buffers of stage kt / kt + 1.
-        // Sub-steps 0..2 run against `cur` while the reads for the following sub-step are in
-        // flight; before sub-step 3 every wave has all its operands of `cur` in registers, so
-        // after the barrier `cur` is refilled with stage kt + 2 and the first operands of
-        // stage kt + 1 are fetched from `nxt` underneath the last 16 matrix instructions.
+        // One K stage.  `cur` / `nxt` are the LDS buffers of stage kt / kt + 1.  Operand registers
+        // are indexed by sub-step and fetched two sub-steps ahead (LDS is shared by four waves and
+        // the direct loads, so a read can take several hundred cycles): during sub-steps 0 and 1
+        // the operands of sub-steps 2 and 3 arrive; then every wave holds the rest of `cur` in
+        // registers, so after the barrier `cur` is refilled with stage kt + 2 and the operands of
+        // sub-steps 0 and 1 of stage kt + 1 are fetched from `nxt` underneath sub-steps 2 and 3.
         auto stageBody = [&](uint32_t kt, char* cur, char* nxt, auto refill, auto hasNext) {
             constexpr bool REFILL = decltype(refill)::value; // stage kt + 2 exists
             constexpr bool NEXT   = decltype(hasNext)::value; // stage kt + 1 exists
@@ -428,47 +430,49 @@ namespace
                 return;
             }
 #pragma unroll
-            for(uint32_t s = 0; s < 3; ++s)
+            for(uint32_t s = 0; s < 2; ++s)
             {
 #pragma unroll
                 for(uint32_t i = 0; i < 4; ++i)
                 {
-                    fa[(s + 1) & 1][i] = readA(cur, i, s + 1);
-                    fb[(s + 1) & 1][i] = readB(cur, i, s + 1);
+                    fa[s + 2][i] = readA(cur, i, s + 2);
+                    fb[s + 2][i] = readB(cur, i, s + 2);
                 }
-                mfmaStep(fa[s & 1], fb[s & 1]);
-                // LDS reads early in the sub-step, matrix instructions throughout
+                mfmaStep(fa[s], fb[s]);
 #pragma unroll
                 for(uint32_t g = 0; g < 8; ++g)
-                    schedGroup<1, READS_PER_SUB / 8u, 0>();
-                schedGroup<8, 0, 0>();
+                {
+                    schedGroup<1, READS_PER_SUB / 8u - READS_PER_SUB / 16u, 0>();
+                    schedGroup<1, READS_PER_SUB / 16u, 0>();
+                }
             }
             if constexpr(!DIRECT && NEXT)
                 commitLds(nxt);
-            // Direct-to-LDS loads are tracked by vmcnt of the issuing wave only: every wave must
-            // see its own loads of stage kt + 1 land before the barrier publishes them to the others.
             if constexpr(DIRECT)
                 __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
-            __syncthreads(); // also waits for this wave's LDS reads of `cur`
+            __syncthreads();
             if constexpr(REFILL)
                 issueGlobal(kt + 2, cur);
-            if constexpr(NEXT)
+#pragma unroll
+            for(uint32_t s = 2; s < 4; ++s)
             {
-#pragma unroll
-                for(uint32_t i = 0; i < 4; ++i)
+                if constexpr(NEXT)
                 {
-                    fa[0][i] = readA(nxt, i, 0);
-                    fb[0][i] = readB(nxt, i, 0);
+#pragma unroll
+                    for(uint32_t i = 0; i < 4; ++i)
+                    {
+                        fa[s - 2][i] = readA(nxt, i, s - 2);
+                        fb[s - 2][i] = readB(nxt, i, s - 2);
+                    }
                 }
+                mfmaStep(fa[s], fb[s]);
             }
-            mfmaStep(fa[1], fb[1]);
-            // reads early (their data is needed first), one global load per matrix instruction
 #pragma unroll
-            for(uint32_t g = 0; g < 8; ++g)
-                schedGroup<1, NEXT ? READS_PER_SUB / 8u : 0u, REFILL ? 1u : 0u>();
-#pragma unroll
-            for(uint32_t g = 0; g < 8; ++g)
-                schedGroup<1, 0, REFILL ? 1u : 0u>();
+            for(uint32_t g = 0; g < 16; ++g)
+            {
+                schedGroup<1, NEXT ? READS_PER_SUB / 8u - READS_PER_SUB / 16u : 0u, REFILL ? 1u : 0u>();
+                schedGroup<1, NEXT ? READS_PER_SUB / 16u : 0u, 0>();
+            }
         };
         constexpr std::true_type  yes{};
         constexpr std::false_type no{};
@@ -487,7 +491,7 @@ namespace
         }
         __syncthreads();
 #pragma unroll
-        for(uint32_t s = 0; s < (PAIRED ? 2u : 1u); ++s)
+        for(uint32_t s = 0; s < 2u; ++s)
 #pragma unroll
             for(uint32_t i = 0; i < 4; ++i)
             {
