@@ -8,10 +8,11 @@
 //
 //   * one wave owns one sample at a time; a workgroup (4 waves) owns 8 consecutive samples,
 //     whose outputs form one contiguous, 16-byte aligned run of 8 * (k + m(m-1)/2) elements;
-//   * X (m x k, m <= 32) is read once with fully coalesced 128-bit loads, parked in LDS with
-//     a per-row XOR swizzle, and fed to v_mfma_f32_32x32x16 with the same register as both
-//     operands (X X^T): k / 16 matrix instructions, one 128-bit LDS read each; rows >= m are
-//     kept zero in LDS, which is the 27 -> 32 padding;
+//   * X (m x k, m <= 32) is read once with fully coalesced 128-bit loads (both samples of a
+//     wave are requested before either is consumed), parked in LDS with a per-row XOR swizzle,
+//     and fed to v_mfma_f32_32x32x16 with the same register as both operands (X X^T): k / 16
+//     matrix instructions, one 128-bit LDS read each; lanes of rows >= m feed zeros, which is
+//     the 27 -> 32 padding;
 //   * the strict lower triangle and the copied first row are assembled in an LDS image of
 //     the output and leave with coalesced 128-bit stores.  No global scratch.
 //
@@ -56,13 +57,15 @@ namespace
     }
 
     // K is a template parameter (32, 64, 128, 256): rows of X are K * 2 bytes = K / 8 chunks.
-    template <bool BF16, uint32_t K>
+    // ROWS (28 or 32) bounds m: the LDS image of a sample holds ROWS rows, which at m <= 28 and
+    // K = 128 lets four workgroups share a CU instead of three.
+    template <bool BF16, uint32_t K, uint32_t ROWS>
     __global__ void __launch_bounds__(THREADS)
         dlrmFwdKernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out, uint32_t m, uint32_t batch)
     {
         constexpr uint32_t ROW_CHUNKS = K / 8; // 16-byte chunks per row
-        constexpr uint32_t X_BYTES    = MAX_M * K * 2; // LDS image of one padded sample
-        constexpr uint32_t MAX_OUT    = K + MAX_M * (MAX_M - 1) / 2;
+        constexpr uint32_t X_BYTES    = ROWS * K * 2; // LDS image of one sample
+        constexpr uint32_t MAX_OUT    = K + ROWS * (ROWS - 1) / 2;
 
         __shared__ __attribute__((aligned(16))) char     xLds[WAVES][X_BYTES];
         __shared__ __attribute__((aligned(16))) uint16_t outLds[SAMPLES_PER_WG * MAX_OUT + 8];
@@ -75,14 +78,12 @@ namespace
         const uint32_t inChunks  = m * ROW_CHUNKS; // 16-byte chunks of one sample
 
         char* xw = xLds[wave];
-        // rows m..31 stay zero for the whole kernel: the padding rows of the 32 x 32 product
-        for(uint32_t c = inChunks + lane; c < MAX_M * ROW_CHUNKS; c += 64)
-            *reinterpret_cast<i32x4*>(xw + c * 16u) = i32x4{0, 0, 0, 0};
+        // rows m..31 of the 32 x 32 product are padding: their lanes feed zeros (see below)
 
         // Both samples of this wave are requested from HBM before either is consumed: the kernel is
         // bandwidth-bound, and bytes in flight per CU are what keeps HBM busy.
         constexpr uint32_t PER_WAVE   = SAMPLES_PER_WG / WAVES; // 2
-        constexpr uint32_t MAX_CHUNKS = (MAX_M * ROW_CHUNKS + 63u) / 64u; // loads per lane per sample
+        constexpr uint32_t MAX_CHUNKS = (ROWS * ROW_CHUNKS + 63u) / 64u; // loads per lane per sample
         i32x4              stash[PER_WAVE][MAX_CHUNKS];
 #pragma unroll
         for(uint32_t q = 0; q < PER_WAVE; ++q)
@@ -124,15 +125,18 @@ namespace
             __builtin_amdgcn_wave_barrier();
 
             // ---- Gram matrix: acc(i, j) = sum_k X(i, k) X(j, k)
-            f32x16         acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-            const uint32_t row = lane & 31u;
+            f32x16         acc   = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            const bool     valid = (lane & 31u) < m;
+            const uint32_t row   = valid ? (lane & 31u) : 0u; // padding lanes read row 0 and discard it
 #pragma unroll
             for(uint32_t s = 0; s < K / 16; ++s)
             {
                 const uint32_t col  = 2u * s + (lane >> 5);
                 const uint32_t slot = col ^ (row & (ROW_CHUNKS - 1u) & 15u);
-                const i32x4    x    = *reinterpret_cast<const i32x4*>(xw + (row * ROW_CHUNKS + slot) * 16u);
-                acc                 = mfma16<BF16>(acc, x, x);
+                i32x4          x    = *reinterpret_cast<const i32x4*>(xw + (row * ROW_CHUNKS + slot) * 16u);
+                if(!valid)
+                    x = i32x4{0, 0, 0, 0};
+                acc = mfma16<BF16>(acc, x, x);
             }
 
             // ---- output image: first row, then strict lower triangle (i, j < i) row-major
@@ -283,7 +287,14 @@ extern "C" int r355_dlrm_fwd(int32_t dtype, const void* in, void* out, uint32_t 
     hipStream_t s  = static_cast<hipStream_t>(stream);
     auto*       pi = static_cast<const uint16_t*>(in);
     auto*       po = static_cast<uint16_t*>(out);
-#define R355_FWD(BF, KK) hipLaunchKernelGGL((dlrmFwdKernel<BF, KK>), grid, block, 0, s, pi, po, m, batch)
+#define R355_FWD(BF, KK)                                                                         \
+    do                                                                                            \
+    {                                                                                             \
+        if(m <= 28)                                                                               \
+            hipLaunchKernelGGL((dlrmFwdKernel<BF, KK, 28>), grid, block, 0, s, pi, po, m, batch); \
+        else                                                                                      \
+            hipLaunchKernelGGL((dlrmFwdKernel<BF, KK, 32>), grid, block, 0, s, pi, po, m, batch); \
+    } while(0)
 #define R355_FWD_K(BF)   \
     switch(k)            \
     {                    \

@@ -5,8 +5,8 @@
 // Takes the place of samples/simple_sgemv.cpp:103-150, which feeds 16x16x16 f32 fragments
 // (the B fragment being x broadcast 16 times) to the matrix core.  At 0.5 flop per byte
 // the matrix core contributes nothing; the kernel is organised for memory bandwidth.
-//   col-major A (the sample's layout): a workgroup owns 256 * 4 rows; lane t holds rows
-//     4 t .. 4 t + 3 and walks k, one 128-bit load per column.
+//   col-major A (the sample's layout): a workgroup owns 64 (or 256) rows; its 16 waves split
+//     the columns and combine their partial sums through LDS in a fixed order.
 //   row-major A: one wave per row, lanes stride k in float4, then a wave reduction.
 #include <hip/hip_runtime.h>
 
@@ -18,39 +18,60 @@ namespace
 
     constexpr uint32_t THREADS = 256;
 
-    __global__ void __launch_bounds__(THREADS) gemvColMajor(uint32_t     m,
-                                                           uint32_t     k,
-                                                           const float* a,
-                                                           uint32_t     lda,
-                                                           const float* x,
-                                                           const float* yIn,
-                                                           float*       yOut,
-                                                           float        alpha,
-                                                           float        beta,
-                                                           uint32_t     kSplit)
+    // col-major A (m contiguous): a wave reads V * 64 consecutive rows of one column per load;
+    // the 16 waves of a workgroup split the columns and their partial sums meet in LDS in a fixed
+    // order, so the result does not depend on scheduling.
+    constexpr uint32_t COL_WAVES = 16;
+
+    template <uint32_t V>
+    __global__ void __launch_bounds__(COL_WAVES * 64) gemvColMajor(uint32_t     m,
+                                                                  uint32_t     k,
+                                                                  const float* a,
+                                                                  uint32_t     lda,
+                                                                  const float* x,
+                                                                  const float* yIn,
+                                                                  float*       yOut,
+                                                                  float        alpha,
+                                                                  float        beta)
     {
-        // grid.x: row blocks of 1024 rows; each thread 4 rows; all of k per thread
-        const uint32_t r0 = (blockIdx.x * THREADS + threadIdx.x) * 4u;
-        if(r0 >= m)
-            return;
-        f32x4        acc = {0, 0, 0, 0};
-        const float* p   = a + r0;
-#pragma unroll 8
-        for(uint32_t kk = 0; kk < k; ++kk)
-        {
-            const f32x4 v  = *reinterpret_cast<const f32x4*>(p + (uint64_t)kk * lda);
-            const float xv = x[kk];
-            acc[0] += v[0] * xv;
-            acc[1] += v[1] * xv;
-            acc[2] += v[2] * xv;
-            acc[3] += v[3] * xv;
-        }
-        (void)kSplit;
-        f32x4 out;
+        using VecT = float __attribute__((ext_vector_type(V)));
+        __shared__ float partial[COL_WAVES][64 * V];
+        const uint32_t   lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+        const uint32_t   r0   = (blockIdx.x * 64u + lane) * V;
+        VecT             acc;
 #pragma unroll
-        for(uint32_t e = 0; e < 4; ++e)
-            out[e] = beta != 0.0f ? alpha * acc[e] + beta * yIn[r0 + e] : alpha * acc[e];
-        *reinterpret_cast<f32x4*>(yOut + r0) = out;
+        for(uint32_t e = 0; e < V; ++e)
+            acc[e] = 0.0f;
+        if(r0 < m)
+        {
+            const float* p = a + r0;
+#pragma unroll 8
+            for(uint32_t kk = wave; kk < k; kk += COL_WAVES)
+            {
+                const VecT  v  = *reinterpret_cast<const VecT*>(p + (uint64_t)kk * lda);
+                const float xv = x[kk];
+#pragma unroll
+                for(uint32_t e = 0; e < V; ++e)
+                    acc[e] += v[e] * xv;
+            }
+        }
+#pragma unroll
+        for(uint32_t e = 0; e < V; ++e)
+            partial[wave][lane * V + e] = acc[e];
+        __syncthreads();
+        // 64 * V rows, summed over the waves in wave order
+        for(uint32_t r = threadIdx.x; r < 64u * V; r += COL_WAVES * 64u)
+        {
+            const uint32_t row = blockIdx.x * 64u * V + r;
+            if(row < m)
+            {
+                float sum = 0.0f;
+#pragma unroll
+                for(uint32_t w = 0; w < COL_WAVES; ++w)
+                    sum += partial[w][r];
+                yOut[row] = beta != 0.0f ? alpha * sum + beta * yIn[row] : alpha * sum;
+            }
+        }
     }
 
     __global__ void __launch_bounds__(THREADS) gemvRowMajor(uint32_t     m,
@@ -102,8 +123,13 @@ extern "C" int r355_gemv(int32_t layout_a, uint32_t m, uint32_t k, const float* 
     {
         if(lda < m)
             return r355::fail(R355_ERR_BAD_ARG, "gemv: lda < m");
-        hipLaunchKernelGGL(gemvColMajor, dim3((m / 4 + THREADS - 1) / THREADS), dim3(THREADS), 0, s, m, k, a, lda, x,
-                           y_in, y_out, alpha, beta, 1u);
+        // narrow loads while they are what it takes to give every CU a workgroup
+        if(m >= 256u * 256u)
+            hipLaunchKernelGGL(gemvColMajor<4>, dim3((m + 255u) / 256u), dim3(COL_WAVES * 64), 0, s, m, k, a, lda, x,
+                               y_in, y_out, alpha, beta);
+        else
+            hipLaunchKernelGGL(gemvColMajor<1>, dim3((m + 63u) / 64u), dim3(COL_WAVES * 64), 0, s, m, k, a, lda, x,
+                               y_in, y_out, alpha, beta);
     }
     else if(layout_a == R355_ROW_MAJOR)
     {

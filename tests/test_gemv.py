@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("layout", [O.ROW, O.COL])
-@pytest.mark.parametrize("m,k", [(256, 256), (1024, 512), (8192, 8192), (4100, 260)])
+@pytest.mark.parametrize("m,k", [(256, 256), (1024, 512), (8192, 8192), (4100, 260), (65536 + 256, 64)])
 def test_gemv_vs_oracle(layout, m, k):
     a, x, y = O.uniform_pm1(1, m * k), O.uniform_pm1(2, k), O.uniform_pm1(3, m)
     want = O.gemm(O.F32, O.F32, layout, O.COL, O.COL, O.COL, m, 1, k, a, x, y, 2.0, 2.0)

@@ -24,7 +24,7 @@ def _sparse_inputs(in_t, m, n, k, seed):
 
 
 @pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32)])
-@pytest.mark.parametrize("m,n,k", [(32, 32, 64), (96, 64, 256), (256, 128, 1024)])
+@pytest.mark.parametrize("m,n,k", [(32, 32, 64), (96, 64, 256), (256, 128, 1024), (256, 256, 512), (512, 768, 256)])
 @pytest.mark.parametrize("ldl", [O.ROW, O.COL])
 def test_sparse_gemm_vs_dense_oracle(in_t, out_t, m, n, k, ldl):
     dense, b = _sparse_inputs(in_t, m, n, k, 40)
@@ -37,6 +37,8 @@ def test_sparse_gemm_vs_dense_oracle(in_t, out_t, m, n, k, ldl):
     dd = device_filled(m * n, O.NP_STORAGE[out_t], 0xFF)
     R.gemm(in_t, out_t, m, n, k, dv, db, dc, dd, 1.0, 1.0, O.ROW, O.COL, ldl, ldl, a_meta=dm)
     got = to_host(dd, O.NP_STORAGE[out_t])
+    plan = R.gemm_query(R.gemm_args(in_t, out_t, m, n, k, dv, db, dc, dd, 1.0, 1.0, O.ROW, O.COL, ldl, ldl, a_meta=dm))
+    assert plan.kernel == (R.KERNEL_TILED if (m % 256 == 0 and n % 256 == 0 and k % 256 == 0) else R.KERNEL_SIMPLE)
     if in_t == O.I8:
         assert np.array_equal(got, want)
     else:
