@@ -576,7 +576,8 @@ namespace
                     else
                         v = *reinterpret_cast<const i32x4*>(wl + row * ROW_BYTES + ((c ^ (row & 31u)) * CHUNK));
                     const uint64_t offD = (uint64_t)(m0 + pass * ROWS_PASS + row) * p.ldd + n0;
-                    *reinterpret_cast<i32x4*>(p.d + offD * OS + c * CHUNK) = v;
+                    // D is written once and not read again: stream it past the caches
+                    __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(p.d + offD * OS + c * CHUNK));
                 }
                 __builtin_amdgcn_wave_barrier();
             }
