@@ -29,10 +29,10 @@ HBM_PEAK_GBPS = 8000.0
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--size", type=int, default=8192, help="M = N = K (default: the BASELINE size)")
-    ap.add_argument("--cpu-rows", type=int, default=48, help="output rows the CPU baseline computes")
+    ap.add_argument("--cpu-rows", type=int, default=512, help="output rows the CPU baseline computes")
     ap.add_argument("--quick", action="store_true", help="skip the extra configurations")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -83,7 +83,7 @@ def main():
     value = flop / wall_ms / 1e9
 
     # kernel duration by HIP events on the launch stream
-    ev_ms = R.gemm_timed(g, 1, args.steps)
+    ev_ms = R.gemm_timed(g, args.warmup, args.steps)
     achieved = flop / ev_ms / 1e9
 
     # ---- CPU baseline on a bounded sample (complete rows of D), doubling as validation

@@ -114,8 +114,9 @@ int r355_gemm_timed(const r355_gemm_args* args, void* stream, int warmup, int it
 /*
  * DLRM dot-interaction forward.  in: [batch][m][k], out: [batch][k + m(m-1)/2]:
  * out[b][0:k] = in[b][0][:], then the strict lower triangle of X X^T in row-major (i, j<i)
- * order, f32 accumulation, rounded to dtype (R355_F16, R355_BF16 or R355_F32).  Any m <= 32,
- * k a multiple of 32 up to 256.  No scratch buffer (the reference's `acc` argument is gone).
+ * order, f32 accumulation, rounded to dtype (R355_F16, R355_BF16 or R355_F32).  2 <= m <= 32,
+ * k in {32, 64, 128, 256} (R355_F32: up to 128).  No scratch buffer (the reference's `acc`
+ * argument is gone).
  * Replaces: dlrmDotFwd launch, test/dlrm/dlrm_kernel_base_impl.hpp:78-96,
  * test/dlrm/device/dlrm_dot_fwd.hpp:35-138, samples/simple_dlrm.cpp:184-284.
  */

@@ -97,7 +97,7 @@ namespace
                 {
                     const uint32_t c = j * 64u + lane;
                     if(c < inChunks)
-                        stash[q][j] = *reinterpret_cast<const i32x4*>(src + c * 16u);
+                        stash[q][j] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(src + c * 16u)); // read once
                 }
             }
         }
@@ -162,8 +162,91 @@ namespace
         uint16_t*      dst      = out + (uint64_t)b0 * outStride;
         const uint32_t vecs     = total / 8u;
         for(uint32_t v = tid; v < vecs; v += THREADS)
-            reinterpret_cast<i32x4*>(dst)[v] = reinterpret_cast<const i32x4*>(outLds)[v];
+            __builtin_nontemporal_store(reinterpret_cast<const i32x4*>(outLds)[v], reinterpret_cast<i32x4*>(dst) + v);
         for(uint32_t e = vecs * 8u + tid; e < total; e += THREADS)
+            dst[e] = outLds[e];
+    }
+
+    // f32 variant: one sample per wave, four per workgroup (4 * out_row_bytes is a multiple of 16),
+    // v_mfma_f32_32x32x2f32 on an LDS image of X with 16-byte chunks XOR-swizzled by row.
+    template <uint32_t K>
+    __global__ void __launch_bounds__(THREADS)
+        dlrmFwdF32Kernel(const float* __restrict__ in, float* __restrict__ out, uint32_t m, uint32_t batch)
+    {
+        constexpr uint32_t ROW_CHUNKS = K / 4; // 16-byte chunks per row
+        constexpr uint32_t MAX_OUT    = K + MAX_M * (MAX_M - 1) / 2;
+        constexpr uint32_t MAX_CHUNKS = (MAX_M * ROW_CHUNKS + 63u) / 64u;
+        using f32x4                   = float __attribute__((ext_vector_type(4)));
+
+        __shared__ __attribute__((aligned(16))) float xLds[WAVES][MAX_M * K];
+        __shared__ __attribute__((aligned(16))) float outLds[WAVES * MAX_OUT + 4];
+
+        const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+        const uint32_t outStride = K + m * (m - 1) / 2;
+        const uint32_t b0        = blockIdx.x * WAVES;
+        const uint32_t inChunks  = m * ROW_CHUNKS;
+        const uint32_t b         = b0 + wave;
+        char*          xw        = reinterpret_cast<char*>(xLds[wave]);
+
+        if(b < batch)
+        {
+            const char* src = reinterpret_cast<const char*>(in) + (uint64_t)b * m * K * 4u;
+            f32x4       stash[MAX_CHUNKS];
+#pragma unroll
+            for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
+            {
+                const uint32_t c = j * 64u + lane;
+                if(c < inChunks)
+                    stash[j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src + c * 16u));
+            }
+#pragma unroll
+            for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
+            {
+                const uint32_t c = j * 64u + lane;
+                if(c < inChunks)
+                {
+                    const uint32_t row = c / ROW_CHUNKS, col = c % ROW_CHUNKS;
+                    *reinterpret_cast<f32x4*>(xw + (row * ROW_CHUNKS + (col ^ (row & (ROW_CHUNKS - 1u) & 31u))) * 16u) = stash[j];
+                }
+            }
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_wave_barrier();
+
+            f32x16         acc   = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            const bool     valid = (lane & 31u) < m;
+            const uint32_t row   = valid ? (lane & 31u) : 0u;
+#pragma unroll 8
+            for(uint32_t s = 0; s < K / 2; ++s)
+            {
+                const uint32_t kk  = 2u * s + (lane >> 5);
+                const uint32_t col = kk >> 2;
+                float          x   = *reinterpret_cast<const float*>(
+                    xw + (row * ROW_CHUNKS + (col ^ (row & (ROW_CHUNKS - 1u) & 31u))) * 16u + (kk & 3u) * 4u);
+                if(!valid)
+                    x = 0.0f;
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x, x, acc, 0, 0, 0);
+            }
+
+            float* o = outLds + wave * outStride;
+            for(uint32_t e = lane; e < K; e += 64)
+                o[e] = reinterpret_cast<const float*>(xw)[e]; // row 0 is stored unswizzled
+            const uint32_t j = lane & 31u;
+#pragma unroll
+            for(uint32_t r = 0; r < 16; ++r)
+            {
+                const uint32_t i = 8u * (r >> 2) + 4u * (lane >> 5) + (r & 3u);
+                if(j < i && i < m)
+                    o[K + i * (i - 1u) / 2u + j] = acc[r];
+            }
+        }
+        __syncthreads();
+        const uint32_t nSamples = (batch - b0) < WAVES ? (batch - b0) : WAVES;
+        const uint32_t total    = nSamples * outStride;
+        float*         dst      = out + (uint64_t)b0 * outStride;
+        const uint32_t vecs     = total / 4u;
+        for(uint32_t v = tid; v < vecs; v += THREADS)
+            __builtin_nontemporal_store(reinterpret_cast<const f32x4*>(outLds)[v], reinterpret_cast<f32x4*>(dst) + v);
+        for(uint32_t e = vecs * 4u + tid; e < total; e += THREADS)
             dst[e] = outLds[e];
     }
 
@@ -260,12 +343,15 @@ namespace
         }
     }
 
-    int checkArgs(const char* what, int32_t dtype, const void* in, const void* out, uint32_t m, uint32_t k, uint32_t batch)
+    int checkArgs(const char* what, int32_t dtype, const void* in, const void* out, uint32_t m, uint32_t k, uint32_t batch,
+                  bool allowF32)
     {
         if(!in || !out)
             return r355::fail(R355_ERR_BAD_ARG, "%s: null pointer", what);
-        if(dtype != R355_F16 && dtype != R355_BF16)
-            return r355::fail(R355_ERR_UNSUPPORTED, "%s: dtype must be R355_F16 or R355_BF16", what);
+        if(dtype != R355_F16 && dtype != R355_BF16 && !(allowF32 && dtype == R355_F32))
+            return r355::fail(R355_ERR_UNSUPPORTED, "%s: dtype must be R355_F16, R355_BF16%s", what, allowF32 ? " or R355_F32" : "");
+        if(dtype == R355_F32 && k > 128)
+            return r355::fail(R355_ERR_BAD_SIZE, "%s: k=%u must be at most 128 for R355_F32", what, k);
         if(m < 2 || m > MAX_M)
             return r355::fail(R355_ERR_BAD_SIZE, "%s: m=%u must be in [2, %u]", what, m, MAX_M);
         if(k != 32 && k != 64 && k != 128 && k != 256)
@@ -280,11 +366,24 @@ namespace
 
 extern "C" int r355_dlrm_fwd(int32_t dtype, const void* in, void* out, uint32_t m, uint32_t k, uint32_t batch, void* stream)
 {
-    int rc = checkArgs("dlrm_fwd", dtype, in, out, m, k, batch);
+    int rc = checkArgs("dlrm_fwd", dtype, in, out, m, k, batch, true);
     if(rc != R355_OK)
         return rc;
-    const dim3  grid((batch + SAMPLES_PER_WG - 1) / SAMPLES_PER_WG), block(THREADS);
-    hipStream_t s  = static_cast<hipStream_t>(stream);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if(dtype == R355_F32)
+    {
+        const dim3 grid32((batch + WAVES - 1) / WAVES), block32(THREADS);
+        auto*      fi = static_cast<const float*>(in);
+        auto*      fo = static_cast<float*>(out);
+        switch(k)
+        {
+        case 32: hipLaunchKernelGGL(dlrmFwdF32Kernel<32>, grid32, block32, 0, s, fi, fo, m, batch); break;
+        case 64: hipLaunchKernelGGL(dlrmFwdF32Kernel<64>, grid32, block32, 0, s, fi, fo, m, batch); break;
+        default: hipLaunchKernelGGL(dlrmFwdF32Kernel<128>, grid32, block32, 0, s, fi, fo, m, batch); break;
+        }
+        return r355::checkLaunch("dlrm_fwd");
+    }
+    const dim3 grid((batch + SAMPLES_PER_WG - 1) / SAMPLES_PER_WG), block(THREADS);
     auto*       pi = static_cast<const uint16_t*>(in);
     auto*       po = static_cast<uint16_t*>(out);
 #define R355_FWD(BF, KK)                                                                         \
@@ -319,7 +418,7 @@ extern "C" int r355_dlrm_fwd(int32_t dtype, const void* in, void* out, uint32_t 
 extern "C" int r355_dlrm_bwd(int32_t dtype, const void* in, const void* upstream, void* mlp_grad, void* in_grad,
                              uint32_t m, uint32_t k, uint32_t batch, void* stream)
 {
-    int rc = checkArgs("dlrm_bwd", dtype, in, in_grad, m, k, batch);
+    int rc = checkArgs("dlrm_bwd", dtype, in, in_grad, m, k, batch, false);
     if(rc != R355_OK)
         return rc;
     if(!upstream || !mlp_grad)

@@ -5,9 +5,13 @@
 // published peak.  Usage:
 //   host_bench gemm  [--type f16|bf16|i8|e4m3] [--out f16|bf16|f32|i32] [--layout nt|tn|nn|tt]
 //                    [--m M --n N --k K] [--kernel auto|simple|tiled] [--warmup W --iters I]
-//   host_bench dlrm  [--batch B --m M --k K] [--warmup W --iters I]
+//                    [--sparse 1]   A is 2:4 structured sparse (compressed values + index nibbles)
+//   host_bench dlrm  [--type f16|bf16|f32] [--batch B --m M --k K] [--warmup W --iters I]
 //   host_bench gemv  [--m M --k K --layout n|t]
 //   host_bench copy  [--bytes N]      plain device copy of known size (counter calibration)
+//   host_bench mfma  [--iters I]      register-resident MFMA loops, one wave per SIMD, 16 independent
+//                                     accumulators: the rate the matrix cores sustain under the board's
+//                                     power limit with all-zero and with random operands
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
@@ -83,6 +87,75 @@ namespace
         return (t == R355_F16 || t == R355_BF16) ? 2 : ((t == R355_F32 || t == R355_I32) ? 4 : 1);
     }
 
+    using f32x16 = float __attribute__((ext_vector_type(16)));
+    using i32x16 = int __attribute__((ext_vector_type(16)));
+    using i32x4  = int __attribute__((ext_vector_type(4)));
+    using i32x8  = int __attribute__((ext_vector_type(8)));
+    using f16x8  = _Float16 __attribute__((ext_vector_type(8)));
+    using bf16x8 = __bf16 __attribute__((ext_vector_type(8)));
+
+    enum MfmaKind { MF_F16, MF_BF16, MF_I8, MF_FP8_K64, MF_SPARSE_I8, MF_KINDS };
+
+    // 16 MFMAs per loop trip on 4 x 4 operand registers; no memory traffic inside the loop.
+    template <int T>
+    __global__ void __launch_bounds__(256) mfmaLoop(const i32x4* __restrict__ in, float* __restrict__ out, int iters)
+    {
+        i32x4 a[4], b[4];
+        for(int i = 0; i < 4; ++i)
+        {
+            a[i] = in[(threadIdx.x + i * 256) % 1024];
+            b[i] = in[(threadIdx.x * 3 + i * 131) % 1024];
+        }
+        f32x16 acc[16];
+        i32x16 iacc[16];
+        for(int i = 0; i < 16; ++i)
+            for(int e = 0; e < 16; ++e)
+                acc[i][e] = 0.0f, iacc[i][e] = 0;
+        for(int it = 0; it < iters; ++it)
+        {
+#pragma unroll
+            for(int i = 0; i < 4; ++i)
+#pragma unroll
+                for(int j = 0; j < 4; ++j)
+                {
+                    const int  x  = i * 4 + j;
+                    const auto a8 = __builtin_shufflevector(a[i], a[(i + 1) & 3], 0, 1, 2, 3, 4, 5, 6, 7);
+                    const auto b8 = __builtin_shufflevector(b[j], b[(j + 1) & 3], 0, 1, 2, 3, 4, 5, 6, 7);
+                    if constexpr(T == MF_F16)
+                        acc[x] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a[i]),
+                                                                        __builtin_bit_cast(f16x8, b[j]), acc[x], 0, 0, 0);
+                    else if constexpr(T == MF_BF16)
+                        acc[x] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a[i]),
+                                                                         __builtin_bit_cast(bf16x8, b[j]), acc[x], 0, 0, 0);
+                    else if constexpr(T == MF_I8)
+                        iacc[x] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], iacc[x], 0, 0, 0);
+                    else if constexpr(T == MF_FP8_K64)
+                        acc[x] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, acc[x], 0, 0, 0, 0x7F7F7F7F, 0,
+                                                                                 0x7F7F7F7F);
+                    else
+                        iacc[x] = __builtin_amdgcn_smfmac_i32_32x32x64_i8(a[i], b8, iacc[x], 0x84848484, 0, 0);
+                }
+        }
+        float s = 0.0f;
+        for(int i = 0; i < 16; ++i)
+            for(int e = 0; e < 16; ++e)
+                s += acc[i][e] + static_cast<float>(iacc[i][e]);
+        out[blockIdx.x * 256 + threadIdx.x] = s;
+    }
+
+    void launchMfma(int kind, int cus, const i32x4* in, float* out, int iters)
+    {
+        const dim3 g(cus), b(256);
+        switch(kind)
+        {
+        case MF_F16: hipLaunchKernelGGL(mfmaLoop<MF_F16>, g, b, 0, 0, in, out, iters); break;
+        case MF_BF16: hipLaunchKernelGGL(mfmaLoop<MF_BF16>, g, b, 0, 0, in, out, iters); break;
+        case MF_I8: hipLaunchKernelGGL(mfmaLoop<MF_I8>, g, b, 0, 0, in, out, iters); break;
+        case MF_FP8_K64: hipLaunchKernelGGL(mfmaLoop<MF_FP8_K64>, g, b, 0, 0, in, out, iters); break;
+        default: hipLaunchKernelGGL(mfmaLoop<MF_SPARSE_I8>, g, b, 0, 0, in, out, iters); break;
+        }
+    }
+
     __global__ void copyKernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n)
     {
         for(size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
@@ -94,11 +167,12 @@ int main(int argc, char** argv)
 {
     if(argc < 2)
     {
-        fprintf(stderr, "usage: host_bench gemm|dlrm|gemv|copy [options]\n");
+        fprintf(stderr, "usage: host_bench gemm|dlrm|gemv|copy|mfma [options]\n");
         return 2;
     }
     const std::string op = argv[1];
     std::string       type = "f16", out = "", layout = "nt", kernel = "auto";
+    bool              sparse = false, itersSet = false;
     uint32_t          m = 8192, n = 8192, k = 8192, batch = 65536;
     bool              mSet = false, kSet = false;
     int               warmup = 2, iters = 10;
@@ -115,7 +189,8 @@ int main(int argc, char** argv)
         else if(a == "--k") k = atoi(v.c_str()), kSet = true;
         else if(a == "--batch") batch = atoi(v.c_str());
         else if(a == "--warmup") warmup = atoi(v.c_str());
-        else if(a == "--iters") iters = atoi(v.c_str());
+        else if(a == "--iters") iters = atoi(v.c_str()), itersSet = true;
+        else if(a == "--sparse") sparse = atoi(v.c_str()) != 0;
         else if(a == "--bytes") bytes = strtoull(v.c_str(), nullptr, 10);
         else
         {
@@ -149,10 +224,21 @@ int main(int argc, char** argv)
         g.ldc = g.ldd = n;
         g.alpha = 1.0f, g.beta = 0.0f;
         g.kernel = kernel == "simple" ? R355_KERNEL_SIMPLE : (kernel == "tiled" ? R355_KERNEL_TILED : R355_KERNEL_AUTO);
-        std::vector<uint8_t> ha((size_t)m * k * bytesOf(inT)), hb((size_t)k * n * bytesOf(inT));
+        std::vector<uint8_t> ha((size_t)m * k * bytesOf(inT) / (sparse ? 2 : 1)), hb((size_t)k * n * bytesOf(inT));
         fillBytes(ha, inT, 1);
         fillBytes(hb, inT, 2);
-        void *da, *db, *dd;
+        void *da, *db, *dd, *dmeta = nullptr;
+        if(sparse)
+        {
+            // compressed A is m x k/2 row-major; one index nibble per group of four dense columns:
+            // 0x4 keeps positions (0, 1), 0x8 keeps positions (0, 2)
+            g.sparse24 = 1;
+            g.lda      = k / 2;
+            std::vector<uint8_t> hm((size_t)m * k / 8, 0x84);
+            HIP_OK(hipMalloc(&dmeta, hm.size()));
+            HIP_OK(hipMemcpy(dmeta, hm.data(), hm.size(), hipMemcpyHostToDevice));
+            g.a_meta = dmeta;
+        }
         HIP_OK(hipMalloc(&da, ha.size()));
         HIP_OK(hipMalloc(&db, hb.size()));
         HIP_OK(hipMalloc(&dd, (size_t)m * n * bytesOf(outT)));
@@ -168,13 +254,13 @@ int main(int argc, char** argv)
         }
         const double flop   = 2.0 * m * n * k;
         const double tflops = flop / ms / 1e9;
-        const double vendor = (inT == R355_I8 || inT == R355_E4M3) ? 5000.0 : 2500.0; // dense TFLOP/s | TOP/s
+        const double vendor = ((inT == R355_I8 || inT == R355_E4M3) ? 5000.0 : 2500.0) * (sparse ? 2.0 : 1.0);
         const double perClk = (inT == R355_I8 || inT == R355_E4M3) ? 8192.0 : 4096.0; // flop / CU / clk
         const double model  = perClk * dev.compute_units * dev.clock_mhz * 1e-6; // TFLOP/s at the reported clock
-        printf("{\"op\": \"gemm\", \"type\": \"%s\", \"out\": \"%s\", \"layout\": \"%s\", \"m\": %u, \"n\": %u, \"k\": %u, "
+        printf("{\"op\": \"%s\", \"type\": \"%s\", \"out\": \"%s\", \"layout\": \"%s\", \"m\": %u, \"n\": %u, \"k\": %u, "
                "\"kernel\": %d, \"macro_tile\": [%u, %u, %u], \"lds_bytes\": %u, \"ms\": %.4f, \"tflops\": %.1f, "
                "\"frac_vendor_peak\": %.4f, \"frac_clock_model_peak\": %.4f, \"cus\": %d, \"clock_mhz\": %d}\n",
-               type.c_str(), out.c_str(), layout.c_str(), m, n, k, plan.kernel, plan.macro_tile_m, plan.macro_tile_n,
+               sparse ? "gemm_sparse24" : "gemm", type.c_str(), out.c_str(), layout.c_str(), m, n, k, plan.kernel, plan.macro_tile_m, plan.macro_tile_n,
                plan.macro_tile_k, plan.lds_bytes, ms, tflops, tflops / vendor, tflops / model, dev.compute_units,
                dev.clock_mhz);
     }
@@ -183,21 +269,24 @@ int main(int argc, char** argv)
         if(!mSet) m = 27;
         if(!kSet) k = 128;
         const size_t inElems = (size_t)batch * m * k, outElems = (size_t)batch * (k + m * (m - 1) / 2);
-        std::vector<uint8_t> hx(inElems * 2);
-        fillBytes(hx, R355_F16, 3);
+        const int    dt = parseType(type);
+        const size_t es = bytesOf(dt);
+        std::vector<uint8_t> hx(inElems * es);
+        fillBytes(hx, dt, 3);
         void *dx, *dout;
         HIP_OK(hipMalloc(&dx, hx.size()));
-        HIP_OK(hipMalloc(&dout, outElems * 2));
+        HIP_OK(hipMalloc(&dout, outElems * es));
         HIP_OK(hipMemcpy(dx, hx.data(), hx.size(), hipMemcpyHostToDevice));
-        if(r355_dlrm_fwd_timed(R355_F16, dx, dout, m, k, batch, nullptr, warmup, iters, &ms) != R355_OK)
+        if(r355_dlrm_fwd_timed(dt, dx, dout, m, k, batch, nullptr, warmup, iters, &ms) != R355_OK)
         {
             fprintf(stderr, "%s\n", r355_last_error());
             return 1;
         }
-        const double byts = (double)(inElems + outElems) * 2.0;
-        printf("{\"op\": \"dlrm_fwd\", \"batch\": %u, \"m\": %u, \"k\": %u, \"ms\": %.4f, \"gbps\": %.1f, "
+        const double byts = (double)(inElems + outElems) * es;
+        printf("{\"op\": \"dlrm_fwd\", \"type\": \"%s\", \"batch\": %u, \"m\": %u, \"k\": %u, \"ms\": %.4f, \"gbps\": %.1f, "
                "\"frac_hbm_peak\": %.4f, \"gflops_ref_convention\": %.1f}\n",
-               batch, m, k, ms, byts / ms / 1e6, byts / ms / 1e6 / 8000.0, 2.0 * m * m * k * batch / ms / 1e6);
+               type.c_str(), batch, m, k, ms, byts / ms / 1e6, byts / ms / 1e6 / 8000.0,
+               2.0 * m * m * k * batch / ms / 1e6);
     }
     else if(op == "gemv")
     {
@@ -223,6 +312,49 @@ int main(int argc, char** argv)
         const double byts = (double)m * k * 4.0 + (double)(m + k) * 4.0;
         printf("{\"op\": \"gemv\", \"m\": %u, \"k\": %u, \"ms\": %.4f, \"gbps\": %.1f, \"frac_hbm_peak\": %.4f}\n", m, k,
                ms, byts / ms / 1e6, byts / ms / 1e6 / 8000.0);
+    }
+    else if(op == "mfma")
+    {
+        const int loops = itersSet ? iters : 20000;
+        i32x4*    in;
+        float*    outBuf;
+        HIP_OK(hipMalloc(&in, 1024 * sizeof(i32x4)));
+        HIP_OK(hipMalloc(&outBuf, (size_t)dev.compute_units * 256 * sizeof(float)));
+        hipEvent_t e0, e1;
+        HIP_OK(hipEventCreate(&e0));
+        HIP_OK(hipEventCreate(&e1));
+        static const char*  names[MF_KINDS] = {"f16 32x32x16", "bf16 32x32x16", "i8 32x32x32", "fp8 f8f6f4 32x32x64",
+                                               "sparse i8 smfmac 32x32x64 (dense-equivalent ops)"};
+        static const double flopPer[MF_KINDS]
+            = {2.0 * 32 * 32 * 16, 2.0 * 32 * 32 * 16, 2.0 * 32 * 32 * 32, 2.0 * 32 * 32 * 64, 2.0 * 32 * 32 * 64};
+        static const double vendorPeak[MF_KINDS] = {2500.0, 2500.0, 5000.0, 5000.0, 10000.0};
+        printf("[");
+        for(int random = 0; random < 2; ++random)
+            for(int kind = 0; kind < MF_KINDS; ++kind)
+            {
+                std::vector<uint32_t> h(4096, 0u);
+                for(size_t i = 0; random && i < h.size(); ++i)
+                {
+                    const uint32_t r = static_cast<uint32_t>(splitmix(7 + kind, i));
+                    h[i] = kind == MF_F16    ? ((r & 0x8FFF8FFFu) | 0x30003000u)  // |x| in [1/8, 1)
+                           : kind == MF_BF16 ? ((r & 0x807F807Fu) | 0x3E003E00u)  // |x| in [1/8, 1/4)
+                           : kind == MF_FP8_K64 ? ((r & 0x87878787u) | 0x30303030u) // |x| in [1/2, 1)
+                                                : r;
+                }
+                HIP_OK(hipMemcpy(in, h.data(), h.size() * 4, hipMemcpyHostToDevice));
+                launchMfma(kind, dev.compute_units, in, outBuf, 1000);
+                HIP_OK(hipDeviceSynchronize());
+                HIP_OK(hipEventRecord(e0));
+                launchMfma(kind, dev.compute_units, in, outBuf, loops);
+                HIP_OK(hipEventRecord(e1));
+                HIP_OK(hipEventSynchronize(e1));
+                HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+                const double tf = (double)dev.compute_units * 4 * loops * 16 * flopPer[kind] / ms / 1e9;
+                printf("%s\n {\"op\": \"mfma\", \"instr\": \"%s\", \"operands\": \"%s\", \"ms\": %.3f, \"tflops\": %.1f, "
+                       "\"frac_vendor_peak\": %.4f}",
+                       (random || kind) ? "," : "", names[kind], random ? "random" : "zero", ms, tf, tf / vendorPeak[kind]);
+            }
+        printf("\n]\n");
     }
     else if(op == "copy")
     {

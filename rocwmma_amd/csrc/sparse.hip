@@ -331,7 +331,7 @@ namespace
                     for(uint32_t e = 0; e < 4; ++e)
                         v[e] += beta * cv[e];
                 }
-                *reinterpret_cast<V4*>(p.d + (off * p.ldd + n0) * 4u + c * 16u) = v;
+                __builtin_nontemporal_store(v, reinterpret_cast<V4*>(p.d + (off * p.ldd + n0) * 4u + c * 16u));
             }
             __builtin_amdgcn_wave_barrier();
         }

@@ -81,8 +81,11 @@ def test_dlrm_and_gemv_validation_without_gpu():
         R.dlrm_fwd(R.F16, 0x1000, 0x2000, 27, 100, 8)
     assert e.value.code == -3
     with pytest.raises(R.R355Error) as e:
-        R.dlrm_fwd(R.F32, 0x1000, 0x2000, 27, 128, 8)
+        R.dlrm_fwd(R.I8, 0x1000, 0x2000, 27, 128, 8)
     assert e.value.code == -2
+    with pytest.raises(R.R355Error) as e:
+        R.dlrm_fwd(R.F32, 0x1000, 0x2000, 27, 256, 8)
+    assert e.value.code == -3
     with pytest.raises(R.R355Error) as e:
         R.gemv(R.COL_MAJOR, 10, 16, 0x1000, 0x2000, None, 0x3000)
     assert e.value.code == -3

@@ -23,6 +23,61 @@ def _fwd(dtype, x, m, k, batch):
     return full[:out_elems].reshape(batch, -1)
 
 
+def _exact_fwd_f32(x, m, k, batch):
+    """float64 evaluation of the interaction terms (inputs are exact in float64)."""
+    X = x.reshape(batch, m, k).astype(np.float64)
+    T = np.einsum("bik,bjk->bij", X, X)
+    ii, jj = np.tril_indices(m, -1)
+    return T[:, ii, jj]
+
+
+def _rel(a, b):
+    a, b = a.astype(np.float64), b.astype(np.float64)
+    return float(np.max(np.abs(a - b) / (np.abs(a) + np.abs(b) + 1.0)))
+
+
+# f32 bar.  Any two f32 summation orders of a k = 128 dot product differ by more than the
+# reference's 10 eps (the reference-held output_fp32 fixture itself sits 12 eps from a sequential
+# f32 sum and 13 eps from the exact value), so the f32 checks are: within 40 eps(f32) of the oracle
+# and of the fixture in the reference's relative-error metric, and no further from the float64-exact
+# value than 1.5 x the sequential-f32 oracle's own distance from it.
+F32_TOL_EPS = 40.0
+
+
+def _check_f32(got, want_oracle, x, m, k, batch):
+    assert np.array_equal(got[:, :k], want_oracle[:, :k])
+    ok, mx = O.compare(O.F32, got, want_oracle, F32_TOL_EPS)
+    assert ok, mx
+    exact = _exact_fwd_f32(x, m, k, batch)
+    assert _rel(got[:, k:], exact) <= 1.5 * _rel(want_oracle[:, k:], exact) + 1e-9
+
+
+def test_fwd_reference_fixture_fp32():
+    x = np.fromfile(os.path.join(GOLD, "input_fp32"), dtype=np.float32)
+    want = np.fromfile(os.path.join(GOLD, "output_fp32"), dtype=np.float32).reshape(64, 479)
+    dx = to_device(x)
+    dout = device_filled(64 * 479 + 4, np.float32, 0xFF)
+    R.dlrm_fwd(R.F32, dx, dout, 27, 128, 64)
+    full = to_host(dout, np.float32)
+    assert np.all(np.isnan(full[64 * 479:]))
+    got = full[:64 * 479].reshape(64, 479)
+    assert np.array_equal(got[:, :128], want[:, :128])
+    ok, mx = O.compare(O.F32, got, want, F32_TOL_EPS)
+    assert ok, mx
+    _check_f32(got, O.dlrm_fwd(O.F32, x, 27, 128, 64), x, 27, 128, 64)
+
+
+@pytest.mark.parametrize("m,k,batch", [(32, 32, 64), (27, 128, 13), (2, 64, 5), (32, 128, 3)])
+def test_fwd_f32_shapes_vs_oracle(m, k, batch):
+    x = O.normal(3, batch * m * k)
+    want = O.dlrm_fwd(O.F32, x, m, k, batch)
+    dx = to_device(x)
+    dout = device_filled(want.size, np.float32, 0xFF)
+    R.dlrm_fwd(R.F32, dx, dout, m, k, batch)
+    got = to_host(dout, np.float32).reshape(batch, -1)
+    _check_f32(got, want, x, m, k, batch)
+
+
 def test_fwd_reference_fixture_fp16():
     x = np.fromfile(os.path.join(GOLD, "input_fp16"), dtype=np.uint16)
     want = np.fromfile(os.path.join(GOLD, "output_fp16"), dtype=np.uint16).reshape(64, 479)
