@@ -24,6 +24,12 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "e4m3": 5000.0, "i8": 5000.0}
 HBM_PEAK_GBPS = 8000.0
+# Bytes one 8192^3 f16 NT launch moves across the L2 <-> fabric boundary, from two rocprofv3 --pmc
+# runs of `host_bench gemm --type f16 --layout nt`: FETCH_SIZE 7.866e5 x 2 KiB + WRITE_SIZE 1.311e5
+# x 1 KiB (unit sizes calibrated with `host_bench copy --bytes 1073741824`, which reads 5.243e5 and
+# writes 1.049e6 units for 1 GiB each way).  The fetch side is 6 x the 256 MiB of A and B: each
+# 4 MiB operand panel is fetched once per group of tiles that share an XCD's L2.
+TRAFFIC_F16_NT_8192 = int(7.866e5 * 2048 + 1.311e5 * 1024)
 
 
 def main():
@@ -124,7 +130,8 @@ def main():
         "validated": validated,
         "max_rel_error_vs_oracle": max_rel,
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_TFLOPS["f16"], 4), "traffic": None,
+                     "frac": round(achieved / PEAK_TFLOPS["f16"], 4),
+                     "traffic": TRAFFIC_F16_NT_8192 if args.size == 8192 else None,
                      "kernel_ms": round(ev_ms, 4), "algorithmic_flop": flop,
                      "algorithmic_bytes": (m * k + k * n) * 2 + m * n * 2},
         "cpu_baseline": {"value": round(cpu_tflops, 6), "unit": "TFLOP/s", "cores": O.lib().orc_num_threads(),

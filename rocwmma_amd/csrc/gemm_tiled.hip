@@ -619,7 +619,7 @@ namespace
     Variant chosenVariant()
     {
         static const Variant v = [] {
-            Variant     r{true, false};
+            Variant     r{true, true};
             const char* e = getenv("R355_TILED_VARIANT");
             if(e)
             {

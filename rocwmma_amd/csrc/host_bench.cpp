@@ -44,7 +44,7 @@ namespace
         return z ^ (z >> 31);
     }
 
-    // cheap bit patterns in a sane range for each type: small values, no NaN / inf
+    // seeded values in a sane range for each type, no NaN / inf
     void fillBytes(std::vector<uint8_t>& buf, int dtype, uint64_t seed)
     {
         const size_t es = (dtype == R355_F16 || dtype == R355_BF16) ? 2 : (dtype == R355_F32 ? 4 : 1);
@@ -54,14 +54,21 @@ namespace
             const uint64_t r = splitmix(seed, i);
             switch(dtype)
             {
-            case R355_F16: // sign, exponent 2^-4..2^-1, random mantissa: |x| in [1/16, 1)
-                reinterpret_cast<uint16_t*>(buf.data())[i]
-                    = static_cast<uint16_t>(((r & 1) << 15) | ((11 + ((r >> 1) & 3)) << 10) | ((r >> 8) & 0x3FF));
+            case R355_F16: // U[-1, 1) rounded to the type, like bench.py's operands
+            {
+                const _Float16 h = static_cast<_Float16>(static_cast<float>(r >> 40) * (2.0f / 16777216.0f) - 1.0f);
+                memcpy(buf.data() + 2 * i, &h, 2);
                 break;
+            }
             case R355_BF16:
-                reinterpret_cast<uint16_t*>(buf.data())[i]
-                    = static_cast<uint16_t>(((r & 1) << 15) | ((123 + ((r >> 1) & 3)) << 7) | ((r >> 8) & 0x7F));
+            {
+                const float f = static_cast<float>(r >> 40) * (2.0f / 16777216.0f) - 1.0f;
+                uint32_t    u;
+                memcpy(&u, &f, 4);
+                u += 0x7FFFu + ((u >> 16) & 1u); // round to nearest even
+                reinterpret_cast<uint16_t*>(buf.data())[i] = static_cast<uint16_t>(u >> 16);
                 break;
+            }
             case R355_E4M3: // exponent 3..6: |x| in [1/16, 1)
                 buf[i] = static_cast<uint8_t>(((r & 1) << 7) | ((3 + ((r >> 1) & 3)) << 3) | ((r >> 8) & 7));
                 break;
