@@ -168,17 +168,19 @@ def run_extras(R, O, np, torch, args):
               PEAK_TFLOPS["f16"], "TFLOP/s")
     i8 = lambda nel: torch.randint(-128, 128, (nel,), dtype=torch.int16, device="cuda").to(torch.int8)
     gemm_case("gemm_i8_tn_8192", R.I8, R.I32, R.ROW_MAJOR, R.COL_MAJOR, i8(s * s), i8(s * s), PEAK_TFLOPS["i8"], "TOP/s")
-    # e4m3 codes with exponent 3..9: |x| in [1/16, 8), no NaN
-    f8 = lambda nel: ((torch.randint(0x18, 0x50, (nel,), dtype=torch.int16, device="cuda")
-                       | (torch.randint(0, 2, (nel,), dtype=torch.int16, device="cuda") << 7)).to(torch.uint8))
+    # e4m3: N(0, 1) draws rounded to nearest-even and saturated to the finite range (|x| <= 448;
+    # scale 1.0, so saturation never triggers in practice)
+    f8 = lambda nel: torch.randn(nel, device="cuda").clamp_(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8)
     gemm_case("gemm_e4m3_tn_8192", R.E4M3, R.F32, R.ROW_MAJOR, R.COL_MAJOR, f8(s * s), f8(s * s), PEAK_TFLOPS["e4m3"],
               "TFLOP/s")
     # 2:4 sparse, BASELINE config 4: M = N = 4096, dense-equivalent K = 8192, int8; dense-equivalent ops
-    # against the sparse peak (2 x dense)
+    # against the sparse peak (2 x dense).  Every group of 4 keeps 2 values at random positions:
+    # one index nibble idx0 | idx1 << 2 (idx0 < idx1) per group, two groups per metadata byte.
     sm, sn, sk = 4096, 4096, 8192
     vals = i8(sm * sk // 2)
-    # index nibbles 0x4 = positions (0, 1) and 0x8 = positions (0, 2): idx0 < idx1 in every group
-    meta = torch.full((sm * sk // 8,), 0x84, dtype=torch.uint8, device="cuda")
+    pairs = torch.tensor([0x4, 0x8, 0xC, 0x9, 0xD, 0xE], dtype=torch.uint8, device="cuda")
+    nib = pairs[torch.randint(0, 6, (sm * sk // 4,), device="cuda")].view(-1, 2)
+    meta = (nib[:, 0] | (nib[:, 1] << 4)).contiguous()
     gemm_case("gemm_i8_sparse24_4096x4096x8192", R.I8, R.I32, R.ROW_MAJOR, R.COL_MAJOR, vals, i8(sk * sn),
               PEAK_TFLOPS["i8"], "TOP/s (dense-equivalent)", sparse_meta=meta, mm=sm, nn=sn, kk=sk, peak_scale=2.0)
     # DLRM dot interaction forward, BASELINE config 5

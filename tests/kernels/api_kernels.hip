@@ -121,6 +121,8 @@ namespace
 } // namespace
 
 // ---- dispatch tables.  A case id selects (role, BlockM, BlockN, BlockK, type, layout).
+// Cases 26..89 sample the reference's unit-test matrix (test/unit/unit_test_params.hpp:86-146:
+// block extents 16..256 x 8..256, 8/16/32-bit types, both layouts) within 64 registers per lane.
 #define FRAG_CASES(X)                                                                  \
     X(0, matrix_a, 16, 16, 16, float16_t, row_major)                                   \
     X(1, matrix_a, 16, 16, 16, float16_t, col_major)                                   \
@@ -147,7 +149,71 @@ namespace
     X(22, accumulator, 32, 32, 16, int32_t, row_major)                                 \
     X(23, matrix_a, 32, 32, 32, float16_t, row_major)                                  \
     X(24, matrix_b, 16, 16, 4, float32_t, col_major)                                   \
-    X(25, accumulator, 64, 64, 16, float32_t, col_major)
+    X(25, accumulator, 64, 64, 16, float32_t, col_major)                               \
+    X(26, matrix_a, 16, 16, 128, bfloat16_t, row_major)                                \
+    X(27, matrix_b, 16, 32, 16, bfloat16_t, row_major)                                 \
+    X(28, matrix_a, 32, 16, 32, bfloat16_t, col_major)                                 \
+    X(29, matrix_b, 16, 32, 64, bfloat16_t, col_major)                                 \
+    X(30, matrix_a, 32, 16, 256, bfloat16_t, row_major)                                \
+    X(31, matrix_b, 16, 64, 8, bfloat16_t, row_major)                                  \
+    X(32, matrix_a, 64, 16, 64, bfloat16_t, col_major)                                 \
+    X(33, matrix_b, 16, 128, 8, bfloat16_t, col_major)                                 \
+    X(34, matrix_a, 128, 16, 16, bfloat16_t, row_major)                                \
+    X(35, matrix_b, 16, 256, 16, bfloat16_t, row_major)                                \
+    X(36, matrix_a, 16, 16, 16, float16_t, col_major)                                  \
+    X(37, matrix_b, 16, 16, 256, float16_t, col_major)                                 \
+    X(38, matrix_a, 32, 16, 8, float16_t, row_major)                                   \
+    X(39, matrix_b, 16, 32, 16, float16_t, row_major)                                  \
+    X(40, matrix_a, 32, 16, 128, float16_t, col_major)                                 \
+    X(41, matrix_b, 16, 32, 256, float16_t, col_major)                                 \
+    X(42, matrix_a, 64, 16, 16, float16_t, row_major)                                  \
+    X(43, matrix_b, 16, 64, 128, float16_t, row_major)                                 \
+    X(44, matrix_a, 128, 16, 16, float16_t, col_major)                                 \
+    X(45, matrix_b, 16, 128, 32, float16_t, col_major)                                 \
+    X(46, matrix_a, 128, 16, 64, float16_t, row_major)                                 \
+    X(47, matrix_b, 16, 256, 8, float16_t, row_major)                                  \
+    X(48, matrix_a, 256, 16, 32, float16_t, col_major)                                 \
+    X(49, matrix_b, 16, 16, 32, float32_t, col_major)                                  \
+    X(50, matrix_a, 32, 16, 32, float32_t, row_major)                                  \
+    X(51, matrix_b, 16, 64, 8, float32_t, row_major)                                   \
+    X(52, matrix_a, 64, 16, 64, float32_t, col_major)                                  \
+    X(53, matrix_b, 16, 16, 32, float8_t, col_major)                                   \
+    X(54, matrix_a, 16, 16, 128, float8_t, row_major)                                  \
+    X(55, matrix_b, 16, 32, 32, float8_t, row_major)                                   \
+    X(56, matrix_a, 32, 16, 64, float8_t, col_major)                                   \
+    X(57, matrix_b, 16, 32, 256, float8_t, col_major)                                  \
+    X(58, matrix_a, 64, 16, 64, float8_t, row_major)                                   \
+    X(59, matrix_b, 16, 64, 128, float8_t, row_major)                                  \
+    X(60, matrix_a, 128, 16, 16, float8_t, col_major)                                  \
+    X(61, matrix_b, 16, 128, 64, float8_t, col_major)                                  \
+    X(62, matrix_a, 256, 16, 8, float8_t, row_major)                                   \
+    X(63, matrix_b, 16, 256, 32, float8_t, row_major)                                  \
+    X(64, matrix_a, 256, 16, 64, float8_t, col_major)                                  \
+    X(65, matrix_b, 16, 16, 128, int8_t, col_major)                                    \
+    X(66, matrix_a, 32, 16, 32, int8_t, row_major)                                     \
+    X(67, matrix_b, 16, 32, 128, int8_t, row_major)                                    \
+    X(68, matrix_a, 32, 16, 256, int8_t, col_major)                                    \
+    X(69, matrix_b, 16, 64, 32, int8_t, col_major)                                     \
+    X(70, matrix_a, 64, 16, 64, int8_t, row_major)                                     \
+    X(71, matrix_b, 16, 128, 8, int8_t, row_major)                                     \
+    X(72, matrix_a, 128, 16, 64, int8_t, col_major)                                    \
+    X(73, matrix_b, 16, 256, 32, int8_t, col_major)                                    \
+    X(74, accumulator, 16, 64, 16, float32_t, row_major)                               \
+    X(75, accumulator, 16, 64, 16, float32_t, col_major)                               \
+    X(76, accumulator, 64, 16, 16, float32_t, row_major)                               \
+    X(77, accumulator, 64, 16, 16, float32_t, col_major)                               \
+    X(78, accumulator, 128, 32, 16, float32_t, row_major)                              \
+    X(79, accumulator, 128, 32, 16, float32_t, col_major)                              \
+    X(80, accumulator, 32, 128, 16, int32_t, row_major)                                \
+    X(81, accumulator, 32, 128, 16, int32_t, col_major)                                \
+    X(82, accumulator, 64, 64, 16, float16_t, row_major)                               \
+    X(83, accumulator, 64, 64, 16, float16_t, col_major)                               \
+    X(84, accumulator, 256, 16, 16, float32_t, row_major)                              \
+    X(85, accumulator, 256, 16, 16, float32_t, col_major)                              \
+    X(86, accumulator, 16, 16, 16, int32_t, row_major)                                 \
+    X(87, accumulator, 16, 16, 16, int32_t, col_major)                                 \
+    X(88, accumulator, 16, 256, 16, float16_t, row_major)                              \
+    X(89, accumulator, 16, 256, 16, float16_t, col_major)
 
 extern "C" {
 

@@ -14,7 +14,7 @@ from gpuutil import api_lib, device_filled, to_device, to_host
 
 pytestmark = pytest.mark.gpu
 
-CASES = list(range(26))
+CASES = list(range(90))
 
 
 def _info(cid):
@@ -60,7 +60,7 @@ def test_load_store_round_trip_leaves_padding_untouched(cid):
     assert np.all(out2d[mask] == canary)
 
 
-@pytest.mark.parametrize("cid", [0, 3, 8, 9, 10, 11, 12, 22])
+@pytest.mark.parametrize("cid", [0, 3, 8, 9, 10, 11, 12, 22, 30, 41, 52, 57, 66, 75, 78, 81, 83, 88])
 def test_runtime_layout_overloads(cid):
     rows, cols, eb, rm, _ = _info(cid)
     mat, flat, ld, _ = _padded(rows, cols, eb, rm, 0, 77 + cid)
@@ -69,7 +69,17 @@ def test_runtime_layout_overloads(cid):
     assert np.array_equal(to_host(d_out, flat.dtype), flat)
 
 
-@pytest.mark.parametrize("cid", [0, 5, 6, 8, 11, 13, 15, 17, 20, 22, 25])
+# element type of each case, for the expected fill pattern (mirrors FRAG_CASES in api_kernels.hip)
+def _case_types():
+    import os, re
+    src = open(os.path.join(os.path.dirname(__file__), "kernels", "api_kernels.hip")).read()
+    return {int(m.group(1)): m.group(2) for m in re.finditer(r"X\((\d+), \w+, \d+, \d+, \d+, (\w+), \w+\)", src)}
+
+
+CASE_TYPE = _case_types()
+
+
+@pytest.mark.parametrize("cid", [0, 5, 6, 8, 11, 13, 15, 17, 20, 22, 25] + list(range(26, 90, 3)))
 def test_fill_fragment(cid):
     rows, cols, eb, rm, ne = _info(cid)
     assert ne == rows * cols // 64
@@ -77,22 +87,17 @@ def test_fill_fragment(cid):
     d_out = device_filled(rows * cols, _np_dtype(eb), 0xEE)
     assert api_lib().api_fill(cid, ctypes.c_void_p(d_out.data_ptr()), ld, ctypes.c_float(-3.0)) == 0
     out = to_host(d_out, _np_dtype(eb))
-    if cid in (13, 21):
-        want = np.int8(-3).view(np.uint8)
-    elif cid == 22:
-        want = np.int32(-3).view(np.uint32)
-    elif cid in (15, 16):
-        want = O.f32_to_storage(np.float32([-3.0]), O.E4M3)[0]
-    elif cid in (6, 7):
-        want = O.f32_to_storage(np.float32([-3.0]), O.BF16)[0]
-    elif eb == 2:
-        want = np.float16(-3.0).view(np.uint16)
-    else:
-        want = np.float32(-3.0).view(np.uint32)
+    t = CASE_TYPE[cid]
+    want = {"int8_t": lambda: np.int8(-3).view(np.uint8),
+            "int32_t": lambda: np.int32(-3).view(np.uint32),
+            "float8_t": lambda: O.f32_to_storage(np.float32([-3.0]), O.E4M3)[0],
+            "bfloat16_t": lambda: O.f32_to_storage(np.float32([-3.0]), O.BF16)[0],
+            "float16_t": lambda: np.float16(-3.0).view(np.uint16),
+            "float32_t": lambda: np.float32(-3.0).view(np.uint32)}[t]()
     assert np.all(out == want)
 
 
-@pytest.mark.parametrize("cid", [4, 7, 10, 17, 18, 19, 20, 21, 25])
+@pytest.mark.parametrize("cid", [4, 7, 10, 17, 18, 19, 20, 21, 25, 32, 36, 48, 51, 61, 64, 72, 73, 79, 80, 85, 89])
 @pytest.mark.parametrize("waves", [(1, 1), (2, 1), (2, 2), (4, 2)])
 @pytest.mark.parametrize("use_lds", [0, 1])
 def test_cooperative_round_trip(cid, waves, use_lds):

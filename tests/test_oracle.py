@@ -304,3 +304,19 @@ def test_sparse24_format_invariants():
     few = dense.copy(); few[1, :8] = 0; few[2, 0:4] = [0, 0, 0, 9]
     v2, m2 = O.compress24(few.view(np.uint8), m, k)
     assert np.array_equal(O.decompress24(v2, m2, m, k), few.view(np.uint8))
+
+
+def test_e4m3_matches_torch_float8_e4m3fn():
+    """An independent implementation of the same OCP format: torch's float8_e4m3fn cast (round to
+    nearest even; values beyond +-448 clamped first, as the saturating conversion does)."""
+    torch = pytest.importorskip("torch")
+    if not hasattr(torch, "float8_e4m3fn"):
+        pytest.skip("torch without float8_e4m3fn")
+    x = np.concatenate([O.normal(11, 1 << 18), O.normal(12, 1 << 16) * 200.0, O.uniform_pm1(13, 1 << 16) * 2.0 ** -7,
+                        np.float32([0.0, -0.0, 448.0, -448.0, 1e9, -1e9, 2.0 ** -9, 2.0 ** -10, 3 * 2.0 ** -11])])
+    t = torch.from_numpy(x.copy()).clamp_(-448.0, 448.0).to(torch.float8_e4m3fn)
+    got = O.f32_to_storage(x, O.E4M3)
+    want = t.view(torch.uint8).numpy()
+    # -0.0 and +0.0 encode to 0x80 / 0x00 in both; compare bytes
+    assert np.array_equal(got, want)
+    assert np.array_equal(O.storage_to_f32(got, O.E4M3), t.to(torch.float32).numpy())
