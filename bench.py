@@ -193,6 +193,22 @@ def run_extras(R, O, np, torch, args):
                                        "peak": HBM_PEAK_GBPS, "frac": round(byts / ms / 1e6 / HBM_PEAK_GBPS, 4),
                                        "algorithmic_bytes": byts,
                                        "gflops_ref_convention": round(2.0 * mm * mm * kk * bsz / ms / 1e6, 1)}
+    # DLRM backward on the same shape: reads X and the upstream gradient, writes both gradients
+    up = torch.randn(bsz * (kk + mm * (mm - 1) // 2), device="cuda").to(torch.float16)
+    gmlp = torch.empty(bsz * kk, dtype=torch.float16, device="cuda")
+    gin = torch.empty(bsz * mm * kk, dtype=torch.float16, device="cuda")
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for it in range(args.warmup + args.steps):
+        if it == args.warmup:
+            e0.record()  # the C ABI launches on the null stream, which torch's default stream is
+        R.dlrm_bwd(R.F16, x, up, gmlp, gin, mm, kk, bsz)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / args.steps
+    byts = (2 * bsz * mm * kk + bsz * (kk + mm * (mm - 1) // 2) + bsz * kk) * 2
+    out["dlrm_bwd_b65536_f27_d128"] = {"ms": round(ms, 4), "value": round(byts / ms / 1e6, 1), "unit": "GB/s",
+                                       "peak": HBM_PEAK_GBPS, "frac": round(byts / ms / 1e6 / HBM_PEAK_GBPS, 4),
+                                       "algorithmic_bytes": byts}
     return out
 
 

@@ -442,7 +442,7 @@ int orc_dlrm_bwd(int         dtype,
 {
     size_t in_stride = (size_t)m * k;
     size_t up_stride = ((size_t)m * (m - 1)) / 2 + k;
-    if(dtype != ORC_F16 && dtype != ORC_F32)
+    if(dtype != ORC_F16 && dtype != ORC_F32 && dtype != ORC_BF16)
         return -1;
 #pragma omp parallel for schedule(static)
     for(int64_t b = 0; b < (int64_t)batch; ++b)

@@ -16,9 +16,9 @@
 //   * the strict lower triangle and the copied first row are assembled in an LDS image of
 //     the output and leave with coalesced 128-bit stores.  No global scratch.
 //
-// Backward takes the place of test/dlrm/device/dlrm_dot_bwd.hpp:35-176: the upstream
-// triangle is rebuilt symmetric in LDS (trilReconstruct) and multiplied into X with the
-// same matrix instruction, again without global scratch.
+// Backward takes the place of test/dlrm/device/dlrm_dot_bwd.hpp:35-176: the symmetric matrix
+// of the upstream triangle (trilReconstruct) is formed directly as a matrix-instruction operand
+// and multiplied into X, read from LDS with transposing reads, again without global scratch.
 #include <hip/hip_runtime.h>
 
 #include "common.hpp"
@@ -167,38 +167,50 @@ namespace
             dst[e] = outLds[e];
     }
 
-    // f32 variant: one sample per wave, four per workgroup (4 * out_row_bytes is a multiple of 16),
-    // v_mfma_f32_32x32x2f32 on an LDS image of X with 16-byte chunks XOR-swizzled by row.
-    template <uint32_t K>
+    // f32 variant.  An f32 sample is 13.8 KB, so only a few fit in LDS per CU and the matrix core
+    // (v_mfma_f32_32x32x2f32, 64 instructions per sample) is busy almost half of the time: the loads
+    // of a wave's next sample are therefore issued before the current sample is computed, and every
+    // wave walks F32_PER_WAVE consecutive samples, writing each result row from its own LDS image
+    // with coalesced 4-byte stores (a sample's output row is only 4-byte aligned).
+    constexpr uint32_t F32_PER_WAVE = 8;
+
+    template <uint32_t K, uint32_t ROWS>
     __global__ void __launch_bounds__(THREADS)
         dlrmFwdF32Kernel(const float* __restrict__ in, float* __restrict__ out, uint32_t m, uint32_t batch)
     {
         constexpr uint32_t ROW_CHUNKS = K / 4; // 16-byte chunks per row
-        constexpr uint32_t MAX_OUT    = K + MAX_M * (MAX_M - 1) / 2;
-        constexpr uint32_t MAX_CHUNKS = (MAX_M * ROW_CHUNKS + 63u) / 64u;
+        constexpr uint32_t MAX_OUT    = K + ROWS * (ROWS - 1) / 2;
+        constexpr uint32_t MAX_CHUNKS = (ROWS * ROW_CHUNKS + 63u) / 64u;
+        constexpr uint32_t SWZ        = 31u & (ROW_CHUNKS - 1u);
         using f32x4                   = float __attribute__((ext_vector_type(4)));
 
-        __shared__ __attribute__((aligned(16))) float xLds[WAVES][MAX_M * K];
-        __shared__ __attribute__((aligned(16))) float outLds[WAVES * MAX_OUT + 4];
+        __shared__ __attribute__((aligned(16))) float xLds[WAVES][ROWS * K];
+        __shared__ __attribute__((aligned(16))) float outLds[WAVES][MAX_OUT];
 
         const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
         const uint32_t outStride = K + m * (m - 1) / 2;
-        const uint32_t b0        = blockIdx.x * WAVES;
         const uint32_t inChunks  = m * ROW_CHUNKS;
-        const uint32_t b         = b0 + wave;
+        const uint32_t first     = (blockIdx.x * WAVES + wave) * F32_PER_WAVE; // this wave's first sample
         char*          xw        = reinterpret_cast<char*>(xLds[wave]);
+        float*         o         = outLds[wave];
 
-        if(b < batch)
-        {
-            const char* src = reinterpret_cast<const char*>(in) + (uint64_t)b * m * K * 4u;
-            f32x4       stash[MAX_CHUNKS];
-#pragma unroll
-            for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
+        f32x4 stash[2][MAX_CHUNKS];
+        auto  request = [&](uint32_t b, f32x4 (&dst)[MAX_CHUNKS]) {
+            if(b < batch)
             {
-                const uint32_t c = j * 64u + lane;
-                if(c < inChunks)
-                    stash[j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src + c * 16u));
+                const char* src = reinterpret_cast<const char*>(in) + (uint64_t)b * m * K * 4u;
+#pragma unroll
+                for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
+                {
+                    const uint32_t c = j * 64u + lane;
+                    if(c < inChunks)
+                        dst[j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src + c * 16u));
+                }
             }
+        };
+        auto process = [&](uint32_t b, const f32x4 (&src)[MAX_CHUNKS]) {
+            if(b >= batch)
+                return;
 #pragma unroll
             for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
             {
@@ -206,28 +218,30 @@ namespace
                 if(c < inChunks)
                 {
                     const uint32_t row = c / ROW_CHUNKS, col = c % ROW_CHUNKS;
-                    *reinterpret_cast<f32x4*>(xw + (row * ROW_CHUNKS + (col ^ (row & (ROW_CHUNKS - 1u) & 31u))) * 16u) = stash[j];
+                    *reinterpret_cast<f32x4*>(xw + (row * ROW_CHUNKS + (col ^ (row & SWZ))) * 16u) = src[j];
                 }
             }
             __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_wave_barrier();
 
-            f32x16         acc   = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            // two independent accumulator chains (even / odd k pairs) keep the matrix core pipelined
+            f32x16         acc0  = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            f32x16         acc1  = acc0;
             const bool     valid = (lane & 31u) < m;
             const uint32_t row   = valid ? (lane & 31u) : 0u;
 #pragma unroll 8
-            for(uint32_t s = 0; s < K / 2; ++s)
+            for(uint32_t s = 0; s < K / 4; ++s)
             {
-                const uint32_t kk  = 2u * s + (lane >> 5);
-                const uint32_t col = kk >> 2;
-                float          x   = *reinterpret_cast<const float*>(
-                    xw + (row * ROW_CHUNKS + (col ^ (row & (ROW_CHUNKS - 1u) & 31u))) * 16u + (kk & 3u) * 4u);
+                // lane half h holds k = 4 s + h and 4 s + 2 + h: one 16-byte chunk feeds two instructions
+                const char* src4 = xw + (row * ROW_CHUNKS + (s ^ (row & SWZ))) * 16u + (lane >> 5) * 4u;
+                float       x0   = *reinterpret_cast<const float*>(src4);
+                float       x1   = *reinterpret_cast<const float*>(src4 + 8u);
                 if(!valid)
-                    x = 0.0f;
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x, x, acc, 0, 0, 0);
+                    x0 = 0.0f, x1 = 0.0f;
+                acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(x0, x0, acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(x1, x1, acc1, 0, 0, 0);
             }
 
-            float* o = outLds + wave * outStride;
             for(uint32_t e = lane; e < K; e += 64)
                 o[e] = reinterpret_cast<const float*>(xw)[e]; // row 0 is stored unswizzled
             const uint32_t j = lane & 31u;
@@ -236,23 +250,41 @@ namespace
             {
                 const uint32_t i = 8u * (r >> 2) + 4u * (lane >> 5) + (r & 3u);
                 if(j < i && i < m)
-                    o[K + i * (i - 1u) / 2u + j] = acc[r];
+                    o[K + i * (i - 1u) / 2u + j] = acc0[r] + acc1[r];
             }
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_wave_barrier();
+            float* dst = out + (uint64_t)b * outStride;
+            for(uint32_t e = lane; e < outStride; e += 64)
+                __builtin_nontemporal_store(o[e], dst + e);
+            __builtin_amdgcn_s_waitcnt(0xC07F); // the image is rewritten by the next sample
+            __builtin_amdgcn_wave_barrier();
+        };
+
+        request(first, stash[0]);
+#pragma unroll 1
+        for(uint32_t it = 0; it < F32_PER_WAVE; it += 2)
+        {
+            request(first + it + 1u, stash[1]);
+            process(first + it, stash[0]);
+            if(it + 2u < F32_PER_WAVE)
+                request(first + it + 2u, stash[0]);
+            process(first + it + 1u, stash[1]);
         }
-        __syncthreads();
-        const uint32_t nSamples = (batch - b0) < WAVES ? (batch - b0) : WAVES;
-        const uint32_t total    = nSamples * outStride;
-        float*         dst      = out + (uint64_t)b0 * outStride;
-        const uint32_t vecs     = total / 4u;
-        for(uint32_t v = tid; v < vecs; v += THREADS)
-            __builtin_nontemporal_store(reinterpret_cast<const f32x4*>(outLds)[v], reinterpret_cast<f32x4*>(dst) + v);
-        for(uint32_t e = vecs * 4u + tid; e < total; e += THREADS)
-            dst[e] = outLds[e];
     }
 
-    // Backward: S = T + T^T (T = strict lower triangle from the upstream gradient),
-    // grad(m x k) = S X, computed as acc(i, c) = sum_j S(i, j) X(j, c) per 32-column slab of k.
-    template <bool BF16, uint32_t K>
+    // Backward: S = T + T^T (T = strict lower triangle from the upstream gradient, zero diagonal),
+    // grad (m x k) = S X.  Same organisation as the forward kernel: a workgroup owns 8 consecutive
+    // samples (their upstream rows form one 16-byte aligned run, staged in LDS with 128-bit loads),
+    // a wave owns one sample at a time with the X of both of its samples requested up front.
+    // X sits in LDS as [j][c] rows; the matrix instruction wants X^T (lane = column c, 8
+    // consecutive j), which the transposing LDS read delivers: 16 lanes address a 4 (j) x 16 (c)
+    // block and lane t receives column t.  Per 32-column slab of k: acc(c, i) = sum_j X(j, c) S(j, i),
+    // i.e. every lane ends up with runs of 4 consecutive c of one gradient row i.  The gradient
+    // image replaces X in LDS (rows < m) and leaves with 128-bit nontemporal stores.
+    typedef __fp16 trv4 __attribute__((__vector_size__(4 * sizeof(__fp16))));
+
+    template <bool BF16, uint32_t K, uint32_t ROWS>
     __global__ void __launch_bounds__(THREADS) dlrmBwdKernel(const uint16_t* __restrict__ in,
                                                             const uint16_t* __restrict__ upstream,
                                                             uint16_t* __restrict__ mlpGrad,
@@ -260,71 +292,148 @@ namespace
                                                             uint32_t m,
                                                             uint32_t batch)
     {
-        // S: 32 x 32 elements, row i holds S(i, 0..31) -> K-contiguous operand X-role "A" (32 x 32, K = j)
-        // X^T is needed as the other operand: lane (c = lane % 32, j-run) -> X(j, c) for 8 consecutive j;
-        // X is stored (j, c) row-major in memory, i.e. contiguous along c: keep X in LDS as [j][c]
-        // and gather the 8 values of a lane's j-run with 16-bit LDS reads.
-        __shared__ uint16_t sLds[WAVES][32 * 32];
-        __shared__ uint16_t xLds[WAVES][32 * MAX_K];
+        constexpr uint32_t ROW_CHUNKS = K / 8; // 16-byte chunks per row
+        constexpr uint32_t ROWB       = K * 2;
+        constexpr uint32_t X_BYTES    = MAX_M * ROWB; // always 32 rows: rows >= m stay zero
+        constexpr uint32_t SLABS      = K / 32;
+        constexpr uint32_t MAX_UP     = K + ROWS * (ROWS - 1) / 2;
+        constexpr uint32_t PER_WAVE   = SAMPLES_PER_WG / WAVES;
+        constexpr uint32_t MAX_CHUNKS = (ROWS * ROW_CHUNKS + 63u) / 64u;
+        constexpr uint32_t SWZ_IN     = 12u & (ROW_CHUNKS - 1u); // (j & 3) << 2: four j rows -> four 64-byte groups
+        constexpr uint32_t SWZ_OUT    = 15u & (ROW_CHUNKS - 1u);
+
+        __shared__ __attribute__((aligned(16))) char     xLds[WAVES][X_BYTES];
+        __shared__ __attribute__((aligned(16))) uint16_t upLds[SAMPLES_PER_WG * MAX_UP + 8];
 
         const uint32_t tid      = threadIdx.x;
         const uint32_t lane     = tid & 63u;
         const uint32_t wave     = tid >> 6;
         const uint32_t upStride = K + m * (m - 1) / 2;
-        uint16_t*      sw       = sLds[wave];
-        uint16_t*      xw       = xLds[wave];
+        const uint32_t b0       = blockIdx.x * SAMPLES_PER_WG;
+        const uint32_t inChunks = m * ROW_CHUNKS;
+        char*          xw       = xLds[wave];
 
-        for(uint32_t b = blockIdx.x * WAVES + wave; b < batch; b += gridDim.x * WAVES)
+        i32x4 stash[PER_WAVE][MAX_CHUNKS];
+#pragma unroll
+        for(uint32_t q = 0; q < PER_WAVE; ++q)
         {
-            const uint16_t* up = upstream + (uint64_t)b * upStride;
-            const uint16_t* x  = in + (uint64_t)b * m * K;
-            for(uint32_t e = lane; e < K; e += 64)
-                mlpGrad[(uint64_t)b * K + e] = up[e];
-            // symmetric S with zero diagonal and zero padding
-            for(uint32_t e = lane; e < 32 * 32; e += 64)
+            const uint32_t b = b0 + wave + q * WAVES;
+            if(b < batch)
             {
-                const uint32_t i = e >> 5, j = e & 31u;
-                uint16_t       v = 0;
-                if(i < m && j < m && i != j)
+                const char* src = reinterpret_cast<const char*>(in) + (uint64_t)b * m * K * 2u;
+#pragma unroll
+                for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
                 {
-                    const uint32_t hi = i > j ? i : j, lo = i > j ? j : i;
-                    v                 = up[K + hi * (hi - 1u) / 2u + lo];
+                    const uint32_t c = j * 64u + lane;
+                    if(c < inChunks)
+                        stash[q][j] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(src + c * 16u));
                 }
-                sw[e] = v;
             }
-            for(uint32_t e = lane; e < 32 * K; e += 64)
-                xw[e] = e < m * K ? x[e] : (uint16_t)0;
-            __builtin_amdgcn_s_waitcnt(0xC07F);
+        }
+
+        // ---- upstream rows of the workgroup's samples -> LDS; zero rows m..31 of the X image
+        const uint32_t nSamples = (batch - b0) < SAMPLES_PER_WG ? (batch - b0) : SAMPLES_PER_WG;
+        {
+            const uint32_t  total = nSamples * upStride;
+            const uint16_t* src   = upstream + (uint64_t)b0 * upStride;
+            const uint32_t  vecs  = total / 8u;
+            for(uint32_t v = tid; v < vecs; v += THREADS)
+                reinterpret_cast<i32x4*>(upLds)[v] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(src) + v);
+            for(uint32_t e = vecs * 8u + tid; e < total; e += THREADS)
+                upLds[e] = src[e];
+            for(uint32_t c = inChunks + lane; c < MAX_M * ROW_CHUNKS; c += 64u)
+                *reinterpret_cast<i32x4*>(xw + c * 16u) = i32x4{0, 0, 0, 0};
+        }
+        __syncthreads();
+
+        // ---- bottom-MLP gradient: the first k values of every upstream row
+        for(uint32_t t = tid; t < nSamples * ROW_CHUNKS; t += THREADS)
+        {
+            const uint32_t sIdx = t / ROW_CHUNKS, cc = t % ROW_CHUNKS;
+            union
+            {
+                uint16_t h[8];
+                i32x4    v;
+            } o;
+#pragma unroll
+            for(uint32_t e = 0; e < 8; ++e)
+                o.h[e] = upLds[sIdx * upStride + cc * 8u + e];
+            __builtin_nontemporal_store(o.v, reinterpret_cast<i32x4*>(mlpGrad + ((uint64_t)(b0 + sIdx) * K + cc * 8u)));
+        }
+
+        const uint32_t i = lane & 31u, half = lane >> 5, t16 = lane & 15u;
+#pragma unroll
+        for(uint32_t q = 0; q < PER_WAVE; ++q)
+        {
+            const uint32_t sIdx = wave + q * WAVES;
+            const uint32_t b    = b0 + sIdx;
+            if(b >= batch)
+                break;
+            // ---- X -> LDS: chunk c goes to row j = c / ROW_CHUNKS, slot (c % ROW_CHUNKS) ^ ((j & 3) << 2)
+#pragma unroll
+            for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
+            {
+                const uint32_t c = j * 64u + lane;
+                if(c < inChunks)
+                {
+                    const uint32_t row = c / ROW_CHUNKS, col = c % ROW_CHUNKS;
+                    *reinterpret_cast<i32x4*>(xw + (row * ROW_CHUNKS + (col ^ ((row << 2) & SWZ_IN))) * 16u) = stash[q][j];
+                }
+            }
+            // ---- S operand: lane holds S(i, j) for its 8-wide runs of j (zero diagonal, zero padding)
+            const uint16_t* tril = upLds + sIdx * upStride + K;
+            i32x4           sReg[2];
+#pragma unroll
+            for(uint32_t s = 0; s < 2; ++s)
+            {
+                union
+                {
+                    uint16_t h[8];
+                    i32x4    v;
+                } so;
+#pragma unroll
+                for(uint32_t e = 0; e < 8; ++e)
+                {
+                    const uint32_t j  = 16u * s + 8u * half + e;
+                    const uint32_t hi = i > j ? i : j, lo = i > j ? j : i;
+                    uint16_t       v  = 0;
+                    if(hi < m && hi != lo)
+                        v = tril[hi * (hi - 1u) / 2u + lo];
+                    so.h[e] = v;
+                }
+                sReg[s] = so.v;
+            }
+            __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): this wave's LDS writes are done
             __builtin_amdgcn_wave_barrier();
 
-            const uint32_t idx = lane & 31u, run = 8u * (lane >> 5);
-            for(uint32_t c0 = 0; c0 < K; c0 += 32)
+            f32x16 acc[SLABS];
+#pragma unroll
+            for(uint32_t slab = 0; slab < SLABS; ++slab)
             {
-                f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                acc[slab] = f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-                for(uint32_t s = 0; s < 2; ++s) // j = 16 s + run .. + 7
+                for(uint32_t s = 0; s < 2; ++s)
                 {
-                    // swapped operands: "rows" of the instruction = c, "cols" = i, so that a lane
-                    // ends up with 4 consecutive c of one output row i
-                    union
-                    {
-                        uint16_t h[8];
-                        i32x4    v;
-                    } xo, so;
-#pragma unroll
-                    for(uint32_t e = 0; e < 8; ++e)
-                    {
-                        const uint32_t j = 16u * s + run + e;
-                        xo.h[e]          = xw[j * K + c0 + idx]; // X(j, c0 + idx)
-                        so.h[e]          = sw[idx * 32u + j]; // S(idx, j)
-                    }
-                    acc = mfma16<BF16>(acc, xo.v, so.v);
+                    using lp             = __attribute__((address_space(3))) trv4*;
+                    const uint32_t row   = 16u * s + 8u * half + (t16 >> 2);
+                    const uint32_t piece = 8u * slab + 4u * ((lane >> 4) & 1u) + (t16 & 3u); // 8-byte pieces
+                    const char*    p0    = xw + row * ROWB + (((piece >> 1) ^ ((row << 2) & SWZ_IN)) * 16u) + (piece & 1u) * 8u;
+                    using i32x2          = int __attribute__((ext_vector_type(2)));
+                    const i32x2 lo = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lp)p0));
+                    const i32x2 hi = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lp)(p0 + 4u * ROWB)));
+                    acc[slab]      = mfma16<BF16>(acc[slab], i32x4{lo[0], lo[1], hi[0], hi[1]}, sReg[s]);
                 }
-                // lane: i = idx, c = c0 + 8 (r / 4) + 4 (lane / 32) + r % 4
-                if(idx < m)
-                {
+            }
+            __builtin_amdgcn_s_waitcnt(0xC07F); // every read of X has returned before rows are overwritten
+            __builtin_amdgcn_wave_barrier();
+
+            // ---- gradient image over rows < m: lane has c = 32 slab + 8 r + 4 half + (0..3) of row i
+            if(i < m)
+            {
 #pragma unroll
-                    for(uint32_t q = 0; q < 4; ++q)
+                for(uint32_t slab = 0; slab < SLABS; ++slab)
+#pragma unroll
+                    for(uint32_t r = 0; r < 4; ++r)
                     {
                         union
                         {
@@ -333,12 +442,27 @@ namespace
                         } o;
 #pragma unroll
                         for(uint32_t e = 0; e < 4; ++e)
-                            o.h[e] = roundOut<BF16>(acc[4 * q + e]);
-                        const uint32_t c = c0 + 8u * q + 4u * (lane >> 5);
-                        *reinterpret_cast<uint64_t*>(inGrad + (uint64_t)b * m * K + idx * K + c) = o.v;
+                            o.h[e] = roundOut<BF16>(acc[slab][4 * r + e]);
+                        const uint32_t chunk = 4u * slab + r;
+                        *reinterpret_cast<uint64_t*>(xw + i * ROWB + ((chunk ^ (i & SWZ_OUT)) * 16u) + half * 8u) = o.v;
                     }
+            }
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_wave_barrier();
+
+            char* dst = reinterpret_cast<char*>(inGrad) + (uint64_t)b * m * K * 2u;
+#pragma unroll
+            for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
+            {
+                const uint32_t c = j * 64u + lane;
+                if(c < inChunks)
+                {
+                    const uint32_t row = c / ROW_CHUNKS, col = c % ROW_CHUNKS;
+                    const i32x4    v   = *reinterpret_cast<const i32x4*>(xw + (row * ROW_CHUNKS + (col ^ (row & SWZ_OUT))) * 16u);
+                    __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(dst + c * 16u));
                 }
             }
+            __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_wave_barrier();
         }
     }
@@ -372,15 +496,25 @@ extern "C" int r355_dlrm_fwd(int32_t dtype, const void* in, void* out, uint32_t 
     hipStream_t s = static_cast<hipStream_t>(stream);
     if(dtype == R355_F32)
     {
-        const dim3 grid32((batch + WAVES - 1) / WAVES), block32(THREADS);
+        const uint32_t perWg = WAVES * F32_PER_WAVE;
+        const dim3     grid32((batch + perWg - 1) / perWg), block32(THREADS);
         auto*      fi = static_cast<const float*>(in);
         auto*      fo = static_cast<float*>(out);
+#define R355_FWD32(KK)                                                                                \
+    do                                                                                                \
+    {                                                                                                 \
+        if(m <= 28)                                                                                   \
+            hipLaunchKernelGGL((dlrmFwdF32Kernel<KK, 28>), grid32, block32, 0, s, fi, fo, m, batch);  \
+        else                                                                                          \
+            hipLaunchKernelGGL((dlrmFwdF32Kernel<KK, 32>), grid32, block32, 0, s, fi, fo, m, batch);  \
+    } while(0)
         switch(k)
         {
-        case 32: hipLaunchKernelGGL(dlrmFwdF32Kernel<32>, grid32, block32, 0, s, fi, fo, m, batch); break;
-        case 64: hipLaunchKernelGGL(dlrmFwdF32Kernel<64>, grid32, block32, 0, s, fi, fo, m, batch); break;
-        default: hipLaunchKernelGGL(dlrmFwdF32Kernel<128>, grid32, block32, 0, s, fi, fo, m, batch); break;
+        case 32: R355_FWD32(32); break;
+        case 64: R355_FWD32(64); break;
+        default: R355_FWD32(128); break;
         }
+#undef R355_FWD32
         return r355::checkLaunch("dlrm_fwd");
     }
     const dim3 grid((batch + SAMPLES_PER_WG - 1) / SAMPLES_PER_WG), block(THREADS);
@@ -423,14 +557,22 @@ extern "C" int r355_dlrm_bwd(int32_t dtype, const void* in, const void* upstream
         return rc;
     if(!upstream || !mlp_grad)
         return r355::fail(R355_ERR_BAD_ARG, "dlrm_bwd: null pointer");
-    const uint32_t wgs = (batch + WAVES - 1) / WAVES;
-    const dim3     grid(wgs < 4096 ? wgs : 4096), block(THREADS);
-    hipStream_t    s  = static_cast<hipStream_t>(stream);
-    auto*          pi = static_cast<const uint16_t*>(in);
-    auto*          pu = static_cast<const uint16_t*>(upstream);
-    auto*          pm = static_cast<uint16_t*>(mlp_grad);
-    auto*          pg = static_cast<uint16_t*>(in_grad);
-#define R355_BWD(BF, KK) hipLaunchKernelGGL((dlrmBwdKernel<BF, KK>), grid, block, 0, s, pi, pu, pm, pg, m, batch)
+    if(!r355::aligned(upstream, 16) || !r355::aligned(mlp_grad, 16))
+        return r355::fail(R355_ERR_MISALIGNED, "dlrm_bwd: upstream and mlp_grad must be 16-byte aligned");
+    const dim3  grid((batch + SAMPLES_PER_WG - 1) / SAMPLES_PER_WG), block(THREADS);
+    hipStream_t s  = static_cast<hipStream_t>(stream);
+    auto*       pi = static_cast<const uint16_t*>(in);
+    auto*       pu = static_cast<const uint16_t*>(upstream);
+    auto*       pm = static_cast<uint16_t*>(mlp_grad);
+    auto*       pg = static_cast<uint16_t*>(in_grad);
+#define R355_BWD(BF, KK)                                                                                          \
+    do                                                                                                            \
+    {                                                                                                             \
+        if(m <= 28)                                                                                               \
+            hipLaunchKernelGGL((dlrmBwdKernel<BF, KK, 28>), grid, block, 0, s, pi, pu, pm, pg, m, batch);          \
+        else                                                                                                      \
+            hipLaunchKernelGGL((dlrmBwdKernel<BF, KK, 32>), grid, block, 0, s, pi, pu, pm, pg, m, batch);          \
+    } while(0)
 #define R355_BWD_K(BF)   \
     switch(k)            \
     {                    \
@@ -441,11 +583,11 @@ extern "C" int r355_dlrm_bwd(int32_t dtype, const void* in, const void* upstream
     }
     if(dtype == R355_BF16)
     {
-        R355_BWD_K(true)
+        R355_BWD_K(true);
     }
     else
     {
-        R355_BWD_K(false)
+        R355_BWD_K(false);
     }
 #undef R355_BWD_K
 #undef R355_BWD

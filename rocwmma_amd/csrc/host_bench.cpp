@@ -6,7 +6,7 @@
 //   host_bench gemm  [--type f16|bf16|i8|e4m3] [--out f16|bf16|f32|i32] [--layout nt|tn|nn|tt]
 //                    [--m M --n N --k K] [--kernel auto|simple|tiled] [--warmup W --iters I]
 //                    [--sparse 1]   A is 2:4 structured sparse (compressed values + index nibbles)
-//   host_bench dlrm  [--type f16|bf16|f32] [--batch B --m M --k K] [--warmup W --iters I]
+//   host_bench dlrm  [--type f16|bf16|f32] [--bwd 1] [--batch B --m M --k K] [--warmup W --iters I]
 //   host_bench gemv  [--m M --k K --layout n|t]
 //   host_bench copy  [--bytes N]      plain device copy of known size (counter calibration)
 //   host_bench mfma  [--iters I]      register-resident MFMA loops, one wave per SIMD, 16 independent
@@ -179,7 +179,7 @@ int main(int argc, char** argv)
     }
     const std::string op = argv[1];
     std::string       type = "f16", out = "", layout = "nt", kernel = "auto";
-    bool              sparse = false, itersSet = false;
+    bool              sparse = false, itersSet = false, bwd = false;
     uint32_t          m = 8192, n = 8192, k = 8192, batch = 65536;
     bool              mSet = false, kSet = false;
     int               warmup = 2, iters = 10;
@@ -198,6 +198,7 @@ int main(int argc, char** argv)
         else if(a == "--warmup") warmup = atoi(v.c_str());
         else if(a == "--iters") iters = atoi(v.c_str()), itersSet = true;
         else if(a == "--sparse") sparse = atoi(v.c_str()) != 0;
+        else if(a == "--bwd") bwd = atoi(v.c_str()) != 0;
         else if(a == "--bytes") bytes = strtoull(v.c_str(), nullptr, 10);
         else
         {
@@ -284,6 +285,39 @@ int main(int argc, char** argv)
         HIP_OK(hipMalloc(&dx, hx.size()));
         HIP_OK(hipMalloc(&dout, outElems * es));
         HIP_OK(hipMemcpy(dx, hx.data(), hx.size(), hipMemcpyHostToDevice));
+        if(bwd)
+        {
+            // upstream gradient has the forward output's shape; outputs: mlp gradient [batch][k]
+            // and input gradient [batch][m][k]
+            std::vector<uint8_t> hu(outElems * es);
+            fillBytes(hu, dt, 9);
+            void *dmlp, *dgrad;
+            HIP_OK(hipMemcpy(dout, hu.data(), hu.size(), hipMemcpyHostToDevice));
+            HIP_OK(hipMalloc(&dmlp, (size_t)batch * k * es));
+            HIP_OK(hipMalloc(&dgrad, inElems * es));
+            hipEvent_t e0, e1;
+            HIP_OK(hipEventCreate(&e0));
+            HIP_OK(hipEventCreate(&e1));
+            for(int i = 0; i < warmup + iters; ++i)
+            {
+                if(i == warmup)
+                    HIP_OK(hipEventRecord(e0));
+                if(r355_dlrm_bwd(dt, dx, dout, dmlp, dgrad, m, k, batch, nullptr) != R355_OK)
+                {
+                    fprintf(stderr, "%s\n", r355_last_error());
+                    return 1;
+                }
+            }
+            HIP_OK(hipEventRecord(e1));
+            HIP_OK(hipEventSynchronize(e1));
+            HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+            ms /= iters;
+            const double byts = (double)(2 * inElems + outElems + (size_t)batch * k) * es;
+            printf("{\"op\": \"dlrm_bwd\", \"type\": \"%s\", \"batch\": %u, \"m\": %u, \"k\": %u, \"ms\": %.4f, \"gbps\": %.1f, "
+                   "\"frac_hbm_peak\": %.4f}\n",
+                   type.c_str(), batch, m, k, ms, byts / ms / 1e6, byts / ms / 1e6 / 8000.0);
+            return 0;
+        }
         if(r355_dlrm_fwd_timed(dt, dx, dout, m, k, batch, nullptr, warmup, iters, &ms) != R355_OK)
         {
             fprintf(stderr, "%s\n", r355_last_error());

@@ -145,3 +145,38 @@ def test_bwd_reference_fixture(suffix):
     omlp, ograd = O.dlrm_bwd(O.F16, x, up, 27, 128, 64)
     ok, mx = O.compare(O.F16, got, ograd.ravel(), 10.0)
     assert ok, mx
+
+
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16])
+@pytest.mark.parametrize("m,k,batch", [(27, 128, 13), (32, 128, 8), (32, 32, 64), (2, 64, 5), (17, 256, 9), (28, 128, 1),
+                                       (29, 64, 17)])
+def test_bwd_shapes_vs_oracle(dtype, m, k, batch):
+    """Ragged batches (not a multiple of the 8 samples a workgroup owns), both row bounds (m <= 28, m > 28),
+    every supported k; padding bytes after both outputs must stay untouched."""
+    stride = k + m * (m - 1) // 2
+    x = O.f32_to_storage(O.normal(5, batch * m * k) * 0.5, dtype)
+    up = O.f32_to_storage(O.normal(6, batch * stride) * 0.5, dtype)
+    want_mlp, want = O.dlrm_bwd(dtype, x, up, m, k, batch)
+    dx, dup = to_device(x), to_device(up)
+    dmlp = device_filled(batch * k + 8, np.uint16, 0xEE)
+    dgrad = device_filled(batch * m * k + 8, np.uint16, 0xEE)
+    R.dlrm_bwd(R.F16 if dtype == O.F16 else R.BF16, dx, dup, dmlp, dgrad, m, k, batch)
+    mlp, grad = to_host(dmlp, np.uint16), to_host(dgrad, np.uint16)
+    assert np.all(mlp[batch * k:] == 0xEEEE) and np.all(grad[batch * m * k:] == 0xEEEE)
+    assert np.array_equal(mlp[:batch * k], want_mlp.ravel())
+    ok, mx = O.compare(dtype, grad[:batch * m * k], want.ravel(), 10.0)  # the reference's DLRM tolerance
+    assert ok, mx
+
+
+def test_bwd_integer_inputs_exact():
+    """Small integers: every product and partial sum is exact, so any summation order gives the oracle's bits."""
+    m, k, batch = 27, 128, 24
+    stride = k + m * (m - 1) // 2
+    x = O.f32_to_storage(np.round(O.uniform_pm1(7, batch * m * k) * 3.0), O.F16)
+    up = O.f32_to_storage(np.round(O.uniform_pm1(8, batch * stride) * 3.0), O.F16)
+    want_mlp, want = O.dlrm_bwd(O.F16, x, up, m, k, batch)
+    dx, dup = to_device(x), to_device(up)
+    dmlp, dgrad = device_filled(batch * k, np.uint16), device_filled(batch * m * k, np.uint16)
+    R.dlrm_bwd(R.F16, dx, dup, dmlp, dgrad, m, k, batch)
+    assert np.array_equal(to_host(dmlp, np.uint16), want_mlp.ravel())
+    assert np.array_equal(to_host(dgrad, np.uint16), want.ravel())
