@@ -213,3 +213,46 @@ def test_full_size_8192_sampled_rows(in_t, out_t, la, lb):
         assert np.max(np.abs(gs - colsum) / scale) < (2e-3 if in_t != O.E4M3 else 1e-3)
     del da, db, dd
     torch.cuda.empty_cache()
+
+
+def _embed(flat, rows, cols, layout, ld, fill):
+    """Packed rows x cols matrix (layout) -> storage with leading dimension ld, padding = fill."""
+    major, minor = (rows, cols) if layout == O.ROW else (cols, rows)
+    out = np.full(major * ld, fill, dtype=flat.dtype)
+    out.reshape(major, ld)[:, :minor] = flat.reshape(major, minor)
+    return out
+
+
+@pytest.mark.parametrize("kernel", ["tiled", "simple"])
+@pytest.mark.parametrize("in_t,out_t,la,lb,ldl", [(O.F16, O.F16, O.COL, O.ROW, O.ROW), (O.F16, O.F32, O.ROW, O.COL, O.COL),
+                                                  (O.BF16, O.BF16, O.ROW, O.ROW, O.ROW), (O.I8, O.I32, O.ROW, O.COL, O.ROW),
+                                                  (O.E4M3, O.F32, O.ROW, O.COL, O.COL)])
+def test_padded_leading_dimensions(kernel, in_t, out_t, la, lb, ldl):
+    """Operands and result embedded in wider buffers (ld > extent): the reference kernels take lda..ldd
+    (test/gemm/gemm_kernel_base.hpp:101-114); bytes outside the m x n block of D must stay untouched."""
+    m, n, k = (256, 512, 512) if kernel == "tiled" else (96, 64, 128)
+    a, b, c = _inputs(in_t, out_t, m, n, k, seed=41)
+    alpha, beta = (1.0, 1.0) if in_t in (O.I8, O.E4M3) else (2.0, -1.0)
+    want = O.gemm(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, c, alpha, beta)
+    es_in, es_out = a.dtype.itemsize, c.dtype.itemsize
+    pad_in, pad_out = 48 // es_in * 2, 32 // es_out * 2  # keeps 16-byte alignment of every row / column
+    lda = (k if la == O.ROW else m) + pad_in
+    ldb = (n if lb == O.ROW else k) + pad_in
+    ldc = (n if ldl == O.ROW else m) + pad_out
+    ldd = ldc + pad_out
+    canary = np.array([0xEE] * es_out, dtype=np.uint8).view(c.dtype)[0]
+    ea, eb = _embed(a, m, k, la, lda, 1), _embed(b, k, n, lb, ldb, 1)
+    ec = _embed(c, m, n, ldl, ldc, canary)
+    da, db, dc = to_device(ea), to_device(eb), to_device(ec)
+    major = m if ldl == O.ROW else n
+    dd = device_filled(major * ldd, O.NP_STORAGE[out_t], 0xEE)
+    R.gemm(in_t, out_t, m, n, k, da, db, dc, dd, alpha, beta, la, lb, ldl, ldl, lda=lda, ldb=ldb, ldc=ldc, ldd=ldd,
+           kernel=R.KERNEL_TILED if kernel == "tiled" else R.KERNEL_SIMPLE)
+    full = to_host(dd, O.NP_STORAGE[out_t]).reshape(major, ldd)
+    minor = n if ldl == O.ROW else m
+    assert np.all(full[:, minor:] == canary)
+    got = np.ascontiguousarray(full[:, :minor]).ravel()
+    w32 = None
+    if out_t in (O.F16, O.BF16):
+        w32 = O.gemm(in_t, O.F32, la, lb, ldl, ldl, m, n, k, a, b, O.storage_to_f32(c, out_t), alpha, beta)
+    _check(in_t, out_t, got, want, w32)
