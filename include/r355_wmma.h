@@ -40,7 +40,8 @@ typedef enum
     R355_E4M3 = 2, /* OCP FP8 E4M3 (gfx950 native)       */
     R355_I8   = 3, /* signed 8-bit integer               */
     R355_F32  = 4,
-    R355_I32  = 5
+    R355_I32  = 5,
+    R355_F64  = 6 /* GEMM f64 -> f64 on the block-per-wave kernel only */
 } r355_dtype;
 
 /* memory orientation; BLAS letters: row-major = "T", col-major = "N" for A (m x k) */

@@ -46,7 +46,7 @@
 #include <omp.h>
 #endif
 
-enum { ORC_F16 = 0, ORC_BF16 = 1, ORC_E4M3 = 2, ORC_I8 = 3, ORC_F32 = 4, ORC_I32 = 5 };
+enum { ORC_F16 = 0, ORC_BF16 = 1, ORC_E4M3 = 2, ORC_I8 = 3, ORC_F32 = 4, ORC_I32 = 5, ORC_F64 = 6 };
 enum { ORC_ROW_MAJOR = 0, ORC_COL_MAJOR = 1 };
 
 /* ---------------------------------------------------------------- scalars */
@@ -244,7 +244,7 @@ static inline size_t mat_index(uint32_t row, uint32_t col, uint32_t ld, int layo
  * multiply, and the epilogue alpha*accum + beta*C is rounded once to the
  * output type (lines 76-77).  Rows are spread over OpenMP threads (line 65).
  *
- * Floating inputs (f16, bf16, e4m3, f32) compute in f32; int8 computes in
+ * Floating inputs (f16, bf16, e4m3, f32) compute in f32, f64 in f64; int8 computes in
  * int32 with int32 alpha/beta passed as integers-in-float.  Returns 0, or
  * -1 for an unsupported type combination.
  */
@@ -294,6 +294,30 @@ int orc_gemm(int         in_type,
                     = (int32_t)((uint32_t)ia * (uint32_t)accum
                                 + (uint32_t)ib
                                       * (uint32_t)pc[mat_index((uint32_t)i, j, ldc, layout_c)]);
+            }
+        }
+        return 0;
+    }
+
+    if(in_type == ORC_F64)
+    {
+        /* f64 in, f64 compute, f64 out (the reference's dgemm instantiation) */
+        const double* pa = (const double*)a;
+        const double* pb = (const double*)b;
+        const double* pc = (const double*)c;
+        double*       pd = (double*)d;
+        if(out_type != ORC_F64)
+            return -1;
+#pragma omp parallel for schedule(static)
+        for(int64_t i = 0; i < (int64_t)m; ++i)
+        {
+            for(uint32_t j = 0; j < n; ++j)
+            {
+                double accum = 0.0;
+                for(uint32_t h = 0; h < k; ++h)
+                    accum += pa[mat_index((uint32_t)i, h, lda, layout_a)] * pb[mat_index(h, j, ldb, layout_b)];
+                pd[mat_index((uint32_t)i, j, ldd, layout_d)]
+                    = (double)alpha * accum + (double)beta * pc[mat_index((uint32_t)i, j, ldc, layout_c)];
             }
         }
         return 0;
@@ -513,14 +537,17 @@ int orc_compare(
     case ORC_E4M3:
         eps = 0.125;
         break; /* float8.hpp:549-580: epsilon code 0x20 = 2^-3 */
+    case ORC_F64:
+        eps = 2.220446049250313e-16;
+        break;
     default:
         return -1;
     }
 #pragma omp parallel for reduction(max : mx) reduction(| : is_inf, is_nan)
     for(int64_t i = 0; i < (int64_t)count; ++i)
     {
-        double a   = (double)load_as_f32(x, (size_t)i, dtype);
-        double b   = (double)load_as_f32(y, (size_t)i, dtype);
+        double a   = dtype == ORC_F64 ? ((const double*)x)[i] : (double)load_as_f32(x, (size_t)i, dtype);
+        double b   = dtype == ORC_F64 ? ((const double*)y)[i] : (double)load_as_f32(y, (size_t)i, dtype);
         double num = fabs(a - b);
         double den = fabs(a) + fabs(b) + 1.0;
         if(isinf(num) || isinf(den))
@@ -582,6 +609,9 @@ int orc_fill_ref(int dtype, void* mat, uint32_t m, uint32_t n, int layout)
                 break;
             case ORC_I32:
                 ((int32_t*)mat)[idx] = -v;
+                break;
+            case ORC_F64:
+                ((double*)mat)[idx] = (double)fv;
                 break;
             default:
                 return -1;

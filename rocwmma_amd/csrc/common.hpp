@@ -25,6 +25,7 @@ namespace r355
         case R355_I8: return 1;
         case R355_F32:
         case R355_I32: return 4;
+        case R355_F64: return 8;
         default: return 0;
         }
     }

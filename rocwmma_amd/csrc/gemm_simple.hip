@@ -99,7 +99,7 @@ namespace
         else if constexpr(sizeof(InT) == 1)
             return Blk == 32 ? 16 : 32;
         else
-            return Blk == 32 ? 2 : 4;
+            return Blk == 32 ? 2 : 4; // f32; f64 exists for 16 x 16 blocks only (K 4)
     }
 
     template <typename InT, typename OutT, typename CompT, typename LayoutA, typename LayoutB, uint32_t Blk>
@@ -147,8 +147,11 @@ namespace
     template <typename InT, typename OutT, typename CompT>
     int launchBlocks(const r355_gemm_args& g, hipStream_t stream, uint32_t blk)
     {
-        return blk == 32 ? launchLayouts<InT, OutT, CompT, 32>(g, stream)
-                         : launchLayouts<InT, OutT, CompT, 16>(g, stream);
+        if constexpr(std::is_same_v<InT, float64_t>)
+            return launchLayouts<InT, OutT, CompT, 16>(g, stream);
+        else
+            return blk == 32 ? launchLayouts<InT, OutT, CompT, 32>(g, stream)
+                             : launchLayouts<InT, OutT, CompT, 16>(g, stream);
     }
 
     uint32_t kGranule(int32_t inType, uint32_t blk)
@@ -160,6 +163,7 @@ namespace
         case R355_I8: return 32;
         case R355_E4M3: return blk == 32 ? 16 : 32;
         case R355_F32: return blk == 32 ? 2 : 4;
+        case R355_F64: return 4;
         default: return 0;
         }
     }
@@ -167,12 +171,12 @@ namespace
     // Widest vector a fragment access may use: pointers and leading dimensions must keep it aligned
     uint32_t vectorBytes(int32_t inType)
     {
-        return inType == R355_F32 ? 4 : (inType == R355_I8 ? 16 : 16);
+        return inType == R355_F32 ? 4 : (inType == R355_F64 ? 8 : 16);
     }
 
     uint32_t pickBlock(const r355_gemm_args& g)
     {
-        if(g.m % 32 == 0 && g.n % 32 == 0 && g.k % kGranule(g.in_type, 32) == 0)
+        if(g.in_type != R355_F64 && g.m % 32 == 0 && g.n % 32 == 0 && g.k % kGranule(g.in_type, 32) == 0)
             return 32;
         if(g.m % 16 == 0 && g.n % 16 == 0 && g.k % kGranule(g.in_type, 16) == 0)
             return 16;
@@ -188,6 +192,7 @@ namespace
         case R355_E4M3: return out == R355_F32;
         case R355_I8: return out == R355_I32;
         case R355_F32: return out == R355_F32;
+        case R355_F64: return out == R355_F64;
         default: return false;
         }
     }
@@ -208,8 +213,10 @@ namespace r355
         const uint32_t eb = dtypeBytes(g.in_type), ob = dtypeBytes(g.out_type);
         const uint32_t va = g.layout_a == R355_ROW_MAJOR ? vectorBytes(g.in_type) : eb;
         const uint32_t vb = g.layout_b == R355_COL_MAJOR ? vectorBytes(g.in_type) : eb;
-        const uint32_t vd = g.layout_d == R355_COL_MAJOR ? 4 * ob : ob;
-        const uint32_t vc = g.layout_c == R355_COL_MAJOR ? 4 * ob : ob;
+        // accumulator fragments hold 4 consecutive rows per lane (f64: one row per register)
+        const uint32_t accRun = g.out_type == R355_F64 ? 1u : 4u;
+        const uint32_t vd = g.layout_d == R355_COL_MAJOR ? accRun * ob : ob;
+        const uint32_t vc = g.layout_c == R355_COL_MAJOR ? accRun * ob : ob;
         if(!aligned(g.a, va) || (g.lda * eb) % va || !aligned(g.b, vb) || (g.ldb * eb) % vb
            || !aligned(g.d, vd) || (g.ldd * ob) % vd
            || (g.beta != 0.0f && (!aligned(g.c, vc) || (g.ldc * ob) % vc)))
@@ -243,6 +250,7 @@ namespace r355
         case R355_E4M3: return launchBlocks<float8_t, float32_t, float32_t>(g, stream, blk);
         case R355_I8: return launchBlocks<int8_t, int32_t, int32_t>(g, stream, blk);
         case R355_F32: return launchBlocks<float32_t, float32_t, float32_t>(g, stream, blk);
+        case R355_F64: return launchBlocks<float64_t, float64_t, float64_t>(g, stream, blk);
         default: return fail(R355_ERR_UNSUPPORTED, "gemm: unknown in_type %d", g.in_type);
         }
     }

@@ -22,7 +22,8 @@
 //   int8      : KW 16 -> v_mfma_i32_32x32x32 / 16x16x64, KW 8 -> 32x32x16 / 16x16x32
 //   fp8 e4m3  : KW 8 -> v_mfma_f32_32x32x16 / 16x16x32 (fp8_fp8)
 //   f32       : KW 1 -> v_mfma_f32_32x32x2 / 16x16x4
-// Accumulators use KW 4, which is the MFMA C/D layout
+//   f64       : KW 1 -> v_mfma_f64_16x16x4 (BlockDim 16 only)
+// Accumulators use KW 4, which is the MFMA C/D layout (f64: KW 1, row = 4 e + lane / 16)
 //   (32x32: col = l % 32, row = 8 * (e / 4) + 4 * (l / 32) + e % 4;
 //    16x16: col = l % 16, row = 4 * (l / 16) + e)
 // for every element type, so `fragC.x[i]` and `fragAcc.x[i]` always name the same (row, col).
@@ -116,8 +117,10 @@ namespace rocwmma
             static constexpr uint32_t D    = cmin(BlockDim, WaveSize);
             static constexpr uint32_t G    = WaveSize / D;
             static constexpr uint32_t Segs = BlockDim / D;
+            // f64 accumulators follow v_mfma_f64_16x16x4: one row per register, rows G apart
             static constexpr uint32_t KW
-                = IsAcc ? 4u : inputKW<DataT>(KDim, G, BlockDim == 16u || BlockDim == 32u);
+                = IsAcc ? (sizeof(DataT) == 8u ? 1u : 4u)
+                        : inputKW<DataT>(KDim, G, BlockDim == 16u || BlockDim == 32u);
 
             static_assert(KDim % (KW * G) == 0u,
                           "KDim is not a multiple of the K extent one wave holds per register chunk");

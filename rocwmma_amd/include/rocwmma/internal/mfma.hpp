@@ -9,6 +9,7 @@
 //   int8 16/lane: v_mfma_i32_32x32x32_i8    / 16x16x64_i8     8/lane: 32x32x16_i8 / 16x16x32_i8
 //   e4m3  8/lane: v_mfma_f32_32x32x16_fp8_fp8 / 16x16x32_fp8_fp8   (OCP encoding on gfx950)
 //   f32   1/lane: v_mfma_f32_32x32x2f32     / 16x16x4f32
+//   f64   1/lane: v_mfma_f64_16x16x4f64 (16x16 blocks only)
 #ifndef ROCWMMA_MFMA_HPP
 #define ROCWMMA_MFMA_HPP
 
@@ -30,7 +31,10 @@ namespace rocwmma
         {
             static_assert(BlockDim == 16u || BlockDim == 32u, "MFMA blocks are 16x16 or 32x32");
 
-            using AccT = std::conditional_t<is_i8_v<InputT>, acc_i32_t<BlockDim>, acc_f32_t<BlockDim>>;
+            using AccT = std::conditional_t<
+                is_i8_v<InputT>,
+                acc_i32_t<BlockDim>,
+                std::conditional_t<std::is_same_v<InputT, float64_t>, vec_t<double, 4>, acc_f32_t<BlockDim>>>;
 
             ROCWMMA_DEVICE static inline void exec(AccT& acc, InputT const* a, InputT const* b)
             {
@@ -116,6 +120,11 @@ namespace rocwmma
                         acc = __builtin_amdgcn_mfma_f32_32x32x2f32(*a, *b, acc, 0, 0, 0);
                     else
                         acc = __builtin_amdgcn_mfma_f32_16x16x4f32(*a, *b, acc, 0, 0, 0);
+                }
+                else if constexpr(std::is_same_v<InputT, float64_t> && KW == 1u)
+                {
+                    static_assert(BlockDim == 16u, "f64 matrix instructions exist for 16x16 blocks only");
+                    acc = __builtin_amdgcn_mfma_f64_16x16x4f64(*a, *b, acc, 0, 0, 0);
                 }
                 else
                 {

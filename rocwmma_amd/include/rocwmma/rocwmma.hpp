@@ -302,7 +302,9 @@ namespace rocwmma
                       "A and B register layouts must mirror each other");
         using Op   = detail::MfmaChunk<InputT, BlockM, LayoutAReg::KW>;
         using AccT = typename Op::AccT;
-        using AccE = std::conditional_t<detail::is_i8_v<InputT>, int32_t, float32_t>;
+        using AccE = std::conditional_t<detail::is_i8_v<InputT>,
+                                        int32_t,
+                                        std::conditional_t<std::is_same_v<InputT, float64_t>, float64_t, float32_t>>;
         constexpr uint32_t AccN = BlockM == 32u ? 16u : 4u;
 
         AccT acc;

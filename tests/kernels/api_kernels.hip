@@ -213,7 +213,11 @@ namespace
     X(86, accumulator, 16, 16, 16, int32_t, row_major)                                 \
     X(87, accumulator, 16, 16, 16, int32_t, col_major)                                 \
     X(88, accumulator, 16, 256, 16, float16_t, row_major)                              \
-    X(89, accumulator, 16, 256, 16, float16_t, col_major)
+    X(89, accumulator, 16, 256, 16, float16_t, col_major)                              \
+    X(90, matrix_a, 16, 16, 16, float64_t, row_major)                                  \
+    X(91, matrix_b, 16, 16, 16, float64_t, row_major)                                  \
+    X(92, accumulator, 16, 16, 16, float64_t, col_major)                               \
+    X(93, matrix_a, 64, 16, 8, float64_t, col_major)
 
 extern "C" {
 
@@ -338,7 +342,7 @@ int api_relayout_store(const void* in, void* out, uint32_t ldIn, uint32_t ldOut)
     return hipDeviceSynchronize() == hipSuccess ? 0 : -2;
 }
 
-// one tile D = A B + C.  type: 0 f16, 1 bf16, 2 e4m3, 3 i8, 4 f32; blk 16 | 32; bk per the table in the test
+// one tile D = A B + C.  type: 0 f16, 1 bf16, 2 e4m3, 3 i8, 4 f32, 5 f16 accumulate, 6 f64; blk 16 | 32; bk per the table in the test
 int api_mma_tile(int type, uint32_t blk, uint32_t bk, int aRow, int bRow, int cRow, const void* a, const void* b,
                  const void* c, void* d, uint32_t lda, uint32_t ldb, uint32_t ldc)
 {
@@ -377,6 +381,7 @@ int api_mma_tile(int type, uint32_t blk, uint32_t bk, int aRow, int bRow, int cR
     case 3: SHAPE(int8_t, int32_t, 16, 32, 16, 64, 32, 16, 32, 32); break;
     case 4: SHAPE(float32_t, float32_t, 16, 4, 16, 16, 32, 2, 32, 8); break;
     case 5: SHAPE(float16_t, float16_t, 16, 16, 16, 32, 32, 8, 32, 16); break; // 16-bit accumulate type
+    case 6: SHAPE(float64_t, float64_t, 16, 4, 16, 8, 16, 16, 16, 32); break;
     default: return -1;
     }
     return hipDeviceSynchronize() == hipSuccess ? 0 : -2;

@@ -12,10 +12,11 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _ORACLE_DIR = os.path.join(os.path.dirname(_HERE), "oracle")
 
-F16, BF16, E4M3, I8, F32, I32 = range(6)
+F16, BF16, E4M3, I8, F32, I32, F64 = range(7)
 ROW, COL = 0, 1  # row_major ("T" in BLAS letters), col_major ("N")
 
-NP_STORAGE = {F16: np.uint16, BF16: np.uint16, E4M3: np.uint8, I8: np.int8, F32: np.float32, I32: np.int32}
+NP_STORAGE = {F16: np.uint16, BF16: np.uint16, E4M3: np.uint8, I8: np.int8, F32: np.float32, I32: np.int32,
+              F64: np.float64}
 
 _lib = None
 
@@ -156,6 +157,8 @@ def f32_to_storage(x, dtype):
         return x
     if dtype == I32:
         return x.astype(np.int32)
+    if dtype == F64:
+        return x.astype(np.float64)
     raise ValueError(dtype)
 
 

@@ -14,7 +14,7 @@ from gpuutil import api_lib, device_filled, to_device, to_host
 
 pytestmark = pytest.mark.gpu
 
-CASES = list(range(90))
+CASES = list(range(94))
 
 
 def _info(cid):
@@ -24,7 +24,7 @@ def _info(cid):
 
 
 def _np_dtype(eb):
-    return {1: np.uint8, 2: np.uint16, 4: np.uint32}[eb]
+    return {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[eb]
 
 
 def _padded(rows, cols, eb, row_major, pad, seed):
@@ -34,6 +34,8 @@ def _padded(rows, cols, eb, row_major, pad, seed):
     vals = (np.arange(R_ * C_, dtype=np.uint64) * 2654435761 + seed) % (1 << (8 * eb) - 1)
     if eb == 4:
         vals = vals % (1 << 22)  # keep f32 patterns finite
+    if eb == 8:
+        vals = vals % (1 << 52)
     mat = vals.astype(dt).reshape(R_, C_)
     ld = C_ if row_major else R_
     off = pad * ld + pad
@@ -150,10 +152,11 @@ def test_mapping_util_coordinates():
                     assert out[w, 6] == mat[0] * ld + mat[1] and out[w, 7] == out[w, 6]
 
 
-TYPES = {0: (O.F16, O.F32), 1: (O.BF16, O.F32), 2: (O.E4M3, O.F32), 3: (O.I8, O.I32), 4: (O.F32, O.F32), 5: (O.F16, O.F16)}
+TYPES = {0: (O.F16, O.F32), 1: (O.BF16, O.F32), 2: (O.E4M3, O.F32), 3: (O.I8, O.I32), 4: (O.F32, O.F32), 5: (O.F16, O.F16),
+         6: (O.F64, O.F64)}
 SHAPES = {0: [(16, 16), (16, 32), (32, 8), (32, 16)], 1: [(16, 16), (16, 32), (32, 8), (32, 16)],
           2: [(16, 32), (16, 64), (32, 16), (32, 32)], 3: [(16, 32), (16, 64), (32, 16), (32, 32)],
-          4: [(16, 4), (16, 16), (32, 2), (32, 8)], 5: [(16, 16), (32, 16)]}
+          4: [(16, 4), (16, 16), (32, 2), (32, 8)], 5: [(16, 16), (32, 16)], 6: [(16, 4), (16, 8), (16, 16), (16, 32)]}
 
 
 @pytest.mark.parametrize("type_id", sorted(TYPES))

@@ -61,6 +61,10 @@ def _check(in_t, out_t, got, want, want_f32=None):
     if in_t == O.I8:
         assert np.array_equal(got, want)
         return
+    if out_t == O.F64:
+        ok, mx = O.compare(O.F64, got, want, 10.0)  # the reference's 10 eps(f64), test/gemm/gemm_kernel_base_impl.hpp:906-918
+        assert ok, mx
+        return
     tol = REL_TOL.get(in_t, 1e-5)
     if out_t == O.F32:
         assert _max_rel(out_t, got, want) <= tol
@@ -94,7 +98,8 @@ def test_config1_256_cubed_f16_tn_alpha_beta_2():
         assert ok and mx == 0.0, mx
 
 
-TYPE_PAIRS = [(O.F16, O.F32), (O.F16, O.F16), (O.BF16, O.F32), (O.BF16, O.BF16), (O.E4M3, O.F32), (O.I8, O.I32), (O.F32, O.F32)]
+TYPE_PAIRS = [(O.F16, O.F32), (O.F16, O.F16), (O.BF16, O.F32), (O.BF16, O.BF16), (O.E4M3, O.F32), (O.I8, O.I32), (O.F32, O.F32),
+              (O.F64, O.F64)]
 
 
 @pytest.mark.parametrize("in_t,out_t", TYPE_PAIRS)

@@ -320,3 +320,23 @@ def test_e4m3_matches_torch_float8_e4m3fn():
     # -0.0 and +0.0 encode to 0x80 / 0x00 in both; compare bytes
     assert np.array_equal(got, want)
     assert np.array_equal(O.storage_to_f32(got, O.E4M3), t.to(torch.float32).numpy())
+
+
+def test_gemm_f64_against_numpy():
+    """f64 path (the reference's dgemm instantiation): exact on the reference's integer pattern in every
+    layout combination; on random data equal to numpy's sequential float64 accumulation bit for bit."""
+    m, n, k = 24, 40, 56
+    for la in (O.ROW, O.COL):
+        for lb in (O.ROW, O.COL):
+            for ld in (O.ROW, O.COL):
+                a, b, c = O.fill_ref(O.F64, m, k, la), O.fill_ref(O.F64, k, n, lb), O.fill_ref(O.F64, m, n, ld)
+                A, B, C = O.as_matrix(a, m, k, la), O.as_matrix(b, k, n, lb), O.as_matrix(c, m, n, ld)
+                got = O.as_matrix(O.gemm(O.F64, O.F64, la, lb, ld, ld, m, n, k, a, b, c, 2.0, -3.0), m, n, ld)
+                assert np.array_equal(got, 2.0 * (A @ B) - 3.0 * C)
+    a = O.normal(21, m * k).astype(np.float64) * 1.2345678901234
+    b = O.normal(22, k * n).astype(np.float64) / 3.0
+    A, B = a.reshape(m, k), b.reshape(k, n)
+    got = O.gemm(O.F64, O.F64, O.ROW, O.ROW, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0).reshape(m, n)
+    prod = A[:, :, None] * B[None, :, :]  # (m, k, n): products in k order
+    seq = np.add.accumulate(prod, axis=1)[:, -1, :]  # sequential left-to-right sums
+    assert np.array_equal(got, seq)

@@ -12,7 +12,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 REF = "/root/reference/samples"
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-SAMPLES = ["simple_hgemm", "perf_hgemm", "simple_sgemv", "simple_dlrm", "simple_sgemm", "perf_sgemm"]
+SAMPLES = ["simple_hgemm", "perf_hgemm", "simple_sgemv", "simple_dlrm", "simple_sgemm", "perf_sgemm", "simple_dgemm",
+           "perf_dgemm", "simple_dgemv"]
 
 
 @pytest.mark.skipif(not os.path.isdir(REF) or not os.path.exists(HIPCC), reason="needs the reference tree and hipcc")
