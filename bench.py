@@ -9,7 +9,7 @@ One "step" is one GEMM launch on device-resident operands.  Prints ONE JSON line
                published dense f16 MFMA peak (2.5 PFLOP/s)
   cpu_baseline the CPU oracle (port of the reference's OpenMP gemm_CPU) timed on a bounded sample
                of complete output rows of the same workload; the same rows validate the GPU result
-  extra        the other BASELINE configurations (bf16, int8, fp8, 2:4 sparse, DLRM) with their
+  extra        the other benchmark configurations (bf16, int8, fp8, 2:4 sparse, DLRM) with their
                own roofline fractions (skipped with --quick)
 """
 import argparse
@@ -37,7 +37,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--size", type=int, default=8192, help="M = N = K (default: the BASELINE size)")
+    ap.add_argument("--size", type=int, default=8192, help="M = N = K (default: the headline size)")
     ap.add_argument("--cpu-rows", type=int, default=512, help="output rows the CPU baseline computes")
     ap.add_argument("--quick", action="store_true", help="skip the extra configurations")
     args = ap.parse_args()
@@ -121,7 +121,7 @@ def main():
         "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": "dense GEMM M=N=K=%d, f16 A (col-major) x f16 B (row-major) -> f16 row-major, "
-                               "f32 accumulate, alpha=1 beta=0 (BASELINE configs[1])" % m,
+                               "f32 accumulate, alpha=1 beta=0 (headline configuration)" % m,
                    "kernel": {1: "block-per-wave", 2: "macro-tile"}[plan.kernel],
                    "macro_tile": [plan.macro_tile_m, plan.macro_tile_n, plan.macro_tile_k],
                    "lds_bytes": plan.lds_bytes, "grid": plan.grid_x, "block": plan.block_x,
@@ -145,7 +145,7 @@ def main():
 
 
 def run_extras(R, O, np, torch, args):
-    """The remaining BASELINE configurations, each timed with HIP events over args.steps launches."""
+    """The remaining benchmark configurations, each timed with HIP events over args.steps launches."""
     out = {}
     s = args.size
 
@@ -173,7 +173,7 @@ def run_extras(R, O, np, torch, args):
     f8 = lambda nel: torch.randn(nel, device="cuda").clamp_(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8)
     gemm_case("gemm_e4m3_tn_8192", R.E4M3, R.F32, R.ROW_MAJOR, R.COL_MAJOR, f8(s * s), f8(s * s), PEAK_TFLOPS["e4m3"],
               "TFLOP/s")
-    # 2:4 sparse, BASELINE config 4: M = N = 4096, dense-equivalent K = 8192, int8; dense-equivalent ops
+    # 2:4 sparse, benchmark configuration 4: M = N = 4096, dense-equivalent K = 8192, int8; dense-equivalent ops
     # against the sparse peak (2 x dense).  Every group of 4 keeps 2 values at random positions:
     # one index nibble idx0 | idx1 << 2 (idx0 < idx1) per group, two groups per metadata byte.
     sm, sn, sk = 4096, 4096, 8192
@@ -183,7 +183,7 @@ def run_extras(R, O, np, torch, args):
     meta = (nib[:, 0] | (nib[:, 1] << 4)).contiguous()
     gemm_case("gemm_i8_sparse24_4096x4096x8192", R.I8, R.I32, R.ROW_MAJOR, R.COL_MAJOR, vals, i8(sk * sn),
               PEAK_TFLOPS["i8"], "TOP/s (dense-equivalent)", sparse_meta=meta, mm=sm, nn=sn, kk=sk, peak_scale=2.0)
-    # DLRM dot interaction forward, BASELINE config 5
+    # DLRM dot interaction forward, benchmark configuration 5
     bsz, mm, kk = 65536, 27, 128
     x = torch.randn(bsz * mm * kk, device="cuda").to(torch.float16)
     o = torch.empty(bsz * (kk + mm * (mm - 1) // 2), dtype=torch.float16, device="cuda")

@@ -111,7 +111,7 @@ def test_fwd_integer_inputs_exact():
 
 
 def test_fwd_full_batch_65536_properties():
-    # BASELINE config 5 at full size: oracle on a sample of the batch + symmetric-product identity
+    # benchmark configuration 5 at full size: oracle on a sample of the batch + symmetric-product identity
     m, k, batch = 27, 128, 65536
     x = O.f32_to_storage(O.normal(5, batch * m * k), O.F16)
     got = _fwd(O.F16, x, m, k, batch)

@@ -81,7 +81,7 @@ def _check(in_t, out_t, got, want, want_f32=None):
 
 
 def test_config1_256_cubed_f16_tn_alpha_beta_2():
-    # BASELINE config 1: A row-major (T), B col-major (N), C/D f32 row-major, alpha = beta = 2
+    # benchmark configuration 1: A row-major (T), B col-major (N), C/D f32 row-major, alpha = beta = 2
     m = n = k = 256
     a, b, c = _inputs(O.F16, O.F32, m, n, k, seed=1)
     want = O.gemm(O.F16, O.F32, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, 2.0)
@@ -184,7 +184,7 @@ def test_auto_falls_back_and_bad_sizes_error():
 @pytest.mark.parametrize("in_t,out_t,la,lb", [(O.F16, O.F16, O.COL, O.ROW), (O.BF16, O.BF16, O.COL, O.ROW),
                                                (O.I8, O.I32, O.ROW, O.COL), (O.E4M3, O.F32, O.ROW, O.COL)])
 def test_full_size_8192_sampled_rows(in_t, out_t, la, lb):
-    # BASELINE configs 2 / 3 at full size.  Each element of the oracle depends only on its own row
+    # benchmark configurations 2 and 3 at full size.  Each element of the oracle depends only on its own row
     # of A and column of B, so complete rows computed by the oracle are exactly its values.
     import torch
 

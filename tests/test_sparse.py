@@ -47,7 +47,7 @@ def test_sparse_gemm_vs_dense_oracle(in_t, out_t, m, n, k, ldl):
 
 
 def test_sparse_config4_sampled_rows():
-    # BASELINE config 4: M = N = 4096, dense-equivalent K = 8192, int8
+    # benchmark configuration 4: M = N = 4096, dense-equivalent K = 8192, int8
     m, n, k = 4096, 4096, 8192
     dense, b = _sparse_inputs(O.I8, m, n, k, 60)
     vals, meta = R.compress_24(dense)
