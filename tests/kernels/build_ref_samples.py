@@ -1,0 +1,35 @@
+"""Builds the reference's own sample kernels against this library's headers into shared objects the
+GPU tests can call: the sample sources are compiled where they lie (REFERENCE_ROOT, default
+/root/reference) -- nothing of them is copied -- and the outputs go to tests/kernels/_ref/, which is
+kept out of version control.  Without the reference tree this is a no-op and the tests skip."""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+REF = os.environ.get("REFERENCE_ROOT", "/root/reference")
+OUT = os.path.join(HERE, "_ref")
+WRAPPERS = ["simple_hgemm", "perf_hgemm", "simple_dlrm", "simple_sgemv", "simple_sgemm", "simple_dgemm", "perf_sgemm",
+            "perf_dgemm"]
+
+
+def build():
+    samples = os.path.join(REF, "samples")
+    if not os.path.isdir(samples):
+        return []
+    os.makedirs(OUT, exist_ok=True)
+    built = []
+    for name in WRAPPERS:
+        out = os.path.join(OUT, "libref_%s.so" % name)
+        subprocess.check_call([
+            os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), "--offload-arch=gfx950", "-std=c++17", "-O3", "-fPIC", "-shared",
+            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-w",
+            "-I" + os.path.join(ROOT, "rocwmma_amd", "include"), "-I" + samples,
+            os.path.join(HERE, "ref_samples", "wrap_%s.hip" % name), "-o", out])
+        built.append(out)
+    return built
+
+
+if __name__ == "__main__":
+    print("\n".join(build()) or "reference tree not found at %s: nothing built" % REF, file=sys.stderr)
