@@ -11,6 +11,19 @@ namespace rocwmma
     {
         static constexpr uint32_t AMDGCN_ARCH_ID_GFX950 = 0x950;
         static constexpr uint32_t AMDGCN_ARCH_ID_NONE   = 0x0;
+        // Identifiers of the targets the reference knows (constants.hpp:39-49).  They exist so that
+        // code comparing AMDGCN_CURRENT_ARCH_ID against them still compiles; none of them is ever
+        // the current architecture here.
+        static constexpr uint32_t AMDGCN_ARCH_ID_GFX908  = 0x908;
+        static constexpr uint32_t AMDGCN_ARCH_ID_GFX90A  = 0x90A;
+        static constexpr uint32_t AMDGCN_ARCH_ID_GFX940  = 0x940;
+        static constexpr uint32_t AMDGCN_ARCH_ID_GFX941  = 0x941;
+        static constexpr uint32_t AMDGCN_ARCH_ID_GFX942  = 0x942;
+        static constexpr uint32_t AMDGCN_ARCH_ID_GFX1100 = 0x1100;
+        static constexpr uint32_t AMDGCN_ARCH_ID_GFX1101 = 0x1101;
+        static constexpr uint32_t AMDGCN_ARCH_ID_GFX1102 = 0x1102;
+        static constexpr uint32_t AMDGCN_ARCH_ID_GFX1200 = 0x1200;
+        static constexpr uint32_t AMDGCN_ARCH_ID_GFX1201 = 0x1201;
 
         static constexpr uint32_t AMDGCN_WAVE_SIZE_64   = 64u;
         static constexpr uint32_t AMDGCN_WAVE_SIZE_32   = 32u;

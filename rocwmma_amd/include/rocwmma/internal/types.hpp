@@ -90,6 +90,24 @@ namespace rocwmma
     template <typename L>
     using orthogonal_layout_t = typename detail::orthogonal_layout<L>::type;
 
+    // How many elements of DataT share one 32-bit register, and the register's element type
+    // (same names as the reference's pack_util.hpp:42-53 / pack_util_impl.hpp:36-200).
+    template <typename DataT>
+    struct PackTraits
+    {
+        enum : uint32_t
+        {
+            PackRatio = sizeof(DataT) >= 4u ? 1u : 4u / sizeof(DataT)
+        };
+        using UnpackedT = DataT;
+        using PackedT   = std::conditional_t<
+            sizeof(DataT) >= 4u,
+            DataT,
+            std::conditional_t<std::is_integral_v<DataT>,
+                               std::conditional_t<std::is_signed_v<DataT>, int32_t, uint32_t>,
+                               float32_t>>;
+    };
+
 } // namespace rocwmma
 
 #endif // ROCWMMA_TYPES_HPP
