@@ -127,3 +127,35 @@ def test_f32_f64_gemm_sample_kernels(sample, dtype, la, lb, mnk):
     assert fn(m, n, k, _p(da), _p(db), _p(dc), _p(dd), lda, ldb, n, n, ctypes.c_double(2.0), ctypes.c_double(2.0)) == 0
     want = O.gemm(dtype, dtype, la, lb, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, 2.0)
     assert np.array_equal(to_host(dd, O.NP_STORAGE[dtype]), want)
+
+
+@pytest.mark.parametrize("dtype,tile", [(O.F16, 16), (O.F16, 32), (O.F32, 16), (O.F32, 32)])
+def test_reference_dlrm_test_kernels_forward_and_backward(dtype, tile):
+    # test/dlrm/device/dlrm_dot_fwd.hpp:37-138 and dlrm_dot_bwd.hpp:35-176 (trilReconstruct + dlrmDotBwd)
+    L = _lib("test_dlrm")
+    m, k, batch = 32, 128, 5
+    stride = k + m * (m - 1) // 2
+    st = O.NP_STORAGE[dtype]
+    x = O.f32_to_storage(O.normal(14, batch * m * k) * 0.5, dtype)
+    up = O.f32_to_storage(O.normal(15, batch * stride) * 0.5, dtype)
+    dx, dup = to_device(x), to_device(up)
+    dout = device_filled(batch * stride, st, 0xFF)
+    dacc = device_filled(batch * m * m, np.float32, 0x00)
+    assert L.ref_test_dlrm_fwd(dtype, tile, _p(dx), _p(dout), _p(dacc), m, k, batch) == 0
+    want = O.dlrm_fwd(dtype, x, m, k, batch).ravel()
+    tol = 10.0 if dtype == O.F16 else 40.0  # f32: two summation orders of 128 terms (see tests/test_dlrm.py)
+    ok, mx = O.compare(dtype, to_host(dout, st), want, tol)
+    assert ok, mx
+    dgrad, dmlp = device_filled(batch * m * k, st, 0xFF), device_filled(batch * k, st, 0xFF)
+    dacc2 = device_filled(batch * m * m, st, 0x00)
+    assert L.ref_test_dlrm_bwd(dtype, tile, _p(dx), _p(dup), _p(dgrad), _p(dmlp), _p(dacc2), m, k, batch) == 0
+    if dtype == O.F16:
+        want_mlp, want_grad = O.dlrm_bwd(dtype, x, up, m, k, batch)
+        assert np.array_equal(to_host(dmlp, st), want_mlp.ravel())
+        ok, mx = O.compare(dtype, to_host(dgrad, st), want_grad.ravel(), 10.0)
+        assert ok, mx
+    else:
+        want_mlp, want_grad = O.dlrm_bwd(dtype, x, up, m, k, batch)
+        assert np.array_equal(to_host(dmlp, st), want_mlp.ravel())
+        ok, mx = O.compare(dtype, to_host(dgrad, st), want_grad.ravel(), 40.0)
+        assert ok, mx

@@ -30,3 +30,41 @@ def test_reference_sample_compiles_unchanged(sample):
         asm = open(out).read()
         assert "v_mfma_" in asm  # the fragment API lowered to matrix instructions
         assert "scratch_" not in asm  # fragments stay in registers
+
+
+# Device headers of the reference's own test suites that stay inside the fragment API surface.
+TEST_DEVICE_HEADERS = [
+    "unit/load_store_matrix_sync_test/device/load_store_matrix_sync.hpp",
+    "unit/load_store_matrix_coop_sync_test/device/load_store_matrix_coop_sync.hpp",
+    "unit/fill_fragment_test/device/fill_fragment.hpp",
+    "unit/contamination_test/device/load_contamination.hpp",
+    "unit/contamination_test/device/store_contamination.hpp",
+    "unit/map_util_test/device/map_block_to_matrix.hpp",
+    "unit/map_util_test/device/map_block_to_matrix_override.hpp",
+    "unit/map_util_test/device/map_matrix_to_data.hpp",
+    "unit/map_util_test/device/map_matrix_to_data_override.hpp",
+    "unit/map_util_test/device/map_thread_to_matrix.hpp",
+    "unit/map_util_test/device/map_wave_to_matrix.hpp",
+    "dlrm/device/dlrm_dot_fwd.hpp",
+    "dlrm/device/dlrm_dot_bwd.hpp",
+]
+REF_TEST = "/root/reference/test"
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_TEST) or not os.path.exists(HIPCC), reason="needs the reference tree and hipcc")
+@pytest.mark.parametrize("header", TEST_DEVICE_HEADERS)
+def test_reference_test_device_header_compiles_unchanged(header):
+    """The kernels in these headers are templates; the translation unit here only has to parse and
+    semantically check them against this library's headers (the run-time check of the DLRM ones is
+    tests/test_ref_samples_run.py)."""
+    with tempfile.TemporaryDirectory() as tmp:
+        src = os.path.join(tmp, "tu.hip")
+        with open(src, "w") as f:
+            f.write('#include <hip/hip_runtime.h>\n#include <rocwmma/rocwmma.hpp>\n#include <rocwmma/rocwmma_coop.hpp>\n'
+                    '#include <rocwmma/rocwmma_transforms.hpp>\n#include "%s"\n' % header)
+        r = subprocess.run(
+            [HIPCC, "--offload-arch=gfx950", "-std=c++17", "-O1", "-c", "--cuda-device-only", "-w",
+             "-I" + os.path.join(ROOT, "rocwmma_amd", "include"), "-I" + REF_TEST, "-I" + os.path.join(REF_TEST, "unit"),
+             "-I" + os.path.join(REF_TEST, "dlrm"), src, "-o", os.path.join(tmp, "tu.o")],
+            capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr[-2000:]
