@@ -19,6 +19,8 @@
 
 using hip_fp8_e4m3 = __hip_fp8_e4m3;
 using hip_fp8_e5m2 = __hip_fp8_e5m2;
+using hip_fp8_e4m3_fnuz = __hip_fp8_e4m3_fnuz;
+using hip_fp8_e5m2_fnuz = __hip_fp8_e5m2_fnuz;
 
 namespace rocwmma
 {
@@ -27,6 +29,14 @@ namespace rocwmma
     using bfloat16_t = hip_bfloat16;
     using float8_t   = hip_fp8_e4m3;
     using bfloat8_t  = hip_fp8_e5m2;
+    // Storage-only names kept for source compatibility (types.hpp:108-114 of the reference): gfx950's
+    // matrix cores take the OCP encodings only and have no xf32 form, so mma_sync rejects these.
+    using float8_fnuz_t  = hip_fp8_e4m3_fnuz;
+    using bfloat8_fnuz_t = hip_fp8_e5m2_fnuz;
+    struct xfloat32_t
+    {
+        float data;
+    };
     using float32_t  = float;
     using float64_t  = double;
     using int8_t     = ::int8_t;

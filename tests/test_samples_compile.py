@@ -47,6 +47,7 @@ TEST_DEVICE_HEADERS = [
     "unit/map_util_test/device/map_wave_to_matrix.hpp",
     "dlrm/device/dlrm_dot_fwd.hpp",
     "dlrm/device/dlrm_dot_bwd.hpp",
+    "gemm/gemm_PGR0_LB0_MP0_SB_NC/device/kernel_device_func.hpp",
 ]
 REF_TEST = "/root/reference/test"
 
@@ -60,11 +61,12 @@ def test_reference_test_device_header_compiles_unchanged(header):
     with tempfile.TemporaryDirectory() as tmp:
         src = os.path.join(tmp, "tu.hip")
         with open(src, "w") as f:
-            f.write('#include <hip/hip_runtime.h>\n#include <rocwmma/rocwmma.hpp>\n#include <rocwmma/rocwmma_coop.hpp>\n'
+            f.write('#include <iostream>\n#include <hip/hip_runtime.h>\n#include <rocwmma/rocwmma.hpp>\n#include <rocwmma/rocwmma_coop.hpp>\n'
                     '#include <rocwmma/rocwmma_transforms.hpp>\n#include "%s"\n' % header)
         r = subprocess.run(
             [HIPCC, "--offload-arch=gfx950", "-std=c++17", "-O1", "-c", "--cuda-device-only", "-w",
              "-I" + os.path.join(ROOT, "rocwmma_amd", "include"), "-I" + REF_TEST, "-I" + os.path.join(REF_TEST, "unit"),
-             "-I" + os.path.join(REF_TEST, "dlrm"), src, "-o", os.path.join(tmp, "tu.o")],
+             "-I" + os.path.join(REF_TEST, "dlrm"), "-I" + os.path.join(REF_TEST, "gemm"), src, "-o",
+             os.path.join(tmp, "tu.o")],
             capture_output=True, text=True)
         assert r.returncode == 0, r.stderr[-2000:]
