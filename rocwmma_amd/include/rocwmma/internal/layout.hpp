@@ -156,6 +156,16 @@ namespace rocwmma
             = std::is_same_v<MatrixT, matrix_a> ? std::is_same_v<DataLayoutT, row_major>
                                                 : std::is_same_v<DataLayoutT, col_major>;
     } // namespace detail
+    // Public names of the 1-d data spaces (reference: layout/data_layout.hpp, used by kernels as
+    // DataLayout::Array1d<row_major>::fromMatrixCoord(coord, ld)).
+    namespace DataLayout
+    {
+        template <typename DataOrientation>
+        using Array1d = detail::DataSpace<DataOrientation>;
+        using RowMajor = Array1d<row_major>;
+        using ColMajor = Array1d<col_major>;
+    } // namespace DataLayout
+
 } // namespace rocwmma
 
 #endif // ROCWMMA_LAYOUT_HPP

@@ -101,6 +101,38 @@ namespace rocwmma
         }
     } // namespace detail
 
+    // Short printable tag of a type, for logs and benchmark tables (utils.hpp:196-325 of the reference).
+    // Primary template has no definition: user code may specialise it for its own tag types.
+    template <typename DataT>
+    constexpr const char* dataTypeToString();
+
+#define ROCWMMA_TYPE_TAG(TYPE, TAG)                            \
+    template <>                                                \
+    constexpr const char* dataTypeToString<TYPE>()             \
+    {                                                          \
+        return TAG;                                            \
+    }
+    ROCWMMA_TYPE_TAG(float8_t, "f8")
+    ROCWMMA_TYPE_TAG(bfloat8_t, "bf8")
+    ROCWMMA_TYPE_TAG(float8_fnuz_t, "f8(fnuz)")
+    ROCWMMA_TYPE_TAG(bfloat8_fnuz_t, "bf8(fnuz)")
+    ROCWMMA_TYPE_TAG(float16_t, "f16")
+    ROCWMMA_TYPE_TAG(hfloat16_t, "h16")
+    ROCWMMA_TYPE_TAG(bfloat16_t, "bf16")
+    ROCWMMA_TYPE_TAG(float32_t, "f32")
+    ROCWMMA_TYPE_TAG(xfloat32_t, "xf32")
+    ROCWMMA_TYPE_TAG(float64_t, "f64")
+    ROCWMMA_TYPE_TAG(int8_t, "i8")
+    ROCWMMA_TYPE_TAG(uint8_t, "u8")
+    ROCWMMA_TYPE_TAG(int16_t, "i16")
+    ROCWMMA_TYPE_TAG(uint16_t, "u16")
+    ROCWMMA_TYPE_TAG(int32_t, "i32")
+    ROCWMMA_TYPE_TAG(uint32_t, "u32")
+    ROCWMMA_TYPE_TAG(uint64_t, "u64")
+    ROCWMMA_TYPE_TAG(row_major, "T")
+    ROCWMMA_TYPE_TAG(col_major, "N")
+#undef ROCWMMA_TYPE_TAG
+
 } // namespace rocwmma
 
 #endif // ROCWMMA_UTILS_HPP

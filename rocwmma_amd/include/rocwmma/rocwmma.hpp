@@ -11,6 +11,7 @@
 #include "internal/config.hpp"
 #include "internal/constants.hpp"
 #include "internal/convert.hpp"
+#include "internal/flow_control.hpp"
 #include "internal/io.hpp"
 #include "internal/layout.hpp"
 #include "internal/mapping_util.hpp"
@@ -177,7 +178,10 @@ namespace rocwmma
 
     template <typename FragT>
     using GetIOConfig_t = typename detail::FragmentTraits<std::decay_t<FragT>>::IOConfigT;
-    template <typename FragT>
+    // Cooperative configuration: the register layout does not depend on how many waves share the
+    // fragment (waves take whole register chunks), so WaveCount only parameterises the name
+    // (reference: coop_io_config.hpp:63-108, accessors_impl.hpp:99-112).
+    template <typename FragT, uint32_t WaveCount = 1u>
     using GetCoopIOConfig_t = GetIOConfig_t<FragT>;
     template <typename FragT>
     using GetIOShape_t = typename GetIOConfig_t<FragT>::IOShape;

@@ -48,6 +48,7 @@ TEST_DEVICE_HEADERS = [
     "dlrm/device/dlrm_dot_fwd.hpp",
     "dlrm/device/dlrm_dot_bwd.hpp",
     "gemm/gemm_PGR0_LB0_MP0_SB_NC/device/kernel_device_func.hpp",
+    "gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp",
 ]
 REF_TEST = "/root/reference/test"
 
