@@ -13,6 +13,7 @@
 #include "internal/convert.hpp"
 #include "internal/flow_control.hpp"
 #include "internal/io.hpp"
+#include "internal/io_traits.hpp"
 #include "internal/layout.hpp"
 #include "internal/mapping_util.hpp"
 #include "internal/mfma.hpp"

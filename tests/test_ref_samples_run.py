@@ -159,3 +159,12 @@ def test_reference_dlrm_test_kernels_forward_and_backward(dtype, tile):
         assert np.array_equal(to_host(dmlp, st), want_mlp.ravel())
         ok, mx = O.compare(dtype, to_host(dgrad, st), want_grad.ravel(), 40.0)
         assert ok, mx
+
+
+def test_reference_io_traits_unit_kernel():
+    # test/unit/io_traits_test/device/io_traits.hpp:34-101: PackTraits and IOTraits identities checked on the
+    # device; 0 = SUCCESS_VALUE
+    L = _lib("test_io_traits")
+    n = L.ref_test_io_traits_cases()
+    assert n >= 20
+    assert [L.ref_test_io_traits(i) for i in range(n)] == [0] * n

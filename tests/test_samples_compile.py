@@ -49,6 +49,8 @@ TEST_DEVICE_HEADERS = [
     "dlrm/device/dlrm_dot_bwd.hpp",
     "gemm/gemm_PGR0_LB0_MP0_SB_NC/device/kernel_device_func.hpp",
     "gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp",
+    "dlrm/device/dlrm_dot_fwd_lds.hpp",
+    "dlrm/device/dlrm_dot_bwd_lds.hpp",
 ]
 REF_TEST = "/root/reference/test"
 
