@@ -168,3 +168,27 @@ def test_reference_io_traits_unit_kernel():
     n = L.ref_test_io_traits_cases()
     assert n >= 20
     assert [L.ref_test_io_traits(i) for i in range(n)] == [0] * n
+
+
+@pytest.mark.parametrize("tile", [16, 32])
+def test_reference_dlrm_lds_test_kernels(tile):
+    # test/dlrm/device/dlrm_dot_fwd_lds.hpp / dlrm_dot_bwd_lds.hpp with the register-file LDS mapping
+    # (test/dlrm/lds_mapping_util.hpp:63-367): fragments parked in LDS and re-read between K steps
+    L = _lib("test_dlrm")
+    m, k, batch = 32, 128, 5
+    stride = k + m * (m - 1) // 2
+    x = O.f32_to_storage(O.normal(16, batch * m * k) * 0.5, O.F16)
+    up = O.f32_to_storage(O.normal(17, batch * stride) * 0.5, O.F16)
+    dx, dup = to_device(x), to_device(up)
+    dout = device_filled(batch * stride, np.uint16, 0xFF)
+    dacc = device_filled(batch * m * m, np.float32, 0x00)
+    assert L.ref_test_dlrm_fwd_lds(tile, _p(dx), _p(dout), _p(dacc), m, k, batch) == 0
+    ok, mx = O.compare(O.F16, to_host(dout, np.uint16), O.dlrm_fwd(O.F16, x, m, k, batch).ravel(), 10.0)
+    assert ok, mx
+    dgrad, dmlp = device_filled(batch * m * k, np.uint16, 0xFF), device_filled(batch * k, np.uint16, 0xFF)
+    dacc2 = device_filled(batch * m * m, np.uint16, 0x00)
+    assert L.ref_test_dlrm_bwd_lds(tile, _p(dx), _p(dup), _p(dgrad), _p(dmlp), _p(dacc2), m, k, batch) == 0
+    want_mlp, want_grad = O.dlrm_bwd(O.F16, x, up, m, k, batch)
+    assert np.array_equal(to_host(dmlp, np.uint16), want_mlp.ravel())
+    ok, mx = O.compare(O.F16, to_host(dgrad, np.uint16), want_grad.ravel(), 10.0)
+    assert ok, mx
