@@ -29,7 +29,13 @@ namespace rocwmma
         static constexpr uint32_t AMDGCN_WAVE_SIZE_32   = 32u;
         static constexpr uint32_t AMDGCN_WAVE_SIZE_NONE = 0u;
 
-#if ROCWMMA_ARCH_GFX950
+        // Code written before gfx950 existed often gates its wave64 matrix-core branch on one of the
+        // gfx90a / gfx94x ids above.  Compiling it with -DROCWMMA_REPORT_ARCH_ID=0x942 makes the device
+        // pass report that id instead, so such gates pick the branch this hardware can run; nothing else
+        // in the library depends on the value.
+#if ROCWMMA_ARCH_GFX950 && defined(ROCWMMA_REPORT_ARCH_ID)
+        static constexpr uint32_t AMDGCN_CURRENT_ARCH_ID = ROCWMMA_REPORT_ARCH_ID;
+#elif ROCWMMA_ARCH_GFX950
         static constexpr uint32_t AMDGCN_CURRENT_ARCH_ID = AMDGCN_ARCH_ID_GFX950;
 #else
         static constexpr uint32_t AMDGCN_CURRENT_ARCH_ID = AMDGCN_ARCH_ID_NONE;

@@ -25,7 +25,8 @@ namespace rocwmma
             {
                 return make_coord2d(threadIdx.x / Constants::AMDGCN_WAVE_SIZE, threadIdx.y);
             }
-            ROCWMMA_DEVICE static inline WorkgroupDimT workgroupDim()
+            // Compile-time constant when the workgroup shape is given as template arguments
+            ROCWMMA_DEVICE constexpr static inline WorkgroupDimT workgroupDim()
             {
                 if constexpr(TBlockX > 0u && TBlockY > 0u)
                     return make_coord2d(TBlockX / Constants::AMDGCN_WAVE_SIZE, TBlockY);

@@ -11,7 +11,7 @@ ROOT = os.path.dirname(os.path.dirname(HERE))
 REF = os.environ.get("REFERENCE_ROOT", "/root/reference")
 OUT = os.path.join(HERE, "_ref")
 WRAPPERS = ["simple_hgemm", "perf_hgemm", "simple_dlrm", "simple_sgemv", "simple_sgemm", "simple_dgemm", "perf_sgemm",
-            "perf_dgemm", "test_dlrm", "test_io_traits"]
+            "perf_dgemm", "test_dlrm", "test_io_traits", "test_gemm_simple", "test_gemm_coop"]
 
 
 def build():
@@ -26,7 +26,8 @@ def build():
             os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), "--offload-arch=gfx950", "-std=c++17", "-O3", "-fPIC", "-shared",
             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-w",
             "-I" + os.path.join(ROOT, "rocwmma_amd", "include"), "-I" + samples, "-I" + os.path.join(REF, "test", "dlrm"),
-            "-I" + os.path.join(REF, "test"), "-I" + os.path.join(REF, "test", "unit"), "-I" + REF,
+            "-I" + os.path.join(REF, "test"), "-I" + os.path.join(REF, "test", "unit"), "-I" + os.path.join(REF, "test", "gemm"),
+            "-I" + REF,
             os.path.join(HERE, "ref_samples", "wrap_%s.hip" % name), "-o", out])
         built.append(out)
     return built

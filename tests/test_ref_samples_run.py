@@ -192,3 +192,51 @@ def test_reference_dlrm_lds_test_kernels(tile):
     assert np.array_equal(to_host(dmlp, np.uint16), want_mlp.ravel())
     ok, mx = O.compare(O.F16, to_host(dgrad, np.uint16), want_grad.ravel(), 10.0)
     assert ok, mx
+
+
+def _gemm_args(m, n, k, da, db, dc, dd, lda, ldb, alpha, beta):
+    return (m, n, k, _p(da), _p(db), _p(dc), _p(dd), lda, ldb, n, n, ctypes.c_float(alpha), ctypes.c_float(beta))
+
+
+@pytest.mark.parametrize("cid,in_t,out_t,la,lb", [(0, O.F16, O.F32, O.ROW, O.COL), (1, O.F16, O.F16, O.COL, O.ROW),
+                                                  (2, O.I8, O.I32, O.ROW, O.COL)])
+def test_reference_gemm_test_kernel_block_per_wave(cid, in_t, out_t, la, lb):
+    # test/gemm/gemm_PGR0_LB0_MP0_SB_NC/device/kernel_device_func.hpp:50-175
+    L = _lib("test_gemm_simple")
+    m, n, k = 128, 192, 96
+    if in_t == O.I8:
+        a, b = O.uniform_int8(21, m * k), O.uniform_int8(22, k * n)
+        c = O.uniform_int8(23, m * n).astype(np.int32) * 11
+    else:
+        a = O.f32_to_storage(O.uniform_pm1(21, m * k), in_t)
+        b = O.f32_to_storage(O.uniform_pm1(22, k * n), in_t)
+        c = O.f32_to_storage(O.uniform_pm1(23, m * n), out_t)
+    st = O.NP_STORAGE[out_t]
+    da, db, dc, dd = to_device(a), to_device(b), to_device(c), device_filled(m * n, st, 0xFF)
+    lda, ldb = (k if la == O.ROW else m), (n if lb == O.ROW else k)
+    assert L.ref_test_gemm_simple(cid, *_gemm_args(m, n, k, da, db, dc, dd, lda, ldb, 2.0, 2.0)) == 0
+    want = O.gemm(in_t, out_t, la, lb, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, 2.0)
+    got = to_host(dd, st)
+    if in_t == O.I8:
+        assert np.array_equal(got, want)
+    else:
+        ok, mx = O.compare(out_t, got, want, 10.0 if out_t == O.F16 else k / 2.0)
+        assert ok, mx
+
+
+@pytest.mark.parametrize("lds_col_major", [0, 1])
+@pytest.mark.parametrize("cid", range(6))
+def test_reference_gemm_test_kernel_cooperative(cid, lds_col_major):
+    # test/gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp:52-283 with the six CooperativeGemm
+    # configurations of test/gemm/gemm_config.hpp:64-431 (workgroup / block / wave level cooperation, LDS
+    # holding NT, TN or register-file images), both LDS data layouts
+    L = _lib("test_gemm_coop")
+    m, n, k = 256, 384, 128
+    a = O.f32_to_storage(O.uniform_pm1(31, m * k), O.F16)
+    b = O.f32_to_storage(O.uniform_pm1(32, k * n), O.F16)
+    c = O.f32_to_storage(O.uniform_pm1(33, m * n), O.F16)
+    da, db, dc, dd = to_device(a), to_device(b), to_device(c), device_filled(m * n, np.uint16, 0xFF)
+    assert L.ref_test_gemm_coop(cid, lds_col_major, *_gemm_args(m, n, k, da, db, dc, dd, m, n, 2.0, 2.0)) == 0
+    want = O.gemm(O.F16, O.F16, O.COL, O.ROW, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, 2.0)
+    ok, mx = O.compare(O.F16, to_host(dd, np.uint16), want, 10.0)
+    assert ok, mx
