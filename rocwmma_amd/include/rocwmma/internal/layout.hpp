@@ -88,14 +88,13 @@ namespace rocwmma
                     kw >>= 1;
                 return kw;
             }
-            if constexpr(bytes == 2u)
-                return (kDim % (8u * groups)) == 0u ? 8u : 4u;
-            else if constexpr(is_i8_v<DataT>)
-                return (kDim % (16u * groups)) == 0u ? 16u : 8u;
-            else if constexpr(bytes == 1u)
-                return 8u;
-            else
-                return 1u;
+            // 16 x 16 and 32 x 32 blocks: start from the widest matrix-instruction operand of the type and
+            // halve until the wave's chunk tiles KDim.  Widths below the narrowest instruction form (4 for
+            // 16-bit types, 8 for 8-bit types) still load, store and fill; mma_sync rejects them.
+            uint32_t kw = bytes == 2u ? 8u : (is_i8_v<DataT> ? 16u : (bytes == 1u ? 8u : 1u));
+            while(kw > 1u && (kDim % (kw * groups)) != 0u)
+                kw >>= 1;
+            return kw;
         }
 
         template <typename MatrixT, uint32_t BlockM, uint32_t BlockN, uint32_t BlockK, typename DataT>
@@ -112,7 +111,7 @@ namespace rocwmma
             static constexpr uint32_t BlockDim    = IsA ? BlockM : BlockN;
             static constexpr uint32_t KDim        = IsAcc ? BlockM : BlockK;
 
-            static_assert(isPow2(BlockDim) && BlockDim >= 16u, "BlockDim must be a power of two >= 16");
+            static_assert(isPow2(BlockDim), "BlockDim must be a power of two");
 
             static constexpr uint32_t D    = cmin(BlockDim, WaveSize);
             static constexpr uint32_t G    = WaveSize / D;
