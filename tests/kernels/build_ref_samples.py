@@ -14,23 +14,27 @@ WRAPPERS = ["simple_hgemm", "perf_hgemm", "simple_dlrm", "simple_sgemv", "simple
             "perf_dgemm", "test_dlrm", "test_io_traits", "test_gemm_simple", "test_gemm_coop", "test_unit"]
 
 
+def _compile(name, samples):
+    out = os.path.join(OUT, "libref_%s.so" % name)
+    subprocess.check_call([
+        os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), "--offload-arch=gfx950", "-std=c++17", "-O3", "-fPIC", "-shared",
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-w",
+        "-I" + os.path.join(ROOT, "rocwmma_amd", "include"), "-I" + samples, "-I" + os.path.join(REF, "test", "dlrm"),
+        "-I" + os.path.join(REF, "test"), "-I" + os.path.join(REF, "test", "unit"), "-I" + os.path.join(REF, "test", "gemm"),
+        "-I" + REF,
+        os.path.join(HERE, "ref_samples", "wrap_%s.hip" % name), "-o", out])
+    return out
+
+
 def build():
     samples = os.path.join(REF, "samples")
     if not os.path.isdir(samples):
         return []
     os.makedirs(OUT, exist_ok=True)
-    built = []
-    for name in WRAPPERS:
-        out = os.path.join(OUT, "libref_%s.so" % name)
-        subprocess.check_call([
-            os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), "--offload-arch=gfx950", "-std=c++17", "-O3", "-fPIC", "-shared",
-            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-w",
-            "-I" + os.path.join(ROOT, "rocwmma_amd", "include"), "-I" + samples, "-I" + os.path.join(REF, "test", "dlrm"),
-            "-I" + os.path.join(REF, "test"), "-I" + os.path.join(REF, "test", "unit"), "-I" + os.path.join(REF, "test", "gemm"),
-            "-I" + REF,
-            os.path.join(HERE, "ref_samples", "wrap_%s.hip" % name), "-o", out])
-        built.append(out)
-    return built
+    from concurrent.futures import ThreadPoolExecutor
+
+    with ThreadPoolExecutor(max_workers=min(6, os.cpu_count() or 1)) as pool:
+        return list(pool.map(lambda n: _compile(n, samples), WRAPPERS))
 
 
 if __name__ == "__main__":
