@@ -10,7 +10,9 @@
 //   macro tile   256 x 256, K stage of 128 bytes (64 f16/bf16, 128 int8/fp8 elements)
 //   workgroup    256 threads = 4 waves in a 2 x 2 grid, wave tile 128 x 128
 //                = 4 x 4 v_mfma_*_32x32x{16,32} accumulators (256 accumulator registers)
-//   LDS          2 stages x (A 32 KiB + B 32 KiB) = 128 KiB, one workgroup per CU
+//   LDS          16-bit types: 2 stages x (A 32 KiB + B 32 KiB) = 128 KiB;
+//                8-bit types: 2 A buffers + 3 B buffers x 32 KiB = 160 KiB (gemmTiledKernel8);
+//                one workgroup per CU either way
 //   global->LDS  128-bit loads, either staged through registers or written straight
 //                into LDS by the memory pipeline (global_load_lds_dwordx4)
 //   LDS layout   16-byte chunks, XOR-swizzled inside each row so that both the
@@ -152,6 +154,112 @@ namespace
             __builtin_amdgcn_sched_group_barrier(0x020, VMEM, 0);
     }
 
+    // D = alpha * acc + beta * C for one wave's 128 x 128 tile, row-major.  `scratch` is 32 KiB of LDS
+    // owned by this wave (the stage buffers are idle by then).
+    template <Elem E, typename OutT>
+    __device__ __forceinline__ void storeTile(typename ElemTraits<E>::Acc (&acc)[4][4], const Params& p, uint32_t tm,
+                                              uint32_t tn, uint32_t wm, uint32_t wn, uint32_t lane, char* scratch)
+    {
+        // ---------------- epilogue: D = alpha * acc + beta * C, row-major
+        // lane holds D(m = lane % 32, n = 8 (e / 4) + 4 (lane / 32) + e % 4) of each 32 x 32 block
+        using AccE = std::conditional_t<E == Elem::I8, int, float>;
+        using OutV = OutT __attribute__((ext_vector_type(4)));
+        const AccE     alpha = static_cast<AccE>(p.alpha), beta = static_cast<AccE>(p.beta);
+        const uint32_t m0 = tm * TILE_M + wm * 128u, n0 = tn * TILE_N + wn * 128u;
+
+        if(beta == static_cast<AccE>(0))
+        {
+            // The stage buffers are idle now: every wave transposes its 128 x 128 result through its
+            // own 32 KiB of LDS so that a store instruction covers whole 256- or 512-byte rows of D
+            // (128-bit per lane) instead of 8- / 16-byte pieces of 32 different rows.
+            constexpr uint32_t OS         = sizeof(OutT);
+            constexpr uint32_t ROW_BYTES  = 128u * OS; // one row of the wave tile
+            constexpr uint32_t ROW_CHUNKS = ROW_BYTES / CHUNK; // 16 (2-byte) or 32 (4-byte)
+            constexpr uint32_t ROWS_PASS  = 32768u / ROW_BYTES; // 128 or 64 rows per pass
+            constexpr uint32_t BLOCKS_I   = ROWS_PASS / 32u; // 32-row blocks per pass
+            char*              wl         = scratch;
+            const uint32_t     r32 = lane & 31u, h = lane >> 5;
+#pragma unroll
+            for(uint32_t pass = 0; pass < 4u / BLOCKS_I; ++pass)
+            {
+#pragma unroll
+                for(uint32_t ii = 0; ii < BLOCKS_I; ++ii)
+                {
+                    const uint32_t i   = pass * BLOCKS_I + ii;
+                    const uint32_t row = 32u * ii + r32; // row inside the pass
+#pragma unroll
+                    for(uint32_t j = 0; j < 4; ++j)
+#pragma unroll
+                        for(uint32_t q = 0; q < 4; ++q)
+                        {
+                            OutV out;
+#pragma unroll
+                            for(uint32_t e = 0; e < 4; ++e)
+                                out[e] = static_cast<OutT>(alpha * static_cast<AccE>(acc[i][j][4 * q + e]));
+                            if constexpr(OS == 2)
+                            {
+                                // 8 bytes: chunk 4 j + q, half h; rows 16 apart share a chunk slot, so
+                                // they take opposite halves
+                                const uint32_t c = 4u * j + q;
+                                char* dst = wl + row * ROW_BYTES + ((c ^ (row & 15u)) * CHUNK) + ((h ^ ((row >> 4) & 1u)) * 8u);
+                                *reinterpret_cast<OutV*>(dst) = out;
+                            }
+                            else
+                            {
+                                const uint32_t c = 8u * j + 2u * q + h;
+                                char* dst = wl + row * ROW_BYTES + ((c ^ (row & 31u)) * CHUNK);
+                                *reinterpret_cast<OutV*>(dst) = out;
+                            }
+                        }
+                }
+                __builtin_amdgcn_wave_barrier(); // same wave reads back what it wrote (LDS is in order per wave)
+#pragma unroll
+                for(uint32_t it = 0; it < ROWS_PASS * ROW_CHUNKS / 64u; ++it)
+                {
+                    const uint32_t L = it * 64u + lane, row = L / ROW_CHUNKS, c = L % ROW_CHUNKS;
+                    i32x4          v;
+                    if constexpr(OS == 2)
+                    {
+                        v = *reinterpret_cast<const i32x4*>(wl + row * ROW_BYTES + ((c ^ (row & 15u)) * CHUNK));
+                        if((row >> 4) & 1u)
+                            v = i32x4{v[2], v[3], v[0], v[1]};
+                    }
+                    else
+                        v = *reinterpret_cast<const i32x4*>(wl + row * ROW_BYTES + ((c ^ (row & 31u)) * CHUNK));
+                    const uint64_t offD = (uint64_t)(m0 + pass * ROWS_PASS + row) * p.ldd + n0;
+                    // D is written once and not read again: stream it past the caches
+                    __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(p.d + offD * OS + c * CHUNK));
+                }
+                __builtin_amdgcn_wave_barrier();
+            }
+            return;
+        }
+
+#pragma unroll
+        for(uint32_t i = 0; i < 4; ++i)
+        {
+#pragma unroll
+            for(uint32_t j = 0; j < 4; ++j)
+            {
+#pragma unroll
+                for(uint32_t q = 0; q < 4; ++q)
+                {
+                    const uint32_t row  = m0 + 32u * i + (lane & 31u);
+                    const uint32_t col  = n0 + 32u * j + 8u * q + 4u * (lane >> 5);
+                    const uint64_t offD = (uint64_t)row * p.ldd + col;
+                    const uint64_t offC = (uint64_t)row * p.ldc + col;
+                    const OutV     cv   = *reinterpret_cast<const OutV*>(p.c + offC * sizeof(OutT));
+                    OutV           out;
+#pragma unroll
+                    for(uint32_t e = 0; e < 4; ++e)
+                        out[e] = static_cast<OutT>(alpha * static_cast<AccE>(acc[i][j][4 * q + e])
+                                                   + beta * static_cast<AccE>(cv[e]));
+                    *reinterpret_cast<OutV*>(p.d + offD * sizeof(OutT)) = out;
+                }
+            }
+        }
+    }
+
     template <Elem E, typename OutT, bool A_KCONTIG, bool B_KCONTIG, bool DIRECT>
     __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
         gemmTiledKernel(Params p)
@@ -160,7 +268,7 @@ namespace
         using Acc             = typename Traits::Acc;
         constexpr uint32_t ES = Traits::Bytes;
         constexpr uint32_t TK = STAGE_KB / ES; // K elements per stage
-        static_assert(ES == 2 || (A_KCONTIG && B_KCONTIG), "8-bit operands must be K-contiguous");
+        static_assert(ES == 2, "16-bit element types only; 8-bit types run gemmTiledKernel8");
         // LDS reads per operand block: one 128-bit read, or two transposing 64-bit reads
         constexpr uint32_t READS_PER_SUB = (A_KCONTIG ? 4u : 8u) + (B_KCONTIG ? 4u : 8u);
 
@@ -361,20 +469,7 @@ namespace
                     mfma32<E>(acc[i][j], fb[j], fa[i]);
         };
 
-        // fp8: one matrix instruction spans two 16-byte sub-steps of K
-        constexpr bool     PAIRED = (E == Elem::E4M3);
-        constexpr uint32_t NBUF   = 4u;
-        auto mfmaPair = [&](const i32x4 (&fa0)[4], const i32x4 (&fa1)[4], const i32x4 (&fb0)[4], const i32x4 (&fb1)[4]) {
-            if constexpr(PAIRED)
-            {
-#pragma unroll
-                for(uint32_t i = 0; i < 4; ++i)
-#pragma unroll
-                    for(uint32_t j = 0; j < 4; ++j)
-                        mfma64Fp8(acc[i][j], fb0[j], fb1[j], fa0[i], fa1[i]);
-            }
-        };
-
+        constexpr uint32_t NBUF = 4u;
         i32x4 fa[NBUF][4], fb[NBUF][4];
 
         // One K stage.  `cur` / `nxt` are the LDS buffers of stage kt / kt + 1.  Operand registers
@@ -386,49 +481,6 @@ namespace
         auto stageBody = [&](uint32_t kt, char* cur, char* nxt, auto refill, auto hasNext) {
             constexpr bool REFILL = decltype(refill)::value; // stage kt + 2 exists
             constexpr bool NEXT   = decltype(hasNext)::value; // stage kt + 1 exists
-            if constexpr(PAIRED)
-            {
-                // sub-steps (0, 1) are in registers; fetch (2, 3) under the first 16 instructions
-#pragma unroll
-                for(uint32_t s = 2; s < 4; ++s)
-#pragma unroll
-                    for(uint32_t i = 0; i < 4; ++i)
-                    {
-                        fa[s][i] = readA(cur, i, s);
-                        fb[s][i] = readB(cur, i, s);
-                    }
-                mfmaPair(fa[0], fa[1], fb[0], fb[1]);
-#pragma unroll
-                for(uint32_t g = 0; g < 8; ++g)
-                    schedGroup<1, 2, 0>();
-                schedGroup<8, 0, 0>();
-                if constexpr(DIRECT)
-                    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
-                else if constexpr(NEXT)
-                    commitLds(nxt);
-                __syncthreads();
-                if constexpr(REFILL)
-                    issueGlobal(kt + 2, cur);
-                if constexpr(NEXT)
-                {
-#pragma unroll
-                    for(uint32_t s = 0; s < 2; ++s)
-#pragma unroll
-                        for(uint32_t i = 0; i < 4; ++i)
-                        {
-                            fa[s][i] = readA(nxt, i, s);
-                            fb[s][i] = readB(nxt, i, s);
-                        }
-                }
-                mfmaPair(fa[2], fa[3], fb[2], fb[3]);
-#pragma unroll
-                for(uint32_t g = 0; g < 8; ++g)
-                    schedGroup<1, NEXT ? 2u : 0u, REFILL ? 1u : 0u>();
-#pragma unroll
-                for(uint32_t g = 0; g < 8; ++g)
-                    schedGroup<1, 0, REFILL ? 1u : 0u>();
-                return;
-            }
 #pragma unroll
             for(uint32_t s = 0; s < 2; ++s)
             {
@@ -509,104 +561,243 @@ namespace
         stageBody(kt, stage0, stage1, no, yes);
         stageBody(kt + 1, stage1, stage0, no, no);
 
-        // ---------------- epilogue: D = alpha * acc + beta * C, row-major
-        // lane holds D(m = lane % 32, n = 8 (e / 4) + 4 (lane / 32) + e % 4) of each 32 x 32 block
-        using AccE = std::conditional_t<E == Elem::I8, int, float>;
-        using OutV = OutT __attribute__((ext_vector_type(4)));
-        const AccE     alpha = static_cast<AccE>(p.alpha), beta = static_cast<AccE>(p.beta);
-        const uint32_t m0 = tm * TILE_M + wm * 128u, n0 = tn * TILE_N + wn * 128u;
+        storeTile<E, OutT>(acc, p, tm, tn, wm, wn, lane, ((wave < 2u) ? stage0 : stage1) + (wave & 1u) * 32768u);
+    }
 
-        if(beta == static_cast<AccE>(0))
-        {
-            // The stage buffers are idle now: every wave transposes its 128 x 128 result through its
-            // own 32 KiB of LDS so that a store instruction covers whole 256- or 512-byte rows of D
-            // (128-bit per lane) instead of 8- / 16-byte pieces of 32 different rows.
-            constexpr uint32_t OS         = sizeof(OutT);
-            constexpr uint32_t ROW_BYTES  = 128u * OS; // one row of the wave tile
-            constexpr uint32_t ROW_CHUNKS = ROW_BYTES / CHUNK; // 16 (2-byte) or 32 (4-byte)
-            constexpr uint32_t ROWS_PASS  = 32768u / ROW_BYTES; // 128 or 64 rows per pass
-            constexpr uint32_t BLOCKS_I   = ROWS_PASS / 32u; // 32-row blocks per pass
-            char*              wl         = ((wave < 2u) ? stage0 : stage1) + (wave & 1u) * 32768u;
-            const uint32_t     r32 = lane & 31u, h = lane >> 5;
-#pragma unroll
-            for(uint32_t pass = 0; pass < 4u / BLOCKS_I; ++pass)
-            {
-#pragma unroll
-                for(uint32_t ii = 0; ii < BLOCKS_I; ++ii)
-                {
-                    const uint32_t i   = pass * BLOCKS_I + ii;
-                    const uint32_t row = 32u * ii + r32; // row inside the pass
-#pragma unroll
-                    for(uint32_t j = 0; j < 4; ++j)
-#pragma unroll
-                        for(uint32_t q = 0; q < 4; ++q)
-                        {
-                            OutV out;
-#pragma unroll
-                            for(uint32_t e = 0; e < 4; ++e)
-                                out[e] = static_cast<OutT>(alpha * static_cast<AccE>(acc[i][j][4 * q + e]));
-                            if constexpr(OS == 2)
-                            {
-                                // 8 bytes: chunk 4 j + q, half h; rows 16 apart share a chunk slot, so
-                                // they take opposite halves
-                                const uint32_t c = 4u * j + q;
-                                char* dst = wl + row * ROW_BYTES + ((c ^ (row & 15u)) * CHUNK) + ((h ^ ((row >> 4) & 1u)) * 8u);
-                                *reinterpret_cast<OutV*>(dst) = out;
-                            }
-                            else
-                            {
-                                const uint32_t c = 8u * j + 2u * q + h;
-                                char* dst = wl + row * ROW_BYTES + ((c ^ (row & 31u)) * CHUNK);
-                                *reinterpret_cast<OutV*>(dst) = out;
-                            }
-                        }
-                }
-                __builtin_amdgcn_wave_barrier(); // same wave reads back what it wrote (LDS is in order per wave)
-#pragma unroll
-                for(uint32_t it = 0; it < ROWS_PASS * ROW_CHUNKS / 64u; ++it)
-                {
-                    const uint32_t L = it * 64u + lane, row = L / ROW_CHUNKS, c = L % ROW_CHUNKS;
-                    i32x4          v;
-                    if constexpr(OS == 2)
-                    {
-                        v = *reinterpret_cast<const i32x4*>(wl + row * ROW_BYTES + ((c ^ (row & 15u)) * CHUNK));
-                        if((row >> 4) & 1u)
-                            v = i32x4{v[2], v[3], v[0], v[1]};
-                    }
-                    else
-                        v = *reinterpret_cast<const i32x4*>(wl + row * ROW_BYTES + ((c ^ (row & 31u)) * CHUNK));
-                    const uint64_t offD = (uint64_t)(m0 + pass * ROWS_PASS + row) * p.ldd + n0;
-                    // D is written once and not read again: stream it past the caches
-                    __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(p.d + offD * OS + c * CHUNK));
-                }
-                __builtin_amdgcn_wave_barrier();
-            }
+    // ------------------------------------------------------------------------------------------
+    // 8-bit operands (int8, e4m3; A row-major, B col-major).  At twice the matrix-instruction rate a
+    // K stage lasts about as long as a direct load takes to arrive, so the two-buffer scheme above
+    // leaves the memory pipe idle while a refill waits for its consumer.  Here LDS holds two buffers
+    // for A and three for B (5 x 32 KiB = all 160 KiB): the B half of a stage is requested three
+    // stages ahead and the A half two, which keeps 96 KiB per CU in flight instead of 64.
+    // Stage kt lives in A buffer kt % 2 and B buffer kt % 3, so six stages bring every buffer back
+    // to its starting role.  Loads past the last stage are clamped to it -- they land in buffers
+    // nobody reads any more -- so every stage issues the same 16 loads and the wait before its
+    // barrier is always "all but the youngest 8".
+    //
+    // The direct loads are inline assembly: for the builtin the compiler cannot tell which buffer a
+    // later ds_read depends on and waits for vmcnt(0) every time, which would serialise exactly the
+    // loads that are meant to stay in flight.  Issued this way the only vmcnt waits are the ones
+    // written here.  The "memory" clobber keeps each load between the two ds_reads it is written
+    // between, which is what spreads them over the matrix instructions.
+    __device__ inline void loadToLds(i32x4 rsrc, uint32_t laneOffset, uint32_t uniformOffset, uint32_t ldsAddr)
+    {
+        asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
+                     :
+                     : "v"(laneOffset), "s"(rsrc), "s"(uniformOffset), "s"(ldsAddr)
+                     : "memory");
+    }
+
+    template <uint32_t N>
+    __device__ inline void waitVmcnt()
+    {
+        // vmcnt is split over bits [3:0] and [15:14]; expcnt and lgkmcnt stay at their maxima
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15u) | ((N >> 4) << 14));
+    }
+
+    // barrier that orders LDS traffic only: __syncthreads() also fences global memory
+    __device__ inline void ldsBarrier()
+    {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    }
+
+    template <Elem E, typename OutT>
+    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
+        gemmTiledKernel8(Params p)
+    {
+        using Traits = ElemTraits<E>;
+        using Acc    = typename Traits::Acc;
+        static_assert(Traits::Bytes == 1, "8-bit element types only");
+        constexpr uint32_t TK     = STAGE_KB; // K elements per stage
+        constexpr bool     PAIRED = (E == Elem::E4M3);
+        // LDS map: A buffers at 0 and 32 KiB, B buffers at 64, 96 and 128 KiB
+        constexpr uint32_t A_AT[2] = {0u, OPER_BYTES};
+        constexpr uint32_t B_AT[3] = {2u * OPER_BYTES, 3u * OPER_BYTES, 4u * OPER_BYTES};
+
+        __shared__ __attribute__((aligned(1024))) char lds[5u * OPER_BYTES];
+
+        uint32_t tm, tn;
+        if(!r355::tileCoord(blockIdx.x, p.tilesM, p.tilesN, tm, tn))
             return;
-        }
 
+        const uint32_t tid  = threadIdx.x;
+        const uint32_t lane = tid & 63u;
+        const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const uint32_t wm = wave >> 1, wn = wave & 1u;
+        auto           swzK = [](uint32_t row) { return (row >> 1) & 7u; };
+        const uint32_t ldsBase
+            = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds));
+
+        // global -> LDS: chunk L = j * 256 + tid of an operand tile sits at LDS byte 16 L (row L / 8)
+        const uint32_t gr = tid >> 3, gslot = tid & 7u;
+        const uint32_t gOffA = gr * p.lda + ((gslot ^ swzK(gr)) * CHUNK), gStepA = 32u * p.lda;
+        const uint32_t gOffB = gr * p.ldb + ((gslot ^ swzK(gr)) * CHUNK), gStepB = 32u * p.ldb;
+        const char*    gA = p.a + (uint64_t)tm * TILE_M * p.lda;
+        const char*    gB = p.b + (uint64_t)tn * TILE_N * p.ldb;
+        const uint32_t numStages = p.k / TK;
+        const uint32_t dmaDst    = ldsBase + wave * 64u * CHUNK; // + buffer + j * 4 KiB
+
+        // buffer resource over one stage of an operand panel (clamped to the last stage)
+        auto resource = [&](const char* panel, uint32_t stage) {
+            const uint32_t st = stage < numStages ? stage : numStages - 1u;
+            const uint64_t v  = reinterpret_cast<uint64_t>(panel + (uint64_t)st * STAGE_KB);
+            return i32x4{static_cast<int>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v))),
+                         static_cast<int>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32)) & 0xFFFF),
+                         0x7FFFFFFF, 0x00020000};
+        };
+        auto issueHalf = [&](i32x4 rsrc, uint32_t gOff, uint32_t gStep, uint32_t at) {
+#pragma unroll
+            for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
+                loadToLds(rsrc, gOff, j * gStep, dmaDst + at + j * THREADS * CHUNK);
+        };
+
+        // LDS -> registers: block i rows are i * 32 + lane % 32; sub-step s reads chunk 2 s + lane / 32
+        uint32_t rdA[4], rdB[4];
+        {
+            const uint32_t ra = wm * 128u + (lane & 31u), rb = wn * 128u + (lane & 31u);
+#pragma unroll
+            for(uint32_t s = 0; s < 4; ++s)
+            {
+                rdA[s] = ra * STAGE_KB + (((2u * s + (lane >> 5)) ^ swzK(ra)) * CHUNK);
+                rdB[s] = rb * STAGE_KB + (((2u * s + (lane >> 5)) ^ swzK(rb)) * CHUNK);
+            }
+        }
+        auto readA = [&](uint32_t at, uint32_t i, uint32_t s) -> i32x4 {
+            return *reinterpret_cast<const i32x4*>(lds + at + rdA[s] + i * 32u * STAGE_KB);
+        };
+        auto readB = [&](uint32_t at, uint32_t i, uint32_t s) -> i32x4 {
+            return *reinterpret_cast<const i32x4*>(lds + at + rdB[s] + i * 32u * STAGE_KB);
+        };
+
+        Acc acc[4][4];
 #pragma unroll
         for(uint32_t i = 0; i < 4; ++i)
-        {
 #pragma unroll
             for(uint32_t j = 0; j < 4; ++j)
+#pragma unroll
+                for(uint32_t e = 0; e < 16; ++e)
+                    acc[i][j][e] = 0;
+
+        i32x4 fa[4][4], fb[4][4];
+        auto  mfmaHalf = [&](uint32_t s0) {
+            if constexpr(PAIRED)
             {
 #pragma unroll
-                for(uint32_t q = 0; q < 4; ++q)
-                {
-                    const uint32_t row  = m0 + 32u * i + (lane & 31u);
-                    const uint32_t col  = n0 + 32u * j + 8u * q + 4u * (lane >> 5);
-                    const uint64_t offD = (uint64_t)row * p.ldd + col;
-                    const uint64_t offC = (uint64_t)row * p.ldc + col;
-                    const OutV     cv   = *reinterpret_cast<const OutV*>(p.c + offC * sizeof(OutT));
-                    OutV           out;
+                for(uint32_t i = 0; i < 4; ++i)
 #pragma unroll
-                    for(uint32_t e = 0; e < 4; ++e)
-                        out[e] = static_cast<OutT>(alpha * static_cast<AccE>(acc[i][j][4 * q + e])
-                                                   + beta * static_cast<AccE>(cv[e]));
-                    *reinterpret_cast<OutV*>(p.d + offD * sizeof(OutT)) = out;
+                    for(uint32_t j = 0; j < 4; ++j)
+                        mfma64Fp8(acc[i][j], fb[s0][j], fb[s0 + 1][j], fa[s0][i], fa[s0 + 1][i]);
+            }
+            else
+            {
+#pragma unroll
+                for(uint32_t s = s0; s < s0 + 2u; ++s)
+#pragma unroll
+                    for(uint32_t i = 0; i < 4; ++i)
+#pragma unroll
+                        for(uint32_t j = 0; j < 4; ++j)
+                            mfma32<E>(acc[i][j], fb[s][j], fa[s][i]);
+            }
+        };
+        constexpr uint32_t MFMA_PER_HALF = PAIRED ? 16u : 32u;
+
+        // One K stage: operands of sub-steps 0, 1 are in registers; 2, 3 arrive under the first half of
+        // the matrix instructions; then every wave is done with this stage's buffers, they are refilled
+        // (A two stages ahead, B three), and sub-steps 0, 1 of the next stage arrive under the second half.
+        auto stageBody = [&](uint32_t kt, uint32_t aCur, uint32_t aNxt, uint32_t bCur, uint32_t bNxt) {
+#pragma unroll
+            for(uint32_t s = 2; s < 4; ++s)
+#pragma unroll
+                for(uint32_t i = 0; i < 4; ++i)
+                {
+                    fa[s][i] = readA(aCur, i, s);
+                    fb[s][i] = readB(bCur, i, s);
+                }
+            mfmaHalf(0);
+#pragma unroll
+            for(uint32_t g = 0; g < 16; ++g)
+                schedGroup<MFMA_PER_HALF / 16u, 1, 0>();
+
+            waitVmcnt<8>(); // this wave's part of stage kt + 1 has landed (the youngest 8 loads are B of kt + 2)
+            ldsBarrier();
+
+            const i32x4 rsrcA = resource(gA, kt + 2u), rsrcB = resource(gB, kt + 3u);
+#pragma unroll
+            for(uint32_t g = 0; g < 16; ++g)
+            {
+                const uint32_t s = g >> 3, i = (g >> 1) & 3u;
+                if(g & 1u)
+                    fb[s][i] = readB(bNxt, i, s);
+                else
+                    fa[s][i] = readA(aNxt, i, s);
+                if(g < 8u)
+                    loadToLds(rsrcA, gOffA, g * gStepA, dmaDst + aCur + g * THREADS * CHUNK);
+                else
+                    loadToLds(rsrcB, gOffB, (g - 8u) * gStepB, dmaDst + bCur + (g - 8u) * THREADS * CHUNK);
+            }
+            mfmaHalf(2);
+#pragma unroll
+            for(uint32_t g = 0; g < 16; ++g)
+                schedGroup<MFMA_PER_HALF / 16u, 1, 0>();
+            __builtin_amdgcn_sched_barrier(0); // one scheduling region per stage
+        };
+
+        // prologue: stages 0 and 1 and the B half of stage 2 requested; stage 0 published
+        issueHalf(resource(gA, 0u), gOffA, gStepA, A_AT[0]);
+        issueHalf(resource(gB, 0u), gOffB, gStepB, B_AT[0]);
+        issueHalf(resource(gA, 1u), gOffA, gStepA, A_AT[1]);
+        issueHalf(resource(gB, 1u), gOffB, gStepB, B_AT[1]);
+        issueHalf(resource(gB, 2u), gOffB, gStepB, B_AT[2]);
+        waitVmcnt<24>();
+        ldsBarrier();
+#pragma unroll
+        for(uint32_t s = 0; s < 2u; ++s)
+#pragma unroll
+            for(uint32_t i = 0; i < 4; ++i)
+            {
+                fa[s][i] = readA(A_AT[0], i, s);
+                fb[s][i] = readB(B_AT[0], i, s);
+            }
+
+        // Six stages per trip.  The loop has a single exit: with an exit after every stage the register
+        // allocator rotates the accumulators through the loop and spills hundreds of registers.  The up
+        // to five remaining stages follow as straight-line code.
+        uint32_t kt = 0;
+        for(uint32_t trips = numStages / 6u; trips > 0; --trips, kt += 6u)
+        {
+            stageBody(kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1]);
+            stageBody(kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2]);
+            stageBody(kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0]);
+            stageBody(kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1]);
+            stageBody(kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2]);
+            stageBody(kt + 5u, A_AT[1], A_AT[0], B_AT[2], B_AT[0]);
+        }
+        const uint32_t rem = numStages - kt;
+        if(rem > 0u)
+        {
+            stageBody(kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1]);
+            if(rem > 1u)
+            {
+                stageBody(kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2]);
+                if(rem > 2u)
+                {
+                    stageBody(kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0]);
+                    if(rem > 3u)
+                    {
+                        stageBody(kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1]);
+                        if(rem > 4u)
+                            stageBody(kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2]);
+                    }
                 }
             }
         }
+
+        // the clamped loads of the last stages are still landing in buffers the epilogue reuses
+        waitVmcnt<0>();
+        ldsBarrier();
+        storeTile<E, OutT>(acc, p, tm, tn, wm, wn, lane, lds + wave * OPER_BYTES);
     }
 
     struct Variant
@@ -615,7 +806,7 @@ namespace
         bool banks64;
     };
     // Defaults chosen from measurements on MI355X; R355_TILED_VARIANT=<bit0: direct-to-LDS loads,
-    // bit1: 64-bank swizzle> overrides them for experiments.
+    // bit1: 64-bank swizzle> overrides them for experiments (16-bit types).
     Variant chosenVariant()
     {
         static const Variant v = [] {
@@ -649,7 +840,11 @@ namespace
     int launchLayouts(bool aK, bool bK, const Params& p, hipStream_t stream)
     {
         if constexpr(ElemTraits<E>::Bytes == 1)
-            return launchVariant<E, OutT, true, true>(p, stream);
+        {
+            const uint32_t grid = ((p.tilesM * p.tilesN + 7u) / 8u) * 8u;
+            hipLaunchKernelGGL((gemmTiledKernel8<E, OutT>), dim3(grid), dim3(THREADS), 0, stream, p);
+            return r355::checkLaunch("gemm (macro tile, 8-bit)");
+        }
         else
         {
             if(aK && bK)
@@ -679,8 +874,11 @@ namespace r355
         if(g.beta != 0.0f && g.layout_c != g.layout_d)
             return fail(R355_ERR_UNSUPPORTED, "tiled gemm: C and D must share an orientation");
         const uint32_t tk = STAGE_KB / es;
-        if(g.m % TILE_M || g.n % TILE_N || g.k % (2 * tk) || g.k == 0)
-            return fail(R355_ERR_BAD_SIZE, "tiled gemm: m=%u n=%u must be multiples of 256 and k=%u of %u", g.m, g.n, g.k, 2 * tk);
+        // the two-buffer kernel consumes K stages in pairs; the five-buffer 8-bit kernel takes any count
+        const bool     fiveBuffers = es == 1;
+        const uint32_t kGranule    = fiveBuffers ? tk : 2 * tk;
+        if(g.m % TILE_M || g.n % TILE_N || g.k % kGranule || g.k == 0)
+            return fail(R355_ERR_BAD_SIZE, "tiled gemm: m=%u n=%u must be multiples of 256 and k=%u of %u", g.m, g.n, g.k, kGranule);
         if(!aligned(g.a, 16) || !aligned(g.b, 16) || (g.lda * es) % 16 || (g.ldb * es) % 16 || !aligned(g.d, 16)
            || (g.ldd * os) % 16 || (g.beta != 0.0f && (!aligned(g.c, 16) || (g.ldc * os) % 16)))
             return fail(R355_ERR_MISALIGNED, "tiled gemm: pointers and leading dimensions of A, B, C, D must keep 16-byte alignment");
@@ -694,7 +892,7 @@ namespace r355
             plan->grid_y       = 1;
             plan->block_x      = THREADS;
             plan->block_y      = 1;
-            plan->lds_bytes    = NUM_STAGES * STAGE_BYTES;
+            plan->lds_bytes    = fiveBuffers ? 5u * OPER_BYTES : NUM_STAGES * STAGE_BYTES;
         }
         return R355_OK;
     }

@@ -161,6 +161,18 @@ def test_tiled_kernel_8bit(in_t, out_t, ldl):
     _check(in_t, out_t, got, want)
 
 
+@pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32)])
+@pytest.mark.parametrize("stages", [1, 2, 3, 4, 5, 6, 7, 11, 13])
+def test_tiled_kernel_8bit_stage_counts(in_t, out_t, stages):
+    # The 8-bit kernel rotates five LDS buffers with period six; cover every remainder of the K
+    # stage count, including a single stage and counts beyond one period.
+    m, n, k = 256, 256, 128 * stages
+    a, b, _ = _inputs(in_t, out_t, m, n, k, seed=40 + stages)
+    want = O.gemm(in_t, out_t, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0)
+    got = _run(in_t, out_t, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0, R.KERNEL_TILED)
+    _check(in_t, out_t, got, want)
+
+
 def test_tiled_kernel_many_tiles_xcd_mapping():
     # 5 x 3 tiles: a tile count that is not a multiple of 8 and a partial row group
     m, n, k = 1280, 768, 256
