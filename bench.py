@@ -162,17 +162,19 @@ def run_extras(R, O, np, torch, args):
         out[name] = {"ms": round(ms, 4), "value": round(tf, 2), "unit": unit, "peak": peak * peak_scale,
                      "frac": round(tf / (peak * peak_scale), 4)}
 
-    gemm_case("gemm_bf16_nt_8192", R.BF16, R.BF16, R.COL_MAJOR, R.ROW_MAJOR, rnd16(s * s, True), rnd16(s * s, True),
-              PEAK_TFLOPS["bf16"], "TFLOP/s")
-    gemm_case("gemm_f16_tn_8192", R.F16, R.F16, R.ROW_MAJOR, R.COL_MAJOR, rnd16(s * s, False), rnd16(s * s, False),
-              PEAK_TFLOPS["f16"], "TFLOP/s")
+    abf, bbf = rnd16(s * s, True), rnd16(s * s, True)
+    gemm_case("gemm_bf16_nt_8192", R.BF16, R.BF16, R.COL_MAJOR, R.ROW_MAJOR, abf, bbf, PEAK_TFLOPS["bf16"], "TFLOP/s")
+    af16, bf16_ = rnd16(s * s, False), rnd16(s * s, False)
+    gemm_case("gemm_f16_tn_8192", R.F16, R.F16, R.ROW_MAJOR, R.COL_MAJOR, af16, bf16_, PEAK_TFLOPS["f16"], "TFLOP/s")
     i8 = lambda nel: torch.randint(-128, 128, (nel,), dtype=torch.int16, device="cuda").to(torch.int8)
-    gemm_case("gemm_i8_tn_8192", R.I8, R.I32, R.ROW_MAJOR, R.COL_MAJOR, i8(s * s), i8(s * s), PEAK_TFLOPS["i8"], "TOP/s")
+    ai8, bi8 = i8(s * s), i8(s * s)
+    gemm_case("gemm_i8_tn_8192", R.I8, R.I32, R.ROW_MAJOR, R.COL_MAJOR, ai8, bi8, PEAK_TFLOPS["i8"], "TOP/s")
     # e4m3: N(0, 1) draws rounded to nearest-even and saturated to the finite range (|x| <= 448;
     # scale 1.0, so saturation never triggers in practice)
     f8 = lambda nel: torch.randn(nel, device="cuda").clamp_(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8)
-    gemm_case("gemm_e4m3_tn_8192", R.E4M3, R.F32, R.ROW_MAJOR, R.COL_MAJOR, f8(s * s), f8(s * s), PEAK_TFLOPS["e4m3"],
-              "TFLOP/s")
+    af8, bf8 = f8(s * s), f8(s * s)
+    gemm_case("gemm_e4m3_tn_8192", R.E4M3, R.F32, R.ROW_MAJOR, R.COL_MAJOR, af8, bf8, PEAK_TFLOPS["e4m3"], "TFLOP/s")
+    out["same_box_comparison"] = same_box_comparison(torch, args, s, af16, bf16_, abf, bbf, ai8, bi8, af8, bf8)
     # 2:4 sparse, benchmark configuration 4: M = N = 4096, dense-equivalent K = 8192, int8; dense-equivalent ops
     # against the sparse peak (2 x dense).  Every group of 4 keeps 2 values at random positions:
     # one index nibble idx0 | idx1 << 2 (idx0 < idx1) per group, two groups per metadata byte.
@@ -210,6 +212,58 @@ def run_extras(R, O, np, torch, args):
                                        "peak": HBM_PEAK_GBPS, "frac": round(byts / ms / 1e6 / HBM_PEAK_GBPS, 4),
                                        "algorithmic_bytes": byts}
     return out
+
+
+def same_box_comparison(torch, args, s, af16, bf16_, abf, bbf, ai8, bi8, af8, bf8):
+    """Context only, never part of `value`: the vendor GEMM library as torch dispatches it, on the same
+    operand bits and shapes as the cases above, and -- where its shared object was built -- the kernel of
+    the reference's samples/perf_hgemm.cpp (macro tile 128 x 128 x 16, samples/perf_hgemm.cpp:224-237,
+    515-711) compiled unchanged against this library's headers."""
+    res, flop = {}, 2.0 * s * s * s
+
+    def timed(fn):
+        for _ in range(min(args.warmup, 3)):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        n = min(args.steps, 10)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    def case(name, fn, unit="TFLOP/s"):
+        try:
+            ms = timed(fn)
+            res[name] = {"ms": round(ms, 4), "value": round(flop / ms / 1e9, 2), "unit": unit}
+        except Exception as e:  # a library without this type pair is not an error of this benchmark
+            res[name] = {"error": repr(e)[:160]}
+
+    v = lambda t, dt=None: (t if dt is None else t.view(dt)).view(s, s)
+    case("torch_matmul_f16_nt", lambda: torch.matmul(v(af16).t(), v(bf16_)))
+    case("torch_matmul_f16_tn", lambda: torch.matmul(v(af16), v(bf16_).t()))
+    case("torch_matmul_bf16_nt", lambda: torch.matmul(v(abf).t(), v(bbf)))
+    case("torch_int_mm_i8_tn", lambda: torch._int_mm(v(ai8), v(bi8).t()), "TOP/s")
+    one = torch.ones((), device="cuda")
+    f8t = torch.float8_e4m3fn
+    case("torch_scaled_mm_e4m3_tn_f32", lambda: torch._scaled_mm(v(af8, f8t), v(bf8, f8t).t(), scale_a=one, scale_b=one,
+                                                                 out_dtype=torch.float32))
+    lib = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "kernels", "_ref", "libref_perf_hgemm.so")
+    if os.path.exists(lib):
+        import ctypes
+
+        L = ctypes.CDLL(lib)
+        d = torch.empty(s * s, dtype=torch.float16, device="cuda")
+        P = lambda t: ctypes.c_void_p(t.data_ptr())
+
+        def ref():  # the wrapper synchronises after each launch
+            if L.ref_perf_hgemm(s, s, s, P(af16), P(bf16_), P(d), P(d), s, s, s, s, ctypes.c_float(1.0),
+                                ctypes.c_float(0.0)) != 0:
+                raise RuntimeError("reference sample kernel failed")
+
+        case("reference_perf_hgemm_kernel_f16_nt", ref)
+    return res
 
 
 if __name__ == "__main__":

@@ -565,6 +565,347 @@ namespace
     }
 
     // ------------------------------------------------------------------------------------------
+    // The same macro tile on the 16 x 16 matrix-instruction shapes (v_mfma_f32_16x16x32_{f16,bf16}).
+    // Under the board's power limit these sustain about a fifth more than the 32 x 32 shapes of the
+    // same types (measured with register-resident loops), and the kernel is power-bound, so it is the
+    // default for the 16-bit types.  What changes against gemmTiledKernel:
+    //   * wave tile 128 x 128 = 8 x 8 accumulators of 4 registers; a stage is two K steps of 32;
+    //     the operands of one K step (8 + 8 blocks, 128 registers for both steps) are fetched one step
+    //     ahead of their use;
+    //   * lane -> operand mapping: row lane % 16, 16-byte chunk lane / 16 of the 64-byte K step;
+    //   * the M/N-contiguous swizzle also depends on bit 3 of the k-row (a 32-lane transposing read
+    //     covers k-rows 0..3 and 8..11), which makes the global -> LDS lane offset alternate between two
+    //     values from one load to the next;
+    //   * accumulator block (i, j): lane holds D(16 i + lane % 16, 16 j + 4 (lane / 16) + 0..3).
+    using f32x4 = float __attribute__((ext_vector_type(4)));
+
+    // The compiler selects these 4-register-result instructions with a destination that is not tied
+    // to the C operand, and its register allocator then moves the 64 accumulators around inside the K
+    // loop (thousands of copies).  Written as inline assembly the accumulator is updated in place, in an
+    // AGPR.  The price: the compiler no longer knows these are matrix instructions, so the K loop below
+    // fixes the instruction order itself, and the epilogue waits out the result latency by hand.
+    template <Elem E>
+    __device__ __forceinline__ void mfma16(f32x4& acc, i32x4 x, i32x4 y)
+    {
+        if constexpr(E == Elem::F16)
+            asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc) : "v"(x), "v"(y));
+        else
+            asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(x), "v"(y));
+    }
+
+    // D = alpha * acc + beta * C for one wave's 128 x 128 tile of 16 x 16 accumulator blocks, row-major.
+    // `scratch` is 32 KiB of LDS owned by this wave.
+    template <typename AccV, typename OutT>
+    __device__ __forceinline__ void storeTile16(AccV (&acc)[8][8], const Params& p, uint32_t tm, uint32_t tn, uint32_t wm,
+                                                uint32_t wn, uint32_t lane, char* scratch)
+    {
+        using AccE = std::remove_reference_t<decltype(acc[0][0][0])>;
+        using OutV = OutT __attribute__((ext_vector_type(4)));
+        const AccE     alpha = static_cast<AccE>(p.alpha), beta = static_cast<AccE>(p.beta);
+        const uint32_t m0 = tm * TILE_M + wm * 128u, n0 = tn * TILE_N + wn * 128u;
+        const uint32_t r16 = lane & 15u, g = lane >> 4;
+
+        if(beta == static_cast<AccE>(0))
+        {
+            // Transpose through the wave's own LDS so that a store instruction covers whole 256- or
+            // 512-byte rows of D with 128 bits per lane.
+            constexpr uint32_t OS         = sizeof(OutT);
+            constexpr uint32_t ROW_BYTES  = 128u * OS;
+            constexpr uint32_t ROW_CHUNKS = ROW_BYTES / CHUNK; // 16 or 32
+            constexpr uint32_t ROWS_PASS  = 32768u / ROW_BYTES; // 128 or 64
+            constexpr uint32_t BLOCKS_I   = ROWS_PASS / 16u; // 8 or 4 row blocks per pass
+#pragma unroll
+            for(uint32_t pass = 0; pass < 8u / BLOCKS_I; ++pass)
+            {
+#pragma unroll
+                for(uint32_t ii = 0; ii < BLOCKS_I; ++ii)
+                {
+                    const uint32_t i = pass * BLOCKS_I + ii, row = 16u * ii + r16;
+#pragma unroll
+                    for(uint32_t j = 0; j < 8; ++j)
+                    {
+                        OutV out;
+#pragma unroll
+                        for(uint32_t e = 0; e < 4; ++e)
+                            out[e] = static_cast<OutT>(alpha * acc[i][j][e]);
+                        // 16 consecutive rows take 16 different chunk slots
+                        const uint32_t byteInRow = (16u * j + 4u * g) * OS;
+                        const uint32_t c = byteInRow / CHUNK, within = byteInRow % CHUNK;
+                        *reinterpret_cast<OutV*>(scratch + row * ROW_BYTES + ((c ^ (row & 15u)) * CHUNK) + within) = out;
+                    }
+                }
+                __builtin_amdgcn_wave_barrier(); // the same wave reads back what it wrote (LDS is in order per wave)
+#pragma unroll
+                for(uint32_t it = 0; it < ROWS_PASS * ROW_CHUNKS / 64u; ++it)
+                {
+                    const uint32_t L = it * 64u + lane, row = L / ROW_CHUNKS, c = L % ROW_CHUNKS;
+                    const i32x4    v = *reinterpret_cast<const i32x4*>(scratch + row * ROW_BYTES + ((c ^ (row & 15u)) * CHUNK));
+                    const uint64_t offD = (uint64_t)(m0 + pass * ROWS_PASS + row) * p.ldd + n0;
+                    // D is written once and not read again: stream it past the caches
+                    __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(p.d + offD * OS + c * CHUNK));
+                }
+                __builtin_amdgcn_wave_barrier();
+            }
+            return;
+        }
+        // C may alias D, so loads cannot move above earlier stores: fetch a block row of C at a time
+#pragma unroll
+        for(uint32_t i = 0; i < 8; ++i)
+        {
+            const uint32_t row = m0 + 16u * i + r16;
+            OutV           cv[8];
+#pragma unroll
+            for(uint32_t j = 0; j < 8; ++j)
+                cv[j] = *reinterpret_cast<const OutV*>(p.c + ((uint64_t)row * p.ldc + n0 + 16u * j + 4u * g) * sizeof(OutT));
+#pragma unroll
+            for(uint32_t j = 0; j < 8; ++j)
+            {
+                OutV out;
+#pragma unroll
+                for(uint32_t e = 0; e < 4; ++e)
+                    out[e] = static_cast<OutT>(alpha * acc[i][j][e] + beta * static_cast<AccE>(cv[j][e]));
+                *reinterpret_cast<OutV*>(p.d + ((uint64_t)row * p.ldd + n0 + 16u * j + 4u * g) * sizeof(OutT)) = out;
+            }
+        }
+    }
+
+    template <Elem E, typename OutT, bool A_KCONTIG, bool B_KCONTIG>
+    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
+        gemmTiledKernel16(Params p)
+    {
+        constexpr uint32_t ES = ElemTraits<E>::Bytes;
+        constexpr uint32_t TK = STAGE_KB / ES; // 64 K elements per stage = two K steps of 32
+        static_assert(ES == 2, "16-bit element types only");
+        // LDS reads per K step: one 128-bit read per operand block, or two transposing 64-bit reads
+        constexpr uint32_t READS_A = A_KCONTIG ? 8u : 16u, READS_B = B_KCONTIG ? 8u : 16u;
+        constexpr uint32_t READS   = READS_A + READS_B; // 16, 24 or 32
+
+        // One variable per stage: the compiler tracks outstanding direct-to-LDS loads per LDS variable.
+        __shared__ __attribute__((aligned(1024))) char stage0[STAGE_BYTES];
+        __shared__ __attribute__((aligned(1024))) char stage1[STAGE_BYTES];
+
+        uint32_t tm, tn;
+        if(!r355::tileCoord(blockIdx.x, p.tilesM, p.tilesN, tm, tn))
+            return;
+
+        const uint32_t tid  = threadIdx.x;
+        const uint32_t lane = tid & 63u;
+        const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const uint32_t wm = wave >> 1, wn = wave & 1u;
+        auto           swzK  = [](uint32_t row) { return (row >> 1) & 7u; };
+        auto           swzMN = [](uint32_t krow) { return ((krow & 3u) << 2) | (((krow >> 3) & 1u) << 1); };
+
+        // ---------------- global -> LDS: chunk L = j * 256 + tid of an operand tile sits at LDS byte 16 L.
+        // K-contiguous: row L / 8, and the swizzle does not change with j (32 rows per load).
+        // M/N-contiguous: k-row L / 32 = 8 j + tid / 32; the swizzle alternates with bit 3 of the k-row.
+        uint32_t gOffA[2], gOffB[2], gStepA, gStepB;
+        uint64_t gStageA, gStageB;
+        if constexpr(A_KCONTIG)
+        {
+            const uint32_t r = tid >> 3, slot = tid & 7u;
+            gOffA[0] = gOffA[1] = r * p.lda * ES + ((slot ^ swzK(r)) * CHUNK);
+            gStepA = 32u * p.lda * ES, gStageA = STAGE_KB;
+        }
+        else
+        {
+            const uint32_t r = tid >> 5, slot = tid & 31u;
+            gOffA[0] = r * p.lda * ES + ((slot ^ swzMN(r)) * CHUNK);
+            gOffA[1] = r * p.lda * ES + ((slot ^ swzMN(r + 8u)) * CHUNK);
+            gStepA = 8u * p.lda * ES, gStageA = (uint64_t)TK * p.lda * ES;
+        }
+        if constexpr(B_KCONTIG)
+        {
+            const uint32_t r = tid >> 3, slot = tid & 7u;
+            gOffB[0] = gOffB[1] = r * p.ldb * ES + ((slot ^ swzK(r)) * CHUNK);
+            gStepB = 32u * p.ldb * ES, gStageB = STAGE_KB;
+        }
+        else
+        {
+            const uint32_t r = tid >> 5, slot = tid & 31u;
+            gOffB[0] = r * p.ldb * ES + ((slot ^ swzMN(r)) * CHUNK);
+            gOffB[1] = r * p.ldb * ES + ((slot ^ swzMN(r + 8u)) * CHUNK);
+            gStepB = 8u * p.ldb * ES, gStageB = (uint64_t)TK * p.ldb * ES;
+        }
+        const char* gA = p.a + (A_KCONTIG ? (uint64_t)tm * TILE_M * p.lda * ES : (uint64_t)tm * TILE_M * ES);
+        const char* gB = p.b + (B_KCONTIG ? (uint64_t)tn * TILE_N * p.ldb * ES : (uint64_t)tn * TILE_N * ES);
+
+        // ---------------- LDS -> registers (per lane, fixed)
+        // K-contiguous: block i rows are 16 i + lane % 16; K step s reads chunk 4 s + lane / 16.
+        // M/N-contiguous: K step s, half h: k-row 32 s + 8 (lane / 16) + 4 h + (lane % 16) / 4,
+        //                 8-byte piece m / 4 with m = 16 i + 4 (lane % 4).
+        uint32_t rdA[8], rdB[8];
+        const uint32_t t = lane & 15u, g = lane >> 4;
+        if constexpr(A_KCONTIG)
+        {
+            const uint32_t r = wm * 128u + t;
+            rdA[0] = r * STAGE_KB + ((g ^ swzK(r)) * CHUNK);
+            rdA[1] = r * STAGE_KB + (((4u + g) ^ swzK(r)) * CHUNK);
+        }
+        else
+        {
+            const uint32_t kr = 8u * g + (t >> 2);
+#pragma unroll
+            for(uint32_t i = 0; i < 8; ++i)
+            {
+                const uint32_t piece = wm * 32u + 4u * i + (t & 3u);
+                rdA[i] = kr * 512u + (((piece >> 1) ^ swzMN(kr)) * CHUNK) + (piece & 1u) * 8u;
+            }
+        }
+        if constexpr(B_KCONTIG)
+        {
+            const uint32_t r = wn * 128u + t;
+            rdB[0] = OPER_BYTES + r * STAGE_KB + ((g ^ swzK(r)) * CHUNK);
+            rdB[1] = OPER_BYTES + r * STAGE_KB + (((4u + g) ^ swzK(r)) * CHUNK);
+        }
+        else
+        {
+            const uint32_t kr = 8u * g + (t >> 2);
+#pragma unroll
+            for(uint32_t i = 0; i < 8; ++i)
+            {
+                const uint32_t piece = wn * 32u + 4u * i + (t & 3u);
+                rdB[i] = OPER_BYTES + kr * 512u + (((piece >> 1) ^ swzMN(kr)) * CHUNK) + (piece & 1u) * 8u;
+            }
+        }
+        using lpt = __attribute__((address_space(3))) trv4*;
+        auto readA = [&](const char* base, uint32_t i, uint32_t s) -> i32x4 {
+            if constexpr(A_KCONTIG)
+                return *reinterpret_cast<const i32x4*>(base + rdA[s] + i * 16u * STAGE_KB);
+            else
+            {
+                const char* q  = base + rdA[i] + s * 32u * 512u;
+                const i32x2 lo = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lpt)q));
+                const i32x2 hi = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lpt)(q + 4u * 512u)));
+                return i32x4{lo[0], lo[1], hi[0], hi[1]};
+            }
+        };
+        auto readB = [&](const char* base, uint32_t i, uint32_t s) -> i32x4 {
+            if constexpr(B_KCONTIG)
+                return *reinterpret_cast<const i32x4*>(base + rdB[s] + i * 16u * STAGE_KB);
+            else
+            {
+                const char* q  = base + rdB[i] + s * 32u * 512u;
+                const i32x2 lo = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lpt)q));
+                const i32x2 hi = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lpt)(q + 4u * 512u)));
+                return i32x4{lo[0], lo[1], hi[0], hi[1]};
+            }
+        };
+
+        // ---------------- global -> LDS, written by the memory pipeline: 16 loads per stage
+        auto stageRsrc = [&](const char* panel) {
+            const uint64_t v  = reinterpret_cast<uint64_t>(panel);
+            const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+            const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+            // raw buffer, 32-bit data format, no swizzle
+            return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>((static_cast<uint64_t>(hi) << 32) | lo), 0,
+                                                     0x7FFFFFFF, 0x00020000);
+        };
+        // load x of a stage: x = 2 j loads piece j of A, x = 2 j + 1 piece j of B
+        auto issueLoad = [&](__amdgpu_buffer_rsrc_t srcA, __amdgpu_buffer_rsrc_t srcB, char* stage, uint32_t x) {
+            using lp         = __attribute__((address_space(3))) void*;
+            const uint32_t j = x >> 1;
+            char*          dst = stage + (j * THREADS + wave * 64u) * CHUNK;
+            if(x & 1u)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(srcB, (lp)(dst + OPER_BYTES), 16, gOffB[j & 1u], j * gStepB, 0, 0);
+            else
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(srcA, (lp)dst, 16, gOffA[j & 1u], j * gStepA, 0, 0);
+        };
+        auto issueGlobal = [&](uint32_t kt, char* stage) {
+            const __amdgpu_buffer_rsrc_t srcA = stageRsrc(gA + kt * gStageA), srcB = stageRsrc(gB + kt * gStageB);
+#pragma unroll
+            for(uint32_t x = 0; x < 2u * LOADS_PER_OPER; ++x)
+                issueLoad(srcA, srcB, stage, x);
+        };
+
+        f32x4          acc[8][8];
+        const uint32_t numStages = p.k / TK;
+#pragma unroll
+        for(uint32_t i = 0; i < 8; ++i)
+#pragma unroll
+            for(uint32_t j = 0; j < 8; ++j)
+                acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+        i32x4 fa[2][8], fb[2][8];
+        // Matrix instruction n (0..63) of a K step works on accumulator block (i, j) = blockOf(n): block
+        // row / column d is first needed after d * d instructions, and the operands arrive in the
+        // order A0 B0 A1 B1 ...  Operands swapped: each lane then holds 4 consecutive columns of a row of D.
+        auto mfmaAt = [&](uint32_t s, uint32_t n) {
+            uint32_t d = 0;
+            while((d + 1u) * (d + 1u) <= n)
+                ++d;
+            const uint32_t r = n - d * d; // 0..2d within the L-shaped shell d
+            const uint32_t i = r <= d ? d : r - d - 1u, j = r <= d ? r : d;
+            mfma16<E>(acc[i][j], fb[s][j], fa[s][i]);
+        };
+        // operand block x of K step s: x = 2 i is A block i, x = 2 i + 1 is B block i
+        auto readAt = [&](const char* base, uint32_t s, uint32_t x) {
+            if(x & 1u)
+                fb[s][x >> 1] = readB(base, x >> 1, s);
+            else
+                fa[s][x >> 1] = readA(base, x >> 1, s);
+        };
+        auto readStep = [&](const char* base, uint32_t s) {
+#pragma unroll
+            for(uint32_t x = 0; x < 16; ++x)
+                readAt(base, s, x);
+        };
+
+        // One K stage; `cur` / `nxt` are the LDS buffers of stage kt / kt + 1.  K step 0 is in registers:
+        // step 1 arrives under its matrix instructions; then every wave holds the rest of `cur` in
+        // registers, so after the barrier `cur` is refilled with stage kt + 2 while step 0 of stage
+        // kt + 1 arrives from `nxt` under the matrix instructions of step 1.  Sixteen groups per K step:
+        // four matrix instructions, one operand block read, (second step) one direct load; nothing
+        // moves between groups.  Every stage runs the same code: past the end the refill is clamped to
+        // the last stage and the operands read ahead are never used.
+        auto stageBody = [&](uint32_t kt, char* cur, char* nxt) {
+#pragma unroll
+            for(uint32_t x = 0; x < 16; ++x)
+            {
+#pragma unroll
+                for(uint32_t n = 4u * x; n < 4u * x + 4u; ++n)
+                    mfmaAt(0, n);
+                readAt(cur, 1, x);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): stage kt + 1 has landed
+            __syncthreads();
+            const uint32_t               kr   = kt + 2u < numStages ? kt + 2u : numStages - 1u;
+            const __amdgpu_buffer_rsrc_t srcA = stageRsrc(gA + kr * gStageA), srcB = stageRsrc(gB + kr * gStageB);
+#pragma unroll
+            for(uint32_t x = 0; x < 16; ++x)
+            {
+#pragma unroll
+                for(uint32_t n = 4u * x; n < 4u * x + 4u; ++n)
+                    mfmaAt(1, n);
+                readAt(nxt, 0, x);
+                issueLoad(srcA, srcB, cur, x);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+
+        // prologue: stage 0 resident, stage 1 in flight, first operands in registers
+        issueGlobal(0, stage0);
+        issueGlobal(1, stage1);
+        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+        __syncthreads();
+        readStep(stage0, 0);
+
+        // numStages is even (checked on the host)
+        for(uint32_t kt = 0; kt < numStages; kt += 2)
+        {
+            stageBody(kt, stage0, stage1);
+            stageBody(kt + 1, stage1, stage0);
+        }
+
+        // the clamped refills of the last two stages are still landing in the buffers the epilogue reuses
+        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+        __syncthreads();
+        // the last matrix instructions are still in the pipeline and the compiler does not know it
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+        storeTile16<f32x4, OutT>(acc, p, tm, tn, wm, wn, lane, ((wave < 2u) ? stage0 : stage1) + (wave & 1u) * 32768u);
+    }
+
+    // ------------------------------------------------------------------------------------------
     // 8-bit operands (int8, e4m3; A row-major, B col-major).  At twice the matrix-instruction rate a
     // K stage lasts about as long as a direct load takes to arrive, so the two-buffer scheme above
     // leaves the memory pipe idle while a refill waits for its consumer.  Here LDS holds two buffers
@@ -804,19 +1145,21 @@ namespace
     {
         bool direct;
         bool banks64;
+        bool shape32; // 16-bit types on the 32 x 32 x 16 instruction shapes (the earlier kernel)
     };
     // Defaults chosen from measurements on MI355X; R355_TILED_VARIANT=<bit0: direct-to-LDS loads,
-    // bit1: 64-bank swizzle> overrides them for experiments (16-bit types).
+    // bit1: 64-bank swizzle, bit2: 32 x 32 instruction shapes> overrides them for experiments (16-bit types).
     Variant chosenVariant()
     {
         static const Variant v = [] {
-            Variant     r{true, true};
+            Variant     r{true, true, false};
             const char* e = getenv("R355_TILED_VARIANT");
             if(e)
             {
                 int x     = atoi(e);
                 r.direct  = x & 1;
                 r.banks64 = x & 2;
+                r.shape32 = x & 4;
             }
             return r;
         }();
@@ -829,7 +1172,9 @@ namespace
         const Variant  v    = chosenVariant();
         const uint32_t grid = ((p.tilesM * p.tilesN + 7u) / 8u) * 8u;
         p.banks64           = v.banks64;
-        if(v.direct)
+        if(!v.shape32)
+            hipLaunchKernelGGL((gemmTiledKernel16<E, OutT, AK, BK>), dim3(grid), dim3(THREADS), 0, stream, p);
+        else if(v.direct)
             hipLaunchKernelGGL((gemmTiledKernel<E, OutT, AK, BK, true>), dim3(grid), dim3(THREADS), 0, stream, p);
         else
             hipLaunchKernelGGL((gemmTiledKernel<E, OutT, AK, BK, false>), dim3(grid), dim3(THREADS), 0, stream, p);

@@ -6,6 +6,7 @@
 //   host_bench gemm  [--type f16|bf16|i8|e4m3] [--out f16|bf16|f32|i32] [--layout nt|tn|nn|tt]
 //                    [--m M --n N --k K] [--kernel auto|simple|tiled] [--warmup W --iters I]
 //                    [--sparse 1]   A is 2:4 structured sparse (compressed values + index nibbles)
+//                    [--ldpad E]    lda and ldb grow by E elements (power-of-two strides cost L2 efficiency)
 //   host_bench dlrm  [--type f16|bf16|f32] [--bwd 1] [--batch B --m M --k K] [--warmup W --iters I]
 //   host_bench gemv  [--m M --k K --layout n|t]
 //   host_bench copy  [--bytes N]      plain device copy of known size (counter calibration)
@@ -101,7 +102,7 @@ namespace
     using f16x8  = _Float16 __attribute__((ext_vector_type(8)));
     using bf16x8 = __bf16 __attribute__((ext_vector_type(8)));
 
-    enum MfmaKind { MF_F16, MF_BF16, MF_I8, MF_FP8_K64, MF_SPARSE_I8, MF_KINDS };
+    enum MfmaKind { MF_F16, MF_BF16, MF_I8, MF_FP8_K64, MF_SPARSE_I8, MF_F16_16, MF_I8_16, MF_FP8_16, MF_KINDS };
 
     // 16 MFMAs per loop trip on 4 x 4 operand registers; no memory traffic inside the loop.
     template <int T>
@@ -150,6 +151,48 @@ namespace
         out[blockIdx.x * 256 + threadIdx.x] = s;
     }
 
+    // The 16 x 16 shapes of the same types: 64 independent 4-register accumulators (same register
+    // footprint and flop per loop trip as the 32 x 32 loop above).
+    using f32x4 = float __attribute__((ext_vector_type(4)));
+    template <int T>
+    __global__ void __launch_bounds__(256) mfmaLoop16(const i32x4* __restrict__ in, float* __restrict__ out, int iters)
+    {
+        i32x4 a[4], b[4];
+        for(int i = 0; i < 4; ++i)
+        {
+            a[i] = in[(threadIdx.x + i * 256) % 1024];
+            b[i] = in[(threadIdx.x * 3 + i * 131) % 1024];
+        }
+        f32x4 acc[64];
+        i32x4 iacc[64];
+        for(int i = 0; i < 64; ++i)
+            for(int e = 0; e < 4; ++e)
+                acc[i][e] = 0.0f, iacc[i][e] = 0;
+        for(int it = 0; it < iters; ++it)
+        {
+#pragma unroll
+            for(int x = 0; x < 64; ++x)
+            {
+                const int  i = x & 3, j = (x >> 2) & 3;
+                const auto a8 = __builtin_shufflevector(a[i], a[(i + 1) & 3], 0, 1, 2, 3, 4, 5, 6, 7);
+                const auto b8 = __builtin_shufflevector(b[j], b[(j + 1) & 3], 0, 1, 2, 3, 4, 5, 6, 7);
+                if constexpr(T == MF_F16_16)
+                    acc[x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a[i]),
+                                                                    __builtin_bit_cast(f16x8, b[j]), acc[x], 0, 0, 0);
+                else if constexpr(T == MF_I8_16)
+                    iacc[x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i], b[j], iacc[x], 0, 0, 0);
+                else
+                    acc[x] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, acc[x], 0, 0, 0, 0x7F7F7F7F, 0,
+                                                                              0x7F7F7F7F);
+            }
+        }
+        float s = 0.0f;
+        for(int i = 0; i < 64; ++i)
+            for(int e = 0; e < 4; ++e)
+                s += acc[i][e] + static_cast<float>(iacc[i][e]);
+        out[blockIdx.x * 256 + threadIdx.x] = s;
+    }
+
     void launchMfma(int kind, int cus, const i32x4* in, float* out, int iters)
     {
         const dim3 g(cus), b(256);
@@ -159,7 +202,10 @@ namespace
         case MF_BF16: hipLaunchKernelGGL(mfmaLoop<MF_BF16>, g, b, 0, 0, in, out, iters); break;
         case MF_I8: hipLaunchKernelGGL(mfmaLoop<MF_I8>, g, b, 0, 0, in, out, iters); break;
         case MF_FP8_K64: hipLaunchKernelGGL(mfmaLoop<MF_FP8_K64>, g, b, 0, 0, in, out, iters); break;
-        default: hipLaunchKernelGGL(mfmaLoop<MF_SPARSE_I8>, g, b, 0, 0, in, out, iters); break;
+        case MF_SPARSE_I8: hipLaunchKernelGGL(mfmaLoop<MF_SPARSE_I8>, g, b, 0, 0, in, out, iters); break;
+        case MF_F16_16: hipLaunchKernelGGL(mfmaLoop16<MF_F16_16>, g, b, 0, 0, in, out, iters); break;
+        case MF_I8_16: hipLaunchKernelGGL(mfmaLoop16<MF_I8_16>, g, b, 0, 0, in, out, iters); break;
+        default: hipLaunchKernelGGL(mfmaLoop16<MF_FP8_16>, g, b, 0, 0, in, out, iters); break;
         }
     }
 
@@ -180,7 +226,7 @@ int main(int argc, char** argv)
     const std::string op = argv[1];
     std::string       type = "f16", out = "", layout = "nt", kernel = "auto";
     bool              sparse = false, itersSet = false, bwd = false;
-    uint32_t          m = 8192, n = 8192, k = 8192, batch = 65536;
+    uint32_t          m = 8192, n = 8192, k = 8192, batch = 65536, ldpad = 0;
     bool              mSet = false, kSet = false;
     int               warmup = 2, iters = 10;
     size_t            bytes = 1ull << 30;
@@ -195,6 +241,7 @@ int main(int argc, char** argv)
         else if(a == "--n") n = atoi(v.c_str());
         else if(a == "--k") k = atoi(v.c_str()), kSet = true;
         else if(a == "--batch") batch = atoi(v.c_str());
+        else if(a == "--ldpad") ldpad = atoi(v.c_str()); // elements added to lda and ldb (dense GEMM)
         else if(a == "--warmup") warmup = atoi(v.c_str());
         else if(a == "--iters") iters = atoi(v.c_str()), itersSet = true;
         else if(a == "--sparse") sparse = atoi(v.c_str()) != 0;
@@ -227,12 +274,14 @@ int main(int argc, char** argv)
         g.layout_b = layout[1] == 't' ? R355_ROW_MAJOR : R355_COL_MAJOR;
         g.layout_c = g.layout_d = R355_ROW_MAJOR;
         g.m = m, g.n = n, g.k = k;
-        g.lda = g.layout_a == R355_ROW_MAJOR ? k : m;
-        g.ldb = g.layout_b == R355_ROW_MAJOR ? n : k;
+        g.lda = (g.layout_a == R355_ROW_MAJOR ? k : m) + ldpad;
+        g.ldb = (g.layout_b == R355_ROW_MAJOR ? n : k) + ldpad;
         g.ldc = g.ldd = n;
         g.alpha = 1.0f, g.beta = 0.0f;
         g.kernel = kernel == "simple" ? R355_KERNEL_SIMPLE : (kernel == "tiled" ? R355_KERNEL_TILED : R355_KERNEL_AUTO);
-        std::vector<uint8_t> ha((size_t)m * k * bytesOf(inT) / (sparse ? 2 : 1)), hb((size_t)k * n * bytesOf(inT));
+        const size_t rowsA = g.layout_a == R355_ROW_MAJOR ? m : k, rowsB = g.layout_b == R355_ROW_MAJOR ? k : n;
+        std::vector<uint8_t> ha(sparse ? (size_t)m * k * bytesOf(inT) / 2 : rowsA * g.lda * bytesOf(inT)),
+            hb(rowsB * g.ldb * bytesOf(inT));
         fillBytes(ha, inT, 1);
         fillBytes(hb, inT, 2);
         void *da, *db, *dd, *dmeta = nullptr;
@@ -365,10 +414,13 @@ int main(int argc, char** argv)
         HIP_OK(hipEventCreate(&e0));
         HIP_OK(hipEventCreate(&e1));
         static const char*  names[MF_KINDS] = {"f16 32x32x16", "bf16 32x32x16", "i8 32x32x32", "fp8 f8f6f4 32x32x64",
-                                               "sparse i8 smfmac 32x32x64 (dense-equivalent ops)"};
+                                               "sparse i8 smfmac 32x32x64 (dense-equivalent ops)", "f16 16x16x32",
+                                               "i8 16x16x64", "fp8 f8f6f4 16x16x128"};
+        // flop per loop trip and wave: 16 instructions of the 32 x 32 shapes, 64 of the 16 x 16 shapes
         static const double flopPer[MF_KINDS]
-            = {2.0 * 32 * 32 * 16, 2.0 * 32 * 32 * 16, 2.0 * 32 * 32 * 32, 2.0 * 32 * 32 * 64, 2.0 * 32 * 32 * 64};
-        static const double vendorPeak[MF_KINDS] = {2500.0, 2500.0, 5000.0, 5000.0, 10000.0};
+            = {2.0 * 32 * 32 * 16, 2.0 * 32 * 32 * 16, 2.0 * 32 * 32 * 32, 2.0 * 32 * 32 * 64, 2.0 * 32 * 32 * 64,
+               4 * 2.0 * 16 * 16 * 32, 4 * 2.0 * 16 * 16 * 64, 4 * 2.0 * 16 * 16 * 128};
+        static const double vendorPeak[MF_KINDS] = {2500.0, 2500.0, 5000.0, 5000.0, 10000.0, 2500.0, 5000.0, 5000.0};
         printf("[");
         for(int random = 0; random < 2; ++random)
             for(int kind = 0; kind < MF_KINDS; ++kind)
@@ -379,7 +431,8 @@ int main(int argc, char** argv)
                     const uint32_t r = static_cast<uint32_t>(splitmix(7 + kind, i));
                     h[i] = kind == MF_F16    ? ((r & 0x8FFF8FFFu) | 0x30003000u)  // |x| in [1/8, 1)
                            : kind == MF_BF16 ? ((r & 0x807F807Fu) | 0x3E003E00u)  // |x| in [1/8, 1/4)
-                           : kind == MF_FP8_K64 ? ((r & 0x87878787u) | 0x30303030u) // |x| in [1/2, 1)
+                           : kind == MF_F16_16 ? ((r & 0x8FFF8FFFu) | 0x30003000u)
+                           : (kind == MF_FP8_K64 || kind == MF_FP8_16) ? ((r & 0x87878787u) | 0x30303030u) // |x| in [1/2, 1)
                                                 : r;
                 }
                 HIP_OK(hipMemcpy(in, h.data(), h.size() * 4, hipMemcpyHostToDevice));
