@@ -699,7 +699,7 @@ namespace
         // K-contiguous: row L / 8, and the swizzle does not change with j (32 rows per load).
         // M/N-contiguous: k-row L / 32 = 8 j + tid / 32; the swizzle alternates with bit 3 of the k-row.
         uint32_t gOffA[2], gOffB[2], gStepA, gStepB;
-        uint64_t gStageA, gStageB;
+        uint64_t gStageA, gStageB; // bytes between consecutive K stages
         if constexpr(A_KCONTIG)
         {
             const uint32_t r = tid >> 3, slot = tid & 7u;
@@ -767,39 +767,48 @@ namespace
                 rdB[i] = OPER_BYTES + kr * 512u + (((piece >> 1) ^ swzMN(kr)) * CHUNK) + (piece & 1u) * 8u;
             }
         }
+        // An operand block arrives in one 128-bit read (part 0) or in two transposing 64-bit reads
+        // (parts 0 and 1, the low and high four K values of each lane).
         using lpt = __attribute__((address_space(3))) trv4*;
-        auto readA = [&](const char* base, uint32_t i, uint32_t s) -> i32x4 {
+        auto readA = [&](const char* base, uint32_t i, uint32_t s, uint32_t part, i32x4& dst) {
             if constexpr(A_KCONTIG)
-                return *reinterpret_cast<const i32x4*>(base + rdA[s] + i * 16u * STAGE_KB);
+            {
+                if(part == 0u)
+                    dst = *reinterpret_cast<const i32x4*>(base + rdA[s] + i * 16u * STAGE_KB);
+            }
             else
             {
-                const char* q  = base + rdA[i] + s * 32u * 512u;
-                const i32x2 lo = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lpt)q));
-                const i32x2 hi = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lpt)(q + 4u * 512u)));
-                return i32x4{lo[0], lo[1], hi[0], hi[1]};
+                const char* q = base + rdA[i] + s * 32u * 512u + part * 4u * 512u;
+                const i32x2 v = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lpt)q));
+                dst[2u * part] = v[0], dst[2u * part + 1u] = v[1];
             }
         };
-        auto readB = [&](const char* base, uint32_t i, uint32_t s) -> i32x4 {
+        auto readB = [&](const char* base, uint32_t i, uint32_t s, uint32_t part, i32x4& dst) {
             if constexpr(B_KCONTIG)
-                return *reinterpret_cast<const i32x4*>(base + rdB[s] + i * 16u * STAGE_KB);
+            {
+                if(part == 0u)
+                    dst = *reinterpret_cast<const i32x4*>(base + rdB[s] + i * 16u * STAGE_KB);
+            }
             else
             {
-                const char* q  = base + rdB[i] + s * 32u * 512u;
-                const i32x2 lo = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lpt)q));
-                const i32x2 hi = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lpt)(q + 4u * 512u)));
-                return i32x4{lo[0], lo[1], hi[0], hi[1]};
+                const char* q = base + rdB[i] + s * 32u * 512u + part * 4u * 512u;
+                const i32x2 v = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lpt)q));
+                dst[2u * part] = v[0], dst[2u * part + 1u] = v[1];
             }
         };
 
         // ---------------- global -> LDS, written by the memory pipeline: 16 loads per stage
-        auto stageRsrc = [&](const char* panel) {
-            const uint64_t v  = reinterpret_cast<uint64_t>(panel);
+        // wave-uniform addresses are kept as integers the compiler can see are uniform
+        auto uniform64 = [](const char* ptr) {
+            const uint64_t v  = reinterpret_cast<uint64_t>(ptr);
             const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
             const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
-            // raw buffer, 32-bit data format, no swizzle
-            return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>((static_cast<uint64_t>(hi) << 32) | lo), 0,
-                                                     0x7FFFFFFF, 0x00020000);
+            return (static_cast<uint64_t>(hi) << 32) | lo;
         };
+        auto rsrcAt = [](uint64_t addr) { // raw buffer, 32-bit data format, no swizzle
+            return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>(addr), 0, 0x7FFFFFFF, 0x00020000);
+        };
+        auto stageRsrc = [&](const char* panel) { return rsrcAt(uniform64(panel)); };
         // load x of a stage: x = 2 j loads piece j of A, x = 2 j + 1 piece j of B
         auto issueLoad = [&](__amdgpu_buffer_rsrc_t srcA, __amdgpu_buffer_rsrc_t srcB, char* stage, uint32_t x) {
             using lp         = __attribute__((address_space(3))) void*;
@@ -825,7 +834,8 @@ namespace
             for(uint32_t j = 0; j < 8; ++j)
                 acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-        i32x4 fa[2][8], fb[2][8];
+        i32x4    fa[2][8], fb[2][8];
+        uint64_t refillA, refillB; // where the next refill reads from (stage kt + 2, clamped to the last stage)
         // Matrix instruction n (0..63) of a K step works on accumulator block (i, j) = blockOf(n): block
         // row / column d is first needed after d * d instructions, and the operands arrive in the
         // order A0 B0 A1 B1 ...  Operands swapped: each lane then holds 4 consecutive columns of a row of D.
@@ -838,48 +848,61 @@ namespace
             mfma16<E>(acc[i][j], fb[s][j], fa[s][i]);
         };
         // operand block x of K step s: x = 2 i is A block i, x = 2 i + 1 is B block i
-        auto readAt = [&](const char* base, uint32_t s, uint32_t x) {
+        auto readAt = [&](const char* base, uint32_t s, uint32_t x, uint32_t part) {
             if(x & 1u)
-                fb[s][x >> 1] = readB(base, x >> 1, s);
+                readB(base, x >> 1, s, part, fb[s][x >> 1]);
             else
-                fa[s][x >> 1] = readA(base, x >> 1, s);
+                readA(base, x >> 1, s, part, fa[s][x >> 1]);
         };
         auto readStep = [&](const char* base, uint32_t s) {
 #pragma unroll
             for(uint32_t x = 0; x < 16; ++x)
-                readAt(base, s, x);
+            {
+                readAt(base, s, x, 0);
+                readAt(base, s, x, 1);
+            }
         };
 
         // One K stage; `cur` / `nxt` are the LDS buffers of stage kt / kt + 1.  K step 0 is in registers:
         // step 1 arrives under its matrix instructions; then every wave holds the rest of `cur` in
         // registers, so after the barrier `cur` is refilled with stage kt + 2 while step 0 of stage
-        // kt + 1 arrives from `nxt` under the matrix instructions of step 1.  Sixteen groups per K step:
-        // four matrix instructions, one operand block read, (second step) one direct load; nothing
-        // moves between groups.  Every stage runs the same code: past the end the refill is clamped to
-        // the last stage and the operands read ahead are never used.
+        // kt + 1 arrives from `nxt` under the matrix instructions of step 1.  A matrix instruction
+        // occupies its pipeline for 16 cycles and the wave can issue about three other instructions
+        // in that time, so the other work is dealt out one piece per matrix instruction, in groups of
+        // four: read (part 0), read (part 1), direct load (second step), nothing -- and nothing moves
+        // between pieces.  Every stage runs the same code: past the end the refill is clamped to the
+        // last stage and the operands read ahead are never used.
         auto stageBody = [&](uint32_t kt, char* cur, char* nxt) {
 #pragma unroll
             for(uint32_t x = 0; x < 16; ++x)
             {
 #pragma unroll
-                for(uint32_t n = 4u * x; n < 4u * x + 4u; ++n)
-                    mfmaAt(0, n);
-                readAt(cur, 1, x);
-                __builtin_amdgcn_sched_barrier(0);
+                for(uint32_t q = 0; q < 4; ++q)
+                {
+                    mfmaAt(0, 4u * x + q);
+                    if(q < 2u)
+                        readAt(cur, 1, x, q);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
             __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): stage kt + 1 has landed
             __syncthreads();
-            const uint32_t               kr   = kt + 2u < numStages ? kt + 2u : numStages - 1u;
-            const __amdgpu_buffer_rsrc_t srcA = stageRsrc(gA + kr * gStageA), srcB = stageRsrc(gB + kr * gStageB);
+            const __amdgpu_buffer_rsrc_t srcA = rsrcAt(refillA), srcB = rsrcAt(refillB);
+            if(kt + 3u < numStages) // the refill of the next stage is one stage further, or the last again
+                refillA += gStageA, refillB += gStageB;
 #pragma unroll
             for(uint32_t x = 0; x < 16; ++x)
             {
 #pragma unroll
-                for(uint32_t n = 4u * x; n < 4u * x + 4u; ++n)
-                    mfmaAt(1, n);
-                readAt(nxt, 0, x);
-                issueLoad(srcA, srcB, cur, x);
-                __builtin_amdgcn_sched_barrier(0);
+                for(uint32_t q = 0; q < 4; ++q)
+                {
+                    mfmaAt(1, 4u * x + q);
+                    if(q < 2u)
+                        readAt(nxt, 0, x, q);
+                    else if(q == 2u)
+                        issueLoad(srcA, srcB, cur, x);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
         };
 
@@ -889,6 +912,8 @@ namespace
         __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
         __syncthreads();
         readStep(stage0, 0);
+        refillA = uniform64(gA + (numStages > 2u ? 2u : numStages - 1u) * gStageA);
+        refillB = uniform64(gB + (numStages > 2u ? 2u : numStages - 1u) * gStageB);
 
         // numStages is even (checked on the host)
         for(uint32_t kt = 0; kt < numStages; kt += 2)
