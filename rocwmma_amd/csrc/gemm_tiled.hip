@@ -1166,6 +1166,195 @@ namespace
         storeTile<E, OutT>(acc, p, tm, tn, wm, wn, lane, lds + wave * OPER_BYTES);
     }
 
+    // ------------------------------------------------------------------------------------------
+    // int8 on v_mfma_i32_16x16x64_i8: the five-buffer scheme of gemmTiledKernel8 with the K-step
+    // structure and the in-place inline-assembly accumulators of gemmTiledKernel16.  A stage is two
+    // K steps of 64 bytes; lane -> operand mapping: row lane % 16, 16-byte chunk lane / 16 of the step.
+    using i32x4v = int __attribute__((ext_vector_type(4)));
+    __device__ __forceinline__ void mfma16i8(i32x4v& acc, i32x4 x, i32x4 y)
+    {
+        asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc) : "v"(x), "v"(y));
+    }
+
+    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) gemmTiledKernelI8(Params p)
+    {
+        // LDS map: A buffers at 0 and 32 KiB, B buffers at 64, 96 and 128 KiB
+        constexpr uint32_t A_AT[2] = {0u, OPER_BYTES};
+        constexpr uint32_t B_AT[3] = {2u * OPER_BYTES, 3u * OPER_BYTES, 4u * OPER_BYTES};
+        __shared__ __attribute__((aligned(1024))) char lds[5u * OPER_BYTES];
+
+        uint32_t tm, tn;
+        if(!r355::tileCoord(blockIdx.x, p.tilesM, p.tilesN, tm, tn))
+            return;
+
+        const uint32_t tid  = threadIdx.x;
+        const uint32_t lane = tid & 63u;
+        const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const uint32_t wm = wave >> 1, wn = wave & 1u;
+        auto           swzK = [](uint32_t row) { return (row >> 1) & 7u; };
+        const uint32_t ldsBase
+            = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds));
+
+        // global -> LDS: chunk L = j * 256 + tid of an operand tile sits at LDS byte 16 L (row L / 8)
+        const uint32_t gr = tid >> 3, gslot = tid & 7u;
+        const uint32_t gOffA = gr * p.lda + ((gslot ^ swzK(gr)) * CHUNK), gStepA = 32u * p.lda;
+        const uint32_t gOffB = gr * p.ldb + ((gslot ^ swzK(gr)) * CHUNK), gStepB = 32u * p.ldb;
+        const uint32_t numStages = p.k / STAGE_KB;
+        const uint32_t dmaDst    = ldsBase + wave * 64u * CHUNK; // + buffer + j * 4 KiB
+        auto           uniform64 = [](const char* ptr) {
+            const uint64_t v  = reinterpret_cast<uint64_t>(ptr);
+            const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+            const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+            return (static_cast<uint64_t>(hi) << 32) | lo;
+        };
+        const uint64_t gA = uniform64(p.a + (uint64_t)tm * TILE_M * p.lda);
+        const uint64_t gB = uniform64(p.b + (uint64_t)tn * TILE_N * p.ldb);
+        auto rsrcAt = [](uint64_t addr) { // raw buffer over a stage of an operand panel
+            return i32x4{static_cast<int>(static_cast<uint32_t>(addr)), static_cast<int>(static_cast<uint32_t>(addr >> 32) & 0xFFFFu),
+                         0x7FFFFFFF, 0x00020000};
+        };
+        auto stageAddr = [&](uint64_t panel, uint32_t stage) { // clamped to the last stage
+            return panel + (uint64_t)(stage < numStages ? stage : numStages - 1u) * STAGE_KB;
+        };
+        auto issueHalf = [&](uint64_t addr, uint32_t gOff, uint32_t gStep, uint32_t at) {
+            const i32x4 rsrc = rsrcAt(addr);
+#pragma unroll
+            for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
+                loadToLds(rsrc, gOff, j * gStep, dmaDst + at + j * THREADS * CHUNK);
+        };
+
+        // LDS -> registers: block i rows are 16 i + lane % 16; K step s reads chunk 4 s + lane / 16
+        uint32_t rdA[2], rdB[2];
+        {
+            const uint32_t ra = wm * 128u + (lane & 15u), rb = wn * 128u + (lane & 15u), g = lane >> 4;
+#pragma unroll
+            for(uint32_t s = 0; s < 2; ++s)
+            {
+                rdA[s] = ra * STAGE_KB + (((4u * s + g) ^ swzK(ra)) * CHUNK);
+                rdB[s] = rb * STAGE_KB + (((4u * s + g) ^ swzK(rb)) * CHUNK);
+            }
+        }
+
+        i32x4v acc[8][8];
+#pragma unroll
+        for(uint32_t i = 0; i < 8; ++i)
+#pragma unroll
+            for(uint32_t j = 0; j < 8; ++j)
+                acc[i][j] = i32x4v{0, 0, 0, 0};
+
+        i32x4 fa[2][8], fb[2][8];
+        // matrix instruction n of a K step: L-shaped shells, as in gemmTiledKernel16
+        auto mfmaAt = [&](uint32_t s, uint32_t n) {
+            uint32_t d = 0;
+            while((d + 1u) * (d + 1u) <= n)
+                ++d;
+            const uint32_t r = n - d * d;
+            const uint32_t i = r <= d ? d : r - d - 1u, j = r <= d ? r : d;
+            mfma16i8(acc[i][j], fb[s][j], fa[s][i]);
+        };
+        // operand block x of K step s: x = 2 i is A block i, x = 2 i + 1 is B block i
+        auto readAt = [&](uint32_t aAt, uint32_t bAt, uint32_t s, uint32_t x) {
+            const uint32_t i = x >> 1;
+            if(x & 1u)
+                fb[s][i] = *reinterpret_cast<const i32x4*>(lds + bAt + rdB[s] + i * 16u * STAGE_KB);
+            else
+                fa[s][i] = *reinterpret_cast<const i32x4*>(lds + aAt + rdA[s] + i * 16u * STAGE_KB);
+        };
+
+        uint64_t refillA, refillB; // stage kt + 2 of A, stage kt + 3 of B (clamped)
+        // One K stage: K step 0 is in registers; step 1 arrives under its matrix instructions; then the
+        // stage's buffers are refilled (A two stages ahead, B three) while step 0 of the next stage
+        // arrives under the matrix instructions of step 1.  One read per four matrix instructions, one
+        // direct load per four; nothing moves between the pieces.
+        auto stageBody = [&](uint32_t kt, uint32_t aCur, uint32_t aNxt, uint32_t bCur, uint32_t bNxt) {
+#pragma unroll
+            for(uint32_t x = 0; x < 16; ++x)
+#pragma unroll
+                for(uint32_t q = 0; q < 4; ++q)
+                {
+                    mfmaAt(0, 4u * x + q);
+                    if(q == 0u)
+                        readAt(aCur, bCur, 1, x);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            waitVmcnt<8>(); // this wave's part of stage kt + 1 has landed (the youngest 8 loads are B of kt + 2)
+            ldsBarrier();
+            const i32x4 rsrcA = rsrcAt(refillA), rsrcB = rsrcAt(refillB);
+            if(kt + 3u < numStages)
+                refillA += STAGE_KB;
+            if(kt + 4u < numStages)
+                refillB += STAGE_KB;
+#pragma unroll
+            for(uint32_t x = 0; x < 16; ++x)
+#pragma unroll
+                for(uint32_t q = 0; q < 4; ++q)
+                {
+                    mfmaAt(1, 4u * x + q);
+                    if(q == 0u)
+                        readAt(aNxt, bNxt, 0, x);
+                    if(q == 2u)
+                    {
+                        if(x < 8u)
+                            loadToLds(rsrcA, gOffA, x * gStepA, dmaDst + aCur + x * THREADS * CHUNK);
+                        else
+                            loadToLds(rsrcB, gOffB, (x - 8u) * gStepB, dmaDst + bCur + (x - 8u) * THREADS * CHUNK);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+        };
+
+        // prologue: stages 0 and 1 and the B half of stage 2 requested; stage 0 published
+        issueHalf(stageAddr(gA, 0u), gOffA, gStepA, A_AT[0]);
+        issueHalf(stageAddr(gB, 0u), gOffB, gStepB, B_AT[0]);
+        issueHalf(stageAddr(gA, 1u), gOffA, gStepA, A_AT[1]);
+        issueHalf(stageAddr(gB, 1u), gOffB, gStepB, B_AT[1]);
+        issueHalf(stageAddr(gB, 2u), gOffB, gStepB, B_AT[2]);
+        refillA = stageAddr(gA, 2u), refillB = stageAddr(gB, 3u);
+        waitVmcnt<24>();
+        ldsBarrier();
+#pragma unroll
+        for(uint32_t x = 0; x < 16; ++x)
+            readAt(A_AT[0], B_AT[0], 0, x);
+
+        // six stages per trip bring every buffer back to its role; single-exit loop, then the remainder
+        uint32_t kt = 0;
+        for(uint32_t trips = numStages / 6u; trips > 0; --trips, kt += 6u)
+        {
+            stageBody(kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1]);
+            stageBody(kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2]);
+            stageBody(kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0]);
+            stageBody(kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1]);
+            stageBody(kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2]);
+            stageBody(kt + 5u, A_AT[1], A_AT[0], B_AT[2], B_AT[0]);
+        }
+        const uint32_t rem = numStages - kt;
+        if(rem > 0u)
+        {
+            stageBody(kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1]);
+            if(rem > 1u)
+            {
+                stageBody(kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2]);
+                if(rem > 2u)
+                {
+                    stageBody(kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0]);
+                    if(rem > 3u)
+                    {
+                        stageBody(kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1]);
+                        if(rem > 4u)
+                            stageBody(kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2]);
+                    }
+                }
+            }
+        }
+
+        // the clamped loads of the last stages are still landing in buffers the epilogue reuses, and the
+        // last matrix instructions are still in the pipeline (the compiler does not know either)
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+        waitVmcnt<0>();
+        ldsBarrier();
+        storeTile16<i32x4v, int>(acc, p, tm, tn, wm, wn, lane, lds + wave * OPER_BYTES);
+    }
+
     struct Variant
     {
         bool direct;
@@ -1212,6 +1401,14 @@ namespace
         if constexpr(ElemTraits<E>::Bytes == 1)
         {
             const uint32_t grid = ((p.tilesM * p.tilesN + 7u) / 8u) * 8u;
+            if constexpr(E == Elem::I8)
+            {
+                if(!chosenVariant().shape32)
+                {
+                    hipLaunchKernelGGL(gemmTiledKernelI8, dim3(grid), dim3(THREADS), 0, stream, p);
+                    return r355::checkLaunch("gemm (macro tile, int8)");
+                }
+            }
             hipLaunchKernelGGL((gemmTiledKernel8<E, OutT>), dim3(grid), dim3(THREADS), 0, stream, p);
             return r355::checkLaunch("gemm (macro tile, 8-bit)");
         }
