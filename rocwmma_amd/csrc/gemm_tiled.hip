@@ -1355,6 +1355,202 @@ namespace
         storeTile16<i32x4v, int>(acc, p, tm, tn, wm, wn, lane, lds + wave * OPER_BYTES);
     }
 
+    // ------------------------------------------------------------------------------------------
+    // fp8 e4m3 on v_mfma_f32_16x16x128_f8f6f4.  One instruction spans the whole 128-byte K stage
+    // (32 bytes per lane: chunks lane / 16 and 4 + lane / 16, a K permutation shared by A and B), so
+    // a stage cannot be split along K.  It is split into quadrants of the wave tile instead:
+    //     Q1 = A[0..3] x B[0..3]   Q2 = A[0..3] x B[4..7]   Q3 = A[4..7] x B[4..7]   Q4 = A[4..7] x B[0..3]
+    // Consecutive quadrants share one operand group (4 blocks, 32 registers), so each quadrant's 16
+    // matrix instructions hide the 8 LDS reads of the one group the next quadrant needs:
+    //     under Q1: B[4..7] of this stage       under Q3: A[0..3] of the next stage
+    //     under Q2: A[4..7] of this stage       under Q4: B[0..3] of the next stage
+    // After Q2 the stage's buffers are no longer read: barrier, then the refills are issued under Q3
+    // (A) and Q4 (B).  Four register groups suffice; the two B groups swap roles every stage.
+    using i32x8 = int __attribute__((ext_vector_type(8)));
+    __device__ __forceinline__ void mfma16f8(f32x4& acc, const i32x8& x, const i32x8& y)
+    {
+        // cbsz = blgp = 0: both operands e4m3; the unscaled form multiplies by 2^0
+        asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc) : "v"(x), "v"(y));
+    }
+
+    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) gemmTiledKernelF8(Params p)
+    {
+        constexpr uint32_t A_AT[2] = {0u, OPER_BYTES};
+        constexpr uint32_t B_AT[3] = {2u * OPER_BYTES, 3u * OPER_BYTES, 4u * OPER_BYTES};
+        __shared__ __attribute__((aligned(1024))) char lds[5u * OPER_BYTES];
+
+        uint32_t tm, tn;
+        if(!r355::tileCoord(blockIdx.x, p.tilesM, p.tilesN, tm, tn))
+            return;
+
+        const uint32_t tid  = threadIdx.x;
+        const uint32_t lane = tid & 63u;
+        const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const uint32_t wm = wave >> 1, wn = wave & 1u;
+        auto           swzK = [](uint32_t row) { return (row >> 1) & 7u; };
+        const uint32_t ldsBase
+            = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds));
+
+        // global -> LDS: chunk L = j * 256 + tid of an operand tile sits at LDS byte 16 L (row L / 8)
+        const uint32_t gr = tid >> 3, gslot = tid & 7u;
+        const uint32_t gOffA = gr * p.lda + ((gslot ^ swzK(gr)) * CHUNK), gStepA = 32u * p.lda;
+        const uint32_t gOffB = gr * p.ldb + ((gslot ^ swzK(gr)) * CHUNK), gStepB = 32u * p.ldb;
+        const uint32_t numStages = p.k / STAGE_KB;
+        const uint32_t dmaDst    = ldsBase + wave * 64u * CHUNK;
+        auto           uniform64 = [](const char* ptr) {
+            const uint64_t v  = reinterpret_cast<uint64_t>(ptr);
+            const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+            const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+            return (static_cast<uint64_t>(hi) << 32) | lo;
+        };
+        const uint64_t gA = uniform64(p.a + (uint64_t)tm * TILE_M * p.lda);
+        const uint64_t gB = uniform64(p.b + (uint64_t)tn * TILE_N * p.ldb);
+        auto rsrcAt = [](uint64_t addr) {
+            return i32x4{static_cast<int>(static_cast<uint32_t>(addr)), static_cast<int>(static_cast<uint32_t>(addr >> 32) & 0xFFFFu),
+                         0x7FFFFFFF, 0x00020000};
+        };
+        auto stageAddr = [&](uint64_t panel, uint32_t stage) {
+            return panel + (uint64_t)(stage < numStages ? stage : numStages - 1u) * STAGE_KB;
+        };
+        auto issueHalf = [&](uint64_t addr, uint32_t gOff, uint32_t gStep, uint32_t at) {
+            const i32x4 rsrc = rsrcAt(addr);
+#pragma unroll
+            for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
+                loadToLds(rsrc, gOff, j * gStep, dmaDst + at + j * THREADS * CHUNK);
+        };
+
+        // LDS -> registers: block rows are 16 i + lane % 16; piece q of a block is chunk 4 q + lane / 16
+        uint32_t rdA[2], rdB[2];
+        {
+            const uint32_t ra = wm * 128u + (lane & 15u), rb = wn * 128u + (lane & 15u), g = lane >> 4;
+#pragma unroll
+            for(uint32_t q = 0; q < 2; ++q)
+            {
+                rdA[q] = ra * STAGE_KB + (((4u * q + g) ^ swzK(ra)) * CHUNK);
+                rdB[q] = rb * STAGE_KB + (((4u * q + g) ^ swzK(rb)) * CHUNK);
+            }
+        }
+        // read r (0..7) of an operand group: block 4 half + r / 2, piece r % 2
+        auto readPiece = [&](i32x8 (&grp)[4], uint32_t at, const uint32_t (&rd)[2], uint32_t half, uint32_t r) {
+            const uint32_t b = r >> 1, q = r & 1u;
+            const i32x4    v = *reinterpret_cast<const i32x4*>(lds + at + rd[q] + (4u * half + b) * 16u * STAGE_KB);
+            grp[b][4u * q] = v[0], grp[b][4u * q + 1u] = v[1], grp[b][4u * q + 2u] = v[2], grp[b][4u * q + 3u] = v[3];
+        };
+
+        f32x4 acc[8][8];
+#pragma unroll
+        for(uint32_t i = 0; i < 8; ++i)
+#pragma unroll
+            for(uint32_t j = 0; j < 8; ++j)
+                acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+        i32x8 aLo[4], aHi[4], bX[4], bY[4]; // bX / bY alternate as B[0..3] / B[4..7]
+
+        uint64_t refillA, refillB; // stage kt + 2 of A, stage kt + 3 of B (clamped)
+        auto stageBody = [&](uint32_t kt, uint32_t aCur, uint32_t aNxt, uint32_t bCur, uint32_t bNxt, i32x8 (&bLo)[4],
+                             i32x8 (&bHi)[4]) {
+            // Q1: A[0..3] x B[0..3]; B[4..7] arrives
+#pragma unroll
+            for(uint32_t n = 0; n < 16; ++n)
+            {
+                mfma16f8(acc[n & 3u][n >> 2], bLo[n >> 2], aLo[n & 3u]);
+                if(!(n & 1u))
+                    readPiece(bHi, bCur, rdB, 1, n >> 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // Q2: A[0..3] x B[4..7] (column by column, in the order B arrived); A[4..7] arrives
+#pragma unroll
+            for(uint32_t n = 0; n < 16; ++n)
+            {
+                mfma16f8(acc[n & 3u][4u + (n >> 2)], bHi[n >> 2], aLo[n & 3u]);
+                if(!(n & 1u))
+                    readPiece(aHi, aCur, rdA, 1, n >> 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            waitVmcnt<8>(); // this wave's part of stage kt + 1 has landed (the youngest 8 loads are B of kt + 2)
+            ldsBarrier();
+            const i32x4 rsrcA = rsrcAt(refillA), rsrcB = rsrcAt(refillB);
+            if(kt + 3u < numStages)
+                refillA += STAGE_KB;
+            if(kt + 4u < numStages)
+                refillB += STAGE_KB;
+            // Q3: A[4..7] x B[4..7] (row by row, in the order A arrived); next A[0..3] arrives; A refill
+#pragma unroll
+            for(uint32_t n = 0; n < 16; ++n)
+            {
+                mfma16f8(acc[4u + (n >> 2)][4u + (n & 3u)], bHi[n & 3u], aHi[n >> 2]);
+                if(!(n & 1u))
+                    readPiece(aLo, aNxt, rdA, 0, n >> 1);
+                else
+                    loadToLds(rsrcA, gOffA, (n >> 1) * gStepA, dmaDst + aCur + (n >> 1) * THREADS * CHUNK);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // Q4: A[4..7] x B[0..3]; next B[0..3] arrives in the registers B[4..7] has left; B refill
+#pragma unroll
+            for(uint32_t n = 0; n < 16; ++n)
+            {
+                mfma16f8(acc[4u + (n & 3u)][n >> 2], bLo[n >> 2], aHi[n & 3u]);
+                if(!(n & 1u))
+                    readPiece(bHi, bNxt, rdB, 0, n >> 1);
+                else
+                    loadToLds(rsrcB, gOffB, (n >> 1) * gStepB, dmaDst + bCur + (n >> 1) * THREADS * CHUNK);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+
+        // prologue: stages 0 and 1 and the B half of stage 2 requested; stage 0 published
+        issueHalf(stageAddr(gA, 0u), gOffA, gStepA, A_AT[0]);
+        issueHalf(stageAddr(gB, 0u), gOffB, gStepB, B_AT[0]);
+        issueHalf(stageAddr(gA, 1u), gOffA, gStepA, A_AT[1]);
+        issueHalf(stageAddr(gB, 1u), gOffB, gStepB, B_AT[1]);
+        issueHalf(stageAddr(gB, 2u), gOffB, gStepB, B_AT[2]);
+        refillA = stageAddr(gA, 2u), refillB = stageAddr(gB, 3u);
+        waitVmcnt<24>();
+        ldsBarrier();
+#pragma unroll
+        for(uint32_t r = 0; r < 8; ++r)
+        {
+            readPiece(aLo, A_AT[0], rdA, 0, r);
+            readPiece(bX, B_AT[0], rdB, 0, r);
+        }
+
+        // six stages per trip bring every buffer and both B register groups back to their roles
+        uint32_t kt = 0;
+        for(uint32_t trips = numStages / 6u; trips > 0; --trips, kt += 6u)
+        {
+            stageBody(kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1], bX, bY);
+            stageBody(kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2], bY, bX);
+            stageBody(kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0], bX, bY);
+            stageBody(kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1], bY, bX);
+            stageBody(kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2], bX, bY);
+            stageBody(kt + 5u, A_AT[1], A_AT[0], B_AT[2], B_AT[0], bY, bX);
+        }
+        const uint32_t rem = numStages - kt;
+        if(rem > 0u)
+        {
+            stageBody(kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1], bX, bY);
+            if(rem > 1u)
+            {
+                stageBody(kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2], bY, bX);
+                if(rem > 2u)
+                {
+                    stageBody(kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0], bX, bY);
+                    if(rem > 3u)
+                    {
+                        stageBody(kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1], bY, bX);
+                        if(rem > 4u)
+                            stageBody(kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2], bX, bY);
+                    }
+                }
+            }
+        }
+
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); // the last matrix instructions are still in the pipeline
+        waitVmcnt<0>();
+        ldsBarrier();
+        storeTile16<f32x4, float>(acc, p, tm, tn, wm, wn, lane, lds + wave * OPER_BYTES);
+    }
+
     struct Variant
     {
         bool direct;
@@ -1407,6 +1603,14 @@ namespace
                 {
                     hipLaunchKernelGGL(gemmTiledKernelI8, dim3(grid), dim3(THREADS), 0, stream, p);
                     return r355::checkLaunch("gemm (macro tile, int8)");
+                }
+            }
+            if constexpr(E == Elem::E4M3)
+            {
+                if(!chosenVariant().shape32)
+                {
+                    hipLaunchKernelGGL(gemmTiledKernelF8, dim3(grid), dim3(THREADS), 0, stream, p);
+                    return r355::checkLaunch("gemm (macro tile, e4m3)");
                 }
             }
             hipLaunchKernelGGL((gemmTiledKernel8<E, OutT>), dim3(grid), dim3(THREADS), 0, stream, p);
