@@ -1,5 +1,5 @@
-// LDS-staged, double-buffered macro-tile GEMM for gfx950, written directly against the
-// hardware (no fragment-API composition).
+// LDS-staged macro-tile GEMM for gfx950, written directly against the hardware (no fragment-API
+// composition).
 //
 // Takes the place of samples/perf_hgemm.cpp:515-711 and
 // test/gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp:52-283.  The reference
@@ -9,18 +9,27 @@
 //
 //   macro tile   256 x 256, K stage of 128 bytes (64 f16/bf16, 128 int8/fp8 elements)
 //   workgroup    256 threads = 4 waves in a 2 x 2 grid, wave tile 128 x 128
-//                = 4 x 4 v_mfma_*_32x32x{16,32} accumulators (256 accumulator registers)
+//                = 8 x 8 accumulators of the 16 x 16 matrix-instruction shapes (256 registers):
+//                v_mfma_f32_16x16x32_{f16,bf16}, v_mfma_i32_16x16x64_i8, v_mfma_f32_16x16x128_f8f6f4.
+//                Under the board's power limit these sustain 12-20 % more than the 32 x 32 shapes of
+//                the same types (register-resident loops, random operands), and the kernels are
+//                power-bound.
 //   LDS          16-bit types: 2 stages x (A 32 KiB + B 32 KiB) = 128 KiB;
-//                8-bit types: 2 A buffers + 3 B buffers x 32 KiB = 160 KiB (gemmTiledKernel8);
+//                8-bit types: 2 A buffers + 3 B buffers x 32 KiB = 160 KiB;
 //                one workgroup per CU either way
-//   global->LDS  128-bit loads, either staged through registers or written straight
-//                into LDS by the memory pipeline (global_load_lds_dwordx4)
+//   global->LDS  128-bit loads written straight into LDS by the memory pipeline
+//                (buffer_load_dwordx4 ... lds), no register staging
 //   LDS layout   16-byte chunks, XOR-swizzled inside each row so that both the
 //                row-contiguous writes and the MFMA-shaped reads are bank-conflict free
-//   LDS->regs    K-contiguous operands: one ds_read_b128 per 32x(16|32) operand block;
+//   LDS->regs    K-contiguous operands: one ds_read_b128 per 16-row operand block;
 //                M/N-contiguous 16-bit operands: two ds_read_b64_tr_b16 (transposing
-//                read) -- no element-wise reads anywhere; operands are fetched two
-//                matrix-instruction K steps (32 instructions) ahead of their use
+//                read) -- no element-wise reads anywhere; operands are fetched one K step
+//                (64 matrix instructions; fp8: one quadrant, 16) ahead of their use
+//   schedule     the matrix instructions are inline assembly with the accumulator tied in place
+//                (the compiler's own selection leaves the 64 small accumulators untied and its
+//                register allocator then shuffles them through the K loop), so the kernels fix
+//                the instruction order themselves: one LDS read or direct load per matrix
+//                instruction, pinned by scheduling barriers
 //   grid         1-D, remapped so that each XCD (workgroup id mod 8) owns a compact
 //                rectangle of tiles and walks it in 4-row groups (L2 reuse of A and B)
 //
@@ -34,12 +43,9 @@
 
 namespace
 {
-    using f32x16 = float __attribute__((ext_vector_type(16)));
-    using i32x16 = int __attribute__((ext_vector_type(16)));
     using i32x4  = int __attribute__((ext_vector_type(4)));
     using i32x2  = int __attribute__((ext_vector_type(2)));
     using f16x8  = _Float16 __attribute__((ext_vector_type(8)));
-    using f16x4  = _Float16 __attribute__((ext_vector_type(4)));
     using bf16x8 = __bf16 __attribute__((ext_vector_type(8)));
     typedef __fp16 trv4 __attribute__((__vector_size__(4 * sizeof(__fp16)))); // operand type of the transposing LDS read
 
@@ -56,7 +62,7 @@ namespace
     constexpr uint32_t STAGE_KB    = 128; // bytes of K per stage per row
     constexpr uint32_t OPER_BYTES  = TILE_M * STAGE_KB; // 32 KiB per operand per stage
     constexpr uint32_t STAGE_BYTES = 2 * OPER_BYTES;
-    constexpr uint32_t NUM_STAGES  = 2;
+    constexpr uint32_t NUM_STAGES  = 2; // 16-bit kernel
     constexpr uint32_t THREADS     = 256;
     constexpr uint32_t CHUNK       = 16; // bytes moved per lane per access
     constexpr uint32_t LOADS_PER_OPER = OPER_BYTES / CHUNK / THREADS; // 8
@@ -67,68 +73,23 @@ namespace
     struct ElemTraits<Elem::F16>
     {
         static constexpr uint32_t Bytes = 2;
-        using Acc                       = f32x16;
     };
     template <>
     struct ElemTraits<Elem::BF16>
     {
         static constexpr uint32_t Bytes = 2;
-        using Acc                       = f32x16;
     };
     template <>
     struct ElemTraits<Elem::E4M3>
     {
         static constexpr uint32_t Bytes = 1;
-        using Acc                       = f32x16;
     };
     template <>
     struct ElemTraits<Elem::I8>
     {
         static constexpr uint32_t Bytes = 1;
-        using Acc                       = i32x16;
     };
 
-    // acc += X(32 x k) * Y(k x 32) with 16 bytes of K per lane per operand
-    template <Elem E>
-    __device__ inline void mfma32(typename ElemTraits<E>::Acc& acc, i32x4 x, i32x4 y)
-    {
-        if constexpr(E == Elem::F16)
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                __builtin_bit_cast(f16x8, x), __builtin_bit_cast(f16x8, y), acc, 0, 0, 0);
-        else if constexpr(E == Elem::BF16)
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                __builtin_bit_cast(bf16x8, x), __builtin_bit_cast(bf16x8, y), acc, 0, 0, 0);
-        else if constexpr(E == Elem::I8)
-            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(x, y, acc, 0, 0, 0);
-        else
-        {
-            // fp8: two 32x32x16 steps on the low / high 8 bytes (a K permutation shared by X and Y)
-            using l2 = long __attribute__((ext_vector_type(2)));
-            l2 xl    = __builtin_bit_cast(l2, x);
-            l2 yl    = __builtin_bit_cast(l2, y);
-            acc      = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(xl[0], yl[0], acc, 0, 0, 0);
-            acc      = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(xl[1], yl[1], acc, 0, 0, 0);
-        }
-    }
-
-    // fp8 e4m3 at full rate: v_mfma_f32_32x32x64_f8f6f4 takes 32 bytes of K per lane per operand
-    // (two 16-byte pieces here: any K permutation shared by both operands is legal).  Formats
-    // cbsz = blgp = 0 select e4m3 for both operands; the E8M0 block scales are 127 = 2^0.
-    __device__ inline void mfma64Fp8(f32x16& acc, i32x4 x0, i32x4 x1, i32x4 y0, i32x4 y1)
-    {
-        using i32x8 = int __attribute__((ext_vector_type(8)));
-        const i32x8 x = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
-        const i32x8 y = {y0[0], y0[1], y0[2], y0[3], y1[0], y1[1], y1[2], y1[3]};
-        acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, acc, 0, 0, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
-    }
-
-    // ---- LDS swizzles.  A tile is `rows` rows of `rowBytes`; chunk c of row r lives in
-    // chunk slot (c ^ swz(r)) of that row.
-    //   K-contiguous tile: 256 rows x 128 B (8 slots).   Readers: lane -> row, 8 (or 16)
-    //     lanes share a chunk index, so consecutive rows must land in different slots.
-    //   M/N-contiguous tile: 64 k-rows x 512 B (32 slots).  Readers: 16 lanes cover
-    //     4 k-rows x 32 B, so consecutive k-rows must land in different 32-byte pairs.
-    // BANKS64 selects the pattern for a 256-byte-per-clock LDS (64 banks) instead of 128.
     struct Params
     {
         uint32_t    m, n, k;
@@ -139,443 +100,19 @@ namespace
         uint32_t    lda, ldb, ldc, ldd; // elements
         float       alpha, beta;
         uint32_t    tilesM, tilesN;
-        uint32_t    banks64; // LDS swizzle tuned for 64 banks instead of 32
     };
 
-    // Scheduling hint for the current region: next come MFMAS matrix instructions, then DSREADS
-    // LDS reads, then VMEM global loads.
-    template <uint32_t MFMAS, uint32_t DSREADS, uint32_t VMEM>
-    __device__ inline void schedGroup()
-    {
-        __builtin_amdgcn_sched_group_barrier(0x008, MFMAS, 0);
-        if constexpr(DSREADS > 0)
-            __builtin_amdgcn_sched_group_barrier(0x100, DSREADS, 0);
-        if constexpr(VMEM > 0)
-            __builtin_amdgcn_sched_group_barrier(0x020, VMEM, 0);
-    }
-
-    // D = alpha * acc + beta * C for one wave's 128 x 128 tile, row-major.  `scratch` is 32 KiB of LDS
-    // owned by this wave (the stage buffers are idle by then).
-    template <Elem E, typename OutT>
-    __device__ __forceinline__ void storeTile(typename ElemTraits<E>::Acc (&acc)[4][4], const Params& p, uint32_t tm,
-                                              uint32_t tn, uint32_t wm, uint32_t wn, uint32_t lane, char* scratch)
-    {
-        // ---------------- epilogue: D = alpha * acc + beta * C, row-major
-        // lane holds D(m = lane % 32, n = 8 (e / 4) + 4 (lane / 32) + e % 4) of each 32 x 32 block
-        using AccE = std::conditional_t<E == Elem::I8, int, float>;
-        using OutV = OutT __attribute__((ext_vector_type(4)));
-        const AccE     alpha = static_cast<AccE>(p.alpha), beta = static_cast<AccE>(p.beta);
-        const uint32_t m0 = tm * TILE_M + wm * 128u, n0 = tn * TILE_N + wn * 128u;
-
-        if(beta == static_cast<AccE>(0))
-        {
-            // The stage buffers are idle now: every wave transposes its 128 x 128 result through its
-            // own 32 KiB of LDS so that a store instruction covers whole 256- or 512-byte rows of D
-            // (128-bit per lane) instead of 8- / 16-byte pieces of 32 different rows.
-            constexpr uint32_t OS         = sizeof(OutT);
-            constexpr uint32_t ROW_BYTES  = 128u * OS; // one row of the wave tile
-            constexpr uint32_t ROW_CHUNKS = ROW_BYTES / CHUNK; // 16 (2-byte) or 32 (4-byte)
-            constexpr uint32_t ROWS_PASS  = 32768u / ROW_BYTES; // 128 or 64 rows per pass
-            constexpr uint32_t BLOCKS_I   = ROWS_PASS / 32u; // 32-row blocks per pass
-            char*              wl         = scratch;
-            const uint32_t     r32 = lane & 31u, h = lane >> 5;
-#pragma unroll
-            for(uint32_t pass = 0; pass < 4u / BLOCKS_I; ++pass)
-            {
-#pragma unroll
-                for(uint32_t ii = 0; ii < BLOCKS_I; ++ii)
-                {
-                    const uint32_t i   = pass * BLOCKS_I + ii;
-                    const uint32_t row = 32u * ii + r32; // row inside the pass
-#pragma unroll
-                    for(uint32_t j = 0; j < 4; ++j)
-#pragma unroll
-                        for(uint32_t q = 0; q < 4; ++q)
-                        {
-                            OutV out;
-#pragma unroll
-                            for(uint32_t e = 0; e < 4; ++e)
-                                out[e] = static_cast<OutT>(alpha * static_cast<AccE>(acc[i][j][4 * q + e]));
-                            if constexpr(OS == 2)
-                            {
-                                // 8 bytes: chunk 4 j + q, half h; rows 16 apart share a chunk slot, so
-                                // they take opposite halves
-                                const uint32_t c = 4u * j + q;
-                                char* dst = wl + row * ROW_BYTES + ((c ^ (row & 15u)) * CHUNK) + ((h ^ ((row >> 4) & 1u)) * 8u);
-                                *reinterpret_cast<OutV*>(dst) = out;
-                            }
-                            else
-                            {
-                                const uint32_t c = 8u * j + 2u * q + h;
-                                char* dst = wl + row * ROW_BYTES + ((c ^ (row & 31u)) * CHUNK);
-                                *reinterpret_cast<OutV*>(dst) = out;
-                            }
-                        }
-                }
-                __builtin_amdgcn_wave_barrier(); // same wave reads back what it wrote (LDS is in order per wave)
-#pragma unroll
-                for(uint32_t it = 0; it < ROWS_PASS * ROW_CHUNKS / 64u; ++it)
-                {
-                    const uint32_t L = it * 64u + lane, row = L / ROW_CHUNKS, c = L % ROW_CHUNKS;
-                    i32x4          v;
-                    if constexpr(OS == 2)
-                    {
-                        v = *reinterpret_cast<const i32x4*>(wl + row * ROW_BYTES + ((c ^ (row & 15u)) * CHUNK));
-                        if((row >> 4) & 1u)
-                            v = i32x4{v[2], v[3], v[0], v[1]};
-                    }
-                    else
-                        v = *reinterpret_cast<const i32x4*>(wl + row * ROW_BYTES + ((c ^ (row & 31u)) * CHUNK));
-                    const uint64_t offD = (uint64_t)(m0 + pass * ROWS_PASS + row) * p.ldd + n0;
-                    // D is written once and not read again: stream it past the caches
-                    __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(p.d + offD * OS + c * CHUNK));
-                }
-                __builtin_amdgcn_wave_barrier();
-            }
-            return;
-        }
-
-#pragma unroll
-        for(uint32_t i = 0; i < 4; ++i)
-        {
-#pragma unroll
-            for(uint32_t j = 0; j < 4; ++j)
-            {
-#pragma unroll
-                for(uint32_t q = 0; q < 4; ++q)
-                {
-                    const uint32_t row  = m0 + 32u * i + (lane & 31u);
-                    const uint32_t col  = n0 + 32u * j + 8u * q + 4u * (lane >> 5);
-                    const uint64_t offD = (uint64_t)row * p.ldd + col;
-                    const uint64_t offC = (uint64_t)row * p.ldc + col;
-                    const OutV     cv   = *reinterpret_cast<const OutV*>(p.c + offC * sizeof(OutT));
-                    OutV           out;
-#pragma unroll
-                    for(uint32_t e = 0; e < 4; ++e)
-                        out[e] = static_cast<OutT>(alpha * static_cast<AccE>(acc[i][j][4 * q + e])
-                                                   + beta * static_cast<AccE>(cv[e]));
-                    *reinterpret_cast<OutV*>(p.d + offD * sizeof(OutT)) = out;
-                }
-            }
-        }
-    }
-
-    template <Elem E, typename OutT, bool A_KCONTIG, bool B_KCONTIG, bool DIRECT>
-    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
-        gemmTiledKernel(Params p)
-    {
-        using Traits          = ElemTraits<E>;
-        using Acc             = typename Traits::Acc;
-        constexpr uint32_t ES = Traits::Bytes;
-        constexpr uint32_t TK = STAGE_KB / ES; // K elements per stage
-        static_assert(ES == 2, "16-bit element types only; 8-bit types run gemmTiledKernel8");
-        // LDS reads per operand block: one 128-bit read, or two transposing 64-bit reads
-        constexpr uint32_t READS_PER_SUB = (A_KCONTIG ? 4u : 8u) + (B_KCONTIG ? 4u : 8u);
-
-        // One variable per stage: the compiler tracks outstanding direct-to-LDS loads per LDS
-        // variable, so reads of one stage need not wait for loads in flight to the other.
-        __shared__ __attribute__((aligned(1024))) char stage0[STAGE_BYTES];
-        __shared__ __attribute__((aligned(1024))) char stage1[STAGE_BYTES];
-
-        uint32_t tm, tn;
-        if(!r355::tileCoord(blockIdx.x, p.tilesM, p.tilesN, tm, tn))
-            return;
-
-        const uint32_t tid   = threadIdx.x;
-        const uint32_t lane  = tid & 63u;
-        const uint32_t wave  = __builtin_amdgcn_readfirstlane(tid >> 6);
-        const uint32_t wm    = wave >> 1; // wave row in the 2 x 2 wave grid
-        const uint32_t wn    = wave & 1u;
-        const bool     b64   = p.banks64 != 0;
-        auto           swzK  = [&](uint32_t row) { return b64 ? ((row >> 1) & 7u) : (row & 7u); };
-        auto           swzMN = [&](uint32_t krow) { return b64 ? ((krow & 3u) << 2) : ((krow & 3u) << 1); };
-
-        // ---------------- global -> LDS addressing (per thread, fixed for the whole K loop)
-        // chunk L = j * 256 + tid of an operand tile sits at LDS byte 16 L.  The swizzle terms
-        // depend on the row only through bits that j does not change (j * 32 rows for the
-        // K-contiguous tile, j * 8 k-rows for the other), so one lane offset serves all j.
-        uint32_t gOffA, gOffB; // byte offset of this thread's j = 0 chunk from the tile origin
-        uint32_t gStepA, gStepB; // bytes between consecutive j
-        uint64_t gStageA, gStageB; // bytes between consecutive K stages
-        if constexpr(A_KCONTIG)
-        {
-            const uint32_t r = tid >> 3, slot = tid & 7u;
-            gOffA   = r * p.lda * ES + ((slot ^ swzK(r)) * CHUNK);
-            gStepA  = 32u * p.lda * ES;
-            gStageA = STAGE_KB;
-        }
-        else
-        {
-            const uint32_t r = tid >> 5, slot = tid & 31u;
-            gOffA   = r * p.lda * ES + ((slot ^ swzMN(r)) * CHUNK);
-            gStepA  = 8u * p.lda * ES;
-            gStageA = (uint64_t)TK * p.lda * ES;
-        }
-        if constexpr(B_KCONTIG)
-        {
-            const uint32_t r = tid >> 3, slot = tid & 7u;
-            gOffB   = r * p.ldb * ES + ((slot ^ swzK(r)) * CHUNK);
-            gStepB  = 32u * p.ldb * ES;
-            gStageB = STAGE_KB;
-        }
-        else
-        {
-            const uint32_t r = tid >> 5, slot = tid & 31u;
-            gOffB   = r * p.ldb * ES + ((slot ^ swzMN(r)) * CHUNK);
-            gStepB  = 8u * p.ldb * ES;
-            gStageB = (uint64_t)TK * p.ldb * ES;
-        }
-        const char* gA = p.a + (A_KCONTIG ? (uint64_t)tm * TILE_M * p.lda * ES : (uint64_t)tm * TILE_M * ES);
-        const char* gB = p.b + (B_KCONTIG ? (uint64_t)tn * TILE_N * p.ldb * ES : (uint64_t)tn * TILE_N * ES);
-
-        // ---------------- LDS -> register addressing (per lane, fixed)
-        // K-contiguous: block i rows are (i * 32 + lane % 32); sub-step s reads chunk 2 s + lane / 32.
-        // M/N-contiguous: sub-step s, half h: k-row 16 s + 8 (lane / 32) + 4 h + (lane % 16) / 4,
-        //                 8-byte piece m / 4 with m = 32 i + 16 ((lane / 16) & 1) + 4 (lane % 4).
-        uint32_t rdA[4], rdB[4];
-        if constexpr(A_KCONTIG)
-        {
-            const uint32_t r = wm * 128u + (lane & 31u);
-#pragma unroll
-            for(uint32_t s = 0; s < 4; ++s)
-                rdA[s] = r * STAGE_KB + (((2u * s + (lane >> 5)) ^ swzK(r)) * CHUNK);
-        }
-        else
-        {
-            const uint32_t t = lane & 15u, kr = 8u * (lane >> 5) + (t >> 2);
-#pragma unroll
-            for(uint32_t i = 0; i < 4; ++i)
-            {
-                const uint32_t piece = wm * 32u + 8u * i + 4u * ((lane >> 4) & 1u) + (t & 3u);
-                rdA[i] = kr * 512u + (((piece >> 1) ^ swzMN(kr)) * CHUNK) + (piece & 1u) * 8u;
-            }
-        }
-        if constexpr(B_KCONTIG)
-        {
-            const uint32_t r = wn * 128u + (lane & 31u);
-#pragma unroll
-            for(uint32_t s = 0; s < 4; ++s)
-                rdB[s] = OPER_BYTES + r * STAGE_KB + (((2u * s + (lane >> 5)) ^ swzK(r)) * CHUNK);
-        }
-        else
-        {
-            const uint32_t t = lane & 15u, kr = 8u * (lane >> 5) + (t >> 2);
-#pragma unroll
-            for(uint32_t i = 0; i < 4; ++i)
-            {
-                const uint32_t piece = wn * 32u + 8u * i + 4u * ((lane >> 4) & 1u) + (t & 3u);
-                rdB[i] = OPER_BYTES + kr * 512u + (((piece >> 1) ^ swzMN(kr)) * CHUNK) + (piece & 1u) * 8u;
-            }
-        }
-
-        // operand block i of sub-step s from a stage buffer
-        auto readA = [&](const char* base, uint32_t i, uint32_t s) -> i32x4 {
-            if constexpr(A_KCONTIG)
-                return *reinterpret_cast<const i32x4*>(base + rdA[s] + i * 32u * STAGE_KB);
-            else
-            {
-                using lp        = __attribute__((address_space(3))) trv4*;
-                const char* q   = base + rdA[i] + s * 16u * 512u;
-                const i32x2 lo  = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lp)q));
-                const i32x2 hi  = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lp)(q + 4u * 512u)));
-                return i32x4{lo[0], lo[1], hi[0], hi[1]};
-            }
-        };
-        auto readB = [&](const char* base, uint32_t i, uint32_t s) -> i32x4 {
-            if constexpr(B_KCONTIG)
-                return *reinterpret_cast<const i32x4*>(base + rdB[s] + i * 32u * STAGE_KB);
-            else
-            {
-                using lp        = __attribute__((address_space(3))) trv4*;
-                const char* q   = base + rdB[i] + s * 16u * 512u;
-                const i32x2 lo  = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lp)q));
-                const i32x2 hi  = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lp)(q + 4u * 512u)));
-                return i32x4{lo[0], lo[1], hi[0], hi[1]};
-            }
-        };
-
-        // ---------------- stage movement
-        i32x4 stageRegs[DIRECT ? 1 : 2 * LOADS_PER_OPER];
-
-        auto issueGlobal = [&](uint32_t kt, char* stage) {
-            // Buffer addressing keeps every per-load term scalar: resource = origin of this stage's
-            // panel (uniform), soffset = j * step (uniform), voffset = the lane's fixed offset.
-            const char* srcA = gA + kt * gStageA;
-            const char* srcB = gB + kt * gStageB;
-            if constexpr(DIRECT)
-            {
-                // the panel origins are wave-uniform; say so, or the resource ends up in VGPRs
-                auto uniform = [](const char* ptr) {
-                    const uint64_t v  = reinterpret_cast<uint64_t>(ptr);
-                    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
-                    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
-                    return reinterpret_cast<char*>((static_cast<uint64_t>(hi) << 32) | lo);
-                };
-                constexpr int RSRC_FLAGS = 0x00020000; // raw buffer, 32-bit data format, no swizzle
-                const __amdgpu_buffer_rsrc_t rsrcA
-                    = __builtin_amdgcn_make_buffer_rsrc(uniform(srcA), 0, 0x7FFFFFFF, RSRC_FLAGS);
-                const __amdgpu_buffer_rsrc_t rsrcB
-                    = __builtin_amdgcn_make_buffer_rsrc(uniform(srcB), 0, 0x7FFFFFFF, RSRC_FLAGS);
-                using lp = __attribute__((address_space(3))) void*;
-#pragma unroll
-                for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
-                {
-                    // the memory pipeline writes lane l's 16 bytes at (uniform LDS base + 16 l)
-                    char* dstA = stage + (j * THREADS + wave * 64u) * CHUNK;
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcA, (lp)dstA, 16, gOffA, j * gStepA, 0, 0);
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrcB, (lp)(dstA + OPER_BYTES), 16, gOffB, j * gStepB, 0, 0);
-                }
-            }
-            else
-            {
-#pragma unroll
-                for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
-                {
-                    stageRegs[j]                  = *reinterpret_cast<const i32x4*>(srcA + (uint64_t)j * gStepA + gOffA);
-                    stageRegs[LOADS_PER_OPER + j] = *reinterpret_cast<const i32x4*>(srcB + (uint64_t)j * gStepB + gOffB);
-                }
-            }
-        };
-
-        auto commitLds = [&](char* stage) {
-            if constexpr(!DIRECT)
-            {
-#pragma unroll
-                for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
-                {
-                    char* dstA = stage + (j * THREADS + tid) * CHUNK;
-                    *reinterpret_cast<i32x4*>(dstA)              = stageRegs[j];
-                    *reinterpret_cast<i32x4*>(dstA + OPER_BYTES) = stageRegs[LOADS_PER_OPER + j];
-                }
-            }
-        };
-
-        Acc            acc[4][4];
-        const uint32_t numStages = p.k / TK;
-#pragma unroll
-        for(uint32_t i = 0; i < 4; ++i)
-#pragma unroll
-            for(uint32_t j = 0; j < 4; ++j)
-#pragma unroll
-                for(uint32_t e = 0; e < 16; ++e)
-                    acc[i][j][e] = 0;
-
-        // operands swapped: each lane then holds 4 consecutive columns of a row of D
-        auto mfmaStep = [&](const i32x4 (&fa)[4], const i32x4 (&fb)[4]) {
-#pragma unroll
-            for(uint32_t i = 0; i < 4; ++i)
-#pragma unroll
-                for(uint32_t j = 0; j < 4; ++j)
-                    mfma32<E>(acc[i][j], fb[j], fa[i]);
-        };
-
-        constexpr uint32_t NBUF = 4u;
-        i32x4 fa[NBUF][4], fb[NBUF][4];
-
-        // One K stage.  `cur` / `nxt` are the LDS buffers of stage kt / kt + 1.  Operand registers
-        // are indexed by sub-step and fetched two sub-steps ahead (LDS is shared by four waves and
-        // the direct loads, so a read can take several hundred cycles): during sub-steps 0 and 1
-        // the operands of sub-steps 2 and 3 arrive; then every wave holds the rest of `cur` in
-        // registers, so after the barrier `cur` is refilled with stage kt + 2 and the operands of
-        // sub-steps 0 and 1 of stage kt + 1 are fetched from `nxt` underneath sub-steps 2 and 3.
-        auto stageBody = [&](uint32_t kt, char* cur, char* nxt, auto refill, auto hasNext) {
-            constexpr bool REFILL = decltype(refill)::value; // stage kt + 2 exists
-            constexpr bool NEXT   = decltype(hasNext)::value; // stage kt + 1 exists
-#pragma unroll
-            for(uint32_t s = 0; s < 2; ++s)
-            {
-#pragma unroll
-                for(uint32_t i = 0; i < 4; ++i)
-                {
-                    fa[s + 2][i] = readA(cur, i, s + 2);
-                    fb[s + 2][i] = readB(cur, i, s + 2);
-                }
-                mfmaStep(fa[s], fb[s]);
-#pragma unroll
-                for(uint32_t g = 0; g < 8; ++g)
-                {
-                    schedGroup<1, READS_PER_SUB / 8u - READS_PER_SUB / 16u, 0>();
-                    schedGroup<1, READS_PER_SUB / 16u, 0>();
-                }
-            }
-            if constexpr(!DIRECT && NEXT)
-                commitLds(nxt);
-            if constexpr(DIRECT)
-                __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
-            __syncthreads();
-            if constexpr(REFILL)
-                issueGlobal(kt + 2, cur);
-#pragma unroll
-            for(uint32_t s = 2; s < 4; ++s)
-            {
-                if constexpr(NEXT)
-                {
-#pragma unroll
-                    for(uint32_t i = 0; i < 4; ++i)
-                    {
-                        fa[s - 2][i] = readA(nxt, i, s - 2);
-                        fb[s - 2][i] = readB(nxt, i, s - 2);
-                    }
-                }
-                mfmaStep(fa[s], fb[s]);
-            }
-#pragma unroll
-            for(uint32_t g = 0; g < 16; ++g)
-            {
-                schedGroup<1, NEXT ? READS_PER_SUB / 8u - READS_PER_SUB / 16u : 0u, REFILL ? 1u : 0u>();
-                schedGroup<1, NEXT ? READS_PER_SUB / 16u : 0u, 0>();
-            }
-        };
-        constexpr std::true_type  yes{};
-        constexpr std::false_type no{};
-
-        // prologue: stage 0 resident, stage 1 in flight, first operands in registers
-        issueGlobal(0, stage0);
-        if constexpr(DIRECT)
-        {
-            issueGlobal(1, stage1);
-            __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
-        }
-        else
-        {
-            commitLds(stage0);
-            issueGlobal(1, stage1);
-        }
-        __syncthreads();
-#pragma unroll
-        for(uint32_t s = 0; s < 2u; ++s)
-#pragma unroll
-            for(uint32_t i = 0; i < 4; ++i)
-            {
-                fa[s][i] = readA(stage0, i, s);
-                fb[s][i] = readB(stage0, i, s);
-            }
-
-        // numStages is even (checked on the host): steady state in pairs, last pair peeled
-        uint32_t kt = 0;
-        for(; kt + 2 < numStages; kt += 2)
-        {
-            stageBody(kt, stage0, stage1, yes, yes);
-            stageBody(kt + 1, stage1, stage0, yes, yes);
-        }
-        stageBody(kt, stage0, stage1, no, yes);
-        stageBody(kt + 1, stage1, stage0, no, no);
-
-        storeTile<E, OutT>(acc, p, tm, tn, wm, wn, lane, ((wave < 2u) ? stage0 : stage1) + (wave & 1u) * 32768u);
-    }
-
     // ------------------------------------------------------------------------------------------
-    // The same macro tile on the 16 x 16 matrix-instruction shapes (v_mfma_f32_16x16x32_{f16,bf16}).
-    // Under the board's power limit these sustain about a fifth more than the 32 x 32 shapes of the
-    // same types (measured with register-resident loops), and the kernel is power-bound, so it is the
-    // default for the 16-bit types.  What changes against gemmTiledKernel:
+    // f16 / bf16 on v_mfma_f32_16x16x32_{f16,bf16}.
     //   * wave tile 128 x 128 = 8 x 8 accumulators of 4 registers; a stage is two K steps of 32;
     //     the operands of one K step (8 + 8 blocks, 128 registers for both steps) are fetched one step
     //     ahead of their use;
     //   * lane -> operand mapping: row lane % 16, 16-byte chunk lane / 16 of the 64-byte K step;
-    //   * the M/N-contiguous swizzle also depends on bit 3 of the k-row (a 32-lane transposing read
-    //     covers k-rows 0..3 and 8..11), which makes the global -> LDS lane offset alternate between two
-    //     values from one load to the next;
+    //   * K-contiguous tile in LDS: 256 rows x 128 B, chunk c of row r in slot c ^ ((r >> 1) & 7): 16
+    //     consecutive rows of one chunk index cover all 64 banks once;
+    //   * M/N-contiguous tile in LDS: 64 k-rows x 512 B; a 32-lane transposing read covers k-rows 0..3
+    //     and 8..11 times 32 bytes, so the swizzle depends on bits 0, 1 and 3 of the k-row, which makes
+    //     the global -> LDS lane offset alternate between two values from one load to the next;
     //   * accumulator block (i, j): lane holds D(16 i + lane % 16, 16 j + 4 (lane / 16) + 0..3).
     using f32x4 = float __attribute__((ext_vector_type(4)));
 
@@ -931,21 +468,22 @@ namespace
     }
 
     // ------------------------------------------------------------------------------------------
-    // 8-bit operands (int8, e4m3; A row-major, B col-major).  At twice the matrix-instruction rate a
-    // K stage lasts about as long as a direct load takes to arrive, so the two-buffer scheme above
-    // leaves the memory pipe idle while a refill waits for its consumer.  Here LDS holds two buffers
-    // for A and three for B (5 x 32 KiB = all 160 KiB): the B half of a stage is requested three
-    // stages ahead and the A half two, which keeps 96 KiB per CU in flight instead of 64.
-    // Stage kt lives in A buffer kt % 2 and B buffer kt % 3, so six stages bring every buffer back
-    // to its starting role.  Loads past the last stage are clamped to it -- they land in buffers
-    // nobody reads any more -- so every stage issues the same 16 loads and the wait before its
-    // barrier is always "all but the youngest 8".
+    // 8-bit operands (int8, e4m3; A row-major, B col-major): five LDS buffers.  At twice the
+    // matrix-instruction rate a K stage lasts about as long as a direct load takes to arrive, so a
+    // two-buffer scheme leaves the memory pipe idle while a refill waits for its consumer.  Here LDS
+    // holds two buffers for A and three for B (5 x 32 KiB = all 160 KiB): the B half of a stage is
+    // requested three stages ahead and the A half two, which keeps 96 KiB per CU in flight instead
+    // of 64.  Stage kt lives in A buffer kt % 2 and B buffer kt % 3, so six stages bring every buffer
+    // back to its starting role; the K loop is unrolled six times with a single exit (an exit after
+    // every stage makes the register allocator spill hundreds of registers) and the up to five
+    // remaining stages follow as straight-line code, so K may be any multiple of 128.  Loads past the
+    // last stage are clamped to it -- they land in buffers nobody reads any more -- so every stage
+    // issues the same 16 loads and the wait before its barrier is always "all but the youngest 8".
     //
     // The direct loads are inline assembly: for the builtin the compiler cannot tell which buffer a
     // later ds_read depends on and waits for vmcnt(0) every time, which would serialise exactly the
     // loads that are meant to stay in flight.  Issued this way the only vmcnt waits are the ones
-    // written here.  The "memory" clobber keeps each load between the two ds_reads it is written
-    // between, which is what spreads them over the matrix instructions.
+    // written here.
     __device__ inline void loadToLds(i32x4 rsrc, uint32_t laneOffset, uint32_t uniformOffset, uint32_t ldsAddr)
     {
         asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
@@ -969,206 +507,9 @@ namespace
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     }
 
-    template <Elem E, typename OutT>
-    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
-        gemmTiledKernel8(Params p)
-    {
-        using Traits = ElemTraits<E>;
-        using Acc    = typename Traits::Acc;
-        static_assert(Traits::Bytes == 1, "8-bit element types only");
-        constexpr uint32_t TK     = STAGE_KB; // K elements per stage
-        constexpr bool     PAIRED = (E == Elem::E4M3);
-        // LDS map: A buffers at 0 and 32 KiB, B buffers at 64, 96 and 128 KiB
-        constexpr uint32_t A_AT[2] = {0u, OPER_BYTES};
-        constexpr uint32_t B_AT[3] = {2u * OPER_BYTES, 3u * OPER_BYTES, 4u * OPER_BYTES};
-
-        __shared__ __attribute__((aligned(1024))) char lds[5u * OPER_BYTES];
-
-        uint32_t tm, tn;
-        if(!r355::tileCoord(blockIdx.x, p.tilesM, p.tilesN, tm, tn))
-            return;
-
-        const uint32_t tid  = threadIdx.x;
-        const uint32_t lane = tid & 63u;
-        const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-        const uint32_t wm = wave >> 1, wn = wave & 1u;
-        auto           swzK = [](uint32_t row) { return (row >> 1) & 7u; };
-        const uint32_t ldsBase
-            = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds));
-
-        // global -> LDS: chunk L = j * 256 + tid of an operand tile sits at LDS byte 16 L (row L / 8)
-        const uint32_t gr = tid >> 3, gslot = tid & 7u;
-        const uint32_t gOffA = gr * p.lda + ((gslot ^ swzK(gr)) * CHUNK), gStepA = 32u * p.lda;
-        const uint32_t gOffB = gr * p.ldb + ((gslot ^ swzK(gr)) * CHUNK), gStepB = 32u * p.ldb;
-        const char*    gA = p.a + (uint64_t)tm * TILE_M * p.lda;
-        const char*    gB = p.b + (uint64_t)tn * TILE_N * p.ldb;
-        const uint32_t numStages = p.k / TK;
-        const uint32_t dmaDst    = ldsBase + wave * 64u * CHUNK; // + buffer + j * 4 KiB
-
-        // buffer resource over one stage of an operand panel (clamped to the last stage)
-        auto resource = [&](const char* panel, uint32_t stage) {
-            const uint32_t st = stage < numStages ? stage : numStages - 1u;
-            const uint64_t v  = reinterpret_cast<uint64_t>(panel + (uint64_t)st * STAGE_KB);
-            return i32x4{static_cast<int>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v))),
-                         static_cast<int>(__builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32)) & 0xFFFF),
-                         0x7FFFFFFF, 0x00020000};
-        };
-        auto issueHalf = [&](i32x4 rsrc, uint32_t gOff, uint32_t gStep, uint32_t at) {
-#pragma unroll
-            for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
-                loadToLds(rsrc, gOff, j * gStep, dmaDst + at + j * THREADS * CHUNK);
-        };
-
-        // LDS -> registers: block i rows are i * 32 + lane % 32; sub-step s reads chunk 2 s + lane / 32
-        uint32_t rdA[4], rdB[4];
-        {
-            const uint32_t ra = wm * 128u + (lane & 31u), rb = wn * 128u + (lane & 31u);
-#pragma unroll
-            for(uint32_t s = 0; s < 4; ++s)
-            {
-                rdA[s] = ra * STAGE_KB + (((2u * s + (lane >> 5)) ^ swzK(ra)) * CHUNK);
-                rdB[s] = rb * STAGE_KB + (((2u * s + (lane >> 5)) ^ swzK(rb)) * CHUNK);
-            }
-        }
-        auto readA = [&](uint32_t at, uint32_t i, uint32_t s) -> i32x4 {
-            return *reinterpret_cast<const i32x4*>(lds + at + rdA[s] + i * 32u * STAGE_KB);
-        };
-        auto readB = [&](uint32_t at, uint32_t i, uint32_t s) -> i32x4 {
-            return *reinterpret_cast<const i32x4*>(lds + at + rdB[s] + i * 32u * STAGE_KB);
-        };
-
-        Acc acc[4][4];
-#pragma unroll
-        for(uint32_t i = 0; i < 4; ++i)
-#pragma unroll
-            for(uint32_t j = 0; j < 4; ++j)
-#pragma unroll
-                for(uint32_t e = 0; e < 16; ++e)
-                    acc[i][j][e] = 0;
-
-        i32x4 fa[4][4], fb[4][4];
-        auto  mfmaHalf = [&](uint32_t s0) {
-            if constexpr(PAIRED)
-            {
-#pragma unroll
-                for(uint32_t i = 0; i < 4; ++i)
-#pragma unroll
-                    for(uint32_t j = 0; j < 4; ++j)
-                        mfma64Fp8(acc[i][j], fb[s0][j], fb[s0 + 1][j], fa[s0][i], fa[s0 + 1][i]);
-            }
-            else
-            {
-#pragma unroll
-                for(uint32_t s = s0; s < s0 + 2u; ++s)
-#pragma unroll
-                    for(uint32_t i = 0; i < 4; ++i)
-#pragma unroll
-                        for(uint32_t j = 0; j < 4; ++j)
-                            mfma32<E>(acc[i][j], fb[s][j], fa[s][i]);
-            }
-        };
-        constexpr uint32_t MFMA_PER_HALF = PAIRED ? 16u : 32u;
-
-        // One K stage: operands of sub-steps 0, 1 are in registers; 2, 3 arrive under the first half of
-        // the matrix instructions; then every wave is done with this stage's buffers, they are refilled
-        // (A two stages ahead, B three), and sub-steps 0, 1 of the next stage arrive under the second half.
-        auto stageBody = [&](uint32_t kt, uint32_t aCur, uint32_t aNxt, uint32_t bCur, uint32_t bNxt) {
-#pragma unroll
-            for(uint32_t s = 2; s < 4; ++s)
-#pragma unroll
-                for(uint32_t i = 0; i < 4; ++i)
-                {
-                    fa[s][i] = readA(aCur, i, s);
-                    fb[s][i] = readB(bCur, i, s);
-                }
-            mfmaHalf(0);
-#pragma unroll
-            for(uint32_t g = 0; g < 16; ++g)
-                schedGroup<MFMA_PER_HALF / 16u, 1, 0>();
-
-            waitVmcnt<8>(); // this wave's part of stage kt + 1 has landed (the youngest 8 loads are B of kt + 2)
-            ldsBarrier();
-
-            const i32x4 rsrcA = resource(gA, kt + 2u), rsrcB = resource(gB, kt + 3u);
-#pragma unroll
-            for(uint32_t g = 0; g < 16; ++g)
-            {
-                const uint32_t s = g >> 3, i = (g >> 1) & 3u;
-                if(g & 1u)
-                    fb[s][i] = readB(bNxt, i, s);
-                else
-                    fa[s][i] = readA(aNxt, i, s);
-                if(g < 8u)
-                    loadToLds(rsrcA, gOffA, g * gStepA, dmaDst + aCur + g * THREADS * CHUNK);
-                else
-                    loadToLds(rsrcB, gOffB, (g - 8u) * gStepB, dmaDst + bCur + (g - 8u) * THREADS * CHUNK);
-            }
-            mfmaHalf(2);
-#pragma unroll
-            for(uint32_t g = 0; g < 16; ++g)
-                schedGroup<MFMA_PER_HALF / 16u, 1, 0>();
-            __builtin_amdgcn_sched_barrier(0); // one scheduling region per stage
-        };
-
-        // prologue: stages 0 and 1 and the B half of stage 2 requested; stage 0 published
-        issueHalf(resource(gA, 0u), gOffA, gStepA, A_AT[0]);
-        issueHalf(resource(gB, 0u), gOffB, gStepB, B_AT[0]);
-        issueHalf(resource(gA, 1u), gOffA, gStepA, A_AT[1]);
-        issueHalf(resource(gB, 1u), gOffB, gStepB, B_AT[1]);
-        issueHalf(resource(gB, 2u), gOffB, gStepB, B_AT[2]);
-        waitVmcnt<24>();
-        ldsBarrier();
-#pragma unroll
-        for(uint32_t s = 0; s < 2u; ++s)
-#pragma unroll
-            for(uint32_t i = 0; i < 4; ++i)
-            {
-                fa[s][i] = readA(A_AT[0], i, s);
-                fb[s][i] = readB(B_AT[0], i, s);
-            }
-
-        // Six stages per trip.  The loop has a single exit: with an exit after every stage the register
-        // allocator rotates the accumulators through the loop and spills hundreds of registers.  The up
-        // to five remaining stages follow as straight-line code.
-        uint32_t kt = 0;
-        for(uint32_t trips = numStages / 6u; trips > 0; --trips, kt += 6u)
-        {
-            stageBody(kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1]);
-            stageBody(kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2]);
-            stageBody(kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0]);
-            stageBody(kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1]);
-            stageBody(kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2]);
-            stageBody(kt + 5u, A_AT[1], A_AT[0], B_AT[2], B_AT[0]);
-        }
-        const uint32_t rem = numStages - kt;
-        if(rem > 0u)
-        {
-            stageBody(kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1]);
-            if(rem > 1u)
-            {
-                stageBody(kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2]);
-                if(rem > 2u)
-                {
-                    stageBody(kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0]);
-                    if(rem > 3u)
-                    {
-                        stageBody(kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1]);
-                        if(rem > 4u)
-                            stageBody(kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2]);
-                    }
-                }
-            }
-        }
-
-        // the clamped loads of the last stages are still landing in buffers the epilogue reuses
-        waitVmcnt<0>();
-        ldsBarrier();
-        storeTile<E, OutT>(acc, p, tm, tn, wm, wn, lane, lds + wave * OPER_BYTES);
-    }
-
     // ------------------------------------------------------------------------------------------
-    // int8 on v_mfma_i32_16x16x64_i8: the five-buffer scheme of gemmTiledKernel8 with the K-step
-    // structure and the in-place inline-assembly accumulators of gemmTiledKernel16.  A stage is two
+    // int8 on v_mfma_i32_16x16x64_i8: the five-buffer scheme with the K-step structure and the
+    // in-place inline-assembly accumulators of gemmTiledKernel16.  A stage is two
     // K steps of 64 bytes; lane -> operand mapping: row lane % 16, 16-byte chunk lane / 16 of the step.
     using i32x4v = int __attribute__((ext_vector_type(4)));
     __device__ __forceinline__ void mfma16i8(i32x4v& acc, i32x4 x, i32x4 y)
@@ -1551,81 +892,23 @@ namespace
         storeTile16<f32x4, float>(acc, p, tm, tn, wm, wn, lane, lds + wave * OPER_BYTES);
     }
 
-    struct Variant
-    {
-        bool direct;
-        bool banks64;
-        bool shape32; // 16-bit types on the 32 x 32 x 16 instruction shapes (the earlier kernel)
-    };
-    // Defaults chosen from measurements on MI355X; R355_TILED_VARIANT=<bit0: direct-to-LDS loads,
-    // bit1: 64-bank swizzle, bit2: 32 x 32 instruction shapes> overrides them for experiments (16-bit types).
-    Variant chosenVariant()
-    {
-        static const Variant v = [] {
-            Variant     r{true, true, false};
-            const char* e = getenv("R355_TILED_VARIANT");
-            if(e)
-            {
-                int x     = atoi(e);
-                r.direct  = x & 1;
-                r.banks64 = x & 2;
-                r.shape32 = x & 4;
-            }
-            return r;
-        }();
-        return v;
-    }
-
-    template <Elem E, typename OutT, bool AK, bool BK>
-    int launchVariant(Params p, hipStream_t stream)
-    {
-        const Variant  v    = chosenVariant();
-        const uint32_t grid = ((p.tilesM * p.tilesN + 7u) / 8u) * 8u;
-        p.banks64           = v.banks64;
-        if(!v.shape32)
-            hipLaunchKernelGGL((gemmTiledKernel16<E, OutT, AK, BK>), dim3(grid), dim3(THREADS), 0, stream, p);
-        else if(v.direct)
-            hipLaunchKernelGGL((gemmTiledKernel<E, OutT, AK, BK, true>), dim3(grid), dim3(THREADS), 0, stream, p);
-        else
-            hipLaunchKernelGGL((gemmTiledKernel<E, OutT, AK, BK, false>), dim3(grid), dim3(THREADS), 0, stream, p);
-        return r355::checkLaunch("gemm (macro tile)");
-    }
-
     template <Elem E, typename OutT>
     int launchLayouts(bool aK, bool bK, const Params& p, hipStream_t stream)
     {
-        if constexpr(ElemTraits<E>::Bytes == 1)
-        {
-            const uint32_t grid = ((p.tilesM * p.tilesN + 7u) / 8u) * 8u;
-            if constexpr(E == Elem::I8)
-            {
-                if(!chosenVariant().shape32)
-                {
-                    hipLaunchKernelGGL(gemmTiledKernelI8, dim3(grid), dim3(THREADS), 0, stream, p);
-                    return r355::checkLaunch("gemm (macro tile, int8)");
-                }
-            }
-            if constexpr(E == Elem::E4M3)
-            {
-                if(!chosenVariant().shape32)
-                {
-                    hipLaunchKernelGGL(gemmTiledKernelF8, dim3(grid), dim3(THREADS), 0, stream, p);
-                    return r355::checkLaunch("gemm (macro tile, e4m3)");
-                }
-            }
-            hipLaunchKernelGGL((gemmTiledKernel8<E, OutT>), dim3(grid), dim3(THREADS), 0, stream, p);
-            return r355::checkLaunch("gemm (macro tile, 8-bit)");
-        }
+        const dim3 grid(((p.tilesM * p.tilesN + 7u) / 8u) * 8u), block(THREADS);
+        if constexpr(E == Elem::I8)
+            hipLaunchKernelGGL(gemmTiledKernelI8, grid, block, 0, stream, p);
+        else if constexpr(E == Elem::E4M3)
+            hipLaunchKernelGGL(gemmTiledKernelF8, grid, block, 0, stream, p);
+        else if(aK && bK)
+            hipLaunchKernelGGL((gemmTiledKernel16<E, OutT, true, true>), grid, block, 0, stream, p);
+        else if(aK)
+            hipLaunchKernelGGL((gemmTiledKernel16<E, OutT, true, false>), grid, block, 0, stream, p);
+        else if(bK)
+            hipLaunchKernelGGL((gemmTiledKernel16<E, OutT, false, true>), grid, block, 0, stream, p);
         else
-        {
-            if(aK && bK)
-                return launchVariant<E, OutT, true, true>(p, stream);
-            if(aK && !bK)
-                return launchVariant<E, OutT, true, false>(p, stream);
-            if(!aK && bK)
-                return launchVariant<E, OutT, false, true>(p, stream);
-            return launchVariant<E, OutT, false, false>(p, stream);
-        }
+            hipLaunchKernelGGL((gemmTiledKernel16<E, OutT, false, false>), grid, block, 0, stream, p);
+        return r355::checkLaunch("gemm (macro tile)");
     }
 } // namespace
 
@@ -1695,7 +978,6 @@ namespace r355
             aK = g.layout_b == R355_COL_MAJOR, bK = g.layout_a == R355_ROW_MAJOR;
         }
         p.tilesM = p.m / TILE_M, p.tilesN = p.n / TILE_N;
-        p.banks64 = 0;
         switch(g.in_type)
         {
         case R355_F16:
