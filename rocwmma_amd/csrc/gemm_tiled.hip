@@ -39,6 +39,7 @@
 #include <hip/hip_runtime.h>
 
 #include "common.hpp"
+#include "lds_dma.hpp"
 #include "tile_map.hpp"
 
 namespace
@@ -484,28 +485,9 @@ namespace
     // later ds_read depends on and waits for vmcnt(0) every time, which would serialise exactly the
     // loads that are meant to stay in flight.  Issued this way the only vmcnt waits are the ones
     // written here.
-    __device__ inline void loadToLds(i32x4 rsrc, uint32_t laneOffset, uint32_t uniformOffset, uint32_t ldsAddr)
-    {
-        asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
-                     :
-                     : "v"(laneOffset), "s"(rsrc), "s"(uniformOffset), "s"(ldsAddr)
-                     : "memory");
-    }
-
-    template <uint32_t N>
-    __device__ inline void waitVmcnt()
-    {
-        // vmcnt is split over bits [3:0] and [15:14]; expcnt and lgkmcnt stay at their maxima
-        __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15u) | ((N >> 4) << 14));
-    }
-
-    // barrier that orders LDS traffic only: __syncthreads() also fences global memory
-    __device__ inline void ldsBarrier()
-    {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-    }
+    using r355::ldsBarrier;
+    using r355::loadToLds;
+    using r355::waitVmcnt;
 
     // ------------------------------------------------------------------------------------------
     // int8 on v_mfma_i32_16x16x64_i8: the five-buffer scheme with the K-step structure and the

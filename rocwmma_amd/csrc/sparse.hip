@@ -9,10 +9,11 @@
 // B is dense, col-major (k contiguous); D row- or col-major.
 //
 // Two kernels:
-//   sparseTiledKernel    256 x 256 macro tile, 128 dense K per stage, double-buffered LDS filled
-//                        by direct-to-LDS loads (kept values 16 KiB + indices 4 KiB + dense B
-//                        32 KiB per stage), 2 x 2 waves with 4 x 4 v_smfmac_*_32x32x64 accumulators
-//                        each; the result is transposed through LDS so that D leaves in whole rows.
+//   sparseTiledKernel    256 x 256 macro tile, 128 dense K per stage, a ring of three LDS slots filled
+//                        by direct-to-LDS loads two stages ahead (kept values 16 KiB + indices 4 KiB
+//                        + dense B 32 KiB per stage), 2 x 2 waves with 4 x 4 v_smfmac_*_32x32x64
+//                        accumulators each; the result is transposed through LDS so that D leaves in
+//                        whole rows.
 //   sparseBlockPerWave   one 32 x 32 block of D per wave straight from global memory; fallback
 //                        for shapes that do not fill a macro tile.
 // Per 64-wide K step a lane feeds 16 kept bytes + 4 index bytes of A and 2 x 16 dense bytes of B.  Operand formats of v_smfmac_*_32x32x64 as measured on MI355X: index
@@ -22,6 +23,7 @@
 #include <cstring>
 
 #include "common.hpp"
+#include "lds_dma.hpp"
 #include "tile_map.hpp"
 
 namespace
@@ -124,15 +126,25 @@ namespace
         uint32_t       dRow; // D (and C) row-major
     };
 
+    // Three 52 KiB stage slots (156 of 160 KiB): a stage's 32 matrix instructions last about as long
+    // as half the latency of a direct load, so the slot of stage kt is refilled with stage kt + 3 and
+    // two stages of loads (104 KiB per CU) are in flight at any time.  The direct loads are explicit
+    // (lds_dma.hpp) and the only vmcnt wait is "all but the youngest 13" before each barrier; loads
+    // past the last stage are clamped to it, so every stage issues the same 13.  Every matrix
+    // instruction is followed by one LDS read and (second half of a stage) one direct load, pinned
+    // by scheduling barriers.  Three stages bring every slot back to its role: single-exit loop of
+    // three plus up to two stages of straight-line code.
+    constexpr uint32_t RING = 3, LOADS_PER_STAGE = 13;
+
     template <bool FP8>
     __global__ void __launch_bounds__(T_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
         sparseTiledKernel(TiledParams p)
     {
         using Acc  = std::conditional_t<FP8, f32x16, i32x16>;
         using AccE = std::conditional_t<FP8, float, int>;
+        using r355::loadToLds;
 
-        __shared__ __attribute__((aligned(1024))) char stage0[STAGE_BYTES];
-        __shared__ __attribute__((aligned(1024))) char stage1[STAGE_BYTES];
+        __shared__ __attribute__((aligned(1024))) char lds[RING * STAGE_BYTES];
 
         uint32_t tm, tn;
         if(!r355::tileCoord(blockIdx.x, p.tilesM, p.tilesN, tm, tn))
@@ -143,34 +155,34 @@ namespace
         const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const uint32_t wm = wave >> 1, wn = wave & 1u;
         const uint32_t r32 = lane & 31u, g = lane >> 5;
+        const uint32_t ldsBase
+            = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds));
 
         // ---- global -> LDS (per thread, fixed).  LDS chunk L = j * 256 + tid of each operand tile.
         //   kept values: 4 chunks per row, chunk c of row r in slot c ^ ((r >> 2) & 3)
         //   dense B:     8 chunks per row, chunk c of row r in slot c ^ ((r >> 1) & 7)
         //   indices:     one 16-byte chunk per row, thread t <-> row t
         const uint32_t rowA = tid >> 2, slotA = tid & 3u;
-        const uint32_t gOffA = rowA * p.lda + ((slotA ^ ((rowA >> 2) & 3u)) * 16u);
+        const uint32_t gOffA = rowA * p.lda + ((slotA ^ ((rowA >> 2) & 3u)) * 16u), gStepA = 64u * p.lda;
         const uint32_t rowB = tid >> 3, slotB = tid & 7u;
-        const uint32_t gOffB = rowB * p.ldb + ((slotB ^ ((rowB >> 1) & 7u)) * 16u);
+        const uint32_t gOffB = rowB * p.ldb + ((slotB ^ ((rowB >> 1) & 7u)) * 16u), gStepB = 32u * p.ldb;
         const uint32_t gOffM = tid * (p.k / 8u);
-        const uint8_t* gA = p.aVals + (uint64_t)tm * T_M * p.lda;
-        const uint8_t* gM = p.aMeta + (uint64_t)tm * T_M * (p.k / 8u);
-        const uint8_t* gB = p.b + (uint64_t)tn * T_N * p.ldb;
+        const uint32_t numStages = p.k / T_K;
+        const uint64_t gA = r355::uniformAddress(p.aVals + (uint64_t)tm * T_M * p.lda);
+        const uint64_t gM = r355::uniformAddress(p.aMeta + (uint64_t)tm * T_M * (p.k / 8u));
+        const uint64_t gB = r355::uniformAddress(p.b + (uint64_t)tn * T_N * p.ldb);
+        const uint32_t dmaDst = ldsBase + wave * 1024u; // lane l lands at dmaDst + slot + piece + 16 l
 
-        auto issueGlobal = [&](uint32_t kt, char* stage) {
-            using gp = const __attribute__((address_space(1))) void*;
-            using lp = __attribute__((address_space(3))) void*;
-            const uint8_t* srcA = gA + kt * (T_K / 2u);
-            const uint8_t* srcB = gB + kt * T_K;
-            char* dst = stage + wave * 1024u; // lane l lands at dst + 16 l
-#pragma unroll
-            for(uint32_t j = 0; j < 4; ++j) // 64 rows of kept values per j
-                __builtin_amdgcn_global_load_lds((gp)(srcA + (uint64_t)j * 64u * p.lda + gOffA), (lp)(dst + j * 4096u), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((gp)(gM + kt * (T_K / 8u) + gOffM), (lp)(dst + OFF_META), 16, 0, 0);
-#pragma unroll
-            for(uint32_t j = 0; j < 8; ++j) // 32 rows of B per j
-                __builtin_amdgcn_global_load_lds((gp)(srcB + (uint64_t)j * 32u * p.ldb + gOffB), (lp)(dst + OFF_B + j * 4096u), 16, 0, 0);
+        // load x (0..12) of stage `stage` (already clamped) into the slot at byte `at`
+        auto issueLoad = [&](uint32_t stage, uint32_t at, uint32_t x) {
+            if(x < 4u) // 64 rows of kept values per load
+                loadToLds(r355::rawBuffer(gA + stage * (T_K / 2u)), gOffA, x * gStepA, dmaDst + at + x * 4096u);
+            else if(x == 4u)
+                loadToLds(r355::rawBuffer(gM + stage * (T_K / 8u)), gOffM, 0u, dmaDst + at + OFF_META);
+            else // 32 rows of B per load
+                loadToLds(r355::rawBuffer(gB + stage * T_K), gOffB, (x - 5u) * gStepB, dmaDst + at + OFF_B + (x - 5u) * 4096u);
         };
+        auto clampStage = [&](uint32_t stage) { return stage < numStages ? stage : numStages - 1u; };
 
         // ---- LDS -> registers (per lane, fixed)
         const uint32_t rA   = wm * 128u + r32, rB = wn * 128u + r32;
@@ -190,14 +202,16 @@ namespace
             int   idx[4];
             i32x4 b0[4], b1[4];
         };
-        auto readGroup = [&](Frags& f, const char* base, uint32_t q) {
-#pragma unroll
-            for(uint32_t i = 0; i < 4; ++i)
+        // read x (0..15) of K group q: the four operands of block index x / 4, values first
+        auto readPiece = [&](Frags& f, uint32_t at, uint32_t q, uint32_t x) {
+            const uint32_t i = x >> 2;
+            const char*    base = lds + at;
+            switch(x & 3u)
             {
-                f.a[i]   = *reinterpret_cast<const i32x4*>(base + rdA[q] + i * 32u * 64u);
-                f.idx[i] = *reinterpret_cast<const int*>(base + rdM + 8u * q + i * 32u * 16u);
-                f.b0[i]  = *reinterpret_cast<const i32x4*>(base + rdB[2u * q] + i * 32u * 128u);
-                f.b1[i]  = *reinterpret_cast<const i32x4*>(base + rdB[2u * q + 1u] + i * 32u * 128u);
+            case 0: f.a[i] = *reinterpret_cast<const i32x4*>(base + rdA[q] + i * 32u * 64u); break;
+            case 1: f.idx[i] = *reinterpret_cast<const int*>(base + rdM + 8u * q + i * 32u * 16u); break;
+            case 2: f.b0[i] = *reinterpret_cast<const i32x4*>(base + rdB[2u * q] + i * 32u * 128u); break;
+            default: f.b1[i] = *reinterpret_cast<const i32x4*>(base + rdB[2u * q + 1u] + i * 32u * 128u); break;
             }
         };
 
@@ -210,66 +224,73 @@ namespace
                 for(uint32_t e = 0; e < 16; ++e)
                     acc[i][j][e] = 0;
 
-        auto mfmaGroup = [&](const Frags& f) {
-#pragma unroll
-            for(uint32_t i = 0; i < 4; ++i)
-#pragma unroll
-                for(uint32_t j = 0; j < 4; ++j)
-                {
-                    const i32x8 bv = {f.b0[j][0], f.b0[j][1], f.b0[j][2], f.b0[j][3],
-                                      f.b1[j][0], f.b1[j][1], f.b1[j][2], f.b1[j][3]};
-                    if constexpr(FP8)
-                        acc[i][j] = __builtin_amdgcn_smfmac_f32_32x32x64_fp8_fp8(f.a[i], bv, acc[i][j], f.idx[i], 0, 0);
-                    else
-                        acc[i][j] = __builtin_amdgcn_smfmac_i32_32x32x64_i8(f.a[i], bv, acc[i][j], f.idx[i], 0, 0);
-                }
-        };
-        auto hint = [&](bool reads, bool loads) {
-            // 16 LDS reads (4 values + 4 indices + 8 dense) and 13 global loads per 16 matrix instructions
-#pragma unroll
-            for(uint32_t x = 0; x < 8; ++x)
-            {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                if(reads)
-                    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-                if(loads)
-                    __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
-            }
-            __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+        // matrix instruction n (0..15) of a K group: L-shaped shells, so that block index d of either
+        // operand is first needed after d * d instructions (the reads arrive block by block)
+        auto mfmaAt = [&](const Frags& f, uint32_t n) {
+            uint32_t d = 0;
+            while((d + 1u) * (d + 1u) <= n)
+                ++d;
+            const uint32_t r = n - d * d;
+            const uint32_t i = r <= d ? d : r - d - 1u, j = r <= d ? r : d;
+            const i32x8    bv = {f.b0[j][0], f.b0[j][1], f.b0[j][2], f.b0[j][3], f.b1[j][0], f.b1[j][1], f.b1[j][2], f.b1[j][3]};
+            if constexpr(FP8)
+                acc[i][j] = __builtin_amdgcn_smfmac_f32_32x32x64_fp8_fp8(f.a[i], bv, acc[i][j], f.idx[i], 0, 0);
+            else
+                acc[i][j] = __builtin_amdgcn_smfmac_i32_32x32x64_i8(f.a[i], bv, acc[i][j], f.idx[i], 0, 0);
         };
 
         Frags f0, f1;
-        auto  stageBody = [&](uint32_t kt, char* cur, char* nxt, auto refill, auto hasNext) {
-            constexpr bool REFILL = decltype(refill)::value, NEXT = decltype(hasNext)::value;
-            readGroup(f1, cur, 1);
-            mfmaGroup(f0);
-            hint(true, false);
-            __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): own direct loads of stage kt + 1 have landed
-            __syncthreads();
-            if constexpr(REFILL)
-                issueGlobal(kt + 2, cur);
-            if constexpr(NEXT)
-                readGroup(f0, nxt, 0);
-            mfmaGroup(f1);
-            hint(NEXT, REFILL);
+        auto  stageBody = [&](uint32_t kt, uint32_t cur, uint32_t nxt) {
+#pragma unroll
+            for(uint32_t n = 0; n < 16; ++n)
+            {
+                mfmaAt(f0, n);
+                readPiece(f1, cur, 1, n);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            r355::waitVmcnt<LOADS_PER_STAGE>(); // stage kt + 1 has landed; the youngest 13 loads are stage kt + 2
+            r355::ldsBarrier();
+            const uint32_t refill = clampStage(kt + 3u);
+#pragma unroll
+            for(uint32_t n = 0; n < 16; ++n)
+            {
+                mfmaAt(f1, n);
+                readPiece(f0, nxt, 0, n);
+                if(n < LOADS_PER_STAGE)
+                    issueLoad(refill, cur, n);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         };
-        constexpr std::true_type  yes{};
-        constexpr std::false_type no{};
 
-        const uint32_t numStages = p.k / T_K; // even, >= 2 (checked on the host)
-        issueGlobal(0, stage0);
-        issueGlobal(1, stage1);
-        __builtin_amdgcn_s_waitcnt(0x0F70);
-        __syncthreads();
-        readGroup(f0, stage0, 0);
+        constexpr uint32_t SLOT[3] = {0u, STAGE_BYTES, 2u * STAGE_BYTES};
+#pragma unroll
+        for(uint32_t st = 0; st < RING; ++st)
+#pragma unroll
+            for(uint32_t x = 0; x < LOADS_PER_STAGE; ++x)
+                issueLoad(clampStage(st), SLOT[st], x);
+        r355::waitVmcnt<2u * LOADS_PER_STAGE>();
+        r355::ldsBarrier();
+#pragma unroll
+        for(uint32_t x = 0; x < 16; ++x)
+            readPiece(f0, SLOT[0], 0, x);
+
         uint32_t kt = 0;
-        for(; kt + 2 < numStages; kt += 2)
+        for(uint32_t trips = numStages / 3u; trips > 0; --trips, kt += 3u)
         {
-            stageBody(kt, stage0, stage1, yes, yes);
-            stageBody(kt + 1, stage1, stage0, yes, yes);
+            stageBody(kt, SLOT[0], SLOT[1]);
+            stageBody(kt + 1u, SLOT[1], SLOT[2]);
+            stageBody(kt + 2u, SLOT[2], SLOT[0]);
         }
-        stageBody(kt, stage0, stage1, no, yes);
-        stageBody(kt + 1, stage1, stage0, no, no);
+        const uint32_t rem = numStages - kt;
+        if(rem > 0u)
+        {
+            stageBody(kt, SLOT[0], SLOT[1]);
+            if(rem > 1u)
+                stageBody(kt + 1u, SLOT[1], SLOT[2]);
+        }
+        // the clamped loads of the last stages are still landing in the slots the epilogue reuses
+        r355::waitVmcnt<0>();
+        r355::ldsBarrier();
 
         // ---- epilogue.  lane holds D(m = 8 (e / 4) + 4 g + e % 4, n = lane % 32) of each block:
         // four consecutive rows of one column.
@@ -302,9 +323,9 @@ namespace
                     }
             return;
         }
-        // row-major: transpose through this wave's 26 KiB of the idle stage buffers, 32 rows (one
+        // row-major: transpose through this wave's 26 KiB of the idle stage slots, 32 rows (one
         // block row i) at a time: rows of 128 x 4 bytes = 32 chunks, chunk c of row r in slot c ^ r.
-        char* wl = ((wave < 2u) ? stage0 : stage1) + (wave & 1u) * 26624u;
+        char* wl = lds + wave * 26624u;
 #pragma unroll
         for(uint32_t i = 0; i < 4; ++i)
         {
@@ -339,7 +360,7 @@ namespace
 
     bool tiledOk(const r355_gemm_args& g)
     {
-        return g.kernel != R355_KERNEL_SIMPLE && g.m % T_M == 0 && g.n % T_N == 0 && g.k % (2 * T_K) == 0
+        return g.kernel != R355_KERNEL_SIMPLE && g.m % T_M == 0 && g.n % T_N == 0 && g.k % T_K == 0
                && g.layout_c == g.layout_d && (g.ldd % 4) == 0 && r355::aligned(g.d, 16)
                && (g.beta == 0.0f || ((g.ldc % 4) == 0 && r355::aligned(g.c, 16))) && r355::aligned(g.a_meta, 16);
     }
@@ -362,7 +383,7 @@ namespace r355
         if(!aligned(g.a, 16) || g.lda % 16 || !aligned(g.b, 16) || g.ldb % 16 || !aligned(g.a_meta, 4) || !aligned(g.d, 4))
             return fail(R355_ERR_MISALIGNED, "sparse gemm: values / B need 16-byte alignment, metadata 4-byte");
         if(g.kernel == R355_KERNEL_TILED && !tiledOk(g))
-            return fail(R355_ERR_BAD_SIZE, "sparse gemm (macro tile): m=%u n=%u must be multiples of 256, k=%u of 256, C/D same orientation and 16-byte aligned", g.m, g.n, g.k);
+            return fail(R355_ERR_BAD_SIZE, "sparse gemm (macro tile): m=%u n=%u must be multiples of 256, k=%u of 128, C/D same orientation and 16-byte aligned", g.m, g.n, g.k);
         if(plan && tiledOk(g))
         {
             plan->kernel       = R355_KERNEL_TILED;
@@ -373,7 +394,7 @@ namespace r355
             plan->grid_y       = 1;
             plan->block_x      = T_THREADS;
             plan->block_y      = 1;
-            plan->lds_bytes    = 2 * STAGE_BYTES;
+            plan->lds_bytes    = RING * STAGE_BYTES;
         }
         else if(plan)
         {

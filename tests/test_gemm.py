@@ -161,6 +161,22 @@ def test_tiled_kernel_8bit(in_t, out_t, ldl):
     _check(in_t, out_t, got, want)
 
 
+@pytest.mark.parametrize("in_t,out_t", [(O.F16, O.F32), (O.BF16, O.BF16)])
+@pytest.mark.parametrize("la,lb", [(O.COL, O.ROW), (O.ROW, O.COL)])
+@pytest.mark.parametrize("k", [128, 256, 640])
+def test_tiled_kernel_16bit_stage_counts(in_t, out_t, la, lb, k):
+    # the 16-bit kernel runs K stages of 64 in pairs and clamps its refills past the last stage:
+    # the smallest K (one pair), two pairs and an odd number of pairs
+    m, n = 256, 256
+    a, b, _ = _inputs(in_t, out_t, m, n, k, seed=60 + k)
+    want = O.gemm(in_t, out_t, la, lb, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0)
+    got = _run(in_t, out_t, la, lb, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0, R.KERNEL_TILED)
+    w32 = None
+    if out_t != O.F32:
+        w32 = O.gemm(in_t, O.F32, la, lb, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0)
+    _check(in_t, out_t, got, want, w32)
+
+
 @pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32)])
 @pytest.mark.parametrize("stages", [1, 2, 3, 4, 5, 6, 7, 11, 13])
 def test_tiled_kernel_8bit_stage_counts(in_t, out_t, stages):
