@@ -57,7 +57,7 @@ typedef enum
     R355_KERNEL_SIMPLE = 1, /* one MFMA block per wave through the fragment API, no LDS
                                (samples/simple_hgemm.cpp:81-139,
                                 test/gemm/gemm_PGR0_LB0_MP0_SB_NC/device/kernel_device_func.hpp:50-175) */
-    R355_KERNEL_TILED  = 2  /* LDS-staged double-buffered macro tile
+    R355_KERNEL_TILED  = 2  /* LDS-staged 256 x 256 macro tile (m, n multiples of 256, k of 128)
                                (samples/perf_hgemm.cpp:515-711,
                                 test/gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp:52-283) */
 } r355_gemm_kernel;
@@ -67,7 +67,7 @@ typedef enum
  * Argument order and meaning follow the reference kernel signature
  * (test/gemm/gemm_kernel_base.hpp:101-114): leading dimensions in elements.
  * Supported (in -> out, accumulate): f16 -> f32|f16 (f32), bf16 -> f32|bf16 (f32),
- * e4m3 -> f32 (f32), i8 -> i32 (i32, alpha/beta truncated to int32), f32 -> f32 (f32).
+ * e4m3 -> f32 (f32), i8 -> i32 (i32, alpha/beta truncated to int32), f32 -> f32 (f32), f64 -> f64 (f64).
  * beta == 0 means C is never read and may be NULL.
  *
  * sparse24 != 0: A is 2:4 structured-sparse along k, row-major, 1-byte elements:

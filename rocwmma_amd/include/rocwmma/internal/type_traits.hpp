@@ -6,7 +6,9 @@
 #ifndef ROCWMMA_TYPE_TRAITS_HPP
 #define ROCWMMA_TYPE_TRAITS_HPP
 
+#if !defined(__HIPCC_RTC__)
 #include <limits>
+#endif
 
 #include "types.hpp"
 

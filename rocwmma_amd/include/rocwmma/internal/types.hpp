@@ -7,6 +7,9 @@
 #ifndef ROCWMMA_TYPES_HPP
 #define ROCWMMA_TYPES_HPP
 
+#if defined(__HIPCC_RTC__)
+#include "rtc_compat.hpp"
+#else
 #include <cstdint>
 #include <type_traits>
 
@@ -14,6 +17,7 @@
 #include <hip/hip_bfloat16.h>
 #include <hip/hip_fp16.h>
 #include <hip/hip_fp8.h>
+#endif
 
 #include "config.hpp"
 

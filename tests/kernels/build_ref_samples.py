@@ -26,6 +26,19 @@ def _compile(name, samples):
     return out
 
 
+def _compile_hiprtc_sample(samples):
+    """samples/hipRTC_gemm.cpp as the program it is: its host side compiles the kernel string at run
+    time with hipRTC, against whatever <ROCM_PATH>/include/rocwmma holds (samples/hipRTC_gemm.cpp:185-206),
+    runs it and validates against its own CPU GEMM (:359-381)."""
+    out = os.path.join(OUT, "hiprtc_gemm")
+    subprocess.check_call([
+        os.environ.get("HIPCC", "/opt/rocm/bin/hipcc"), "--offload-arch=gfx950", "-std=c++17", "-O2", "-w",
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
+        "-I" + os.path.join(ROOT, "rocwmma_amd", "include"), "-I" + samples,
+        os.path.join(samples, "hipRTC_gemm.cpp"), "-o", out, "-lhiprtc"])
+    return out
+
+
 def build():
     samples = os.path.join(REF, "samples")
     if not os.path.isdir(samples):
@@ -34,7 +47,8 @@ def build():
     from concurrent.futures import ThreadPoolExecutor
 
     with ThreadPoolExecutor(max_workers=min(6, os.cpu_count() or 1)) as pool:
-        return list(pool.map(lambda n: _compile(n, samples), WRAPPERS))
+        rtc = pool.submit(_compile_hiprtc_sample, samples)
+        return list(pool.map(lambda n: _compile(n, samples), WRAPPERS)) + [rtc.result()]
 
 
 if __name__ == "__main__":
