@@ -48,7 +48,10 @@ namespace
             *family = -1;
             return rc;
         }
-        if(g->kernel == R355_KERNEL_TILED || g->kernel == R355_KERNEL_AUTO)
+        // AUTO leaves problems smaller than half a macro tile in either direction to the block-per-wave
+        // kernel: one mostly empty 256 x 256 tile on one CU is slower than many small blocks.
+        const bool worthTiling = g->kernel == R355_KERNEL_TILED || (g->m >= 128 && g->n >= 128);
+        if((g->kernel == R355_KERNEL_TILED || g->kernel == R355_KERNEL_AUTO) && worthTiling)
         {
             rc = r355::gemmTiledCheck(*g, out);
             if(rc == R355_OK)

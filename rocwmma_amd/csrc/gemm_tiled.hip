@@ -178,9 +178,12 @@ namespace
                 {
                     const uint32_t L = it * 64u + lane, row = L / ROW_CHUNKS, c = L % ROW_CHUNKS;
                     const i32x4    v = *reinterpret_cast<const i32x4*>(scratch + row * ROW_BYTES + ((c ^ (row & 15u)) * CHUNK));
-                    const uint64_t offD = (uint64_t)(m0 + pass * ROWS_PASS + row) * p.ldd + n0;
-                    // D is written once and not read again: stream it past the caches
-                    __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(p.d + offD * OS + c * CHUNK));
+                    const uint32_t gRow = m0 + pass * ROWS_PASS + row, gCol = n0 + c * (CHUNK / OS);
+                    const uint64_t offD = (uint64_t)gRow * p.ldd + n0;
+                    // D is written once and not read again: stream it past the caches.  Edge tiles:
+                    // m and n are multiples of 16, so a 16-byte chunk is inside D or outside as a whole.
+                    if(gRow < p.m && gCol < p.n)
+                        __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(p.d + offD * OS + c * CHUNK));
                 }
                 __builtin_amdgcn_wave_barrier();
             }
@@ -194,7 +197,8 @@ namespace
             OutV           cv[8];
 #pragma unroll
             for(uint32_t j = 0; j < 8; ++j)
-                cv[j] = *reinterpret_cast<const OutV*>(p.c + ((uint64_t)row * p.ldc + n0 + 16u * j + 4u * g) * sizeof(OutT));
+                if(row < p.m && n0 + 16u * j < p.n)
+                    cv[j] = *reinterpret_cast<const OutV*>(p.c + ((uint64_t)row * p.ldc + n0 + 16u * j + 4u * g) * sizeof(OutT));
 #pragma unroll
             for(uint32_t j = 0; j < 8; ++j)
             {
@@ -202,7 +206,8 @@ namespace
 #pragma unroll
                 for(uint32_t e = 0; e < 4; ++e)
                     out[e] = static_cast<OutT>(alpha * acc[i][j][e] + beta * static_cast<AccE>(cv[j][e]));
-                *reinterpret_cast<OutV*>(p.d + ((uint64_t)row * p.ldd + n0 + 16u * j + 4u * g) * sizeof(OutT)) = out;
+                if(row < p.m && n0 + 16u * j < p.n)
+                    *reinterpret_cast<OutV*>(p.d + ((uint64_t)row * p.ldd + n0 + 16u * j + 4u * g) * sizeof(OutT)) = out;
             }
         }
     }
@@ -236,34 +241,41 @@ namespace
         // ---------------- global -> LDS: chunk L = j * 256 + tid of an operand tile sits at LDS byte 16 L.
         // K-contiguous: row L / 8, and the swizzle does not change with j (32 rows per load).
         // M/N-contiguous: k-row L / 32 = 8 j + tid / 32; the swizzle alternates with bit 3 of the k-row.
-        uint32_t gOffA[2], gOffB[2], gStepA, gStepB;
-        uint64_t gStageA, gStageB; // bytes between consecutive K stages
-        if constexpr(A_KCONTIG)
-        {
-            const uint32_t r = tid >> 3, slot = tid & 7u;
-            gOffA[0] = gOffA[1] = r * p.lda * ES + ((slot ^ swzK(r)) * CHUNK);
-            gStepA = 32u * p.lda * ES, gStageA = STAGE_KB;
-        }
-        else
-        {
-            const uint32_t r = tid >> 5, slot = tid & 31u;
-            gOffA[0] = r * p.lda * ES + ((slot ^ swzMN(r)) * CHUNK);
-            gOffA[1] = r * p.lda * ES + ((slot ^ swzMN(r + 8u)) * CHUNK);
-            gStepA = 8u * p.lda * ES, gStageA = (uint64_t)TK * p.lda * ES;
-        }
-        if constexpr(B_KCONTIG)
-        {
-            const uint32_t r = tid >> 3, slot = tid & 7u;
-            gOffB[0] = gOffB[1] = r * p.ldb * ES + ((slot ^ swzK(r)) * CHUNK);
-            gStepB = 32u * p.ldb * ES, gStageB = STAGE_KB;
-        }
-        else
-        {
-            const uint32_t r = tid >> 5, slot = tid & 31u;
-            gOffB[0] = r * p.ldb * ES + ((slot ^ swzMN(r)) * CHUNK);
-            gOffB[1] = r * p.ldb * ES + ((slot ^ swzMN(r + 8u)) * CHUNK);
-            gStepB = 8u * p.ldb * ES, gStageB = (uint64_t)TK * p.ldb * ES;
-        }
+        // Edge tiles (m or n not a multiple of 256) must not read outside the operands: a lane whose
+        // row (K-contiguous) or 16-byte chunk (M/N-contiguous) lies beyond the matrix reads the last valid
+        // row / the first chunk instead -- what lands in LDS for it only feeds elements of D that are
+        // never stored.  Hence one lane offset per load (the compiler merges equal ones).
+        uint32_t       gOffA[LOADS_PER_OPER], gOffB[LOADS_PER_OPER], gStepA, gStepB; // gStep: uniform offset per load
+        uint64_t       gStageA, gStageB; // bytes between consecutive K stages
+        const uint32_t validM = p.m - tm * TILE_M < TILE_M ? p.m - tm * TILE_M : TILE_M;
+        const uint32_t validN = p.n - tn * TILE_N < TILE_N ? p.n - tn * TILE_N : TILE_N;
+        auto laneOffsets = [&](bool kContig, uint32_t ld, uint32_t valid, uint32_t (&off)[LOADS_PER_OPER], uint32_t& step,
+                               uint64_t& stage) {
+            if(kContig)
+            {
+                const uint32_t r = tid >> 3, slot = tid & 7u;
+#pragma unroll
+                for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
+                {
+                    const uint32_t row = r + 32u * j < valid ? r + 32u * j : valid - 1u;
+                    off[j]             = row * ld * ES + ((slot ^ swzK(r)) * CHUNK);
+                }
+                step = 0u, stage = STAGE_KB;
+            }
+            else
+            {
+                const uint32_t r = tid >> 5, slot = tid & 31u;
+#pragma unroll
+                for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
+                {
+                    const uint32_t c = slot ^ swzMN(r + 8u * (j & 1u));
+                    off[j]           = r * ld * ES + (c * (CHUNK / ES) < valid ? c : 0u) * CHUNK;
+                }
+                step = 8u * ld * ES, stage = (uint64_t)TK * ld * ES;
+            }
+        };
+        laneOffsets(A_KCONTIG, p.lda, validM, gOffA, gStepA, gStageA);
+        laneOffsets(B_KCONTIG, p.ldb, validN, gOffB, gStepB, gStageB);
         const char* gA = p.a + (A_KCONTIG ? (uint64_t)tm * TILE_M * p.lda * ES : (uint64_t)tm * TILE_M * ES);
         const char* gB = p.b + (B_KCONTIG ? (uint64_t)tn * TILE_N * p.ldb * ES : (uint64_t)tn * TILE_N * ES);
 
@@ -353,9 +365,9 @@ namespace
             const uint32_t j = x >> 1;
             char*          dst = stage + (j * THREADS + wave * 64u) * CHUNK;
             if(x & 1u)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(srcB, (lp)(dst + OPER_BYTES), 16, gOffB[j & 1u], j * gStepB, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(srcB, (lp)(dst + OPER_BYTES), 16, gOffB[j], j * gStepB, 0, 0);
             else
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(srcA, (lp)dst, 16, gOffA[j & 1u], j * gStepA, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(srcA, (lp)dst, 16, gOffA[j], j * gStepA, 0, 0);
         };
         auto issueGlobal = [&](uint32_t kt, char* stage) {
             const __amdgpu_buffer_rsrc_t srcA = stageRsrc(gA + kt * gStageA), srcB = stageRsrc(gB + kt * gStageB);
@@ -520,8 +532,19 @@ namespace
 
         // global -> LDS: chunk L = j * 256 + tid of an operand tile sits at LDS byte 16 L (row L / 8)
         const uint32_t gr = tid >> 3, gslot = tid & 7u;
-        const uint32_t gOffA = gr * p.lda + ((gslot ^ swzK(gr)) * CHUNK), gStepA = 32u * p.lda;
-        const uint32_t gOffB = gr * p.ldb + ((gslot ^ swzK(gr)) * CHUNK), gStepB = 32u * p.ldb;
+        // one lane offset per load: rows beyond an edge tile's valid part read its last valid row instead
+        // (what lands in LDS for them only feeds elements of D that are never stored)
+        uint32_t       gOffA[LOADS_PER_OPER], gOffB[LOADS_PER_OPER];
+        const uint32_t validM = p.m - tm * TILE_M < TILE_M ? p.m - tm * TILE_M : TILE_M;
+        const uint32_t validN = p.n - tn * TILE_N < TILE_N ? p.n - tn * TILE_N : TILE_N;
+#pragma unroll
+        for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
+        {
+            const uint32_t ra = gr + 32u * j < validM ? gr + 32u * j : validM - 1u;
+            const uint32_t rb = gr + 32u * j < validN ? gr + 32u * j : validN - 1u;
+            gOffA[j]          = ra * p.lda + ((gslot ^ swzK(gr)) * CHUNK);
+            gOffB[j]          = rb * p.ldb + ((gslot ^ swzK(gr)) * CHUNK);
+        }
         const uint32_t numStages = p.k / STAGE_KB;
         const uint32_t dmaDst    = ldsBase + wave * 64u * CHUNK; // + buffer + j * 4 KiB
         auto           uniform64 = [](const char* ptr) {
@@ -539,11 +562,11 @@ namespace
         auto stageAddr = [&](uint64_t panel, uint32_t stage) { // clamped to the last stage
             return panel + (uint64_t)(stage < numStages ? stage : numStages - 1u) * STAGE_KB;
         };
-        auto issueHalf = [&](uint64_t addr, uint32_t gOff, uint32_t gStep, uint32_t at) {
+        auto issueHalf = [&](uint64_t addr, const uint32_t (&gOff)[LOADS_PER_OPER], uint32_t at) {
             const i32x4 rsrc = rsrcAt(addr);
 #pragma unroll
             for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
-                loadToLds(rsrc, gOff, j * gStep, dmaDst + at + j * THREADS * CHUNK);
+                loadToLds(rsrc, gOff[j], 0u, dmaDst + at + j * THREADS * CHUNK);
         };
 
         // LDS -> registers: block i rows are 16 i + lane % 16; K step s reads chunk 4 s + lane / 16
@@ -618,20 +641,20 @@ namespace
                     if(q == 2u)
                     {
                         if(x < 8u)
-                            loadToLds(rsrcA, gOffA, x * gStepA, dmaDst + aCur + x * THREADS * CHUNK);
+                            loadToLds(rsrcA, gOffA[x], 0u, dmaDst + aCur + x * THREADS * CHUNK);
                         else
-                            loadToLds(rsrcB, gOffB, (x - 8u) * gStepB, dmaDst + bCur + (x - 8u) * THREADS * CHUNK);
+                            loadToLds(rsrcB, gOffB[x - 8u], 0u, dmaDst + bCur + (x - 8u) * THREADS * CHUNK);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
         };
 
         // prologue: stages 0 and 1 and the B half of stage 2 requested; stage 0 published
-        issueHalf(stageAddr(gA, 0u), gOffA, gStepA, A_AT[0]);
-        issueHalf(stageAddr(gB, 0u), gOffB, gStepB, B_AT[0]);
-        issueHalf(stageAddr(gA, 1u), gOffA, gStepA, A_AT[1]);
-        issueHalf(stageAddr(gB, 1u), gOffB, gStepB, B_AT[1]);
-        issueHalf(stageAddr(gB, 2u), gOffB, gStepB, B_AT[2]);
+        issueHalf(stageAddr(gA, 0u), gOffA, A_AT[0]);
+        issueHalf(stageAddr(gB, 0u), gOffB, B_AT[0]);
+        issueHalf(stageAddr(gA, 1u), gOffA, A_AT[1]);
+        issueHalf(stageAddr(gB, 1u), gOffB, B_AT[1]);
+        issueHalf(stageAddr(gB, 2u), gOffB, B_AT[2]);
         refillA = stageAddr(gA, 2u), refillB = stageAddr(gB, 3u);
         waitVmcnt<24>();
         ldsBarrier();
@@ -716,8 +739,19 @@ namespace
 
         // global -> LDS: chunk L = j * 256 + tid of an operand tile sits at LDS byte 16 L (row L / 8)
         const uint32_t gr = tid >> 3, gslot = tid & 7u;
-        const uint32_t gOffA = gr * p.lda + ((gslot ^ swzK(gr)) * CHUNK), gStepA = 32u * p.lda;
-        const uint32_t gOffB = gr * p.ldb + ((gslot ^ swzK(gr)) * CHUNK), gStepB = 32u * p.ldb;
+        // one lane offset per load: rows beyond an edge tile's valid part read its last valid row instead
+        // (what lands in LDS for them only feeds elements of D that are never stored)
+        uint32_t       gOffA[LOADS_PER_OPER], gOffB[LOADS_PER_OPER];
+        const uint32_t validM = p.m - tm * TILE_M < TILE_M ? p.m - tm * TILE_M : TILE_M;
+        const uint32_t validN = p.n - tn * TILE_N < TILE_N ? p.n - tn * TILE_N : TILE_N;
+#pragma unroll
+        for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
+        {
+            const uint32_t ra = gr + 32u * j < validM ? gr + 32u * j : validM - 1u;
+            const uint32_t rb = gr + 32u * j < validN ? gr + 32u * j : validN - 1u;
+            gOffA[j]          = ra * p.lda + ((gslot ^ swzK(gr)) * CHUNK);
+            gOffB[j]          = rb * p.ldb + ((gslot ^ swzK(gr)) * CHUNK);
+        }
         const uint32_t numStages = p.k / STAGE_KB;
         const uint32_t dmaDst    = ldsBase + wave * 64u * CHUNK;
         auto           uniform64 = [](const char* ptr) {
@@ -735,11 +769,11 @@ namespace
         auto stageAddr = [&](uint64_t panel, uint32_t stage) {
             return panel + (uint64_t)(stage < numStages ? stage : numStages - 1u) * STAGE_KB;
         };
-        auto issueHalf = [&](uint64_t addr, uint32_t gOff, uint32_t gStep, uint32_t at) {
+        auto issueHalf = [&](uint64_t addr, const uint32_t (&gOff)[LOADS_PER_OPER], uint32_t at) {
             const i32x4 rsrc = rsrcAt(addr);
 #pragma unroll
             for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
-                loadToLds(rsrc, gOff, j * gStep, dmaDst + at + j * THREADS * CHUNK);
+                loadToLds(rsrc, gOff[j], 0u, dmaDst + at + j * THREADS * CHUNK);
         };
 
         // LDS -> registers: block rows are 16 i + lane % 16; piece q of a block is chunk 4 q + lane / 16
@@ -805,7 +839,7 @@ namespace
                 if(!(n & 1u))
                     readPiece(aLo, aNxt, rdA, 0, n >> 1);
                 else
-                    loadToLds(rsrcA, gOffA, (n >> 1) * gStepA, dmaDst + aCur + (n >> 1) * THREADS * CHUNK);
+                    loadToLds(rsrcA, gOffA[n >> 1], 0u, dmaDst + aCur + (n >> 1) * THREADS * CHUNK);
                 __builtin_amdgcn_sched_barrier(0);
             }
             // Q4: A[4..7] x B[0..3]; next B[0..3] arrives in the registers B[4..7] has left; B refill
@@ -816,17 +850,17 @@ namespace
                 if(!(n & 1u))
                     readPiece(bHi, bNxt, rdB, 0, n >> 1);
                 else
-                    loadToLds(rsrcB, gOffB, (n >> 1) * gStepB, dmaDst + bCur + (n >> 1) * THREADS * CHUNK);
+                    loadToLds(rsrcB, gOffB[n >> 1], 0u, dmaDst + bCur + (n >> 1) * THREADS * CHUNK);
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
 
         // prologue: stages 0 and 1 and the B half of stage 2 requested; stage 0 published
-        issueHalf(stageAddr(gA, 0u), gOffA, gStepA, A_AT[0]);
-        issueHalf(stageAddr(gB, 0u), gOffB, gStepB, B_AT[0]);
-        issueHalf(stageAddr(gA, 1u), gOffA, gStepA, A_AT[1]);
-        issueHalf(stageAddr(gB, 1u), gOffB, gStepB, B_AT[1]);
-        issueHalf(stageAddr(gB, 2u), gOffB, gStepB, B_AT[2]);
+        issueHalf(stageAddr(gA, 0u), gOffA, A_AT[0]);
+        issueHalf(stageAddr(gB, 0u), gOffB, B_AT[0]);
+        issueHalf(stageAddr(gA, 1u), gOffA, A_AT[1]);
+        issueHalf(stageAddr(gB, 1u), gOffB, B_AT[1]);
+        issueHalf(stageAddr(gB, 2u), gOffB, B_AT[2]);
         refillA = stageAddr(gA, 2u), refillB = stageAddr(gB, 3u);
         waitVmcnt<24>();
         ldsBarrier();
@@ -913,8 +947,8 @@ namespace r355
         // the two-buffer kernel consumes K stages in pairs; the five-buffer 8-bit kernel takes any count
         const bool     fiveBuffers = es == 1;
         const uint32_t kGranule    = fiveBuffers ? tk : 2 * tk;
-        if(g.m % TILE_M || g.n % TILE_N || g.k % kGranule || g.k == 0)
-            return fail(R355_ERR_BAD_SIZE, "tiled gemm: m=%u n=%u must be multiples of 256 and k=%u of %u", g.m, g.n, g.k, kGranule);
+        if(g.m % 16 || g.n % 16 || g.m == 0 || g.n == 0 || g.k % kGranule || g.k == 0)
+            return fail(R355_ERR_BAD_SIZE, "tiled gemm: m=%u n=%u must be multiples of 16 and k=%u of %u", g.m, g.n, g.k, kGranule);
         if(!aligned(g.a, 16) || !aligned(g.b, 16) || (g.lda * es) % 16 || (g.ldb * es) % 16 || !aligned(g.d, 16)
            || (g.ldd * os) % 16 || (g.beta != 0.0f && (!aligned(g.c, 16) || (g.ldc * os) % 16)))
             return fail(R355_ERR_MISALIGNED, "tiled gemm: pointers and leading dimensions of A, B, C, D must keep 16-byte alignment");
@@ -924,7 +958,7 @@ namespace r355
             plan->macro_tile_m = TILE_M;
             plan->macro_tile_n = TILE_N;
             plan->macro_tile_k = tk;
-            plan->grid_x       = (((g.m / TILE_M) * (g.n / TILE_N) + 7u) / 8u) * 8u;
+            plan->grid_x       = ((((g.m + TILE_M - 1) / TILE_M) * ((g.n + TILE_N - 1) / TILE_N) + 7u) / 8u) * 8u;
             plan->grid_y       = 1;
             plan->block_x      = THREADS;
             plan->block_y      = 1;
@@ -959,7 +993,7 @@ namespace r355
             p.lda = g.ldb, p.ldb = g.lda;
             aK = g.layout_b == R355_COL_MAJOR, bK = g.layout_a == R355_ROW_MAJOR;
         }
-        p.tilesM = p.m / TILE_M, p.tilesN = p.n / TILE_N;
+        p.tilesM = (p.m + TILE_M - 1) / TILE_M, p.tilesN = (p.n + TILE_N - 1) / TILE_N;
         switch(g.in_type)
         {
         case R355_F16:

@@ -161,6 +161,52 @@ def test_tiled_kernel_8bit(in_t, out_t, ldl):
     _check(in_t, out_t, got, want)
 
 
+RAGGED_SHAPES = [(272, 304, 256), (16, 528, 128), (1008, 16, 384), (496, 752, 128)]
+
+
+@pytest.mark.parametrize("in_t,out_t", [(O.F16, O.F16), (O.BF16, O.F32)])
+@pytest.mark.parametrize("la,lb", TILED_LAYOUTS_16)
+@pytest.mark.parametrize("m,n,k", RAGGED_SHAPES)
+def test_tiled_kernel_16bit_edge_tiles(in_t, out_t, la, lb, m, n, k):
+    # m and n multiples of 16 that do not fill 256 x 256 tiles: edge tiles read clamped rows / chunks
+    # and store only what lies inside D; beta != 0 exercises the guarded C loads as well
+    a, b, c = _inputs(in_t, out_t, m, n, k, seed=70 + m)
+    for alpha, beta in ((1.0, 0.0), (2.0, 2.0)):
+        cc = None if beta == 0.0 else c
+        want = O.gemm(in_t, out_t, la, lb, O.ROW, O.ROW, m, n, k, a, b, cc, alpha, beta)
+        got = _run(in_t, out_t, la, lb, O.ROW, O.ROW, m, n, k, a, b, cc, alpha, beta, R.KERNEL_TILED)
+        w32 = None
+        if out_t != O.F32:
+            c32 = None if cc is None else O.storage_to_f32(cc, out_t)
+            w32 = O.gemm(in_t, O.F32, la, lb, O.ROW, O.ROW, m, n, k, a, b, c32, alpha, beta)
+        _check(in_t, out_t, got, want, w32)
+
+
+@pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32)])
+@pytest.mark.parametrize("ldl", [O.ROW, O.COL])
+@pytest.mark.parametrize("m,n,k", RAGGED_SHAPES)
+def test_tiled_kernel_8bit_edge_tiles(in_t, out_t, ldl, m, n, k):
+    a, b, c = _inputs(in_t, out_t, m, n, k, seed=80 + n)
+    for alpha, beta in ((1.0, 0.0), (1.0, 1.0)):
+        cc = None if beta == 0.0 else c
+        want = O.gemm(in_t, out_t, O.ROW, O.COL, ldl, ldl, m, n, k, a, b, cc, alpha, beta)
+        got = _run(in_t, out_t, O.ROW, O.COL, ldl, ldl, m, n, k, a, b, cc, alpha, beta, R.KERNEL_TILED)
+        _check(in_t, out_t, got, want)
+
+
+def test_edge_tiles_leave_neighbouring_memory_untouched():
+    # D with a padded leading dimension: the columns between n and ldd must keep their prefill
+    m, n, k, ldd = 272, 304, 128, 320
+    a, b, _ = _inputs(O.F16, O.F32, m, n, k, seed=91)
+    da, db = to_device(a), to_device(b)
+    dd = device_filled(m * ldd, np.float32, 0xFF)
+    R.gemm(R.F16, R.F32, m, n, k, da, db, None, dd, 1.0, 0.0, O.ROW, O.COL, O.ROW, O.ROW, ldd=ldd, kernel=R.KERNEL_TILED)
+    got = to_host(dd, np.float32).reshape(m, ldd)
+    want = O.gemm(O.F16, O.F32, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0).reshape(m, n)
+    _check(O.F16, O.F32, np.ascontiguousarray(got[:, :n]).ravel(), want.ravel())
+    assert np.all(np.ascontiguousarray(got[:, n:]).view(np.uint32) == 0xFFFFFFFF)
+
+
 @pytest.mark.parametrize("in_t,out_t", [(O.F16, O.F32), (O.BF16, O.BF16)])
 @pytest.mark.parametrize("la,lb", [(O.COL, O.ROW), (O.ROW, O.COL)])
 @pytest.mark.parametrize("k", [128, 256, 640])
