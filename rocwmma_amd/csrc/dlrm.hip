@@ -168,7 +168,7 @@ namespace
     }
 
     // f32 variant.  An f32 sample is 13.8 KB, so only a few fit in LDS per CU and the matrix core
-    // (v_mfma_f32_32x32x2f32, 64 instructions per sample) is busy almost half of the time: the loads
+    // (v_mfma_f32_16x16x4_f32, 96 instructions per sample) is busy a good third of the time: the loads
     // of a wave's next sample are therefore issued before the current sample is computed, and every
     // wave walks F32_PER_WAVE consecutive samples, writing each result row from its own LDS image
     // with coalesced 4-byte stores (a sample's output row is only 4-byte aligned).
@@ -224,33 +224,45 @@ namespace
             __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_wave_barrier();
 
-            // two independent accumulator chains (even / odd k pairs) keep the matrix core pipelined
-            f32x16         acc0  = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-            f32x16         acc1  = acc0;
-            const bool     valid = (lane & 31u) < m;
-            const uint32_t row   = valid ? (lane & 31u) : 0u;
+            // v_mfma_f32_16x16x4_f32 on the three 16 x 16 blocks of the Gram matrix that hold its lower
+            // triangle (rows < 16 x rows < 16, rows >= 16 x rows < 16, rows >= 16 x rows >= 16): a quarter
+            // fewer matrix-core cycles than the full 32 x 32 product, and three independent accumulator
+            // chains keep the pipeline full.  Lane l feeds row l % 16 (+ 16) at k = 4 s + l / 16.
+            using f32x4acc = float __attribute__((ext_vector_type(4)));
+            f32x4acc       accLL = {0, 0, 0, 0}, accHL = accLL, accHH = accLL;
+            const uint32_t r16 = lane & 15u, kq = lane >> 4;
+            const bool     validLo = r16 < m, validHi = 16u + r16 < m;
+            const uint32_t rowLo = validLo ? r16 : 0u, rowHi = validHi ? 16u + r16 : 0u;
 #pragma unroll 8
             for(uint32_t s = 0; s < K / 4; ++s)
             {
-                // lane half h holds k = 4 s + h and 4 s + 2 + h: one 16-byte chunk feeds two instructions
-                const char* src4 = xw + (row * ROW_CHUNKS + (s ^ (row & SWZ))) * 16u + (lane >> 5) * 4u;
-                float       x0   = *reinterpret_cast<const float*>(src4);
-                float       x1   = *reinterpret_cast<const float*>(src4 + 8u);
-                if(!valid)
-                    x0 = 0.0f, x1 = 0.0f;
-                acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(x0, x0, acc0, 0, 0, 0);
-                acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(x1, x1, acc1, 0, 0, 0);
+                float xl = *reinterpret_cast<const float*>(xw + (rowLo * ROW_CHUNKS + (s ^ (rowLo & SWZ))) * 16u + kq * 4u);
+                float xh = *reinterpret_cast<const float*>(xw + (rowHi * ROW_CHUNKS + (s ^ (rowHi & SWZ))) * 16u + kq * 4u);
+                if(!validLo)
+                    xl = 0.0f;
+                if(!validHi)
+                    xh = 0.0f;
+                accLL = __builtin_amdgcn_mfma_f32_16x16x4f32(xl, xl, accLL, 0, 0, 0);
+                accHL = __builtin_amdgcn_mfma_f32_16x16x4f32(xh, xl, accHL, 0, 0, 0);
+                accHH = __builtin_amdgcn_mfma_f32_16x16x4f32(xh, xh, accHH, 0, 0, 0);
             }
 
             for(uint32_t e = lane; e < K; e += 64)
                 o[e] = reinterpret_cast<const float*>(xw)[e]; // row 0 is stored unswizzled
-            const uint32_t j = lane & 31u;
+            // a 16 x 16 result block: lane holds rows 4 (lane / 16) + e, column lane % 16
 #pragma unroll
-            for(uint32_t r = 0; r < 16; ++r)
+            for(uint32_t e = 0; e < 4; ++e)
             {
-                const uint32_t i = 8u * (r >> 2) + 4u * (lane >> 5) + (r & 3u);
+                const uint32_t i = 4u * kq + e, j = r16;
                 if(j < i && i < m)
-                    o[K + i * (i - 1u) / 2u + j] = acc0[r] + acc1[r];
+                    o[K + i * (i - 1u) / 2u + j] = accLL[e];
+                const uint32_t ih = 16u + i;
+                if(ih < m)
+                {
+                    o[K + ih * (ih - 1u) / 2u + j] = accHL[e];
+                    if(j < i)
+                        o[K + ih * (ih - 1u) / 2u + 16u + j] = accHH[e];
+                }
             }
             __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_wave_barrier();
