@@ -161,6 +161,23 @@ def test_tiled_kernel_8bit(in_t, out_t, ldl):
     _check(in_t, out_t, got, want)
 
 
+# the sizes the reference's GEMM suites validate (test/gemm/gemm_common_test_params.hpp:336-348) with its
+# alpha = beta = 2 (:363-373)
+REFERENCE_VALIDATED_SIZES = [(64, 64, 1024), (32, 64, 1024), (64, 32, 1024), (256, 256, 1024), (2048, 64, 1024),
+                             (64, 2048, 1024), (512, 512, 512)]
+
+
+@pytest.mark.parametrize("m,n,k", REFERENCE_VALIDATED_SIZES)
+@pytest.mark.parametrize("kernel", ["auto", "tiled"])
+def test_reference_validated_problem_sizes(m, n, k, kernel):
+    sel = R.KERNEL_AUTO if kernel == "auto" else R.KERNEL_TILED
+    for in_t, out_t in ((O.F16, O.F32), (O.I8, O.I32)):
+        a, b, c = _inputs(in_t, out_t, m, n, k, seed=5)
+        want = O.gemm(in_t, out_t, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, 2.0)
+        got = _run(in_t, out_t, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, 2.0, sel)
+        _check(in_t, out_t, got, want)
+
+
 RAGGED_SHAPES = [(272, 304, 256), (16, 528, 128), (1008, 16, 384), (496, 752, 128)]
 
 
