@@ -127,8 +127,9 @@ int r355_dlrm_fwd_timed(int32_t dtype, const void* in, void* out, uint32_t m, ui
 
 /*
  * DLRM dot-interaction backward.  upstream: [batch][k + m(m-1)/2]; mlp_grad: [batch][k];
- * in_grad: [batch][m][k].  Replaces: dlrmDotBwd + trilReconstruct launches,
- * test/dlrm/device/dlrm_dot_bwd.hpp:35-176.
+ * in_grad: [batch][m][k].  dtype R355_F16, R355_BF16 (all four pointers 16-byte aligned) or R355_F32
+ * (k <= 128; in / in_grad 16-byte, upstream / mlp_grad 4-byte aligned).  Replaces: dlrmDotBwd +
+ * trilReconstruct launches, test/dlrm/device/dlrm_dot_bwd.hpp:35-176.
  */
 int r355_dlrm_bwd(int32_t dtype, const void* in, const void* upstream, void* mlp_grad, void* in_grad,
                   uint32_t m, uint32_t k, uint32_t batch, void* stream);

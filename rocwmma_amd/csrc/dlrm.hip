@@ -479,6 +479,160 @@ namespace
         }
     }
 
+    // f32 backward.  grad (m x k) = S X with S = T + T^T from the upstream triangle, on
+    // v_mfma_f32_16x16x4_f32: A operand = a 16 x 4 piece of S (lane l: row l % 16, column l / 16), B
+    // operand = a 4 x 16 piece of X (lane l: row l / 16, column l % 16), 2 x (k / 16) result blocks, 8
+    // steps over the 32 (zero-padded) rows of X.  Every wave walks F32_PER_WAVE consecutive samples with
+    // the loads of the next one in flight.  Per sample: X goes to an LDS image whose 64-byte column
+    // groups are XOR-swizzled with the row (four consecutive rows of one column group land in
+    // different banks), the upstream row to a second image from which each lane gathers its 16 values
+    // of S; the gradient is written over X and leaves with 128-bit nontemporal stores; the first k
+    // upstream values are the bottom-MLP gradient (test/reference_impl.hpp:121-179).
+    template <uint32_t K>
+    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2))) dlrmBwdF32Kernel(const float* __restrict__ in, const float* __restrict__ upstream,
+                                                               float* __restrict__ mlpGrad, float* __restrict__ inGrad,
+                                                               uint32_t m, uint32_t batch)
+    {
+        constexpr uint32_t ROW_CHUNKS = K / 4; // 16-byte chunks per row
+        constexpr uint32_t ROWB       = K * 4;
+        constexpr uint32_t MAX_UP     = K + MAX_M * (MAX_M - 1) / 2;
+        constexpr uint32_t X_CHUNKS   = (MAX_M * ROW_CHUNKS + 63u) / 64u; // per lane
+        constexpr uint32_t UP_WORDS   = (MAX_UP + 63u) / 64u; // per lane
+        constexpr uint32_t CBLOCKS    = K / 16; // 64-byte column groups per row
+        constexpr uint32_t SWZ        = CBLOCKS >= 4 ? 3u : CBLOCKS - 1u;
+        using f32x4                   = float __attribute__((ext_vector_type(4)));
+
+        __shared__ __attribute__((aligned(16))) char  xLds[WAVES][MAX_M * ROWB];
+        __shared__ __attribute__((aligned(16))) float upLds[WAVES][MAX_UP];
+
+        const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+        const uint32_t upStride = K + m * (m - 1) / 2;
+        const uint32_t inChunks = m * ROW_CHUNKS;
+        const uint32_t first    = (blockIdx.x * WAVES + wave) * F32_PER_WAVE;
+        char*          xw       = xLds[wave];
+        float*         uw       = upLds[wave];
+        const uint32_t r16 = lane & 15u, q4 = lane >> 4;
+
+        // byte address of 16-byte chunk c (0 .. ROW_CHUNKS) of row `row` in the swizzled image
+        auto chunkAt = [&](uint32_t row, uint32_t c) { return row * ROWB + ((((c >> 2) ^ (row & SWZ)) << 2) + (c & 3u)) * 16u; };
+
+        // rows >= m of the image stay zero for every sample
+        for(uint32_t c = inChunks + lane; c < MAX_M * ROW_CHUNKS; c += 64u)
+            *reinterpret_cast<f32x4*>(xw + chunkAt(c / ROW_CHUNKS, c % ROW_CHUNKS)) = f32x4{0, 0, 0, 0};
+
+        // where lane l finds S(i, j) in the upstream image: the strict lower triangle is stored row by
+        // row behind the first k values; the diagonal is zero (recomputed per sample: registers are
+        // scarcer than integer instructions here)
+        auto sAt = [&](uint32_t i, uint32_t j) -> float {
+            const uint32_t hi = i > j ? i : j, lo = i > j ? j : i;
+            return (i != j && hi < m) ? uw[K + hi * (hi - 1u) / 2u + lo] : 0.0f;
+        };
+
+        // one register stash: a sample's loads are requested while the previous sample is computed and
+        // unloaded into LDS before the next request reuses the registers
+        f32x4 xs[X_CHUNKS];
+        float us[UP_WORDS];
+        auto  request = [&](uint32_t b) {
+            if(b < batch)
+            {
+                const char*  src = reinterpret_cast<const char*>(in) + (uint64_t)b * m * ROWB;
+                const float* up  = upstream + (uint64_t)b * upStride;
+#pragma unroll
+                for(uint32_t j = 0; j < X_CHUNKS; ++j)
+                    if(j * 64u + lane < inChunks)
+                        xs[j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src + (j * 64u + lane) * 16u));
+#pragma unroll
+                for(uint32_t j = 0; j < UP_WORDS; ++j)
+                    if(j * 64u + lane < upStride)
+                        us[j] = __builtin_nontemporal_load(up + j * 64u + lane);
+            }
+        };
+
+        request(first);
+#pragma unroll 1
+        for(uint32_t it = 0; it < F32_PER_WAVE; ++it)
+        {
+            const uint32_t b = first + it;
+            if(b >= batch)
+                break;
+#pragma unroll
+            for(uint32_t j = 0; j < X_CHUNKS; ++j)
+            {
+                const uint32_t c = j * 64u + lane;
+                if(c < inChunks)
+                    *reinterpret_cast<f32x4*>(xw + chunkAt(c / ROW_CHUNKS, c % ROW_CHUNKS)) = xs[j];
+            }
+#pragma unroll
+            for(uint32_t j = 0; j < UP_WORDS; ++j)
+                if(j * 64u + lane < upStride)
+                    uw[j * 64u + lane] = us[j];
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_wave_barrier();
+            if(it + 1u < F32_PER_WAVE)
+                request(b + 1u);
+
+            // bottom-MLP gradient: the first k upstream values
+            float* mg = mlpGrad + (uint64_t)b * K;
+            for(uint32_t e = lane; e < K; e += 64u)
+                __builtin_nontemporal_store(uw[e], mg + e);
+
+            float sv[2][8];
+#pragma unroll
+            for(uint32_t ib = 0; ib < 2; ++ib)
+#pragma unroll
+                for(uint32_t js = 0; js < 8; ++js)
+                    sv[ib][js] = sAt(16u * ib + r16, 4u * js + q4);
+
+            f32x4 acc[2][CBLOCKS];
+#pragma unroll
+            for(uint32_t ib = 0; ib < 2; ++ib)
+#pragma unroll
+                for(uint32_t cb = 0; cb < CBLOCKS; ++cb)
+                    acc[ib][cb] = f32x4{0, 0, 0, 0};
+#pragma unroll
+            for(uint32_t js = 0; js < 8; ++js)
+            {
+                const uint32_t row = 4u * js + q4;
+#pragma unroll
+                for(uint32_t cb = 0; cb < CBLOCKS; ++cb)
+                {
+                    // X(row, 16 cb + l % 16): 64-byte column group cb, swizzled with the row
+                    const float xv = *reinterpret_cast<const float*>(xw + row * ROWB + ((cb ^ (row & SWZ)) << 6) + r16 * 4u);
+                    acc[0][cb]     = __builtin_amdgcn_mfma_f32_16x16x4f32(sv[0][js], xv, acc[0][cb], 0, 0, 0);
+                    acc[1][cb]     = __builtin_amdgcn_mfma_f32_16x16x4f32(sv[1][js], xv, acc[1][cb], 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0); // keeps the LDS reads of later steps from piling up in registers
+            }
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_wave_barrier(); // every lane has read X: the gradient goes over it
+            // result block (ib, cb): lane holds rows 16 ib + 4 (l / 16) + e, column 16 cb + l % 16
+#pragma unroll
+            for(uint32_t ib = 0; ib < 2; ++ib)
+#pragma unroll
+                for(uint32_t cb = 0; cb < CBLOCKS; ++cb)
+#pragma unroll
+                    for(uint32_t e = 0; e < 4; ++e)
+                    {
+                        const uint32_t row = 16u * ib + 4u * q4 + e;
+                        if(row < m)
+                            *reinterpret_cast<float*>(xw + row * ROWB + ((cb ^ (row & SWZ)) << 6) + r16 * 4u) = acc[ib][cb][e];
+                    }
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_wave_barrier();
+            char* dst = reinterpret_cast<char*>(inGrad) + (uint64_t)b * m * ROWB;
+#pragma unroll
+            for(uint32_t j = 0; j < X_CHUNKS; ++j)
+            {
+                const uint32_t c = j * 64u + lane;
+                if(c < inChunks)
+                    __builtin_nontemporal_store(*reinterpret_cast<const f32x4*>(xw + chunkAt(c / ROW_CHUNKS, c % ROW_CHUNKS)),
+                                                reinterpret_cast<f32x4*>(dst + c * 16u));
+            }
+            __builtin_amdgcn_s_waitcnt(0xC07F); // the images are rewritten by the next sample
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
+
     int checkArgs(const char* what, int32_t dtype, const void* in, const void* out, uint32_t m, uint32_t k, uint32_t batch,
                   bool allowF32)
     {
@@ -564,11 +718,30 @@ extern "C" int r355_dlrm_fwd(int32_t dtype, const void* in, void* out, uint32_t 
 extern "C" int r355_dlrm_bwd(int32_t dtype, const void* in, const void* upstream, void* mlp_grad, void* in_grad,
                              uint32_t m, uint32_t k, uint32_t batch, void* stream)
 {
-    int rc = checkArgs("dlrm_bwd", dtype, in, in_grad, m, k, batch, false);
+    int rc = checkArgs("dlrm_bwd", dtype, in, in_grad, m, k, batch, true);
     if(rc != R355_OK)
         return rc;
     if(!upstream || !mlp_grad)
         return r355::fail(R355_ERR_BAD_ARG, "dlrm_bwd: null pointer");
+    if(dtype == R355_F32)
+    {
+        if(!r355::aligned(upstream, 4) || !r355::aligned(mlp_grad, 4))
+            return r355::fail(R355_ERR_MISALIGNED, "dlrm_bwd: upstream and mlp_grad must be 4-byte aligned");
+        const uint32_t perWg = WAVES * F32_PER_WAVE;
+        const dim3     grid32((batch + perWg - 1) / perWg), block32(THREADS);
+        hipStream_t    s32 = static_cast<hipStream_t>(stream);
+        auto*          fi  = static_cast<const float*>(in);
+        auto*          fu  = static_cast<const float*>(upstream);
+        auto*          fm  = static_cast<float*>(mlp_grad);
+        auto*          fg  = static_cast<float*>(in_grad);
+        switch(k)
+        {
+        case 32: hipLaunchKernelGGL(dlrmBwdF32Kernel<32>, grid32, block32, 0, s32, fi, fu, fm, fg, m, batch); break;
+        case 64: hipLaunchKernelGGL(dlrmBwdF32Kernel<64>, grid32, block32, 0, s32, fi, fu, fm, fg, m, batch); break;
+        default: hipLaunchKernelGGL(dlrmBwdF32Kernel<128>, grid32, block32, 0, s32, fi, fu, fm, fg, m, batch); break;
+        }
+        return r355::checkLaunch("dlrm_bwd");
+    }
     if(!r355::aligned(upstream, 16) || !r355::aligned(mlp_grad, 16))
         return r355::fail(R355_ERR_MISALIGNED, "dlrm_bwd: upstream and mlp_grad must be 16-byte aligned");
     const dim3  grid((batch + SAMPLES_PER_WG - 1) / SAMPLES_PER_WG), block(THREADS);

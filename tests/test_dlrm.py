@@ -147,6 +147,74 @@ def test_bwd_reference_fixture(suffix):
     assert ok, mx
 
 
+def _exact_bwd_f32(x, up, m, k, batch):
+    """float64 gradient of the f32 inputs: S X with S = T + T^T from the upstream triangle."""
+    X = x.reshape(batch, m, k).astype(np.float64)
+    U = up.reshape(batch, k + m * (m - 1) // 2).astype(np.float64)
+    S = np.zeros((batch, m, m))
+    ii, jj = np.tril_indices(m, -1)
+    S[:, ii, jj] = U[:, k:]
+    S = S + S.transpose(0, 2, 1)
+    return S @ X
+
+
+def _check_bwd_f32(got, want_oracle, x, up, m, k, batch):
+    # same bar as the f32 forward: within F32_TOL_EPS of the oracle, and no further from the float64
+    # value than 1.5 x the sequential-f32 oracle's own distance from it
+    ok, mx = O.compare(O.F32, got, want_oracle, F32_TOL_EPS)
+    assert ok, mx
+    exact = _exact_bwd_f32(x, up, m, k, batch).ravel()
+    err_gpu = np.max(np.abs(got.astype(np.float64) - exact) / (np.abs(exact) + 1.0))
+    err_orc = np.max(np.abs(want_oracle.astype(np.float64) - exact) / (np.abs(exact) + 1.0))
+    assert err_gpu <= 1.5 * err_orc + 1e-7, (err_gpu, err_orc)
+
+
+def test_bwd_f32_reference_fixture():
+    x = np.fromfile(os.path.join(GOLD, "input_fp32"), dtype=np.float32)
+    up = np.fromfile(os.path.join(GOLD, "input_grad_fp32"), dtype=np.float32)
+    want = np.fromfile(os.path.join(GOLD, "output_input_grad_fp32"), dtype=np.float32)
+    want_mlp = np.fromfile(os.path.join(GOLD, "output_mlp_input_grad_fp32"), dtype=np.float32)
+    dx, dup = to_device(x), to_device(up)
+    dmlp, dgrad = device_filled(64 * 128, np.float32), device_filled(64 * 27 * 128, np.float32)
+    R.dlrm_bwd(R.F32, dx, dup, dmlp, dgrad, 27, 128, 64)
+    assert np.array_equal(to_host(dmlp, np.float32), want_mlp)
+    got = to_host(dgrad, np.float32)
+    ok, mx = O.compare(O.F32, got, want, F32_TOL_EPS)
+    assert ok, mx
+    _, ograd = O.dlrm_bwd(O.F32, x, up, 27, 128, 64)
+    _check_bwd_f32(got, ograd.ravel(), x, up, 27, 128, 64)
+
+
+@pytest.mark.parametrize("m,k,batch", [(27, 128, 13), (32, 128, 40), (32, 32, 64), (2, 64, 5), (17, 128, 9), (28, 128, 1),
+                                       (29, 64, 33)])
+def test_bwd_f32_shapes_vs_oracle(m, k, batch):
+    stride = k + m * (m - 1) // 2
+    x = (O.normal(5, batch * m * k) * 0.5).astype(np.float32)
+    up = (O.normal(6, batch * stride) * 0.5).astype(np.float32)
+    want_mlp, want = O.dlrm_bwd(O.F32, x, up, m, k, batch)
+    dx, dup = to_device(x), to_device(up)
+    dmlp = device_filled(batch * k + 8, np.float32, 0xEE)
+    dgrad = device_filled(batch * m * k + 8, np.float32, 0xEE)
+    R.dlrm_bwd(R.F32, dx, dup, dmlp, dgrad, m, k, batch)
+    mlp, grad = to_host(dmlp, np.float32), to_host(dgrad, np.float32)
+    assert np.all(mlp[batch * k:].view(np.uint32) == 0xEEEEEEEE) and np.all(grad[batch * m * k:].view(np.uint32) == 0xEEEEEEEE)
+    assert np.array_equal(mlp[:batch * k], want_mlp.ravel())
+    _check_bwd_f32(grad[:batch * m * k], want.ravel(), x, up, m, k, batch)
+
+
+def test_bwd_f32_integer_inputs_exact():
+    m, k, batch = 27, 128, 24
+    stride = k + m * (m - 1) // 2
+    x = np.round(O.uniform_pm1(7, batch * m * k) * 3.0).astype(np.float32)
+    up = np.round(O.uniform_pm1(8, batch * stride) * 3.0).astype(np.float32)
+    want_mlp, want = O.dlrm_bwd(O.F32, x, up, m, k, batch)
+    dx, dup = to_device(x), to_device(up)
+    dmlp, dgrad = device_filled(batch * k, np.float32), device_filled(batch * m * k, np.float32)
+    R.dlrm_bwd(R.F32, dx, dup, dmlp, dgrad, m, k, batch)
+    assert np.array_equal(to_host(dmlp, np.float32), want_mlp.ravel())
+    assert np.array_equal(to_host(dgrad, np.float32), want.ravel())
+
+
 @pytest.mark.parametrize("dtype", [O.F16, O.BF16])
 @pytest.mark.parametrize("m,k,batch", [(27, 128, 13), (32, 128, 8), (32, 32, 64), (2, 64, 5), (17, 256, 9), (28, 128, 1),
                                        (29, 64, 17)])
