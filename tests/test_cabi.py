@@ -62,7 +62,8 @@ def test_query_selects_kernel_family_and_reports_launch_shape():
     (dict(in_type=R.F16, out_type=R.I32), -2),
     (dict(m=100, n=256), -3),
     (dict(k=24), -3),
-    (dict(kernel=R.KERNEL_TILED, m=128), -3),
+    (dict(kernel=R.KERNEL_TILED, m=120), -3),
+    (dict(kernel=R.KERNEL_TILED, k=192), -3),
     (dict(a=0x1002, layout_a=R.ROW_MAJOR), -4),
     (dict(lda=8), -1),
 ])
