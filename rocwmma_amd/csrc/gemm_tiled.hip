@@ -22,8 +22,8 @@
 //   LDS layout   16-byte chunks, XOR-swizzled inside each row so that both the
 //                row-contiguous writes and the MFMA-shaped reads are bank-conflict free
 //   LDS->regs    K-contiguous operands: one ds_read_b128 per 16-row operand block;
-//                M/N-contiguous 16-bit operands: two ds_read_b64_tr_b16 (transposing
-//                read) -- no element-wise reads anywhere; operands are fetched one K step
+//                M/N-contiguous operands: two ds_read_b64_tr_b16 / ds_read_b64_tr_b8 (transposing
+//                reads) -- no element-wise reads anywhere; operands are fetched one K step
 //                (64 matrix instructions; fp8: one quadrant, 16) ahead of their use
 //   schedule     the matrix instructions are inline assembly with the accumulator tied in place
 //                (the compiler's own selection leaves the 64 small accumulators untied and its
@@ -37,6 +37,8 @@
 // B col-major).  The MFMA operands are swapped so that each lane holds four consecutive
 // columns of a row of D; a col-major D is computed as the row-major D^T = B^T A^T.
 #include <hip/hip_runtime.h>
+
+#include <type_traits>
 
 #include "common.hpp"
 #include "lds_dma.hpp"
@@ -481,7 +483,7 @@ namespace
     }
 
     // ------------------------------------------------------------------------------------------
-    // 8-bit operands (int8, e4m3; A row-major, B col-major): five LDS buffers.  At twice the
+    // 8-bit operands (int8, e4m3), either orientation: five LDS buffers.  At twice the
     // matrix-instruction rate a K stage lasts about as long as a direct load takes to arrive, so a
     // two-buffer scheme leaves the memory pipe idle while a refill waits for its consumer.  Here LDS
     // holds two buffers for A and three for B (5 x 32 KiB = all 160 KiB): the B half of a stage is
@@ -497,20 +499,122 @@ namespace
     // later ds_read depends on and waits for vmcnt(0) every time, which would serialise exactly the
     // loads that are meant to stay in flight.  Issued this way the only vmcnt waits are the ones
     // written here.
+    //
+    // Operand tiles in LDS (32 KiB each), chunk L = j * 256 + tid of a tile at byte 16 L:
+    //   * K-contiguous (A row-major / B col-major): 256 rows x 128 B, chunk c of row r in slot
+    //     c ^ ((r >> 1) & 7); a lane reads 16 consecutive K bytes of its row with one ds_read_b128;
+    //   * M/N-contiguous (A col-major / B row-major): 128 k-rows x 256 B, chunk c of k-row q in slot
+    //     c ^ ((q & 7) | ((q >> 1) & 8)).  ds_read_b64_tr_b8 transposes inside each group of 16 lanes:
+    //     lane t supplies the address of 8 bytes, k-row t / 2 and byte columns 8 (t % 2) .. + 7, and
+    //     receives column t of the group's 8 k-rows -- 8 consecutive K values of one row of the operand,
+    //     which is what the matrix instructions want.  Two such reads make the 16 K bytes a
+    //     ds_read_b128 delivers for a K-contiguous operand.  The 32 lanes of one LDS pass touch 16
+    //     k-rows (8 each from two lane groups, 16 k-rows apart), hence bit 4 in the swizzle.
     using r355::ldsBarrier;
     using r355::loadToLds;
     using r355::waitVmcnt;
 
+    __device__ __forceinline__ uint32_t swzK8(uint32_t row)
+    {
+        return (row >> 1) & 7u;
+    }
+    __device__ __forceinline__ uint32_t swzMN8(uint32_t krow)
+    {
+        return (krow & 7u) | ((krow >> 1) & 8u);
+    }
+
+    // global -> LDS lane offsets of one operand: load j brings chunk j * 256 + tid.  Edge tiles (m or
+    // n not a multiple of 256) must not read outside the operand: a lane whose row (K-contiguous) or
+    // chunk (M/N-contiguous) lies beyond the matrix reads the last valid row / the first chunk instead;
+    // what lands in LDS for it only feeds elements of D that are never stored.  `step` is the uniform
+    // offset from one load to the next, `stage` the distance between K stages.
+    template <bool KCONTIG>
+    __device__ __forceinline__ void laneOffsets8(uint32_t tid, uint32_t ld, uint32_t valid, uint32_t (&off)[LOADS_PER_OPER],
+                                                 uint32_t& step, uint64_t& stage)
+    {
+        if constexpr(KCONTIG)
+        {
+            const uint32_t r = tid >> 3, slot = tid & 7u; // row 32 j + r
+#pragma unroll
+            for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
+            {
+                const uint32_t row = r + 32u * j < valid ? r + 32u * j : valid - 1u;
+                off[j]             = row * ld + ((slot ^ swzK8(r)) * CHUNK);
+            }
+            step = 0u, stage = STAGE_KB;
+        }
+        else
+        {
+            const uint32_t r = tid >> 4, slot = tid & 15u; // k-row 16 j + r: the swizzle alternates with j
+#pragma unroll
+            for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
+            {
+                const uint32_t c = slot ^ swzMN8(16u * j + r);
+                off[j]           = r * ld + (c * CHUNK < valid ? c : 0u) * CHUNK;
+            }
+            step = 16u * ld, stage = (uint64_t)STAGE_KB * ld;
+        }
+    }
+
+    // LDS -> register lane offsets of one operand for the wave whose tile starts at row 128 w.
+    // K-contiguous: rd[q] is 64-byte K step q of block 0 (block i is 16 rows further);
+    // M/N-contiguous: rd[i] is block i, the first 8 k-rows of the lane's 16 of K step 0.
+    template <bool KCONTIG>
+    __device__ __forceinline__ void readOffsets8(uint32_t w, uint32_t lane, uint32_t (&rd)[8])
+    {
+        const uint32_t t = lane & 15u, g = lane >> 4;
+#pragma unroll
+        for(uint32_t i = 0; i < 8; ++i)
+            rd[i] = 0u;
+        if constexpr(KCONTIG)
+        {
+            const uint32_t r = w * 128u + t;
+            rd[0]            = r * STAGE_KB + ((g ^ swzK8(r)) * CHUNK);
+            rd[1]            = r * STAGE_KB + (((4u + g) ^ swzK8(r)) * CHUNK);
+        }
+        else
+        {
+            const uint32_t kr = 16u * g + (t >> 1);
+#pragma unroll
+            for(uint32_t i = 0; i < 8; ++i)
+                rd[i] = kr * 256u + (((w * 8u + i) ^ swzMN8(kr)) * CHUNK) + (t & 1u) * 8u;
+        }
+    }
+
+    // 16 K bytes of block i, K step s (64 bytes), of the operand tile at `tile`: they arrive whole with
+    // part 0 (K-contiguous) or as two transposed halves, parts 0 and 1, into registers at, at + 1 and
+    // at + 2, at + 3 of `dst`
+    template <bool KCONTIG, typename V>
+    __device__ __forceinline__ void readBlock8(const char* tile, const uint32_t (&rd)[8], uint32_t i, uint32_t s, uint32_t part,
+                                               V& dst, uint32_t at)
+    {
+        if constexpr(KCONTIG)
+        {
+            if(part == 0u)
+            {
+                const i32x4 v = *reinterpret_cast<const i32x4*>(tile + rd[s] + i * 16u * STAGE_KB);
+                dst[at] = v[0], dst[at + 1u] = v[1], dst[at + 2u] = v[2], dst[at + 3u] = v[3];
+            }
+        }
+        else
+        {
+            using lp      = __attribute__((address_space(3))) i32x2*;
+            const i32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lp)(tile + rd[i] + (64u * s + 8u * part) * 256u));
+            dst[at + 2u * part] = v[0], dst[at + 2u * part + 1u] = v[1];
+        }
+    }
+
     // ------------------------------------------------------------------------------------------
     // int8 on v_mfma_i32_16x16x64_i8: the five-buffer scheme with the K-step structure and the
     // in-place inline-assembly accumulators of gemmTiledKernel16.  A stage is two
-    // K steps of 64 bytes; lane -> operand mapping: row lane % 16, 16-byte chunk lane / 16 of the step.
+    // K steps of 64 bytes; lane -> operand mapping: row lane % 16, K bytes 16 (lane / 16) .. + 15 of the step.
     using i32x4v = int __attribute__((ext_vector_type(4)));
     __device__ __forceinline__ void mfma16i8(i32x4v& acc, i32x4 x, i32x4 y)
     {
         asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc) : "v"(x), "v"(y));
     }
 
+    template <bool A_KCONTIG, bool B_KCONTIG>
     __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) gemmTiledKernelI8(Params p)
     {
         // LDS map: A buffers at 0 and 32 KiB, B buffers at 64, 96 and 128 KiB
@@ -526,25 +630,15 @@ namespace
         const uint32_t lane = tid & 63u;
         const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const uint32_t wm = wave >> 1, wn = wave & 1u;
-        auto           swzK = [](uint32_t row) { return (row >> 1) & 7u; };
         const uint32_t ldsBase
             = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds));
 
-        // global -> LDS: chunk L = j * 256 + tid of an operand tile sits at LDS byte 16 L (row L / 8)
-        const uint32_t gr = tid >> 3, gslot = tid & 7u;
-        // one lane offset per load: rows beyond an edge tile's valid part read its last valid row instead
-        // (what lands in LDS for them only feeds elements of D that are never stored)
-        uint32_t       gOffA[LOADS_PER_OPER], gOffB[LOADS_PER_OPER];
+        uint32_t       gOffA[LOADS_PER_OPER], gOffB[LOADS_PER_OPER], gStepA, gStepB;
+        uint64_t       gStageA, gStageB;
         const uint32_t validM = p.m - tm * TILE_M < TILE_M ? p.m - tm * TILE_M : TILE_M;
         const uint32_t validN = p.n - tn * TILE_N < TILE_N ? p.n - tn * TILE_N : TILE_N;
-#pragma unroll
-        for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
-        {
-            const uint32_t ra = gr + 32u * j < validM ? gr + 32u * j : validM - 1u;
-            const uint32_t rb = gr + 32u * j < validN ? gr + 32u * j : validN - 1u;
-            gOffA[j]          = ra * p.lda + ((gslot ^ swzK(gr)) * CHUNK);
-            gOffB[j]          = rb * p.ldb + ((gslot ^ swzK(gr)) * CHUNK);
-        }
+        laneOffsets8<A_KCONTIG>(tid, p.lda, validM, gOffA, gStepA, gStageA);
+        laneOffsets8<B_KCONTIG>(tid, p.ldb, validN, gOffB, gStepB, gStageB);
         const uint32_t numStages = p.k / STAGE_KB;
         const uint32_t dmaDst    = ldsBase + wave * 64u * CHUNK; // + buffer + j * 4 KiB
         auto           uniform64 = [](const char* ptr) {
@@ -553,33 +647,25 @@ namespace
             const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
             return (static_cast<uint64_t>(hi) << 32) | lo;
         };
-        const uint64_t gA = uniform64(p.a + (uint64_t)tm * TILE_M * p.lda);
-        const uint64_t gB = uniform64(p.b + (uint64_t)tn * TILE_N * p.ldb);
+        const uint64_t gA = uniform64(p.a + (A_KCONTIG ? (uint64_t)tm * TILE_M * p.lda : (uint64_t)tm * TILE_M));
+        const uint64_t gB = uniform64(p.b + (B_KCONTIG ? (uint64_t)tn * TILE_N * p.ldb : (uint64_t)tn * TILE_N));
         auto rsrcAt = [](uint64_t addr) { // raw buffer over a stage of an operand panel
             return i32x4{static_cast<int>(static_cast<uint32_t>(addr)), static_cast<int>(static_cast<uint32_t>(addr >> 32) & 0xFFFFu),
                          0x7FFFFFFF, 0x00020000};
         };
-        auto stageAddr = [&](uint64_t panel, uint32_t stage) { // clamped to the last stage
-            return panel + (uint64_t)(stage < numStages ? stage : numStages - 1u) * STAGE_KB;
+        auto stageAddr = [&](uint64_t panel, uint64_t perStage, uint32_t stage) { // clamped to the last stage
+            return panel + (uint64_t)(stage < numStages ? stage : numStages - 1u) * perStage;
         };
-        auto issueHalf = [&](uint64_t addr, const uint32_t (&gOff)[LOADS_PER_OPER], uint32_t at) {
+        auto issueHalf = [&](uint64_t addr, const uint32_t (&gOff)[LOADS_PER_OPER], uint32_t step, uint32_t at) {
             const i32x4 rsrc = rsrcAt(addr);
 #pragma unroll
             for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
-                loadToLds(rsrc, gOff[j], 0u, dmaDst + at + j * THREADS * CHUNK);
+                loadToLds(rsrc, gOff[j], j * step, dmaDst + at + j * THREADS * CHUNK);
         };
 
-        // LDS -> registers: block i rows are 16 i + lane % 16; K step s reads chunk 4 s + lane / 16
-        uint32_t rdA[2], rdB[2];
-        {
-            const uint32_t ra = wm * 128u + (lane & 15u), rb = wn * 128u + (lane & 15u), g = lane >> 4;
-#pragma unroll
-            for(uint32_t s = 0; s < 2; ++s)
-            {
-                rdA[s] = ra * STAGE_KB + (((4u * s + g) ^ swzK(ra)) * CHUNK);
-                rdB[s] = rb * STAGE_KB + (((4u * s + g) ^ swzK(rb)) * CHUNK);
-            }
-        }
+        uint32_t rdA[8], rdB[8];
+        readOffsets8<A_KCONTIG>(wm, lane, rdA);
+        readOffsets8<B_KCONTIG>(wn, lane, rdB);
 
         i32x4v acc[8][8];
 #pragma unroll
@@ -599,19 +685,19 @@ namespace
             mfma16i8(acc[i][j], fb[s][j], fa[s][i]);
         };
         // operand block x of K step s: x = 2 i is A block i, x = 2 i + 1 is B block i
-        auto readAt = [&](uint32_t aAt, uint32_t bAt, uint32_t s, uint32_t x) {
-            const uint32_t i = x >> 1;
+        auto readAt = [&](uint32_t aAt, uint32_t bAt, uint32_t s, uint32_t x, uint32_t part) {
             if(x & 1u)
-                fb[s][i] = *reinterpret_cast<const i32x4*>(lds + bAt + rdB[s] + i * 16u * STAGE_KB);
+                readBlock8<B_KCONTIG>(lds + bAt, rdB, x >> 1, s, part, fb[s][x >> 1], 0u);
             else
-                fa[s][i] = *reinterpret_cast<const i32x4*>(lds + aAt + rdA[s] + i * 16u * STAGE_KB);
+                readBlock8<A_KCONTIG>(lds + aAt, rdA, x >> 1, s, part, fa[s][x >> 1], 0u);
         };
 
         uint64_t refillA, refillB; // stage kt + 2 of A, stage kt + 3 of B (clamped)
         // One K stage: K step 0 is in registers; step 1 arrives under its matrix instructions; then the
         // stage's buffers are refilled (A two stages ahead, B three) while step 0 of the next stage
-        // arrives under the matrix instructions of step 1.  One read per four matrix instructions, one
-        // direct load per four; nothing moves between the pieces.
+        // arrives under the matrix instructions of step 1.  Per four matrix instructions: one operand
+        // block read (two reads when it is transposed on the way) and, in the second half, one direct
+        // load; nothing moves between the pieces.
         auto stageBody = [&](uint32_t kt, uint32_t aCur, uint32_t aNxt, uint32_t bCur, uint32_t bNxt) {
 #pragma unroll
             for(uint32_t x = 0; x < 16; ++x)
@@ -619,48 +705,51 @@ namespace
                 for(uint32_t q = 0; q < 4; ++q)
                 {
                     mfmaAt(0, 4u * x + q);
-                    if(q == 0u)
-                        readAt(aCur, bCur, 1, x);
+                    if(q < 2u)
+                        readAt(aCur, bCur, 1, x, q);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             waitVmcnt<8>(); // this wave's part of stage kt + 1 has landed (the youngest 8 loads are B of kt + 2)
             ldsBarrier();
             const i32x4 rsrcA = rsrcAt(refillA), rsrcB = rsrcAt(refillB);
             if(kt + 3u < numStages)
-                refillA += STAGE_KB;
+                refillA += gStageA;
             if(kt + 4u < numStages)
-                refillB += STAGE_KB;
+                refillB += gStageB;
 #pragma unroll
             for(uint32_t x = 0; x < 16; ++x)
 #pragma unroll
                 for(uint32_t q = 0; q < 4; ++q)
                 {
                     mfmaAt(1, 4u * x + q);
-                    if(q == 0u)
-                        readAt(aNxt, bNxt, 0, x);
+                    if(q < 2u)
+                        readAt(aNxt, bNxt, 0, x, q);
                     if(q == 2u)
                     {
                         if(x < 8u)
-                            loadToLds(rsrcA, gOffA[x], 0u, dmaDst + aCur + x * THREADS * CHUNK);
+                            loadToLds(rsrcA, gOffA[x], x * gStepA, dmaDst + aCur + x * THREADS * CHUNK);
                         else
-                            loadToLds(rsrcB, gOffB[x - 8u], 0u, dmaDst + bCur + (x - 8u) * THREADS * CHUNK);
+                            loadToLds(rsrcB, gOffB[x - 8u], (x - 8u) * gStepB, dmaDst + bCur + (x - 8u) * THREADS * CHUNK);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
         };
 
         // prologue: stages 0 and 1 and the B half of stage 2 requested; stage 0 published
-        issueHalf(stageAddr(gA, 0u), gOffA, A_AT[0]);
-        issueHalf(stageAddr(gB, 0u), gOffB, B_AT[0]);
-        issueHalf(stageAddr(gA, 1u), gOffA, A_AT[1]);
-        issueHalf(stageAddr(gB, 1u), gOffB, B_AT[1]);
-        issueHalf(stageAddr(gB, 2u), gOffB, B_AT[2]);
-        refillA = stageAddr(gA, 2u), refillB = stageAddr(gB, 3u);
+        issueHalf(stageAddr(gA, gStageA, 0u), gOffA, gStepA, A_AT[0]);
+        issueHalf(stageAddr(gB, gStageB, 0u), gOffB, gStepB, B_AT[0]);
+        issueHalf(stageAddr(gA, gStageA, 1u), gOffA, gStepA, A_AT[1]);
+        issueHalf(stageAddr(gB, gStageB, 1u), gOffB, gStepB, B_AT[1]);
+        issueHalf(stageAddr(gB, gStageB, 2u), gOffB, gStepB, B_AT[2]);
+        refillA = stageAddr(gA, gStageA, 2u), refillB = stageAddr(gB, gStageB, 3u);
         waitVmcnt<24>();
         ldsBarrier();
 #pragma unroll
         for(uint32_t x = 0; x < 16; ++x)
-            readAt(A_AT[0], B_AT[0], 0, x);
+        {
+            readAt(A_AT[0], B_AT[0], 0, x, 0);
+            readAt(A_AT[0], B_AT[0], 0, x, 1);
+        }
 
         // six stages per trip bring every buffer back to its role; single-exit loop, then the remainder
         uint32_t kt = 0;
@@ -703,11 +792,12 @@ namespace
 
     // ------------------------------------------------------------------------------------------
     // fp8 e4m3 on v_mfma_f32_16x16x128_f8f6f4.  One instruction spans the whole 128-byte K stage
-    // (32 bytes per lane: chunks lane / 16 and 4 + lane / 16, a K permutation shared by A and B), so
-    // a stage cannot be split along K.  It is split into quadrants of the wave tile instead:
+    // (32 bytes per lane: K bytes 16 (lane / 16) .. + 15 of each 64-byte half, a K permutation shared by
+    // A and B), so a stage cannot be split along K.  It is split into quadrants of the wave tile instead:
     //     Q1 = A[0..3] x B[0..3]   Q2 = A[0..3] x B[4..7]   Q3 = A[4..7] x B[4..7]   Q4 = A[4..7] x B[0..3]
     // Consecutive quadrants share one operand group (4 blocks, 32 registers), so each quadrant's 16
-    // matrix instructions hide the 8 LDS reads of the one group the next quadrant needs:
+    // matrix instructions hide the LDS reads (8, or 16 transposing ones) of the one group the next
+    // quadrant needs:
     //     under Q1: B[4..7] of this stage       under Q3: A[0..3] of the next stage
     //     under Q2: A[4..7] of this stage       under Q4: B[0..3] of the next stage
     // After Q2 the stage's buffers are no longer read: barrier, then the refills are issued under Q3
@@ -719,6 +809,7 @@ namespace
         asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc) : "v"(x), "v"(y));
     }
 
+    template <bool A_KCONTIG, bool B_KCONTIG>
     __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) gemmTiledKernelF8(Params p)
     {
         constexpr uint32_t A_AT[2] = {0u, OPER_BYTES};
@@ -733,25 +824,15 @@ namespace
         const uint32_t lane = tid & 63u;
         const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const uint32_t wm = wave >> 1, wn = wave & 1u;
-        auto           swzK = [](uint32_t row) { return (row >> 1) & 7u; };
         const uint32_t ldsBase
             = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds));
 
-        // global -> LDS: chunk L = j * 256 + tid of an operand tile sits at LDS byte 16 L (row L / 8)
-        const uint32_t gr = tid >> 3, gslot = tid & 7u;
-        // one lane offset per load: rows beyond an edge tile's valid part read its last valid row instead
-        // (what lands in LDS for them only feeds elements of D that are never stored)
-        uint32_t       gOffA[LOADS_PER_OPER], gOffB[LOADS_PER_OPER];
+        uint32_t       gOffA[LOADS_PER_OPER], gOffB[LOADS_PER_OPER], gStepA, gStepB;
+        uint64_t       gStageA, gStageB;
         const uint32_t validM = p.m - tm * TILE_M < TILE_M ? p.m - tm * TILE_M : TILE_M;
         const uint32_t validN = p.n - tn * TILE_N < TILE_N ? p.n - tn * TILE_N : TILE_N;
-#pragma unroll
-        for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
-        {
-            const uint32_t ra = gr + 32u * j < validM ? gr + 32u * j : validM - 1u;
-            const uint32_t rb = gr + 32u * j < validN ? gr + 32u * j : validN - 1u;
-            gOffA[j]          = ra * p.lda + ((gslot ^ swzK(gr)) * CHUNK);
-            gOffB[j]          = rb * p.ldb + ((gslot ^ swzK(gr)) * CHUNK);
-        }
+        laneOffsets8<A_KCONTIG>(tid, p.lda, validM, gOffA, gStepA, gStageA);
+        laneOffsets8<B_KCONTIG>(tid, p.ldb, validN, gOffB, gStepB, gStageB);
         const uint32_t numStages = p.k / STAGE_KB;
         const uint32_t dmaDst    = ldsBase + wave * 64u * CHUNK;
         auto           uniform64 = [](const char* ptr) {
@@ -760,38 +841,33 @@ namespace
             const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
             return (static_cast<uint64_t>(hi) << 32) | lo;
         };
-        const uint64_t gA = uniform64(p.a + (uint64_t)tm * TILE_M * p.lda);
-        const uint64_t gB = uniform64(p.b + (uint64_t)tn * TILE_N * p.ldb);
+        const uint64_t gA = uniform64(p.a + (A_KCONTIG ? (uint64_t)tm * TILE_M * p.lda : (uint64_t)tm * TILE_M));
+        const uint64_t gB = uniform64(p.b + (B_KCONTIG ? (uint64_t)tn * TILE_N * p.ldb : (uint64_t)tn * TILE_N));
         auto rsrcAt = [](uint64_t addr) {
             return i32x4{static_cast<int>(static_cast<uint32_t>(addr)), static_cast<int>(static_cast<uint32_t>(addr >> 32) & 0xFFFFu),
                          0x7FFFFFFF, 0x00020000};
         };
-        auto stageAddr = [&](uint64_t panel, uint32_t stage) {
-            return panel + (uint64_t)(stage < numStages ? stage : numStages - 1u) * STAGE_KB;
+        auto stageAddr = [&](uint64_t panel, uint64_t perStage, uint32_t stage) {
+            return panel + (uint64_t)(stage < numStages ? stage : numStages - 1u) * perStage;
         };
-        auto issueHalf = [&](uint64_t addr, const uint32_t (&gOff)[LOADS_PER_OPER], uint32_t at) {
+        auto issueHalf = [&](uint64_t addr, const uint32_t (&gOff)[LOADS_PER_OPER], uint32_t step, uint32_t at) {
             const i32x4 rsrc = rsrcAt(addr);
 #pragma unroll
             for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
-                loadToLds(rsrc, gOff[j], 0u, dmaDst + at + j * THREADS * CHUNK);
+                loadToLds(rsrc, gOff[j], j * step, dmaDst + at + j * THREADS * CHUNK);
         };
 
-        // LDS -> registers: block rows are 16 i + lane % 16; piece q of a block is chunk 4 q + lane / 16
-        uint32_t rdA[2], rdB[2];
-        {
-            const uint32_t ra = wm * 128u + (lane & 15u), rb = wn * 128u + (lane & 15u), g = lane >> 4;
-#pragma unroll
-            for(uint32_t q = 0; q < 2; ++q)
-            {
-                rdA[q] = ra * STAGE_KB + (((4u * q + g) ^ swzK(ra)) * CHUNK);
-                rdB[q] = rb * STAGE_KB + (((4u * q + g) ^ swzK(rb)) * CHUNK);
-            }
-        }
-        // read r (0..7) of an operand group: block 4 half + r / 2, piece r % 2
-        auto readPiece = [&](i32x8 (&grp)[4], uint32_t at, const uint32_t (&rd)[2], uint32_t half, uint32_t r) {
-            const uint32_t b = r >> 1, q = r & 1u;
-            const i32x4    v = *reinterpret_cast<const i32x4*>(lds + at + rd[q] + (4u * half + b) * 16u * STAGE_KB);
-            grp[b][4u * q] = v[0], grp[b][4u * q + 1u] = v[1], grp[b][4u * q + 2u] = v[2], grp[b][4u * q + 3u] = v[3];
+        uint32_t rdA[8], rdB[8];
+        readOffsets8<A_KCONTIG>(wm, lane, rdA);
+        readOffsets8<B_KCONTIG>(wn, lane, rdB);
+        // Slot n (0..15) of a quadrant brings a piece of the operand group that holds blocks 4 half .. + 3:
+        // K-contiguous: even slots, 16 bytes -- block n / 4, 64-byte half (n / 2) % 2;
+        // M/N-contiguous: every slot, 8 transposed bytes -- same block and half, part n % 2.
+        auto readSlotA = [&](i32x8 (&grp)[4], uint32_t at, uint32_t half, uint32_t n) {
+            readBlock8<A_KCONTIG>(lds + at, rdA, 4u * half + (n >> 2), (n >> 1) & 1u, n & 1u, grp[n >> 2], 4u * ((n >> 1) & 1u));
+        };
+        auto readSlotB = [&](i32x8 (&grp)[4], uint32_t at, uint32_t half, uint32_t n) {
+            readBlock8<B_KCONTIG>(lds + at, rdB, 4u * half + (n >> 2), (n >> 1) & 1u, n & 1u, grp[n >> 2], 4u * ((n >> 1) & 1u));
         };
 
         f32x4 acc[8][8];
@@ -811,8 +887,7 @@ namespace
             for(uint32_t n = 0; n < 16; ++n)
             {
                 mfma16f8(acc[n & 3u][n >> 2], bLo[n >> 2], aLo[n & 3u]);
-                if(!(n & 1u))
-                    readPiece(bHi, bCur, rdB, 1, n >> 1);
+                readSlotB(bHi, bCur, 1, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
             // Q2: A[0..3] x B[4..7] (column by column, in the order B arrived); A[4..7] arrives
@@ -820,26 +895,24 @@ namespace
             for(uint32_t n = 0; n < 16; ++n)
             {
                 mfma16f8(acc[n & 3u][4u + (n >> 2)], bHi[n >> 2], aLo[n & 3u]);
-                if(!(n & 1u))
-                    readPiece(aHi, aCur, rdA, 1, n >> 1);
+                readSlotA(aHi, aCur, 1, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
             waitVmcnt<8>(); // this wave's part of stage kt + 1 has landed (the youngest 8 loads are B of kt + 2)
             ldsBarrier();
             const i32x4 rsrcA = rsrcAt(refillA), rsrcB = rsrcAt(refillB);
             if(kt + 3u < numStages)
-                refillA += STAGE_KB;
+                refillA += gStageA;
             if(kt + 4u < numStages)
-                refillB += STAGE_KB;
+                refillB += gStageB;
             // Q3: A[4..7] x B[4..7] (row by row, in the order A arrived); next A[0..3] arrives; A refill
 #pragma unroll
             for(uint32_t n = 0; n < 16; ++n)
             {
                 mfma16f8(acc[4u + (n >> 2)][4u + (n & 3u)], bHi[n & 3u], aHi[n >> 2]);
-                if(!(n & 1u))
-                    readPiece(aLo, aNxt, rdA, 0, n >> 1);
-                else
-                    loadToLds(rsrcA, gOffA[n >> 1], 0u, dmaDst + aCur + (n >> 1) * THREADS * CHUNK);
+                readSlotA(aLo, aNxt, 0, n);
+                if(n & 1u)
+                    loadToLds(rsrcA, gOffA[n >> 1], (n >> 1) * gStepA, dmaDst + aCur + (n >> 1) * THREADS * CHUNK);
                 __builtin_amdgcn_sched_barrier(0);
             }
             // Q4: A[4..7] x B[0..3]; next B[0..3] arrives in the registers B[4..7] has left; B refill
@@ -847,28 +920,27 @@ namespace
             for(uint32_t n = 0; n < 16; ++n)
             {
                 mfma16f8(acc[4u + (n & 3u)][n >> 2], bLo[n >> 2], aHi[n & 3u]);
-                if(!(n & 1u))
-                    readPiece(bHi, bNxt, rdB, 0, n >> 1);
-                else
-                    loadToLds(rsrcB, gOffB[n >> 1], 0u, dmaDst + bCur + (n >> 1) * THREADS * CHUNK);
+                readSlotB(bHi, bNxt, 0, n);
+                if(n & 1u)
+                    loadToLds(rsrcB, gOffB[n >> 1], (n >> 1) * gStepB, dmaDst + bCur + (n >> 1) * THREADS * CHUNK);
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
 
         // prologue: stages 0 and 1 and the B half of stage 2 requested; stage 0 published
-        issueHalf(stageAddr(gA, 0u), gOffA, A_AT[0]);
-        issueHalf(stageAddr(gB, 0u), gOffB, B_AT[0]);
-        issueHalf(stageAddr(gA, 1u), gOffA, A_AT[1]);
-        issueHalf(stageAddr(gB, 1u), gOffB, B_AT[1]);
-        issueHalf(stageAddr(gB, 2u), gOffB, B_AT[2]);
-        refillA = stageAddr(gA, 2u), refillB = stageAddr(gB, 3u);
+        issueHalf(stageAddr(gA, gStageA, 0u), gOffA, gStepA, A_AT[0]);
+        issueHalf(stageAddr(gB, gStageB, 0u), gOffB, gStepB, B_AT[0]);
+        issueHalf(stageAddr(gA, gStageA, 1u), gOffA, gStepA, A_AT[1]);
+        issueHalf(stageAddr(gB, gStageB, 1u), gOffB, gStepB, B_AT[1]);
+        issueHalf(stageAddr(gB, gStageB, 2u), gOffB, gStepB, B_AT[2]);
+        refillA = stageAddr(gA, gStageA, 2u), refillB = stageAddr(gB, gStageB, 3u);
         waitVmcnt<24>();
         ldsBarrier();
 #pragma unroll
-        for(uint32_t r = 0; r < 8; ++r)
+        for(uint32_t n = 0; n < 16; ++n)
         {
-            readPiece(aLo, A_AT[0], rdA, 0, r);
-            readPiece(bX, B_AT[0], rdB, 0, r);
+            readSlotA(aLo, A_AT[0], 0, n);
+            readSlotB(bX, B_AT[0], 0, n);
         }
 
         // six stages per trip bring every buffer and both B register groups back to their roles
@@ -912,18 +984,25 @@ namespace
     int launchLayouts(bool aK, bool bK, const Params& p, hipStream_t stream)
     {
         const dim3 grid(((p.tilesM * p.tilesN + 7u) / 8u) * 8u), block(THREADS);
-        if constexpr(E == Elem::I8)
-            hipLaunchKernelGGL(gemmTiledKernelI8, grid, block, 0, stream, p);
-        else if constexpr(E == Elem::E4M3)
-            hipLaunchKernelGGL(gemmTiledKernelF8, grid, block, 0, stream, p);
-        else if(aK && bK)
-            hipLaunchKernelGGL((gemmTiledKernel16<E, OutT, true, true>), grid, block, 0, stream, p);
+        auto launch = [&](auto aKc, auto bKc) {
+            constexpr bool AK = decltype(aKc)::value, BK = decltype(bKc)::value;
+            if constexpr(E == Elem::I8)
+                hipLaunchKernelGGL((gemmTiledKernelI8<AK, BK>), grid, block, 0, stream, p);
+            else if constexpr(E == Elem::E4M3)
+                hipLaunchKernelGGL((gemmTiledKernelF8<AK, BK>), grid, block, 0, stream, p);
+            else
+                hipLaunchKernelGGL((gemmTiledKernel16<E, OutT, AK, BK>), grid, block, 0, stream, p);
+        };
+        using T = std::true_type;
+        using F = std::false_type;
+        if(aK && bK)
+            launch(T{}, T{});
         else if(aK)
-            hipLaunchKernelGGL((gemmTiledKernel16<E, OutT, true, false>), grid, block, 0, stream, p);
+            launch(T{}, F{});
         else if(bK)
-            hipLaunchKernelGGL((gemmTiledKernel16<E, OutT, false, true>), grid, block, 0, stream, p);
+            launch(F{}, T{});
         else
-            hipLaunchKernelGGL((gemmTiledKernel16<E, OutT, false, false>), grid, block, 0, stream, p);
+            launch(F{}, F{});
         return r355::checkLaunch("gemm (macro tile)");
     }
 } // namespace
@@ -939,8 +1018,6 @@ namespace r355
         if(!pairOk)
             return fail(R355_ERR_UNSUPPORTED, "tiled gemm: no kernel for in_type %d -> out_type %d", g.in_type, g.out_type);
         const uint32_t es = dtypeBytes(g.in_type), os = dtypeBytes(g.out_type);
-        if(es == 1 && !(g.layout_a == R355_ROW_MAJOR && g.layout_b == R355_COL_MAJOR))
-            return fail(R355_ERR_UNSUPPORTED, "tiled gemm: 8-bit operands must be K-contiguous (A row-major, B col-major)");
         if(g.beta != 0.0f && g.layout_c != g.layout_d)
             return fail(R355_ERR_UNSUPPORTED, "tiled gemm: C and D must share an orientation");
         const uint32_t tk = STAGE_KB / es;

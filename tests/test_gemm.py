@@ -152,13 +152,39 @@ def test_tiled_kernel_16bit_layouts(in_t, out_t, la, lb, ldl):
 
 
 @pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32)])
+@pytest.mark.parametrize("la,lb", TILED_LAYOUTS_16)
 @pytest.mark.parametrize("ldl", [O.ROW, O.COL])
-def test_tiled_kernel_8bit(in_t, out_t, ldl):
+def test_tiled_kernel_8bit_layouts(in_t, out_t, la, lb, ldl):
+    # K-contiguous operands are read whole, M/N-contiguous ones through the transposing LDS read
     m, n, k = 256, 512, 768
     a, b, c = _inputs(in_t, out_t, m, n, k, seed=21)
-    want = O.gemm(in_t, out_t, O.ROW, O.COL, ldl, ldl, m, n, k, a, b, c, 1.0, 1.0)
-    got = _run(in_t, out_t, O.ROW, O.COL, ldl, ldl, m, n, k, a, b, c, 1.0, 1.0, R.KERNEL_TILED)
+    want = O.gemm(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, c, 1.0, 1.0)
+    got = _run(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, c, 1.0, 1.0, R.KERNEL_TILED)
     _check(in_t, out_t, got, want)
+    # reference-pattern inputs: exact
+    a, b = O.fill_ref(in_t, m, k, la), O.fill_ref(in_t, k, n, lb)
+    want = O.gemm(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, None, 1.0, 0.0)
+    got = _run(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, None, 1.0, 0.0, R.KERNEL_TILED)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("la,lb", TILED_LAYOUTS_16)
+def test_tiled_kernel_8bit_one_hot_operands(la, lb):
+    # A single non-zero in A and in B lands in exactly one element of D only if every (row, k) and
+    # (k, column) of the operand tiles reaches the matrix instruction it belongs to: probes the
+    # global -> LDS placement and the (transposing) LDS reads of both orientations.
+    m, n, k = 256, 256, 256
+    rng = np.random.default_rng(5)
+    for _ in range(6):
+        i, j, h = int(rng.integers(m)), int(rng.integers(n)), int(rng.integers(k))
+        a = np.zeros(m * k, np.int8)
+        b = np.zeros(k * n, np.int8)
+        a[i * k + h if la == O.ROW else h * m + i] = 3
+        b[h * n + j if lb == O.ROW else j * k + h] = 5
+        got = _run(O.I8, O.I32, la, lb, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0, R.KERNEL_TILED).reshape(m, n)
+        want = np.zeros((m, n), np.int32)
+        want[i, j] = 15
+        assert np.array_equal(got, want), (i, j, h)
 
 
 # the sizes the reference's GEMM suites validate (test/gemm/gemm_common_test_params.hpp:336-348) with its
@@ -200,14 +226,15 @@ def test_tiled_kernel_16bit_edge_tiles(in_t, out_t, la, lb, m, n, k):
 
 
 @pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32)])
-@pytest.mark.parametrize("ldl", [O.ROW, O.COL])
+@pytest.mark.parametrize("la,lb,ldl", [(O.ROW, O.COL, O.ROW), (O.ROW, O.COL, O.COL), (O.COL, O.ROW, O.ROW),
+                                       (O.COL, O.COL, O.COL), (O.ROW, O.ROW, O.ROW)])
 @pytest.mark.parametrize("m,n,k", RAGGED_SHAPES)
-def test_tiled_kernel_8bit_edge_tiles(in_t, out_t, ldl, m, n, k):
+def test_tiled_kernel_8bit_edge_tiles(in_t, out_t, la, lb, ldl, m, n, k):
     a, b, c = _inputs(in_t, out_t, m, n, k, seed=80 + n)
     for alpha, beta in ((1.0, 0.0), (1.0, 1.0)):
         cc = None if beta == 0.0 else c
-        want = O.gemm(in_t, out_t, O.ROW, O.COL, ldl, ldl, m, n, k, a, b, cc, alpha, beta)
-        got = _run(in_t, out_t, O.ROW, O.COL, ldl, ldl, m, n, k, a, b, cc, alpha, beta, R.KERNEL_TILED)
+        want = O.gemm(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, cc, alpha, beta)
+        got = _run(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, cc, alpha, beta, R.KERNEL_TILED)
         _check(in_t, out_t, got, want)
 
 
@@ -241,14 +268,15 @@ def test_tiled_kernel_16bit_stage_counts(in_t, out_t, la, lb, k):
 
 
 @pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32)])
+@pytest.mark.parametrize("la,lb", [(O.ROW, O.COL), (O.COL, O.ROW)])
 @pytest.mark.parametrize("stages", [1, 2, 3, 4, 5, 6, 7, 11, 13])
-def test_tiled_kernel_8bit_stage_counts(in_t, out_t, stages):
+def test_tiled_kernel_8bit_stage_counts(in_t, out_t, la, lb, stages):
     # The 8-bit kernel rotates five LDS buffers with period six; cover every remainder of the K
     # stage count, including a single stage and counts beyond one period.
     m, n, k = 256, 256, 128 * stages
     a, b, _ = _inputs(in_t, out_t, m, n, k, seed=40 + stages)
-    want = O.gemm(in_t, out_t, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0)
-    got = _run(in_t, out_t, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0, R.KERNEL_TILED)
+    want = O.gemm(in_t, out_t, la, lb, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0)
+    got = _run(in_t, out_t, la, lb, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0, R.KERNEL_TILED)
     _check(in_t, out_t, got, want)
 
 
@@ -273,7 +301,8 @@ def test_auto_falls_back_and_bad_sizes_error():
 
 
 @pytest.mark.parametrize("in_t,out_t,la,lb", [(O.F16, O.F16, O.COL, O.ROW), (O.BF16, O.BF16, O.COL, O.ROW),
-                                               (O.I8, O.I32, O.ROW, O.COL), (O.E4M3, O.F32, O.ROW, O.COL)])
+                                               (O.I8, O.I32, O.ROW, O.COL), (O.E4M3, O.F32, O.ROW, O.COL),
+                                               (O.I8, O.I32, O.COL, O.ROW)])
 def test_full_size_8192_sampled_rows(in_t, out_t, la, lb):
     # benchmark configurations 2 and 3 at full size.  Each element of the oracle depends only on its own row
     # of A and column of B, so complete rows computed by the oracle are exactly its values.
@@ -322,7 +351,8 @@ def _embed(flat, rows, cols, layout, ld, fill):
 @pytest.mark.parametrize("kernel", ["tiled", "simple"])
 @pytest.mark.parametrize("in_t,out_t,la,lb,ldl", [(O.F16, O.F16, O.COL, O.ROW, O.ROW), (O.F16, O.F32, O.ROW, O.COL, O.COL),
                                                   (O.BF16, O.BF16, O.ROW, O.ROW, O.ROW), (O.I8, O.I32, O.ROW, O.COL, O.ROW),
-                                                  (O.E4M3, O.F32, O.ROW, O.COL, O.COL)])
+                                                  (O.E4M3, O.F32, O.ROW, O.COL, O.COL), (O.I8, O.I32, O.COL, O.ROW, O.ROW),
+                                                  (O.E4M3, O.F32, O.COL, O.COL, O.ROW)])
 def test_padded_leading_dimensions(kernel, in_t, out_t, la, lb, ldl):
     """Operands and result embedded in wider buffers (ld > extent): the reference kernels take lda..ldd
     (test/gemm/gemm_kernel_base.hpp:101-114); bytes outside the m x n block of D must stay untouched."""
