@@ -31,7 +31,8 @@ namespace
         const uint32_t minLdd = g->layout_d == R355_ROW_MAJOR ? g->n : g->m;
         if(g->lda < minLda || g->ldb < minLdb || g->ldd < minLdd || (g->beta != 0.0f && g->ldc < minLdc))
             return r355::fail(R355_ERR_BAD_ARG, "gemm: leading dimension smaller than the contiguous extent");
-        if(g->kernel != R355_KERNEL_AUTO && g->kernel != R355_KERNEL_SIMPLE && g->kernel != R355_KERNEL_TILED)
+        if(g->kernel != R355_KERNEL_AUTO && g->kernel != R355_KERNEL_SIMPLE && g->kernel != R355_KERNEL_TILED
+           && g->kernel != R355_KERNEL_TILED_128)
             return r355::fail(R355_ERR_BAD_ARG, "gemm: unknown kernel selector %d", g->kernel);
         return R355_OK;
     }
@@ -50,8 +51,9 @@ namespace
         }
         // AUTO leaves problems smaller than half a macro tile in either direction to the block-per-wave
         // kernel: one mostly empty 256 x 256 tile on one CU is slower than many small blocks.
-        const bool worthTiling = g->kernel == R355_KERNEL_TILED || (g->m >= 128 && g->n >= 128);
-        if((g->kernel == R355_KERNEL_TILED || g->kernel == R355_KERNEL_AUTO) && worthTiling)
+        const bool forced      = g->kernel == R355_KERNEL_TILED || g->kernel == R355_KERNEL_TILED_128;
+        const bool worthTiling = forced || (g->m >= 128 && g->n >= 128);
+        if((forced || g->kernel == R355_KERNEL_AUTO) && worthTiling)
         {
             rc = r355::gemmTiledCheck(*g, out);
             if(rc == R355_OK)
@@ -59,7 +61,7 @@ namespace
                 *family = R355_KERNEL_TILED;
                 return rc;
             }
-            if(g->kernel == R355_KERNEL_TILED)
+            if(forced)
                 return rc;
         }
         rc = r355::gemmSimpleCheck(*g, out);

@@ -133,45 +133,46 @@ namespace
             asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(x), "v"(y));
     }
 
-    // D = alpha * acc + beta * C for one wave's 128 x 128 tile of 16 x 16 accumulator blocks, row-major.
-    // `scratch` is 32 KiB of LDS owned by this wave.
-    template <typename AccV, typename OutT>
-    __device__ __forceinline__ void storeTile16(AccV (&acc)[8][8], const Params& p, uint32_t tm, uint32_t tn, uint32_t wm,
-                                                uint32_t wn, uint32_t lane, char* scratch)
+    // D = alpha * acc + beta * C for one wave's tile of WB x WB accumulator blocks (16 x 16 each), row-major;
+    // the wave tile starts at (m0, n0).  `scratch` is WB * 4 KiB of LDS owned by this wave.
+    template <typename AccV, typename OutT, uint32_t WB>
+    __device__ __forceinline__ void storeTile16(AccV (&acc)[WB][WB], const Params& p, uint32_t m0, uint32_t n0, uint32_t lane,
+                                                char* scratch)
     {
         using AccE = std::remove_reference_t<decltype(acc[0][0][0])>;
         using OutV = OutT __attribute__((ext_vector_type(4)));
         const AccE     alpha = static_cast<AccE>(p.alpha), beta = static_cast<AccE>(p.beta);
-        const uint32_t m0 = tm * TILE_M + wm * 128u, n0 = tn * TILE_N + wn * 128u;
         const uint32_t r16 = lane & 15u, g = lane >> 4;
 
         if(beta == static_cast<AccE>(0))
         {
-            // Transpose through the wave's own LDS so that a store instruction covers whole 256- or
-            // 512-byte rows of D with 128 bits per lane.
+            // Transpose through the wave's own LDS so that a store instruction covers whole rows of
+            // the wave tile (128 to 512 bytes) with 128 bits per lane.
             constexpr uint32_t OS         = sizeof(OutT);
-            constexpr uint32_t ROW_BYTES  = 128u * OS;
-            constexpr uint32_t ROW_CHUNKS = ROW_BYTES / CHUNK; // 16 or 32
-            constexpr uint32_t ROWS_PASS  = 32768u / ROW_BYTES; // 128 or 64
-            constexpr uint32_t BLOCKS_I   = ROWS_PASS / 16u; // 8 or 4 row blocks per pass
+            constexpr uint32_t ROW_BYTES  = 16u * WB * OS;
+            constexpr uint32_t ROW_CHUNKS = ROW_BYTES / CHUNK; // 8, 16 or 32
+            constexpr uint32_t SWZ        = ROW_CHUNKS < 16u ? ROW_CHUNKS - 1u : 15u;
+            constexpr uint32_t FIT        = WB * 4096u / ROW_BYTES; // rows the scratch holds
+            constexpr uint32_t ROWS_PASS  = FIT < 16u * WB ? FIT : 16u * WB;
+            constexpr uint32_t BLOCKS_I   = ROWS_PASS / 16u; // row blocks per pass
 #pragma unroll
-            for(uint32_t pass = 0; pass < 8u / BLOCKS_I; ++pass)
+            for(uint32_t pass = 0; pass < WB / BLOCKS_I; ++pass)
             {
 #pragma unroll
                 for(uint32_t ii = 0; ii < BLOCKS_I; ++ii)
                 {
                     const uint32_t i = pass * BLOCKS_I + ii, row = 16u * ii + r16;
 #pragma unroll
-                    for(uint32_t j = 0; j < 8; ++j)
+                    for(uint32_t j = 0; j < WB; ++j)
                     {
                         OutV out;
 #pragma unroll
                         for(uint32_t e = 0; e < 4; ++e)
                             out[e] = static_cast<OutT>(alpha * acc[i][j][e]);
-                        // 16 consecutive rows take 16 different chunk slots
+                        // 16 consecutive rows take 16 (8) different chunk slots
                         const uint32_t byteInRow = (16u * j + 4u * g) * OS;
                         const uint32_t c = byteInRow / CHUNK, within = byteInRow % CHUNK;
-                        *reinterpret_cast<OutV*>(scratch + row * ROW_BYTES + ((c ^ (row & 15u)) * CHUNK) + within) = out;
+                        *reinterpret_cast<OutV*>(scratch + row * ROW_BYTES + ((c ^ (row & SWZ)) * CHUNK) + within) = out;
                     }
                 }
                 __builtin_amdgcn_wave_barrier(); // the same wave reads back what it wrote (LDS is in order per wave)
@@ -179,7 +180,7 @@ namespace
                 for(uint32_t it = 0; it < ROWS_PASS * ROW_CHUNKS / 64u; ++it)
                 {
                     const uint32_t L = it * 64u + lane, row = L / ROW_CHUNKS, c = L % ROW_CHUNKS;
-                    const i32x4    v = *reinterpret_cast<const i32x4*>(scratch + row * ROW_BYTES + ((c ^ (row & 15u)) * CHUNK));
+                    const i32x4    v = *reinterpret_cast<const i32x4*>(scratch + row * ROW_BYTES + ((c ^ (row & SWZ)) * CHUNK));
                     const uint32_t gRow = m0 + pass * ROWS_PASS + row, gCol = n0 + c * (CHUNK / OS);
                     const uint64_t offD = (uint64_t)gRow * p.ldd + n0;
                     // D is written once and not read again: stream it past the caches.  Edge tiles:
@@ -193,16 +194,16 @@ namespace
         }
         // C may alias D, so loads cannot move above earlier stores: fetch a block row of C at a time
 #pragma unroll
-        for(uint32_t i = 0; i < 8; ++i)
+        for(uint32_t i = 0; i < WB; ++i)
         {
             const uint32_t row = m0 + 16u * i + r16;
-            OutV           cv[8];
+            OutV           cv[WB];
 #pragma unroll
-            for(uint32_t j = 0; j < 8; ++j)
+            for(uint32_t j = 0; j < WB; ++j)
                 if(row < p.m && n0 + 16u * j < p.n)
                     cv[j] = *reinterpret_cast<const OutV*>(p.c + ((uint64_t)row * p.ldc + n0 + 16u * j + 4u * g) * sizeof(OutT));
 #pragma unroll
-            for(uint32_t j = 0; j < 8; ++j)
+            for(uint32_t j = 0; j < WB; ++j)
             {
                 OutV out;
 #pragma unroll
@@ -214,20 +215,29 @@ namespace
         }
     }
 
-    template <Elem E, typename OutT, bool A_KCONTIG, bool B_KCONTIG>
-    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
-        gemmTiledKernel16(Params p)
+    //
+    // WB is the number of accumulator blocks per wave tile edge: 8 (wave tile 128 x 128, macro tile
+    // 256 x 256, one workgroup per CU) or 4 (wave tile 64 x 64, macro tile 128 x 128, 64 KiB of LDS and
+    // a quarter of the registers) for problems with too few 256 x 256 tiles to fill the CUs.
+    template <Elem E, typename OutT, bool A_KCONTIG, bool B_KCONTIG, uint32_t WB>
+    __device__ __forceinline__ void gemmTiled16(const Params& p)
     {
         constexpr uint32_t ES = ElemTraits<E>::Bytes;
         constexpr uint32_t TK = STAGE_KB / ES; // 64 K elements per stage = two K steps of 32
         static_assert(ES == 2, "16-bit element types only");
-        // LDS reads per K step: one 128-bit read per operand block, or two transposing 64-bit reads
-        constexpr uint32_t READS_A = A_KCONTIG ? 8u : 16u, READS_B = B_KCONTIG ? 8u : 16u;
-        constexpr uint32_t READS   = READS_A + READS_B; // 16, 24 or 32
+        static_assert(WB == 8 || WB == 4, "wave tile of 8 x 8 or 4 x 4 blocks");
+        constexpr uint32_t TILE  = 32u * WB; // macro tile edge
+        constexpr uint32_t WT    = 16u * WB; // wave tile edge
+        constexpr uint32_t OPER  = TILE * STAGE_KB; // bytes of one operand per stage
+        constexpr uint32_t LOADS = OPER / CHUNK / THREADS; // direct loads per operand per stage = WB
+        constexpr uint32_t ROWB  = TILE * ES; // bytes of a k-row of an M/N-contiguous operand tile
+        constexpr uint32_t KROWS = THREADS * CHUNK / ROWB; // k-rows of such a tile one load covers: 8 or 16
+        constexpr uint32_t XS    = 2u * WB; // operand blocks per K step
+        constexpr uint32_t QS    = WB / 2u; // matrix instructions per operand block
 
         // One variable per stage: the compiler tracks outstanding direct-to-LDS loads per LDS variable.
-        __shared__ __attribute__((aligned(1024))) char stage0[STAGE_BYTES];
-        __shared__ __attribute__((aligned(1024))) char stage1[STAGE_BYTES];
+        __shared__ __attribute__((aligned(1024))) char stage0[2u * OPER];
+        __shared__ __attribute__((aligned(1024))) char stage1[2u * OPER];
 
         uint32_t tm, tn;
         if(!r355::tileCoord(blockIdx.x, p.tilesM, p.tilesN, tm, tn))
@@ -242,22 +252,23 @@ namespace
 
         // ---------------- global -> LDS: chunk L = j * 256 + tid of an operand tile sits at LDS byte 16 L.
         // K-contiguous: row L / 8, and the swizzle does not change with j (32 rows per load).
-        // M/N-contiguous: k-row L / 32 = 8 j + tid / 32; the swizzle alternates with bit 3 of the k-row.
+        // M/N-contiguous: k-row L / (ROWB / 16) = KROWS j + tid / (ROWB / 16); with 8 k-rows per load the
+        // swizzle alternates with bit 3 of the k-row.
         // Edge tiles (m or n not a multiple of 256) must not read outside the operands: a lane whose
         // row (K-contiguous) or 16-byte chunk (M/N-contiguous) lies beyond the matrix reads the last valid
         // row / the first chunk instead -- what lands in LDS for it only feeds elements of D that are
         // never stored.  Hence one lane offset per load (the compiler merges equal ones).
-        uint32_t       gOffA[LOADS_PER_OPER], gOffB[LOADS_PER_OPER], gStepA, gStepB; // gStep: uniform offset per load
+        uint32_t       gOffA[LOADS], gOffB[LOADS], gStepA, gStepB; // gStep: uniform offset per load
         uint64_t       gStageA, gStageB; // bytes between consecutive K stages
-        const uint32_t validM = p.m - tm * TILE_M < TILE_M ? p.m - tm * TILE_M : TILE_M;
-        const uint32_t validN = p.n - tn * TILE_N < TILE_N ? p.n - tn * TILE_N : TILE_N;
-        auto laneOffsets = [&](bool kContig, uint32_t ld, uint32_t valid, uint32_t (&off)[LOADS_PER_OPER], uint32_t& step,
+        const uint32_t validM = p.m - tm * TILE < TILE ? p.m - tm * TILE : TILE;
+        const uint32_t validN = p.n - tn * TILE < TILE ? p.n - tn * TILE : TILE;
+        auto laneOffsets = [&](bool kContig, uint32_t ld, uint32_t valid, uint32_t (&off)[LOADS], uint32_t& step,
                                uint64_t& stage) {
             if(kContig)
             {
                 const uint32_t r = tid >> 3, slot = tid & 7u;
 #pragma unroll
-                for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
+                for(uint32_t j = 0; j < LOADS; ++j)
                 {
                     const uint32_t row = r + 32u * j < valid ? r + 32u * j : valid - 1u;
                     off[j]             = row * ld * ES + ((slot ^ swzK(r)) * CHUNK);
@@ -266,30 +277,31 @@ namespace
             }
             else
             {
-                const uint32_t r = tid >> 5, slot = tid & 31u;
+                constexpr uint32_t SLOTS = ROWB / CHUNK; // 32 or 16 chunks per k-row
+                const uint32_t     r = tid / SLOTS, slot = tid % SLOTS;
 #pragma unroll
-                for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
+                for(uint32_t j = 0; j < LOADS; ++j)
                 {
-                    const uint32_t c = slot ^ swzMN(r + 8u * (j & 1u));
+                    const uint32_t c = slot ^ swzMN(r + KROWS * j);
                     off[j]           = r * ld * ES + (c * (CHUNK / ES) < valid ? c : 0u) * CHUNK;
                 }
-                step = 8u * ld * ES, stage = (uint64_t)TK * ld * ES;
+                step = KROWS * ld * ES, stage = (uint64_t)TK * ld * ES;
             }
         };
         laneOffsets(A_KCONTIG, p.lda, validM, gOffA, gStepA, gStageA);
         laneOffsets(B_KCONTIG, p.ldb, validN, gOffB, gStepB, gStageB);
-        const char* gA = p.a + (A_KCONTIG ? (uint64_t)tm * TILE_M * p.lda * ES : (uint64_t)tm * TILE_M * ES);
-        const char* gB = p.b + (B_KCONTIG ? (uint64_t)tn * TILE_N * p.ldb * ES : (uint64_t)tn * TILE_N * ES);
+        const char* gA = p.a + (A_KCONTIG ? (uint64_t)tm * TILE * p.lda * ES : (uint64_t)tm * TILE * ES);
+        const char* gB = p.b + (B_KCONTIG ? (uint64_t)tn * TILE * p.ldb * ES : (uint64_t)tn * TILE * ES);
 
         // ---------------- LDS -> registers (per lane, fixed)
         // K-contiguous: block i rows are 16 i + lane % 16; K step s reads chunk 4 s + lane / 16.
         // M/N-contiguous: K step s, half h: k-row 32 s + 8 (lane / 16) + 4 h + (lane % 16) / 4,
         //                 8-byte piece m / 4 with m = 16 i + 4 (lane % 4).
-        uint32_t rdA[8], rdB[8];
+        uint32_t rdA[WB], rdB[WB];
         const uint32_t t = lane & 15u, g = lane >> 4;
         if constexpr(A_KCONTIG)
         {
-            const uint32_t r = wm * 128u + t;
+            const uint32_t r = wm * WT + t;
             rdA[0] = r * STAGE_KB + ((g ^ swzK(r)) * CHUNK);
             rdA[1] = r * STAGE_KB + (((4u + g) ^ swzK(r)) * CHUNK);
         }
@@ -297,26 +309,26 @@ namespace
         {
             const uint32_t kr = 8u * g + (t >> 2);
 #pragma unroll
-            for(uint32_t i = 0; i < 8; ++i)
+            for(uint32_t i = 0; i < WB; ++i)
             {
-                const uint32_t piece = wm * 32u + 4u * i + (t & 3u);
-                rdA[i] = kr * 512u + (((piece >> 1) ^ swzMN(kr)) * CHUNK) + (piece & 1u) * 8u;
+                const uint32_t piece = wm * (WT / 4u) + 4u * i + (t & 3u);
+                rdA[i] = kr * ROWB + (((piece >> 1) ^ swzMN(kr)) * CHUNK) + (piece & 1u) * 8u;
             }
         }
         if constexpr(B_KCONTIG)
         {
-            const uint32_t r = wn * 128u + t;
-            rdB[0] = OPER_BYTES + r * STAGE_KB + ((g ^ swzK(r)) * CHUNK);
-            rdB[1] = OPER_BYTES + r * STAGE_KB + (((4u + g) ^ swzK(r)) * CHUNK);
+            const uint32_t r = wn * WT + t;
+            rdB[0] = OPER + r * STAGE_KB + ((g ^ swzK(r)) * CHUNK);
+            rdB[1] = OPER + r * STAGE_KB + (((4u + g) ^ swzK(r)) * CHUNK);
         }
         else
         {
             const uint32_t kr = 8u * g + (t >> 2);
 #pragma unroll
-            for(uint32_t i = 0; i < 8; ++i)
+            for(uint32_t i = 0; i < WB; ++i)
             {
-                const uint32_t piece = wn * 32u + 4u * i + (t & 3u);
-                rdB[i] = OPER_BYTES + kr * 512u + (((piece >> 1) ^ swzMN(kr)) * CHUNK) + (piece & 1u) * 8u;
+                const uint32_t piece = wn * (WT / 4u) + 4u * i + (t & 3u);
+                rdB[i] = OPER + kr * ROWB + (((piece >> 1) ^ swzMN(kr)) * CHUNK) + (piece & 1u) * 8u;
             }
         }
         // An operand block arrives in one 128-bit read (part 0) or in two transposing 64-bit reads
@@ -330,7 +342,7 @@ namespace
             }
             else
             {
-                const char* q = base + rdA[i] + s * 32u * 512u + part * 4u * 512u;
+                const char* q = base + rdA[i] + s * 32u * ROWB + part * 4u * ROWB;
                 const i32x2 v = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lpt)q));
                 dst[2u * part] = v[0], dst[2u * part + 1u] = v[1];
             }
@@ -343,7 +355,7 @@ namespace
             }
             else
             {
-                const char* q = base + rdB[i] + s * 32u * 512u + part * 4u * 512u;
+                const char* q = base + rdB[i] + s * 32u * ROWB + part * 4u * ROWB;
                 const i32x2 v = __builtin_bit_cast(i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lpt)q));
                 dst[2u * part] = v[0], dst[2u * part + 1u] = v[1];
             }
@@ -367,28 +379,28 @@ namespace
             const uint32_t j = x >> 1;
             char*          dst = stage + (j * THREADS + wave * 64u) * CHUNK;
             if(x & 1u)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(srcB, (lp)(dst + OPER_BYTES), 16, gOffB[j], j * gStepB, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(srcB, (lp)(dst + OPER), 16, gOffB[j], j * gStepB, 0, 0);
             else
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(srcA, (lp)dst, 16, gOffA[j], j * gStepA, 0, 0);
         };
         auto issueGlobal = [&](uint32_t kt, char* stage) {
             const __amdgpu_buffer_rsrc_t srcA = stageRsrc(gA + kt * gStageA), srcB = stageRsrc(gB + kt * gStageB);
 #pragma unroll
-            for(uint32_t x = 0; x < 2u * LOADS_PER_OPER; ++x)
+            for(uint32_t x = 0; x < 2u * LOADS; ++x)
                 issueLoad(srcA, srcB, stage, x);
         };
 
-        f32x4          acc[8][8];
+        f32x4          acc[WB][WB];
         const uint32_t numStages = p.k / TK;
 #pragma unroll
-        for(uint32_t i = 0; i < 8; ++i)
+        for(uint32_t i = 0; i < WB; ++i)
 #pragma unroll
-            for(uint32_t j = 0; j < 8; ++j)
+            for(uint32_t j = 0; j < WB; ++j)
                 acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-        i32x4    fa[2][8], fb[2][8];
+        i32x4    fa[2][WB], fb[2][WB];
         uint64_t refillA, refillB; // where the next refill reads from (stage kt + 2, clamped to the last stage)
-        // Matrix instruction n (0..63) of a K step works on accumulator block (i, j) = blockOf(n): block
+        // Matrix instruction n (0 .. WB * WB - 1) of a K step works on accumulator block (i, j) = blockOf(n): block
         // row / column d is first needed after d * d instructions, and the operands arrive in the
         // order A0 B0 A1 B1 ...  Operands swapped: each lane then holds 4 consecutive columns of a row of D.
         auto mfmaAt = [&](uint32_t s, uint32_t n) {
@@ -408,7 +420,7 @@ namespace
         };
         auto readStep = [&](const char* base, uint32_t s) {
 #pragma unroll
-            for(uint32_t x = 0; x < 16; ++x)
+            for(uint32_t x = 0; x < XS; ++x)
             {
                 readAt(base, s, x, 0);
                 readAt(base, s, x, 1);
@@ -422,16 +434,18 @@ namespace
         // occupies its pipeline for 16 cycles and the wave can issue about three other instructions
         // in that time, so the other work is dealt out one piece per matrix instruction, in groups of
         // four: read (part 0), read (part 1), direct load (second step), nothing -- and nothing moves
-        // between pieces.  Every stage runs the same code: past the end the refill is clamped to the
-        // last stage and the operands read ahead are never used.
+        // between pieces (groups of two with the small wave tile: read, read + direct load).  Every stage
+        // runs the same code: past the end the refill is clamped to the last stage and the operands read
+        // ahead are never used.
+        constexpr uint32_t LOAD_Q = QS > 2u ? 2u : QS - 1u;
         auto stageBody = [&](uint32_t kt, char* cur, char* nxt) {
 #pragma unroll
-            for(uint32_t x = 0; x < 16; ++x)
+            for(uint32_t x = 0; x < XS; ++x)
             {
 #pragma unroll
-                for(uint32_t q = 0; q < 4; ++q)
+                for(uint32_t q = 0; q < QS; ++q)
                 {
-                    mfmaAt(0, 4u * x + q);
+                    mfmaAt(0, QS * x + q);
                     if(q < 2u)
                         readAt(cur, 1, x, q);
                     __builtin_amdgcn_sched_barrier(0);
@@ -443,15 +457,15 @@ namespace
             if(kt + 3u < numStages) // the refill of the next stage is one stage further, or the last again
                 refillA += gStageA, refillB += gStageB;
 #pragma unroll
-            for(uint32_t x = 0; x < 16; ++x)
+            for(uint32_t x = 0; x < XS; ++x)
             {
 #pragma unroll
-                for(uint32_t q = 0; q < 4; ++q)
+                for(uint32_t q = 0; q < QS; ++q)
                 {
-                    mfmaAt(1, 4u * x + q);
+                    mfmaAt(1, QS * x + q);
                     if(q < 2u)
                         readAt(nxt, 0, x, q);
-                    else if(q == 2u)
+                    if(q == LOAD_Q)
                         issueLoad(srcA, srcB, cur, x);
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -479,7 +493,21 @@ namespace
         __syncthreads();
         // the last matrix instructions are still in the pipeline and the compiler does not know it
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-        storeTile16<f32x4, OutT>(acc, p, tm, tn, wm, wn, lane, ((wave < 2u) ? stage0 : stage1) + (wave & 1u) * 32768u);
+        storeTile16<f32x4, OutT, WB>(acc, p, tm * TILE + wm * WT, tn * TILE + wn * WT, lane,
+                                     ((wave < 2u) ? stage0 : stage1) + (wave & 1u) * (WB * 4096u));
+    }
+
+    // (a waves-per-EU attribute that depends on a template parameter makes the compiler drop the host-side
+    // launch stub without a diagnostic, hence one kernel per tile size around a common body)
+    template <Elem E, typename OutT, bool A_KCONTIG, bool B_KCONTIG>
+    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) gemmTiledKernel16(Params p)
+    {
+        gemmTiled16<E, OutT, A_KCONTIG, B_KCONTIG, 8>(p);
+    }
+    template <Elem E, typename OutT, bool A_KCONTIG, bool B_KCONTIG>
+    __global__ void __launch_bounds__(THREADS) gemmTiledKernel16Small(Params p)
+    {
+        gemmTiled16<E, OutT, A_KCONTIG, B_KCONTIG, 4>(p);
     }
 
     // ------------------------------------------------------------------------------------------
@@ -787,7 +815,7 @@ namespace
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
         waitVmcnt<0>();
         ldsBarrier();
-        storeTile16<i32x4v, int>(acc, p, tm, tn, wm, wn, lane, lds + wave * OPER_BYTES);
+        storeTile16<i32x4v, int, 8>(acc, p, tm * TILE_M + wm * 128u, tn * TILE_N + wn * 128u, lane, lds + wave * OPER_BYTES);
     }
 
     // ------------------------------------------------------------------------------------------
@@ -977,11 +1005,11 @@ namespace
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); // the last matrix instructions are still in the pipeline
         waitVmcnt<0>();
         ldsBarrier();
-        storeTile16<f32x4, float>(acc, p, tm, tn, wm, wn, lane, lds + wave * OPER_BYTES);
+        storeTile16<f32x4, float, 8>(acc, p, tm * TILE_M + wm * 128u, tn * TILE_N + wn * 128u, lane, lds + wave * OPER_BYTES);
     }
 
     template <Elem E, typename OutT>
-    int launchLayouts(bool aK, bool bK, const Params& p, hipStream_t stream)
+    int launchLayouts(bool aK, bool bK, uint32_t tile, const Params& p, hipStream_t stream)
     {
         const dim3 grid(((p.tilesM * p.tilesN + 7u) / 8u) * 8u), block(THREADS);
         auto launch = [&](auto aKc, auto bKc) {
@@ -990,6 +1018,8 @@ namespace
                 hipLaunchKernelGGL((gemmTiledKernelI8<AK, BK>), grid, block, 0, stream, p);
             else if constexpr(E == Elem::E4M3)
                 hipLaunchKernelGGL((gemmTiledKernelF8<AK, BK>), grid, block, 0, stream, p);
+            else if(tile == 128u)
+                hipLaunchKernelGGL((gemmTiledKernel16Small<E, OutT, AK, BK>), grid, block, 0, stream, p);
             else
                 hipLaunchKernelGGL((gemmTiledKernel16<E, OutT, AK, BK>), grid, block, 0, stream, p);
         };
@@ -1005,6 +1035,38 @@ namespace
             launch(F{}, F{});
         return r355::checkLaunch("gemm (macro tile)");
     }
+
+    // CUs of the current device; where the query fails (no device: plan queries on a build host) MI355X's 256
+    uint32_t computeUnits()
+    {
+        static const uint32_t cus = [] {
+            int dev = 0, n = 0;
+            if(hipGetDevice(&dev) != hipSuccess
+               || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            {
+                (void)hipGetLastError();
+                return 256u;
+            }
+            return static_cast<uint32_t>(n);
+        }();
+        return cus;
+    }
+
+    // Macro tile edge for a problem.  The 128 x 128 tile (16-bit types) is a quarter of the work of the
+    // 256 x 256 one at about 0.55 of its efficiency (measured with one workgroup per CU): it pays when
+    // the large tiles would leave most CUs idle.
+    uint32_t macroTile(const r355_gemm_args& g)
+    {
+        if(g.kernel == R355_KERNEL_TILED)
+            return 256u;
+        if(g.kernel == R355_KERNEL_TILED_128)
+            return 128u;
+        if(r355::dtypeBytes(g.in_type) != 2)
+            return 256u;
+        const uint64_t cus    = computeUnits();
+        auto           rounds = [&](uint32_t t) { return ((uint64_t)((g.m + t - 1) / t) * ((g.n + t - 1) / t) + cus - 1) / cus; };
+        return rounds(128u) * 5u < rounds(256u) * 11u ? 128u : 256u;
+    }
 } // namespace
 
 namespace r355
@@ -1018,6 +1080,9 @@ namespace r355
         if(!pairOk)
             return fail(R355_ERR_UNSUPPORTED, "tiled gemm: no kernel for in_type %d -> out_type %d", g.in_type, g.out_type);
         const uint32_t es = dtypeBytes(g.in_type), os = dtypeBytes(g.out_type);
+        const uint32_t tile = macroTile(g);
+        if(tile == 128u && es != 2)
+            return fail(R355_ERR_UNSUPPORTED, "tiled gemm: the 128 x 128 macro tile takes 16-bit operands only");
         if(g.beta != 0.0f && g.layout_c != g.layout_d)
             return fail(R355_ERR_UNSUPPORTED, "tiled gemm: C and D must share an orientation");
         const uint32_t tk = STAGE_KB / es;
@@ -1032,14 +1097,14 @@ namespace r355
         if(plan)
         {
             plan->kernel       = R355_KERNEL_TILED;
-            plan->macro_tile_m = TILE_M;
-            plan->macro_tile_n = TILE_N;
+            plan->macro_tile_m = tile;
+            plan->macro_tile_n = tile;
             plan->macro_tile_k = tk;
-            plan->grid_x       = ((((g.m + TILE_M - 1) / TILE_M) * ((g.n + TILE_N - 1) / TILE_N) + 7u) / 8u) * 8u;
+            plan->grid_x       = ((((g.m + tile - 1) / tile) * ((g.n + tile - 1) / tile) + 7u) / 8u) * 8u;
             plan->grid_y       = 1;
             plan->block_x      = THREADS;
             plan->block_y      = 1;
-            plan->lds_bytes    = fiveBuffers ? 5u * OPER_BYTES : NUM_STAGES * STAGE_BYTES;
+            plan->lds_bytes    = fiveBuffers ? 5u * OPER_BYTES : NUM_STAGES * STAGE_BYTES * tile / 256u;
         }
         return R355_OK;
     }
@@ -1070,17 +1135,18 @@ namespace r355
             p.lda = g.ldb, p.ldb = g.lda;
             aK = g.layout_b == R355_COL_MAJOR, bK = g.layout_a == R355_ROW_MAJOR;
         }
-        p.tilesM = (p.m + TILE_M - 1) / TILE_M, p.tilesN = (p.n + TILE_N - 1) / TILE_N;
+        const uint32_t tile = macroTile(g);
+        p.tilesM = (p.m + tile - 1) / tile, p.tilesN = (p.n + tile - 1) / tile;
         switch(g.in_type)
         {
         case R355_F16:
-            return g.out_type == R355_F16 ? launchLayouts<Elem::F16, _Float16>(aK, bK, p, stream)
-                                          : launchLayouts<Elem::F16, float>(aK, bK, p, stream);
+            return g.out_type == R355_F16 ? launchLayouts<Elem::F16, _Float16>(aK, bK, tile, p, stream)
+                                          : launchLayouts<Elem::F16, float>(aK, bK, tile, p, stream);
         case R355_BF16:
-            return g.out_type == R355_BF16 ? launchLayouts<Elem::BF16, __bf16>(aK, bK, p, stream)
-                                           : launchLayouts<Elem::BF16, float>(aK, bK, p, stream);
-        case R355_E4M3: return launchLayouts<Elem::E4M3, float>(aK, bK, p, stream);
-        case R355_I8: return launchLayouts<Elem::I8, int>(aK, bK, p, stream);
+            return g.out_type == R355_BF16 ? launchLayouts<Elem::BF16, __bf16>(aK, bK, tile, p, stream)
+                                           : launchLayouts<Elem::BF16, float>(aK, bK, tile, p, stream);
+        case R355_E4M3: return launchLayouts<Elem::E4M3, float>(aK, bK, tile, p, stream);
+        case R355_I8: return launchLayouts<Elem::I8, int>(aK, bK, tile, p, stream);
         default: return fail(R355_ERR_UNSUPPORTED, "tiled gemm: unknown in_type %d", g.in_type);
         }
     }

@@ -50,6 +50,16 @@ def test_query_selects_kernel_family_and_reports_launch_shape():
     # int8: 128 elements of K per stage
     plan = R.gemm_query(_args(in_type=R.I8, out_type=R.I32, m=512, n=256, k=1024, layout_a=R.ROW_MAJOR, layout_b=R.COL_MAJOR))
     assert plan.kernel == R.KERNEL_TILED and plan.macro_tile_k == 128 and plan.grid_x == 8
+    # 16-bit problems whose 256 x 256 tiles would leave most of the 256 CUs idle take the 128 x 128 tile
+    plan = R.gemm_query(_args(m=2048, n=2048, k=2048))
+    assert plan.kernel == R.KERNEL_TILED and (plan.macro_tile_m, plan.macro_tile_n) == (128, 128)
+    assert plan.grid_x == 256 and plan.lds_bytes == 65536
+    plan = R.gemm_query(_args(m=4096, n=4096, k=4096))
+    assert (plan.macro_tile_m, plan.grid_x) == (256, 256)
+    plan = R.gemm_query(_args(m=2048, n=2048, k=2048, kernel=R.KERNEL_TILED))
+    assert (plan.macro_tile_m, plan.grid_x) == (256, 64)
+    plan = R.gemm_query(_args(m=8192, n=8192, k=256, kernel=R.KERNEL_TILED_128))
+    assert (plan.macro_tile_m, plan.grid_x) == (128, 4096)
     # shapes that do not fill a macro tile fall back to one block per wave
     plan = R.gemm_query(_args(m=64, n=48, k=80, a=0x1000))
     assert plan.kernel == R.KERNEL_SIMPLE and plan.lds_bytes == 0 and plan.macro_tile_m == 32
@@ -64,6 +74,9 @@ def test_query_selects_kernel_family_and_reports_launch_shape():
     (dict(k=24), -3),
     (dict(kernel=R.KERNEL_TILED, m=120), -3),
     (dict(kernel=R.KERNEL_TILED, k=192), -3),
+    (dict(kernel=R.KERNEL_TILED_128, m=120), -3),
+    (dict(kernel=R.KERNEL_TILED_128, in_type=R.I8, out_type=R.I32, layout_a=R.ROW_MAJOR, layout_b=R.COL_MAJOR), -2),
+    (dict(kernel=4), -1),
     (dict(a=0x1002, layout_a=R.ROW_MAJOR), -4),
     (dict(lda=8), -1),
 ])

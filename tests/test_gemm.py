@@ -151,6 +151,72 @@ def test_tiled_kernel_16bit_layouts(in_t, out_t, la, lb, ldl):
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("in_t,out_t", [(O.F16, O.F16), (O.F16, O.F32), (O.BF16, O.BF16), (O.BF16, O.F32)])
+@pytest.mark.parametrize("la,lb", TILED_LAYOUTS_16)
+@pytest.mark.parametrize("ldl", [O.ROW, O.COL])
+def test_small_tile_kernel_16bit_layouts(in_t, out_t, la, lb, ldl):
+    # the 128 x 128 macro tile (wave tile 4 x 4 blocks): 3 x 2 tiles
+    m, n, k = 384, 256, 384
+    a, b, c = _inputs(in_t, out_t, m, n, k, seed=12)
+    want = O.gemm(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, c, 2.0, 2.0)
+    got = _run(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, c, 2.0, 2.0, R.KERNEL_TILED_128)
+    w32 = None
+    if out_t != O.F32:
+        w32 = O.gemm(in_t, O.F32, la, lb, ldl, ldl, m, n, k, a, b, O.storage_to_f32(c, out_t), 2.0, 2.0)
+    _check(in_t, out_t, got, want, w32)
+    a, b = O.fill_ref(in_t, m, k, la), O.fill_ref(in_t, k, n, lb)
+    want = O.gemm(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, None, 1.0, 0.0)
+    got = _run(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, None, 1.0, 0.0, R.KERNEL_TILED_128)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("la,lb", TILED_LAYOUTS_16)
+@pytest.mark.parametrize("kernel", ["tiled", "tiled_128"])
+def test_tiled_kernel_16bit_one_hot_operands(la, lb, kernel):
+    # one non-zero in A and one in B: exactly one element of D, for both tile sizes and every orientation
+    m, n, k = 256, 256, 128
+    rng = np.random.default_rng(6)
+    sel = R.KERNEL_TILED if kernel == "tiled" else R.KERNEL_TILED_128
+    for _ in range(6):
+        i, j, h = int(rng.integers(m)), int(rng.integers(n)), int(rng.integers(k))
+        a = np.zeros(m * k, np.float16)
+        b = np.zeros(k * n, np.float16)
+        a[i * k + h if la == O.ROW else h * m + i] = 3
+        b[h * n + j if lb == O.ROW else j * k + h] = 5
+        got = _run(O.F16, O.F32, la, lb, O.ROW, O.ROW, m, n, k, a.view(np.uint16), b.view(np.uint16), None, 1.0, 0.0, sel)
+        want = np.zeros((m, n), np.float32)
+        want[i, j] = 15
+        assert np.array_equal(got.reshape(m, n), want), (i, j, h)
+
+
+@pytest.mark.parametrize("in_t,out_t", [(O.F16, O.F16), (O.BF16, O.F32)])
+@pytest.mark.parametrize("la,lb", [(O.COL, O.ROW), (O.ROW, O.COL)])
+@pytest.mark.parametrize("m,n,k", [(272, 304, 256), (16, 528, 128), (1008, 16, 384), (144, 112, 640)])
+def test_small_tile_kernel_edge_tiles_and_stage_counts(in_t, out_t, la, lb, m, n, k):
+    a, b, c = _inputs(in_t, out_t, m, n, k, seed=75 + m)
+    for alpha, beta in ((1.0, 0.0), (2.0, 2.0)):
+        cc = None if beta == 0.0 else c
+        want = O.gemm(in_t, out_t, la, lb, O.ROW, O.ROW, m, n, k, a, b, cc, alpha, beta)
+        got = _run(in_t, out_t, la, lb, O.ROW, O.ROW, m, n, k, a, b, cc, alpha, beta, R.KERNEL_TILED_128)
+        w32 = None
+        if out_t != O.F32:
+            c32 = None if cc is None else O.storage_to_f32(cc, out_t)
+            w32 = O.gemm(in_t, O.F32, la, lb, O.ROW, O.ROW, m, n, k, a, b, c32, alpha, beta)
+        _check(in_t, out_t, got, want, w32)
+
+
+def test_auto_takes_the_small_tile_for_few_tile_problems():
+    # 1024 x 768 has 12 tiles of 256 x 256 on 256 CUs: AUTO must resolve to the 128 x 128 tile and agree with the oracle
+    m, n, k = 1024, 768, 512
+    a, b, _ = _inputs(O.F16, O.F16, m, n, k, seed=77)
+    g = R.gemm_args(R.F16, R.F16, m, n, k, 0x1000, 0x2000, None, 0x3000, 1.0, 0.0, O.COL, O.ROW, O.ROW, O.ROW)
+    assert R.gemm_query(g).macro_tile_m == 128
+    want = O.gemm(O.F16, O.F16, O.COL, O.ROW, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0)
+    got = _run(O.F16, O.F16, O.COL, O.ROW, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0, R.KERNEL_AUTO)
+    w32 = O.gemm(O.F16, O.F32, O.COL, O.ROW, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0)
+    _check(O.F16, O.F16, got, want, w32)
+
+
 @pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32)])
 @pytest.mark.parametrize("la,lb", TILED_LAYOUTS_16)
 @pytest.mark.parametrize("ldl", [O.ROW, O.COL])
