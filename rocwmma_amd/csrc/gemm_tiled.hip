@@ -546,9 +546,13 @@ namespace
     {
         return (row >> 1) & 7u;
     }
+    template <uint32_t WB>
     __device__ __forceinline__ uint32_t swzMN8(uint32_t krow)
     {
-        return (krow & 7u) | ((krow >> 1) & 8u);
+        if constexpr(WB == 8)
+            return (krow & 7u) | ((krow >> 1) & 8u); // 256-byte k-rows, 16 chunks
+        else
+            return ((krow >> 1) & 3u) | ((krow >> 2) & 4u); // 128-byte k-rows, 8 chunks: rows 2 apart share banks
     }
 
     // global -> LDS lane offsets of one operand: load j brings chunk j * 256 + tid.  Edge tiles (m or
@@ -556,15 +560,15 @@ namespace
     // chunk (M/N-contiguous) lies beyond the matrix reads the last valid row / the first chunk instead;
     // what lands in LDS for it only feeds elements of D that are never stored.  `step` is the uniform
     // offset from one load to the next, `stage` the distance between K stages.
-    template <bool KCONTIG>
-    __device__ __forceinline__ void laneOffsets8(uint32_t tid, uint32_t ld, uint32_t valid, uint32_t (&off)[LOADS_PER_OPER],
-                                                 uint32_t& step, uint64_t& stage)
+    template <bool KCONTIG, uint32_t WB>
+    __device__ __forceinline__ void laneOffsets8(uint32_t tid, uint32_t ld, uint32_t valid, uint32_t (&off)[WB], uint32_t& step,
+                                                 uint64_t& stage)
     {
         if constexpr(KCONTIG)
         {
             const uint32_t r = tid >> 3, slot = tid & 7u; // row 32 j + r
 #pragma unroll
-            for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
+            for(uint32_t j = 0; j < WB; ++j)
             {
                 const uint32_t row = r + 32u * j < valid ? r + 32u * j : valid - 1u;
                 off[j]             = row * ld + ((slot ^ swzK8(r)) * CHUNK);
@@ -573,21 +577,22 @@ namespace
         }
         else
         {
-            const uint32_t r = tid >> 4, slot = tid & 15u; // k-row 16 j + r: the swizzle alternates with j
+            constexpr uint32_t SLOTS = 2u * WB, KROWS = THREADS / SLOTS; // chunks per k-row, k-rows per load
+            const uint32_t     r = tid / SLOTS, slot = tid % SLOTS; // k-row KROWS j + r (256-byte rows: the swizzle alternates with j)
 #pragma unroll
-            for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
+            for(uint32_t j = 0; j < WB; ++j)
             {
-                const uint32_t c = slot ^ swzMN8(16u * j + r);
+                const uint32_t c = slot ^ swzMN8<WB>(KROWS * j + r);
                 off[j]           = r * ld + (c * CHUNK < valid ? c : 0u) * CHUNK;
             }
-            step = 16u * ld, stage = (uint64_t)STAGE_KB * ld;
+            step = KROWS * ld, stage = (uint64_t)STAGE_KB * ld;
         }
     }
 
-    // LDS -> register lane offsets of one operand for the wave whose tile starts at row 128 w.
+    // LDS -> register lane offsets of one operand for the wave whose tile starts at row 16 WB w.
     // K-contiguous: rd[q] is 64-byte K step q of block 0 (block i is 16 rows further);
     // M/N-contiguous: rd[i] is block i, the first 8 k-rows of the lane's 16 of K step 0.
-    template <bool KCONTIG>
+    template <bool KCONTIG, uint32_t WB>
     __device__ __forceinline__ void readOffsets8(uint32_t w, uint32_t lane, uint32_t (&rd)[8])
     {
         const uint32_t t = lane & 15u, g = lane >> 4;
@@ -596,7 +601,7 @@ namespace
             rd[i] = 0u;
         if constexpr(KCONTIG)
         {
-            const uint32_t r = w * 128u + t;
+            const uint32_t r = w * 16u * WB + t;
             rd[0]            = r * STAGE_KB + ((g ^ swzK8(r)) * CHUNK);
             rd[1]            = r * STAGE_KB + (((4u + g) ^ swzK8(r)) * CHUNK);
         }
@@ -604,15 +609,15 @@ namespace
         {
             const uint32_t kr = 16u * g + (t >> 1);
 #pragma unroll
-            for(uint32_t i = 0; i < 8; ++i)
-                rd[i] = kr * 256u + (((w * 8u + i) ^ swzMN8(kr)) * CHUNK) + (t & 1u) * 8u;
+            for(uint32_t i = 0; i < WB; ++i)
+                rd[i] = kr * 32u * WB + (((w * WB + i) ^ swzMN8<WB>(kr)) * CHUNK) + (t & 1u) * 8u;
         }
     }
 
     // 16 K bytes of block i, K step s (64 bytes), of the operand tile at `tile`: they arrive whole with
     // part 0 (K-contiguous) or as two transposed halves, parts 0 and 1, into registers at, at + 1 and
     // at + 2, at + 3 of `dst`
-    template <bool KCONTIG, typename V>
+    template <bool KCONTIG, uint32_t WB, typename V>
     __device__ __forceinline__ void readBlock8(const char* tile, const uint32_t (&rd)[8], uint32_t i, uint32_t s, uint32_t part,
                                                V& dst, uint32_t at)
     {
@@ -627,7 +632,7 @@ namespace
         else
         {
             using lp      = __attribute__((address_space(3))) i32x2*;
-            const i32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lp)(tile + rd[i] + (64u * s + 8u * part) * 256u));
+            const i32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lp)(tile + rd[i] + (64u * s + 8u * part) * 32u * WB));
             dst[at + 2u * part] = v[0], dst[at + 2u * part + 1u] = v[1];
         }
     }
@@ -642,13 +647,18 @@ namespace
         asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc) : "v"(x), "v"(y));
     }
 
-    template <bool A_KCONTIG, bool B_KCONTIG>
-    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) gemmTiledKernelI8(Params p)
+    template <bool A_KCONTIG, bool B_KCONTIG, uint32_t WB>
+    __device__ __forceinline__ void gemmTiledI8(const Params& p)
     {
-        // LDS map: A buffers at 0 and 32 KiB, B buffers at 64, 96 and 128 KiB
-        constexpr uint32_t A_AT[2] = {0u, OPER_BYTES};
-        constexpr uint32_t B_AT[3] = {2u * OPER_BYTES, 3u * OPER_BYTES, 4u * OPER_BYTES};
-        __shared__ __attribute__((aligned(1024))) char lds[5u * OPER_BYTES];
+        static_assert(WB == 8 || WB == 4, "wave tile of 8 x 8 or 4 x 4 blocks");
+        constexpr uint32_t TILE = 32u * WB, WT = 16u * WB; // macro tile and wave tile edge
+        constexpr uint32_t OPER = TILE * STAGE_KB; // bytes of one operand per stage: 32 or 16 KiB
+        constexpr uint32_t XS = 2u * WB, QS = WB / 2u; // operand blocks per K step, matrix instructions per block
+        constexpr uint32_t LOAD_Q = QS > 2u ? 2u : QS - 1u;
+        // LDS map: A buffers at 0 and OPER, B buffers at 2, 3 and 4 OPER
+        constexpr uint32_t A_AT[2] = {0u, OPER};
+        constexpr uint32_t B_AT[3] = {2u * OPER, 3u * OPER, 4u * OPER};
+        __shared__ __attribute__((aligned(1024))) char lds[5u * OPER];
 
         uint32_t tm, tn;
         if(!r355::tileCoord(blockIdx.x, p.tilesM, p.tilesN, tm, tn))
@@ -661,12 +671,12 @@ namespace
         const uint32_t ldsBase
             = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds));
 
-        uint32_t       gOffA[LOADS_PER_OPER], gOffB[LOADS_PER_OPER], gStepA, gStepB;
+        uint32_t       gOffA[WB], gOffB[WB], gStepA, gStepB; // WB direct loads per operand per stage
         uint64_t       gStageA, gStageB;
-        const uint32_t validM = p.m - tm * TILE_M < TILE_M ? p.m - tm * TILE_M : TILE_M;
-        const uint32_t validN = p.n - tn * TILE_N < TILE_N ? p.n - tn * TILE_N : TILE_N;
-        laneOffsets8<A_KCONTIG>(tid, p.lda, validM, gOffA, gStepA, gStageA);
-        laneOffsets8<B_KCONTIG>(tid, p.ldb, validN, gOffB, gStepB, gStageB);
+        const uint32_t validM = p.m - tm * TILE < TILE ? p.m - tm * TILE : TILE;
+        const uint32_t validN = p.n - tn * TILE < TILE ? p.n - tn * TILE : TILE;
+        laneOffsets8<A_KCONTIG, WB>(tid, p.lda, validM, gOffA, gStepA, gStageA);
+        laneOffsets8<B_KCONTIG, WB>(tid, p.ldb, validN, gOffB, gStepB, gStageB);
         const uint32_t numStages = p.k / STAGE_KB;
         const uint32_t dmaDst    = ldsBase + wave * 64u * CHUNK; // + buffer + j * 4 KiB
         auto           uniform64 = [](const char* ptr) {
@@ -675,8 +685,8 @@ namespace
             const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
             return (static_cast<uint64_t>(hi) << 32) | lo;
         };
-        const uint64_t gA = uniform64(p.a + (A_KCONTIG ? (uint64_t)tm * TILE_M * p.lda : (uint64_t)tm * TILE_M));
-        const uint64_t gB = uniform64(p.b + (B_KCONTIG ? (uint64_t)tn * TILE_N * p.ldb : (uint64_t)tn * TILE_N));
+        const uint64_t gA = uniform64(p.a + (A_KCONTIG ? (uint64_t)tm * TILE * p.lda : (uint64_t)tm * TILE));
+        const uint64_t gB = uniform64(p.b + (B_KCONTIG ? (uint64_t)tn * TILE * p.ldb : (uint64_t)tn * TILE));
         auto rsrcAt = [](uint64_t addr) { // raw buffer over a stage of an operand panel
             return i32x4{static_cast<int>(static_cast<uint32_t>(addr)), static_cast<int>(static_cast<uint32_t>(addr >> 32) & 0xFFFFu),
                          0x7FFFFFFF, 0x00020000};
@@ -684,25 +694,25 @@ namespace
         auto stageAddr = [&](uint64_t panel, uint64_t perStage, uint32_t stage) { // clamped to the last stage
             return panel + (uint64_t)(stage < numStages ? stage : numStages - 1u) * perStage;
         };
-        auto issueHalf = [&](uint64_t addr, const uint32_t (&gOff)[LOADS_PER_OPER], uint32_t step, uint32_t at) {
+        auto issueHalf = [&](uint64_t addr, const uint32_t (&gOff)[WB], uint32_t step, uint32_t at) {
             const i32x4 rsrc = rsrcAt(addr);
 #pragma unroll
-            for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
+            for(uint32_t j = 0; j < WB; ++j)
                 loadToLds(rsrc, gOff[j], j * step, dmaDst + at + j * THREADS * CHUNK);
         };
 
         uint32_t rdA[8], rdB[8];
-        readOffsets8<A_KCONTIG>(wm, lane, rdA);
-        readOffsets8<B_KCONTIG>(wn, lane, rdB);
+        readOffsets8<A_KCONTIG, WB>(wm, lane, rdA);
+        readOffsets8<B_KCONTIG, WB>(wn, lane, rdB);
 
-        i32x4v acc[8][8];
+        i32x4v acc[WB][WB];
 #pragma unroll
-        for(uint32_t i = 0; i < 8; ++i)
+        for(uint32_t i = 0; i < WB; ++i)
 #pragma unroll
-            for(uint32_t j = 0; j < 8; ++j)
+            for(uint32_t j = 0; j < WB; ++j)
                 acc[i][j] = i32x4v{0, 0, 0, 0};
 
-        i32x4 fa[2][8], fb[2][8];
+        i32x4 fa[2][WB], fb[2][WB];
         // matrix instruction n of a K step: L-shaped shells, as in gemmTiledKernel16
         auto mfmaAt = [&](uint32_t s, uint32_t n) {
             uint32_t d = 0;
@@ -715,29 +725,29 @@ namespace
         // operand block x of K step s: x = 2 i is A block i, x = 2 i + 1 is B block i
         auto readAt = [&](uint32_t aAt, uint32_t bAt, uint32_t s, uint32_t x, uint32_t part) {
             if(x & 1u)
-                readBlock8<B_KCONTIG>(lds + bAt, rdB, x >> 1, s, part, fb[s][x >> 1], 0u);
+                readBlock8<B_KCONTIG, WB>(lds + bAt, rdB, x >> 1, s, part, fb[s][x >> 1], 0u);
             else
-                readBlock8<A_KCONTIG>(lds + aAt, rdA, x >> 1, s, part, fa[s][x >> 1], 0u);
+                readBlock8<A_KCONTIG, WB>(lds + aAt, rdA, x >> 1, s, part, fa[s][x >> 1], 0u);
         };
 
         uint64_t refillA, refillB; // stage kt + 2 of A, stage kt + 3 of B (clamped)
         // One K stage: K step 0 is in registers; step 1 arrives under its matrix instructions; then the
         // stage's buffers are refilled (A two stages ahead, B three) while step 0 of the next stage
-        // arrives under the matrix instructions of step 1.  Per four matrix instructions: one operand
-        // block read (two reads when it is transposed on the way) and, in the second half, one direct
-        // load; nothing moves between the pieces.
+        // arrives under the matrix instructions of step 1.  Per four (small wave tile: two) matrix
+        // instructions: one operand block read (two reads when it is transposed on the way) and, in the
+        // second half, one direct load; nothing moves between the pieces.
         auto stageBody = [&](uint32_t kt, uint32_t aCur, uint32_t aNxt, uint32_t bCur, uint32_t bNxt) {
 #pragma unroll
-            for(uint32_t x = 0; x < 16; ++x)
+            for(uint32_t x = 0; x < XS; ++x)
 #pragma unroll
-                for(uint32_t q = 0; q < 4; ++q)
+                for(uint32_t q = 0; q < QS; ++q)
                 {
-                    mfmaAt(0, 4u * x + q);
+                    mfmaAt(0, QS * x + q);
                     if(q < 2u)
                         readAt(aCur, bCur, 1, x, q);
                     __builtin_amdgcn_sched_barrier(0);
                 }
-            waitVmcnt<8>(); // this wave's part of stage kt + 1 has landed (the youngest 8 loads are B of kt + 2)
+            waitVmcnt<WB>(); // this wave's part of stage kt + 1 has landed (the youngest WB loads are B of kt + 2)
             ldsBarrier();
             const i32x4 rsrcA = rsrcAt(refillA), rsrcB = rsrcAt(refillB);
             if(kt + 3u < numStages)
@@ -745,19 +755,19 @@ namespace
             if(kt + 4u < numStages)
                 refillB += gStageB;
 #pragma unroll
-            for(uint32_t x = 0; x < 16; ++x)
+            for(uint32_t x = 0; x < XS; ++x)
 #pragma unroll
-                for(uint32_t q = 0; q < 4; ++q)
+                for(uint32_t q = 0; q < QS; ++q)
                 {
-                    mfmaAt(1, 4u * x + q);
+                    mfmaAt(1, QS * x + q);
                     if(q < 2u)
                         readAt(aNxt, bNxt, 0, x, q);
-                    if(q == 2u)
+                    if(q == LOAD_Q)
                     {
-                        if(x < 8u)
+                        if(x < WB)
                             loadToLds(rsrcA, gOffA[x], x * gStepA, dmaDst + aCur + x * THREADS * CHUNK);
                         else
-                            loadToLds(rsrcB, gOffB[x - 8u], (x - 8u) * gStepB, dmaDst + bCur + (x - 8u) * THREADS * CHUNK);
+                            loadToLds(rsrcB, gOffB[x - WB], (x - WB) * gStepB, dmaDst + bCur + (x - WB) * THREADS * CHUNK);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -770,10 +780,10 @@ namespace
         issueHalf(stageAddr(gB, gStageB, 1u), gOffB, gStepB, B_AT[1]);
         issueHalf(stageAddr(gB, gStageB, 2u), gOffB, gStepB, B_AT[2]);
         refillA = stageAddr(gA, gStageA, 2u), refillB = stageAddr(gB, gStageB, 3u);
-        waitVmcnt<24>();
+        waitVmcnt<3u * WB>();
         ldsBarrier();
 #pragma unroll
-        for(uint32_t x = 0; x < 16; ++x)
+        for(uint32_t x = 0; x < XS; ++x)
         {
             readAt(A_AT[0], B_AT[0], 0, x, 0);
             readAt(A_AT[0], B_AT[0], 0, x, 1);
@@ -815,7 +825,18 @@ namespace
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
         waitVmcnt<0>();
         ldsBarrier();
-        storeTile16<i32x4v, int, 8>(acc, p, tm * TILE_M + wm * 128u, tn * TILE_N + wn * 128u, lane, lds + wave * OPER_BYTES);
+        storeTile16<i32x4v, int, WB>(acc, p, tm * TILE + wm * WT, tn * TILE + wn * WT, lane, lds + wave * (WB * 4096u));
+    }
+
+    template <bool A_KCONTIG, bool B_KCONTIG>
+    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) gemmTiledKernelI8(Params p)
+    {
+        gemmTiledI8<A_KCONTIG, B_KCONTIG, 8>(p);
+    }
+    template <bool A_KCONTIG, bool B_KCONTIG>
+    __global__ void __launch_bounds__(THREADS) gemmTiledKernelI8Small(Params p)
+    {
+        gemmTiledI8<A_KCONTIG, B_KCONTIG, 4>(p);
     }
 
     // ------------------------------------------------------------------------------------------
@@ -837,12 +858,16 @@ namespace
         asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc) : "v"(x), "v"(y));
     }
 
-    template <bool A_KCONTIG, bool B_KCONTIG>
-    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) gemmTiledKernelF8(Params p)
+    template <bool A_KCONTIG, bool B_KCONTIG, uint32_t WB>
+    __device__ __forceinline__ void gemmTiledF8(const Params& p)
     {
-        constexpr uint32_t A_AT[2] = {0u, OPER_BYTES};
-        constexpr uint32_t B_AT[3] = {2u * OPER_BYTES, 3u * OPER_BYTES, 4u * OPER_BYTES};
-        __shared__ __attribute__((aligned(1024))) char lds[5u * OPER_BYTES];
+        static_assert(WB == 8 || WB == 4, "wave tile of 8 x 8 or 4 x 4 blocks");
+        constexpr uint32_t TILE = 32u * WB, WT = 16u * WB; // macro tile and wave tile edge
+        constexpr uint32_t OPER = TILE * STAGE_KB; // bytes of one operand per stage: 32 or 16 KiB
+        constexpr uint32_t H = WB / 2u, NQ = H * H; // blocks per operand group, matrix instructions per quadrant
+        constexpr uint32_t A_AT[2] = {0u, OPER};
+        constexpr uint32_t B_AT[3] = {2u * OPER, 3u * OPER, 4u * OPER};
+        __shared__ __attribute__((aligned(1024))) char lds[5u * OPER];
 
         uint32_t tm, tn;
         if(!r355::tileCoord(blockIdx.x, p.tilesM, p.tilesN, tm, tn))
@@ -855,12 +880,12 @@ namespace
         const uint32_t ldsBase
             = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds));
 
-        uint32_t       gOffA[LOADS_PER_OPER], gOffB[LOADS_PER_OPER], gStepA, gStepB;
+        uint32_t       gOffA[WB], gOffB[WB], gStepA, gStepB; // WB direct loads per operand per stage
         uint64_t       gStageA, gStageB;
-        const uint32_t validM = p.m - tm * TILE_M < TILE_M ? p.m - tm * TILE_M : TILE_M;
-        const uint32_t validN = p.n - tn * TILE_N < TILE_N ? p.n - tn * TILE_N : TILE_N;
-        laneOffsets8<A_KCONTIG>(tid, p.lda, validM, gOffA, gStepA, gStageA);
-        laneOffsets8<B_KCONTIG>(tid, p.ldb, validN, gOffB, gStepB, gStageB);
+        const uint32_t validM = p.m - tm * TILE < TILE ? p.m - tm * TILE : TILE;
+        const uint32_t validN = p.n - tn * TILE < TILE ? p.n - tn * TILE : TILE;
+        laneOffsets8<A_KCONTIG, WB>(tid, p.lda, validM, gOffA, gStepA, gStageA);
+        laneOffsets8<B_KCONTIG, WB>(tid, p.ldb, validN, gOffB, gStepB, gStageB);
         const uint32_t numStages = p.k / STAGE_KB;
         const uint32_t dmaDst    = ldsBase + wave * 64u * CHUNK;
         auto           uniform64 = [](const char* ptr) {
@@ -869,8 +894,8 @@ namespace
             const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
             return (static_cast<uint64_t>(hi) << 32) | lo;
         };
-        const uint64_t gA = uniform64(p.a + (A_KCONTIG ? (uint64_t)tm * TILE_M * p.lda : (uint64_t)tm * TILE_M));
-        const uint64_t gB = uniform64(p.b + (B_KCONTIG ? (uint64_t)tn * TILE_N * p.ldb : (uint64_t)tn * TILE_N));
+        const uint64_t gA = uniform64(p.a + (A_KCONTIG ? (uint64_t)tm * TILE * p.lda : (uint64_t)tm * TILE));
+        const uint64_t gB = uniform64(p.b + (B_KCONTIG ? (uint64_t)tn * TILE * p.ldb : (uint64_t)tn * TILE));
         auto rsrcAt = [](uint64_t addr) {
             return i32x4{static_cast<int>(static_cast<uint32_t>(addr)), static_cast<int>(static_cast<uint32_t>(addr >> 32) & 0xFFFFu),
                          0x7FFFFFFF, 0x00020000};
@@ -878,79 +903,95 @@ namespace
         auto stageAddr = [&](uint64_t panel, uint64_t perStage, uint32_t stage) {
             return panel + (uint64_t)(stage < numStages ? stage : numStages - 1u) * perStage;
         };
-        auto issueHalf = [&](uint64_t addr, const uint32_t (&gOff)[LOADS_PER_OPER], uint32_t step, uint32_t at) {
+        auto issueHalf = [&](uint64_t addr, const uint32_t (&gOff)[WB], uint32_t step, uint32_t at) {
             const i32x4 rsrc = rsrcAt(addr);
 #pragma unroll
-            for(uint32_t j = 0; j < LOADS_PER_OPER; ++j)
+            for(uint32_t j = 0; j < WB; ++j)
                 loadToLds(rsrc, gOff[j], j * step, dmaDst + at + j * THREADS * CHUNK);
         };
 
         uint32_t rdA[8], rdB[8];
-        readOffsets8<A_KCONTIG>(wm, lane, rdA);
-        readOffsets8<B_KCONTIG>(wn, lane, rdB);
-        // Slot n (0..15) of a quadrant brings a piece of the operand group that holds blocks 4 half .. + 3:
-        // K-contiguous: even slots, 16 bytes -- block n / 4, 64-byte half (n / 2) % 2;
-        // M/N-contiguous: every slot, 8 transposed bytes -- same block and half, part n % 2.
-        auto readSlotA = [&](i32x8 (&grp)[4], uint32_t at, uint32_t half, uint32_t n) {
-            readBlock8<A_KCONTIG>(lds + at, rdA, 4u * half + (n >> 2), (n >> 1) & 1u, n & 1u, grp[n >> 2], 4u * ((n >> 1) & 1u));
+        readOffsets8<A_KCONTIG, WB>(wm, lane, rdA);
+        readOffsets8<B_KCONTIG, WB>(wn, lane, rdB);
+        // An operand group (blocks H half .. + H - 1) arrives in 2 H pieces of 16 bytes (K-contiguous:
+        // piece r is block r / 2, 64-byte half r % 2) or 4 H transposed pieces of 8 bytes (block r / 4,
+        // half (r / 2) % 2, part r % 2), dealt out evenly over the NQ slots of a quadrant.
+        auto readSlotA = [&](i32x8 (&grp)[H], uint32_t at, uint32_t half, uint32_t n) {
+            constexpr uint32_t P = A_KCONTIG ? 2u * H : 4u * H;
+#pragma unroll
+            for(uint32_t r = (n * P + NQ - 1u) / NQ; r < ((n + 1u) * P + NQ - 1u) / NQ; ++r)
+            {
+                const uint32_t b = A_KCONTIG ? r >> 1 : r >> 2, kh = A_KCONTIG ? r & 1u : (r >> 1) & 1u, part = A_KCONTIG ? 0u : r & 1u;
+                readBlock8<A_KCONTIG, WB>(lds + at, rdA, H * half + b, kh, part, grp[b], 4u * kh);
+            }
         };
-        auto readSlotB = [&](i32x8 (&grp)[4], uint32_t at, uint32_t half, uint32_t n) {
-            readBlock8<B_KCONTIG>(lds + at, rdB, 4u * half + (n >> 2), (n >> 1) & 1u, n & 1u, grp[n >> 2], 4u * ((n >> 1) & 1u));
+        auto readSlotB = [&](i32x8 (&grp)[H], uint32_t at, uint32_t half, uint32_t n) {
+            constexpr uint32_t P = B_KCONTIG ? 2u * H : 4u * H;
+#pragma unroll
+            for(uint32_t r = (n * P + NQ - 1u) / NQ; r < ((n + 1u) * P + NQ - 1u) / NQ; ++r)
+            {
+                const uint32_t b = B_KCONTIG ? r >> 1 : r >> 2, kh = B_KCONTIG ? r & 1u : (r >> 1) & 1u, part = B_KCONTIG ? 0u : r & 1u;
+                readBlock8<B_KCONTIG, WB>(lds + at, rdB, H * half + b, kh, part, grp[b], 4u * kh);
+            }
+        };
+        // direct load j of an operand goes out in slot n when [n WB / NQ, (n + 1) WB / NQ) contains j
+        auto loadSlot = [&](const i32x4& rsrc, const uint32_t (&gOff)[WB], uint32_t step, uint32_t at, uint32_t n) {
+#pragma unroll
+            for(uint32_t j = n * WB / NQ; j < (n + 1u) * WB / NQ; ++j)
+                loadToLds(rsrc, gOff[j], j * step, dmaDst + at + j * THREADS * CHUNK);
         };
 
-        f32x4 acc[8][8];
+        f32x4 acc[WB][WB];
 #pragma unroll
-        for(uint32_t i = 0; i < 8; ++i)
+        for(uint32_t i = 0; i < WB; ++i)
 #pragma unroll
-            for(uint32_t j = 0; j < 8; ++j)
+            for(uint32_t j = 0; j < WB; ++j)
                 acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-        i32x8 aLo[4], aHi[4], bX[4], bY[4]; // bX / bY alternate as B[0..3] / B[4..7]
+        i32x8 aLo[H], aHi[H], bX[H], bY[H]; // bX / bY alternate as the low / high half of B's blocks
 
         uint64_t refillA, refillB; // stage kt + 2 of A, stage kt + 3 of B (clamped)
-        auto stageBody = [&](uint32_t kt, uint32_t aCur, uint32_t aNxt, uint32_t bCur, uint32_t bNxt, i32x8 (&bLo)[4],
-                             i32x8 (&bHi)[4]) {
-            // Q1: A[0..3] x B[0..3]; B[4..7] arrives
+        auto stageBody = [&](uint32_t kt, uint32_t aCur, uint32_t aNxt, uint32_t bCur, uint32_t bNxt, i32x8 (&bLo)[H],
+                             i32x8 (&bHi)[H]) {
+            // Q1: A low x B low; B high arrives
 #pragma unroll
-            for(uint32_t n = 0; n < 16; ++n)
+            for(uint32_t n = 0; n < NQ; ++n)
             {
-                mfma16f8(acc[n & 3u][n >> 2], bLo[n >> 2], aLo[n & 3u]);
+                mfma16f8(acc[n % H][n / H], bLo[n / H], aLo[n % H]);
                 readSlotB(bHi, bCur, 1, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            // Q2: A[0..3] x B[4..7] (column by column, in the order B arrived); A[4..7] arrives
+            // Q2: A low x B high (column by column, in the order B arrived); A high arrives
 #pragma unroll
-            for(uint32_t n = 0; n < 16; ++n)
+            for(uint32_t n = 0; n < NQ; ++n)
             {
-                mfma16f8(acc[n & 3u][4u + (n >> 2)], bHi[n >> 2], aLo[n & 3u]);
+                mfma16f8(acc[n % H][H + n / H], bHi[n / H], aLo[n % H]);
                 readSlotA(aHi, aCur, 1, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            waitVmcnt<8>(); // this wave's part of stage kt + 1 has landed (the youngest 8 loads are B of kt + 2)
+            waitVmcnt<WB>(); // this wave's part of stage kt + 1 has landed (the youngest WB loads are B of kt + 2)
             ldsBarrier();
             const i32x4 rsrcA = rsrcAt(refillA), rsrcB = rsrcAt(refillB);
             if(kt + 3u < numStages)
                 refillA += gStageA;
             if(kt + 4u < numStages)
                 refillB += gStageB;
-            // Q3: A[4..7] x B[4..7] (row by row, in the order A arrived); next A[0..3] arrives; A refill
+            // Q3: A high x B high (row by row, in the order A arrived); next A low arrives; A refill
 #pragma unroll
-            for(uint32_t n = 0; n < 16; ++n)
+            for(uint32_t n = 0; n < NQ; ++n)
             {
-                mfma16f8(acc[4u + (n >> 2)][4u + (n & 3u)], bHi[n & 3u], aHi[n >> 2]);
+                mfma16f8(acc[H + n / H][H + n % H], bHi[n % H], aHi[n / H]);
                 readSlotA(aLo, aNxt, 0, n);
-                if(n & 1u)
-                    loadToLds(rsrcA, gOffA[n >> 1], (n >> 1) * gStepA, dmaDst + aCur + (n >> 1) * THREADS * CHUNK);
+                loadSlot(rsrcA, gOffA, gStepA, aCur, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            // Q4: A[4..7] x B[0..3]; next B[0..3] arrives in the registers B[4..7] has left; B refill
+            // Q4: A high x B low; next B low arrives in the registers B high has left; B refill
 #pragma unroll
-            for(uint32_t n = 0; n < 16; ++n)
+            for(uint32_t n = 0; n < NQ; ++n)
             {
-                mfma16f8(acc[4u + (n & 3u)][n >> 2], bLo[n >> 2], aHi[n & 3u]);
+                mfma16f8(acc[H + n % H][n / H], bLo[n / H], aHi[n % H]);
                 readSlotB(bHi, bNxt, 0, n);
-                if(n & 1u)
-                    loadToLds(rsrcB, gOffB[n >> 1], (n >> 1) * gStepB, dmaDst + bCur + (n >> 1) * THREADS * CHUNK);
+                loadSlot(rsrcB, gOffB, gStepB, bCur, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
@@ -962,10 +1003,10 @@ namespace
         issueHalf(stageAddr(gB, gStageB, 1u), gOffB, gStepB, B_AT[1]);
         issueHalf(stageAddr(gB, gStageB, 2u), gOffB, gStepB, B_AT[2]);
         refillA = stageAddr(gA, gStageA, 2u), refillB = stageAddr(gB, gStageB, 3u);
-        waitVmcnt<24>();
+        waitVmcnt<3u * WB>();
         ldsBarrier();
 #pragma unroll
-        for(uint32_t n = 0; n < 16; ++n)
+        for(uint32_t n = 0; n < NQ; ++n)
         {
             readSlotA(aLo, A_AT[0], 0, n);
             readSlotB(bX, B_AT[0], 0, n);
@@ -1005,7 +1046,18 @@ namespace
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); // the last matrix instructions are still in the pipeline
         waitVmcnt<0>();
         ldsBarrier();
-        storeTile16<f32x4, float, 8>(acc, p, tm * TILE_M + wm * 128u, tn * TILE_N + wn * 128u, lane, lds + wave * OPER_BYTES);
+        storeTile16<f32x4, float, WB>(acc, p, tm * TILE + wm * WT, tn * TILE + wn * WT, lane, lds + wave * (WB * 4096u));
+    }
+
+    template <bool A_KCONTIG, bool B_KCONTIG>
+    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) gemmTiledKernelF8(Params p)
+    {
+        gemmTiledF8<A_KCONTIG, B_KCONTIG, 8>(p);
+    }
+    template <bool A_KCONTIG, bool B_KCONTIG>
+    __global__ void __launch_bounds__(THREADS) gemmTiledKernelF8Small(Params p)
+    {
+        gemmTiledF8<A_KCONTIG, B_KCONTIG, 4>(p);
     }
 
     template <Elem E, typename OutT>
@@ -1015,9 +1067,19 @@ namespace
         auto launch = [&](auto aKc, auto bKc) {
             constexpr bool AK = decltype(aKc)::value, BK = decltype(bKc)::value;
             if constexpr(E == Elem::I8)
-                hipLaunchKernelGGL((gemmTiledKernelI8<AK, BK>), grid, block, 0, stream, p);
+            {
+                if(tile == 128u)
+                    hipLaunchKernelGGL((gemmTiledKernelI8Small<AK, BK>), grid, block, 0, stream, p);
+                else
+                    hipLaunchKernelGGL((gemmTiledKernelI8<AK, BK>), grid, block, 0, stream, p);
+            }
             else if constexpr(E == Elem::E4M3)
-                hipLaunchKernelGGL((gemmTiledKernelF8<AK, BK>), grid, block, 0, stream, p);
+            {
+                if(tile == 128u)
+                    hipLaunchKernelGGL((gemmTiledKernelF8Small<AK, BK>), grid, block, 0, stream, p);
+                else
+                    hipLaunchKernelGGL((gemmTiledKernelF8<AK, BK>), grid, block, 0, stream, p);
+            }
             else if(tile == 128u)
                 hipLaunchKernelGGL((gemmTiledKernel16Small<E, OutT, AK, BK>), grid, block, 0, stream, p);
             else
@@ -1061,8 +1123,6 @@ namespace
             return 256u;
         if(g.kernel == R355_KERNEL_TILED_128)
             return 128u;
-        if(r355::dtypeBytes(g.in_type) != 2)
-            return 256u;
         const uint64_t cus    = computeUnits();
         auto           rounds = [&](uint32_t t) { return ((uint64_t)((g.m + t - 1) / t) * ((g.n + t - 1) / t) + cus - 1) / cus; };
         return rounds(128u) * 5u < rounds(256u) * 11u ? 128u : 256u;
@@ -1081,8 +1141,6 @@ namespace r355
             return fail(R355_ERR_UNSUPPORTED, "tiled gemm: no kernel for in_type %d -> out_type %d", g.in_type, g.out_type);
         const uint32_t es = dtypeBytes(g.in_type), os = dtypeBytes(g.out_type);
         const uint32_t tile = macroTile(g);
-        if(tile == 128u && es != 2)
-            return fail(R355_ERR_UNSUPPORTED, "tiled gemm: the 128 x 128 macro tile takes 16-bit operands only");
         if(g.beta != 0.0f && g.layout_c != g.layout_d)
             return fail(R355_ERR_UNSUPPORTED, "tiled gemm: C and D must share an orientation");
         const uint32_t tk = STAGE_KB / es;
@@ -1104,7 +1162,7 @@ namespace r355
             plan->grid_y       = 1;
             plan->block_x      = THREADS;
             plan->block_y      = 1;
-            plan->lds_bytes    = fiveBuffers ? 5u * OPER_BYTES : NUM_STAGES * STAGE_BYTES * tile / 256u;
+            plan->lds_bytes    = (fiveBuffers ? 5u * OPER_BYTES : NUM_STAGES * STAGE_BYTES) * tile / 256u;
         }
         return R355_OK;
     }

@@ -130,6 +130,7 @@ def test_simple_kernel_random_inputs_and_block16(in_t, out_t):
 
 
 TILED_LAYOUTS_16 = list(itertools.product([O.ROW, O.COL], repeat=2))
+TILE_SELECTORS = {"tiled": R.KERNEL_TILED, "tiled_128": R.KERNEL_TILED_128}  # 256 x 256 and 128 x 128 macro tiles
 
 
 @pytest.mark.parametrize("in_t,out_t", [(O.F16, O.F16), (O.F16, O.F32), (O.BF16, O.BF16), (O.BF16, O.F32)])
@@ -176,7 +177,7 @@ def test_tiled_kernel_16bit_one_hot_operands(la, lb, kernel):
     # one non-zero in A and one in B: exactly one element of D, for both tile sizes and every orientation
     m, n, k = 256, 256, 128
     rng = np.random.default_rng(6)
-    sel = R.KERNEL_TILED if kernel == "tiled" else R.KERNEL_TILED_128
+    sel = TILE_SELECTORS[kernel]
     for _ in range(6):
         i, j, h = int(rng.integers(m)), int(rng.integers(n)), int(rng.integers(k))
         a = np.zeros(m * k, np.float16)
@@ -220,22 +221,24 @@ def test_auto_takes_the_small_tile_for_few_tile_problems():
 @pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32)])
 @pytest.mark.parametrize("la,lb", TILED_LAYOUTS_16)
 @pytest.mark.parametrize("ldl", [O.ROW, O.COL])
-def test_tiled_kernel_8bit_layouts(in_t, out_t, la, lb, ldl):
+@pytest.mark.parametrize("kernel", list(TILE_SELECTORS))
+def test_tiled_kernel_8bit_layouts(in_t, out_t, la, lb, ldl, kernel):
     # K-contiguous operands are read whole, M/N-contiguous ones through the transposing LDS read
     m, n, k = 256, 512, 768
     a, b, c = _inputs(in_t, out_t, m, n, k, seed=21)
     want = O.gemm(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, c, 1.0, 1.0)
-    got = _run(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, c, 1.0, 1.0, R.KERNEL_TILED)
+    got = _run(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, c, 1.0, 1.0, TILE_SELECTORS[kernel])
     _check(in_t, out_t, got, want)
     # reference-pattern inputs: exact
     a, b = O.fill_ref(in_t, m, k, la), O.fill_ref(in_t, k, n, lb)
     want = O.gemm(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, None, 1.0, 0.0)
-    got = _run(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, None, 1.0, 0.0, R.KERNEL_TILED)
+    got = _run(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, None, 1.0, 0.0, TILE_SELECTORS[kernel])
     assert np.array_equal(got, want)
 
 
 @pytest.mark.parametrize("la,lb", TILED_LAYOUTS_16)
-def test_tiled_kernel_8bit_one_hot_operands(la, lb):
+@pytest.mark.parametrize("kernel", list(TILE_SELECTORS))
+def test_tiled_kernel_8bit_one_hot_operands(la, lb, kernel):
     # A single non-zero in A and in B lands in exactly one element of D only if every (row, k) and
     # (k, column) of the operand tiles reaches the matrix instruction it belongs to: probes the
     # global -> LDS placement and the (transposing) LDS reads of both orientations.
@@ -247,7 +250,7 @@ def test_tiled_kernel_8bit_one_hot_operands(la, lb):
         b = np.zeros(k * n, np.int8)
         a[i * k + h if la == O.ROW else h * m + i] = 3
         b[h * n + j if lb == O.ROW else j * k + h] = 5
-        got = _run(O.I8, O.I32, la, lb, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0, R.KERNEL_TILED).reshape(m, n)
+        got = _run(O.I8, O.I32, la, lb, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0, TILE_SELECTORS[kernel]).reshape(m, n)
         want = np.zeros((m, n), np.int32)
         want[i, j] = 15
         assert np.array_equal(got, want), (i, j, h)
@@ -295,12 +298,13 @@ def test_tiled_kernel_16bit_edge_tiles(in_t, out_t, la, lb, m, n, k):
 @pytest.mark.parametrize("la,lb,ldl", [(O.ROW, O.COL, O.ROW), (O.ROW, O.COL, O.COL), (O.COL, O.ROW, O.ROW),
                                        (O.COL, O.COL, O.COL), (O.ROW, O.ROW, O.ROW)])
 @pytest.mark.parametrize("m,n,k", RAGGED_SHAPES)
-def test_tiled_kernel_8bit_edge_tiles(in_t, out_t, la, lb, ldl, m, n, k):
+@pytest.mark.parametrize("kernel", list(TILE_SELECTORS))
+def test_tiled_kernel_8bit_edge_tiles(in_t, out_t, la, lb, ldl, m, n, k, kernel):
     a, b, c = _inputs(in_t, out_t, m, n, k, seed=80 + n)
     for alpha, beta in ((1.0, 0.0), (1.0, 1.0)):
         cc = None if beta == 0.0 else c
         want = O.gemm(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, cc, alpha, beta)
-        got = _run(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, cc, alpha, beta, R.KERNEL_TILED)
+        got = _run(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, cc, alpha, beta, TILE_SELECTORS[kernel])
         _check(in_t, out_t, got, want)
 
 
@@ -336,13 +340,14 @@ def test_tiled_kernel_16bit_stage_counts(in_t, out_t, la, lb, k):
 @pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32)])
 @pytest.mark.parametrize("la,lb", [(O.ROW, O.COL), (O.COL, O.ROW)])
 @pytest.mark.parametrize("stages", [1, 2, 3, 4, 5, 6, 7, 11, 13])
-def test_tiled_kernel_8bit_stage_counts(in_t, out_t, la, lb, stages):
+@pytest.mark.parametrize("kernel", list(TILE_SELECTORS))
+def test_tiled_kernel_8bit_stage_counts(in_t, out_t, la, lb, stages, kernel):
     # The 8-bit kernel rotates five LDS buffers with period six; cover every remainder of the K
     # stage count, including a single stage and counts beyond one period.
     m, n, k = 256, 256, 128 * stages
     a, b, _ = _inputs(in_t, out_t, m, n, k, seed=40 + stages)
     want = O.gemm(in_t, out_t, la, lb, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0)
-    got = _run(in_t, out_t, la, lb, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0, R.KERNEL_TILED)
+    got = _run(in_t, out_t, la, lb, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0, TILE_SELECTORS[kernel])
     _check(in_t, out_t, got, want)
 
 
