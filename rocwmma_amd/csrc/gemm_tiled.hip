@@ -133,6 +133,26 @@ namespace
             asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(x), "v"(y));
     }
 
+    // K tails.  A K stage with only `valid` (< 128) bytes of K left per row is completed with zeros by the
+    // loads themselves: a buffer load whose offset lies outside its buffer writes zeros to LDS.  For an
+    // M/N-contiguous operand the buffer of a stage ends after its last valid k-row (`valid` bytes of K are
+    // valid / element size rows of ld elements: valid * ld bytes; the range check of a raw buffer on this
+    // hardware covers lane offset + scalar offset); a K-contiguous lane whose chunk lies beyond K uses an
+    // offset no buffer contains.
+    __device__ __forceinline__ uint32_t stageRecords(bool kContig, uint32_t valid, uint32_t ld)
+    {
+        return kContig ? 0x7FFFFFFFu : valid * ld;
+    }
+    __device__ __forceinline__ i32x4 stageRsrc8(bool kContig, uint64_t addr, uint32_t valid, uint32_t ld)
+    {
+        return i32x4{static_cast<int>(static_cast<uint32_t>(addr)), static_cast<int>(static_cast<uint32_t>(addr >> 32) & 0xFFFFu),
+                     static_cast<int>(stageRecords(kContig, valid, ld)), 0x00020000};
+    }
+    __device__ __forceinline__ uint32_t tailOffset(bool kContig, uint32_t laneOffset, uint32_t kByte, uint32_t valid)
+    {
+        return kContig && kByte >= valid ? 0x80000000u : laneOffset;
+    }
+
     // D = alpha * acc + beta * C for one wave's tile of WB x WB accumulator blocks (16 x 16 each), row-major;
     // the wave tile starts at (m0, n0).  `scratch` is WB * 4 KiB of LDS owned by this wave.
     template <typename AccV, typename OutT, uint32_t WB>
@@ -259,14 +279,16 @@ namespace
         // row / the first chunk instead -- what lands in LDS for it only feeds elements of D that are
         // never stored.  Hence one lane offset per load (the compiler merges equal ones).
         uint32_t       gOffA[LOADS], gOffB[LOADS], gStepA, gStepB; // gStep: uniform offset per load
+        uint32_t       kByteA = 0u, kByteB = 0u; // K-contiguous: K offset inside a stage of this lane's chunks
         uint64_t       gStageA, gStageB; // bytes between consecutive K stages
         const uint32_t validM = p.m - tm * TILE < TILE ? p.m - tm * TILE : TILE;
         const uint32_t validN = p.n - tn * TILE < TILE ? p.n - tn * TILE : TILE;
         auto laneOffsets = [&](bool kContig, uint32_t ld, uint32_t valid, uint32_t (&off)[LOADS], uint32_t& step,
-                               uint64_t& stage) {
+                               uint64_t& stage, uint32_t& kByte) {
             if(kContig)
             {
                 const uint32_t r = tid >> 3, slot = tid & 7u;
+                kByte = (slot ^ swzK(r)) * CHUNK;
 #pragma unroll
                 for(uint32_t j = 0; j < LOADS; ++j)
                 {
@@ -288,8 +310,8 @@ namespace
                 step = KROWS * ld * ES, stage = (uint64_t)TK * ld * ES;
             }
         };
-        laneOffsets(A_KCONTIG, p.lda, validM, gOffA, gStepA, gStageA);
-        laneOffsets(B_KCONTIG, p.ldb, validN, gOffB, gStepB, gStageB);
+        laneOffsets(A_KCONTIG, p.lda, validM, gOffA, gStepA, gStageA, kByteA);
+        laneOffsets(B_KCONTIG, p.ldb, validN, gOffB, gStepB, gStageB, kByteB);
         const char* gA = p.a + (A_KCONTIG ? (uint64_t)tm * TILE * p.lda * ES : (uint64_t)tm * TILE * ES);
         const char* gB = p.b + (B_KCONTIG ? (uint64_t)tn * TILE * p.ldb * ES : (uint64_t)tn * TILE * ES);
 
@@ -369,29 +391,40 @@ namespace
             const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
             return (static_cast<uint64_t>(hi) << 32) | lo;
         };
-        auto rsrcAt = [](uint64_t addr) { // raw buffer, 32-bit data format, no swizzle
-            return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>(addr), 0, 0x7FFFFFFF, 0x00020000);
+        // K stages come in pairs; K need not fill the last pair: stage st holds validOf(st) = 0 .. 128 valid
+        // bytes per row and the loads fill the rest with zeros
+        const uint32_t kBytes    = p.k * ES;
+        const uint32_t numStages = (kBytes + 2u * STAGE_KB - 1u) / (2u * STAGE_KB) * 2u;
+        auto           validOf   = [&](uint32_t st) {
+            st = st < numStages ? st : numStages - 1u;
+            return st * STAGE_KB >= kBytes ? 0u : (kBytes - st * STAGE_KB < STAGE_KB ? kBytes - st * STAGE_KB : STAGE_KB);
         };
-        auto stageRsrc = [&](const char* panel) { return rsrcAt(uniform64(panel)); };
-        // load x of a stage: x = 2 j loads piece j of A, x = 2 j + 1 piece j of B
-        auto issueLoad = [&](__amdgpu_buffer_rsrc_t srcA, __amdgpu_buffer_rsrc_t srcB, char* stage, uint32_t x) {
+        auto rsrcAt = [](uint64_t addr, uint32_t records) { // raw buffer, 32-bit data format, no swizzle
+            return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>(addr), 0, static_cast<int>(records), 0x00020000);
+        };
+        // load x of a stage with vA / vB valid bytes of K: x = 2 j loads piece j of A, x = 2 j + 1 piece j of B
+        auto issueLoad = [&](__amdgpu_buffer_rsrc_t srcA, __amdgpu_buffer_rsrc_t srcB, uint32_t vA, uint32_t vB, char* stage,
+                             uint32_t x) {
             using lp         = __attribute__((address_space(3))) void*;
             const uint32_t j = x >> 1;
             char*          dst = stage + (j * THREADS + wave * 64u) * CHUNK;
             if(x & 1u)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(srcB, (lp)(dst + OPER), 16, gOffB[j], j * gStepB, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(srcB, (lp)(dst + OPER), 16, tailOffset(B_KCONTIG, gOffB[j], kByteB, vB),
+                                                         j * gStepB, 0, 0);
             else
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(srcA, (lp)dst, 16, gOffA[j], j * gStepA, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(srcA, (lp)dst, 16, tailOffset(A_KCONTIG, gOffA[j], kByteA, vA), j * gStepA, 0,
+                                                         0);
         };
         auto issueGlobal = [&](uint32_t kt, char* stage) {
-            const __amdgpu_buffer_rsrc_t srcA = stageRsrc(gA + kt * gStageA), srcB = stageRsrc(gB + kt * gStageB);
+            const uint32_t               v    = validOf(kt);
+            const __amdgpu_buffer_rsrc_t srcA = rsrcAt(uniform64(gA + kt * gStageA), stageRecords(A_KCONTIG, v, p.lda)),
+                                         srcB = rsrcAt(uniform64(gB + kt * gStageB), stageRecords(B_KCONTIG, v, p.ldb));
 #pragma unroll
             for(uint32_t x = 0; x < 2u * LOADS; ++x)
-                issueLoad(srcA, srcB, stage, x);
+                issueLoad(srcA, srcB, v, v, stage, x);
         };
 
         f32x4          acc[WB][WB];
-        const uint32_t numStages = p.k / TK;
 #pragma unroll
         for(uint32_t i = 0; i < WB; ++i)
 #pragma unroll
@@ -453,7 +486,9 @@ namespace
             }
             __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): stage kt + 1 has landed
             __syncthreads();
-            const __amdgpu_buffer_rsrc_t srcA = rsrcAt(refillA), srcB = rsrcAt(refillB);
+            const uint32_t               v    = validOf(kt + 2u);
+            const __amdgpu_buffer_rsrc_t srcA = rsrcAt(refillA, stageRecords(A_KCONTIG, v, p.lda)),
+                                         srcB = rsrcAt(refillB, stageRecords(B_KCONTIG, v, p.ldb));
             if(kt + 3u < numStages) // the refill of the next stage is one stage further, or the last again
                 refillA += gStageA, refillB += gStageB;
 #pragma unroll
@@ -466,7 +501,7 @@ namespace
                     if(q < 2u)
                         readAt(nxt, 0, x, q);
                     if(q == LOAD_Q)
-                        issueLoad(srcA, srcB, cur, x);
+                        issueLoad(srcA, srcB, v, v, cur, x);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -481,7 +516,6 @@ namespace
         refillA = uniform64(gA + (numStages > 2u ? 2u : numStages - 1u) * gStageA);
         refillB = uniform64(gB + (numStages > 2u ? 2u : numStages - 1u) * gStageB);
 
-        // numStages is even (checked on the host)
         for(uint32_t kt = 0; kt < numStages; kt += 2)
         {
             stageBody(kt, stage0, stage1);
@@ -559,14 +593,17 @@ namespace
     // n not a multiple of 256) must not read outside the operand: a lane whose row (K-contiguous) or
     // chunk (M/N-contiguous) lies beyond the matrix reads the last valid row / the first chunk instead;
     // what lands in LDS for it only feeds elements of D that are never stored.  `step` is the uniform
-    // offset from one load to the next, `stage` the distance between K stages.
+    // offset from one load to the next, `stage` the distance between K stages, `kByte` the K offset
+    // inside a stage of a K-contiguous lane's chunks.
     template <bool KCONTIG, uint32_t WB>
     __device__ __forceinline__ void laneOffsets8(uint32_t tid, uint32_t ld, uint32_t valid, uint32_t (&off)[WB], uint32_t& step,
-                                                 uint64_t& stage)
+                                                 uint64_t& stage, uint32_t& kByte)
     {
+        kByte = 0u;
         if constexpr(KCONTIG)
         {
             const uint32_t r = tid >> 3, slot = tid & 7u; // row 32 j + r
+            kByte = (slot ^ swzK8(r)) * CHUNK;
 #pragma unroll
             for(uint32_t j = 0; j < WB; ++j)
             {
@@ -671,13 +708,17 @@ namespace
         const uint32_t ldsBase
             = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds));
 
-        uint32_t       gOffA[WB], gOffB[WB], gStepA, gStepB; // WB direct loads per operand per stage
+        uint32_t       gOffA[WB], gOffB[WB], gStepA, gStepB, kByteA, kByteB; // WB direct loads per operand per stage
         uint64_t       gStageA, gStageB;
         const uint32_t validM = p.m - tm * TILE < TILE ? p.m - tm * TILE : TILE;
         const uint32_t validN = p.n - tn * TILE < TILE ? p.n - tn * TILE : TILE;
-        laneOffsets8<A_KCONTIG, WB>(tid, p.lda, validM, gOffA, gStepA, gStageA);
-        laneOffsets8<B_KCONTIG, WB>(tid, p.ldb, validN, gOffB, gStepB, gStageB);
-        const uint32_t numStages = p.k / STAGE_KB;
+        laneOffsets8<A_KCONTIG, WB>(tid, p.lda, validM, gOffA, gStepA, gStageA, kByteA);
+        laneOffsets8<B_KCONTIG, WB>(tid, p.ldb, validN, gOffB, gStepB, gStageB, kByteB);
+        // K need not fill the last stage: its lastBytes (16 .. 128) valid bytes per row are followed by zeros
+        // the loads produce themselves (see tailOffset)
+        const uint32_t numStages = (p.k + STAGE_KB - 1u) / STAGE_KB;
+        const uint32_t lastBytes = p.k - (numStages - 1u) * STAGE_KB;
+        auto           validOf   = [&](uint32_t stage) { return stage + 1u >= numStages ? lastBytes : STAGE_KB; };
         const uint32_t dmaDst    = ldsBase + wave * 64u * CHUNK; // + buffer + j * 4 KiB
         auto           uniform64 = [](const char* ptr) {
             const uint64_t v  = reinterpret_cast<uint64_t>(ptr);
@@ -687,18 +728,15 @@ namespace
         };
         const uint64_t gA = uniform64(p.a + (A_KCONTIG ? (uint64_t)tm * TILE * p.lda : (uint64_t)tm * TILE));
         const uint64_t gB = uniform64(p.b + (B_KCONTIG ? (uint64_t)tn * TILE * p.ldb : (uint64_t)tn * TILE));
-        auto rsrcAt = [](uint64_t addr) { // raw buffer over a stage of an operand panel
-            return i32x4{static_cast<int>(static_cast<uint32_t>(addr)), static_cast<int>(static_cast<uint32_t>(addr >> 32) & 0xFFFFu),
-                         0x7FFFFFFF, 0x00020000};
-        };
         auto stageAddr = [&](uint64_t panel, uint64_t perStage, uint32_t stage) { // clamped to the last stage
             return panel + (uint64_t)(stage < numStages ? stage : numStages - 1u) * perStage;
         };
-        auto issueHalf = [&](uint64_t addr, const uint32_t (&gOff)[WB], uint32_t step, uint32_t at) {
-            const i32x4 rsrc = rsrcAt(addr);
+        auto issueHalf = [&](bool kContig, uint64_t addr, const uint32_t (&gOff)[WB], uint32_t step, uint32_t kByte, uint32_t ld,
+                             uint32_t valid, uint32_t at) {
+            const i32x4 rsrc = stageRsrc8(kContig, addr, valid, ld);
 #pragma unroll
             for(uint32_t j = 0; j < WB; ++j)
-                loadToLds(rsrc, gOff[j], j * step, dmaDst + at + j * THREADS * CHUNK);
+                loadToLds(rsrc, tailOffset(kContig, gOff[j], kByte, valid), j * step, dmaDst + at + j * THREADS * CHUNK);
         };
 
         uint32_t rdA[8], rdB[8];
@@ -749,7 +787,8 @@ namespace
                 }
             waitVmcnt<WB>(); // this wave's part of stage kt + 1 has landed (the youngest WB loads are B of kt + 2)
             ldsBarrier();
-            const i32x4 rsrcA = rsrcAt(refillA), rsrcB = rsrcAt(refillB);
+            const uint32_t vA = validOf(kt + 2u), vB = validOf(kt + 3u);
+            const i32x4    rsrcA = stageRsrc8(A_KCONTIG, refillA, vA, p.lda), rsrcB = stageRsrc8(B_KCONTIG, refillB, vB, p.ldb);
             if(kt + 3u < numStages)
                 refillA += gStageA;
             if(kt + 4u < numStages)
@@ -765,20 +804,21 @@ namespace
                     if(q == LOAD_Q)
                     {
                         if(x < WB)
-                            loadToLds(rsrcA, gOffA[x], x * gStepA, dmaDst + aCur + x * THREADS * CHUNK);
+                            loadToLds(rsrcA, tailOffset(A_KCONTIG, gOffA[x], kByteA, vA), x * gStepA, dmaDst + aCur + x * THREADS * CHUNK);
                         else
-                            loadToLds(rsrcB, gOffB[x - WB], (x - WB) * gStepB, dmaDst + bCur + (x - WB) * THREADS * CHUNK);
+                            loadToLds(rsrcB, tailOffset(B_KCONTIG, gOffB[x - WB], kByteB, vB), (x - WB) * gStepB,
+                                      dmaDst + bCur + (x - WB) * THREADS * CHUNK);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
         };
 
         // prologue: stages 0 and 1 and the B half of stage 2 requested; stage 0 published
-        issueHalf(stageAddr(gA, gStageA, 0u), gOffA, gStepA, A_AT[0]);
-        issueHalf(stageAddr(gB, gStageB, 0u), gOffB, gStepB, B_AT[0]);
-        issueHalf(stageAddr(gA, gStageA, 1u), gOffA, gStepA, A_AT[1]);
-        issueHalf(stageAddr(gB, gStageB, 1u), gOffB, gStepB, B_AT[1]);
-        issueHalf(stageAddr(gB, gStageB, 2u), gOffB, gStepB, B_AT[2]);
+        issueHalf(A_KCONTIG, stageAddr(gA, gStageA, 0u), gOffA, gStepA, kByteA, p.lda, validOf(0u), A_AT[0]);
+        issueHalf(B_KCONTIG, stageAddr(gB, gStageB, 0u), gOffB, gStepB, kByteB, p.ldb, validOf(0u), B_AT[0]);
+        issueHalf(A_KCONTIG, stageAddr(gA, gStageA, 1u), gOffA, gStepA, kByteA, p.lda, validOf(1u), A_AT[1]);
+        issueHalf(B_KCONTIG, stageAddr(gB, gStageB, 1u), gOffB, gStepB, kByteB, p.ldb, validOf(1u), B_AT[1]);
+        issueHalf(B_KCONTIG, stageAddr(gB, gStageB, 2u), gOffB, gStepB, kByteB, p.ldb, validOf(2u), B_AT[2]);
         refillA = stageAddr(gA, gStageA, 2u), refillB = stageAddr(gB, gStageB, 3u);
         waitVmcnt<3u * WB>();
         ldsBarrier();
@@ -880,13 +920,17 @@ namespace
         const uint32_t ldsBase
             = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds));
 
-        uint32_t       gOffA[WB], gOffB[WB], gStepA, gStepB; // WB direct loads per operand per stage
+        uint32_t       gOffA[WB], gOffB[WB], gStepA, gStepB, kByteA, kByteB; // WB direct loads per operand per stage
         uint64_t       gStageA, gStageB;
         const uint32_t validM = p.m - tm * TILE < TILE ? p.m - tm * TILE : TILE;
         const uint32_t validN = p.n - tn * TILE < TILE ? p.n - tn * TILE : TILE;
-        laneOffsets8<A_KCONTIG, WB>(tid, p.lda, validM, gOffA, gStepA, gStageA);
-        laneOffsets8<B_KCONTIG, WB>(tid, p.ldb, validN, gOffB, gStepB, gStageB);
-        const uint32_t numStages = p.k / STAGE_KB;
+        laneOffsets8<A_KCONTIG, WB>(tid, p.lda, validM, gOffA, gStepA, gStageA, kByteA);
+        laneOffsets8<B_KCONTIG, WB>(tid, p.ldb, validN, gOffB, gStepB, gStageB, kByteB);
+        // K need not fill the last stage: its lastBytes (16 .. 128) valid bytes per row are followed by zeros
+        // the loads produce themselves (see tailOffset)
+        const uint32_t numStages = (p.k + STAGE_KB - 1u) / STAGE_KB;
+        const uint32_t lastBytes = p.k - (numStages - 1u) * STAGE_KB;
+        auto           validOf   = [&](uint32_t stage) { return stage + 1u >= numStages ? lastBytes : STAGE_KB; };
         const uint32_t dmaDst    = ldsBase + wave * 64u * CHUNK;
         auto           uniform64 = [](const char* ptr) {
             const uint64_t v  = reinterpret_cast<uint64_t>(ptr);
@@ -896,18 +940,15 @@ namespace
         };
         const uint64_t gA = uniform64(p.a + (A_KCONTIG ? (uint64_t)tm * TILE * p.lda : (uint64_t)tm * TILE));
         const uint64_t gB = uniform64(p.b + (B_KCONTIG ? (uint64_t)tn * TILE * p.ldb : (uint64_t)tn * TILE));
-        auto rsrcAt = [](uint64_t addr) {
-            return i32x4{static_cast<int>(static_cast<uint32_t>(addr)), static_cast<int>(static_cast<uint32_t>(addr >> 32) & 0xFFFFu),
-                         0x7FFFFFFF, 0x00020000};
-        };
         auto stageAddr = [&](uint64_t panel, uint64_t perStage, uint32_t stage) {
             return panel + (uint64_t)(stage < numStages ? stage : numStages - 1u) * perStage;
         };
-        auto issueHalf = [&](uint64_t addr, const uint32_t (&gOff)[WB], uint32_t step, uint32_t at) {
-            const i32x4 rsrc = rsrcAt(addr);
+        auto issueHalf = [&](bool kContig, uint64_t addr, const uint32_t (&gOff)[WB], uint32_t step, uint32_t kByte, uint32_t ld,
+                             uint32_t valid, uint32_t at) {
+            const i32x4 rsrc = stageRsrc8(kContig, addr, valid, ld);
 #pragma unroll
             for(uint32_t j = 0; j < WB; ++j)
-                loadToLds(rsrc, gOff[j], j * step, dmaDst + at + j * THREADS * CHUNK);
+                loadToLds(rsrc, tailOffset(kContig, gOff[j], kByte, valid), j * step, dmaDst + at + j * THREADS * CHUNK);
         };
 
         uint32_t rdA[8], rdB[8];
@@ -935,10 +976,11 @@ namespace
             }
         };
         // direct load j of an operand goes out in slot n when [n WB / NQ, (n + 1) WB / NQ) contains j
-        auto loadSlot = [&](const i32x4& rsrc, const uint32_t (&gOff)[WB], uint32_t step, uint32_t at, uint32_t n) {
+        auto loadSlot = [&](bool kContig, const i32x4& rsrc, const uint32_t (&gOff)[WB], uint32_t step, uint32_t kByte,
+                            uint32_t valid, uint32_t at, uint32_t n) {
 #pragma unroll
             for(uint32_t j = n * WB / NQ; j < (n + 1u) * WB / NQ; ++j)
-                loadToLds(rsrc, gOff[j], j * step, dmaDst + at + j * THREADS * CHUNK);
+                loadToLds(rsrc, tailOffset(kContig, gOff[j], kByte, valid), j * step, dmaDst + at + j * THREADS * CHUNK);
         };
 
         f32x4 acc[WB][WB];
@@ -971,7 +1013,8 @@ namespace
             }
             waitVmcnt<WB>(); // this wave's part of stage kt + 1 has landed (the youngest WB loads are B of kt + 2)
             ldsBarrier();
-            const i32x4 rsrcA = rsrcAt(refillA), rsrcB = rsrcAt(refillB);
+            const uint32_t vA = validOf(kt + 2u), vB = validOf(kt + 3u);
+            const i32x4    rsrcA = stageRsrc8(A_KCONTIG, refillA, vA, p.lda), rsrcB = stageRsrc8(B_KCONTIG, refillB, vB, p.ldb);
             if(kt + 3u < numStages)
                 refillA += gStageA;
             if(kt + 4u < numStages)
@@ -982,7 +1025,7 @@ namespace
             {
                 mfma16f8(acc[H + n / H][H + n % H], bHi[n % H], aHi[n / H]);
                 readSlotA(aLo, aNxt, 0, n);
-                loadSlot(rsrcA, gOffA, gStepA, aCur, n);
+                loadSlot(A_KCONTIG, rsrcA, gOffA, gStepA, kByteA, vA, aCur, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
             // Q4: A high x B low; next B low arrives in the registers B high has left; B refill
@@ -991,17 +1034,17 @@ namespace
             {
                 mfma16f8(acc[H + n % H][n / H], bLo[n / H], aHi[n % H]);
                 readSlotB(bHi, bNxt, 0, n);
-                loadSlot(rsrcB, gOffB, gStepB, bCur, n);
+                loadSlot(B_KCONTIG, rsrcB, gOffB, gStepB, kByteB, vB, bCur, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
 
         // prologue: stages 0 and 1 and the B half of stage 2 requested; stage 0 published
-        issueHalf(stageAddr(gA, gStageA, 0u), gOffA, gStepA, A_AT[0]);
-        issueHalf(stageAddr(gB, gStageB, 0u), gOffB, gStepB, B_AT[0]);
-        issueHalf(stageAddr(gA, gStageA, 1u), gOffA, gStepA, A_AT[1]);
-        issueHalf(stageAddr(gB, gStageB, 1u), gOffB, gStepB, B_AT[1]);
-        issueHalf(stageAddr(gB, gStageB, 2u), gOffB, gStepB, B_AT[2]);
+        issueHalf(A_KCONTIG, stageAddr(gA, gStageA, 0u), gOffA, gStepA, kByteA, p.lda, validOf(0u), A_AT[0]);
+        issueHalf(B_KCONTIG, stageAddr(gB, gStageB, 0u), gOffB, gStepB, kByteB, p.ldb, validOf(0u), B_AT[0]);
+        issueHalf(A_KCONTIG, stageAddr(gA, gStageA, 1u), gOffA, gStepA, kByteA, p.lda, validOf(1u), A_AT[1]);
+        issueHalf(B_KCONTIG, stageAddr(gB, gStageB, 1u), gOffB, gStepB, kByteB, p.ldb, validOf(1u), B_AT[1]);
+        issueHalf(B_KCONTIG, stageAddr(gB, gStageB, 2u), gOffB, gStepB, kByteB, p.ldb, validOf(2u), B_AT[2]);
         refillA = stageAddr(gA, gStageA, 2u), refillB = stageAddr(gB, gStageB, 3u);
         waitVmcnt<3u * WB>();
         ldsBarrier();
@@ -1144,11 +1187,14 @@ namespace r355
         if(g.beta != 0.0f && g.layout_c != g.layout_d)
             return fail(R355_ERR_UNSUPPORTED, "tiled gemm: C and D must share an orientation");
         const uint32_t tk = STAGE_KB / es;
-        // the two-buffer kernel consumes K stages in pairs; the five-buffer 8-bit kernel takes any count
+        // K moves in 16-byte chunks; a last K stage that is not full is completed with zeros by the loads
         const bool     fiveBuffers = es == 1;
-        const uint32_t kGranule    = fiveBuffers ? tk : 2 * tk;
+        const uint32_t kGranule    = CHUNK / es;
         if(g.m % 16 || g.n % 16 || g.m == 0 || g.n == 0 || g.k % kGranule || g.k == 0)
             return fail(R355_ERR_BAD_SIZE, "tiled gemm: m=%u n=%u must be multiples of 16 and k=%u of %u", g.m, g.n, g.k, kGranule);
+        // lane offsets are 32-bit (255 rows of ld elements) and a K stage of an M/N-contiguous operand is one buffer
+        if((uint64_t)g.lda * es > (1u << 23) || (uint64_t)g.ldb * es > (1u << 23))
+            return fail(R355_ERR_UNSUPPORTED, "tiled gemm: leading dimensions above 8 MiB per row / column");
         if(!aligned(g.a, 16) || !aligned(g.b, 16) || (g.lda * es) % 16 || (g.ldb * es) % 16 || !aligned(g.d, 16)
            || (g.ldd * os) % 16 || (g.beta != 0.0f && (!aligned(g.c, 16) || (g.ldc * os) % 16)))
             return fail(R355_ERR_MISALIGNED, "tiled gemm: pointers and leading dimensions of A, B, C, D must keep 16-byte alignment");

@@ -73,9 +73,9 @@ def test_query_selects_kernel_family_and_reports_launch_shape():
     (dict(layout_a=7), -1),
     (dict(in_type=R.F16, out_type=R.I32), -2),
     (dict(m=100, n=256), -3),
-    (dict(k=24), -3),
+    (dict(k=20), -3),
     (dict(kernel=R.KERNEL_TILED, m=120), -3),
-    (dict(kernel=R.KERNEL_TILED, k=192), -3),
+    (dict(kernel=R.KERNEL_TILED, k=100), -3),
     (dict(kernel=R.KERNEL_TILED_128, m=120), -3),
     (dict(kernel=4), -1),
     (dict(a=0x1002, layout_a=R.ROW_MAJOR), -4),

@@ -351,6 +351,31 @@ def test_tiled_kernel_8bit_stage_counts(in_t, out_t, la, lb, stages, kernel):
     _check(in_t, out_t, got, want)
 
 
+@pytest.mark.parametrize("in_t,out_t,ks", [(O.F16, O.F32, (8, 72, 136, 328)), (O.BF16, O.BF16, (24, 200)),
+                                           (O.I8, O.I32, (16, 144, 400, 784)), (O.E4M3, O.F32, (48, 272))])
+@pytest.mark.parametrize("la,lb", TILED_LAYOUTS_16)
+@pytest.mark.parametrize("kernel", list(TILE_SELECTORS))
+def test_tiled_kernel_k_tails(in_t, out_t, ks, la, lb, kernel):
+    # K that does not fill the last 128-byte stage (16-bit: the last pair of stages): the loads complete it
+    # with zeros, for K-contiguous operands per lane, for M/N-contiguous ones through the buffer's end.
+    # The operands sit in the middle of a larger allocation filled with a value that would show up in D.
+    m, n = 272, 144
+    for k in ks:
+        a, b, c = _inputs(in_t, out_t, m, n, k, seed=300 + k)
+        want = O.gemm(in_t, out_t, la, lb, O.ROW, O.ROW, m, n, k, a, b, c, 1.0, 1.0)
+        poison = np.full(4096, 0x40 if a.dtype.itemsize == 1 else 0x4000, dtype=a.dtype)  # 2.0 in e4m3 / f16 / bf16, 64 as int8
+        da = to_device(np.concatenate([poison, a, poison]))
+        db = to_device(np.concatenate([poison, b, poison]))
+        dc = to_device(c)
+        dd = device_filled(m * n, O.NP_STORAGE[out_t], 0xFF)
+        R.gemm(in_t, out_t, m, n, k, da[4096:], db[4096:], dc, dd, 1.0, 1.0, la, lb, O.ROW, O.ROW, kernel=TILE_SELECTORS[kernel])
+        got = to_host(dd, O.NP_STORAGE[out_t])
+        w32 = None
+        if out_t not in (O.F32, O.I32):
+            w32 = O.gemm(in_t, O.F32, la, lb, O.ROW, O.ROW, m, n, k, a, b, O.storage_to_f32(c, out_t), 1.0, 1.0)
+        _check(in_t, out_t, got, want, w32)
+
+
 def test_tiled_kernel_many_tiles_xcd_mapping():
     # 5 x 3 tiles: a tile count that is not a multiple of 8 and a partial row group
     m, n, k = 1280, 768, 256
