@@ -49,11 +49,11 @@ namespace
             *family = -1;
             return rc;
         }
-        // AUTO leaves problems smaller than half a macro tile in either direction to the block-per-wave
-        // kernel: one mostly empty 256 x 256 tile on one CU is slower than many small blocks.
-        const bool forced      = g->kernel == R355_KERNEL_TILED || g->kernel == R355_KERNEL_TILED_128;
-        const bool worthTiling = forced || (g->m >= 128 && g->n >= 128);
-        if((forced || g->kernel == R355_KERNEL_AUTO) && worthTiling)
+        // AUTO takes a macro-tile kernel wherever its checks pass (down to m = n = 16 the 128 x 128 tile with
+        // clamped edge loads is faster than one block per wave without LDS); the block-per-wave kernel
+        // covers the rest: f32 / f64, strides or pointers off 16-byte alignment, k off a 16-byte chunk.
+        const bool forced = g->kernel == R355_KERNEL_TILED || g->kernel == R355_KERNEL_TILED_128;
+        if(forced || g->kernel == R355_KERNEL_AUTO)
         {
             rc = r355::gemmTiledCheck(*g, out);
             if(rc == R355_OK)

@@ -4,7 +4,7 @@
 // reference does (2 m n k flop, test/performance.hpp:424-442), plus the fraction of MI355X's
 // published peak.  Usage:
 //   host_bench gemm  [--type f16|bf16|i8|e4m3] [--out f16|bf16|f32|i32] [--layout nt|tn|nn|tt]
-//                    [--m M --n N --k K] [--kernel auto|simple|tiled] [--warmup W --iters I]
+//                    [--m M --n N --k K] [--kernel auto|simple|tiled|tiled128] [--warmup W --iters I]
 //                    [--sparse 1]   A is 2:4 structured sparse (compressed values + index nibbles)
 //                    [--ldpad E]    lda and ldb grow by E elements (power-of-two strides cost L2 efficiency)
 //   host_bench dlrm  [--type f16|bf16|f32] [--bwd 1] [--batch B --m M --k K] [--warmup W --iters I]
@@ -278,7 +278,10 @@ int main(int argc, char** argv)
         g.ldb = (g.layout_b == R355_ROW_MAJOR ? n : k) + ldpad;
         g.ldc = g.ldd = n;
         g.alpha = 1.0f, g.beta = 0.0f;
-        g.kernel = kernel == "simple" ? R355_KERNEL_SIMPLE : (kernel == "tiled" ? R355_KERNEL_TILED : R355_KERNEL_AUTO);
+        g.kernel = kernel == "simple"     ? R355_KERNEL_SIMPLE
+                   : kernel == "tiled"    ? R355_KERNEL_TILED
+                   : kernel == "tiled128" ? R355_KERNEL_TILED_128
+                                          : R355_KERNEL_AUTO;
         const size_t rowsA = g.layout_a == R355_ROW_MAJOR ? m : k, rowsB = g.layout_b == R355_ROW_MAJOR ? k : n;
         std::vector<uint8_t> ha(sparse ? (size_t)m * k * bytesOf(inT) / 2 : rowsA * g.lda * bytesOf(inT)),
             hb(rowsB * g.ldb * bytesOf(inT));
