@@ -7,7 +7,8 @@
 // and eight matrix instructions per wave between barriers; this one is shaped for
 // MI355X's 160 KB LDS and 256 CUs:
 //
-//   macro tile   256 x 256, K stage of 128 bytes (64 f16/bf16, 128 int8/fp8 elements)
+//   macro tile   256 x 256, K stage of 128 bytes (64 f16/bf16, 128 int8/fp8 elements); 128 x 128 (wave tile
+//                64 x 64, five 16 KiB LDS buffers, two workgroups per CU) for problems with too few large tiles
 //   workgroup    256 threads = 4 waves in a 2 x 2 grid, wave tile 128 x 128
 //                = 8 x 8 accumulators of the 16 x 16 matrix-instruction shapes (256 registers):
 //                v_mfma_f32_16x16x32_{f16,bf16}, v_mfma_i32_16x16x64_i8, v_mfma_f32_16x16x128_f8f6f4.
@@ -237,8 +238,9 @@ namespace
 
     //
     // WB is the number of accumulator blocks per wave tile edge: 8 (wave tile 128 x 128, macro tile
-    // 256 x 256, one workgroup per CU) or 4 (wave tile 64 x 64, macro tile 128 x 128, 64 KiB of LDS and
-    // a quarter of the registers) for problems with too few 256 x 256 tiles to fill the CUs.
+    // 256 x 256, one workgroup per CU).  The body also works with 4 (wave tile 64 x 64, macro tile
+    // 128 x 128, 64 KiB of LDS), but the small tile is served by the five-buffer body further down, which
+    // keeps more loads in flight.
     template <Elem E, typename OutT, bool A_KCONTIG, bool B_KCONTIG, uint32_t WB>
     __device__ __forceinline__ void gemmTiled16(const Params& p)
     {
@@ -532,22 +534,18 @@ namespace
     }
 
     // (a waves-per-EU attribute that depends on a template parameter makes the compiler drop the host-side
-    // launch stub without a diagnostic, hence one kernel per tile size around a common body)
+    // launch stub without a diagnostic, hence separate kernels per tile size around common bodies)
     template <Elem E, typename OutT, bool A_KCONTIG, bool B_KCONTIG>
     __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) gemmTiledKernel16(Params p)
     {
         gemmTiled16<E, OutT, A_KCONTIG, B_KCONTIG, 8>(p);
     }
-    template <Elem E, typename OutT, bool A_KCONTIG, bool B_KCONTIG>
-    __global__ void __launch_bounds__(THREADS) gemmTiledKernel16Small(Params p)
-    {
-        gemmTiled16<E, OutT, A_KCONTIG, B_KCONTIG, 4>(p);
-    }
 
     // ------------------------------------------------------------------------------------------
-    // 8-bit operands (int8, e4m3), either orientation: five LDS buffers.  At twice the
-    // matrix-instruction rate a K stage lasts about as long as a direct load takes to arrive, so a
-    // two-buffer scheme leaves the memory pipe idle while a refill waits for its consumer.  Here LDS
+    // 8-bit operands (int8, e4m3), either orientation, and the small macro tile of every type: five LDS
+    // buffers.  At twice the matrix-instruction rate (or a quarter of the tile) a K stage lasts about as
+    // long as a direct load takes to arrive, so a two-buffer scheme leaves the memory pipe idle while a
+    // refill waits for its consumer.  Here LDS
     // holds two buffers for A and three for B (5 x 32 KiB = all 160 KiB): the B half of a stage is
     // requested three stages ahead and the A half two, which keeps 96 KiB per CU in flight instead
     // of 64.  Stage kt lives in A buffer kt % 2 and B buffer kt % 3, so six stages bring every buffer
@@ -580,10 +578,12 @@ namespace
     {
         return (row >> 1) & 7u;
     }
-    template <uint32_t WB>
+    template <uint32_t WB, uint32_t ES = 1>
     __device__ __forceinline__ uint32_t swzMN8(uint32_t krow)
     {
-        if constexpr(WB == 8)
+        if constexpr(ES == 2)
+            return ((krow & 3u) << 2) | (((krow >> 3) & 1u) << 1); // 16-bit elements: as in gemmTiled16
+        else if constexpr(WB == 8)
             return (krow & 7u) | ((krow >> 1) & 8u); // 256-byte k-rows, 16 chunks
         else
             return ((krow >> 1) & 3u) | ((krow >> 2) & 4u); // 128-byte k-rows, 8 chunks: rows 2 apart share banks
@@ -595,7 +595,9 @@ namespace
     // what lands in LDS for it only feeds elements of D that are never stored.  `step` is the uniform
     // offset from one load to the next, `stage` the distance between K stages, `kByte` the K offset
     // inside a stage of a K-contiguous lane's chunks.
-    template <bool KCONTIG, uint32_t WB>
+    // (ES = element size in bytes: the five-buffer kernel body below also serves 16-bit operands, whose
+    // M/N-contiguous tiles are 64 k-rows of 64 WB bytes read with ds_read_b64_tr_b16)
+    template <bool KCONTIG, uint32_t WB, uint32_t ES = 1>
     __device__ __forceinline__ void laneOffsets8(uint32_t tid, uint32_t ld, uint32_t valid, uint32_t (&off)[WB], uint32_t& step,
                                                  uint64_t& stage, uint32_t& kByte)
     {
@@ -608,28 +610,28 @@ namespace
             for(uint32_t j = 0; j < WB; ++j)
             {
                 const uint32_t row = r + 32u * j < valid ? r + 32u * j : valid - 1u;
-                off[j]             = row * ld + ((slot ^ swzK8(r)) * CHUNK);
+                off[j]             = row * ld * ES + ((slot ^ swzK8(r)) * CHUNK);
             }
             step = 0u, stage = STAGE_KB;
         }
         else
         {
-            constexpr uint32_t SLOTS = 2u * WB, KROWS = THREADS / SLOTS; // chunks per k-row, k-rows per load
-            const uint32_t     r = tid / SLOTS, slot = tid % SLOTS; // k-row KROWS j + r (256-byte rows: the swizzle alternates with j)
+            constexpr uint32_t SLOTS = 2u * WB * ES, KROWS = THREADS / SLOTS; // chunks per k-row, k-rows per load
+            const uint32_t     r = tid / SLOTS, slot = tid % SLOTS; // k-row KROWS j + r (the swizzle may alternate with j)
 #pragma unroll
             for(uint32_t j = 0; j < WB; ++j)
             {
-                const uint32_t c = slot ^ swzMN8<WB>(KROWS * j + r);
-                off[j]           = r * ld + (c * CHUNK < valid ? c : 0u) * CHUNK;
+                const uint32_t c = slot ^ swzMN8<WB, ES>(KROWS * j + r);
+                off[j]           = r * ld * ES + (c * (CHUNK / ES) < valid ? c : 0u) * CHUNK;
             }
-            step = KROWS * ld, stage = (uint64_t)STAGE_KB * ld;
+            step = KROWS * ld * ES, stage = (uint64_t)STAGE_KB * ld;
         }
     }
 
     // LDS -> register lane offsets of one operand for the wave whose tile starts at row 16 WB w.
     // K-contiguous: rd[q] is 64-byte K step q of block 0 (block i is 16 rows further);
     // M/N-contiguous: rd[i] is block i, the first 8 k-rows of the lane's 16 of K step 0.
-    template <bool KCONTIG, uint32_t WB>
+    template <bool KCONTIG, uint32_t WB, uint32_t ES = 1>
     __device__ __forceinline__ void readOffsets8(uint32_t w, uint32_t lane, uint32_t (&rd)[8])
     {
         const uint32_t t = lane & 15u, g = lane >> 4;
@@ -642,19 +644,30 @@ namespace
             rd[0]            = r * STAGE_KB + ((g ^ swzK8(r)) * CHUNK);
             rd[1]            = r * STAGE_KB + (((4u + g) ^ swzK8(r)) * CHUNK);
         }
-        else
+        else if constexpr(ES == 1)
         {
             const uint32_t kr = 16u * g + (t >> 1);
 #pragma unroll
             for(uint32_t i = 0; i < WB; ++i)
                 rd[i] = kr * 32u * WB + (((w * WB + i) ^ swzMN8<WB>(kr)) * CHUNK) + (t & 1u) * 8u;
         }
+        else
+        {
+            // 16-bit: k-row 8 (lane / 16) + (lane % 16) / 4 of the K step's first half, 8-byte piece 4 i + lane % 4
+            const uint32_t kr = 8u * g + (t >> 2);
+#pragma unroll
+            for(uint32_t i = 0; i < WB; ++i)
+            {
+                const uint32_t piece = w * 4u * WB + 4u * i + (t & 3u);
+                rd[i] = kr * 64u * WB + (((piece >> 1) ^ swzMN8<WB, 2>(kr)) * CHUNK) + (piece & 1u) * 8u;
+            }
+        }
     }
 
     // 16 K bytes of block i, K step s (64 bytes), of the operand tile at `tile`: they arrive whole with
     // part 0 (K-contiguous) or as two transposed halves, parts 0 and 1, into registers at, at + 1 and
     // at + 2, at + 3 of `dst`
-    template <bool KCONTIG, uint32_t WB, typename V>
+    template <bool KCONTIG, uint32_t WB, uint32_t ES = 1, typename V>
     __device__ __forceinline__ void readBlock8(const char* tile, const uint32_t (&rd)[8], uint32_t i, uint32_t s, uint32_t part,
                                                V& dst, uint32_t at)
     {
@@ -666,10 +679,17 @@ namespace
                 dst[at] = v[0], dst[at + 1u] = v[1], dst[at + 2u] = v[2], dst[at + 3u] = v[3];
             }
         }
-        else
+        else if constexpr(ES == 1)
         {
             using lp      = __attribute__((address_space(3))) i32x2*;
             const i32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lp)(tile + rd[i] + (64u * s + 8u * part) * 32u * WB));
+            dst[at + 2u * part] = v[0], dst[at + 2u * part + 1u] = v[1];
+        }
+        else
+        {
+            using lp      = __attribute__((address_space(3))) trv4*;
+            const i32x2 v = __builtin_bit_cast(
+                i32x2, __builtin_amdgcn_ds_read_tr16_b64_v4f16((lp)(tile + rd[i] + (32u * s + 4u * part) * 64u * WB)));
             dst[at + 2u * part] = v[0], dst[at + 2u * part + 1u] = v[1];
         }
     }
@@ -684,10 +704,13 @@ namespace
         asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc) : "v"(x), "v"(y));
     }
 
-    template <bool A_KCONTIG, bool B_KCONTIG, uint32_t WB>
-    __device__ __forceinline__ void gemmTiledI8(const Params& p)
+    template <Elem E, typename OutT, bool A_KCONTIG, bool B_KCONTIG, uint32_t WB>
+    __device__ __forceinline__ void gemmTiled5(const Params& p)
     {
         static_assert(WB == 8 || WB == 4, "wave tile of 8 x 8 or 4 x 4 blocks");
+        static_assert(E != Elem::E4M3, "e4m3 has its own stage structure");
+        constexpr uint32_t ES = ElemTraits<E>::Bytes;
+        using AccV            = std::conditional_t<E == Elem::I8, i32x4v, f32x4>;
         constexpr uint32_t TILE = 32u * WB, WT = 16u * WB; // macro tile and wave tile edge
         constexpr uint32_t OPER = TILE * STAGE_KB; // bytes of one operand per stage: 32 or 16 KiB
         constexpr uint32_t XS = 2u * WB, QS = WB / 2u; // operand blocks per K step, matrix instructions per block
@@ -712,12 +735,13 @@ namespace
         uint64_t       gStageA, gStageB;
         const uint32_t validM = p.m - tm * TILE < TILE ? p.m - tm * TILE : TILE;
         const uint32_t validN = p.n - tn * TILE < TILE ? p.n - tn * TILE : TILE;
-        laneOffsets8<A_KCONTIG, WB>(tid, p.lda, validM, gOffA, gStepA, gStageA, kByteA);
-        laneOffsets8<B_KCONTIG, WB>(tid, p.ldb, validN, gOffB, gStepB, gStageB, kByteB);
+        laneOffsets8<A_KCONTIG, WB, ES>(tid, p.lda, validM, gOffA, gStepA, gStageA, kByteA);
+        laneOffsets8<B_KCONTIG, WB, ES>(tid, p.ldb, validN, gOffB, gStepB, gStageB, kByteB);
         // K need not fill the last stage: its lastBytes (16 .. 128) valid bytes per row are followed by zeros
         // the loads produce themselves (see tailOffset)
-        const uint32_t numStages = (p.k + STAGE_KB - 1u) / STAGE_KB;
-        const uint32_t lastBytes = p.k - (numStages - 1u) * STAGE_KB;
+        const uint32_t kBytes    = p.k * ES;
+        const uint32_t numStages = (kBytes + STAGE_KB - 1u) / STAGE_KB;
+        const uint32_t lastBytes = kBytes - (numStages - 1u) * STAGE_KB;
         auto           validOf   = [&](uint32_t stage) { return stage + 1u >= numStages ? lastBytes : STAGE_KB; };
         const uint32_t dmaDst    = ldsBase + wave * 64u * CHUNK; // + buffer + j * 4 KiB
         auto           uniform64 = [](const char* ptr) {
@@ -726,8 +750,8 @@ namespace
             const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
             return (static_cast<uint64_t>(hi) << 32) | lo;
         };
-        const uint64_t gA = uniform64(p.a + (A_KCONTIG ? (uint64_t)tm * TILE * p.lda : (uint64_t)tm * TILE));
-        const uint64_t gB = uniform64(p.b + (B_KCONTIG ? (uint64_t)tn * TILE * p.ldb : (uint64_t)tn * TILE));
+        const uint64_t gA = uniform64(p.a + (A_KCONTIG ? (uint64_t)tm * TILE * p.lda : (uint64_t)tm * TILE) * ES);
+        const uint64_t gB = uniform64(p.b + (B_KCONTIG ? (uint64_t)tn * TILE * p.ldb : (uint64_t)tn * TILE) * ES);
         auto stageAddr = [&](uint64_t panel, uint64_t perStage, uint32_t stage) { // clamped to the last stage
             return panel + (uint64_t)(stage < numStages ? stage : numStages - 1u) * perStage;
         };
@@ -740,15 +764,15 @@ namespace
         };
 
         uint32_t rdA[8], rdB[8];
-        readOffsets8<A_KCONTIG, WB>(wm, lane, rdA);
-        readOffsets8<B_KCONTIG, WB>(wn, lane, rdB);
+        readOffsets8<A_KCONTIG, WB, ES>(wm, lane, rdA);
+        readOffsets8<B_KCONTIG, WB, ES>(wn, lane, rdB);
 
-        i32x4v acc[WB][WB];
+        AccV acc[WB][WB];
 #pragma unroll
         for(uint32_t i = 0; i < WB; ++i)
 #pragma unroll
             for(uint32_t j = 0; j < WB; ++j)
-                acc[i][j] = i32x4v{0, 0, 0, 0};
+                acc[i][j] = AccV{0, 0, 0, 0};
 
         i32x4 fa[2][WB], fb[2][WB];
         // matrix instruction n of a K step: L-shaped shells, as in gemmTiledKernel16
@@ -758,14 +782,17 @@ namespace
                 ++d;
             const uint32_t r = n - d * d;
             const uint32_t i = r <= d ? d : r - d - 1u, j = r <= d ? r : d;
-            mfma16i8(acc[i][j], fb[s][j], fa[s][i]);
+            if constexpr(E == Elem::I8)
+                mfma16i8(acc[i][j], fb[s][j], fa[s][i]);
+            else
+                mfma16<E>(acc[i][j], fb[s][j], fa[s][i]);
         };
         // operand block x of K step s: x = 2 i is A block i, x = 2 i + 1 is B block i
         auto readAt = [&](uint32_t aAt, uint32_t bAt, uint32_t s, uint32_t x, uint32_t part) {
             if(x & 1u)
-                readBlock8<B_KCONTIG, WB>(lds + bAt, rdB, x >> 1, s, part, fb[s][x >> 1], 0u);
+                readBlock8<B_KCONTIG, WB, ES>(lds + bAt, rdB, x >> 1, s, part, fb[s][x >> 1], 0u);
             else
-                readBlock8<A_KCONTIG, WB>(lds + aAt, rdA, x >> 1, s, part, fa[s][x >> 1], 0u);
+                readBlock8<A_KCONTIG, WB, ES>(lds + aAt, rdA, x >> 1, s, part, fa[s][x >> 1], 0u);
         };
 
         uint64_t refillA, refillB; // stage kt + 2 of A, stage kt + 3 of B (clamped)
@@ -865,18 +892,26 @@ namespace
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
         waitVmcnt<0>();
         ldsBarrier();
-        storeTile16<i32x4v, int, WB>(acc, p, tm * TILE + wm * WT, tn * TILE + wn * WT, lane, lds + wave * (WB * 4096u));
+        storeTile16<AccV, OutT, WB>(acc, p, tm * TILE + wm * WT, tn * TILE + wn * WT, lane, lds + wave * (WB * 4096u));
     }
 
     template <bool A_KCONTIG, bool B_KCONTIG>
     __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) gemmTiledKernelI8(Params p)
     {
-        gemmTiledI8<A_KCONTIG, B_KCONTIG, 8>(p);
+        gemmTiled5<Elem::I8, int, A_KCONTIG, B_KCONTIG, 8>(p);
     }
     template <bool A_KCONTIG, bool B_KCONTIG>
     __global__ void __launch_bounds__(THREADS) gemmTiledKernelI8Small(Params p)
     {
-        gemmTiledI8<A_KCONTIG, B_KCONTIG, 4>(p);
+        gemmTiled5<Elem::I8, int, A_KCONTIG, B_KCONTIG, 4>(p);
+    }
+    // The 128 x 128 tile of f16 / bf16 runs the five-buffer body as well: with a stage lasting a quarter as
+    // long, the two-buffer scheme of gemmTiled16 keeps too little in flight (2048^3 f16: 710 TFLOP/s against 887
+    // here).  For the 256 x 256 tile the two-buffer kernel stays 1-2 % ahead (it is power-bound, not latency-bound).
+    template <Elem E, typename OutT, bool A_KCONTIG, bool B_KCONTIG>
+    __global__ void __launch_bounds__(THREADS) gemmTiledKernel16Small(Params p)
+    {
+        gemmTiled5<E, OutT, A_KCONTIG, B_KCONTIG, 4>(p);
     }
 
     // ------------------------------------------------------------------------------------------
@@ -1208,7 +1243,7 @@ namespace r355
             plan->grid_y       = 1;
             plan->block_x      = THREADS;
             plan->block_y      = 1;
-            plan->lds_bytes    = (fiveBuffers ? 5u * OPER_BYTES : NUM_STAGES * STAGE_BYTES) * tile / 256u;
+            plan->lds_bytes    = (fiveBuffers || tile == 128u ? 5u * OPER_BYTES : NUM_STAGES * STAGE_BYTES) * tile / 256u;
         }
         return R355_OK;
     }

@@ -53,7 +53,7 @@ def test_query_selects_kernel_family_and_reports_launch_shape():
     # 16-bit problems whose 256 x 256 tiles would leave most of the 256 CUs idle take the 128 x 128 tile
     plan = R.gemm_query(_args(m=2048, n=2048, k=2048))
     assert plan.kernel == R.KERNEL_TILED and (plan.macro_tile_m, plan.macro_tile_n) == (128, 128)
-    assert plan.grid_x == 256 and plan.lds_bytes == 65536
+    assert plan.grid_x == 256 and plan.lds_bytes == 81920
     plan = R.gemm_query(_args(m=4096, n=4096, k=4096))
     assert (plan.macro_tile_m, plan.grid_x) == (256, 256)
     plan = R.gemm_query(_args(m=2048, n=2048, k=2048, kernel=R.KERNEL_TILED))
