@@ -168,7 +168,10 @@ namespace
         if(beta == static_cast<AccE>(0))
         {
             // Transpose through the wave's own LDS so that a store instruction covers whole rows of
-            // the wave tile (128 to 512 bytes) with 128 bits per lane.
+            // the wave tile (128 to 512 bytes) with 128 bits per lane.  (The epilogue of a 256 x 256 int32 tile
+            // takes 7-9 us whatever else the chip is doing and however few instructions it is made of -- skipping
+            // the alpha multiplication and the per-store address arithmetic changed nothing: 256 KiB leave a CU at
+            // about 16 bytes per clock.)
             constexpr uint32_t OS         = sizeof(OutT);
             constexpr uint32_t ROW_BYTES  = 16u * WB * OS;
             constexpr uint32_t ROW_CHUNKS = ROW_BYTES / CHUNK; // 8, 16 or 32
@@ -397,8 +400,7 @@ namespace
         // bytes per row and the loads fill the rest with zeros
         const uint32_t kBytes    = p.k * ES;
         const uint32_t numStages = (kBytes + 2u * STAGE_KB - 1u) / (2u * STAGE_KB) * 2u;
-        auto           validOf   = [&](uint32_t st) {
-            st = st < numStages ? st : numStages - 1u;
+        auto           validOf   = [&](uint32_t st) { // 0 for the padding stage and for refills past the end: no traffic
             return st * STAGE_KB >= kBytes ? 0u : (kBytes - st * STAGE_KB < STAGE_KB ? kBytes - st * STAGE_KB : STAGE_KB);
         };
         auto rsrcAt = [](uint64_t addr, uint32_t records) { // raw buffer, 32-bit data format, no swizzle
@@ -470,7 +472,7 @@ namespace
         // in that time, so the other work is dealt out one piece per matrix instruction, in groups of
         // four: read (part 0), read (part 1), direct load (second step), nothing -- and nothing moves
         // between pieces (groups of two with the small wave tile: read, read + direct load).  Every stage
-        // runs the same code: past the end the refill is clamped to the last stage and the operands read
+        // runs the same code: past the end the refill has nothing in range (it writes zeros) and the operands read
         // ahead are never used.
         constexpr uint32_t LOAD_Q = QS > 2u ? 2u : QS - 1u;
         auto stageBody = [&](uint32_t kt, char* cur, char* nxt) {
@@ -524,7 +526,7 @@ namespace
             stageBody(kt + 1, stage1, stage0);
         }
 
-        // the clamped refills of the last two stages are still landing in the buffers the epilogue reuses
+        // the refills past the end (zeros) are still landing in the buffers the epilogue reuses
         __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
         __syncthreads();
         // the last matrix instructions are still in the pipeline and the compiler does not know it
@@ -551,8 +553,8 @@ namespace
     // of 64.  Stage kt lives in A buffer kt % 2 and B buffer kt % 3, so six stages bring every buffer
     // back to its starting role; the K loop is unrolled six times with a single exit (an exit after
     // every stage makes the register allocator spill hundreds of registers) and the up to five
-    // remaining stages follow as straight-line code, so K may be any multiple of 128.  Loads past the
-    // last stage are clamped to it -- they land in buffers nobody reads any more -- so every stage
+    // remaining stages follow as straight-line code, so any number of stages runs.  Loads past the
+    // last stage have nothing in range -- they write zeros into buffers nobody reads any more -- so every stage
     // issues the same 16 loads and the wait before its barrier is always "all but the youngest 8".
     //
     // The direct loads are inline assembly: for the builtin the compiler cannot tell which buffer a
@@ -742,7 +744,8 @@ namespace
         const uint32_t kBytes    = p.k * ES;
         const uint32_t numStages = (kBytes + STAGE_KB - 1u) / STAGE_KB;
         const uint32_t lastBytes = kBytes - (numStages - 1u) * STAGE_KB;
-        auto           validOf   = [&](uint32_t stage) { return stage + 1u >= numStages ? lastBytes : STAGE_KB; };
+        // (refills past the last stage are issued like all others but with nothing in range: they cost no memory traffic)
+        auto validOf = [&](uint32_t stage) { return stage + 1u < numStages ? STAGE_KB : (stage + 1u == numStages ? lastBytes : 0u); };
         const uint32_t dmaDst    = ldsBase + wave * 64u * CHUNK; // + buffer + j * 4 KiB
         auto           uniform64 = [](const char* ptr) {
             const uint64_t v  = reinterpret_cast<uint64_t>(ptr);
@@ -887,7 +890,7 @@ namespace
             }
         }
 
-        // the clamped loads of the last stages are still landing in buffers the epilogue reuses, and the
+        // the loads past the last stage (zeros) are still landing in buffers the epilogue reuses, and the
         // last matrix instructions are still in the pipeline (the compiler does not know either)
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
         waitVmcnt<0>();
@@ -965,7 +968,8 @@ namespace
         // the loads produce themselves (see tailOffset)
         const uint32_t numStages = (p.k + STAGE_KB - 1u) / STAGE_KB;
         const uint32_t lastBytes = p.k - (numStages - 1u) * STAGE_KB;
-        auto           validOf   = [&](uint32_t stage) { return stage + 1u >= numStages ? lastBytes : STAGE_KB; };
+        // (refills past the last stage are issued like all others but with nothing in range: they cost no memory traffic)
+        auto validOf = [&](uint32_t stage) { return stage + 1u < numStages ? STAGE_KB : (stage + 1u == numStages ? lastBytes : 0u); };
         const uint32_t dmaDst    = ldsBase + wave * 64u * CHUNK;
         auto           uniform64 = [](const char* ptr) {
             const uint64_t v  = reinterpret_cast<uint64_t>(ptr);
