@@ -31,6 +31,8 @@
 //                register allocator then shuffles them through the K loop), so the kernels fix
 //                the instruction order themselves: one LDS read or direct load per matrix
 //                instruction, pinned by scheduling barriers
+//   shapes       m, n multiples of 16 and k a multiple of a 16-byte chunk: edge tiles clamp their loads and guard
+//                their stores, a partial last K stage is completed with zeros by out-of-range buffer loads
 //   grid         1-D, remapped so that each XCD (workgroup id mod 8) owns a compact
 //                rectangle of tiles and walks it in 4-row groups (L2 reuse of A and B)
 //
