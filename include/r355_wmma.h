@@ -69,7 +69,8 @@ typedef enum
  * Argument order and meaning follow the reference kernel signature
  * (test/gemm/gemm_kernel_base.hpp:101-114): leading dimensions in elements.
  * Supported (in -> out, accumulate): f16 -> f32|f16 (f32), bf16 -> f32|bf16 (f32),
- * e4m3 -> f32 (f32), i8 -> i32 (i32, alpha/beta truncated to int32), f32 -> f32 (f32), f64 -> f64 (f64).
+ * e4m3 -> f32 (f32), i8 -> i32|i8 (i32, alpha/beta truncated to int32; an i8 result is the low 8 bits, as the
+ * reference's static_cast narrows it), f32 -> f32 (f32), f64 -> f64 (f64).
  * beta == 0 means C is never read and may be NULL.
  *
  * sparse24 != 0: A is 2:4 structured-sparse along k, row-major, 1-byte elements:

@@ -276,6 +276,31 @@ int orc_gemm(int         in_type,
         const int32_t* pc = (const int32_t*)c;
         int32_t*       pd = (int32_t*)d;
         int32_t        ia = (int32_t)alpha, ib = (int32_t)beta;
+        if(out_type == ORC_I8)
+        {
+            /* (int8, int8, int32) of test/gemm/gemm_common_test_params.hpp:52: C and D are int8, the
+             * arithmetic is int32 and the result is narrowed by static_cast (test/reference_impl.hpp:74-77),
+             * i.e. its low 8 bits */
+            const int8_t* qc = (const int8_t*)c;
+            int8_t*       qd = (int8_t*)d;
+#pragma omp parallel for schedule(static)
+            for(int64_t i = 0; i < (int64_t)m; ++i)
+            {
+                for(uint32_t j = 0; j < n; ++j)
+                {
+                    int32_t accum = 0;
+                    for(uint32_t h = 0; h < k; ++h)
+                    {
+                        accum += (int32_t)pa[mat_index((uint32_t)i, h, lda, layout_a)]
+                                 * (int32_t)pb[mat_index(h, j, ldb, layout_b)];
+                    }
+                    const uint32_t cterm
+                        = ib == 0 ? 0u : (uint32_t)ib * (uint32_t)(int32_t)qc[mat_index((uint32_t)i, j, ldc, layout_c)];
+                    qd[mat_index((uint32_t)i, j, ldd, layout_d)] = (int8_t)(uint8_t)((uint32_t)ia * (uint32_t)accum + cterm);
+                }
+            }
+            return 0;
+        }
         if(out_type != ORC_I32)
             return -1;
 #pragma omp parallel for schedule(static)

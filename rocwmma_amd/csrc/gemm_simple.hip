@@ -190,7 +190,7 @@ namespace
         case R355_F16: return out == R355_F32 || out == R355_F16;
         case R355_BF16: return out == R355_F32 || out == R355_BF16;
         case R355_E4M3: return out == R355_F32;
-        case R355_I8: return out == R355_I32;
+        case R355_I8: return out == R355_I32 || out == R355_I8;
         case R355_F32: return out == R355_F32;
         case R355_F64: return out == R355_F64;
         default: return false;
@@ -248,7 +248,9 @@ namespace r355
             return g.out_type == R355_F32 ? launchBlocks<bfloat16_t, float32_t, float32_t>(g, stream, blk)
                                           : launchBlocks<bfloat16_t, bfloat16_t, float32_t>(g, stream, blk);
         case R355_E4M3: return launchBlocks<float8_t, float32_t, float32_t>(g, stream, blk);
-        case R355_I8: return launchBlocks<int8_t, int32_t, int32_t>(g, stream, blk);
+        case R355_I8:
+            return g.out_type == R355_I32 ? launchBlocks<int8_t, int32_t, int32_t>(g, stream, blk)
+                                          : launchBlocks<int8_t, int8_t, int32_t>(g, stream, blk);
         case R355_F32: return launchBlocks<float32_t, float32_t, float32_t>(g, stream, blk);
         case R355_F64: return launchBlocks<float64_t, float64_t, float64_t>(g, stream, blk);
         default: return fail(R355_ERR_UNSUPPORTED, "gemm: unknown in_type %d", g.in_type);

@@ -900,15 +900,15 @@ namespace
         storeTile16<AccV, OutT, WB>(acc, p, tm * TILE + wm * WT, tn * TILE + wn * WT, lane, lds + wave * (WB * 4096u));
     }
 
-    template <bool A_KCONTIG, bool B_KCONTIG>
+    template <typename OutT, bool A_KCONTIG, bool B_KCONTIG>
     __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) gemmTiledKernelI8(Params p)
     {
-        gemmTiled5<Elem::I8, int, A_KCONTIG, B_KCONTIG, 8>(p);
+        gemmTiled5<Elem::I8, OutT, A_KCONTIG, B_KCONTIG, 8>(p);
     }
-    template <bool A_KCONTIG, bool B_KCONTIG>
+    template <typename OutT, bool A_KCONTIG, bool B_KCONTIG>
     __global__ void __launch_bounds__(THREADS) gemmTiledKernelI8Small(Params p)
     {
-        gemmTiled5<Elem::I8, int, A_KCONTIG, B_KCONTIG, 4>(p);
+        gemmTiled5<Elem::I8, OutT, A_KCONTIG, B_KCONTIG, 4>(p);
     }
     // The 128 x 128 tile of f16 / bf16 runs the five-buffer body as well: with a stage lasting a quarter as
     // long, the two-buffer scheme of gemmTiled16 keeps too little in flight (2048^3 f16: 710 TFLOP/s against 887
@@ -1153,9 +1153,9 @@ namespace
             if constexpr(E == Elem::I8)
             {
                 if(tile == 128u)
-                    hipLaunchKernelGGL((gemmTiledKernelI8Small<AK, BK>), grid, block, 0, stream, p);
+                    hipLaunchKernelGGL((gemmTiledKernelI8Small<OutT, AK, BK>), grid, block, 0, stream, p);
                 else
-                    hipLaunchKernelGGL((gemmTiledKernelI8<AK, BK>), grid, block, 0, stream, p);
+                    hipLaunchKernelGGL((gemmTiledKernelI8<OutT, AK, BK>), grid, block, 0, stream, p);
             }
             else if constexpr(E == Elem::E4M3)
             {
@@ -1220,7 +1220,7 @@ namespace r355
         const bool pairOk = (g.in_type == R355_F16 && (g.out_type == R355_F16 || g.out_type == R355_F32))
                             || (g.in_type == R355_BF16 && (g.out_type == R355_BF16 || g.out_type == R355_F32))
                             || (g.in_type == R355_E4M3 && g.out_type == R355_F32)
-                            || (g.in_type == R355_I8 && g.out_type == R355_I32);
+                            || (g.in_type == R355_I8 && (g.out_type == R355_I32 || g.out_type == R355_I8));
         if(!pairOk)
             return fail(R355_ERR_UNSUPPORTED, "tiled gemm: no kernel for in_type %d -> out_type %d", g.in_type, g.out_type);
         const uint32_t es = dtypeBytes(g.in_type), os = dtypeBytes(g.out_type);
@@ -1291,7 +1291,9 @@ namespace r355
             return g.out_type == R355_BF16 ? launchLayouts<Elem::BF16, __bf16>(aK, bK, tile, p, stream)
                                            : launchLayouts<Elem::BF16, float>(aK, bK, tile, p, stream);
         case R355_E4M3: return launchLayouts<Elem::E4M3, float>(aK, bK, tile, p, stream);
-        case R355_I8: return launchLayouts<Elem::I8, int>(aK, bK, tile, p, stream);
+        case R355_I8:
+            return g.out_type == R355_I32 ? launchLayouts<Elem::I8, int>(aK, bK, tile, p, stream)
+                                          : launchLayouts<Elem::I8, signed char>(aK, bK, tile, p, stream);
         default: return fail(R355_ERR_UNSUPPORTED, "tiled gemm: unknown in_type %d", g.in_type);
         }
     }

@@ -376,6 +376,22 @@ def test_tiled_kernel_k_tails(in_t, out_t, ks, la, lb, kernel):
         _check(in_t, out_t, got, want, w32)
 
 
+@pytest.mark.parametrize("kernel", ["simple", "tiled", "tiled_128"])
+@pytest.mark.parametrize("la,lb,ldl", [(O.ROW, O.COL, O.ROW), (O.COL, O.ROW, O.COL), (O.ROW, O.ROW, O.ROW)])
+def test_int8_to_int8_output(kernel, la, lb, ldl):
+    # the reference's (int8, int8, int32) type tuple (test/gemm/gemm_common_test_params.hpp:52): int8 C and D,
+    # int32 arithmetic, the result narrowed to its low byte; bit-exact, edge tiles and a K tail included
+    sel = {"simple": R.KERNEL_SIMPLE, **TILE_SELECTORS}[kernel]
+    for m, n, k in ((256, 384, 512), (272, 144, 160)):
+        a, b = O.uniform_int8(91, m * k), O.uniform_int8(92, k * n)
+        c = O.uniform_int8(93, m * n)
+        for alpha, beta in ((1.0, 0.0), (3.0, -2.0)):
+            cc = None if beta == 0.0 else c
+            want = O.gemm(O.I8, O.I8, la, lb, ldl, ldl, m, n, k, a, b, cc, alpha, beta)
+            got = _run(O.I8, O.I8, la, lb, ldl, ldl, m, n, k, a, b, cc, alpha, beta, sel)
+            assert np.array_equal(got, want), (m, n, k, alpha, beta)
+
+
 def test_tiled_kernel_many_tiles_xcd_mapping():
     # 5 x 3 tiles: a tile count that is not a multiple of 8 and a partial row group
     m, n, k = 1280, 768, 256

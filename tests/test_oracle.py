@@ -96,6 +96,21 @@ def test_gemm_int8_all_layouts_vs_numpy(la, lb, lc, ld):
     assert np.array_equal(O.as_matrix(d, m, n, ld).astype(np.int64), want)
 
 
+@pytest.mark.parametrize("la,lb,lc,ld", [(O.ROW, O.COL, O.ROW, O.ROW), (O.COL, O.ROW, O.COL, O.ROW), (O.ROW, O.ROW, O.COL, O.COL)])
+def test_gemm_int8_to_int8_is_the_low_byte_of_the_int32_result(la, lb, lc, ld):
+    # (int8, int8, int32) of the reference's extended type list: int32 arithmetic, static_cast<int8_t> at the end,
+    # pinned here by exact int64 arithmetic reduced modulo 256 (sums well beyond the int8 range)
+    m, n, k = 17, 21, 48
+    A = O.uniform_int8(21, m * k).reshape(m, k)
+    B = O.uniform_int8(22, k * n).reshape(k, n)
+    C = O.uniform_int8(23, m * n).reshape(m, n)
+    full = 3 * (A.astype(np.int64) @ B.astype(np.int64)) + (-2) * C.astype(np.int64)
+    want = (full & 0xFF).astype(np.uint8).view(np.int8)
+    assert np.abs(full).max() > 1000
+    d = O.gemm(O.I8, O.I8, la, lb, lc, ld, m, n, k, O.to_flat(A, la), O.to_flat(B, lb), O.to_flat(C, lc), 3.0, -2.0)
+    assert d.dtype == np.int8 and np.array_equal(O.as_matrix(d, m, n, ld), want)
+
+
 def test_gemm_int8_max_magnitude_k8192():
     # |sum| reaches 8192 * 128 * 128 = 2^27 exactly: no overflow, closed form
     m, n, k = 2, 3, 8192
