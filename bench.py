@@ -173,6 +173,9 @@ def run_extras(R, O, np, torch, args):
         out[name] = {"ms": round(ms, 4), "value": round(tf, 2), "unit": unit, "peak": peak * peak_scale,
                      "frac": round(tf / (peak * peak_scale), 4)}
 
+    if s == 8192:  # a problem with too few 256 x 256 tiles for the 256 CUs: the 128 x 128 macro tile
+        gemm_case("gemm_f16_nt_2048x2048x8192", R.F16, R.F16, R.COL_MAJOR, R.ROW_MAJOR, rnd16(2048 * s, False),
+                  rnd16(s * 2048, False), PEAK_TFLOPS["f16"], "TFLOP/s", mm=2048, nn=2048, kk=s)
     abf, bbf = rnd16(s * s, True), rnd16(s * s, True)
     gemm_case("gemm_bf16_nt_8192", R.BF16, R.BF16, R.COL_MAJOR, R.ROW_MAJOR, abf, bbf, PEAK_TFLOPS["bf16"], "TFLOP/s")
     af16, bf16_ = rnd16(s * s, False), rnd16(s * s, False)
@@ -180,6 +183,7 @@ def run_extras(R, O, np, torch, args):
     i8 = lambda nel: torch.randint(-128, 128, (nel,), dtype=torch.int16, device="cuda").to(torch.int8)
     ai8, bi8 = i8(s * s), i8(s * s)
     gemm_case("gemm_i8_tn_8192", R.I8, R.I32, R.ROW_MAJOR, R.COL_MAJOR, ai8, bi8, PEAK_TFLOPS["i8"], "TOP/s")
+    gemm_case("gemm_i8_nt_8192", R.I8, R.I32, R.COL_MAJOR, R.ROW_MAJOR, ai8, bi8, PEAK_TFLOPS["i8"], "TOP/s")
     # e4m3: N(0, 1) draws rounded to nearest-even and saturated to the finite range (|x| <= 448;
     # scale 1.0, so saturation never triggers in practice)
     f8 = lambda nel: torch.randn(nel, device="cuda").clamp_(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8)

@@ -125,3 +125,50 @@ def test_compress_24_host_roundtrip_and_rejection():
     with pytest.raises(R.R355Error) as e:
         R.compress_24(bad)
     assert e.value.code == -6 and "row 3" in str(e.value)
+
+
+@pytest.mark.gpu
+def test_entry_points_can_be_captured_in_a_hip_graph():
+    """The C ABI allocates nothing and only launches kernels on the stream it is given, so its calls can be
+    recorded into a HIP graph.  Replayed three times with the operands changed in between (by eager work of
+    the same process), every replay must reproduce the eager results bit for bit."""
+    import torch
+
+    m, n, k = 512, 384, 640
+    bsz, feat, dim = 256, 27, 128
+    a16 = (torch.rand(m * k, device="cuda") * 2 - 1).half()
+    b16 = (torch.rand(k * n, device="cuda") * 2 - 1).half()
+    a8 = torch.randint(-128, 128, (m * k,), dtype=torch.int16, device="cuda").to(torch.int8)
+    b8 = torch.randint(-128, 128, (k * n,), dtype=torch.int16, device="cuda").to(torch.int8)
+    x = torch.randn(bsz * feat * dim, device="cuda").half()
+    d16, d8 = torch.empty(m * n, dtype=torch.float16, device="cuda"), torch.empty(m * n, dtype=torch.int32, device="cuda")
+    o = torch.empty(bsz * (dim + feat * (feat - 1) // 2), dtype=torch.float16, device="cuda")
+
+    def launch(stream):
+        R.gemm(R.F16, R.F16, m, n, k, a16, b16, None, d16, 1.0, 0.0, R.COL_MAJOR, R.ROW_MAJOR, R.ROW_MAJOR, R.ROW_MAJOR,
+               stream=stream)
+        R.gemm(R.I8, R.I32, m, n, k, a8, b8, None, d8, 1.0, 0.0, R.ROW_MAJOR, R.COL_MAJOR, R.ROW_MAJOR, R.ROW_MAJOR,
+               kernel=R.KERNEL_TILED, stream=stream)
+        R.dlrm_fwd(R.F16, x, o, feat, dim, bsz, stream=stream)
+
+    side = torch.cuda.Stream()  # default priority
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        launch(side)  # warm-up outside the capture
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            launch(side)
+    torch.cuda.synchronize()
+    for rep in range(3):
+        a16.copy_((torch.rand(m * k, device="cuda") * 2 - 1).half())
+        a8.copy_(torch.randint(-128, 128, (m * k,), dtype=torch.int16, device="cuda").to(torch.int8))
+        x.copy_(torch.randn(bsz * feat * dim, device="cuda").half())
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = (d16.clone(), d8.clone(), o.clone())
+        d16.zero_(), d8.zero_(), o.zero_()
+        launch(None)
+        torch.cuda.synchronize()
+        for g, e in zip(got, (d16, d8, o)):
+            assert torch.equal(g.view(torch.uint8), e.view(torch.uint8)), rep
