@@ -8,6 +8,7 @@
 //   bf16  8/lane: v_mfma_f32_32x32x16_bf16  / 16x16x32_bf16   4/lane: 32x32x8bf16_1k / 16x16x16bf16_1k
 //   int8 16/lane: v_mfma_i32_32x32x32_i8    / 16x16x64_i8     8/lane: 32x32x16_i8 / 16x16x32_i8
 //   e4m3  8/lane: v_mfma_f32_32x32x16_fp8_fp8 / 16x16x32_fp8_fp8   (OCP encoding on gfx950)
+//   e5m2  8/lane: v_mfma_f32_32x32x16_bf8_bf8 / 16x16x32_bf8_bf8   (OCP encoding on gfx950)
 //   f32   1/lane: v_mfma_f32_32x32x2f32     / 16x16x4f32
 //   f64   1/lane: v_mfma_f64_16x16x4f64 (16x16 blocks only)
 #ifndef ROCWMMA_MFMA_HPP
@@ -113,6 +114,16 @@ namespace rocwmma
                         acc = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(av, bv, acc, 0, 0, 0);
                     else
                         acc = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(av, bv, acc, 0, 0, 0);
+                }
+                else if constexpr(is_bf8_v<InputT> && KW == 8u)
+                {
+                    long av, bv;
+                    __builtin_memcpy(&av, a, 8);
+                    __builtin_memcpy(&bv, b, 8);
+                    if constexpr(BlockDim == 32u)
+                        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf8_bf8(av, bv, acc, 0, 0, 0);
+                    else
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf8_bf8(av, bv, acc, 0, 0, 0);
                 }
                 else if constexpr(std::is_same_v<InputT, float32_t> && KW == 1u)
                 {

@@ -81,6 +81,8 @@ namespace rocwmma
         template <typename T>
         inline constexpr bool is_fp8_v = std::is_same_v<T, float8_t>;
         template <typename T>
+        inline constexpr bool is_bf8_v = std::is_same_v<T, bfloat8_t>;
+        template <typename T>
         inline constexpr bool is_i8_v = std::is_same_v<T, int8_t> || std::is_same_v<T, uint8_t>;
 
         // Orthogonal orientation

@@ -159,6 +159,34 @@ SHAPES = {0: [(16, 16), (16, 32), (32, 8), (32, 16)], 1: [(16, 16), (16, 32), (3
           4: [(16, 4), (16, 16), (32, 2), (32, 8)], 5: [(16, 16), (32, 16)], 6: [(16, 4), (16, 8), (16, 16), (16, 32)]}
 
 
+@pytest.mark.parametrize("a_row,b_row,c_row", [(1, 0, 1), (0, 1, 0), (1, 1, 1), (0, 0, 0)])
+def test_mma_sync_e5m2_single_tile(a_row, b_row, c_row):
+    """bfloat8_t (OCP e5m2) fragments: an e5m2 code is the high byte of the f16 with the same value, so the
+    operands decode exactly through numpy's float16 and the oracle runs its f32 GEMM on the decoded values
+    (the reference lists the type in its test tuples, test/gemm/gemm_common_test_params.hpp:73-87, but has no
+    matrix instruction for it on any gfx9, mfma_impl.hpp:1113-1170: parity is pinned by the decode alone)."""
+    rng = np.random.default_rng(7)
+    for blk, bk in [(16, 32), (16, 64), (32, 16), (32, 32)]:
+        m = n = blk
+        # finite codes only (exponent field 31 is inf / NaN): sign | exponent 0..30 | 2 mantissa bits
+        a = (rng.integers(0, 0x7C, m * bk) | (rng.integers(0, 2, m * bk) << 7)).astype(np.uint8)
+        b = (rng.integers(0, 0x7C, bk * n) | (rng.integers(0, 2, bk * n) << 7)).astype(np.uint8)
+        a = np.where((a & 0x7F) > 0x47, a & 0xC7 | 0x40, a).astype(np.uint8)  # keep |x| <= 7 so that sums stay small
+        b = np.where((b & 0x7F) > 0x47, b & 0xC7 | 0x40, b).astype(np.uint8)
+        dec = lambda x: (x.astype(np.uint16) << 8).view(np.float16).astype(np.float32)
+        c = O.uniform_pm1(3, m * n)
+        la, lb, lc = (O.ROW if a_row else O.COL), (O.ROW if b_row else O.COL), (O.ROW if c_row else O.COL)
+        want = O.gemm(O.F32, O.F32, la, lb, lc, lc, m, n, bk, dec(a), dec(b), c, 1.0, 1.0)
+        da, db, dc = to_device(a), to_device(b), to_device(c)
+        dd = device_filled(m * n, np.float32, 0xFF)
+        rc = api_lib().api_mma_tile(7, blk, bk, a_row, b_row, c_row, ctypes.c_void_p(da.data_ptr()),
+                                    ctypes.c_void_p(db.data_ptr()), ctypes.c_void_p(dc.data_ptr()),
+                                    ctypes.c_void_p(dd.data_ptr()), bk if a_row else m, n if b_row else bk, n if c_row else m)
+        assert rc == 0, (blk, bk)
+        g, w = to_host(dd, np.float32).astype(np.float64), want.astype(np.float64)
+        assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= 1e-2, (blk, bk)
+
+
 @pytest.mark.parametrize("type_id", sorted(TYPES))
 @pytest.mark.parametrize("a_row,b_row,c_row", [(1, 0, 1), (0, 1, 0), (1, 1, 1), (0, 0, 0)])
 def test_mma_sync_single_tile_matches_oracle(type_id, a_row, b_row, c_row):
