@@ -60,7 +60,9 @@ namespace
         F16,
         BF16,
         E4M3,
-        I8
+        I8,
+        F32,
+        F64
     };
 
     constexpr uint32_t TILE_M      = 256;
@@ -94,6 +96,16 @@ namespace
     struct ElemTraits<Elem::I8>
     {
         static constexpr uint32_t Bytes = 1;
+    };
+    template <>
+    struct ElemTraits<Elem::F32>
+    {
+        static constexpr uint32_t Bytes = 4;
+    };
+    template <>
+    struct ElemTraits<Elem::F64>
+    {
+        static constexpr uint32_t Bytes = 8;
     };
 
     struct Params
@@ -191,14 +203,29 @@ namespace
 #pragma unroll
                     for(uint32_t j = 0; j < WB; ++j)
                     {
-                        OutV out;
+                        if constexpr(sizeof(AccE) == 8)
+                        {
+                            // f64 accumulators: element e is column 4 e + lane / 16 of the block
 #pragma unroll
-                        for(uint32_t e = 0; e < 4; ++e)
-                            out[e] = static_cast<OutT>(alpha * acc[i][j][e]);
-                        // 16 consecutive rows take 16 (8) different chunk slots
-                        const uint32_t byteInRow = (16u * j + 4u * g) * OS;
-                        const uint32_t c = byteInRow / CHUNK, within = byteInRow % CHUNK;
-                        *reinterpret_cast<OutV*>(scratch + row * ROW_BYTES + ((c ^ (row & SWZ)) * CHUNK) + within) = out;
+                            for(uint32_t e = 0; e < 4; ++e)
+                            {
+                                const uint32_t byteInRow = (16u * j + 4u * e + g) * OS;
+                                const uint32_t c = byteInRow / CHUNK, within = byteInRow % CHUNK;
+                                *reinterpret_cast<OutT*>(scratch + row * ROW_BYTES + ((c ^ (row & SWZ)) * CHUNK) + within)
+                                    = static_cast<OutT>(alpha * acc[i][j][e]);
+                            }
+                        }
+                        else
+                        {
+                            OutV out;
+#pragma unroll
+                            for(uint32_t e = 0; e < 4; ++e)
+                                out[e] = static_cast<OutT>(alpha * acc[i][j][e]);
+                            // 16 consecutive rows take 16 (8) different chunk slots
+                            const uint32_t byteInRow = (16u * j + 4u * g) * OS;
+                            const uint32_t c = byteInRow / CHUNK, within = byteInRow % CHUNK;
+                            *reinterpret_cast<OutV*>(scratch + row * ROW_BYTES + ((c ^ (row & SWZ)) * CHUNK) + within) = out;
+                        }
                     }
                 }
                 __builtin_amdgcn_wave_barrier(); // the same wave reads back what it wrote (LDS is in order per wave)
@@ -219,6 +246,30 @@ namespace
             return;
         }
         // C may alias D, so loads cannot move above earlier stores: fetch a block row of C at a time
+        if constexpr(sizeof(AccE) == 8)
+        {
+            // f64 accumulators: element e is column 4 e + lane / 16 of the block
+#pragma unroll
+            for(uint32_t i = 0; i < WB; ++i)
+            {
+                const uint32_t row = m0 + 16u * i + r16;
+                OutT           cv[WB][4];
+#pragma unroll
+                for(uint32_t j = 0; j < WB; ++j)
+#pragma unroll
+                    for(uint32_t e = 0; e < 4; ++e)
+                        if(row < p.m && n0 + 16u * j < p.n)
+                            cv[j][e] = *reinterpret_cast<const OutT*>(p.c + ((uint64_t)row * p.ldc + n0 + 16u * j + 4u * e + g) * sizeof(OutT));
+#pragma unroll
+                for(uint32_t j = 0; j < WB; ++j)
+#pragma unroll
+                    for(uint32_t e = 0; e < 4; ++e)
+                        if(row < p.m && n0 + 16u * j < p.n)
+                            *reinterpret_cast<OutT*>(p.d + ((uint64_t)row * p.ldd + n0 + 16u * j + 4u * e + g) * sizeof(OutT))
+                                = static_cast<OutT>(alpha * acc[i][j][e] + beta * static_cast<AccE>(cv[j][e]));
+            }
+            return;
+        }
 #pragma unroll
         for(uint32_t i = 0; i < WB; ++i)
         {
@@ -585,7 +636,11 @@ namespace
     template <uint32_t WB, uint32_t ES = 1>
     __device__ __forceinline__ uint32_t swzMN8(uint32_t krow)
     {
-        if constexpr(ES == 2)
+        if constexpr(ES == 8)
+            return ((krow >> 1) & 1u) << 3; // f64: a 32-lane pass reads two k-rows 2 apart, 128 bytes each
+        else if constexpr(ES == 4)
+            return ((krow >> 2) & 3u) << 2; // f32: a wave reads k-rows 4 apart, 64 bytes each
+        else if constexpr(ES == 2)
             return ((krow & 3u) << 2) | (((krow >> 3) & 1u) << 1); // 16-bit elements: as in gemmTiled16
         else if constexpr(WB == 8)
             return (krow & 7u) | ((krow >> 1) & 8u); // 256-byte k-rows, 16 chunks
@@ -655,6 +710,23 @@ namespace
             for(uint32_t i = 0; i < WB; ++i)
                 rd[i] = kr * 32u * WB + (((w * WB + i) ^ swzMN8<WB>(kr)) * CHUNK) + (t & 1u) * 8u;
         }
+        else if constexpr(ES == 8)
+        {
+            // f64: element e of the lane's two K values is k-row 2 (lane / 16) + e of the K step, column lane % 16
+            const uint32_t kr = 2u * g;
+#pragma unroll
+            for(uint32_t i = 0; i < WB; ++i)
+                rd[i] = kr * 256u * WB + ((((w * 8u * WB + 8u * i) ^ swzMN8<WB, 8>(kr)) + (t >> 1)) * CHUNK) + (t & 1u) * 8u;
+        }
+        else if constexpr(ES == 4)
+        {
+            // f32 (no transposing read for 32-bit elements): element e of the lane's four K values is k-row
+            // 4 (lane / 16) + e of the K step, column lane % 16 of the block -- 64 consecutive bytes per 16 lanes
+            const uint32_t kr = 4u * g;
+#pragma unroll
+            for(uint32_t i = 0; i < WB; ++i)
+                rd[i] = kr * 128u * WB + ((((w * 4u * WB + 4u * i) ^ swzMN8<WB, 4>(kr)) + (t >> 2)) * CHUNK) + (t & 3u) * 4u;
+        }
         else
         {
             // 16-bit: k-row 8 (lane / 16) + (lane % 16) / 4 of the K step's first half, 8-byte piece 4 i + lane % 4
@@ -689,6 +761,17 @@ namespace
             const i32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lp)(tile + rd[i] + (64u * s + 8u * part) * 32u * WB));
             dst[at + 2u * part] = v[0], dst[at + 2u * part + 1u] = v[1];
         }
+        else if constexpr(ES == 8)
+        {
+            const i32x2 v = *reinterpret_cast<const i32x2*>(tile + rd[i] + (8u * s + part) * 256u * WB);
+            dst[at + 2u * part] = v[0], dst[at + 2u * part + 1u] = v[1];
+        }
+        else if constexpr(ES == 4)
+        {
+            const char* q = tile + rd[i] + (16u * s + 2u * part) * 128u * WB;
+            dst[at + 2u * part]      = *reinterpret_cast<const int*>(q);
+            dst[at + 2u * part + 1u] = *reinterpret_cast<const int*>(q + 128u * WB);
+        }
         else
         {
             using lp      = __attribute__((address_space(3))) trv4*;
@@ -708,13 +791,39 @@ namespace
         asm volatile("v_mfma_i32_16x16x64_i8 %0, %1, %2, %0" : "+a"(acc) : "v"(x), "v"(y));
     }
 
+    // f32 on v_mfma_f32_16x16x4_f32: a lane's 16 bytes are four K values, consumed by four instructions
+    // (instruction e multiplies element e of every lane: k = 4 (lane / 16) + e of each 16-wide K step)
+    __device__ __forceinline__ void mfma16f32(f32x4& acc, i32x4 x, i32x4 y)
+    {
+#pragma unroll
+        for(uint32_t e = 0; e < 4; ++e)
+            asm volatile("v_mfma_f32_16x16x4_f32 %0, %1, %2, %0" : "+a"(acc) : "v"(x[e]), "v"(y[e]));
+    }
+
+    // f64 on v_mfma_f64_16x16x4_f64: a lane's 16 bytes are two K values (k = 2 (lane / 16) + e of each 8-wide K
+    // step) for two instructions.  An accumulator block is 8 registers, so only the 4 x 4 wave tile fits; its
+    // elements are rows lane / 16 + 4 e of column lane % 16 (with the operands swapped as everywhere here:
+    // columns lane / 16 + 4 e of row lane % 16), unlike the four consecutive ones of the 32-bit accumulators.
+    using f64x4 = double __attribute__((ext_vector_type(4)));
+    __device__ __forceinline__ void mfma16f64(f64x4& acc, i32x4 x, i32x4 y)
+    {
+#pragma unroll
+        for(uint32_t e = 0; e < 2; ++e)
+        {
+            const double xe = __builtin_bit_cast(double, i32x2{x[2u * e], x[2u * e + 1u]});
+            const double ye = __builtin_bit_cast(double, i32x2{y[2u * e], y[2u * e + 1u]});
+            asm volatile("v_mfma_f64_16x16x4_f64 %0, %1, %2, %0" : "+a"(acc) : "v"(xe), "v"(ye));
+        }
+    }
+
     template <Elem E, typename OutT, bool A_KCONTIG, bool B_KCONTIG, uint32_t WB>
     __device__ __forceinline__ void gemmTiled5(const Params& p)
     {
         static_assert(WB == 8 || WB == 4, "wave tile of 8 x 8 or 4 x 4 blocks");
+        static_assert(E != Elem::F64 || WB == 4, "f64 accumulators of an 8 x 8 wave tile would need 512 registers");
         static_assert(E != Elem::E4M3, "e4m3 has its own stage structure");
         constexpr uint32_t ES = ElemTraits<E>::Bytes;
-        using AccV            = std::conditional_t<E == Elem::I8, i32x4v, f32x4>;
+        using AccV            = std::conditional_t<E == Elem::I8, i32x4v, std::conditional_t<E == Elem::F64, f64x4, f32x4>>;
         constexpr uint32_t TILE = 32u * WB, WT = 16u * WB; // macro tile and wave tile edge
         constexpr uint32_t OPER = TILE * STAGE_KB; // bytes of one operand per stage: 32 or 16 KiB
         constexpr uint32_t XS = 2u * WB, QS = WB / 2u; // operand blocks per K step, matrix instructions per block
@@ -789,6 +898,10 @@ namespace
             const uint32_t i = r <= d ? d : r - d - 1u, j = r <= d ? r : d;
             if constexpr(E == Elem::I8)
                 mfma16i8(acc[i][j], fb[s][j], fa[s][i]);
+            else if constexpr(E == Elem::F32)
+                mfma16f32(acc[i][j], fb[s][j], fa[s][i]);
+            else if constexpr(E == Elem::F64)
+                mfma16f64(acc[i][j], fb[s][j], fa[s][i]);
             else
                 mfma16<E>(acc[i][j], fb[s][j], fa[s][i]);
         };
@@ -909,6 +1022,21 @@ namespace
     __global__ void __launch_bounds__(THREADS) gemmTiledKernelI8Small(Params p)
     {
         gemmTiled5<Elem::I8, OutT, A_KCONTIG, B_KCONTIG, 4>(p);
+    }
+    template <bool A_KCONTIG, bool B_KCONTIG>
+    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) gemmTiledKernelF32(Params p)
+    {
+        gemmTiled5<Elem::F32, float, A_KCONTIG, B_KCONTIG, 8>(p);
+    }
+    template <bool A_KCONTIG, bool B_KCONTIG>
+    __global__ void __launch_bounds__(THREADS) gemmTiledKernelF32Small(Params p)
+    {
+        gemmTiled5<Elem::F32, float, A_KCONTIG, B_KCONTIG, 4>(p);
+    }
+    template <bool A_KCONTIG, bool B_KCONTIG>
+    __global__ void __launch_bounds__(THREADS) gemmTiledKernelF64Small(Params p)
+    {
+        gemmTiled5<Elem::F64, double, A_KCONTIG, B_KCONTIG, 4>(p);
     }
     // The 128 x 128 tile of f16 / bf16 runs the five-buffer body as well: with a stage lasting a quarter as
     // long, the two-buffer scheme of gemmTiled16 keeps too little in flight (2048^3 f16: 710 TFLOP/s against 887
@@ -1164,6 +1292,15 @@ namespace
                 else
                     hipLaunchKernelGGL((gemmTiledKernelF8<AK, BK>), grid, block, 0, stream, p);
             }
+            else if constexpr(E == Elem::F64)
+                hipLaunchKernelGGL((gemmTiledKernelF64Small<AK, BK>), grid, block, 0, stream, p); // 128 x 128 only
+            else if constexpr(E == Elem::F32)
+            {
+                if(tile == 128u)
+                    hipLaunchKernelGGL((gemmTiledKernelF32Small<AK, BK>), grid, block, 0, stream, p);
+                else
+                    hipLaunchKernelGGL((gemmTiledKernelF32<AK, BK>), grid, block, 0, stream, p);
+            }
             else if(tile == 128u)
                 hipLaunchKernelGGL((gemmTiledKernel16Small<E, OutT, AK, BK>), grid, block, 0, stream, p);
             else
@@ -1204,9 +1341,9 @@ namespace
     uint32_t macroTile(const r355_gemm_args& g)
     {
         if(g.kernel == R355_KERNEL_TILED)
-            return 256u;
-        if(g.kernel == R355_KERNEL_TILED_128)
-            return 128u;
+            return 256u; // (f64 is then refused by the check)
+        if(g.kernel == R355_KERNEL_TILED_128 || g.in_type == R355_F64)
+            return 128u; // f64 accumulators only fit the small wave tile
         const uint64_t cus    = computeUnits();
         auto           rounds = [&](uint32_t t) { return ((uint64_t)((g.m + t - 1) / t) * ((g.n + t - 1) / t) + cus - 1) / cus; };
         return rounds(128u) * 5u < rounds(256u) * 11u ? 128u : 256u;
@@ -1220,16 +1357,20 @@ namespace r355
         const bool pairOk = (g.in_type == R355_F16 && (g.out_type == R355_F16 || g.out_type == R355_F32))
                             || (g.in_type == R355_BF16 && (g.out_type == R355_BF16 || g.out_type == R355_F32))
                             || (g.in_type == R355_E4M3 && g.out_type == R355_F32)
+                            || (g.in_type == R355_F32 && g.out_type == R355_F32)
+                            || (g.in_type == R355_F64 && g.out_type == R355_F64)
                             || (g.in_type == R355_I8 && (g.out_type == R355_I32 || g.out_type == R355_I8));
         if(!pairOk)
             return fail(R355_ERR_UNSUPPORTED, "tiled gemm: no kernel for in_type %d -> out_type %d", g.in_type, g.out_type);
         const uint32_t es = dtypeBytes(g.in_type), os = dtypeBytes(g.out_type);
         const uint32_t tile = macroTile(g);
+        if(g.in_type == R355_F64 && tile != 128u)
+            return fail(R355_ERR_UNSUPPORTED, "tiled gemm: f64 runs the 128 x 128 macro tile only");
         if(g.beta != 0.0f && g.layout_c != g.layout_d)
             return fail(R355_ERR_UNSUPPORTED, "tiled gemm: C and D must share an orientation");
         const uint32_t tk = STAGE_KB / es;
         // K moves in 16-byte chunks; a last K stage that is not full is completed with zeros by the loads
-        const bool     fiveBuffers = es == 1;
+        const bool     fiveBuffers = es != 2;
         const uint32_t kGranule    = CHUNK / es;
         if(g.m % 16 || g.n % 16 || g.m == 0 || g.n == 0 || g.k % kGranule || g.k == 0)
             return fail(R355_ERR_BAD_SIZE, "tiled gemm: m=%u n=%u must be multiples of 16 and k=%u of %u", g.m, g.n, g.k, kGranule);
@@ -1291,6 +1432,8 @@ namespace r355
             return g.out_type == R355_BF16 ? launchLayouts<Elem::BF16, __bf16>(aK, bK, tile, p, stream)
                                            : launchLayouts<Elem::BF16, float>(aK, bK, tile, p, stream);
         case R355_E4M3: return launchLayouts<Elem::E4M3, float>(aK, bK, tile, p, stream);
+        case R355_F32: return launchLayouts<Elem::F32, float>(aK, bK, tile, p, stream);
+        case R355_F64: return launchLayouts<Elem::F64, double>(aK, bK, tile, p, stream);
         case R355_I8:
             return g.out_type == R355_I32 ? launchLayouts<Elem::I8, int>(aK, bK, tile, p, stream)
                                           : launchLayouts<Elem::I8, signed char>(aK, bK, tile, p, stream);

@@ -63,10 +63,13 @@ def test_query_selects_kernel_family_and_reports_launch_shape():
     plan = R.gemm_query(_args(in_type=R.E4M3, out_type=R.F32, m=1024, n=1024, k=1024))
     assert (plan.macro_tile_m, plan.macro_tile_k, plan.grid_x, plan.lds_bytes) == (128, 128, 64, 81920)
     # small problems take the 128 x 128 tile with clamped edge loads; what the macro-tile kernels do not
-    # take (here k off a 16-byte chunk) falls back to one block per wave
+    # take (here f64 rows off 16-byte alignment) falls back to one block per wave
     plan = R.gemm_query(_args(m=64, n=48, k=80))
     assert plan.kernel == R.KERNEL_TILED and plan.macro_tile_m == 128 and plan.grid_x == 8
     plan = R.gemm_query(_args(m=64, n=48, k=80, in_type=R.F32, out_type=R.F32))
+    assert plan.kernel == R.KERNEL_TILED and plan.macro_tile_k == 32 and plan.lds_bytes == 81920
+    plan = R.gemm_query(_args(m=64, n=48, k=80, in_type=R.F64, out_type=R.F64, layout_a=R.ROW_MAJOR, layout_b=R.COL_MAJOR,
+                              lda=81, ldb=81))
     assert plan.kernel == R.KERNEL_SIMPLE and plan.lds_bytes == 0 and plan.macro_tile_m == 32
 
 

@@ -392,6 +392,67 @@ def test_int8_to_int8_output(kernel, la, lb, ldl):
             assert np.array_equal(got, want), (m, n, k, alpha, beta)
 
 
+@pytest.mark.parametrize("la,lb", TILED_LAYOUTS_16)
+@pytest.mark.parametrize("ldl", [O.ROW, O.COL])
+@pytest.mark.parametrize("kernel", list(TILE_SELECTORS))
+def test_tiled_kernel_f32_layouts_edges_and_k_tails(la, lb, ldl, kernel):
+    # f32 on v_mfma_f32_16x16x4_f32 through the five-buffer body: K-contiguous operands arrive as 128-bit LDS reads,
+    # M/N-contiguous ones element by element (there is no 32-bit transposing read); full tiles, edge tiles, K tails
+    for m, n, k in ((256, 512, 160), (272, 144, 36), (16, 400, 260)):
+        a, b, c = _inputs(O.F32, O.F32, m, n, k, seed=500 + k)
+        want = O.gemm(O.F32, O.F32, la, lb, ldl, ldl, m, n, k, a, b, c, 2.0, -1.0)
+        got = _run(O.F32, O.F32, la, lb, ldl, ldl, m, n, k, a, b, c, 2.0, -1.0, TILE_SELECTORS[kernel])
+        _check(O.F32, O.F32, got, want)
+        # integer-valued inputs: every partial sum is exact, so the result is bit-identical to the oracle's
+        a, b = O.fill_ref(O.F32, m, k, la), O.fill_ref(O.F32, k, n, lb)
+        want = O.gemm(O.F32, O.F32, la, lb, ldl, ldl, m, n, k, a, b, None, 1.0, 0.0)
+        got = _run(O.F32, O.F32, la, lb, ldl, ldl, m, n, k, a, b, None, 1.0, 0.0, TILE_SELECTORS[kernel])
+        assert np.array_equal(got, want), (m, n, k)
+
+
+@pytest.mark.parametrize("la,lb", TILED_LAYOUTS_16)
+@pytest.mark.parametrize("ldl", [O.ROW, O.COL])
+def test_tiled_kernel_f64_layouts_edges_and_k_tails(la, lb, ldl):
+    # f64 on v_mfma_f64_16x16x4_f64, 128 x 128 macro tile only (an accumulator block is 8 registers); the
+    # accumulator elements of a lane are 4 columns apart, unlike every other type
+    for m, n, k in ((256, 384, 48), (272, 144, 18), (16, 400, 130)):
+        a, b, c = _inputs(O.F64, O.F64, m, n, k, seed=600 + k)
+        if k <= 48:  # random operands: the reference's 10 eps(f64) holds for short sums in any order
+            want = O.gemm(O.F64, O.F64, la, lb, ldl, ldl, m, n, k, a, b, c, 2.0, -1.0)
+            got = _run(O.F64, O.F64, la, lb, ldl, ldl, m, n, k, a, b, c, 2.0, -1.0, R.KERNEL_AUTO)
+            _check(O.F64, O.F64, got, want)
+        a, b = O.fill_ref(O.F64, m, k, la), O.fill_ref(O.F64, k, n, lb)
+        ci = np.round(c * 8.0)
+        for alpha, beta in ((1.0, 0.0), (2.0, -1.0)):
+            cc = None if beta == 0.0 else ci
+            want = O.gemm(O.F64, O.F64, la, lb, ldl, ldl, m, n, k, a, b, cc, alpha, beta)
+            got = _run(O.F64, O.F64, la, lb, ldl, ldl, m, n, k, a, b, cc, alpha, beta, R.KERNEL_TILED_128)
+            assert np.array_equal(got, want), (m, n, k, alpha, beta)
+    g = R.gemm_args(R.F64, R.F64, 256, 256, 64, 0x1000, 0x2000, None, 0x3000, 1.0, 0.0, la, lb, ldl, ldl)
+    plan = R.gemm_query(g)
+    assert plan.kernel == R.KERNEL_TILED and plan.macro_tile_m == 128 and plan.macro_tile_k == 16
+    with pytest.raises(R.R355Error) as e:
+        _run(O.F64, O.F64, la, lb, ldl, ldl, 256, 256, 64, a[:256 * 64], b[:64 * 256], None, 1.0, 0.0, R.KERNEL_TILED)
+    assert e.value.code == -2
+
+
+@pytest.mark.parametrize("la,lb", TILED_LAYOUTS_16)
+@pytest.mark.parametrize("kernel", list(TILE_SELECTORS))
+def test_tiled_kernel_f32_one_hot_operands(la, lb, kernel):
+    m, n, k = 256, 256, 64
+    rng = np.random.default_rng(8)
+    for _ in range(6):
+        i, j, h = int(rng.integers(m)), int(rng.integers(n)), int(rng.integers(k))
+        a = np.zeros(m * k, np.float32)
+        b = np.zeros(k * n, np.float32)
+        a[i * k + h if la == O.ROW else h * m + i] = 3
+        b[h * n + j if lb == O.ROW else j * k + h] = 5
+        got = _run(O.F32, O.F32, la, lb, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0, TILE_SELECTORS[kernel]).reshape(m, n)
+        want = np.zeros((m, n), np.float32)
+        want[i, j] = 15
+        assert np.array_equal(got, want), (i, j, h)
+
+
 def test_tiled_kernel_many_tiles_xcd_mapping():
     # 5 x 3 tiles: a tile count that is not a multiple of 8 and a partial row group
     m, n, k = 1280, 768, 256
