@@ -23,7 +23,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
-PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "e4m3": 5000.0, "i8": 5000.0}
+PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "e4m3": 5000.0, "i8": 5000.0, "f32": 157.3, "f64": 78.6}
 HBM_PEAK_GBPS = 8000.0
 # Bytes one 8192^3 f16 NT launch moves across the L2 <-> fabric boundary, from two rocprofv3 --pmc
 # runs of `host_bench gemm --type f16 --layout nt`: FETCH_SIZE 7.866e5 x 2 KiB + WRITE_SIZE 1.311e5
@@ -176,6 +176,10 @@ def run_extras(R, O, np, torch, args):
     if s == 8192:  # a problem with too few 256 x 256 tiles for the 256 CUs: the 128 x 128 macro tile
         gemm_case("gemm_f16_nt_2048x2048x8192", R.F16, R.F16, R.COL_MAJOR, R.ROW_MAJOR, rnd16(2048 * s, False),
                   rnd16(s * 2048, False), PEAK_TFLOPS["f16"], "TFLOP/s", mm=2048, nn=2048, kk=s)
+    # f32 and f64 (the reference's perf_sgemm / perf_dgemm samples), TN
+    for nm, it, dt, key in (("gemm_f32_tn_%d" % s, R.F32, torch.float32, "f32"), ("gemm_f64_tn_%d" % s, R.F64, torch.float64, "f64")):
+        gemm_case(nm, it, it, R.ROW_MAJOR, R.COL_MAJOR, torch.rand(s * s, device="cuda", dtype=dt) * 2 - 1,
+                  torch.rand(s * s, device="cuda", dtype=dt) * 2 - 1, PEAK_TFLOPS[key], "TFLOP/s")
     abf, bbf = rnd16(s * s, True), rnd16(s * s, True)
     gemm_case("gemm_bf16_nt_8192", R.BF16, R.BF16, R.COL_MAJOR, R.ROW_MAJOR, abf, bbf, PEAK_TFLOPS["bf16"], "TFLOP/s")
     af16, bf16_ = rnd16(s * s, False), rnd16(s * s, False)

@@ -60,7 +60,7 @@ typedef enum
     R355_KERNEL_TILED  = 2, /* LDS-staged 256 x 256 macro tile (m, n multiples of 16; k of 8 for 16-bit, 16 for 8-bit operands)
                                (samples/perf_hgemm.cpp:515-711,
                                 test/gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp:52-283) */
-    R355_KERNEL_TILED_128 = 3 /* the same kernel with a 128 x 128 macro tile (f16 / bf16 operands): what AUTO
+    R355_KERNEL_TILED_128 = 3 /* the same kernels with a 128 x 128 macro tile (the only one for f64): what AUTO
                                picks when the 256 x 256 tiles of a problem would leave most CUs idle */
 } r355_gemm_kernel;
 

@@ -3,7 +3,7 @@
 // hipEvents: test/gemm/gemm_kernel_base_impl.hpp:647-676) and reports throughput the way the
 // reference does (2 m n k flop, test/performance.hpp:424-442), plus the fraction of MI355X's
 // published peak.  Usage:
-//   host_bench gemm  [--type f16|bf16|i8|e4m3] [--out f16|bf16|f32|i32] [--layout nt|tn|nn|tt]
+//   host_bench gemm  [--type f16|bf16|i8|e4m3|f32|f64] [--out f16|bf16|f32|i32|f64] [--layout nt|tn|nn|tt]
 //                    [--m M --n N --k K] [--kernel auto|simple|tiled|tiled128] [--warmup W --iters I]
 //                    [--sparse 1]   A is 2:4 structured sparse (compressed values + index nibbles)
 //                    [--ldpad E]    lda and ldb grow by E elements (power-of-two strides cost L2 efficiency)
@@ -48,7 +48,7 @@ namespace
     // seeded values in a sane range for each type, no NaN / inf
     void fillBytes(std::vector<uint8_t>& buf, int dtype, uint64_t seed)
     {
-        const size_t es = (dtype == R355_F16 || dtype == R355_BF16) ? 2 : (dtype == R355_F32 ? 4 : 1);
+        const size_t es = (dtype == R355_F16 || dtype == R355_BF16) ? 2 : (dtype == R355_F32 ? 4 : (dtype == R355_F64 ? 8 : 1));
         const size_t n  = buf.size() / es;
         for(size_t i = 0; i < n; ++i)
         {
@@ -74,6 +74,7 @@ namespace
                 buf[i] = static_cast<uint8_t>(((r & 1) << 7) | ((3 + ((r >> 1) & 3)) << 3) | ((r >> 8) & 7));
                 break;
             case R355_I8: buf[i] = static_cast<uint8_t>(r >> 32); break;
+            case R355_F64: reinterpret_cast<double*>(buf.data())[i] = static_cast<double>(r >> 11) * (2.0 / 9007199254740992.0) - 1.0; break;
             default: reinterpret_cast<float*>(buf.data())[i] = static_cast<float>((r >> 40) & 0xFFFF) / 65536.0f - 0.5f;
             }
         }
@@ -86,13 +87,14 @@ namespace
         if(s == "e4m3" || s == "fp8") return R355_E4M3;
         if(s == "i8") return R355_I8;
         if(s == "f32") return R355_F32;
+        if(s == "f64") return R355_F64;
         if(s == "i32") return R355_I32;
         return -1;
     }
 
     size_t bytesOf(int t)
     {
-        return (t == R355_F16 || t == R355_BF16) ? 2 : ((t == R355_F32 || t == R355_I32) ? 4 : 1);
+        return (t == R355_F16 || t == R355_BF16) ? 2 : ((t == R355_F32 || t == R355_I32) ? 4 : (t == R355_F64 ? 8 : 1));
     }
 
     using f32x16 = float __attribute__((ext_vector_type(16)));
@@ -314,8 +316,12 @@ int main(int argc, char** argv)
         }
         const double flop   = 2.0 * m * n * k;
         const double tflops = flop / ms / 1e9;
-        const double vendor = ((inT == R355_I8 || inT == R355_E4M3) ? 5000.0 : 2500.0) * (sparse ? 2.0 : 1.0);
-        const double perClk = (inT == R355_I8 || inT == R355_E4M3) ? 8192.0 : 4096.0; // flop / CU / clk
+        const double vendor = (inT == R355_F64   ? 78.6
+                               : inT == R355_F32 ? 157.3
+                               : (inT == R355_I8 || inT == R355_E4M3) ? 5000.0
+                                                                      : 2500.0)
+                              * (sparse ? 2.0 : 1.0);
+        const double perClk = inT == R355_F64 ? 128.0 : inT == R355_F32 ? 256.0 : (inT == R355_I8 || inT == R355_E4M3) ? 8192.0 : 4096.0; // flop / CU / clk
         const double model  = perClk * dev.compute_units * dev.clock_mhz * 1e-6; // TFLOP/s at the reported clock
         printf("{\"op\": \"%s\", \"type\": \"%s\", \"out\": \"%s\", \"layout\": \"%s\", \"m\": %u, \"n\": %u, \"k\": %u, "
                "\"kernel\": %d, \"macro_tile\": [%u, %u, %u], \"lds_bytes\": %u, \"ms\": %.4f, \"tflops\": %.1f, "
