@@ -146,6 +146,9 @@ int r355_gemv(int32_t layout_a, uint32_t m, uint32_t k, const float* a, uint32_t
 int r355_gemv_timed(int32_t layout_a, uint32_t m, uint32_t k, const float* a, uint32_t lda, const float* x,
                     const float* y_in, float* y_out, float alpha, float beta, void* stream, int warmup,
                     int iters, float* avg_ms);
+/* The f64 twin (samples/simple_dgemv.cpp:103): m, k multiples of 2, lda % 2 == 0, 16-byte aligned pointers. */
+int r355_dgemv(int32_t layout_a, uint32_t m, uint32_t k, const double* a, uint32_t lda, const double* x,
+               const double* y_in, double* y_out, double alpha, double beta, void* stream);
 
 /*
  * Host-side 2:4 compressor for a row-major m x k matrix of 1-byte elements (host pointers).

@@ -25,7 +25,7 @@ DTYPE_BYTES = {F16: 2, BF16: 2, E4M3: 1, I8: 1, F32: 4, I32: 4, F64: 8}
 
 EXPORTS = [
     "r355_gemm", "r355_gemm_query", "r355_gemm_timed", "r355_dlrm_fwd", "r355_dlrm_fwd_timed",
-    "r355_dlrm_bwd", "r355_gemv", "r355_gemv_timed", "r355_compress_24", "r355_decompress_24",
+    "r355_dlrm_bwd", "r355_gemv", "r355_gemv_timed", "r355_dgemv", "r355_compress_24", "r355_decompress_24",
     "r355_get_device_info", "r355_last_error", "r355_version",
 ]
 
@@ -90,6 +90,7 @@ def lib():
         L.r355_dlrm_bwd.argtypes = [i32, vp, vp, vp, vp, u32, u32, u32, vp]
         L.r355_gemv.argtypes = [i32, u32, u32, vp, u32, vp, vp, vp, f32, f32, vp]
         L.r355_gemv_timed.argtypes = [i32, u32, u32, vp, u32, vp, vp, vp, f32, f32, vp, ctypes.c_int, ctypes.c_int, fp]
+        L.r355_dgemv.argtypes = [i32, u32, u32, vp, u32, vp, vp, vp, ctypes.c_double, ctypes.c_double, vp]
         L.r355_compress_24.argtypes = [vp, u32, u32, vp, vp]
         L.r355_decompress_24.argtypes = [vp, vp, u32, u32, vp]
         L.r355_get_device_info.argtypes = [ctypes.POINTER(DeviceInfo)]
@@ -188,6 +189,13 @@ def gemv(layout_a, m, k, a, x, y_in, y_out, alpha=1.0, beta=0.0, lda=None, strea
     lda = lda if lda is not None else default_ld(m, k, layout_a)
     _check(lib().r355_gemv(layout_a, m, k, _ptr(a), lda, _ptr(x), _ptr(y_in), _ptr(y_out), alpha, beta,
                            _stream_handle(stream)))
+
+
+def dgemv(layout_a, m, k, a, x, y_in, y_out, alpha=1.0, beta=0.0, lda=None, stream=None):
+    """f64 GEMV (the reference's simple_dgemv sample)."""
+    lda = lda if lda is not None else default_ld(m, k, layout_a)
+    _check(lib().r355_dgemv(layout_a, m, k, _ptr(a), lda, _ptr(x), _ptr(y_in), _ptr(y_out), alpha, beta,
+                            _stream_handle(stream)))
 
 
 def gemv_timed(layout_a, m, k, a, x, y_in, y_out, alpha, beta, warmup, iters, lda=None, stream=None):

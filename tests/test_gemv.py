@@ -27,3 +27,25 @@ def test_gemv_vs_oracle(layout, m, k):
     exact = 2.0 * (A @ x.astype(np.float64)) + 2.0 * y.astype(np.float64)
     g = got.astype(np.float64)
     assert np.max(np.abs(g - exact) / (np.abs(g) + np.abs(exact) + 1.0)) <= 1e-7 * k
+
+
+@pytest.mark.parametrize("layout", [O.ROW, O.COL])
+@pytest.mark.parametrize("m,k", [(256, 256), (4098, 262), (32768 + 128, 64)])
+def test_dgemv_vs_oracle(layout, m, k):
+    """The f64 twin (samples/simple_dgemv.cpp): against the oracle's f64 GEMM with n = 1 and the exact integer case."""
+    a = O.uniform_pm1(4, m * k).astype(np.float64) + O.uniform_pm1(5, m * k).astype(np.float64) * 2.0 ** -30
+    x = O.uniform_pm1(6, k).astype(np.float64)
+    y = O.uniform_pm1(7, m).astype(np.float64)
+    want = O.gemm(O.F64, O.F64, layout, O.COL, O.COL, O.COL, m, 1, k, a, x, y, 2.0, 2.0)
+    da, dx, dy = to_device(a), to_device(x), to_device(y)
+    dout = device_filled(m, np.float64, 0xFF)
+    R.dgemv(layout, m, k, da, dx, dy, dout, 2.0, 2.0)
+    got = to_host(dout, np.float64)
+    A = O.as_matrix(a, m, k, layout)
+    bound = (np.abs(A) @ np.abs(x)) * 2.0 * k * 1.2e-16 + 1e-15
+    assert np.all(np.abs(got - want) <= bound)
+    # integer-valued operands: exact in any summation order
+    ai, xi = np.round(a * 8.0), np.round(x * 8.0)
+    want = O.gemm(O.F64, O.F64, layout, O.COL, O.COL, O.COL, m, 1, k, ai, xi, None, 1.0, 0.0)
+    R.dgemv(layout, m, k, to_device(ai), to_device(xi), None, dout, 1.0, 0.0)
+    assert np.array_equal(to_host(dout, np.float64), want)
