@@ -1344,6 +1344,9 @@ namespace
             return 256u; // (f64 is then refused by the check)
         if(g.kernel == R355_KERNEL_TILED_128 || g.in_type == R355_F64)
             return 128u; // f64 accumulators only fit the small wave tile
+        if(g.in_type == R355_F32)
+            return 128u; // bound by the matrix-instruction rate either way (146 TFLOP/s at 4096^2 x 2048 with both
+                         // tiles), and four times finer rounds: 6144^2 x 2048 runs at 148 TFLOP/s against 111
         const uint64_t cus    = computeUnits();
         auto           rounds = [&](uint32_t t) { return ((uint64_t)((g.m + t - 1) / t) * ((g.n + t - 1) / t) + cus - 1) / cus; };
         return rounds(128u) * 5u < rounds(256u) * 11u ? 128u : 256u;
