@@ -41,7 +41,8 @@ typedef enum
     R355_I8   = 3, /* signed 8-bit integer               */
     R355_F32  = 4,
     R355_I32  = 5,
-    R355_F64  = 6 /* GEMM f64 -> f64 on the block-per-wave kernel only */
+    R355_F64  = 6,
+    R355_E5M2 = 7 /* OCP FP8 E5M2 ("bf8", the reference's bfloat8_t): GEMM operands, f32 result */
 } r355_dtype;
 
 /* memory orientation; BLAS letters: row-major = "T", col-major = "N" for A (m x k) */
@@ -69,7 +70,7 @@ typedef enum
  * Argument order and meaning follow the reference kernel signature
  * (test/gemm/gemm_kernel_base.hpp:101-114): leading dimensions in elements.
  * Supported (in -> out, accumulate): f16 -> f32|f16 (f32), bf16 -> f32|bf16 (f32),
- * e4m3 -> f32 (f32), i8 -> i32|i8 (i32, alpha/beta truncated to int32; an i8 result is the low 8 bits, as the
+ * e4m3 -> f32 (f32), e5m2 -> f32 (f32), i8 -> i32|i8 (i32, alpha/beta truncated to int32; an i8 result is the low 8 bits, as the
  * reference's static_cast narrows it), f32 -> f32 (f32), f64 -> f64 (f64).
  * beta == 0 means C is never read and may be NULL.
  *

@@ -46,7 +46,7 @@
 #include <omp.h>
 #endif
 
-enum { ORC_F16 = 0, ORC_BF16 = 1, ORC_E4M3 = 2, ORC_I8 = 3, ORC_F32 = 4, ORC_I32 = 5, ORC_F64 = 6 };
+enum { ORC_F16 = 0, ORC_BF16 = 1, ORC_E4M3 = 2, ORC_I8 = 3, ORC_F32 = 4, ORC_I32 = 5, ORC_F64 = 6, ORC_E5M2 = 7 };
 enum { ORC_ROW_MAJOR = 0, ORC_COL_MAJOR = 1 };
 
 /* ---------------------------------------------------------------- scalars */
@@ -199,6 +199,8 @@ static inline float load_as_f32(const void* p, size_t idx, int dtype)
         return orc_bf16_to_f32(((const uint16_t*)p)[idx]);
     case ORC_E4M3:
         return orc_e4m3_to_f32(((const uint8_t*)p)[idx]);
+    case ORC_E5M2: /* OCP e5m2 is binary16 cut after two mantissa bits: the code is the f16's high byte */
+        return orc_f16_to_f32((uint16_t)(((const uint8_t*)p)[idx] << 8));
     case ORC_I8:
         return (float)((const int8_t*)p)[idx];
     case ORC_F32:
@@ -348,7 +350,7 @@ int orc_gemm(int         in_type,
         return 0;
     }
 
-    if(in_type != ORC_F16 && in_type != ORC_BF16 && in_type != ORC_E4M3 && in_type != ORC_F32)
+    if(in_type != ORC_F16 && in_type != ORC_BF16 && in_type != ORC_E4M3 && in_type != ORC_E5M2 && in_type != ORC_F32)
         return -1;
     if(out_type != ORC_F16 && out_type != ORC_BF16 && out_type != ORC_F32)
         return -1;

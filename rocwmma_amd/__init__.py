@@ -15,13 +15,13 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "librocwmma_amd.so")
 
 # r355_dtype
-F16, BF16, E4M3, I8, F32, I32, F64 = range(7)
+F16, BF16, E4M3, I8, F32, I32, F64, E5M2 = range(8)
 # r355_layout
 ROW_MAJOR, COL_MAJOR = 0, 1
 # r355_gemm_kernel
 KERNEL_AUTO, KERNEL_SIMPLE, KERNEL_TILED, KERNEL_TILED_128 = 0, 1, 2, 3
 
-DTYPE_BYTES = {F16: 2, BF16: 2, E4M3: 1, I8: 1, F32: 4, I32: 4, F64: 8}
+DTYPE_BYTES = {F16: 2, BF16: 2, E4M3: 1, I8: 1, F32: 4, I32: 4, F64: 8, E5M2: 1}
 
 EXPORTS = [
     "r355_gemm", "r355_gemm_query", "r355_gemm_timed", "r355_dlrm_fwd", "r355_dlrm_fwd_timed",

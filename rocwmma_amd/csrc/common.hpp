@@ -22,6 +22,7 @@ namespace r355
         case R355_F16:
         case R355_BF16: return 2;
         case R355_E4M3:
+        case R355_E5M2:
         case R355_I8: return 1;
         case R355_F32:
         case R355_I32: return 4;

@@ -161,7 +161,8 @@ namespace
         case R355_F16:
         case R355_BF16: return 16;
         case R355_I8: return 32;
-        case R355_E4M3: return blk == 32 ? 16 : 32;
+        case R355_E4M3:
+        case R355_E5M2: return blk == 32 ? 16 : 32;
         case R355_F32: return blk == 32 ? 2 : 4;
         case R355_F64: return 4;
         default: return 0;
@@ -189,7 +190,8 @@ namespace
         {
         case R355_F16: return out == R355_F32 || out == R355_F16;
         case R355_BF16: return out == R355_F32 || out == R355_BF16;
-        case R355_E4M3: return out == R355_F32;
+        case R355_E4M3:
+        case R355_E5M2: return out == R355_F32;
         case R355_I8: return out == R355_I32 || out == R355_I8;
         case R355_F32: return out == R355_F32;
         case R355_F64: return out == R355_F64;
@@ -248,6 +250,7 @@ namespace r355
             return g.out_type == R355_F32 ? launchBlocks<bfloat16_t, float32_t, float32_t>(g, stream, blk)
                                           : launchBlocks<bfloat16_t, bfloat16_t, float32_t>(g, stream, blk);
         case R355_E4M3: return launchBlocks<float8_t, float32_t, float32_t>(g, stream, blk);
+        case R355_E5M2: return launchBlocks<bfloat8_t, float32_t, float32_t>(g, stream, blk);
         case R355_I8:
             return g.out_type == R355_I32 ? launchBlocks<int8_t, int32_t, int32_t>(g, stream, blk)
                                           : launchBlocks<int8_t, int8_t, int32_t>(g, stream, blk);

@@ -62,7 +62,8 @@ namespace
         E4M3,
         I8,
         F32,
-        F64
+        F64,
+        E5M2
     };
 
     constexpr uint32_t TILE_M      = 256;
@@ -106,6 +107,11 @@ namespace
     struct ElemTraits<Elem::F64>
     {
         static constexpr uint32_t Bytes = 8;
+    };
+    template <>
+    struct ElemTraits<Elem::E5M2>
+    {
+        static constexpr uint32_t Bytes = 1;
     };
 
     struct Params
@@ -821,7 +827,7 @@ namespace
     {
         static_assert(WB == 8 || WB == 4, "wave tile of 8 x 8 or 4 x 4 blocks");
         static_assert(E != Elem::F64 || WB == 4, "f64 accumulators of an 8 x 8 wave tile would need 512 registers");
-        static_assert(E != Elem::E4M3, "e4m3 has its own stage structure");
+        static_assert(E != Elem::E4M3 && E != Elem::E5M2, "fp8 has its own stage structure");
         constexpr uint32_t ES = ElemTraits<E>::Bytes;
         using AccV            = std::conditional_t<E == Elem::I8, i32x4v, std::conditional_t<E == Elem::F64, f64x4, f32x4>>;
         constexpr uint32_t TILE = 32u * WB, WT = 16u * WB; // macro tile and wave tile edge
@@ -1060,13 +1066,17 @@ namespace
     // After Q2 the stage's buffers are no longer read: barrier, then the refills are issued under Q3
     // (A) and Q4 (B).  Four register groups suffice; the two B groups swap roles every stage.
     using i32x8 = int __attribute__((ext_vector_type(8)));
+    template <bool E5M2>
     __device__ __forceinline__ void mfma16f8(f32x4& acc, const i32x8& x, const i32x8& y)
     {
-        // cbsz = blgp = 0: both operands e4m3; the unscaled form multiplies by 2^0
-        asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc) : "v"(x), "v"(y));
+        // cbsz / blgp give the formats of the two operands: 0 = e4m3, 1 = e5m2; the unscaled form multiplies by 2^0
+        if constexpr(E5M2)
+            asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:1 blgp:1" : "+a"(acc) : "v"(x), "v"(y));
+        else
+            asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(acc) : "v"(x), "v"(y));
     }
 
-    template <bool A_KCONTIG, bool B_KCONTIG, uint32_t WB>
+    template <bool E5M2, bool A_KCONTIG, bool B_KCONTIG, uint32_t WB>
     __device__ __forceinline__ void gemmTiledF8(const Params& p)
     {
         static_assert(WB == 8 || WB == 4, "wave tile of 8 x 8 or 4 x 4 blocks");
@@ -1168,7 +1178,7 @@ namespace
 #pragma unroll
             for(uint32_t n = 0; n < NQ; ++n)
             {
-                mfma16f8(acc[n % H][n / H], bLo[n / H], aLo[n % H]);
+                mfma16f8<E5M2>(acc[n % H][n / H], bLo[n / H], aLo[n % H]);
                 readSlotB(bHi, bCur, 1, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -1176,7 +1186,7 @@ namespace
 #pragma unroll
             for(uint32_t n = 0; n < NQ; ++n)
             {
-                mfma16f8(acc[n % H][H + n / H], bHi[n / H], aLo[n % H]);
+                mfma16f8<E5M2>(acc[n % H][H + n / H], bHi[n / H], aLo[n % H]);
                 readSlotA(aHi, aCur, 1, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -1192,7 +1202,7 @@ namespace
 #pragma unroll
             for(uint32_t n = 0; n < NQ; ++n)
             {
-                mfma16f8(acc[H + n / H][H + n % H], bHi[n % H], aHi[n / H]);
+                mfma16f8<E5M2>(acc[H + n / H][H + n % H], bHi[n % H], aHi[n / H]);
                 readSlotA(aLo, aNxt, 0, n);
                 loadSlot(A_KCONTIG, rsrcA, gOffA, gStepA, kByteA, vA, aCur, n);
                 __builtin_amdgcn_sched_barrier(0);
@@ -1201,7 +1211,7 @@ namespace
 #pragma unroll
             for(uint32_t n = 0; n < NQ; ++n)
             {
-                mfma16f8(acc[H + n % H][n / H], bLo[n / H], aHi[n % H]);
+                mfma16f8<E5M2>(acc[H + n % H][n / H], bLo[n / H], aHi[n % H]);
                 readSlotB(bHi, bNxt, 0, n);
                 loadSlot(B_KCONTIG, rsrcB, gOffB, gStepB, kByteB, vB, bCur, n);
                 __builtin_amdgcn_sched_barrier(0);
@@ -1261,15 +1271,15 @@ namespace
         storeTile16<f32x4, float, WB>(acc, p, tm * TILE + wm * WT, tn * TILE + wn * WT, lane, lds + wave * (WB * 4096u));
     }
 
-    template <bool A_KCONTIG, bool B_KCONTIG>
+    template <bool E5M2, bool A_KCONTIG, bool B_KCONTIG>
     __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) gemmTiledKernelF8(Params p)
     {
-        gemmTiledF8<A_KCONTIG, B_KCONTIG, 8>(p);
+        gemmTiledF8<E5M2, A_KCONTIG, B_KCONTIG, 8>(p);
     }
-    template <bool A_KCONTIG, bool B_KCONTIG>
+    template <bool E5M2, bool A_KCONTIG, bool B_KCONTIG>
     __global__ void __launch_bounds__(THREADS) gemmTiledKernelF8Small(Params p)
     {
-        gemmTiledF8<A_KCONTIG, B_KCONTIG, 4>(p);
+        gemmTiledF8<E5M2, A_KCONTIG, B_KCONTIG, 4>(p);
     }
 
     template <Elem E, typename OutT>
@@ -1285,12 +1295,12 @@ namespace
                 else
                     hipLaunchKernelGGL((gemmTiledKernelI8<OutT, AK, BK>), grid, block, 0, stream, p);
             }
-            else if constexpr(E == Elem::E4M3)
+            else if constexpr(E == Elem::E4M3 || E == Elem::E5M2)
             {
                 if(tile == 128u)
-                    hipLaunchKernelGGL((gemmTiledKernelF8Small<AK, BK>), grid, block, 0, stream, p);
+                    hipLaunchKernelGGL((gemmTiledKernelF8Small<E == Elem::E5M2, AK, BK>), grid, block, 0, stream, p);
                 else
-                    hipLaunchKernelGGL((gemmTiledKernelF8<AK, BK>), grid, block, 0, stream, p);
+                    hipLaunchKernelGGL((gemmTiledKernelF8<E == Elem::E5M2, AK, BK>), grid, block, 0, stream, p);
             }
             else if constexpr(E == Elem::F64)
                 hipLaunchKernelGGL((gemmTiledKernelF64Small<AK, BK>), grid, block, 0, stream, p); // 128 x 128 only
@@ -1359,7 +1369,7 @@ namespace r355
     {
         const bool pairOk = (g.in_type == R355_F16 && (g.out_type == R355_F16 || g.out_type == R355_F32))
                             || (g.in_type == R355_BF16 && (g.out_type == R355_BF16 || g.out_type == R355_F32))
-                            || (g.in_type == R355_E4M3 && g.out_type == R355_F32)
+                            || ((g.in_type == R355_E4M3 || g.in_type == R355_E5M2) && g.out_type == R355_F32)
                             || (g.in_type == R355_F32 && g.out_type == R355_F32)
                             || (g.in_type == R355_F64 && g.out_type == R355_F64)
                             || (g.in_type == R355_I8 && (g.out_type == R355_I32 || g.out_type == R355_I8));
@@ -1435,6 +1445,7 @@ namespace r355
             return g.out_type == R355_BF16 ? launchLayouts<Elem::BF16, __bf16>(aK, bK, tile, p, stream)
                                            : launchLayouts<Elem::BF16, float>(aK, bK, tile, p, stream);
         case R355_E4M3: return launchLayouts<Elem::E4M3, float>(aK, bK, tile, p, stream);
+        case R355_E5M2: return launchLayouts<Elem::E5M2, float>(aK, bK, tile, p, stream);
         case R355_F32: return launchLayouts<Elem::F32, float>(aK, bK, tile, p, stream);
         case R355_F64: return launchLayouts<Elem::F64, double>(aK, bK, tile, p, stream);
         case R355_I8:

@@ -12,11 +12,11 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _ORACLE_DIR = os.path.join(os.path.dirname(_HERE), "oracle")
 
-F16, BF16, E4M3, I8, F32, I32, F64 = range(7)
+F16, BF16, E4M3, I8, F32, I32, F64, E5M2 = range(8)
 ROW, COL = 0, 1  # row_major ("T" in BLAS letters), col_major ("N")
 
 NP_STORAGE = {F16: np.uint16, BF16: np.uint16, E4M3: np.uint8, I8: np.int8, F32: np.float32, I32: np.int32,
-              F64: np.float64}
+              F64: np.float64, E5M2: np.uint8}
 
 _lib = None
 
@@ -170,6 +170,8 @@ def storage_to_f32(s, dtype):
         return (s.astype(np.uint32) << 16).view(np.float32)
     if dtype == E4M3:
         return E4M3_TABLE[s.view(np.uint8)]
+    if dtype == E5M2:  # the high byte of the binary16 with the same value
+        return (s.view(np.uint8).astype(np.uint16) << 8).view(np.float16).astype(np.float32)
     return s.astype(np.float32)
 
 

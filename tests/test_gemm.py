@@ -453,6 +453,35 @@ def test_tiled_kernel_f32_one_hot_operands(la, lb, kernel):
         assert np.array_equal(got, want), (i, j, h)
 
 
+def _e5m2_operand(seed, n):
+    """n finite e5m2 codes of magnitude 2^-4 .. 2 (random sign, exponent 11 .. 15, mantissa)."""
+    rng = np.random.default_rng(seed)
+    return ((rng.integers(0, 2, n) << 7) | (rng.integers(11, 16, n) << 2) | rng.integers(0, 4, n)).astype(np.uint8)
+
+
+@pytest.mark.parametrize("kernel", ["simple", "tiled", "tiled_128"])
+@pytest.mark.parametrize("la,lb,ldl", [(O.ROW, O.COL, O.ROW), (O.COL, O.ROW, O.COL), (O.ROW, O.ROW, O.ROW), (O.COL, O.COL, O.ROW)])
+def test_e5m2_gemm(kernel, la, lb, ldl):
+    # OCP e5m2 operands (the reference's bfloat8_t tuple, test/gemm/gemm_common_test_params.hpp:73-87), f32 result:
+    # v_mfma_f32_16x16x128_f8f6f4 with both format fields set to e5m2 in the macro-tile kernels,
+    # v_mfma_f32_*_bf8_bf8 behind the fragment API in the block-per-wave one
+    sel = {"simple": R.KERNEL_SIMPLE, **TILE_SELECTORS}[kernel]
+    for m, n, k in ((256, 384, 512), (272, 144, 160)):
+        a, b = _e5m2_operand(31, m * k), _e5m2_operand(32, k * n)
+        c = O.uniform_pm1(33, m * n)
+        want = O.gemm(O.E5M2, O.F32, la, lb, ldl, ldl, m, n, k, a, b, c, 1.0, 1.0)
+        got = _run(O.E5M2, O.F32, la, lb, ldl, ldl, m, n, k, a, b, c, 1.0, 1.0, sel)
+        assert _max_rel(O.F32, got, want) <= 1e-2, (m, n, k)
+    # powers of two only: every product and every partial sum is exact, the result must match bit for bit
+    m, n, k = 256, 256, 256
+    rng = np.random.default_rng(34)
+    a = ((rng.integers(0, 2, m * k) << 7) | (rng.integers(13, 17, m * k) << 2)).astype(np.uint8)
+    b = ((rng.integers(0, 2, k * n) << 7) | (rng.integers(13, 17, k * n) << 2)).astype(np.uint8)
+    want = O.gemm(O.E5M2, O.F32, la, lb, ldl, ldl, m, n, k, a, b, None, 1.0, 0.0)
+    got = _run(O.E5M2, O.F32, la, lb, ldl, ldl, m, n, k, a, b, None, 1.0, 0.0, sel)
+    assert np.array_equal(got, want)
+
+
 def test_tiled_kernel_many_tiles_xcd_mapping():
     # 5 x 3 tiles: a tile count that is not a multiple of 8 and a partial row group
     m, n, k = 1280, 768, 256

@@ -337,6 +337,30 @@ def test_e4m3_matches_torch_float8_e4m3fn():
     assert np.array_equal(O.storage_to_f32(got, O.E4M3), t.to(torch.float32).numpy())
 
 
+def test_e5m2_decode_closed_form_and_torch():
+    """OCP e5m2 (the reference's bfloat8_t): sign, 5 exponent bits (bias 15), 2 mantissa bits -- binary16 cut after
+    two mantissa bits.  Every finite code against the closed form, against torch's float8_e5m2 where present, and
+    through the oracle's GEMM (a 1 x 1 x 1 product with 1.0)."""
+    codes = np.arange(256, dtype=np.uint8)
+    dec = O.storage_to_f32(codes, O.E5M2)
+    for v in range(256):
+        s, e, m = v >> 7, (v >> 2) & 0x1F, v & 3
+        if e == 31:
+            assert not np.isfinite(dec[v])
+            continue
+        mag = (m / 4.0) * 2.0 ** -14 if e == 0 else (1.0 + m / 4.0) * 2.0 ** (e - 15)
+        assert dec[v] == np.float32(-mag if s else mag), v
+    finite = codes[((codes >> 2) & 0x1F) != 31]
+    one = np.array([0x3C], dtype=np.uint8)  # 1.0
+    for v in finite[::7]:
+        d = O.gemm(O.E5M2, O.F32, O.ROW, O.COL, O.ROW, O.ROW, 1, 1, 1, np.array([v], np.uint8), one, None, 1.0, 0.0)
+        assert d[0] == dec[v]
+    torch = pytest.importorskip("torch")
+    if hasattr(torch, "float8_e5m2"):
+        t = torch.from_numpy(finite.copy()).view(torch.float8_e5m2).to(torch.float32).numpy()
+        assert np.array_equal(t, dec[finite])
+
+
 def test_gemm_f64_against_numpy():
     """f64 path (the reference's dgemm instantiation): exact on the reference's integer pattern in every
     layout combination; on random data equal to numpy's sequential float64 accumulation bit for bit."""
