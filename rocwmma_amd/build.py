@@ -16,7 +16,12 @@ OBJDIR = os.path.join(HERE, "build")
 LIB = os.path.join(LIBDIR, "librocwmma_amd.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-SOURCES = ["api.cpp", "gemm_simple.hip", "gemm_tiled.hip", "dlrm.hip", "sparse.hip", "gemv.hip"]
+# (source, object stem, extra flags); gemm_tiled.hip is compiled once per kernel family so that the four
+# parts build in parallel
+SOURCES = [("api.cpp", "api", []), ("gemm_simple.hip", "gemm_simple", []),
+           ("gemm_tiled.hip", "gemm_tiled_p0", ["-DR355_TILED_PART=0"]), ("gemm_tiled.hip", "gemm_tiled_p1", ["-DR355_TILED_PART=1"]),
+           ("gemm_tiled.hip", "gemm_tiled_p2", ["-DR355_TILED_PART=2"]), ("gemm_tiled.hip", "gemm_tiled_p3", ["-DR355_TILED_PART=3"]),
+           ("dlrm.hip", "dlrm", []), ("sparse.hip", "sparse", []), ("gemv.hip", "gemv", [])]
 
 # packed-fp32 instructions are disabled on purpose (device pass only; the host pass warns that it
 # does not know the feature, which is harmless)
@@ -35,13 +40,14 @@ def _headers():
     return hs
 
 
-def _compile(src, force):
-    obj = os.path.join(OBJDIR, os.path.splitext(src)[0] + ".o")
+def _compile(item, force):
+    src, stem, extra = item
+    obj = os.path.join(OBJDIR, stem + ".o")
     path = os.path.join(CSRC, src)
     newest = max(os.path.getmtime(p) for p in [path] + _headers())
     if not force and os.path.exists(obj) and os.path.getmtime(obj) >= newest:
         return obj, False
-    r = subprocess.run([HIPCC] + FLAGS + ["-c", path, "-o", obj], capture_output=True, text=True)
+    r = subprocess.run([HIPCC] + FLAGS + extra + ["-c", path, "-o", obj], capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s" % (src, r.stderr))
     return obj, True
@@ -50,7 +56,7 @@ def _compile(src, force):
 def build(force=False, verbose=True):
     os.makedirs(LIBDIR, exist_ok=True)
     os.makedirs(OBJDIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=min(6, os.cpu_count() or 1)) as ex:
+    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as ex:
         results = list(ex.map(lambda s: _compile(s, force), SOURCES))
     objs = [o for o, _ in results]
     if force or any(c for _, c in results) or not os.path.exists(LIB):

@@ -47,6 +47,34 @@
 #include "lds_dma.hpp"
 #include "tile_map.hpp"
 
+// This file is compiled once per part so that its kernel families build in parallel: part 0 holds the host
+// side and the f16 kernels, part 1 bf16, part 2 the 8-bit types, part 3 f32 and f64.  Without the macro one
+// translation unit holds everything.
+#ifndef R355_TILED_PART
+#define R355_TILED_PART (-1)
+#endif
+#define R355_TILED_HAS(part) (R355_TILED_PART < 0 || R355_TILED_PART == (part))
+
+namespace r355
+{
+    struct GemmTileParams
+    {
+        uint32_t    m, n, k;
+        const char* a;
+        const char* b;
+        const char* c;
+        char*       d;
+        uint32_t    lda, ldb, ldc, ldd; // elements
+        float       alpha, beta;
+        uint32_t    tilesM, tilesN;
+    };
+    // launch of one kernel family; aK / bK: operand is K-contiguous; tile: 256 or 128
+    int gemmTiledPart0(const r355_gemm_args& g, bool aK, bool bK, uint32_t tile, const GemmTileParams& p, hipStream_t s);
+    int gemmTiledPart1(const r355_gemm_args& g, bool aK, bool bK, uint32_t tile, const GemmTileParams& p, hipStream_t s);
+    int gemmTiledPart2(const r355_gemm_args& g, bool aK, bool bK, uint32_t tile, const GemmTileParams& p, hipStream_t s);
+    int gemmTiledPart3(const r355_gemm_args& g, bool aK, bool bK, uint32_t tile, const GemmTileParams& p, hipStream_t s);
+} // namespace r355
+
 namespace
 {
     using i32x4  = int __attribute__((ext_vector_type(4)));
@@ -114,17 +142,7 @@ namespace
         static constexpr uint32_t Bytes = 1;
     };
 
-    struct Params
-    {
-        uint32_t    m, n, k;
-        const char* a;
-        const char* b;
-        const char* c;
-        char*       d;
-        uint32_t    lda, ldb, ldc, ldd; // elements
-        float       alpha, beta;
-        uint32_t    tilesM, tilesN;
-    };
+    using Params = r355::GemmTileParams;
 
     // ------------------------------------------------------------------------------------------
     // f16 / bf16 on v_mfma_f32_16x16x32_{f16,bf16}.
@@ -1329,6 +1347,7 @@ namespace
         return r355::checkLaunch("gemm (macro tile)");
     }
 
+#if R355_TILED_HAS(0)
     // CUs of the current device; where the query fails (no device: plan queries on a build host) MI355X's 256
     uint32_t computeUnits()
     {
@@ -1361,10 +1380,12 @@ namespace
         auto           rounds = [&](uint32_t t) { return ((uint64_t)((g.m + t - 1) / t) * ((g.n + t - 1) / t) + cus - 1) / cus; };
         return rounds(128u) * 5u < rounds(256u) * 11u ? 128u : 256u;
     }
+#endif // part 0
 } // namespace
 
 namespace r355
 {
+#if R355_TILED_HAS(0)
     int gemmTiledCheck(const r355_gemm_args& g, r355_gemm_plan* plan)
     {
         const bool pairOk = (g.in_type == R355_F16 && (g.out_type == R355_F16 || g.out_type == R355_F32))
@@ -1438,20 +1459,48 @@ namespace r355
         p.tilesM = (p.m + tile - 1) / tile, p.tilesN = (p.n + tile - 1) / tile;
         switch(g.in_type)
         {
-        case R355_F16:
-            return g.out_type == R355_F16 ? launchLayouts<Elem::F16, _Float16>(aK, bK, tile, p, stream)
-                                          : launchLayouts<Elem::F16, float>(aK, bK, tile, p, stream);
-        case R355_BF16:
-            return g.out_type == R355_BF16 ? launchLayouts<Elem::BF16, __bf16>(aK, bK, tile, p, stream)
-                                           : launchLayouts<Elem::BF16, float>(aK, bK, tile, p, stream);
-        case R355_E4M3: return launchLayouts<Elem::E4M3, float>(aK, bK, tile, p, stream);
-        case R355_E5M2: return launchLayouts<Elem::E5M2, float>(aK, bK, tile, p, stream);
-        case R355_F32: return launchLayouts<Elem::F32, float>(aK, bK, tile, p, stream);
-        case R355_F64: return launchLayouts<Elem::F64, double>(aK, bK, tile, p, stream);
-        case R355_I8:
-            return g.out_type == R355_I32 ? launchLayouts<Elem::I8, int>(aK, bK, tile, p, stream)
-                                          : launchLayouts<Elem::I8, signed char>(aK, bK, tile, p, stream);
+        case R355_F16: return gemmTiledPart0(g, aK, bK, tile, p, stream);
+        case R355_BF16: return gemmTiledPart1(g, aK, bK, tile, p, stream);
+        case R355_E4M3:
+        case R355_E5M2:
+        case R355_I8: return gemmTiledPart2(g, aK, bK, tile, p, stream);
+        case R355_F32:
+        case R355_F64: return gemmTiledPart3(g, aK, bK, tile, p, stream);
         default: return fail(R355_ERR_UNSUPPORTED, "tiled gemm: unknown in_type %d", g.in_type);
         }
     }
+#endif // part 0
+
+#if R355_TILED_HAS(0)
+    int gemmTiledPart0(const r355_gemm_args& g, bool aK, bool bK, uint32_t tile, const GemmTileParams& p, hipStream_t stream)
+    {
+        return g.out_type == R355_F16 ? launchLayouts<Elem::F16, _Float16>(aK, bK, tile, p, stream)
+                                      : launchLayouts<Elem::F16, float>(aK, bK, tile, p, stream);
+    }
+#endif
+#if R355_TILED_HAS(1)
+    int gemmTiledPart1(const r355_gemm_args& g, bool aK, bool bK, uint32_t tile, const GemmTileParams& p, hipStream_t stream)
+    {
+        return g.out_type == R355_BF16 ? launchLayouts<Elem::BF16, __bf16>(aK, bK, tile, p, stream)
+                                       : launchLayouts<Elem::BF16, float>(aK, bK, tile, p, stream);
+    }
+#endif
+#if R355_TILED_HAS(2)
+    int gemmTiledPart2(const r355_gemm_args& g, bool aK, bool bK, uint32_t tile, const GemmTileParams& p, hipStream_t stream)
+    {
+        if(g.in_type == R355_E4M3)
+            return launchLayouts<Elem::E4M3, float>(aK, bK, tile, p, stream);
+        if(g.in_type == R355_E5M2)
+            return launchLayouts<Elem::E5M2, float>(aK, bK, tile, p, stream);
+        return g.out_type == R355_I32 ? launchLayouts<Elem::I8, int>(aK, bK, tile, p, stream)
+                                      : launchLayouts<Elem::I8, signed char>(aK, bK, tile, p, stream);
+    }
+#endif
+#if R355_TILED_HAS(3)
+    int gemmTiledPart3(const r355_gemm_args& g, bool aK, bool bK, uint32_t tile, const GemmTileParams& p, hipStream_t stream)
+    {
+        return g.in_type == R355_F32 ? launchLayouts<Elem::F32, float>(aK, bK, tile, p, stream)
+                                     : launchLayouts<Elem::F64, double>(aK, bK, tile, p, stream);
+    }
+#endif
 } // namespace r355
