@@ -342,7 +342,7 @@ int api_relayout_store(const void* in, void* out, uint32_t ldIn, uint32_t ldOut)
     return hipDeviceSynchronize() == hipSuccess ? 0 : -2;
 }
 
-// one tile D = A B + C.  type: 0 f16, 1 bf16, 2 e4m3, 3 i8, 4 f32, 5 f16 accumulate, 6 f64, 7 e5m2; blk 16 | 32; bk per the table in the test
+// one tile D = A B + C.  type: 0 f16, 1 bf16, 2 e4m3, 3 i8, 4 f32, 5 f16 accumulate, 6 f64, 7 e5m2, 8 bf16 accumulate, 9 / 10 __half (f32 / __half accumulate); blk 16 | 32; bk per the table in the test
 int api_mma_tile(int type, uint32_t blk, uint32_t bk, int aRow, int bRow, int cRow, const void* a, const void* b,
                  const void* c, void* d, uint32_t lda, uint32_t ldb, uint32_t ldc)
 {
@@ -383,6 +383,9 @@ int api_mma_tile(int type, uint32_t blk, uint32_t bk, int aRow, int bRow, int cR
     case 5: SHAPE(float16_t, float16_t, 16, 16, 16, 32, 32, 8, 32, 16); break; // 16-bit accumulate type
     case 6: SHAPE(float64_t, float64_t, 16, 4, 16, 8, 16, 16, 16, 32); break;
     case 7: SHAPE(bfloat8_t, float32_t, 16, 32, 16, 64, 32, 16, 32, 32); break;
+    case 8: SHAPE(bfloat16_t, bfloat16_t, 16, 16, 16, 32, 32, 8, 32, 16); break;
+    case 9: SHAPE(hfloat16_t, float32_t, 16, 16, 16, 32, 32, 8, 32, 16); break; // __half operands
+    case 10: SHAPE(hfloat16_t, hfloat16_t, 16, 16, 16, 32, 32, 8, 32, 16); break;
     default: return -1;
     }
     return hipDeviceSynchronize() == hipSuccess ? 0 : -2;
