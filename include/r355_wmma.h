@@ -74,9 +74,10 @@ typedef enum
  * reference's static_cast narrows it), f32 -> f32 (f32), f64 -> f64 (f64).
  * beta == 0 means C is never read and may be NULL.
  *
- * sparse24 != 0: A is 2:4 structured-sparse along k, row-major, 1-byte elements:
+ * sparse24 != 0: A is 2:4 structured-sparse along k, row-major (i8 -> i32, e4m3 -> f32 with a macro-tile and a
+ * block-per-wave kernel; f16 | bf16 -> f32 with the block-per-wave kernel, k % 32 == 0), B col-major:
  * `a` holds the m x k/2 kept values, `a_meta` the m x k/8 index bytes (format of
- * r355_compress_24); lda is then the leading dimension of the compressed values.
+ * r355_compress_24 / r355_compress_24_16); lda is then the leading dimension of the compressed values.
  * The reference has no sparse path; this form has no counterpart there.
  */
 typedef struct
@@ -159,6 +160,9 @@ int r355_dgemv(int32_t layout_a, uint32_t m, uint32_t k, const double* a, uint32
  */
 int r355_compress_24(const uint8_t* dense, uint32_t m, uint32_t k, uint8_t* values, uint8_t* meta);
 int r355_decompress_24(const uint8_t* values, const uint8_t* meta, uint32_t m, uint32_t k, uint8_t* dense);
+/* The same for 2-byte elements (f16 / bf16 bit patterns; an element is zero when all its bits are). */
+int r355_compress_24_16(const uint16_t* dense, uint32_t m, uint32_t k, uint16_t* values, uint8_t* meta);
+int r355_decompress_24_16(const uint16_t* values, const uint8_t* meta, uint32_t m, uint32_t k, uint16_t* dense);
 
 /* Device facts used by the roofline report (test/hip_device.hpp:101-119 in the reference). */
 typedef struct

@@ -25,7 +25,7 @@ DTYPE_BYTES = {F16: 2, BF16: 2, E4M3: 1, I8: 1, F32: 4, I32: 4, F64: 8, E5M2: 1}
 
 EXPORTS = [
     "r355_gemm", "r355_gemm_query", "r355_gemm_timed", "r355_dlrm_fwd", "r355_dlrm_fwd_timed",
-    "r355_dlrm_bwd", "r355_gemv", "r355_gemv_timed", "r355_dgemv", "r355_compress_24", "r355_decompress_24",
+    "r355_dlrm_bwd", "r355_gemv", "r355_gemv_timed", "r355_dgemv", "r355_compress_24", "r355_decompress_24", "r355_compress_24_16", "r355_decompress_24_16",
     "r355_get_device_info", "r355_last_error", "r355_version",
 ]
 
@@ -93,6 +93,8 @@ def lib():
         L.r355_dgemv.argtypes = [i32, u32, u32, vp, u32, vp, vp, vp, ctypes.c_double, ctypes.c_double, vp]
         L.r355_compress_24.argtypes = [vp, u32, u32, vp, vp]
         L.r355_decompress_24.argtypes = [vp, vp, u32, u32, vp]
+        L.r355_compress_24_16.argtypes = [vp, u32, u32, vp, vp]
+        L.r355_decompress_24_16.argtypes = [vp, vp, u32, u32, vp]
         L.r355_get_device_info.argtypes = [ctypes.POINTER(DeviceInfo)]
         L.r355_last_error.restype = ctypes.c_char_p
         L.r355_version.restype = ctypes.c_char_p
@@ -207,14 +209,16 @@ def gemv_timed(layout_a, m, k, a, x, y_in, y_out, alpha, beta, warmup, iters, ld
 
 
 def compress_24(dense):
-    """Host-side 2:4 compression of a (m, k) uint8/int8 numpy array -> (values, meta)."""
+    """Host-side 2:4 compression of a (m, k) numpy array of 1-byte (uint8 / int8) or 2-byte (uint16: f16 / bf16
+    bit patterns, or float16) elements -> (values, meta)."""
     import numpy as np
 
     dense = np.ascontiguousarray(dense)
     m, k = dense.shape
     values = np.zeros((m, k // 2), dtype=dense.dtype)
     meta = np.zeros((m, k // 8), dtype=np.uint8)
-    _check(lib().r355_compress_24(_ptr(dense), m, k, _ptr(values), _ptr(meta)))
+    fn = {1: lib().r355_compress_24, 2: lib().r355_compress_24_16}[dense.dtype.itemsize]
+    _check(fn(_ptr(dense), m, k, _ptr(values), _ptr(meta)))
     return values, meta
 
 
@@ -224,7 +228,8 @@ def decompress_24(values, meta):
     values, meta = np.ascontiguousarray(values), np.ascontiguousarray(meta)
     m, k = values.shape[0], values.shape[1] * 2
     dense = np.zeros((m, k), dtype=values.dtype)
-    _check(lib().r355_decompress_24(_ptr(values), _ptr(meta), m, k, _ptr(dense)))
+    fn = {1: lib().r355_decompress_24, 2: lib().r355_decompress_24_16}[values.dtype.itemsize]
+    _check(fn(_ptr(values), _ptr(meta), m, k, _ptr(dense)))
     return dense
 
 

@@ -132,6 +132,33 @@ def test_compress_24_host_roundtrip_and_rejection():
     assert e.value.code == -6 and "row 3" in str(e.value)
 
 
+def test_compress_24_16bit_elements_same_format():
+    """2-byte elements: the metadata is what the 1-byte compressor writes for the same non-zero pattern, the kept
+    values are the 2-byte elements at the positions the nibbles name (checked with plain numpy indexing)."""
+    import oraclelib as O
+
+    m, k = 16, 64
+    mask = O.sparse24_mask(11, m, k)
+    dense = np.where(mask, (np.arange(m * k).reshape(m, k) % 60000 + 1), 0).astype(np.uint16)
+    dense[2, 8:12] = 0  # an all-zero group keeps positions 0 and 1
+    dense[5, 16:20] = [0, 0x8000, 0, 0]  # -0.0 is a kept value: all-zero bits are what counts as zero
+    vals, meta = R.compress_24(dense)
+    _, meta8 = R.compress_24((dense != 0).astype(np.uint8))
+    assert np.array_equal(meta, meta8)
+    nib = np.stack([meta & 0xF, meta >> 4], axis=-1).reshape(m, k // 4)
+    pos0, pos1 = nib & 3, nib >> 2
+    assert np.all(pos0 < pos1)
+    grp = dense.reshape(m, k // 4, 4)
+    assert np.array_equal(vals[:, 0::2], np.take_along_axis(grp, pos0[..., None].astype(np.int64), axis=2)[..., 0])
+    assert np.array_equal(vals[:, 1::2], np.take_along_axis(grp, pos1[..., None].astype(np.int64), axis=2)[..., 0])
+    assert np.array_equal(R.decompress_24(vals, meta), dense)
+    bad = dense.copy()
+    bad[3, 4:8] = 1
+    with pytest.raises(R.R355Error) as e:
+        R.compress_24(bad)
+    assert e.value.code == -6
+
+
 @pytest.mark.gpu
 def test_entry_points_can_be_captured_in_a_hip_graph():
     """The C ABI allocates nothing and only launches kernels on the stream it is given, so its calls can be

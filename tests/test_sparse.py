@@ -60,3 +60,46 @@ def test_sparse_config4_sampled_rows():
     assert np.array_equal(got[rows], want)
     B = b.reshape(n, k).astype(np.int64)
     assert int(got.astype(np.int64).sum()) == int(dense.astype(np.int64).sum(axis=0) @ B.sum(axis=0))
+
+
+@pytest.mark.parametrize("in_t", [O.F16, O.BF16])
+@pytest.mark.parametrize("m,n,k", [(32, 32, 32), (96, 64, 96), (256, 128, 1024), (64, 32, 4096)])
+@pytest.mark.parametrize("ldl", [O.ROW, O.COL])
+def test_sparse_gemm_16bit_vs_dense_oracle(in_t, m, n, k, ldl):
+    """f16 / bf16 operands on v_smfmac_f32_32x32x32_{f16,bf16} (block-per-wave kernel), f32 out.  Same products as the
+    oracle's dense GEMM on the decompressed A, summed in another order: the 16-bit bar of 1e-3 on the relative metric."""
+    mask = O.sparse24_mask(70, m, k)
+    a = O.f32_to_storage(O.uniform_pm1(71, m * k), in_t).reshape(m, k)
+    dense = np.where(mask, a, np.uint16(0)).astype(np.uint16)
+    b = O.f32_to_storage(O.uniform_pm1(72, k * n), in_t)
+    vals, meta = R.compress_24(dense)
+    assert vals.dtype == np.uint16 and np.array_equal(R.decompress_24(vals, meta), dense)
+    c = O.uniform_pm1(73, m * n)
+    want = O.gemm(in_t, O.F32, O.ROW, O.COL, ldl, ldl, m, n, k, dense.ravel(), b, c, 2.0, 2.0)
+    dv, dm, db, dc = to_device(vals), to_device(meta), to_device(b), to_device(c)
+    dd = device_filled(m * n, np.float32, 0xFF)
+    R.gemm(in_t, O.F32, m, n, k, dv, db, dc, dd, 2.0, 2.0, O.ROW, O.COL, ldl, ldl, a_meta=dm)
+    got = to_host(dd, np.float32)
+    plan = R.gemm_query(R.gemm_args(in_t, O.F32, m, n, k, dv, db, dc, dd, 2.0, 2.0, O.ROW, O.COL, ldl, ldl, a_meta=dm))
+    assert plan.kernel == R.KERNEL_SIMPLE and plan.macro_tile_k == 32
+    g, w = got.astype(np.float64), want.astype(np.float64)
+    assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= 1e-3
+
+
+def test_sparse_16bit_one_hot_positions():
+    """Every (row, kept position) of A in turn is the only non-zero: D must be that row of B scaled - exact, and it
+    fails for any wrong pairing of lane groups or index bits."""
+    m, n, k = 32, 32, 64
+    b = O.f32_to_storage(((np.arange(k * n) % 2039) - 1000).astype(np.float32), O.F16)  # distinct small integers
+    bf = b.view(np.float16).astype(np.float32).reshape(n, k)  # col-major B: bf[col, kk]
+    db = to_device(b)
+    for kk in range(k):
+        dense = np.zeros((m, k), dtype=np.uint16)
+        cols = (kk + np.arange(m)) % k  # row r has its 1 at column (kk + r) % k
+        dense[np.arange(m), cols] = np.float16(1.0).view(np.uint16)
+        vals, meta = R.compress_24(dense)
+        dv, dm = to_device(vals), to_device(meta)
+        dd = device_filled(m * n, np.float32, 0xFF)
+        R.gemm(O.F16, O.F32, m, n, k, dv, db, None, dd, 1.0, 0.0, O.ROW, O.COL, O.ROW, O.ROW, a_meta=dm)
+        got = to_host(dd, np.float32).reshape(m, n)
+        assert np.array_equal(got, bf[:, cols].T), kk
