@@ -3,6 +3,8 @@
 //   LoadStoreMatrixCoopSync{A,B,Acc}  test/unit/load_store_matrix_coop_sync_test/device/load_store_matrix_coop_sync.hpp
 //   fillFragment{A,B,Acc}             test/unit/fill_fragment_test/device/fill_fragment.hpp
 //   loadContamination{A,B,Acc}, storeContamination{A,B,Acc}   test/unit/contamination_test/device/*.hpp
+//   MapBlockToMatrix[OverrideM|N], MapMatrixToData[OverrideM|N], MapThreadToMatrix, MapWaveToMatrix
+//                                     test/unit/map_util_test/device/*.hpp
 // Every kernel has the suite's uniform signature (m, n, in, out, ld, param1, param2) and is launched on
 // 128 x 2 threads (2 x 2 waves), one block of the matrix per wave, grid from the problem size
 // (test/unit/unit_kernel_base_impl.hpp).  The kernels enable their bodies only for architecture ids
@@ -21,6 +23,12 @@
 #include "unit/fill_fragment_test/device/fill_fragment.hpp"
 #include "unit/load_store_matrix_coop_sync_test/device/load_store_matrix_coop_sync.hpp"
 #include "unit/load_store_matrix_sync_test/device/load_store_matrix_sync.hpp"
+#include "unit/map_util_test/device/map_block_to_matrix.hpp"
+#include "unit/map_util_test/device/map_block_to_matrix_override.hpp"
+#include "unit/map_util_test/device/map_matrix_to_data.hpp"
+#include "unit/map_util_test/device/map_matrix_to_data_override.hpp"
+#include "unit/map_util_test/device/map_thread_to_matrix.hpp"
+#include "unit/map_util_test/device/map_wave_to_matrix.hpp"
 
 // (id, BlockM, BlockN, type, layout): block extents from test/unit/unit_test_params.hpp:89-139
 #define UNIT_CASES(X)                        \
@@ -65,7 +73,8 @@ extern "C" int ref_unit_case_info(int id, uint32_t* blockM, uint32_t* blockN, ui
 }
 
 // kind: 0..2 LoadStoreMatrixSync A/B/Acc, 3..5 LoadStoreMatrixCoopSync A/B/Acc, 6..8 fillFragment A/B/Acc,
-// 9..11 loadContamination A/B/Acc, 12..14 storeContamination A/B/Acc
+// 9..11 loadContamination A/B/Acc, 12..14 storeContamination A/B/Acc, 15..17 MapBlockToMatrix / OverrideM / OverrideN,
+// 18..20 MapMatrixToData / OverrideM / OverrideN, 21 MapThreadToMatrix, 22 MapWaveToMatrix
 extern "C" int ref_unit_run(int kind, int id, uint32_t m, uint32_t n, const void* in, void* out, uint32_t ld, double p1,
                             double p2)
 {
@@ -95,6 +104,14 @@ extern "C" int ref_unit_run(int kind, int id, uint32_t m, uint32_t n, const void
         case 12: LAUNCH(storeContaminationA, BM, BN, T, L); break;         \
         case 13: LAUNCH(storeContaminationB, BM, BN, T, L); break;         \
         case 14: LAUNCH(storeContaminationAcc, BM, BN, T, L); break;       \
+        case 15: LAUNCH(MapBlockToMatrix, BM, BN, T, L); break;            \
+        case 16: LAUNCH(MapBlockToMatrixOverrideM, BM, BN, T, L); break;   \
+        case 17: LAUNCH(MapBlockToMatrixOverrideN, BM, BN, T, L); break;   \
+        case 18: LAUNCH(MapMatrixToData, BM, BN, T, L); break;             \
+        case 19: LAUNCH(MapMatrixToDataOverrideM, BM, BN, T, L); break;    \
+        case 20: LAUNCH(MapMatrixToDataOverrideN, BM, BN, T, L); break;    \
+        case 21: LAUNCH(MapThreadToMatrix, BM, BN, T, L); break;           \
+        case 22: LAUNCH(MapWaveToMatrix, BM, BN, T, L); break;             \
         default: return -1;                                               \
         }                                                                 \
         break;

@@ -1,5 +1,6 @@
 """The reference's unit-test device kernels (test/unit/**/device/*.hpp: load/store round trip, cooperative
-load/store, fill, load and store contamination, for matrix_a / matrix_b / accumulator fragments), compiled
+load/store, fill, load and store contamination, for matrix_a / matrix_b / accumulator fragments, and the
+MappingUtil kernels of test/unit/map_util_test), compiled
 UNCHANGED against this library's headers by tests/kernels/build_ref_samples.py where the reference tree is
 available, checked with the reference suite's own pass criteria on MI355X.  The shared object is a build
 output (tests/kernels/_ref/); when it is absent the tests skip."""
@@ -123,3 +124,45 @@ def test_load_and_store_contamination(cid, role):
     assert np.array_equal(got[pr:pr + m, pc:pc + n], mat)
     got[pr:pr + m, pc:pc + n] = canary
     assert np.all(got == canary)
+
+
+# MappingUtil (test/unit/map_util_test): every wave copies the block its coordinates name; 2 x 2 workgroups of
+# 2 x 2 waves cover a 4 x 4 grid of blocks
+@pytest.mark.parametrize("kind", [15, 18, 21, 22])
+@pytest.mark.parametrize("cid", range(N_CASES))
+def test_map_util_identity_copies(cid, kind):
+    # MapBlockToMatrix, MapMatrixToData, MapThreadToMatrix, MapWaveToMatrix: pass criterion output == input
+    # (test/unit/map_util_test/detail/map_block_to_matrix.hpp:65-79)
+    bm, bn, eb, rm = _info(cid)
+    m, n = 4 * bm, 4 * bn
+    mat = _matrix(m, n, eb, 300 + cid)
+    d_in, d_out = to_device(_flat(mat, rm)), device_filled(m * n, _DT[eb], 0xEE)
+    _run(kind, cid, m, n, d_in, d_out, n if rm else m)
+    assert np.array_equal(_unflat(to_host(d_out, _DT[eb]), m, n, rm), mat)
+
+
+@pytest.mark.parametrize("override", [0, 1, 3])
+@pytest.mark.parametrize("kind", [16, 17, 19, 20])
+@pytest.mark.parametrize("cid", range(0, N_CASES, 2))
+def test_map_util_block_overrides(cid, kind, override):
+    # ...OverrideM / ...OverrideN: every block is read from block row (column) param1 - MapMatrixToData...: from matrix
+    # row (column) param1 - instead of its own, and written to its own place
+    # (test/unit/map_util_test/detail/map_block_to_matrix_override.hpp:118-150, map_matrix_to_data_override.hpp:130-150)
+    bm, bn, eb, rm = _info(cid)
+    m, n = 4 * bm, 4 * bn
+    along_m = kind in (16, 19)
+    blk = bm if along_m else bn
+    if kind in (16, 17):
+        param, first = override, override * blk
+    else:  # a matrix coordinate; kept on 16-element steps so that the fragments' vector accesses stay aligned
+        param = first = min(16 * override * override, 3 * blk) // 16 * 16
+    mat = _matrix(m, n, eb, 400 + cid)
+    d_in, d_out = to_device(_flat(mat, rm)), device_filled(m * n, _DT[eb], 0xEE)
+    _run(kind, cid, m, n, d_in, d_out, n if rm else m, float(param))
+    want = mat.copy()
+    for b in range(4):
+        if along_m:
+            want[b * bm:(b + 1) * bm, :] = mat[first:first + bm, :]
+        else:
+            want[:, b * bn:(b + 1) * bn] = mat[:, first:first + bn]
+    assert np.array_equal(_unflat(to_host(d_out, _DT[eb]), m, n, rm), want)
