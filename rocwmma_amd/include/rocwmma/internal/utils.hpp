@@ -9,11 +9,22 @@ namespace rocwmma
 {
     using Coord2dDataT = uint32_t;
 
-    // (x, y) pair usable in constant expressions on host and device.
+    // (x, y) pair usable in constant expressions on host and device, with the element-wise arithmetic the
+    // reference's two-element vector offers (vector.hpp:157-214 there): user kernels scale and step coordinates
+    // in place (test/gemm/gemm_PGR0_LB0_MP0_MB_NC/device/kernel_device_func.hpp:110).
     struct Coord2d
     {
         Coord2dDataT x;
         Coord2dDataT y;
+
+        ROCWMMA_HOST_DEVICE constexpr inline Coord2dDataT& operator[](unsigned int idx) noexcept
+        {
+            return idx == 0u ? x : y;
+        }
+        ROCWMMA_HOST_DEVICE constexpr inline Coord2dDataT operator[](unsigned int idx) const noexcept
+        {
+            return idx == 0u ? x : y;
+        }
     };
 
     template <uint32_t Idx>
@@ -62,9 +73,52 @@ namespace rocwmma
         return l;
     }
 
+    ROCWMMA_HOST_DEVICE constexpr inline Coord2d operator/(Coord2d const& l, Coord2d const& r)
+    {
+        return Coord2d{l.x / r.x, l.y / r.y};
+    }
+
+    ROCWMMA_HOST_DEVICE constexpr inline Coord2d operator%(Coord2d const& l, Coord2d const& r)
+    {
+        return Coord2d{l.x % r.x, l.y % r.y};
+    }
+
+    ROCWMMA_HOST_DEVICE constexpr inline Coord2d& operator-=(Coord2d& l, Coord2d const& r)
+    {
+        l.x -= r.x;
+        l.y -= r.y;
+        return l;
+    }
+
+    ROCWMMA_HOST_DEVICE constexpr inline Coord2d& operator*=(Coord2d& l, Coord2d const& r)
+    {
+        l.x *= r.x;
+        l.y *= r.y;
+        return l;
+    }
+
+    ROCWMMA_HOST_DEVICE constexpr inline Coord2d& operator/=(Coord2d& l, Coord2d const& r)
+    {
+        l.x /= r.x;
+        l.y /= r.y;
+        return l;
+    }
+
+    ROCWMMA_HOST_DEVICE constexpr inline Coord2d& operator%=(Coord2d& l, Coord2d const& r)
+    {
+        l.x %= r.x;
+        l.y %= r.y;
+        return l;
+    }
+
     ROCWMMA_HOST_DEVICE constexpr inline bool operator==(Coord2d const& l, Coord2d const& r)
     {
         return l.x == r.x && l.y == r.y;
+    }
+
+    ROCWMMA_HOST_DEVICE constexpr inline bool operator!=(Coord2d const& l, Coord2d const& r)
+    {
+        return !(l == r);
     }
 
     template <typename IntT1,

@@ -219,6 +219,25 @@ namespace
     X(92, accumulator, 16, 16, 16, float64_t, col_major)                               \
     X(93, matrix_a, 64, 16, 8, float64_t, col_major)
 
+// Coord2d arithmetic is element-wise and usable in constant expressions (the reference's two-element vector)
+namespace
+{
+    constexpr rocwmma::Coord2d coordOps()
+    {
+        auto c = rocwmma::make_coord2d(6u, 20u);
+        c *= rocwmma::make_coord2d(2u, 3u); // 12, 60
+        c -= rocwmma::make_coord2d(2u, 4u); // 10, 56
+        c /= rocwmma::make_coord2d(2u, 8u); // 5, 7
+        c %= rocwmma::make_coord2d(3u, 4u); // 2, 3
+        c += rocwmma::make_coord2d(1u, 1u); // 3, 4
+        return c;
+    }
+    static_assert(coordOps() == rocwmma::make_coord2d(3u, 4u) && coordOps() != rocwmma::make_coord2d(3u, 5u));
+    static_assert(coordOps()[0] == 3u && coordOps()[1] == 4u && rocwmma::get<1>(coordOps()) == 4u);
+    static_assert(rocwmma::make_coord2d(9u, 8u) / rocwmma::make_coord2d(2u, 4u) == rocwmma::make_coord2d(4u, 2u));
+    static_assert(rocwmma::make_coord2d(9u, 8u) % rocwmma::make_coord2d(2u, 5u) == rocwmma::make_coord2d(1u, 3u));
+} // namespace
+
 extern "C" {
 
 // Describes a case: rows, cols of the block in memory, element bytes; returns 0 if the id exists.

@@ -224,6 +224,33 @@ def test_reference_gemm_test_kernel_block_per_wave(cid, in_t, out_t, la, lb):
         assert ok, mx
 
 
+@pytest.mark.parametrize("cid,in_t,out_t,la,lb", [(0, O.F16, O.F32, O.ROW, O.COL), (1, O.BF16, O.BF16, O.COL, O.ROW),
+                                                  (2, O.I8, O.I32, O.ROW, O.COL), (3, O.F16, O.F16, O.ROW, O.ROW)])
+def test_reference_gemm_test_kernel_multi_block(cid, in_t, out_t, la, lb):
+    # test/gemm/gemm_PGR0_LB0_MP0_MB_NC/device/kernel_device_func.hpp: BlocksX x BlocksY blocks per wave
+    # (2 x 2, 4 x 2, 2 x 4, 8 x 8), no LDS, no cooperation
+    L = _lib("test_gemm_multi")
+    m, n, k = 256, 256, 96
+    if in_t == O.I8:
+        a, b = O.uniform_int8(24, m * k), O.uniform_int8(25, k * n)
+        c = O.uniform_int8(26, m * n).astype(np.int32) * 11
+    else:
+        a = O.f32_to_storage(O.uniform_pm1(24, m * k), in_t)
+        b = O.f32_to_storage(O.uniform_pm1(25, k * n), in_t)
+        c = O.f32_to_storage(O.uniform_pm1(26, m * n), out_t)
+    st = O.NP_STORAGE[out_t]
+    da, db, dc, dd = to_device(a), to_device(b), to_device(c), device_filled(m * n, st, 0xFF)
+    lda, ldb = (k if la == O.ROW else m), (n if lb == O.ROW else k)
+    assert L.ref_test_gemm_multi(cid, *_gemm_args(m, n, k, da, db, dc, dd, lda, ldb, 2.0, 2.0)) == 0
+    want = O.gemm(in_t, out_t, la, lb, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, 2.0)
+    got = to_host(dd, st)
+    if in_t == O.I8:
+        assert np.array_equal(got, want)
+    else:
+        ok, mx = O.compare(out_t, got, want, 10.0 if out_t in (O.F16, O.BF16) else k / 2.0)
+        assert ok, mx
+
+
 @pytest.mark.parametrize("lds_col_major", [0, 1])
 @pytest.mark.parametrize("cid", range(6))
 def test_reference_gemm_test_kernel_cooperative(cid, lds_col_major):
