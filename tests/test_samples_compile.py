@@ -48,6 +48,7 @@ TEST_DEVICE_HEADERS = [
     "dlrm/device/dlrm_dot_fwd.hpp",
     "dlrm/device/dlrm_dot_bwd.hpp",
     "gemm/gemm_PGR0_LB0_MP0_SB_NC/device/kernel_device_func.hpp",
+    "gemm/gemm_PGR0_LB0_MP0_MB_NC/device/kernel_device_func.hpp",
     "gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp",
     "dlrm/device/dlrm_dot_fwd_lds.hpp",
     "dlrm/device/dlrm_dot_bwd_lds.hpp",
@@ -73,3 +74,19 @@ def test_reference_test_device_header_compiles_unchanged(header):
              os.path.join(tmp, "tu.o")],
             capture_output=True, text=True)
         assert r.returncode == 0, r.stderr[-2000:]
+
+
+def test_version_header_reports_the_api_version():
+    """rocwmma/rocwmma-version.hpp: the three macros and rocwmma_get_version() the reference configures at build time
+    (library/include/rocwmma/internal/rocwmma-version.hpp.in), host-only."""
+    gxx = shutil.which("g++")
+    if gxx is None:
+        pytest.skip("needs g++")
+    with tempfile.TemporaryDirectory() as tmp:
+        src, exe = os.path.join(tmp, "v.cpp"), os.path.join(tmp, "v")
+        with open(src, "w") as f:
+            f.write('#include <rocwmma/rocwmma-version.hpp>\n#include <cstdio>\n'
+                    'int main() { std::printf("%s %d", rocwmma_get_version().c_str(), ROCWMMA_VERSION_MAJOR * 10000 + '
+                    'ROCWMMA_VERSION_MINOR * 100 + ROCWMMA_VERSION_PATCH); }\n')
+        subprocess.check_call([gxx, "-std=c++17", "-I" + os.path.join(ROOT, "rocwmma_amd", "include"), src, "-o", exe])
+        assert subprocess.check_output([exe], text=True) == "1.6.0 10600"
