@@ -11,7 +11,8 @@ ROOT = os.path.dirname(os.path.dirname(HERE))
 REF = os.environ.get("REFERENCE_ROOT", "/root/reference")
 OUT = os.path.join(HERE, "_ref")
 WRAPPERS = ["simple_hgemm", "perf_hgemm", "simple_dlrm", "simple_sgemv", "simple_sgemm", "simple_dgemm", "perf_sgemm",
-            "perf_dgemm", "test_dlrm", "test_io_traits", "test_gemm_simple", "test_gemm_multi", "test_gemm_coop", "test_unit"]
+            "perf_dgemm", "test_dlrm", "test_io_traits", "test_gemm_simple", "test_gemm_multi", "test_gemm_coop", "test_gemm_coop_typed",
+            "test_unit"]
 
 
 def _compile(name, samples):

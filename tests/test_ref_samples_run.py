@@ -267,3 +267,39 @@ def test_reference_gemm_test_kernel_cooperative(cid, lds_col_major):
     want = O.gemm(O.F16, O.F16, O.COL, O.ROW, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, 2.0)
     ok, mx = O.compare(O.F16, to_host(dd, np.uint16), want, 10.0)
     assert ok, mx
+
+
+_COOP_TYPED = {0: (O.I8, O.I32, O.ROW, O.COL), 1: (O.BF16, O.F32, O.ROW, O.ROW), 2: (O.F32, O.F32, O.COL, O.COL),
+               3: (O.F64, O.F64, O.ROW, O.COL), 4: (O.E4M3, O.F32, O.COL, O.ROW)}
+
+
+@pytest.mark.parametrize("cfg", range(3))
+@pytest.mark.parametrize("variant", sorted(_COOP_TYPED))
+def test_reference_gemm_test_kernel_cooperative_other_types(variant, cfg):
+    # the same kernel with int8, bf16, f32, f64 and e4m3 operands in the other operand orientations (TN, TT, NN):
+    # the type tuples of test/gemm/gemm_common_test_params.hpp:50-130, three of the CooperativeGemm configurations
+    L = _lib("test_gemm_coop_typed")
+    in_t, out_t, la, lb = _COOP_TYPED[variant]
+    m, n, k = 256, 384, 128
+    if in_t == O.I8:
+        a, b = O.uniform_int8(41, m * k), O.uniform_int8(42, k * n)
+        c = O.uniform_int8(43, m * n).astype(np.int32) * 11
+    else:
+        src = O.normal if in_t == O.E4M3 else O.uniform_pm1
+        a = O.f32_to_storage(src(41, m * k), in_t)
+        b = O.f32_to_storage(src(42, k * n), in_t)
+        c = O.f32_to_storage(O.uniform_pm1(43, m * n), out_t)
+    st = O.NP_STORAGE[out_t]
+    da, db, dc, dd = to_device(a), to_device(b), to_device(c), device_filled(m * n, st, 0xFF)
+    lda, ldb = (k if la == O.ROW else m), (n if lb == O.ROW else k)
+    assert L.ref_test_gemm_coop_typed(variant, cfg, *_gemm_args(m, n, k, da, db, dc, dd, lda, ldb, 2.0, 2.0)) == 0
+    want = O.gemm(in_t, out_t, la, lb, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, 2.0)
+    got = to_host(dd, st)
+    if in_t == O.I8:
+        assert np.array_equal(got, want)
+    elif in_t == O.E4M3:
+        g, w = got.astype(np.float64), want.astype(np.float64)
+        assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= 1e-2
+    else:
+        ok, mx = O.compare(out_t, got, want, k / 2.0)
+        assert ok, mx
