@@ -102,7 +102,10 @@ typedef struct
 int r355_gemm(const r355_gemm_args* args, void* stream);
 
 /* Launch description the AUTO/TILED/SIMPLE choice resolves to, without launching
- * (the values the reference computes on the host: samples/perf_hgemm.cpp:807-817). */
+ * (the values the reference computes on the host: samples/perf_hgemm.cpp:807-817).
+ * R355_KERNEL_AUTO may split a problem of several rounds of 256 x 256 tiles into two launches on the
+ * same stream - whole rounds on that tile, the rest (at most half a round) on 128 x 128 tiles; the
+ * plan then describes the first launch. */
 typedef struct
 {
     int32_t  kernel;                       /* r355_gemm_kernel actually selected */

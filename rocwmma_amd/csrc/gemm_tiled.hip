@@ -67,6 +67,9 @@ namespace r355
         uint32_t    lda, ldb, ldc, ldd; // elements
         float       alpha, beta;
         uint32_t    tilesM, tilesN;
+        // the launch covers tile indices [tileFirst, tileFirst + tileCount) of the tilesM x tilesN walk; with
+        // tileQuad the walk is over tiles of twice the kernel's edge, four workgroups each (tile_map.hpp)
+        uint32_t tileFirst, tileCount, tileQuad;
     };
     // launch of one kernel family; aK / bK: operand is K-contiguous; tile: 256 or 128
     int gemmTiledPart0(const r355_gemm_args& g, bool aK, bool bK, uint32_t tile, const GemmTileParams& p, hipStream_t s);
@@ -342,8 +345,10 @@ namespace
         __shared__ __attribute__((aligned(1024))) char stage1[2u * OPER];
 
         uint32_t tm, tn;
-        if(!r355::tileCoord(blockIdx.x, p.tilesM, p.tilesN, tm, tn))
+        if(!r355::tileCoordRange(blockIdx.x, p.tilesM, p.tilesN, p.tileFirst, p.tileCount, p.tileQuad != 0u, tm, tn))
             return;
+        if(p.tileQuad && (tm * TILE >= p.m || tn * TILE >= p.n))
+            return; // a quarter of a partial edge tile that lies outside the matrix
 
         const uint32_t tid  = threadIdx.x;
         const uint32_t lane = tid & 63u;
@@ -858,8 +863,10 @@ namespace
         __shared__ __attribute__((aligned(1024))) char lds[5u * OPER];
 
         uint32_t tm, tn;
-        if(!r355::tileCoord(blockIdx.x, p.tilesM, p.tilesN, tm, tn))
+        if(!r355::tileCoordRange(blockIdx.x, p.tilesM, p.tilesN, p.tileFirst, p.tileCount, p.tileQuad != 0u, tm, tn))
             return;
+        if(p.tileQuad && (tm * TILE >= p.m || tn * TILE >= p.n))
+            return; // a quarter of a partial edge tile that lies outside the matrix
 
         const uint32_t tid  = threadIdx.x;
         const uint32_t lane = tid & 63u;
@@ -1106,8 +1113,10 @@ namespace
         __shared__ __attribute__((aligned(1024))) char lds[5u * OPER];
 
         uint32_t tm, tn;
-        if(!r355::tileCoord(blockIdx.x, p.tilesM, p.tilesN, tm, tn))
+        if(!r355::tileCoordRange(blockIdx.x, p.tilesM, p.tilesN, p.tileFirst, p.tileCount, p.tileQuad != 0u, tm, tn))
             return;
+        if(p.tileQuad && (tm * TILE >= p.m || tn * TILE >= p.n))
+            return; // a quarter of a partial edge tile that lies outside the matrix
 
         const uint32_t tid  = threadIdx.x;
         const uint32_t lane = tid & 63u;
@@ -1303,7 +1312,8 @@ namespace
     template <Elem E, typename OutT>
     int launchLayouts(bool aK, bool bK, uint32_t tile, const Params& p, hipStream_t stream)
     {
-        const dim3 grid(((p.tilesM * p.tilesN + 7u) / 8u) * 8u), block(THREADS);
+        // every XCD gets ceil(count / 8) tile indices (four workgroups each in a quad launch)
+        const dim3 grid(((p.tileCount + 7u) / 8u) * 8u * (p.tileQuad ? 4u : 1u)), block(THREADS);
         auto launch = [&](auto aKc, auto bKc) {
             constexpr bool AK = decltype(aKc)::value, BK = decltype(bKc)::value;
             if constexpr(E == Elem::I8)
@@ -1380,6 +1390,21 @@ namespace
         auto           rounds = [&](uint32_t t) { return ((uint64_t)((g.m + t - 1) / t) * ((g.n + t - 1) / t) + cus - 1) / cus; };
         return rounds(128u) * 5u < rounds(256u) * 11u ? 128u : 256u;
     }
+
+    // Mixed tiling (R355_KERNEL_AUTO only).  A problem of a few rounds whose last round of 256 x 256 tiles would
+    // occupy at most half of the CUs runs that last part on 128 x 128 tiles instead, in a second launch: four small
+    // tiles per large one, two workgroups per CU, together about 0.4 (up to a quarter of the CUs' worth of large
+    // tiles) or 0.6 of a large-tile round instead of a whole one.  Returns the number of 256 x 256 tile indices the
+    // second launch covers, 0 for a single launch.
+    uint32_t mixedRemainder(const r355_gemm_args& g)
+    {
+        if(g.kernel != R355_KERNEL_AUTO || g.in_type == R355_F32 || g.in_type == R355_F64 || macroTile(g) != 256u)
+            return 0u;
+        const uint32_t cus   = computeUnits();
+        const uint32_t total = ((g.m + 255u) / 256u) * ((g.n + 255u) / 256u);
+        const uint32_t rest  = total % cus;
+        return (total > cus && rest != 0u && rest <= cus / 2u) ? rest : 0u;
+    }
 #endif // part 0
 } // namespace
 
@@ -1420,7 +1445,8 @@ namespace r355
             plan->macro_tile_m = tile;
             plan->macro_tile_n = tile;
             plan->macro_tile_k = tk;
-            plan->grid_x       = ((((g.m + tile - 1) / tile) * ((g.n + tile - 1) / tile) + 7u) / 8u) * 8u;
+            // with mixed tiling: the first launch (the second covers mixedRemainder(g) tile indices on 128 x 128 tiles)
+            plan->grid_x       = ((((g.m + tile - 1) / tile) * ((g.n + tile - 1) / tile) - mixedRemainder(g) + 7u) / 8u) * 8u;
             plan->grid_y       = 1;
             plan->block_x      = THREADS;
             plan->block_y      = 1;
@@ -1457,17 +1483,29 @@ namespace r355
         }
         const uint32_t tile = macroTile(g);
         p.tilesM = (p.m + tile - 1) / tile, p.tilesN = (p.n + tile - 1) / tile;
-        switch(g.in_type)
-        {
-        case R355_F16: return gemmTiledPart0(g, aK, bK, tile, p, stream);
-        case R355_BF16: return gemmTiledPart1(g, aK, bK, tile, p, stream);
-        case R355_E4M3:
-        case R355_E5M2:
-        case R355_I8: return gemmTiledPart2(g, aK, bK, tile, p, stream);
-        case R355_F32:
-        case R355_F64: return gemmTiledPart3(g, aK, bK, tile, p, stream);
-        default: return fail(R355_ERR_UNSUPPORTED, "tiled gemm: unknown in_type %d", g.in_type);
-        }
+        p.tileFirst = 0u, p.tileCount = p.tilesM * p.tilesN, p.tileQuad = 0u;
+        auto part = [&](uint32_t t, const Params& q) {
+            switch(g.in_type)
+            {
+            case R355_F16: return gemmTiledPart0(g, aK, bK, t, q, stream);
+            case R355_BF16: return gemmTiledPart1(g, aK, bK, t, q, stream);
+            case R355_E4M3:
+            case R355_E5M2:
+            case R355_I8: return gemmTiledPart2(g, aK, bK, t, q, stream);
+            case R355_F32:
+            case R355_F64: return gemmTiledPart3(g, aK, bK, t, q, stream);
+            default: return fail(R355_ERR_UNSUPPORTED, "tiled gemm: unknown in_type %d", g.in_type);
+            }
+        };
+        const uint32_t rest = mixedRemainder(g);
+        if(rest == 0u)
+            return part(tile, p);
+        // whole rounds on 256 x 256 tiles, then the rest of the walk on 128 x 128 tiles, four per index
+        Params big = p, small = p;
+        big.tileCount   = p.tileCount - rest;
+        small.tileFirst = big.tileCount, small.tileCount = rest, small.tileQuad = 1u;
+        const int rc = part(256u, big);
+        return rc != R355_OK ? rc : part(128u, small);
     }
 #endif // part 0
 
