@@ -25,12 +25,44 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "e4m3": 5000.0, "i8": 5000.0, "f32": 157.3, "f64": 78.6}
 HBM_PEAK_GBPS = 8000.0
-# Bytes one 8192^3 f16 NT launch moves across the L2 <-> fabric boundary, from two rocprofv3 --pmc
-# runs of `host_bench gemm --type f16 --layout nt`: FETCH_SIZE 7.866e5 x 2 KiB + WRITE_SIZE 1.311e5
-# x 1 KiB (unit sizes calibrated with `host_bench copy --bytes 1073741824`, which reads 5.243e5 and
-# writes 1.049e6 units for 1 GiB each way).  The fetch side is 6 x the 256 MiB of A and B: each
-# 4 MiB operand panel is fetched once per group of tiles that share an XCD's L2.
-TRAFFIC_F16_NT_8192 = int(7.866e5 * 2048 + 1.311e5 * 1024)
+# rocprofv3 --pmc results per benchmark case (MFMA busy, LDS bank conflicts, bytes across the L2 <-> fabric
+# boundary), one table row per case.  Each row carries the SHA-256 (first 16 hex digits) of the kernel sources it
+# was measured on; a row whose digest differs from the sources of this tree is reported as null, so a counter
+# can never outlive the kernel it belongs to.
+COUNTERS_FILE = os.path.join(ROOT, "profiles", "bench_counters.md")
+KERNEL_SOURCES = {"gemm": ["gemm_tiled.hip", "tile_map.hpp", "lds_dma.hpp"], "sparse": ["sparse.hip", "tile_map.hpp", "lds_dma.hpp"],
+                  "dlrm": ["dlrm.hip"]}
+
+
+def source_digest(family):
+    import hashlib
+
+    h = hashlib.sha256()
+    for f in KERNEL_SOURCES[family]:
+        with open(os.path.join(ROOT, "rocwmma_amd", "csrc", f), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+def load_counters():
+    """{case: {"mfma_busy_pct", "lds_bank_conflicts", "fetch_bytes", "write_bytes"}} from the table rows
+    `| case | family | digest | MFMA busy % | LDS bank conflicts | fetch bytes | write bytes |` whose digest matches."""
+    out = {}
+    if not os.path.exists(COUNTERS_FILE):
+        return out
+    digests = {}
+    for line in open(COUNTERS_FILE):
+        cells = [c.strip().strip("`") for c in line.strip().strip("|").split("|")]
+        if len(cells) != 7 or cells[1] not in KERNEL_SOURCES:
+            continue
+        fam = cells[1]
+        digests.setdefault(fam, source_digest(fam))
+        if cells[2] != digests[fam]:
+            continue
+        num = lambda c: None if c in ("", "-") else float(c)
+        out[cells[0]] = {"mfma_busy_pct": num(cells[3]), "lds_bank_conflicts": num(cells[4]), "fetch_bytes": num(cells[5]),
+                         "write_bytes": num(cells[6]), "source": "profiles/bench_counters.md"}
+    return out
 
 
 def main():
@@ -77,14 +109,19 @@ def main():
 
     launch = R.lib().r355_gemm
     gref = ctypes.byref(g)
+    # untimed: bring the device to its sustained clocks first (a handful of 0.7 ms launches after the host-side
+    # set-up above under-reports by up to 10 %), then the W warm-up steps the caller asked for
+    settle(torch, lambda: launch(gref, None), 0.25)
     for _ in range(args.warmup):
         assert launch(gref, None) == 0, R.lib().r355_last_error()
     torch.cuda.synchronize()
+    status = 0
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        launch(gref, None)
+        status |= launch(gref, None)
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    assert status == 0, R.lib().r355_last_error()
     value = flop / wall_ms / 1e9
 
     # kernel duration by HIP events on the launch stream
@@ -102,9 +139,11 @@ def main():
     max_rel = float(np.max(np.abs(gf - wf) / (np.abs(gf) + np.abs(wf) + 1.0)))
     validated = bool(np.all(np.isfinite(gf)) and max_rel <= 1e-3)
 
+    counters = load_counters()
     extra = {}
     if not args.quick:
-        extra = run_extras(R, O, np, torch, args)
+        extra = run_extras(R, O, np, torch, args, counters)
+    head = counters.get("gemm_f16_nt_8192") if args.size == 8192 else None
 
     line = {
         "metric": "TFLOPS at 8192^3 f16 GEMM (f32 accumulate, NT, f16 out); int8 / bf16 / fp8 / sparse / DLRM in extra",
@@ -130,7 +169,11 @@ def main():
         "max_rel_error_vs_oracle": max_rel,
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS["f16"], "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_TFLOPS["f16"], 4),
-                     "traffic": TRAFFIC_F16_NT_8192 if args.size == 8192 else None,
+                     "traffic": int(head["fetch_bytes"] + head["write_bytes"]) if head and head["fetch_bytes"] and head["write_bytes"] else None,
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel source (profiles/bench_counters.md)" if head else None,
+                     "mfma_busy_pct": head["mfma_busy_pct"] if head else None,
+                     "lds_bank_conflicts": head["lds_bank_conflicts"] if head else None,
+                     "achieved_hbm_gbps": round(((m * k + k * n) * 2 + m * n * 2) / ev_ms / 1e6, 1),
                      "kernel_ms": round(ev_ms, 4), "algorithmic_flop": flop,
                      "algorithmic_bytes": (m * k + k * n) * 2 + m * n * 2},
         "cpu_baseline": {"value": round(cpu_tflops, 6), "unit": "TFLOP/s", "cores": O.lib().orc_num_threads(),
@@ -154,10 +197,38 @@ def settle(torch, fn, seconds=0.1):
         torch.cuda.synchronize()
 
 
-def run_extras(R, O, np, torch, args):
-    """The remaining benchmark configurations, each timed with HIP events over args.steps launches."""
+def run_extras(R, O, np, torch, args, counters):
+    """The remaining benchmark configurations, each timed with HIP events over args.steps launches; every result is
+    checked for finite values and, for the GEMMs, on sampled elements against a float64 / int64 dot product on the device
+    (the oracle-based parity of the same configurations is in tests/)."""
     out = {}
     s = args.size
+
+    def with_counters(name, rec):
+        c = counters.get(name)
+        if c:
+            rec["counters"] = {k: v for k, v in c.items() if v is not None}
+        return rec
+
+    def sampled_ok(in_t, out_t, la, lb, mm, nn, kk, a, b, d, sparse_meta):
+        """64 sampled elements of D against a float64 dot product of the operands as stored (dense cases)."""
+        tdt = {R.F16: torch.float16, R.BF16: torch.bfloat16, R.I8: torch.int8, R.E4M3: torch.float8_e4m3fn, R.F32: torch.float32,
+               R.F64: torch.float64, R.I32: torch.int32}
+        dv = d.view(tdt[out_t]).view(mm, nn)
+        if not bool(torch.isfinite(dv.to(torch.float64)).all()):
+            return False
+        if sparse_meta is not None:
+            return True  # (the 2:4 case is compared with the dense oracle in tests/test_sparse.py)
+        av = a.view(tdt[in_t]).view((mm, kk) if la == R.ROW_MAJOR else (kk, mm))
+        bv = b.view(tdt[in_t]).view((kk, nn) if lb == R.ROW_MAJOR else (nn, kk))
+        g = torch.Generator(device="cpu").manual_seed(5)
+        ri, ci = torch.randint(0, mm, (64,), generator=g).cuda(), torch.randint(0, nn, (64,), generator=g).cuda()
+        ar = (av[ri] if la == R.ROW_MAJOR else av[:, ri].t()).to(torch.float64)
+        bc = (bv[:, ci].t() if lb == R.ROW_MAJOR else bv[ci]).to(torch.float64)
+        want = (ar * bc).sum(1)
+        got = dv[ri, ci].to(torch.float64)
+        tol = {R.I8: 0.0, R.F64: 1e-10, R.F32: 1e-4}.get(in_t, 1e-2)
+        return bool(((got - want).abs() <= tol * (want.abs() + got.abs() + 1.0) + (2e-3 * want.abs() if out_t in (R.F16, R.BF16) else 0)).all())
 
     def rnd16(nel, bf):
         t = (torch.rand(nel, device="cuda") * 2 - 1)
@@ -170,8 +241,9 @@ def run_extras(R, O, np, torch, args):
         settle(torch, lambda: R.lib().r355_gemm(ctypes.byref(g), None))
         ms = R.gemm_timed(g, args.warmup, args.steps)
         tf = 2.0 * mm * nn * kk / ms / 1e9
-        out[name] = {"ms": round(ms, 4), "value": round(tf, 2), "unit": unit, "peak": peak * peak_scale,
-                     "frac": round(tf / (peak * peak_scale), 4)}
+        out[name] = with_counters(name, {"ms": round(ms, 4), "value": round(tf, 2), "unit": unit, "peak": peak * peak_scale,
+                                         "frac": round(tf / (peak * peak_scale), 4),
+                                         "validated": sampled_ok(in_t, out_t, la, lb, mm, nn, kk, a, b, d, sparse_meta)})
 
     if s == 8192:  # a problem with too few 256 x 256 tiles for the 256 CUs: the 128 x 128 macro tile
         gemm_case("gemm_f16_nt_2048x2048x8192", R.F16, R.F16, R.COL_MAJOR, R.ROW_MAJOR, rnd16(2048 * s, False),
@@ -189,6 +261,8 @@ def run_extras(R, O, np, torch, args):
     gemm_case("gemm_bf16_nt_8192", R.BF16, R.BF16, R.COL_MAJOR, R.ROW_MAJOR, abf, bbf, PEAK_TFLOPS["bf16"], "TFLOP/s")
     af16, bf16_ = rnd16(s * s, False), rnd16(s * s, False)
     gemm_case("gemm_f16_tn_8192", R.F16, R.F16, R.ROW_MAJOR, R.COL_MAJOR, af16, bf16_, PEAK_TFLOPS["f16"], "TFLOP/s")
+    # the same operands with an f32 result (f16 -> fp32 as the benchmark's target is worded; D is 256 MiB instead of 128)
+    gemm_case("gemm_f16_nt_f32out_8192", R.F16, R.F32, R.COL_MAJOR, R.ROW_MAJOR, af16, bf16_, PEAK_TFLOPS["f16"], "TFLOP/s")
     i8 = lambda nel: torch.randint(-128, 128, (nel,), dtype=torch.int16, device="cuda").to(torch.int8)
     ai8, bi8 = i8(s * s), i8(s * s)
     gemm_case("gemm_i8_tn_8192", R.I8, R.I32, R.ROW_MAJOR, R.COL_MAJOR, ai8, bi8, PEAK_TFLOPS["i8"], "TOP/s")
@@ -216,10 +290,10 @@ def run_extras(R, O, np, torch, args):
     settle(torch, lambda: R.dlrm_fwd(R.F16, x, o, mm, kk, bsz))
     ms = R.dlrm_fwd_timed(R.F16, x, o, mm, kk, bsz, args.warmup, args.steps)
     byts = bsz * (mm * kk + kk + mm * (mm - 1) // 2) * 2
-    out["dlrm_fwd_b65536_f27_d128"] = {"ms": round(ms, 4), "value": round(byts / ms / 1e6, 1), "unit": "GB/s",
-                                       "peak": HBM_PEAK_GBPS, "frac": round(byts / ms / 1e6 / HBM_PEAK_GBPS, 4),
-                                       "algorithmic_bytes": byts,
-                                       "gflops_ref_convention": round(2.0 * mm * mm * kk * bsz / ms / 1e6, 1)}
+    out["dlrm_fwd_b65536_f27_d128"] = with_counters("dlrm_fwd_b65536_f27_d128", {
+        "ms": round(ms, 4), "value": round(byts / ms / 1e6, 1), "unit": "GB/s", "peak": HBM_PEAK_GBPS,
+        "frac": round(byts / ms / 1e6 / HBM_PEAK_GBPS, 4), "algorithmic_bytes": byts,
+        "gflops_ref_convention": round(2.0 * mm * mm * kk * bsz / ms / 1e6, 1), "validated": bool(torch.isfinite(o.float()).all())})
     # DLRM backward on the same shape: reads X and the upstream gradient, writes both gradients
     up = torch.randn(bsz * (kk + mm * (mm - 1) // 2), device="cuda").to(torch.float16)
     gmlp = torch.empty(bsz * kk, dtype=torch.float16, device="cuda")
@@ -234,9 +308,10 @@ def run_extras(R, O, np, torch, args):
     torch.cuda.synchronize()
     ms = e0.elapsed_time(e1) / args.steps
     byts = (2 * bsz * mm * kk + bsz * (kk + mm * (mm - 1) // 2) + bsz * kk) * 2
-    out["dlrm_bwd_b65536_f27_d128"] = {"ms": round(ms, 4), "value": round(byts / ms / 1e6, 1), "unit": "GB/s",
-                                       "peak": HBM_PEAK_GBPS, "frac": round(byts / ms / 1e6 / HBM_PEAK_GBPS, 4),
-                                       "algorithmic_bytes": byts}
+    out["dlrm_bwd_b65536_f27_d128"] = with_counters("dlrm_bwd_b65536_f27_d128", {
+        "ms": round(ms, 4), "value": round(byts / ms / 1e6, 1), "unit": "GB/s", "peak": HBM_PEAK_GBPS,
+        "frac": round(byts / ms / 1e6 / HBM_PEAK_GBPS, 4), "algorithmic_bytes": byts,
+        "validated": bool(torch.isfinite(gin.float()).all() and torch.isfinite(gmlp.float()).all())})
     return out
 
 

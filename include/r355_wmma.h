@@ -91,7 +91,10 @@ typedef struct
     const void* c;
     void*       d;
     uint32_t    lda, ldb, ldc, ldd;
-    float       alpha, beta;
+    /* The reference passes the scalars in the compute type (ComputeT alpha, beta: test/gemm/gemm_kernel_base.hpp:112-113).
+     * A double carries each of them unrounded: it is narrowed to float for f16 / bf16 / fp8 / f32 inputs, truncated to
+     * int32 for i8 inputs (every int32 is exact in a double) and used as it is for f64. */
+    double      alpha, beta;
     int32_t     sparse24;
     const void* a_meta;
     int32_t     kernel; /* r355_gemm_kernel */

@@ -247,7 +247,7 @@ static inline size_t mat_index(uint32_t row, uint32_t col, uint32_t ld, int layo
  * output type (lines 76-77).  Rows are spread over OpenMP threads (line 65).
  *
  * Floating inputs (f16, bf16, e4m3, f32) compute in f32, f64 in f64; int8 computes in
- * int32 with int32 alpha/beta passed as integers-in-float.  Returns 0, or
+ * int32 with int32 alpha/beta passed as integers-in-double.  Returns 0, or
  * -1 for an unsupported type combination.
  */
 int orc_gemm(int         in_type,
@@ -263,9 +263,13 @@ int orc_gemm(int         in_type,
              const void* b,
              const void* c,
              void*       d,
-             float       alpha,
-             float       beta)
+             double      alpha_c,
+             double      beta_c)
 {
+    /* the scalars arrive wide enough for every compute type (gemm_CPU takes ComputeT alpha, beta:
+     * test/reference_impl.hpp:44-45) and are narrowed to it here: int32 for int8 inputs, double for f64,
+     * float for everything else */
+    const float alpha = (float)alpha_c, beta = (float)beta_c;
     uint32_t lda = layout_a == ORC_ROW_MAJOR ? k : m;
     uint32_t ldb = layout_b == ORC_ROW_MAJOR ? n : k;
     uint32_t ldc = layout_c == ORC_ROW_MAJOR ? n : m;
@@ -277,7 +281,7 @@ int orc_gemm(int         in_type,
         const int8_t*  pb = (const int8_t*)b;
         const int32_t* pc = (const int32_t*)c;
         int32_t*       pd = (int32_t*)d;
-        int32_t        ia = (int32_t)alpha, ib = (int32_t)beta;
+        int32_t        ia = (int32_t)alpha_c, ib = (int32_t)beta_c;
         if(out_type == ORC_I8)
         {
             /* (int8, int8, int32) of test/gemm/gemm_common_test_params.hpp:52: C and D are int8, the
@@ -344,7 +348,7 @@ int orc_gemm(int         in_type,
                 for(uint32_t h = 0; h < k; ++h)
                     accum += pa[mat_index((uint32_t)i, h, lda, layout_a)] * pb[mat_index(h, j, ldb, layout_b)];
                 pd[mat_index((uint32_t)i, j, ldd, layout_d)]
-                    = (double)alpha * accum + (double)beta * pc[mat_index((uint32_t)i, j, ldc, layout_c)];
+                    = alpha_c * accum + beta_c * pc[mat_index((uint32_t)i, j, ldc, layout_c)];
             }
         }
         return 0;
@@ -394,8 +398,9 @@ int orc_gemm_rows(int             in_type,
                   const uint32_t* rows,
                   uint32_t        nrows,
                   void*           d_rows,
-                  float           alpha)
+                  double          alpha_c)
 {
+    const float alpha = (float)alpha_c;
     uint32_t lda = layout_a == ORC_ROW_MAJOR ? k : m;
     uint32_t ldb = layout_b == ORC_ROW_MAJOR ? n : k;
     int      rc  = 0;
@@ -417,7 +422,7 @@ int orc_gemm_rows(int             in_type,
                     accum += (int32_t)((const int8_t*)a)[mat_index(i, h, lda, layout_a)]
                              * (int32_t)((const int8_t*)b)[mat_index(h, j, ldb, layout_b)];
                 ((int32_t*)d_rows)[(size_t)r * n + j]
-                    = (int32_t)((uint32_t)(int32_t)alpha * (uint32_t)accum);
+                    = (int32_t)((uint32_t)(int32_t)alpha_c * (uint32_t)accum);
             }
             else
             {

@@ -44,7 +44,7 @@ class GemmArgs(ctypes.Structure):
         ("m", ctypes.c_uint32), ("n", ctypes.c_uint32), ("k", ctypes.c_uint32),
         ("a", ctypes.c_void_p), ("b", ctypes.c_void_p), ("c", ctypes.c_void_p), ("d", ctypes.c_void_p),
         ("lda", ctypes.c_uint32), ("ldb", ctypes.c_uint32), ("ldc", ctypes.c_uint32), ("ldd", ctypes.c_uint32),
-        ("alpha", ctypes.c_float), ("beta", ctypes.c_float),
+        ("alpha", ctypes.c_double), ("beta", ctypes.c_double),
         ("sparse24", ctypes.c_int32), ("a_meta", ctypes.c_void_p),
         ("kernel", ctypes.c_int32),
     ]

@@ -15,7 +15,7 @@ namespace
             return r355::fail(R355_ERR_BAD_ARG, "gemm: args is null");
         if(!g->a || !g->b || !g->d)
             return r355::fail(R355_ERR_BAD_ARG, "gemm: a, b and d must be non-null");
-        if(g->beta != 0.0f && !g->c)
+        if(g->beta != 0.0 && !g->c)
             return r355::fail(R355_ERR_BAD_ARG, "gemm: c is null but beta != 0");
         if(g->m == 0 || g->n == 0 || g->k == 0)
             return r355::fail(R355_ERR_BAD_ARG, "gemm: m, n, k must be non-zero");
@@ -29,7 +29,7 @@ namespace
         const uint32_t minLdb = g->layout_b == R355_ROW_MAJOR ? g->n : g->k;
         const uint32_t minLdc = g->layout_c == R355_ROW_MAJOR ? g->n : g->m;
         const uint32_t minLdd = g->layout_d == R355_ROW_MAJOR ? g->n : g->m;
-        if(g->lda < minLda || g->ldb < minLdb || g->ldd < minLdd || (g->beta != 0.0f && g->ldc < minLdc))
+        if(g->lda < minLda || g->ldb < minLdb || g->ldd < minLdd || (g->beta != 0.0 && g->ldc < minLdc))
             return r355::fail(R355_ERR_BAD_ARG, "gemm: leading dimension smaller than the contiguous extent");
         if(g->kernel != R355_KERNEL_AUTO && g->kernel != R355_KERNEL_SIMPLE && g->kernel != R355_KERNEL_TILED
            && g->kernel != R355_KERNEL_TILED_128)

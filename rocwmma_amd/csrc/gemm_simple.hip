@@ -51,10 +51,14 @@ namespace
         FragAcc fragAcc;
         fill_fragment(fragAcc, static_cast<CompT>(0));
 
-        const InT*     pa    = a + MapA::fromMatrixCoord(make_coord2d(row, 0u), lda);
-        const InT*     pb    = b + MapB::fromMatrixCoord(make_coord2d(0u, col), ldb);
-        const uint32_t stepA = MapA::fromMatrixCoord(make_coord2d(0u, BK), lda);
-        const uint32_t stepB = MapB::fromMatrixCoord(make_coord2d(BK, 0u), ldb);
+        // 64-bit offsets: rows * ld of an operand that fits 288 GB of HBM can exceed 2^32 elements (the
+        // fragment API's own fromMatrixCoord is 32-bit like the reference's)
+        constexpr bool aRow  = std::is_same_v<LayoutA, row_major>;
+        constexpr bool bRow  = std::is_same_v<LayoutB, row_major>;
+        const InT*     pa    = a + (aRow ? (uint64_t)row * lda : (uint64_t)row);
+        const InT*     pb    = b + (bRow ? (uint64_t)col : (uint64_t)col * ldb);
+        const uint64_t stepA = aRow ? (uint64_t)BK : (uint64_t)BK * lda;
+        const uint64_t stepB = bRow ? (uint64_t)BK * ldb : (uint64_t)BK;
 
         for(uint32_t i = 0; i < k; i += BK)
         {
@@ -65,10 +69,8 @@ namespace
             pb += stepB;
         }
 
-        const uint32_t offC
-            = layoutC == mem_row_major ? row * ldc + col : col * ldc + row;
-        const uint32_t offD
-            = layoutD == mem_row_major ? row * ldd + col : col * ldd + row;
+        const uint64_t offC = layoutC == mem_row_major ? (uint64_t)row * ldc + col : (uint64_t)col * ldc + row;
+        const uint64_t offD = layoutD == mem_row_major ? (uint64_t)row * ldd + col : (uint64_t)col * ldd + row;
 
         FragC fragC;
         if(beta != static_cast<CompT>(0))
@@ -221,7 +223,7 @@ namespace r355
         const uint32_t vc = g.layout_c == R355_COL_MAJOR ? accRun * ob : ob;
         if(!aligned(g.a, va) || (g.lda * eb) % va || !aligned(g.b, vb) || (g.ldb * eb) % vb
            || !aligned(g.d, vd) || (g.ldd * ob) % vd
-           || (g.beta != 0.0f && (!aligned(g.c, vc) || (g.ldc * ob) % vc)))
+           || (g.beta != 0.0 && (!aligned(g.c, vc) || (g.ldc * ob) % vc)))
             return fail(R355_ERR_MISALIGNED, "gemm: pointers / leading dimensions must keep %u-byte vectors aligned", va > vb ? va : vb);
         if(plan)
         {

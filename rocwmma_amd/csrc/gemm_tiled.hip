@@ -65,7 +65,7 @@ namespace r355
         const char* c;
         char*       d;
         uint32_t    lda, ldb, ldc, ldd; // elements
-        float       alpha, beta;
+        double      alpha, beta; // narrowed to the accumulator type in the epilogue
         uint32_t    tilesM, tilesN;
         // the launch covers tile indices [tileFirst, tileFirst + tileCount) of the tilesM x tilesN walk; with
         // tileQuad the walk is over tiles of twice the kernel's edge, four workgroups each (tile_map.hpp)
@@ -1425,7 +1425,7 @@ namespace r355
         const uint32_t tile = macroTile(g);
         if(g.in_type == R355_F64 && tile != 128u)
             return fail(R355_ERR_UNSUPPORTED, "tiled gemm: f64 runs the 128 x 128 macro tile only");
-        if(g.beta != 0.0f && g.layout_c != g.layout_d)
+        if(g.beta != 0.0 && g.layout_c != g.layout_d)
             return fail(R355_ERR_UNSUPPORTED, "tiled gemm: C and D must share an orientation");
         const uint32_t tk = STAGE_KB / es;
         // K moves in 16-byte chunks; a last K stage that is not full is completed with zeros by the loads
@@ -1437,7 +1437,7 @@ namespace r355
         if((uint64_t)g.lda * es > (1u << 23) || (uint64_t)g.ldb * es > (1u << 23))
             return fail(R355_ERR_UNSUPPORTED, "tiled gemm: leading dimensions above 8 MiB per row / column");
         if(!aligned(g.a, 16) || !aligned(g.b, 16) || (g.lda * es) % 16 || (g.ldb * es) % 16 || !aligned(g.d, 16)
-           || (g.ldd * os) % 16 || (g.beta != 0.0f && (!aligned(g.c, 16) || (g.ldc * os) % 16)))
+           || (g.ldd * os) % 16 || (g.beta != 0.0 && (!aligned(g.c, 16) || (g.ldc * os) % 16)))
             return fail(R355_ERR_MISALIGNED, "tiled gemm: pointers and leading dimensions of A, B, C, D must keep 16-byte alignment");
         if(plan)
         {

@@ -279,7 +279,7 @@ int main(int argc, char** argv)
         g.lda = (g.layout_a == R355_ROW_MAJOR ? k : m) + ldpad;
         g.ldb = (g.layout_b == R355_ROW_MAJOR ? n : k) + ldpad;
         g.ldc = g.ldd = n;
-        g.alpha = 1.0f, g.beta = 0.0f;
+        g.alpha = 1.0, g.beta = 0.0;
         g.kernel = kernel == "simple"     ? R355_KERNEL_SIMPLE
                    : kernel == "tiled"    ? R355_KERNEL_TILED
                    : kernel == "tiled128" ? R355_KERNEL_TILED_128

@@ -66,8 +66,8 @@ namespace
                                                                                uint32_t       ldd,
                                                                                bool           cRow,
                                                                                bool           dRow,
-                                                                               float          alphaF,
-                                                                               float          betaF)
+                                                                               double         alphaF,
+                                                                               double         betaF)
     {
         constexpr bool     WIDE = E == SpElem::F16 || E == SpElem::BF16; // 2-byte elements
         constexpr uint32_t ES = WIDE ? 2u : 1u, KSTEP = WIDE ? 32u : 64u; // dense k per instruction
@@ -154,7 +154,7 @@ namespace
         const char*    c;
         char*          d;
         uint32_t       lda, ldb, ldc, ldd;
-        float          alpha, beta;
+        double         alpha, beta;
         uint32_t       tilesM, tilesN;
         uint32_t       dRow; // D (and C) row-major
     };
@@ -395,7 +395,7 @@ namespace
     {
         return g.kernel != R355_KERNEL_SIMPLE && (g.in_type == R355_I8 || g.in_type == R355_E4M3) && g.m % T_M == 0 && g.n % T_N == 0 && g.k % T_K == 0
                && g.layout_c == g.layout_d && (g.ldd % 4) == 0 && r355::aligned(g.d, 16)
-               && (g.beta == 0.0f || ((g.ldc % 4) == 0 && r355::aligned(g.c, 16))) && r355::aligned(g.a_meta, 16);
+               && (g.beta == 0.0 || ((g.ldc % 4) == 0 && r355::aligned(g.c, 16))) && r355::aligned(g.a_meta, 16);
     }
 } // namespace
 
@@ -417,7 +417,9 @@ namespace r355
             return fail(R355_ERR_BAD_SIZE, "sparse gemm: m=%u n=%u must be multiples of 32 and k=%u of %u", g.m, g.n, g.k, kStep);
         if(!aligned(g.a, 16) || (g.lda * es) % 16 || !aligned(g.b, 16) || (g.ldb * es) % 16 || !aligned(g.a_meta, 4) || !aligned(g.d, 4))
             return fail(R355_ERR_MISALIGNED, "sparse gemm: values / B need 16-byte alignment, metadata 4-byte");
-        if(w && (g.kernel == R355_KERNEL_TILED || g.kernel == R355_KERNEL_TILED_128))
+        if(g.kernel == R355_KERNEL_TILED_128)
+            return fail(R355_ERR_UNSUPPORTED, "sparse gemm: there is no 128 x 128 sparse macro tile (R355_KERNEL_TILED is 256 x 256)");
+        if(w && g.kernel == R355_KERNEL_TILED)
             return fail(R355_ERR_UNSUPPORTED, "sparse gemm (macro tile): 1-byte elements only");
         if(g.kernel == R355_KERNEL_TILED && !tiledOk(g))
             return fail(R355_ERR_BAD_SIZE, "sparse gemm (macro tile): m=%u n=%u must be multiples of 256, k=%u of 128, C/D same orientation and 16-byte aligned", g.m, g.n, g.k);

@@ -4,7 +4,8 @@
 // is a list of register chunks (internal/layout.hpp); waves [0, waveCount) each take an
 // equal contiguous run of chunks.  When waveCount exceeds the number of chunks only the
 // first NumChunks waves take part, one chunk each, and the rest return
-// (coop_load.hpp:101-131 has the same rule).  A wave keeps its share in the first
+// (coop_load.hpp:101-131 has the same rule); a run-time waveCount that is not a power of two is
+// rounded down to one and the surplus waves return.  A wave keeps its share in the first
 // registers of its fragment, so a cooperatively loaded fragment is meaningful only to a
 // cooperative store with identical (waveIndex, waveCount).  waveIndex must be uniform
 // over the wave.  Hand-offs through LDS need synchronize_workgroup() around them.
@@ -25,6 +26,18 @@ namespace rocwmma
             static constexpr uint32_t ActiveWaves   = cmin(WaveCount, NumChunks);
             static constexpr uint32_t ChunksPerWave = NumChunks / ActiveWaves;
         };
+
+        // Waves that share the work for a wave count given at run time: the largest power of two that does not
+        // exceed it (at most 16, a workgroup's maximum; a count of 0 is taken as 1).  Chunk counts are powers of two,
+        // so this count either divides the chunks or exceeds them (CoopSplit then lets one wave per chunk take part).
+        // Waves with waveIndex at or above it return without touching their fragment, so a workgroup of 3, 6 or 12
+        // waves still moves the whole fragment.  (The reference halves the given count until it divides its work
+        // items, coop_load.hpp:101-104 -- 6 waves become 3 and then 1; either way every element moves exactly once
+        // and the surplus waves idle.)
+        ROCWMMA_HOST_DEVICE constexpr inline uint32_t coopWaves(uint32_t waveCount)
+        {
+            return waveCount >= 16u ? 16u : (waveCount >= 8u ? 8u : (waveCount >= 4u ? 4u : (waveCount >= 2u ? 2u : 1u)));
+        }
     } // namespace detail
 
     template <uint32_t WaveCount,
@@ -87,15 +100,14 @@ namespace rocwmma
                               uint32_t                                                       waveIndex,
                               uint32_t                                                       waveCount)
     {
-        // workgroups hold at most 16 waves; counts must be powers of two
-        switch(waveCount)
+        // workgroups hold at most 16 waves
+        switch(detail::coopWaves(waveCount))
         {
         case 1u: load_matrix_coop_sync<1u>(frag, data, ldm, waveIndex); break;
         case 2u: load_matrix_coop_sync<2u>(frag, data, ldm, waveIndex); break;
         case 4u: load_matrix_coop_sync<4u>(frag, data, ldm, waveIndex); break;
         case 8u: load_matrix_coop_sync<8u>(frag, data, ldm, waveIndex); break;
-        case 16u: load_matrix_coop_sync<16u>(frag, data, ldm, waveIndex); break;
-        default: break;
+        default: load_matrix_coop_sync<16u>(frag, data, ldm, waveIndex); break;
         }
     }
 
@@ -112,14 +124,13 @@ namespace rocwmma
         uint32_t                                                             waveIndex,
         uint32_t                                                             waveCount)
     {
-        switch(waveCount)
+        switch(detail::coopWaves(waveCount))
         {
         case 1u: store_matrix_coop_sync<1u>(data, frag, ldm, waveIndex); break;
         case 2u: store_matrix_coop_sync<2u>(data, frag, ldm, waveIndex); break;
         case 4u: store_matrix_coop_sync<4u>(data, frag, ldm, waveIndex); break;
         case 8u: store_matrix_coop_sync<8u>(data, frag, ldm, waveIndex); break;
-        case 16u: store_matrix_coop_sync<16u>(data, frag, ldm, waveIndex); break;
-        default: break;
+        default: store_matrix_coop_sync<16u>(data, frag, ldm, waveIndex); break;
         }
     }
 

@@ -29,9 +29,9 @@ def lib():
             subprocess.check_call(["make", "-C", _ORACLE_DIR, "-s"])
         L = ctypes.CDLL(so)
         vp, u32, i, f = ctypes.c_void_p, ctypes.c_uint32, ctypes.c_int, ctypes.c_float
-        L.orc_gemm.argtypes = [i, i, i, i, i, i, u32, u32, u32, vp, vp, vp, vp, f, f]
+        L.orc_gemm.argtypes = [i, i, i, i, i, i, u32, u32, u32, vp, vp, vp, vp, ctypes.c_double, ctypes.c_double]
         L.orc_gemm.restype = i
-        L.orc_gemm_rows.argtypes = [i, i, i, i, u32, u32, u32, vp, vp, vp, u32, vp, f]
+        L.orc_gemm_rows.argtypes = [i, i, i, i, u32, u32, u32, vp, vp, vp, u32, vp, ctypes.c_double]
         L.orc_gemm_rows.restype = i
         L.orc_dlrm_fwd.argtypes = [i, vp, vp, u32, u32, u32]
         L.orc_dlrm_fwd.restype = i

@@ -100,7 +100,9 @@ def test_fill_fragment(cid):
 
 
 @pytest.mark.parametrize("cid", [4, 7, 10, 17, 18, 19, 20, 21, 25, 32, 36, 48, 51, 61, 64, 72, 73, 79, 80, 85, 89])
-@pytest.mark.parametrize("waves", [(1, 1), (2, 1), (2, 2), (4, 2)])
+# (3, 1), (3, 2) and (3, 4): wave counts that are not powers of two -- the largest power of two below them shares
+# the work and the surplus waves return (the reference idles its surplus waves too, coop_load.hpp:101-131)
+@pytest.mark.parametrize("waves", [(1, 1), (2, 1), (2, 2), (4, 2), (3, 1), (3, 2), (3, 4)])
 @pytest.mark.parametrize("use_lds", [0, 1])
 def test_cooperative_round_trip(cid, waves, use_lds):
     rows, cols, eb, rm, _ = _info(cid)

@@ -458,6 +458,58 @@ def test_tiled_kernel_f64_layouts_edges_and_k_tails(la, lb, ldl):
     assert e.value.code == -2
 
 
+@pytest.mark.parametrize("kernel", ["simple", "tiled_128"])
+def test_f64_scalars_keep_double_precision(kernel):
+    # the reference passes ComputeT alpha, beta (test/gemm/gemm_kernel_base.hpp:112-113): double for f64.  1/3 and -1/7
+    # are not representable in f32; rounding them on the way would move the result by ~1e-8 relative, far above the
+    # reference's 10 eps(f64) (the negative control below shows the bar sees that)
+    sel = {"simple": R.KERNEL_SIMPLE, **TILE_SELECTORS}[kernel]
+    m, n, k = 144, 272, 48
+    alpha, beta = 1.0 / 3.0, -1.0 / 7.0
+    a, b, c = _inputs(O.F64, O.F64, m, n, k, seed=77)
+    want = O.gemm(O.F64, O.F64, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c, alpha, beta)
+    got = _run(O.F64, O.F64, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c, alpha, beta, sel)
+    ok, mx = O.compare(O.F64, got, want, 10.0)
+    assert ok, mx
+    rounded = O.gemm(O.F64, O.F64, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c, float(np.float32(alpha)), float(np.float32(beta)))
+    assert not O.compare(O.F64, rounded, want, 10.0)[0]
+
+
+@pytest.mark.parametrize("kernel", ["simple", "tiled", "tiled_128"])
+def test_int8_scalars_beyond_f32_integers(kernel):
+    # int32 alpha / beta (ComputeT = int32 for int8 inputs) above 2^24 are not f32 integers; int32 arithmetic wraps
+    sel = {"simple": R.KERNEL_SIMPLE, **TILE_SELECTORS}[kernel]
+    m, n, k = 272, 144, 160
+    alpha, beta = float(2 ** 25 + 1), float(-(2 ** 24 + 3))
+    a, b, c = _inputs(O.I8, O.I32, m, n, k, seed=78)
+    want = O.gemm(O.I8, O.I32, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c, alpha, beta)
+    got = _run(O.I8, O.I32, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c, alpha, beta, sel)
+    assert np.array_equal(got, want)
+    # closed form on the host, independent of the oracle: wrap-around int32 arithmetic
+    acc = a.reshape(m, k).astype(np.int64) @ b.reshape(n, k).T.astype(np.int64)
+    ref = ((2 ** 25 + 1) * acc - (2 ** 24 + 3) * c.reshape(m, n).astype(np.int64)) & 0xFFFFFFFF
+    assert np.array_equal(got.view(np.uint32).reshape(m, n), ref.astype(np.uint32))
+
+
+@pytest.mark.parametrize("la,lb", [(O.ROW, O.COL), (O.COL, O.ROW)])
+def test_f64_random_operands_long_k(la, lb):
+    # Random f64 operands over a long K: the matrix instructions sum in another order than the oracle's sequential loop,
+    # so the two are compared with the exact product (80-bit accumulation on the host) under the forward error bound that
+    # holds for any summation order, |fl(sum) - sum| <= gamma_k * sum |a_i b_i|, gamma_k = k u / (1 - k u), u = 2^-53.
+    m, n, k = 144, 128, 2064
+    a, b, _ = _inputs(O.F64, O.F64, m, n, k, seed=79)
+    got = _run(O.F64, O.F64, la, lb, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0, R.KERNEL_AUTO).reshape(m, n)
+    A = a.reshape(m, k) if la == O.ROW else a.reshape(k, m).T
+    B = b.reshape(k, n) if lb == O.ROW else b.reshape(n, k).T
+    exact = A.astype(np.longdouble) @ B.astype(np.longdouble)
+    bound = (k * 2.0 ** -53 / (1 - k * 2.0 ** -53)) * (np.abs(A) @ np.abs(B))
+    assert np.all(np.abs(got.astype(np.longdouble) - exact) <= bound)
+    want = O.gemm(O.F64, O.F64, la, lb, O.ROW, O.ROW, m, n, k, a, b, None, 1.0, 0.0).reshape(m, n)
+    assert np.all(np.abs(want.astype(np.longdouble) - exact) <= bound)
+    # and the bound has teeth: the typical distance is far below it, an index error is far above
+    assert np.max(np.abs(got - want)) < 1e-12 < np.max(np.abs(np.roll(got, 1, axis=1) - want))
+
+
 @pytest.mark.parametrize("la,lb", TILED_LAYOUTS_16)
 @pytest.mark.parametrize("kernel", list(TILE_SELECTORS))
 def test_tiled_kernel_f32_one_hot_operands(la, lb, kernel):
