@@ -74,10 +74,11 @@ typedef enum
  * reference's static_cast narrows it), f32 -> f32 (f32), f64 -> f64 (f64).
  * beta == 0 means C is never read and may be NULL.
  *
- * sparse24 != 0: A is 2:4 structured-sparse along k, row-major (i8 -> i32, e4m3 -> f32 with a macro-tile and a
- * block-per-wave kernel; f16 | bf16 -> f32 with the block-per-wave kernel, k % 32 == 0), B col-major:
- * `a` holds the m x k/2 kept values, `a_meta` the m x k/8 index bytes (format of
- * r355_compress_24 / r355_compress_24_16); lda is then the leading dimension of the compressed values.
+ * sparse24 != 0: A is 2:4 structured-sparse along k (i8 -> i32, e4m3 -> f32 with a 256 x 256 macro-tile kernel for
+ * m, n % 256 == 0 and a block-per-wave kernel otherwise; f16 | bf16 -> f32 with the block-per-wave kernel), B col-major:
+ * `a` holds the m * k/2 kept values and `a_meta` the m * k/8 index bytes in the K-blocked storage that
+ * r355_compress_24 / r355_compress_24_16 write (layout_a = R355_ROW_MAJOR, lda = k / 2: the storage has no padding);
+ * m, n multiples of 16, k of 128 bytes' worth of elements (128 for 1-byte, 64 for 2-byte elements).
  * The reference has no sparse path; this form has no counterpart there.
  */
 typedef struct
@@ -159,14 +160,22 @@ int r355_dgemv(int32_t layout_a, uint32_t m, uint32_t k, const double* a, uint32
                const double* y_in, double* y_out, double alpha, double beta, void* stream);
 
 /*
- * Host-side 2:4 compressor for a row-major m x k matrix of 1-byte elements (host pointers).
- * values: m x k/2 kept elements (in position order); meta: m x k/8 bytes, one nibble per
- * group of 4 = idx0 | idx1 << 2 with idx0 < idx1, even group in the low nibble.  k % 8 == 0.
- * r355_decompress_24 is the inverse.  No counterpart in the reference.
+ * Host-side 2:4 compressor for a row-major m x k matrix of 1-byte elements (host pointers); m % 16 == 0, k % 128 == 0.
+ * Every aligned group of 4 along k keeps 2 elements (in position order) and a nibble idx0 | idx1 << 2 (idx0 < idx1).
+ * The storage is K-blocked so that a kernel's share of one K stage is contiguous and in matrix-instruction order.
+ * With a stage = 128 dense k and a lane group = 32 of them (8 groups of 4):
+ *   values [k / 128][m / 16][4 lane groups][16 rows][16 kept bytes]     m * k / 2 bytes
+ *   meta   [k / 128][m / 16][4 lane groups][16 rows][4 index bytes]     m * k / 8 bytes, two nibbles per byte, the even
+ *                                                                       group in the low nibble
+ * (a 32-bit word of `meta` is the index register of v_smfmac_*_16x16x128 for the 16 bytes of `values` beside it).
+ * r355_decompress_24 is the inverse.  R355_ERR_BAD_SIZE for sizes off that grid, R355_ERR_NOT_24_SPARSE if a group holds
+ * more than 2 non-zeros.  No counterpart in the reference.
  */
 int r355_compress_24(const uint8_t* dense, uint32_t m, uint32_t k, uint8_t* values, uint8_t* meta);
 int r355_decompress_24(const uint8_t* values, const uint8_t* meta, uint32_t m, uint32_t k, uint8_t* dense);
-/* The same for 2-byte elements (f16 / bf16 bit patterns; an element is zero when all its bits are). */
+/* The same for 2-byte elements (f16 / bf16 bit patterns; an element is zero when all its bits are): a stage is 64 dense
+ * k (128 bytes), a lane group 16 of them: values [k / 64][m / 16][4][16][8 kept elements], meta [k / 64][m / 16][4][16][2 bytes];
+ * k % 64 == 0. */
 int r355_compress_24_16(const uint16_t* dense, uint32_t m, uint32_t k, uint16_t* values, uint8_t* meta);
 int r355_decompress_24_16(const uint16_t* values, const uint8_t* meta, uint32_t m, uint32_t k, uint16_t* dense);
 

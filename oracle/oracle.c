@@ -658,15 +658,33 @@ int orc_fill_ref(int dtype, void* mat, uint32_t m, uint32_t n, int layout)
 /*
  * Build-defined 2:4 structured-sparse storage for a row-major m x k matrix of
  * 1-byte elements (int8 or e4m3): every aligned group of 4 along k keeps 2
- * values.  values[m][k/2] holds the kept pair of each group in increasing
- * position order; meta[m][k/8] holds, per group, a nibble
- * (idx0 | idx1 << 2) with idx0 < idx1, two groups per byte (low nibble first).
- * A group with fewer than 2 non-zeros keeps the non-zeros plus the lowest
- * unused positions.  Returns -1 if a group has more than 2 non-zeros.
+ * values, in increasing position order, plus a nibble (idx0 | idx1 << 2) with
+ * idx0 < idx1.  A group with fewer than 2 non-zeros keeps the non-zeros plus
+ * the lowest unused positions.
+ *
+ * The storage is K-blocked.  A stage is 128 dense k; within a stage a row's 32
+ * groups belong to 4 lane groups of 8.  Kept values:
+ *   values[stage][row / 16][lane group][row % 16][16]   (16 = 8 groups x 2 kept bytes)
+ * and, with the same first four indices, 4 metadata bytes (two nibbles per byte,
+ * the even group in the low nibble):
+ *   meta[stage][row / 16][lane group][row % 16][4]
+ * m must be a multiple of 16 and k of 128.  Returns -1 for other sizes or if a
+ * group has more than 2 non-zeros.
  */
+static size_t orc24_value_at(uint32_t r, uint32_t g, uint32_t m)
+{
+    /* g: group of four along k */
+    return ((((size_t)(g / 32u) * (m / 16u) + r / 16u) * 4u + (g % 32u) / 8u) * 16u + r % 16u) * 16u + 2u * (g % 8u);
+}
+
+static size_t orc24_meta_at(uint32_t r, uint32_t g, uint32_t m)
+{
+    return ((((size_t)(g / 32u) * (m / 16u) + r / 16u) * 4u + (g % 32u) / 8u) * 16u + r % 16u) * 4u + (g % 8u) / 2u;
+}
+
 int orc_compress24(const uint8_t* dense, uint32_t m, uint32_t k, uint8_t* values, uint8_t* meta)
 {
-    if(k % 8u)
+    if(k % 128u || m % 16u)
         return -1;
     for(uint32_t r = 0; r < m; ++r)
     {
@@ -693,10 +711,10 @@ int orc_compress24(const uint8_t* dense, uint32_t m, uint32_t k, uint8_t* values
                 pos[0] = pos[1];
                 pos[1] = t;
             }
-            values[(size_t)r * (k / 2u) + 2u * g]      = p[pos[0]];
-            values[(size_t)r * (k / 2u) + 2u * g + 1u] = p[pos[1]];
-            uint8_t  nib                                = (uint8_t)(pos[0] | (pos[1] << 2));
-            uint8_t* mb                                 = meta + (size_t)r * (k / 8u) + g / 2u;
+            values[orc24_value_at(r, g, m)]      = p[pos[0]];
+            values[orc24_value_at(r, g, m) + 1u] = p[pos[1]];
+            uint8_t  nib                          = (uint8_t)(pos[0] | (pos[1] << 2));
+            uint8_t* mb                           = meta + orc24_meta_at(r, g, m);
             if(g & 1u)
                 *mb = (uint8_t)((*mb & 0x0Fu) | (nib << 4));
             else
@@ -709,18 +727,17 @@ int orc_compress24(const uint8_t* dense, uint32_t m, uint32_t k, uint8_t* values
 int orc_decompress24(
     const uint8_t* values, const uint8_t* meta, uint32_t m, uint32_t k, uint8_t* dense)
 {
-    if(k % 8u)
+    if(k % 128u || m % 16u)
         return -1;
     memset(dense, 0, (size_t)m * k);
     for(uint32_t r = 0; r < m; ++r)
     {
         for(uint32_t g = 0; g < k / 4u; ++g)
         {
-            uint8_t mb  = meta[(size_t)r * (k / 8u) + g / 2u];
+            uint8_t mb  = meta[orc24_meta_at(r, g, m)];
             uint8_t nib = (g & 1u) ? (uint8_t)(mb >> 4) : (uint8_t)(mb & 0xFu);
-            dense[(size_t)r * k + 4u * g + (nib & 3u)] = values[(size_t)r * (k / 2u) + 2u * g];
-            dense[(size_t)r * k + 4u * g + ((nib >> 2) & 3u)]
-                = values[(size_t)r * (k / 2u) + 2u * g + 1u];
+            dense[(size_t)r * k + 4u * g + (nib & 3u)]        = values[orc24_value_at(r, g, m)];
+            dense[(size_t)r * k + 4u * g + ((nib >> 2) & 3u)] = values[orc24_value_at(r, g, m) + 1u];
         }
     }
     return 0;

@@ -210,25 +210,30 @@ def gemv_timed(layout_a, m, k, a, x, y_in, y_out, alpha, beta, warmup, iters, ld
 
 def compress_24(dense):
     """Host-side 2:4 compression of a (m, k) numpy array of 1-byte (uint8 / int8) or 2-byte (uint16: f16 / bf16
-    bit patterns, or float16) elements -> (values, meta)."""
+    bit patterns, or float16) elements -> (values, meta) in the library's K-blocked storage (include/r355_wmma.h):
+    values [stages][m / 16][4][16][16 / es] elements, meta [stages][m / 16][4][16][4 / es] bytes, a stage being
+    128 / es dense elements of k.  m % 16 == 0, k % (128 / es) == 0."""
     import numpy as np
 
     dense = np.ascontiguousarray(dense)
     m, k = dense.shape
-    values = np.zeros((m, k // 2), dtype=dense.dtype)
-    meta = np.zeros((m, k // 8), dtype=np.uint8)
-    fn = {1: lib().r355_compress_24, 2: lib().r355_compress_24_16}[dense.dtype.itemsize]
+    es = dense.dtype.itemsize
+    stages = k * es // 128
+    values = np.zeros(m * k // 2, dtype=dense.dtype)
+    meta = np.zeros(m * k // 8, dtype=np.uint8)
+    fn = {1: lib().r355_compress_24, 2: lib().r355_compress_24_16}[es]
     _check(fn(_ptr(dense), m, k, _ptr(values), _ptr(meta)))
-    return values, meta
+    return values.reshape(stages, m // 16, 4, 16, 16 // es), meta.reshape(stages, m // 16, 4, 16, 4 // es)
 
 
 def decompress_24(values, meta):
     import numpy as np
 
     values, meta = np.ascontiguousarray(values), np.ascontiguousarray(meta)
-    m, k = values.shape[0], values.shape[1] * 2
+    es = values.dtype.itemsize
+    m, k = values.shape[1] * 16, values.shape[0] * 128 // es
     dense = np.zeros((m, k), dtype=values.dtype)
-    fn = {1: lib().r355_decompress_24, 2: lib().r355_decompress_24_16}[values.dtype.itemsize]
+    fn = {1: lib().r355_decompress_24, 2: lib().r355_decompress_24_16}[es]
     _check(fn(_ptr(values), _ptr(meta), m, k, _ptr(dense)))
     return dense
 

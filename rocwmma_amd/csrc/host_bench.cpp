@@ -104,7 +104,7 @@ namespace
     using f16x8  = _Float16 __attribute__((ext_vector_type(8)));
     using bf16x8 = __bf16 __attribute__((ext_vector_type(8)));
 
-    enum MfmaKind { MF_F16, MF_BF16, MF_I8, MF_FP8_K64, MF_SPARSE_I8, MF_F16_16, MF_I8_16, MF_FP8_16, MF_KINDS };
+    enum MfmaKind { MF_F16, MF_BF16, MF_I8, MF_FP8_K64, MF_SPARSE_I8, MF_F16_16, MF_I8_16, MF_FP8_16, MF_SPARSE_I8_16, MF_SPARSE_FP8_16, MF_KINDS };
 
     // 16 MFMAs per loop trip on 4 x 4 operand registers; no memory traffic inside the loop.
     template <int T>
@@ -183,9 +183,13 @@ namespace
                                                                     __builtin_bit_cast(f16x8, b[j]), acc[x], 0, 0, 0);
                 else if constexpr(T == MF_I8_16)
                     iacc[x] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i], b[j], iacc[x], 0, 0, 0);
-                else
+                else if constexpr(T == MF_FP8_16)
                     acc[x] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, acc[x], 0, 0, 0, 0x7F7F7F7F, 0,
                                                                               0x7F7F7F7F);
+                else if constexpr(T == MF_SPARSE_I8_16) // 2:4 sparse A: 16 kept bytes + one index word per lane, 32 dense bytes of B
+                    iacc[x] = __builtin_amdgcn_smfmac_i32_16x16x128_i8(a[i], b8, iacc[x], 0x84848484, 0, 0);
+                else
+                    acc[x] = __builtin_amdgcn_smfmac_f32_16x16x128_fp8_fp8(a[i], b8, acc[x], 0x84848484, 0, 0);
             }
         }
         float s = 0.0f;
@@ -207,7 +211,9 @@ namespace
         case MF_SPARSE_I8: hipLaunchKernelGGL(mfmaLoop<MF_SPARSE_I8>, g, b, 0, 0, in, out, iters); break;
         case MF_F16_16: hipLaunchKernelGGL(mfmaLoop16<MF_F16_16>, g, b, 0, 0, in, out, iters); break;
         case MF_I8_16: hipLaunchKernelGGL(mfmaLoop16<MF_I8_16>, g, b, 0, 0, in, out, iters); break;
-        default: hipLaunchKernelGGL(mfmaLoop16<MF_FP8_16>, g, b, 0, 0, in, out, iters); break;
+        case MF_FP8_16: hipLaunchKernelGGL(mfmaLoop16<MF_FP8_16>, g, b, 0, 0, in, out, iters); break;
+        case MF_SPARSE_I8_16: hipLaunchKernelGGL(mfmaLoop16<MF_SPARSE_I8_16>, g, b, 0, 0, in, out, iters); break;
+        default: hipLaunchKernelGGL(mfmaLoop16<MF_SPARSE_FP8_16>, g, b, 0, 0, in, out, iters); break;
         }
     }
 
@@ -424,12 +430,15 @@ int main(int argc, char** argv)
         HIP_OK(hipEventCreate(&e1));
         static const char*  names[MF_KINDS] = {"f16 32x32x16", "bf16 32x32x16", "i8 32x32x32", "fp8 f8f6f4 32x32x64",
                                                "sparse i8 smfmac 32x32x64 (dense-equivalent ops)", "f16 16x16x32",
-                                               "i8 16x16x64", "fp8 f8f6f4 16x16x128"};
+                                               "i8 16x16x64", "fp8 f8f6f4 16x16x128",
+                                               "sparse i8 smfmac 16x16x128 (dense-equivalent ops)",
+                                               "sparse fp8 smfmac 16x16x128 (dense-equivalent ops)"};
         // flop per loop trip and wave: 16 instructions of the 32 x 32 shapes, 64 of the 16 x 16 shapes
         static const double flopPer[MF_KINDS]
             = {2.0 * 32 * 32 * 16, 2.0 * 32 * 32 * 16, 2.0 * 32 * 32 * 32, 2.0 * 32 * 32 * 64, 2.0 * 32 * 32 * 64,
-               4 * 2.0 * 16 * 16 * 32, 4 * 2.0 * 16 * 16 * 64, 4 * 2.0 * 16 * 16 * 128};
-        static const double vendorPeak[MF_KINDS] = {2500.0, 2500.0, 5000.0, 5000.0, 10000.0, 2500.0, 5000.0, 5000.0};
+               4 * 2.0 * 16 * 16 * 32, 4 * 2.0 * 16 * 16 * 64, 4 * 2.0 * 16 * 16 * 128, 4 * 2.0 * 16 * 16 * 128,
+               4 * 2.0 * 16 * 16 * 128};
+        static const double vendorPeak[MF_KINDS] = {2500.0, 2500.0, 5000.0, 5000.0, 10000.0, 2500.0, 5000.0, 5000.0, 10000.0, 10000.0};
         printf("[");
         for(int random = 0; random < 2; ++random)
             for(int kind = 0; kind < MF_KINDS; ++kind)
@@ -441,7 +450,7 @@ int main(int argc, char** argv)
                     h[i] = kind == MF_F16    ? ((r & 0x8FFF8FFFu) | 0x30003000u)  // |x| in [1/8, 1)
                            : kind == MF_BF16 ? ((r & 0x807F807Fu) | 0x3E003E00u)  // |x| in [1/8, 1/4)
                            : kind == MF_F16_16 ? ((r & 0x8FFF8FFFu) | 0x30003000u)
-                           : (kind == MF_FP8_K64 || kind == MF_FP8_16) ? ((r & 0x87878787u) | 0x30303030u) // |x| in [1/2, 1)
+                           : (kind == MF_FP8_K64 || kind == MF_FP8_16 || kind == MF_SPARSE_FP8_16) ? ((r & 0x87878787u) | 0x30303030u) // |x| in [1/2, 1)
                                                 : r;
                 }
                 HIP_OK(hipMemcpy(in, h.data(), h.size() * 4, hipMemcpyHostToDevice));

@@ -1,30 +1,34 @@
 // 2:4 structured-sparse GEMM on gfx950 sparse matrix cores (v_smfmac_*), plus the host-side
-// compressor.  The reference has no sparse path; the storage format is defined here.
+// compressor.  The reference has no sparse path; the storage format is defined here (and, for device code,
+// in rocwmma/rocwmma_sparse.hpp, which also documents the operand formats of the instructions).
 //
-// A (m x k, row-major; 1-byte elements, or f16 / bf16 for the block-per-wave kernel) keeps 2 of every aligned
-// group of 4 along k:
-//   values  m x k/2   the kept pair of each group, in position order
-//   meta    m x k/8   one nibble per group = idx0 | idx1 << 2 (idx0 < idx1), even group in the
-//                     low nibble -- 32 bits cover 32 dense k, which is exactly the index
-//                     register one lane feeds to v_smfmac_*_32x32x64 for its 16 kept values.
-// B is dense, col-major (k contiguous); D row- or col-major.
+// A (m x k, 1-byte elements, or f16 / bf16 for the block-per-wave kernel) keeps 2 of every aligned group of 4
+// along k and is stored K-blocked: a stage is 128 dense bytes of k, and with ES the element size
+//   values  [stage][row / 16][lane group g = 0..3][row % 16][16 bytes]   kept elements of dense
+//           k in [stage * 128 / ES + g * 32 / ES, ... + 32 / ES) of the row, in position order
+//   meta    the same indexing with 4 / ES bytes: one nibble idx0 | idx1 << 2 (idx0 < idx1) per group of 4,
+//           the lane's first group in the lowest bits = the index register of v_smfmac_*_16x16x(128 / ES)
+// so that all a 256-row macro tile needs of one stage is 16 + 4 KiB of consecutive bytes (whole cache lines;
+// with row-major compressed rows a stage touched 64 + 16 bytes of every row's lines and the direct-to-LDS
+// loads ran at two thirds of the rate), and a fragment's 16 bytes per lane are consecutive across lanes.
+// B is dense, col-major (k contiguous); D row- or col-major.  m % 16 == 0, k % (128 / ES) == 0.
 //
 // Two kernels:
-//   sparseTiledKernel    256 x 256 macro tile, 128 dense K per stage, a ring of three LDS slots filled
+//   sparseTiledKernel    256 x 256 macro tile, one 128-wide K step per stage, a ring of three LDS slots filled
 //                        by direct-to-LDS loads two stages ahead (kept values 16 KiB + indices 4 KiB
-//                        + dense B 32 KiB per stage), 2 x 2 waves with 4 x 4 v_smfmac_*_32x32x64
-//                        accumulators each; the result is transposed through LDS so that D leaves in
-//                        whole rows.
-//   sparseBlockPerWave   one 32 x 32 block of D per wave straight from global memory; fallback
-//                        for shapes that do not fill a macro tile.
-// Per 64-wide K step a lane feeds 16 kept bytes + 4 index bytes of A and 2 x 16 dense bytes of B.  Operand formats of v_smfmac_*_32x32x64 as measured on MI355X: index
-// bits [2 p + 1 : 2 p] give the position within its group of 4 of kept byte p of the lane.
-// 16-bit elements run v_smfmac_f32_32x32x32_{f16,bf16}: 8 kept values + 16 index bits (the half of the index
-// register that ABID names) of A and 2 x 8 dense values of B per lane and 32-wide K step, same pairing of lane
-// groups, same index bits (measured with one-hot A against coded B).
+//                        + dense B 32 KiB per stage), 2 x 2 waves with 8 x 8 accumulators of
+//                        v_smfmac_*_16x16x128 each (under the board's power limit the register-resident loop of
+//                        this shape sustains 7.5 POP/s against 6.5 for 32x32x64); a stage is split into quadrants of
+//                        the wave tile as in the dense fp8 kernel; the result is transposed through LDS so
+//                        that D leaves in whole rows.
+//   sparseBlockPerWave   one 16 x 16 or 32 x 32 block of D per wave through the sparse fragment API
+//                        (rocwmma_sparse.hpp) straight from global memory; fallback for shapes that do not fill a
+//                        macro tile, and the only kernel for f16 / bf16.
 #include <hip/hip_runtime.h>
 
 #include <cstring>
+
+#include <rocwmma/rocwmma_sparse.hpp>
 
 #include "common.hpp"
 #include "lds_dma.hpp"
@@ -32,107 +36,76 @@
 
 namespace
 {
-    using i32x4  = int __attribute__((ext_vector_type(4)));
-    using i32x8  = int __attribute__((ext_vector_type(8)));
-    using i32x16 = int __attribute__((ext_vector_type(16)));
-    using f32x16 = float __attribute__((ext_vector_type(16)));
-    using f16x8   = _Float16 __attribute__((ext_vector_type(8)));
-    using f16x16  = _Float16 __attribute__((ext_vector_type(16)));
-    using bf16x8  = __bf16 __attribute__((ext_vector_type(8)));
-    using bf16x16 = __bf16 __attribute__((ext_vector_type(16)));
+    using namespace rocwmma;
+    using i32x4 = int __attribute__((ext_vector_type(4)));
+    using i32x8 = int __attribute__((ext_vector_type(8)));
+    using f32x4 = float __attribute__((ext_vector_type(4)));
 
     constexpr uint32_t WAVES_X = 2, WAVES_Y = 2;
 
-    enum class SpElem
-    {
-        I8,
-        E4M3,
-        F16,
-        BF16
-    };
-
-    template <SpElem E>
+    // ------------------------------------------------------------------ block per wave, on the fragment API
+    template <typename InT, typename AccE, uint32_t Blk>
     __global__ void __launch_bounds__(WAVES_X* WAVES_Y * 64) sparseBlockPerWave(uint32_t       m,
                                                                                uint32_t       n,
                                                                                uint32_t       k,
-                                                                               const uint8_t* aVals,
+                                                                               const InT*     aVals,
                                                                                const uint8_t* aMeta,
-                                                                               const uint8_t* b,
-                                                                               const void*    c,
-                                                                               void*          d,
-                                                                               uint32_t       lda, // compressed values per row
+                                                                               const InT*     b,
+                                                                               const AccE*    c,
+                                                                               AccE*          d,
                                                                                uint32_t       ldb,
                                                                                uint32_t       ldc,
                                                                                uint32_t       ldd,
-                                                                               bool           cRow,
-                                                                               bool           dRow,
-                                                                               double         alphaF,
-                                                                               double         betaF)
+                                                                               layout_t       layoutC,
+                                                                               layout_t       layoutD,
+                                                                               AccE           alpha,
+                                                                               AccE           beta)
     {
-        constexpr bool     WIDE = E == SpElem::F16 || E == SpElem::BF16; // 2-byte elements
-        constexpr uint32_t ES = WIDE ? 2u : 1u, KSTEP = WIDE ? 32u : 64u; // dense k per instruction
-        using Acc  = std::conditional_t<E == SpElem::I8, i32x16, f32x16>;
-        using AccE = std::conditional_t<E == SpElem::I8, int, float>;
-        const uint32_t lane = threadIdx.x & 63u;
-        const uint32_t row0 = (blockIdx.x * WAVES_X + threadIdx.x / 64u) * 32u;
-        const uint32_t col0 = (blockIdx.y * WAVES_Y + threadIdx.y) * 32u;
-        if(row0 >= m || col0 >= n)
+        using S                 = Sparse24<InT>;
+        constexpr uint32_t BK   = S::StageK; // one stage per trip
+        using FragA             = fragment<sparse_matrix_a, Blk, Blk, BK, InT, row_major>;
+        using FragMeta          = fragment<sparse_metadata, Blk, Blk, BK, InT>;
+        using FragB             = fragment<matrix_b, Blk, Blk, BK, InT, col_major>;
+        using FragAcc           = fragment<accumulator, Blk, Blk, BK, AccE>;
+        const uint32_t row = (blockIdx.x * WAVES_X + threadIdx.x / 64u) * Blk;
+        const uint32_t col = (blockIdx.y * WAVES_Y + threadIdx.y) * Blk;
+        if(row >= m || col >= n)
             return;
-        const uint32_t idx = lane & 31u, g = lane >> 5;
+        const InT*     pa = aVals + S::valueOffset(row, 0u, m);
+        const uint8_t* pm = aMeta + S::metaOffset(row, 0u, m);
+        const InT*     pb = b + (uint64_t)col * ldb;
+        const uint32_t strideV = S::valueStageStride(m), strideM = S::metaStageStride(m);
 
-        // byte pointers; a lane moves 16 bytes of kept values, KSTEP / 16 index bytes and 2 x 16 bytes of B per step
-        const uint8_t* pa = aVals + ((uint64_t)(row0 + idx) * lda) * ES + 16u * g;
-        const uint8_t* pm = aMeta + (uint64_t)(row0 + idx) * (k / 8u) + (KSTEP / 16u) * g;
-        // The instruction pairs A's lane group g, kept bytes [8 q, 8 q + 8) with B's lane group q,
-        // dense bytes [16 g, 16 g + 16).  With A's lane group g holding the kept values of dense
-        // k in [32 g, 32 g + 32), B's lane group h therefore holds dense k in [16 h, 16 h + 16)
-        // and [32 + 16 h, 48 + 16 h) of each 64-wide step (16-bit elements: the same in units of
-        // 2 bytes, a 32-wide step).
-        const uint8_t* pb = b + ((uint64_t)(col0 + idx) * ldb) * ES + 16u * g;
-
-        Acc acc;
-#pragma unroll
-        for(uint32_t e = 0; e < 16; ++e)
-            acc[e] = 0;
-
-        for(uint32_t kd = 0; kd < k; kd += KSTEP)
+        FragA    fragA;
+        FragMeta fragMeta;
+        FragB    fragB;
+        FragAcc  fragAcc;
+        fill_fragment(fragAcc, static_cast<AccE>(0));
+        for(uint32_t kk = 0; kk < k; kk += BK)
         {
-            const i32x4 av = *reinterpret_cast<const i32x4*>(pa + (kd / 2u) * ES);
-            const i32x4 b0 = *reinterpret_cast<const i32x4*>(pb + kd * ES);
-            const i32x4 b1 = *reinterpret_cast<const i32x4*>(pb + kd * ES + 32u);
-            const i32x8 bv = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
-            if constexpr(WIDE)
-            {
-                const int meta = *reinterpret_cast<const uint16_t*>(pm + kd / 8u); // low half, ABID 0
-                if constexpr(E == SpElem::F16)
-                    acc = __builtin_amdgcn_smfmac_f32_32x32x32_f16(__builtin_bit_cast(f16x8, av),
-                                                                   __builtin_bit_cast(f16x16, bv), acc, meta, 0, 0);
-                else
-                    acc = __builtin_amdgcn_smfmac_f32_32x32x32_bf16(__builtin_bit_cast(bf16x8, av),
-                                                                    __builtin_bit_cast(bf16x16, bv), acc, meta, 0, 0);
-            }
-            else
-            {
-                const int meta = *reinterpret_cast<const int*>(pm + kd / 8u);
-                if constexpr(E == SpElem::E4M3)
-                    acc = __builtin_amdgcn_smfmac_f32_32x32x64_fp8_fp8(av, bv, acc, meta, 0, 0);
-                else
-                    acc = __builtin_amdgcn_smfmac_i32_32x32x64_i8(av, bv, acc, meta, 0, 0);
-            }
+            load_matrix_sync(fragA, pa, strideV);
+            load_matrix_sync(fragMeta, pm, strideM);
+            load_matrix_sync(fragB, pb, ldb);
+            mma_sync(fragAcc, fragA, fragMeta, fragB, fragAcc);
+            pa += strideV, pm += strideM, pb += BK;
         }
-
-        // lane holds D(row0 + 8 (e / 4) + 4 g + e % 4, col0 + idx)
-        const AccE alpha = static_cast<AccE>(alphaF), beta = static_cast<AccE>(betaF);
-#pragma unroll
-        for(uint32_t e = 0; e < 16; ++e)
+        const uint64_t offC = layoutC == mem_row_major ? (uint64_t)row * ldc + col : (uint64_t)col * ldc + row;
+        const uint64_t offD = layoutD == mem_row_major ? (uint64_t)row * ldd + col : (uint64_t)col * ldd + row;
+        if(beta != static_cast<AccE>(0))
         {
-            const uint32_t r  = row0 + 8u * (e >> 2) + 4u * g + (e & 3u);
-            const uint32_t cc = col0 + idx;
-            AccE           v  = alpha * acc[e];
-            if(beta != static_cast<AccE>(0))
-                v += beta * static_cast<const AccE*>(c)[cRow ? (uint64_t)r * ldc + cc : (uint64_t)cc * ldc + r];
-            static_cast<AccE*>(d)[dRow ? (uint64_t)r * ldd + cc : (uint64_t)cc * ldd + r] = v;
+            FragAcc fragC;
+            load_matrix_sync(fragC, c + offC, ldc, layoutC);
+#pragma unroll
+            for(uint32_t i = 0; i < FragAcc::num_elements; ++i)
+                fragAcc.x[i] = alpha * fragAcc.x[i] + beta * fragC.x[i];
         }
+        else
+        {
+#pragma unroll
+            for(uint32_t i = 0; i < FragAcc::num_elements; ++i)
+                fragAcc.x[i] = alpha * fragAcc.x[i];
+        }
+        store_matrix_sync(d + offD, fragAcc, ldd, layoutD);
     }
 
     // ------------------------------------------------------------------ macro-tile kernel
@@ -153,28 +126,51 @@ namespace
         const uint8_t* b;
         const char*    c;
         char*          d;
-        uint32_t       lda, ldb, ldc, ldd;
+        uint32_t       ldb, ldc, ldd;
         double         alpha, beta;
         uint32_t       tilesM, tilesN;
         uint32_t       dRow; // D (and C) row-major
     };
 
-    // Three 52 KiB stage slots (156 of 160 KiB): a stage's 32 matrix instructions last about as long
-    // as half the latency of a direct load, so the slot of stage kt is refilled with stage kt + 3 and
-    // two stages of loads (104 KiB per CU) are in flight at any time.  The direct loads are explicit
-    // (lds_dma.hpp) and the only vmcnt wait is "all but the youngest 13" before each barrier; loads
-    // past the last stage are clamped to it, so every stage issues the same 13.  Every matrix
-    // instruction is followed by one LDS read and (second half of a stage) one direct load, pinned
-    // by scheduling barriers.  Three stages bring every slot back to its role: single-exit loop of
-    // three plus up to two stages of straight-line code.
+    // Three 52 KiB stage slots (156 of 160 KiB): the slot of stage kt is refilled with stage kt + 3 once every
+    // wave has its operands in registers, so two stages of loads (104 KiB per CU) are in flight at any time.  The
+    // direct loads are explicit (lds_dma.hpp) and the only vmcnt wait is "all but the youngest 13" before each
+    // barrier; loads past the last stage are issued with nothing in range (zero fill, no memory traffic), so
+    // every stage issues the same 13.
+    //
+    // A stage is one 128-wide K step: 64 matrix instructions per wave.  As in the dense fp8 kernel it is split
+    // into quadrants of the wave tile, consecutive quadrants sharing one operand group of four blocks:
+    //     Q1 = A[0..3] x B[0..3]   Q2 = A[0..3] x B[4..7]   Q3 = A[4..7] x B[4..7]   Q4 = A[4..7] x B[0..3]
+    //     under Q1: B[4..7] of this stage arrives      under Q3: A[0..3] of the next stage + the refill of A
+    //     under Q2: A[4..7] of this stage              under Q4: B[0..3] of the next stage + the refill of B
+    // After Q2 the stage's slot is no longer read: barrier, then its refill.  One LDS read per two matrix
+    // instructions, one direct load per one to three, pinned by scheduling barriers.  The two B register groups
+    // swap roles every stage and the ring has three slots: six stages per loop trip, single exit, then up to five
+    // stages of straight-line code.
     constexpr uint32_t RING = 3, LOADS_PER_STAGE = 13;
+
+    struct AGroup
+    {
+        i32x4 v[4]; // 16 kept bytes per lane and block
+        int   idx[4];
+    };
+
+    template <bool FP8, typename AccV>
+    __device__ __forceinline__ void smfmac16(AccV& acc, const i32x4& a, const i32x8& b, int idx)
+    {
+        // the accumulator is the instruction's destination and addend at once: updated in place, in an AGPR
+        if constexpr(FP8)
+            asm volatile("v_smfmac_f32_16x16x128_fp8_fp8 %0, %1, %2, %3" : "+a"(acc) : "v"(a), "v"(b), "v"(idx));
+        else
+            asm volatile("v_smfmac_i32_16x16x128_i8 %0, %1, %2, %3" : "+a"(acc) : "v"(a), "v"(b), "v"(idx));
+    }
 
     template <bool FP8>
     __global__ void __launch_bounds__(T_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
         sparseTiledKernel(TiledParams p)
     {
-        using Acc  = std::conditional_t<FP8, f32x16, i32x16>;
         using AccE = std::conditional_t<FP8, float, int>;
+        using AccV = std::conditional_t<FP8, f32x4, i32x4>;
         using r355::loadToLds;
 
         __shared__ __attribute__((aligned(1024))) char lds[RING * STAGE_BYTES];
@@ -187,110 +183,119 @@ namespace
         const uint32_t lane = tid & 63u;
         const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const uint32_t wm = wave >> 1, wn = wave & 1u;
-        const uint32_t r32 = lane & 31u, g = lane >> 5;
+        const uint32_t t = lane & 15u, g = lane >> 4;
         const uint32_t ldsBase
             = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds));
 
         // ---- global -> LDS (per thread, fixed).  LDS chunk L = j * 256 + tid of each operand tile.
-        //   kept values: 4 chunks per row, chunk c of row r in slot c ^ ((r >> 2) & 3)
-        //   dense B:     8 chunks per row, chunk c of row r in slot c ^ ((r >> 1) & 7)
-        //   indices:     one 16-byte chunk per row, thread t <-> row t
-        const uint32_t rowA = tid >> 2, slotA = tid & 3u;
-        const uint32_t gOffA = rowA * p.lda + ((slotA ^ ((rowA >> 2) & 3u)) * 16u), gStepA = 64u * p.lda;
+        //   kept values / indices: the tile's share of a stage is 16 / 4 KiB of consecutive bytes, copied as they are
+        //   dense B: 8 chunks per row, chunk c of row r in slot c ^ ((r >> 1) & 7)
+        const uint32_t gOffA = tid * 16u;
         const uint32_t rowB = tid >> 3, slotB = tid & 7u;
         const uint32_t gOffB = rowB * p.ldb + ((slotB ^ ((rowB >> 1) & 7u)) * 16u), gStepB = 32u * p.ldb;
-        const uint32_t gOffM = tid * (p.k / 8u);
         const uint32_t numStages = p.k / T_K;
-        const uint64_t gA = r355::uniformAddress(p.aVals + (uint64_t)tm * T_M * p.lda);
-        const uint64_t gM = r355::uniformAddress(p.aMeta + (uint64_t)tm * T_M * (p.k / 8u));
+        const uint64_t strideV = (uint64_t)p.m * 64u, strideM = (uint64_t)p.m * 16u; // bytes between stages
+        const uint64_t gA = r355::uniformAddress(p.aVals + (uint64_t)tm * A_BYTES);
+        const uint64_t gM = r355::uniformAddress(p.aMeta + (uint64_t)tm * META_BYTES);
         const uint64_t gB = r355::uniformAddress(p.b + (uint64_t)tn * T_N * p.ldb);
         const uint32_t dmaDst = ldsBase + wave * 1024u; // lane l lands at dmaDst + slot + piece + 16 l
 
-        // load x (0..12) of stage `stage` (already clamped) into the slot at byte `at`
-        auto issueLoad = [&](uint32_t stage, uint32_t at, uint32_t x) {
-            if(x < 4u) // 64 rows of kept values per load
-                loadToLds(r355::rawBuffer(gA + stage * (T_K / 2u)), gOffA, x * gStepA, dmaDst + at + x * 4096u);
-            else if(x == 4u)
-                loadToLds(r355::rawBuffer(gM + stage * (T_K / 8u)), gOffM, 0u, dmaDst + at + OFF_META);
-            else // 32 rows of B per load
-                loadToLds(r355::rawBuffer(gB + stage * T_K), gOffB, (x - 5u) * gStepB, dmaDst + at + OFF_B + (x - 5u) * 4096u);
+        // a buffer over [addr, addr + 2 GiB), or over nothing for a stage past the end
+        auto rsrcOf = [](uint64_t addr, bool valid) {
+            return i32x4{static_cast<int>(static_cast<uint32_t>(addr)), static_cast<int>(static_cast<uint32_t>(addr >> 32) & 0xFFFFu),
+                         valid ? 0x7FFFFFFF : 0, 0x00020000};
         };
-        auto clampStage = [&](uint32_t stage) { return stage < numStages ? stage : numStages - 1u; };
+        // load x (0..12) of stage `stage` into the slot at byte `at`: 0..3 kept values, 4 indices, 5..12 dense B
+        auto issueLoad = [&](uint32_t stage, uint32_t at, uint32_t x) {
+            const bool     valid = stage < numStages;
+            const uint32_t st    = valid ? stage : 0u;
+            if(x < 4u)
+                loadToLds(rsrcOf(gA + st * strideV, valid), gOffA, x * 4096u, dmaDst + at + x * 4096u);
+            else if(x == 4u)
+                loadToLds(rsrcOf(gM + st * strideM, valid), gOffA, 0u, dmaDst + at + OFF_META);
+            else // 32 rows of B per load
+                loadToLds(rsrcOf(gB + (uint64_t)st * T_K, valid), gOffB, (x - 5u) * gStepB, dmaDst + at + OFF_B + (x - 5u) * 4096u);
+        };
 
         // ---- LDS -> registers (per lane, fixed)
-        const uint32_t rA   = wm * 128u + r32, rB = wn * 128u + r32;
-        const uint32_t swA  = (r32 >> 2) & 3u, swB = (r32 >> 1) & 7u;
-        uint32_t       rdA[2], rdB[4];
-#pragma unroll
-        for(uint32_t q = 0; q < 2; ++q) // K group q: kept-value chunk 2 q + g
-            rdA[q] = rA * 64u + (((2u * q + g) ^ swA) * 16u);
-        const uint32_t rdM = OFF_META + rA * 16u + 4u * g; // + 8 q
-#pragma unroll
-        for(uint32_t s = 0; s < 4; ++s) // K group q uses dense chunks 4 q + g and 4 q + 2 + g
-            rdB[s] = OFF_B + rB * 128u + (((2u * s + g) ^ swB) * 16u);
+        //   block i of A (rows 16 i .. + 15 of the wave's 128): 1 KiB of values in lane order, 256 B of indices
+        //   block j of B: row 16 j + t, 16-byte chunks g and 4 + g of the row's 128 bytes
+        const uint32_t rdA = wm * 8192u + lane * 16u, rdM = OFF_META + wm * 2048u + lane * 4u;
+        const uint32_t rB  = wn * 128u + t, swB = (t >> 1) & 7u;
+        const uint32_t rdB0 = OFF_B + rB * 128u + ((g ^ swB) * 16u), rdB1 = OFF_B + rB * 128u + (((4u + g) ^ swB) * 16u);
 
-        struct Frags
-        {
-            i32x4 a[4];
-            int   idx[4];
-            i32x4 b0[4], b1[4];
-        };
-        // read x (0..15) of K group q: the four operands of block index x / 4, values first
-        auto readPiece = [&](Frags& f, uint32_t at, uint32_t q, uint32_t x) {
-            const uint32_t i = x >> 2;
-            const char*    base = lds + at;
-            switch(x & 3u)
-            {
-            case 0: f.a[i] = *reinterpret_cast<const i32x4*>(base + rdA[q] + i * 32u * 64u); break;
-            case 1: f.idx[i] = *reinterpret_cast<const int*>(base + rdM + 8u * q + i * 32u * 16u); break;
-            case 2: f.b0[i] = *reinterpret_cast<const i32x4*>(base + rdB[2u * q] + i * 32u * 128u); break;
-            default: f.b1[i] = *reinterpret_cast<const i32x4*>(base + rdB[2u * q + 1u] + i * 32u * 128u); break;
-            }
-        };
-
-        Acc acc[4][4];
-#pragma unroll
-        for(uint32_t i = 0; i < 4; ++i)
-#pragma unroll
-            for(uint32_t j = 0; j < 4; ++j)
-#pragma unroll
-                for(uint32_t e = 0; e < 16; ++e)
-                    acc[i][j][e] = 0;
-
-        // matrix instruction n (0..15) of a K group: L-shaped shells, so that block index d of either
-        // operand is first needed after d * d instructions (the reads arrive block by block)
-        auto mfmaAt = [&](const Frags& f, uint32_t n) {
-            uint32_t d = 0;
-            while((d + 1u) * (d + 1u) <= n)
-                ++d;
-            const uint32_t r = n - d * d;
-            const uint32_t i = r <= d ? d : r - d - 1u, j = r <= d ? r : d;
-            const i32x8    bv = {f.b0[j][0], f.b0[j][1], f.b0[j][2], f.b0[j][3], f.b1[j][0], f.b1[j][1], f.b1[j][2], f.b1[j][3]};
-            if constexpr(FP8)
-                acc[i][j] = __builtin_amdgcn_smfmac_f32_32x32x64_fp8_fp8(f.a[i], bv, acc[i][j], f.idx[i], 0, 0);
+        // piece r (0..7) of an A group: block r / 2 of the half, values (r even) or indices (r odd)
+        auto readA = [&](AGroup& grp, uint32_t at, uint32_t half, uint32_t r) {
+            const uint32_t i = 4u * half + (r >> 1);
+            if(r & 1u)
+                grp.idx[r >> 1] = *reinterpret_cast<const int*>(lds + at + rdM + i * 256u);
             else
-                acc[i][j] = __builtin_amdgcn_smfmac_i32_32x32x64_i8(f.a[i], bv, acc[i][j], f.idx[i], 0, 0);
+                grp.v[r >> 1] = *reinterpret_cast<const i32x4*>(lds + at + rdA + i * 1024u);
+        };
+        // piece r (0..7) of a B group: block r / 2 of the half, 64-byte K half r % 2
+        auto readB = [&](i32x8 (&grp)[4], uint32_t at, uint32_t half, uint32_t r) {
+            const uint32_t j = 4u * half + (r >> 1);
+            const i32x4    v = *reinterpret_cast<const i32x4*>(lds + at + ((r & 1u) ? rdB1 : rdB0) + j * 2048u);
+            const uint32_t o = 4u * (r & 1u);
+            grp[r >> 1][o] = v[0], grp[r >> 1][o + 1u] = v[1], grp[r >> 1][o + 2u] = v[2], grp[r >> 1][o + 3u] = v[3];
+        };
+        // the pieces / loads dealt to slot n (0..15) of a quadrant
+        auto readSlotA = [&](AGroup& grp, uint32_t at, uint32_t half, uint32_t n) {
+            if((n & 1u) == 0u)
+                readA(grp, at, half, n >> 1);
+        };
+        auto readSlotB = [&](i32x8 (&grp)[4], uint32_t at, uint32_t half, uint32_t n) {
+            if((n & 1u) == 0u)
+                readB(grp, at, half, n >> 1);
         };
 
-        Frags f0, f1;
-        auto  stageBody = [&](uint32_t kt, uint32_t cur, uint32_t nxt) {
+        AccV acc[8][8];
+#pragma unroll
+        for(uint32_t i = 0; i < 8; ++i)
+#pragma unroll
+            for(uint32_t j = 0; j < 8; ++j)
+                acc[i][j] = AccV{0, 0, 0, 0};
+
+        AGroup aLo, aHi;
+        i32x8  bX[4], bY[4]; // alternate as the low / high half of B's blocks
+
+        auto stageBody = [&](uint32_t kt, uint32_t cur, uint32_t nxt, i32x8 (&bLo)[4], i32x8 (&bHi)[4]) {
+            // Q1: A low x B low; B high arrives
 #pragma unroll
             for(uint32_t n = 0; n < 16; ++n)
             {
-                mfmaAt(f0, n);
-                readPiece(f1, cur, 1, n);
+                smfmac16<FP8>(acc[n % 4u][n / 4u], aLo.v[n % 4u], bLo[n / 4u], aLo.idx[n % 4u]);
+                readSlotB(bHi, cur, 1, n);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // Q2: A low x B high (column by column, in the order B arrived); A high arrives
+#pragma unroll
+            for(uint32_t n = 0; n < 16; ++n)
+            {
+                smfmac16<FP8>(acc[n % 4u][4u + n / 4u], aLo.v[n % 4u], bHi[n / 4u], aLo.idx[n % 4u]);
+                readSlotA(aHi, cur, 1, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
             r355::waitVmcnt<LOADS_PER_STAGE>(); // stage kt + 1 has landed; the youngest 13 loads are stage kt + 2
             r355::ldsBarrier();
-            const uint32_t refill = clampStage(kt + 3u);
+            // Q3: A high x B high (row by row, in the order A arrived); next A low arrives; refill of A (5 loads)
 #pragma unroll
             for(uint32_t n = 0; n < 16; ++n)
             {
-                mfmaAt(f1, n);
-                readPiece(f0, nxt, 0, n);
-                if(n < LOADS_PER_STAGE)
-                    issueLoad(refill, cur, n);
+                smfmac16<FP8>(acc[4u + n / 4u][4u + n % 4u], aHi.v[n / 4u], bHi[n % 4u], aHi.idx[n / 4u]);
+                readSlotA(aLo, nxt, 0, n);
+                if(n % 3u == 1u && n / 3u < 5u)
+                    issueLoad(kt + 3u, cur, n / 3u);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // Q4: A high x B low; next B low arrives in the registers B high has left; refill of B (8 loads)
+#pragma unroll
+            for(uint32_t n = 0; n < 16; ++n)
+            {
+                smfmac16<FP8>(acc[4u + n % 4u][n / 4u], aHi.v[n % 4u], bLo[n / 4u], aHi.idx[n % 4u]);
+                readSlotB(bHi, nxt, 0, n);
+                if(n & 1u)
+                    issueLoad(kt + 3u, cur, 5u + (n >> 1));
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
@@ -300,33 +305,53 @@ namespace
         for(uint32_t st = 0; st < RING; ++st)
 #pragma unroll
             for(uint32_t x = 0; x < LOADS_PER_STAGE; ++x)
-                issueLoad(clampStage(st), SLOT[st], x);
+                issueLoad(st, SLOT[st], x);
         r355::waitVmcnt<2u * LOADS_PER_STAGE>();
         r355::ldsBarrier();
 #pragma unroll
-        for(uint32_t x = 0; x < 16; ++x)
-            readPiece(f0, SLOT[0], 0, x);
+        for(uint32_t r = 0; r < 8; ++r)
+        {
+            readA(aLo, SLOT[0], 0, r);
+            readB(bX, SLOT[0], 0, r);
+        }
 
         uint32_t kt = 0;
-        for(uint32_t trips = numStages / 3u; trips > 0; --trips, kt += 3u)
+        for(uint32_t trips = numStages / 6u; trips > 0; --trips, kt += 6u)
         {
-            stageBody(kt, SLOT[0], SLOT[1]);
-            stageBody(kt + 1u, SLOT[1], SLOT[2]);
-            stageBody(kt + 2u, SLOT[2], SLOT[0]);
+            stageBody(kt, SLOT[0], SLOT[1], bX, bY);
+            stageBody(kt + 1u, SLOT[1], SLOT[2], bY, bX);
+            stageBody(kt + 2u, SLOT[2], SLOT[0], bX, bY);
+            stageBody(kt + 3u, SLOT[0], SLOT[1], bY, bX);
+            stageBody(kt + 4u, SLOT[1], SLOT[2], bX, bY);
+            stageBody(kt + 5u, SLOT[2], SLOT[0], bY, bX);
         }
         const uint32_t rem = numStages - kt;
         if(rem > 0u)
         {
-            stageBody(kt, SLOT[0], SLOT[1]);
+            stageBody(kt, SLOT[0], SLOT[1], bX, bY);
             if(rem > 1u)
-                stageBody(kt + 1u, SLOT[1], SLOT[2]);
+            {
+                stageBody(kt + 1u, SLOT[1], SLOT[2], bY, bX);
+                if(rem > 2u)
+                {
+                    stageBody(kt + 2u, SLOT[2], SLOT[0], bX, bY);
+                    if(rem > 3u)
+                    {
+                        stageBody(kt + 3u, SLOT[0], SLOT[1], bY, bX);
+                        if(rem > 4u)
+                            stageBody(kt + 4u, SLOT[1], SLOT[2], bX, bY);
+                    }
+                }
+            }
         }
-        // the clamped loads of the last stages are still landing in the slots the epilogue reuses
+        // the loads past the last stage (zeros) are still landing in the slots the epilogue reuses, and the last
+        // matrix instructions are still in the pipeline (the compiler knows neither)
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
         r355::waitVmcnt<0>();
         r355::ldsBarrier();
 
-        // ---- epilogue.  lane holds D(m = 8 (e / 4) + 4 g + e % 4, n = lane % 32) of each block:
-        // four consecutive rows of one column.
+        // ---- epilogue.  A lane holds D(16 i + 4 g + e, 16 j + t), e = 0..3, of each block: four consecutive
+        // rows of one column.
         const AccE     alpha = static_cast<AccE>(p.alpha), beta = static_cast<AccE>(p.beta);
         const uint32_t m0 = tm * T_M + wm * 128u, n0 = tn * T_N + wn * 128u;
         using V4 = AccE __attribute__((ext_vector_type(4)));
@@ -334,50 +359,51 @@ namespace
         {
             // col-major: a lane's four rows are contiguous
 #pragma unroll
-            for(uint32_t i = 0; i < 4; ++i)
+            for(uint32_t i = 0; i < 8; ++i)
 #pragma unroll
-                for(uint32_t j = 0; j < 4; ++j)
+                for(uint32_t j = 0; j < 8; ++j)
+                {
+                    const uint32_t row = m0 + 16u * i + 4u * g, col = n0 + 16u * j + t;
+                    V4             out;
 #pragma unroll
-                    for(uint32_t q = 0; q < 4; ++q)
+                    for(uint32_t e = 0; e < 4; ++e)
+                        out[e] = alpha * acc[i][j][e];
+                    if(beta != static_cast<AccE>(0))
                     {
-                        const uint32_t row = m0 + 32u * i + 8u * q + 4u * g, col = n0 + 32u * j + r32;
-                        V4             out;
+                        const V4 cv = *reinterpret_cast<const V4*>(p.c + ((uint64_t)col * p.ldc + row) * 4u);
 #pragma unroll
                         for(uint32_t e = 0; e < 4; ++e)
-                            out[e] = alpha * acc[i][j][4 * q + e];
-                        if(beta != static_cast<AccE>(0))
-                        {
-                            const V4 cv = *reinterpret_cast<const V4*>(p.c + ((uint64_t)col * p.ldc + row) * 4u);
-#pragma unroll
-                            for(uint32_t e = 0; e < 4; ++e)
-                                out[e] += beta * cv[e];
-                        }
-                        *reinterpret_cast<V4*>(p.d + ((uint64_t)col * p.ldd + row) * 4u) = out;
+                            out[e] += beta * cv[e];
                     }
+                    *reinterpret_cast<V4*>(p.d + ((uint64_t)col * p.ldd + row) * 4u) = out;
+                }
             return;
         }
-        // row-major: transpose through this wave's 26 KiB of the idle stage slots, 32 rows (one
-        // block row i) at a time: rows of 128 x 4 bytes = 32 chunks, chunk c of row r in slot c ^ r.
-        char* wl = lds + wave * 26624u;
+        // row-major: transpose through this wave's 39 KiB of the idle stage slots, 64 rows (four block rows) at a
+        // time: rows of 128 x 4 bytes = 32 chunks, chunk c of row r in slot c ^ (r & 31) -- the 64 lanes of a write
+        // (rows 4 g + e, columns 16 j + t) and of a read (two whole rows) each cover all 64 banks once.
+        char* wl = lds + wave * 39936u;
 #pragma unroll
-        for(uint32_t i = 0; i < 4; ++i)
+        for(uint32_t pass = 0; pass < 2; ++pass)
         {
 #pragma unroll
-            for(uint32_t j = 0; j < 4; ++j)
+            for(uint32_t ii = 0; ii < 4; ++ii)
 #pragma unroll
-                for(uint32_t e = 0; e < 16; ++e)
-                {
-                    const uint32_t row = 8u * (e >> 2) + 4u * g + (e & 3u), col = 32u * j + r32;
-                    *reinterpret_cast<AccE*>(wl + row * 512u + (((col >> 2) ^ row) * 16u) + (col & 3u) * 4u)
-                        = alpha * acc[i][j][e];
-                }
+                for(uint32_t j = 0; j < 8; ++j)
+#pragma unroll
+                    for(uint32_t e = 0; e < 4; ++e)
+                    {
+                        const uint32_t row = 16u * ii + 4u * g + e, col = 16u * j + t;
+                        *reinterpret_cast<AccE*>(wl + row * 512u + (((col >> 2) ^ (row & 31u)) * 16u) + (col & 3u) * 4u)
+                            = alpha * acc[4u * pass + ii][j][e];
+                    }
             __builtin_amdgcn_wave_barrier();
 #pragma unroll
-            for(uint32_t it = 0; it < 16; ++it)
+            for(uint32_t it = 0; it < 32; ++it)
             {
                 const uint32_t L = it * 64u + lane, row = L >> 5, c = L & 31u;
-                V4             v = *reinterpret_cast<const V4*>(wl + row * 512u + ((c ^ row) * 16u));
-                const uint64_t off = (uint64_t)(m0 + 32u * i + row);
+                V4             v = *reinterpret_cast<const V4*>(wl + row * 512u + ((c ^ (row & 31u)) * 16u));
+                const uint64_t off = (uint64_t)(m0 + 64u * pass + row);
                 if(beta != static_cast<AccE>(0))
                 {
                     const V4 cv = *reinterpret_cast<const V4*>(p.c + (off * p.ldc + n0) * 4u + c * 16u);
@@ -397,6 +423,11 @@ namespace
                && g.layout_c == g.layout_d && (g.ldd % 4) == 0 && r355::aligned(g.d, 16)
                && (g.beta == 0.0 || ((g.ldc % 4) == 0 && r355::aligned(g.c, 16))) && r355::aligned(g.a_meta, 16);
     }
+
+    uint32_t simpleBlock(const r355_gemm_args& g)
+    {
+        return (g.m % 32u == 0u && g.n % 32u == 0u) ? 32u : 16u;
+    }
 } // namespace
 
 namespace r355
@@ -409,14 +440,17 @@ namespace r355
         if(!i8 && !f8 && !w)
             return fail(R355_ERR_UNSUPPORTED, "sparse gemm: supported types are i8 -> i32 and e4m3 | f16 | bf16 -> f32");
         if(g.layout_a != R355_ROW_MAJOR || g.layout_b != R355_COL_MAJOR)
-            return fail(R355_ERR_UNSUPPORTED, "sparse gemm: compressed A must be row-major and B col-major");
+            return fail(R355_ERR_UNSUPPORTED, "sparse gemm: compressed A is K-blocked row storage (R355_ROW_MAJOR) and B must be col-major");
         if(!g.a_meta)
             return fail(R355_ERR_BAD_ARG, "sparse gemm: a_meta is null");
-        const uint32_t es = w ? 2u : 1u, kStep = w ? 32u : 64u; // element bytes, dense k per matrix instruction
-        if(g.m % 32 || g.n % 32 || g.k % kStep)
-            return fail(R355_ERR_BAD_SIZE, "sparse gemm: m=%u n=%u must be multiples of 32 and k=%u of %u", g.m, g.n, g.k, kStep);
-        if(!aligned(g.a, 16) || (g.lda * es) % 16 || !aligned(g.b, 16) || (g.ldb * es) % 16 || !aligned(g.a_meta, 4) || !aligned(g.d, 4))
-            return fail(R355_ERR_MISALIGNED, "sparse gemm: values / B need 16-byte alignment, metadata 4-byte");
+        const uint32_t es = w ? 2u : 1u, kStage = 128u / es; // element bytes, dense k per stage of the storage format
+        if(g.m % 16 || g.n % 16 || g.k % kStage)
+            return fail(R355_ERR_BAD_SIZE, "sparse gemm: m=%u n=%u must be multiples of 16 and k=%u of %u", g.m, g.n, g.k, kStage);
+        if(g.lda != g.k / 2u)
+            return fail(R355_ERR_BAD_ARG, "sparse gemm: the K-blocked storage of A has no padding: lda=%u must be k / 2 = %u", g.lda, g.k / 2u);
+        if(!aligned(g.a, 16) || !aligned(g.b, 16) || (g.ldb * es) % 16 || !aligned(g.a_meta, 4) || !aligned(g.d, 16) || (g.ldd % 4)
+           || (g.beta != 0.0 && (!aligned(g.c, 16) || (g.ldc % 4))))
+            return fail(R355_ERR_MISALIGNED, "sparse gemm: values, B, C and D need 16-byte alignment (pointers and leading dimensions), metadata 4-byte");
         if(g.kernel == R355_KERNEL_TILED_128)
             return fail(R355_ERR_UNSUPPORTED, "sparse gemm: there is no 128 x 128 sparse macro tile (R355_KERNEL_TILED is 256 x 256)");
         if(w && g.kernel == R355_KERNEL_TILED)
@@ -437,17 +471,38 @@ namespace r355
         }
         else if(plan)
         {
+            const uint32_t blk = simpleBlock(g);
             plan->kernel       = R355_KERNEL_SIMPLE;
-            plan->macro_tile_m = 32 * WAVES_X;
-            plan->macro_tile_n = 32 * WAVES_Y;
-            plan->macro_tile_k = (g.in_type == R355_F16 || g.in_type == R355_BF16) ? 32 : 64;
-            plan->grid_x       = (g.m + 32 * WAVES_X - 1) / (32 * WAVES_X);
-            plan->grid_y       = (g.n + 32 * WAVES_Y - 1) / (32 * WAVES_Y);
+            plan->macro_tile_m = blk * WAVES_X;
+            plan->macro_tile_n = blk * WAVES_Y;
+            plan->macro_tile_k = kStage;
+            plan->grid_x       = (g.m + blk * WAVES_X - 1) / (blk * WAVES_X);
+            plan->grid_y       = (g.n + blk * WAVES_Y - 1) / (blk * WAVES_Y);
             plan->block_x      = WAVES_X * 64;
             plan->block_y      = WAVES_Y;
             plan->lds_bytes    = 0;
         }
         return R355_OK;
+    }
+
+    template <typename InT, typename AccE>
+    static int launchSimple(const r355_gemm_args& g, hipStream_t stream)
+    {
+        const uint32_t blk = simpleBlock(g);
+        dim3           block(WAVES_X * 64, WAVES_Y);
+        dim3           grid((g.m + blk * WAVES_X - 1) / (blk * WAVES_X), (g.n + blk * WAVES_Y - 1) / (blk * WAVES_Y));
+        const layout_t lc = g.layout_c == R355_ROW_MAJOR ? mem_row_major : mem_col_major;
+        const layout_t ld = g.layout_d == R355_ROW_MAJOR ? mem_row_major : mem_col_major;
+        auto           go = [&](auto kernel) {
+            hipLaunchKernelGGL(kernel, grid, block, 0, stream, g.m, g.n, g.k, static_cast<const InT*>(g.a),
+                               static_cast<const uint8_t*>(g.a_meta), static_cast<const InT*>(g.b), static_cast<const AccE*>(g.c),
+                               static_cast<AccE*>(g.d), g.ldb, g.ldc, g.ldd, lc, ld, static_cast<AccE>(g.alpha), static_cast<AccE>(g.beta));
+        };
+        if(blk == 32u)
+            go(sparseBlockPerWave<InT, AccE, 32>);
+        else
+            go(sparseBlockPerWave<InT, AccE, 16>);
+        return checkLaunch("sparse gemm");
     }
 
     int gemmSparseLaunch(const r355_gemm_args& g, hipStream_t stream)
@@ -459,7 +514,7 @@ namespace r355
             p.aVals = static_cast<const uint8_t*>(g.a), p.aMeta = static_cast<const uint8_t*>(g.a_meta);
             p.b = static_cast<const uint8_t*>(g.b);
             p.c = static_cast<const char*>(g.c), p.d = static_cast<char*>(g.d);
-            p.lda = g.lda, p.ldb = g.ldb, p.ldc = g.ldc, p.ldd = g.ldd;
+            p.ldb = g.ldb, p.ldc = g.ldc, p.ldd = g.ldd;
             p.alpha = g.alpha, p.beta = g.beta;
             p.tilesM = g.m / T_M, p.tilesN = g.n / T_N;
             p.dRow = g.layout_d == R355_ROW_MAJOR;
@@ -470,45 +525,54 @@ namespace r355
                 hipLaunchKernelGGL(sparseTiledKernel<false>, dim3(grid), dim3(T_THREADS), 0, stream, p);
             return checkLaunch("sparse gemm (macro tile)");
         }
-        dim3 block(WAVES_X * 64, WAVES_Y);
-        dim3 grid((g.m + 32 * WAVES_X - 1) / (32 * WAVES_X), (g.n + 32 * WAVES_Y - 1) / (32 * WAVES_Y));
-        auto* av = static_cast<const uint8_t*>(g.a);
-        auto* am = static_cast<const uint8_t*>(g.a_meta);
-        auto* bb = static_cast<const uint8_t*>(g.b);
-        const bool cRow = g.layout_c == R355_ROW_MAJOR, dRow = g.layout_d == R355_ROW_MAJOR;
-#define R355_SPARSE_LAUNCH(E)                                                                                       \
-    hipLaunchKernelGGL(sparseBlockPerWave<SpElem::E>, grid, block, 0, stream, g.m, g.n, g.k, av, am, bb, g.c, g.d, g.lda, \
-                       g.ldb, g.ldc, g.ldd, cRow, dRow, g.alpha, g.beta)
         switch(g.in_type)
         {
-        case R355_E4M3: R355_SPARSE_LAUNCH(E4M3); break;
-        case R355_F16: R355_SPARSE_LAUNCH(F16); break;
-        case R355_BF16: R355_SPARSE_LAUNCH(BF16); break;
-        default: R355_SPARSE_LAUNCH(I8); break;
+        case R355_E4M3: return launchSimple<float8_t, float>(g, stream);
+        case R355_F16: return launchSimple<float16_t, float>(g, stream);
+        case R355_BF16: return launchSimple<bfloat16_t, float>(g, stream);
+        default: return launchSimple<int8_t, int32_t>(g, stream);
         }
-#undef R355_SPARSE_LAUNCH
-        return checkLaunch("sparse gemm");
     }
 } // namespace r355
 
 namespace
 {
+    // Byte offsets of (row, dense group of four `grp`) in the K-blocked storage: the group's two kept elements and
+    // its index nibble.  A stage holds 32 / ES groups of a row, a lane group 8 / ES of them.
+    template <typename T>
+    struct Place
+    {
+        size_t   value; // element index of the first kept element
+        size_t   metaByte;
+        uint32_t metaShift;
+    };
+    template <typename T>
+    Place<T> placeOf(uint32_t row, uint32_t grp, uint32_t m)
+    {
+        using S                  = rocwmma::Sparse24<T>;
+        constexpr uint32_t perLg = S::ChunkElems / 2u; // groups per lane group: 8 (1-byte) or 4 (2-byte elements)
+        const uint32_t stage = grp / (4u * perLg), lg = (grp / perLg) % 4u, within = grp % perLg;
+        Place<T>       pl;
+        pl.value = (size_t)stage * S::valueStageStride(m) + S::valueByteInStage(row, lg) / sizeof(T) + 2u * within;
+        pl.metaByte  = (size_t)stage * S::metaStageStride(m) + S::metaByteInStage(row, lg) + within / 2u;
+        pl.metaShift = 4u * (within & 1u);
+        return pl;
+    }
+
     // An element counts as zero when all its bits are zero (a kept -0.0 stays a kept value: the round trip is exact).
     template <typename T>
     int compress24(const T* dense, uint32_t m, uint32_t k, T* values, uint8_t* meta)
     {
         if(!dense || !values || !meta)
             return r355::fail(R355_ERR_BAD_ARG, "compress_24: null pointer");
-        if(k % 8u)
-            return r355::fail(R355_ERR_BAD_SIZE, "compress_24: k=%u must be a multiple of 8", k);
-        const uint32_t groups = k / 4u;
+        if(m % 16u || k % rocwmma::Sparse24<T>::StageK)
+            return r355::fail(R355_ERR_BAD_SIZE, "compress_24: m=%u must be a multiple of 16 and k=%u of %u", m, k,
+                              rocwmma::Sparse24<T>::StageK);
+        memset(meta, 0, (size_t)m * k / 8u);
         for(uint32_t r = 0; r < m; ++r)
         {
             const T* src = dense + (size_t)r * k;
-            T*       val = values + (size_t)r * (k / 2u);
-            uint8_t* md  = meta + (size_t)r * (k / 8u);
-            memset(md, 0, k / 8u);
-            for(uint32_t g = 0; g < groups; ++g)
+            for(uint32_t g = 0; g < k / 4u; ++g)
             {
                 // positions of the kept pair: the non-zeros first, then the lowest free positions
                 uint32_t keep = 0, count = 0; // bit mask over the 4 positions
@@ -524,9 +588,10 @@ namespace
                 for(uint32_t e = 0; e < 4; ++e)
                     if(keep & (1u << e))
                         pos[p++] = e;
-                val[2 * g]     = src[4 * g + pos[0]];
-                val[2 * g + 1] = src[4 * g + pos[1]];
-                md[g / 2] |= static_cast<uint8_t>((pos[0] | (pos[1] << 2)) << (4 * (g & 1u)));
+                const Place<T> pl    = placeOf<T>(r, g, m);
+                values[pl.value]     = src[4 * g + pos[0]];
+                values[pl.value + 1] = src[4 * g + pos[1]];
+                meta[pl.metaByte] |= static_cast<uint8_t>((pos[0] | (pos[1] << 2)) << pl.metaShift);
             }
         }
         return R355_OK;
@@ -537,15 +602,17 @@ namespace
     {
         if(!dense || !values || !meta)
             return r355::fail(R355_ERR_BAD_ARG, "decompress_24: null pointer");
-        if(k % 8u)
-            return r355::fail(R355_ERR_BAD_SIZE, "decompress_24: k=%u must be a multiple of 8", k);
+        if(m % 16u || k % rocwmma::Sparse24<T>::StageK)
+            return r355::fail(R355_ERR_BAD_SIZE, "decompress_24: m=%u must be a multiple of 16 and k=%u of %u", m, k,
+                              rocwmma::Sparse24<T>::StageK);
         memset(dense, 0, (size_t)m * k * sizeof(T));
         for(uint32_t r = 0; r < m; ++r)
             for(uint32_t g = 0; g < k / 4u; ++g)
             {
-                const uint32_t nib = (meta[(size_t)r * (k / 8u) + g / 2] >> (4 * (g & 1u))) & 0xFu;
-                dense[(size_t)r * k + 4 * g + (nib & 3u)]  = values[(size_t)r * (k / 2u) + 2 * g];
-                dense[(size_t)r * k + 4 * g + (nib >> 2)] = values[(size_t)r * (k / 2u) + 2 * g + 1];
+                const Place<T> pl  = placeOf<T>(r, g, m);
+                const uint32_t nib = (meta[pl.metaByte] >> pl.metaShift) & 0xFu;
+                dense[(size_t)r * k + 4 * g + (nib & 3u)]  = values[pl.value];
+                dense[(size_t)r * k + 4 * g + (nib >> 2)] = values[pl.value + 1];
             }
         return R355_OK;
     }

@@ -20,7 +20,8 @@
 // For BlockDim 16 / 32 a chunk of KW * G along K is exactly one MFMA operand:
 //   f16, bf16 : KW 8 -> v_mfma_f32_32x32x16 / 16x16x32,  KW 4 -> 32x32x8 / 16x16x16
 //   int8      : KW 16 -> v_mfma_i32_32x32x32 / 16x16x64, KW 8 -> 32x32x16 / 16x16x32
-//   fp8 e4m3  : KW 8 -> v_mfma_f32_32x32x16 / 16x16x32 (fp8_fp8)
+//   fp8 / bf8 : KW 16 -> two v_mfma_f32_32x32x16 / 16x16x32 (fp8_fp8 / bf8_bf8) on the lane's two 8-byte halves,
+//               KW 8 -> one (a lane's 16 consecutive K bytes are also what the 2:4 sparse instructions pair with)
 //   f32       : KW 1 -> v_mfma_f32_32x32x2 / 16x16x4
 //   f64       : KW 1 -> v_mfma_f64_16x16x4 (BlockDim 16 only)
 // Accumulators use KW 4, which is the MFMA C/D layout (f64: KW 1, row = 4 e + lane / 16)
@@ -91,7 +92,7 @@ namespace rocwmma
             // 16 x 16 and 32 x 32 blocks: start from the widest matrix-instruction operand of the type and
             // halve until the wave's chunk tiles KDim.  Widths below the narrowest instruction form (4 for
             // 16-bit types, 8 for 8-bit types) still load, store and fill; mma_sync rejects them.
-            uint32_t kw = bytes == 2u ? 8u : (is_i8_v<DataT> ? 16u : (bytes == 1u ? 8u : 1u));
+            uint32_t kw = bytes == 2u ? 8u : (bytes == 1u ? 16u : 1u);
             while(kw > 1u && (kDim % (kw * groups)) != 0u)
                 kw >>= 1;
             return kw;

@@ -7,8 +7,8 @@
 //   f16   8/lane: v_mfma_f32_32x32x16_f16   / 16x16x32_f16    4/lane: 32x32x8f16 / 16x16x16f16
 //   bf16  8/lane: v_mfma_f32_32x32x16_bf16  / 16x16x32_bf16   4/lane: 32x32x8bf16_1k / 16x16x16bf16_1k
 //   int8 16/lane: v_mfma_i32_32x32x32_i8    / 16x16x64_i8     8/lane: 32x32x16_i8 / 16x16x32_i8
-//   e4m3  8/lane: v_mfma_f32_32x32x16_fp8_fp8 / 16x16x32_fp8_fp8   (OCP encoding on gfx950)
-//   e5m2  8/lane: v_mfma_f32_32x32x16_bf8_bf8 / 16x16x32_bf8_bf8   (OCP encoding on gfx950)
+//   e4m3  8/lane: v_mfma_f32_32x32x16_fp8_fp8 / 16x16x32_fp8_fp8   (OCP encoding on gfx950); 16/lane: two of them,
+//   e5m2  8/lane: v_mfma_f32_32x32x16_bf8_bf8 / 16x16x32_bf8_bf8   one per 8-byte half of the lane's K bytes
 //   f32   1/lane: v_mfma_f32_32x32x2f32     / 16x16x4f32
 //   f64   1/lane: v_mfma_f64_16x16x4f64 (16x16 blocks only)
 #ifndef ROCWMMA_MFMA_HPP
@@ -104,6 +104,13 @@ namespace rocwmma
                         acc = __builtin_amdgcn_mfma_i32_32x32x16_i8(av, bv, acc, 0, 0, 0);
                     else
                         acc = __builtin_amdgcn_mfma_i32_16x16x32_i8(av, bv, acc, 0, 0, 0);
+                }
+                else if constexpr((is_fp8_v<InputT> || is_bf8_v<InputT>) && KW == 16u)
+                {
+                    // K is a sum: the low 8 bytes of every lane of A meet the low 8 bytes of every lane of B in one
+                    // instruction, the high 8 bytes in the next
+                    MfmaChunk<InputT, BlockDim, 8u>::exec(acc, a, b);
+                    MfmaChunk<InputT, BlockDim, 8u>::exec(acc, a + 8, b + 8);
                 }
                 else if constexpr(is_fp8_v<InputT> && KW == 8u)
                 {

@@ -4,6 +4,7 @@
 // (tests/test_fragment_api.py) drives them through this C ABI and compares on the host.
 #include <rocwmma/rocwmma.hpp>
 #include <rocwmma/rocwmma_coop.hpp>
+#include <rocwmma/rocwmma_sparse.hpp>
 #include <rocwmma/rocwmma_transforms.hpp>
 
 using namespace rocwmma;
@@ -98,6 +99,24 @@ namespace
         load_matrix_sync(fb, b, ldb);
         load_matrix_sync(fc, c, ldc, layoutC);
         mma_sync(fc, fa, fb, fc);
+        store_matrix_sync(d, fc, ldc, layoutC);
+    }
+
+    // one tile D = A B + C with A 2:4 sparse in the K-blocked storage of a Blk-row matrix (rocwmma_sparse.hpp)
+    template <uint32_t Blk, uint32_t BK, typename InT, typename AccT, typename LB>
+    __global__ void sparseMmaTile(const InT* aVals, const uint8_t* aMeta, const InT* b, const AccT* c, AccT* d, uint32_t ldb,
+                                  uint32_t ldc, layout_t layoutC)
+    {
+        using S = Sparse24<InT>;
+        fragment<sparse_matrix_a, Blk, Blk, BK, InT, row_major> fa;
+        fragment<sparse_metadata, Blk, Blk, BK, InT>            fm;
+        fragment<matrix_b, Blk, Blk, BK, InT, LB>               fb;
+        fragment<accumulator, Blk, Blk, BK, AccT>               fc;
+        load_matrix_sync(fa, aVals + S::valueOffset(0u, 0u, Blk), S::valueStageStride(Blk));
+        load_matrix_sync(fm, aMeta + S::metaOffset(0u, 0u, Blk), S::metaStageStride(Blk));
+        load_matrix_sync(fb, b, ldb);
+        load_matrix_sync(fc, c, ldc, layoutC);
+        mma_sync(fc, fa, fm, fb, fc);
         store_matrix_sync(d, fc, ldc, layoutC);
     }
 
@@ -405,6 +424,49 @@ int api_mma_tile(int type, uint32_t blk, uint32_t bk, int aRow, int bRow, int cR
     case 8: SHAPE(bfloat16_t, bfloat16_t, 16, 16, 16, 32, 32, 8, 32, 16); break;
     case 9: SHAPE(hfloat16_t, float32_t, 16, 16, 16, 32, 32, 8, 32, 16); break; // __half operands
     case 10: SHAPE(hfloat16_t, hfloat16_t, 16, 16, 16, 32, 32, 8, 32, 16); break;
+    default: return -1;
+    }
+    return hipDeviceSynchronize() == hipSuccess ? 0 : -2;
+}
+
+// one sparse tile.  type: 0 f16, 1 bf16, 2 e4m3, 3 i8, 7 e5m2; blk 16 | 32; stages: K stages of 128 bytes (1 | 2)
+int api_sparse_mma_tile(int type, uint32_t blk, uint32_t stages, int bRow, int cRow, const void* aVals, const void* aMeta,
+                        const void* b, const void* c, void* d, uint32_t ldb, uint32_t ldc)
+{
+    const layout_t lc = cRow ? mem_row_major : mem_col_major;
+#define SLAUNCH(BLK, BKK, T, ACC, LB)                                                                              \
+    hipLaunchKernelGGL((sparseMmaTile<BLK, BKK, T, ACC, LB>), dim3(1), dim3(64), 0, 0, static_cast<const T*>(aVals), \
+                       static_cast<const uint8_t*>(aMeta), static_cast<const T*>(b), static_cast<const ACC*>(c),    \
+                       static_cast<ACC*>(d), ldb, ldc, lc)
+#define SSHAPE(T, ACC, SK)                               \
+    do                                                   \
+    {                                                    \
+        if(blk == 16 && stages == 1 && bRow)             \
+            SLAUNCH(16, SK, T, ACC, row_major);          \
+        else if(blk == 16 && stages == 1)                \
+            SLAUNCH(16, SK, T, ACC, col_major);          \
+        else if(blk == 16 && stages == 2 && bRow)        \
+            SLAUNCH(16, 2 * SK, T, ACC, row_major);      \
+        else if(blk == 16 && stages == 2)                \
+            SLAUNCH(16, 2 * SK, T, ACC, col_major);      \
+        else if(blk == 32 && stages == 1 && bRow)        \
+            SLAUNCH(32, SK, T, ACC, row_major);          \
+        else if(blk == 32 && stages == 1)                \
+            SLAUNCH(32, SK, T, ACC, col_major);          \
+        else if(blk == 32 && stages == 2 && bRow)        \
+            SLAUNCH(32, 2 * SK, T, ACC, row_major);      \
+        else if(blk == 32 && stages == 2)                \
+            SLAUNCH(32, 2 * SK, T, ACC, col_major);      \
+        else                                             \
+            return -1;                                   \
+    } while(0)
+    switch(type)
+    {
+    case 0: SSHAPE(float16_t, float32_t, 64); break;
+    case 1: SSHAPE(bfloat16_t, float32_t, 64); break;
+    case 2: SSHAPE(float8_t, float32_t, 128); break;
+    case 3: SSHAPE(int8_t, int32_t, 128); break;
+    case 7: SSHAPE(bfloat8_t, float32_t, 128); break;
     default: return -1;
     }
     return hipDeviceSynchronize() == hipSuccess ? 0 : -2;

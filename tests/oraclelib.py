@@ -122,13 +122,15 @@ def fill_ref(dtype, m, n, layout):
 
 
 def compress24(dense_u8, m, k):
+    """K-blocked 2:4 storage of a (m, k) matrix of 1-byte elements: values [k / 128][m / 16][4][16][16] and
+    meta [k / 128][m / 16][4][16][4] (see orc_compress24)."""
     dense_u8 = np.ascontiguousarray(dense_u8).view(np.uint8)
     vals = np.zeros(m * k // 2, dtype=np.uint8)
     meta = np.zeros(m * k // 8, dtype=np.uint8)
     rc = lib().orc_compress24(_p(dense_u8), m, k, _p(vals), _p(meta))
     if rc != 0:
-        raise ValueError("not a 2:4 matrix")
-    return vals.reshape(m, k // 2), meta.reshape(m, k // 8)
+        raise ValueError("not a 2:4 matrix (or m % 16, k % 128)")
+    return vals.reshape(k // 128, m // 16, 4, 16, 16), meta.reshape(k // 128, m // 16, 4, 16, 4)
 
 
 def decompress24(vals, meta, m, k):
@@ -136,6 +138,16 @@ def decompress24(vals, meta, m, k):
     dense = np.zeros(m * k, dtype=np.uint8)
     assert lib().orc_decompress24(_p(vals), _p(meta), m, k, _p(dense)) == 0
     return dense.reshape(m, k)
+
+
+def plain_to_kblocked(plain, m, k, es=1):
+    """Independent statement of the K-blocked order with array axes instead of offsets: `plain` is (m, bytes per row)
+    with the row's bytes in k order (kept values: k / 2 * es bytes, metadata: k / 8 bytes); a stage is 128 dense bytes
+    of k and splits a row's bytes into 4 equal lane-group pieces."""
+    plain = np.ascontiguousarray(plain).view(np.uint8).reshape(m, -1)
+    stages = k * es // 128
+    piece = plain.shape[1] // stages // 4
+    return plain.reshape(m // 16, 16, stages, 4, piece).transpose(2, 0, 3, 1, 4).copy()
 
 
 # ----------------------------------------------------------------- conversions (vectorised)

@@ -230,3 +230,90 @@ def test_mma_sync_single_tile_matches_oracle(type_id, a_row, b_row, c_row):
             else:
                 ok, mx = O.compare(out_t, got, want, 100.0 if out_t in (O.F16, O.BF16) else 10.0)
                 assert ok, (blk, bk, mx)
+
+
+# ------------------------------------------------------------------ 2:4 sparse fragments (rocwmma_sparse.hpp)
+SPARSE_TYPES = {0: (O.F16, 2), 1: (O.BF16, 2), 2: (O.E4M3, 1), 3: (O.I8, 1), 7: (O.E5M2, 1)}
+
+
+def _sparse_tile(type_id, blk, stages, b_row, c_row, dense, b, c):
+    """dense: (blk, k) storage array with a 2:4 pattern; returns D = A B + C of one tile through the sparse fragment API."""
+    import rocwmma_amd as R
+
+    vals, meta = R.compress_24(dense)
+    assert np.array_equal(R.decompress_24(vals, meta), dense)
+    k = dense.shape[1]
+    acc_dt = np.int32 if type_id == 3 else np.float32
+    dv, dm, db, dc = to_device(vals), to_device(meta), to_device(b), to_device(c)
+    dd = device_filled(blk * blk, acc_dt, 0xFF)
+    rc = api_lib().api_sparse_mma_tile(type_id, blk, stages, b_row, c_row, ctypes.c_void_p(dv.data_ptr()), ctypes.c_void_p(dm.data_ptr()),
+                                       ctypes.c_void_p(db.data_ptr()), ctypes.c_void_p(dc.data_ptr()), ctypes.c_void_p(dd.data_ptr()),
+                                       blk if b_row else k, blk)
+    assert rc == 0, (type_id, blk, stages)
+    return to_host(dd, acc_dt)
+
+
+@pytest.mark.parametrize("type_id", sorted(SPARSE_TYPES))
+@pytest.mark.parametrize("blk,stages", [(16, 1), (16, 2), (32, 1), (32, 2)])
+@pytest.mark.parametrize("b_row,c_row", [(0, 1), (1, 0)])
+def test_sparse_mma_sync_single_tile_matches_dense_oracle(type_id, blk, stages, b_row, c_row):
+    """Random 2:4 operands: the sparse tile equals the oracle's dense GEMM on the decompressed A (int8 bit-exact, fp8
+    1e-2, 16-bit 1e-3 on the reference's metric: same products, another summation order)."""
+    in_t, es = SPARSE_TYPES[type_id]
+    k = stages * 128 // es
+    m = n = blk
+    mask = O.sparse24_mask(20 + type_id, m, k)
+    if in_t == O.I8:
+        a, b = O.uniform_int8(21, m * k).reshape(m, k), O.uniform_int8(22, k * n)
+        c = O.uniform_int8(23, m * n).astype(np.int32) * 100
+        dense = np.where(mask, a, np.int8(0)).astype(np.int8)
+        dec = lambda x: x
+        o_in, o_out = O.I8, O.I32
+    else:
+        if in_t == O.E5M2:  # finite codes with |x| <= 7; decoded exactly through float16
+            rng = np.random.default_rng(5)
+            mk = lambda nel: np.where((rng.integers(0, 0x48, nel) == 0), 1, rng.integers(0, 0x48, nel) | (rng.integers(0, 2, nel) << 7)).astype(np.uint8)
+            a, b = mk(m * k).reshape(m, k), mk(k * n)
+            dec = lambda x: (x.astype(np.uint16) << 8).view(np.float16).astype(np.float32)
+            o_in = O.F32
+        else:
+            src = O.normal if in_t == O.E4M3 else O.uniform_pm1
+            a = O.f32_to_storage(src(21, m * k), in_t).reshape(m, k)
+            b = O.f32_to_storage(src(22, k * n), in_t)
+            dec = lambda x: x
+            o_in = in_t
+        c = O.uniform_pm1(23, m * n)
+        dense = np.where(mask, a, a.dtype.type(0)).astype(a.dtype)
+        o_out = O.F32
+    lb, lc = (O.ROW if b_row else O.COL), (O.ROW if c_row else O.COL)
+    want = O.gemm(o_in, o_out, O.ROW, lb, lc, lc, m, n, k, dec(dense).ravel(), dec(b), c, 1.0, 1.0)
+    got = _sparse_tile(type_id, blk, stages, b_row, c_row, dense, b, c)
+    if in_t == O.I8:
+        assert np.array_equal(got, want)
+    else:
+        g, w = got.astype(np.float64), want.astype(np.float64)
+        tol = 1e-2 if es == 1 else 1e-3
+        assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= tol
+
+
+@pytest.mark.parametrize("type_id,blk", [(3, 16), (3, 32), (0, 16), (0, 32)])
+def test_sparse_mma_sync_one_hot_sweep(type_id, blk):
+    """Every dense position of A in turn holds the only non-zero (row r has it at column (kk + r) % k): D must be the
+    matching rows of B - exact, and wrong for any other pairing of lane groups, index bits or storage offsets."""
+    in_t, es = SPARSE_TYPES[type_id]
+    stages = 2
+    k, m, n = stages * 128 // es, blk, blk
+    if in_t == O.I8:
+        b = ((np.arange(k * n) * 7 + 3) % 251 - 125).astype(np.int8)
+        bf = b.astype(np.int32).reshape(n, k)  # col-major B: bf[col, kk]
+        one, zero_c = np.int8(1), np.zeros(m * n, dtype=np.int32)
+    else:
+        b = O.f32_to_storage(((np.arange(k * n) % 2039) - 1000).astype(np.float32), O.F16)
+        bf = b.view(np.float16).astype(np.float32).reshape(n, k)
+        one, zero_c = np.float16(1.0).view(np.uint16), np.zeros(m * n, dtype=np.float32)
+    for kk in range(k):
+        dense = np.zeros((m, k), dtype=np.int8 if in_t == O.I8 else np.uint16)
+        cols = (kk + np.arange(m)) % k
+        dense[np.arange(m), cols] = one
+        got = _sparse_tile(type_id, blk, stages, 0, 1, dense, b, zero_c).reshape(m, n)
+        assert np.array_equal(got, bf[:, cols].T), kk

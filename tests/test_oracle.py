@@ -294,27 +294,36 @@ def test_compare_closed_forms():
 # ------------------------------------------------------------------ 2:4 format
 
 def test_sparse24_format_invariants():
-    m, k = 16, 64
+    m, k = 32, 256
     mask = O.sparse24_mask(3, m, k)
     assert np.all(mask.reshape(m, k // 4, 4).sum(axis=2) == 2)
     vals_dense = O.uniform_int8(4, m * k).reshape(m, k)
     vals_dense = np.where(vals_dense == 0, np.int8(1), vals_dense)
     dense = np.where(mask, vals_dense, np.int8(0)).astype(np.int8)
     vals, meta = O.compress24(dense.view(np.uint8), m, k)
-    assert vals.shape == (m, k // 2) and meta.shape == (m, k // 8)
-    # indices strictly increasing inside each group and equal to the mask positions
-    for r in range(m):
-        for g in range(k // 4):
-            nib = (meta[r, g // 2] >> (4 * (g % 2))) & 0xF
-            i0, i1 = nib & 3, nib >> 2
-            assert i0 < i1
-            assert list(np.flatnonzero(mask[r, 4 * g : 4 * g + 4])) == [i0, i1]
-            assert vals[r, 2 * g] == dense.view(np.uint8)[r, 4 * g + i0]
+    assert vals.shape == (k // 128, m // 16, 4, 16, 16) and meta.shape == (k // 128, m // 16, 4, 16, 4)
+    # The expected storage from plain numpy: per row, the kept pair of each group in position order and a nibble
+    # idx0 | idx1 << 2 per group (even group in the low nibble), then the K-blocked order by reshaping / transposing
+    grp = dense.view(np.uint8).reshape(m, k // 4, 4)
+    pos = np.argsort(~mask.reshape(m, k // 4, 4), axis=2, kind="stable")[:, :, :2]  # the two kept positions, increasing
+    assert np.all(pos[:, :, 0] < pos[:, :, 1])
+    plain_vals = np.take_along_axis(grp, pos, axis=2).reshape(m, k // 2)
+    nib = (pos[:, :, 0] | (pos[:, :, 1] << 2)).astype(np.uint8)
+    plain_meta = (nib[:, 0::2] | (nib[:, 1::2] << 4)).astype(np.uint8)
+    assert np.array_equal(vals, O.plain_to_kblocked(plain_vals, m, k))
+    assert np.array_equal(meta, O.plain_to_kblocked(plain_meta, m, k))
+    # spot check of one element against the description in words: row 21, dense k 200..203 = stage 1, lane group 2,
+    # its group 2 of 8 -> kept bytes 4, 5 of the lane's 16; the nibble is the low half of index byte 1
+    st, rb, lg, rr = 1, 1, 2, 5
+    assert list(vals[st, rb, lg, rr, 4:6]) == list(plain_vals[21, 100:102])
+    assert (meta[st, rb, lg, rr, 1] & 0xF) == nib[21, 50]
     assert np.array_equal(O.decompress24(vals, meta, m, k), dense.view(np.uint8))
-    # a group with three non-zeros is rejected
+    # a group with three non-zeros is rejected, and so are sizes off the 16 x 128 grid
     bad = dense.copy(); bad[0, :4] = 1
     with pytest.raises(ValueError):
         O.compress24(bad.view(np.uint8), m, k)
+    with pytest.raises(ValueError):
+        O.compress24(dense.view(np.uint8)[:, :64].copy(), m, 64)
     # groups with fewer than two non-zeros still round-trip
     few = dense.copy(); few[1, :8] = 0; few[2, 0:4] = [0, 0, 0, 9]
     v2, m2 = O.compress24(few.view(np.uint8), m, k)

@@ -24,7 +24,8 @@ def _sparse_inputs(in_t, m, n, k, seed):
 
 
 @pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32)])
-@pytest.mark.parametrize("m,n,k", [(32, 32, 64), (96, 64, 256), (256, 128, 1024), (256, 256, 512), (512, 768, 256)])
+@pytest.mark.parametrize("m,n,k", [(32, 32, 128), (16, 48, 128), (96, 64, 256), (256, 128, 1024), (256, 256, 128), (256, 256, 640),
+                                   (512, 768, 384), (256, 512, 896)])
 @pytest.mark.parametrize("ldl", [O.ROW, O.COL])
 def test_sparse_gemm_vs_dense_oracle(in_t, out_t, m, n, k, ldl):
     dense, b = _sparse_inputs(in_t, m, n, k, 40)
@@ -38,7 +39,9 @@ def test_sparse_gemm_vs_dense_oracle(in_t, out_t, m, n, k, ldl):
     R.gemm(in_t, out_t, m, n, k, dv, db, dc, dd, 1.0, 1.0, O.ROW, O.COL, ldl, ldl, a_meta=dm)
     got = to_host(dd, O.NP_STORAGE[out_t])
     plan = R.gemm_query(R.gemm_args(in_t, out_t, m, n, k, dv, db, dc, dd, 1.0, 1.0, O.ROW, O.COL, ldl, ldl, a_meta=dm))
-    assert plan.kernel == (R.KERNEL_TILED if (m % 256 == 0 and n % 256 == 0 and k % 256 == 0) else R.KERNEL_SIMPLE)
+    # the macro tile takes every K that fills whole 128-wide stages (1, 3, 5 and 7 stages above: every remainder of
+    # the six-stage loop trip)
+    assert plan.kernel == (R.KERNEL_TILED if (m % 256 == 0 and n % 256 == 0) else R.KERNEL_SIMPLE)
     if in_t == O.I8:
         assert np.array_equal(got, want)
     else:
@@ -46,27 +49,41 @@ def test_sparse_gemm_vs_dense_oracle(in_t, out_t, m, n, k, ldl):
         assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= 1e-2
 
 
-def test_sparse_config4_sampled_rows():
-    # benchmark configuration 4: M = N = 4096, dense-equivalent K = 8192, int8
+@pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32)])
+def test_sparse_config4_sampled_rows(in_t, out_t):
+    # benchmark configuration 4: M = N = 4096, dense-equivalent K = 8192, int8 and fp8 e4m3
     m, n, k = 4096, 4096, 8192
-    dense, b = _sparse_inputs(O.I8, m, n, k, 60)
+    dense, b = _sparse_inputs(in_t, m, n, k, 60)
     vals, meta = R.compress_24(dense)
     dv, dm, db = to_device(vals), to_device(meta), to_device(b)
-    dd = device_filled(m * n, np.int32, 0xFF)
-    R.gemm(O.I8, O.I32, m, n, k, dv, db, None, dd, 1.0, 0.0, O.ROW, O.COL, O.ROW, O.ROW, a_meta=dm)
-    got = to_host(dd, np.int32).reshape(m, n)
+    dd = device_filled(m * n, O.NP_STORAGE[out_t], 0xFF)
+    R.gemm(in_t, out_t, m, n, k, dv, db, None, dd, 1.0, 0.0, O.ROW, O.COL, O.ROW, O.ROW, a_meta=dm)
+    got = to_host(dd, O.NP_STORAGE[out_t]).reshape(m, n)
     rows = np.array([0, 31, 32, 2047, 4095, 1234], dtype=np.uint32)
-    want = O.gemm_rows(O.I8, O.I32, O.ROW, O.COL, m, n, k, dense.ravel(), b, rows)
-    assert np.array_equal(got[rows], want)
-    B = b.reshape(n, k).astype(np.int64)
-    assert int(got.astype(np.int64).sum()) == int(dense.astype(np.int64).sum(axis=0) @ B.sum(axis=0))
+    storage = dense.view(np.uint8) if in_t == O.E4M3 else dense
+    want = O.gemm_rows(in_t, out_t, O.ROW, O.COL, m, n, k, storage.ravel(), b, rows)
+    if in_t == O.I8:
+        assert np.array_equal(got[rows], want)
+        B = b.reshape(n, k).astype(np.int64)
+        assert int(got.astype(np.int64).sum()) == int(dense.astype(np.int64).sum(axis=0) @ B.sum(axis=0))
+    else:
+        g, w = got[rows].astype(np.float64), want.astype(np.float64)
+        assert np.all(np.isfinite(got))
+        assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= 1e-2
+        # column sums of D against (column sums of A) . B in float64: every element of D takes part
+        A64 = O.storage_to_f32(storage, O.E4M3).astype(np.float64).reshape(m, k)
+        B64 = O.storage_to_f32(b, O.E4M3).astype(np.float64).reshape(n, k)
+        ref = A64.sum(axis=0) @ B64.T
+        scale = np.abs(A64).sum(axis=0) @ np.abs(B64).T
+        assert np.max(np.abs(got.astype(np.float64).sum(axis=0) - ref) / scale) <= 1e-3
 
 
 @pytest.mark.parametrize("in_t", [O.F16, O.BF16])
-@pytest.mark.parametrize("m,n,k", [(32, 32, 32), (96, 64, 96), (256, 128, 1024), (64, 32, 4096)])
+@pytest.mark.parametrize("m,n,k", [(32, 32, 64), (16, 48, 64), (96, 64, 192), (256, 128, 1024), (64, 32, 4096)])
 @pytest.mark.parametrize("ldl", [O.ROW, O.COL])
 def test_sparse_gemm_16bit_vs_dense_oracle(in_t, m, n, k, ldl):
-    """f16 / bf16 operands on v_smfmac_f32_32x32x32_{f16,bf16} (block-per-wave kernel), f32 out.  Same products as the
+    """f16 / bf16 operands on v_smfmac_f32_32x32x32 / 16x16x64_{f16,bf16} (block-per-wave kernel on the sparse fragment
+    API), f32 out.  Same products as the
     oracle's dense GEMM on the decompressed A, summed in another order: the 16-bit bar of 1e-3 on the relative metric."""
     mask = O.sparse24_mask(70, m, k)
     a = O.f32_to_storage(O.uniform_pm1(71, m * k), in_t).reshape(m, k)
@@ -81,7 +98,7 @@ def test_sparse_gemm_16bit_vs_dense_oracle(in_t, m, n, k, ldl):
     R.gemm(in_t, O.F32, m, n, k, dv, db, dc, dd, 2.0, 2.0, O.ROW, O.COL, ldl, ldl, a_meta=dm)
     got = to_host(dd, np.float32)
     plan = R.gemm_query(R.gemm_args(in_t, O.F32, m, n, k, dv, db, dc, dd, 2.0, 2.0, O.ROW, O.COL, ldl, ldl, a_meta=dm))
-    assert plan.kernel == R.KERNEL_SIMPLE and plan.macro_tile_k == 32
+    assert plan.kernel == R.KERNEL_SIMPLE and plan.macro_tile_k == 64
     g, w = got.astype(np.float64), want.astype(np.float64)
     assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= 1e-3
 
@@ -89,7 +106,7 @@ def test_sparse_gemm_16bit_vs_dense_oracle(in_t, m, n, k, ldl):
 def test_sparse_16bit_one_hot_positions():
     """Every (row, kept position) of A in turn is the only non-zero: D must be that row of B scaled - exact, and it
     fails for any wrong pairing of lane groups or index bits."""
-    m, n, k = 32, 32, 64
+    m, n, k = 32, 32, 128
     b = O.f32_to_storage(((np.arange(k * n) % 2039) - 1000).astype(np.float32), O.F16)  # distinct small integers
     bf = b.view(np.float16).astype(np.float32).reshape(n, k)  # col-major B: bf[col, kk]
     db = to_device(b)
@@ -103,3 +120,16 @@ def test_sparse_16bit_one_hot_positions():
         R.gemm(O.F16, O.F32, m, n, k, dv, db, None, dd, 1.0, 0.0, O.ROW, O.COL, O.ROW, O.ROW, a_meta=dm)
         got = to_host(dd, np.float32).reshape(m, n)
         assert np.array_equal(got, bf[:, cols].T), kk
+
+
+def test_sparse_size_and_selector_errors():
+    """Sizes off the storage grid and selectors without a kernel come back as errors, not as silent fallbacks."""
+    g = lambda m, n, k, kernel=R.KERNEL_AUTO, lda=None: R.gemm_args(R.I8, R.I32, m, n, k, 0x1000, 0x2000, None, 0x3000, 1.0, 0.0,
+                                                                  R.ROW_MAJOR, R.COL_MAJOR, R.ROW_MAJOR, R.ROW_MAJOR, a_meta=0x4000,
+                                                                  kernel=kernel, lda=lda)
+    for args, code in ((g(256, 256, 192), -3), (g(24, 256, 128), -3), (g(256, 256, 256, R.KERNEL_TILED_128), -2),
+                       (g(128, 256, 256, R.KERNEL_TILED), -3), (g(256, 256, 256, lda=136), -1)):
+        with pytest.raises(R.R355Error) as e:
+            R.gemm_query(args)
+        assert e.value.code == code
+    assert R.gemm_query(g(256, 256, 128, R.KERNEL_TILED)).macro_tile_k == 128  # k % 128, as the header says
