@@ -28,6 +28,17 @@
 //   (32x32: col = l % 32, row = 8 * (e / 4) + 4 * (l / 32) + e % 4;
 //    16x16: col = l % 16, row = 4 * (l / 16) + e)
 // for every element type, so `fragC.x[i]` and `fragAcc.x[i]` always name the same (row, col).
+//
+// Staging fragments (matrix_a / matrix_b with BlockDim >= 64: the macro-tile buffers of cooperative kernels,
+// which are only loaded and stored, never multiplied) hold vectors along BlockDim instead: a chunk is V = 16 bytes'
+// worth of consecutive BlockDim elements at one k,
+//     BlockDim / V >= 64 :  chunk c, lane l:  k = c / P,  dim = V * (64 * (c % P) + l),   P = BlockDim / V / 64
+//     BlockDim / V <  64 :  chunk c, lane l:  k = c * R + l / (BlockDim / V),  dim = V * (l % (BlockDim / V)),
+//                           R = 64 V / BlockDim k-rows per chunk
+// so that global -> register -> LDS moves of an operand whose BlockDim is the contiguous memory dimension (A
+// col-major, B row-major: the orientation of the reference's perf samples) are 128-bit accesses, and the matrix
+// fragments then come out of such an LDS image with transposing reads (io.hpp).  Like every other layout here it
+// does not depend on the memory orientation: the transforms stay relabels.
 #ifndef ROCWMMA_LAYOUT_HPP
 #define ROCWMMA_LAYOUT_HPP
 
@@ -98,6 +109,23 @@ namespace rocwmma
             return kw;
         }
 
+        // Vector length along BlockDim of a staging fragment; 0: the fragment holds vectors along K
+        template <typename DataT>
+        constexpr inline uint32_t dimVector(uint32_t blockDim, uint32_t kDim, bool input)
+        {
+            if(!input || blockDim < 64u)
+                return 0u;
+            for(uint32_t v = 16u / static_cast<uint32_t>(sizeof(DataT)); v > 1u; v >>= 1)
+            {
+                if(blockDim % v)
+                    continue;
+                const uint32_t lanesPerRow = blockDim / v;
+                if(lanesPerRow >= 64u ? lanesPerRow % 64u == 0u : (64u % lanesPerRow == 0u && kDim % (64u / lanesPerRow) == 0u))
+                    return v;
+            }
+            return 0u;
+        }
+
         template <typename MatrixT, uint32_t BlockM, uint32_t BlockN, uint32_t BlockK, typename DataT>
         struct RegisterLayout
         {
@@ -117,19 +145,27 @@ namespace rocwmma
             static constexpr uint32_t D    = cmin(BlockDim, WaveSize);
             static constexpr uint32_t G    = WaveSize / D;
             static constexpr uint32_t Segs = BlockDim / D;
-            // f64 accumulators follow v_mfma_f64_16x16x4: one row per register, rows G apart
+            // staging fragments: vectors of DimV consecutive BlockDim elements
+            static constexpr uint32_t DimV        = dimVector<DataT>(BlockDim, KDim, !IsAcc);
+            static constexpr bool     VecAlongDim = DimV != 0u;
+            static constexpr uint32_t LanesPerRow = VecAlongDim ? BlockDim / DimV : 1u;
+            static constexpr uint32_t PassesPerRow = LanesPerRow >= WaveSize ? LanesPerRow / WaveSize : 1u;
+            static constexpr uint32_t RowsPerPass  = LanesPerRow >= WaveSize ? 1u : WaveSize / LanesPerRow;
+            // elements per chunk: along K (f64 accumulators follow v_mfma_f64_16x16x4: one row per register, rows G
+            // apart), or along BlockDim for staging fragments
             static constexpr uint32_t KW
-                = IsAcc ? (sizeof(DataT) == 8u ? 1u : 4u)
-                        : inputKW<DataT>(KDim, G, BlockDim == 16u || BlockDim == 32u);
+                = VecAlongDim ? DimV
+                              : (IsAcc ? (sizeof(DataT) == 8u ? 1u : 4u)
+                                       : inputKW<DataT>(KDim, G, BlockDim == 16u || BlockDim == 32u));
 
-            static_assert(KDim % (KW * G) == 0u,
+            static_assert(VecAlongDim || KDim % (KW * G) == 0u,
                           "KDim is not a multiple of the K extent one wave holds per register chunk");
 
             static constexpr uint32_t ElementsPerSeg = KDim / G;
-            static constexpr uint32_t ChunksPerSeg   = ElementsPerSeg / KW;
-            static constexpr uint32_t NumChunks      = Segs * ChunksPerSeg;
+            static constexpr uint32_t ChunksPerSeg   = VecAlongDim ? 1u : ElementsPerSeg / KW;
             static constexpr uint32_t NumElements    = Segs * ElementsPerSeg;
-            static constexpr uint32_t ChunkK         = KW * G; // K extent of one chunk over the wave
+            static constexpr uint32_t NumChunks      = NumElements / KW;
+            static constexpr uint32_t ChunkK         = VecAlongDim ? RowsPerPass : KW * G; // K extent of one chunk over the wave
 
             static_assert(NumElements * sizeof(DataT) >= 4u && (NumElements * sizeof(DataT)) % 4u == 0u,
                           "Fragments must occupy at least one packed register");
@@ -137,11 +173,17 @@ namespace rocwmma
             // (BlockDim index, KDim index) of the first element of chunk c for lane l
             ROCWMMA_DEVICE static inline uint32_t dimOf(uint32_t lane, uint32_t chunk)
             {
-                return (chunk / ChunksPerSeg) * D + lane % D;
+                if constexpr(VecAlongDim)
+                    return DimV * (LanesPerRow >= WaveSize ? WaveSize * (chunk % PassesPerRow) + lane : lane % LanesPerRow);
+                else
+                    return (chunk / ChunksPerSeg) * D + lane % D;
             }
             ROCWMMA_DEVICE static inline uint32_t kOf(uint32_t lane, uint32_t chunk)
             {
-                return (chunk % ChunksPerSeg) * ChunkK + (lane / D) * KW;
+                if constexpr(VecAlongDim)
+                    return LanesPerRow >= WaveSize ? chunk / PassesPerRow : chunk * RowsPerPass + lane / LanesPerRow;
+                else
+                    return (chunk % ChunksPerSeg) * ChunkK + (lane / D) * KW;
             }
             // (row, col) of BlockDim index d and KDim index k
             ROCWMMA_HOST_DEVICE constexpr static inline Coord2d matrixCoord(uint32_t d, uint32_t k)
