@@ -184,6 +184,9 @@ def main():
         "extra": extra,
     }
     print(json.dumps(line))
+    sys.stdout.flush()
+    # leave nothing behind: the OpenMP pool of the oracle and torch's helper threads end with the process
+    os._exit(0)
 
 
 def settle(torch, fn, seconds=0.1):
@@ -275,7 +278,8 @@ def run_extras(R, O, np, torch, args, counters):
     out["same_box_comparison"] = same_box_comparison(torch, args, s, af16, bf16_, abf, bbf, ai8, bi8, af8, bf8)
     # 2:4 sparse, benchmark configuration 4: M = N = 4096, dense-equivalent K = 8192, int8; dense-equivalent ops
     # against the sparse peak (2 x dense).  Every group of 4 keeps 2 values at random positions:
-    # one index nibble idx0 | idx1 << 2 (idx0 < idx1) per group, two groups per metadata byte.
+    # one index nibble idx0 | idx1 << 2 (idx0 < idx1) per group, two groups per metadata byte (in the library's K-blocked
+    # storage any permutation of valid nibbles and values is a valid operand, so both are drawn directly).
     sm, sn, sk = 4096, 4096, 8192
     vals = i8(sm * sk // 2)
     pairs = torch.tensor([0x4, 0x8, 0xC, 0x9, 0xD, 0xE], dtype=torch.uint8, device="cuda")
@@ -283,6 +287,9 @@ def run_extras(R, O, np, torch, args, counters):
     meta = (nib[:, 0] | (nib[:, 1] << 4)).contiguous()
     gemm_case("gemm_i8_sparse24_4096x4096x8192", R.I8, R.I32, R.ROW_MAJOR, R.COL_MAJOR, vals, i8(sk * sn),
               PEAK_TFLOPS["i8"], "TOP/s (dense-equivalent)", sparse_meta=meta, mm=sm, nn=sn, kk=sk, peak_scale=2.0)
+    # the same configuration with fp8 e4m3 operands (f32 result)
+    gemm_case("gemm_e4m3_sparse24_4096x4096x8192", R.E4M3, R.F32, R.ROW_MAJOR, R.COL_MAJOR, f8(sm * sk // 2), f8(sk * sn),
+              PEAK_TFLOPS["e4m3"], "TFLOP/s (dense-equivalent)", sparse_meta=meta, mm=sm, nn=sn, kk=sk, peak_scale=2.0)
     # DLRM dot interaction forward, benchmark configuration 5
     bsz, mm, kk = 65536, 27, 128
     x = torch.randn(bsz * mm * kk, device="cuda").to(torch.float16)

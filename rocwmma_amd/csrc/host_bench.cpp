@@ -298,7 +298,7 @@ int main(int argc, char** argv)
         void *da, *db, *dd, *dmeta = nullptr;
         if(sparse)
         {
-            // compressed A is m x k/2 row-major; one index nibble per group of four dense columns:
+            // compressed A: m * k/2 kept values in the K-blocked storage (any bytes are valid values); one index nibble per group of four dense columns:
             // 0x4 keeps positions (0, 1), 0x8 keeps positions (0, 2)
             g.sparse24 = 1;
             g.lda      = k / 2;

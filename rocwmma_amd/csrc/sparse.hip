@@ -14,16 +14,18 @@
 // B is dense, col-major (k contiguous); D row- or col-major.  m % 16 == 0, k % (128 / ES) == 0.
 //
 // Two kernels:
-//   sparseTiledKernel    256 x 256 macro tile, one 128-wide K step per stage, a ring of three LDS slots filled
-//                        by direct-to-LDS loads two stages ahead (kept values 16 KiB + indices 4 KiB
+//   sparseTiledKernel    256 x 256 macro tile, one K step of 128 bytes per stage, a ring of three LDS slots filled
+//                        by direct-to-LDS loads two stages ahead (kept values 16 KiB + indices 4 or 2 KiB
 //                        + dense B 32 KiB per stage), 2 x 2 waves with 8 x 8 accumulators of
-//                        v_smfmac_*_16x16x128 each (under the board's power limit the register-resident loop of
-//                        this shape sustains 7.5 POP/s against 6.5 for 32x32x64); a stage is split into quadrants of
-//                        the wave tile as in the dense fp8 kernel; the result is transposed through LDS so
-//                        that D leaves in whole rows.
+//                        v_smfmac_*_16x16x128 (int8, e4m3) or v_smfmac_f32_16x16x64 (f16, bf16) each (under the
+//                        board's power limit the register-resident int8 loop of this shape sustains 7.5 POP/s
+//                        against 6.5 for 32x32x64); a stage is split into quadrants of the wave tile as in the
+//                        dense fp8 kernel; the result is transposed through LDS so that D leaves in whole
+//                        rows.  Edge tiles (m, n multiples of 16): rows of A and B beyond the matrix lie outside
+//                        the stage's buffers and load as zeros, the epilogue stores what is inside D.
 //   sparseBlockPerWave   one 16 x 16 or 32 x 32 block of D per wave through the sparse fragment API
 //                        (rocwmma_sparse.hpp) straight from global memory; fallback for shapes that do not fill a
-//                        macro tile, and the only kernel for f16 / bf16.
+//                        macro tile.
 #include <hip/hip_runtime.h>
 
 #include <cstring>
@@ -109,10 +111,10 @@ namespace
     }
 
     // ------------------------------------------------------------------ macro-tile kernel
-    constexpr uint32_t T_M = 256, T_N = 256, T_K = 128; // dense K per stage
+    constexpr uint32_t T_M = 256, T_N = 256, T_K = 128; // dense bytes of K per stage
     constexpr uint32_t T_THREADS   = 256;
     constexpr uint32_t A_BYTES     = T_M * (T_K / 2); // 16 KiB kept values
-    constexpr uint32_t META_BYTES  = T_M * (T_K / 8); // 4 KiB indices
+    constexpr uint32_t META_BYTES  = T_M * (T_K / 8); // 4 KiB indices (2 KiB of them used by 2-byte elements)
     constexpr uint32_t B_BYTES     = T_N * T_K; // 32 KiB dense
     constexpr uint32_t OFF_META    = A_BYTES;
     constexpr uint32_t OFF_B       = A_BYTES + META_BYTES;
@@ -155,22 +157,37 @@ namespace
         int   idx[4];
     };
 
-    template <bool FP8, typename AccV>
+    enum class SpElem
+    {
+        I8,
+        E4M3,
+        F16,
+        BF16
+    };
+
+    template <SpElem E, typename AccV>
     __device__ __forceinline__ void smfmac16(AccV& acc, const i32x4& a, const i32x8& b, int idx)
     {
         // the accumulator is the instruction's destination and addend at once: updated in place, in an AGPR
-        if constexpr(FP8)
+        // (2-byte elements: the index bits are the low half of the register, which is what ABID 0 names)
+        if constexpr(E == SpElem::E4M3)
             asm volatile("v_smfmac_f32_16x16x128_fp8_fp8 %0, %1, %2, %3" : "+a"(acc) : "v"(a), "v"(b), "v"(idx));
-        else
+        else if constexpr(E == SpElem::I8)
             asm volatile("v_smfmac_i32_16x16x128_i8 %0, %1, %2, %3" : "+a"(acc) : "v"(a), "v"(b), "v"(idx));
+        else if constexpr(E == SpElem::F16)
+            asm volatile("v_smfmac_f32_16x16x64_f16 %0, %1, %2, %3" : "+a"(acc) : "v"(a), "v"(b), "v"(idx));
+        else
+            asm volatile("v_smfmac_f32_16x16x64_bf16 %0, %1, %2, %3" : "+a"(acc) : "v"(a), "v"(b), "v"(idx));
     }
 
-    template <bool FP8>
+    template <SpElem E>
     __global__ void __launch_bounds__(T_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
         sparseTiledKernel(TiledParams p)
     {
-        using AccE = std::conditional_t<FP8, float, int>;
-        using AccV = std::conditional_t<FP8, f32x4, i32x4>;
+        constexpr bool     INT = E == SpElem::I8;
+        constexpr uint32_t ES  = (E == SpElem::F16 || E == SpElem::BF16) ? 2u : 1u; // element bytes
+        using AccE = std::conditional_t<INT, int, float>;
+        using AccV = std::conditional_t<INT, i32x4, f32x4>;
         using r355::loadToLds;
 
         __shared__ __attribute__((aligned(1024))) char lds[RING * STAGE_BYTES];
@@ -190,37 +207,45 @@ namespace
         // ---- global -> LDS (per thread, fixed).  LDS chunk L = j * 256 + tid of each operand tile.
         //   kept values / indices: the tile's share of a stage is 16 / 4 KiB of consecutive bytes, copied as they are
         //   dense B: 8 chunks per row, chunk c of row r in slot c ^ ((r >> 1) & 7)
+        //   Edge tiles: the tile's rows of A are the first validM / 16 KiB (values) of its share of a stage and the rows
+        //   of B the first validN * ldb bytes from the tile's first row: each load's buffer ends exactly there, and what
+        //   lies beyond loads as zeros (the raw-buffer range check covers lane offset + scalar offset).
         const uint32_t gOffA = tid * 16u;
         const uint32_t rowB = tid >> 3, slotB = tid & 7u;
-        const uint32_t gOffB = rowB * p.ldb + ((slotB ^ ((rowB >> 1) & 7u)) * 16u), gStepB = 32u * p.ldb;
-        const uint32_t numStages = p.k / T_K;
-        const uint64_t strideV = (uint64_t)p.m * 64u, strideM = (uint64_t)p.m * 16u; // bytes between stages
+        const uint32_t ldbBytes = p.ldb * ES;
+        const uint32_t gOffB = rowB * ldbBytes + ((slotB ^ ((rowB >> 1) & 7u)) * 16u), gStepB = 32u * ldbBytes;
+        const uint32_t numStages = p.k * ES / T_K;
+        const uint64_t strideV = (uint64_t)p.m * 64u, strideM = (uint64_t)p.m * (16u / ES); // bytes between stages
+        // (wave-uniform; the readfirstlane calls only tell the compiler so, which keeps the buffer descriptors in scalar registers)
+        const uint32_t validM = __builtin_amdgcn_readfirstlane(p.m - tm * T_M < T_M ? p.m - tm * T_M : T_M);
+        const uint32_t validN = __builtin_amdgcn_readfirstlane(p.n - tn * T_N < T_N ? p.n - tn * T_N : T_N);
         const uint64_t gA = r355::uniformAddress(p.aVals + (uint64_t)tm * A_BYTES);
-        const uint64_t gM = r355::uniformAddress(p.aMeta + (uint64_t)tm * META_BYTES);
-        const uint64_t gB = r355::uniformAddress(p.b + (uint64_t)tn * T_N * p.ldb);
+        const uint64_t gM = r355::uniformAddress(p.aMeta + (uint64_t)tm * (META_BYTES / ES));
+        const uint64_t gB = r355::uniformAddress(p.b + (uint64_t)tn * T_N * ldbBytes);
         const uint32_t dmaDst = ldsBase + wave * 1024u; // lane l lands at dmaDst + slot + piece + 16 l
 
-        // a buffer over [addr, addr + 2 GiB), or over nothing for a stage past the end
-        auto rsrcOf = [](uint64_t addr, bool valid) {
+        // a buffer of `bytes` bytes at addr, or over nothing for a stage past the end
+        auto rsrcOf = [](uint64_t addr, uint32_t bytes, bool valid) {
             return i32x4{static_cast<int>(static_cast<uint32_t>(addr)), static_cast<int>(static_cast<uint32_t>(addr >> 32) & 0xFFFFu),
-                         valid ? 0x7FFFFFFF : 0, 0x00020000};
+                         static_cast<int>(valid ? bytes : 0u), 0x00020000};
         };
         // load x (0..12) of stage `stage` into the slot at byte `at`: 0..3 kept values, 4 indices, 5..12 dense B
         auto issueLoad = [&](uint32_t stage, uint32_t at, uint32_t x) {
             const bool     valid = stage < numStages;
             const uint32_t st    = valid ? stage : 0u;
             if(x < 4u)
-                loadToLds(rsrcOf(gA + st * strideV, valid), gOffA, x * 4096u, dmaDst + at + x * 4096u);
+                loadToLds(rsrcOf(gA + st * strideV, validM * 64u, valid), gOffA, x * 4096u, dmaDst + at + x * 4096u);
             else if(x == 4u)
-                loadToLds(rsrcOf(gM + st * strideM, valid), gOffA, 0u, dmaDst + at + OFF_META);
-            else // 32 rows of B per load
-                loadToLds(rsrcOf(gB + (uint64_t)st * T_K, valid), gOffB, (x - 5u) * gStepB, dmaDst + at + OFF_B + (x - 5u) * 4096u);
+                loadToLds(rsrcOf(gM + st * strideM, validM * (16u / ES), valid), gOffA, 0u, dmaDst + at + OFF_META);
+            else // 32 rows of B per load; the buffer ends with the tile's last valid row
+                loadToLds(rsrcOf(gB + (uint64_t)st * T_K, validN * ldbBytes - st * T_K, valid), gOffB, (x - 5u) * gStepB,
+                          dmaDst + at + OFF_B + (x - 5u) * 4096u);
         };
 
         // ---- LDS -> registers (per lane, fixed)
         //   block i of A (rows 16 i .. + 15 of the wave's 128): 1 KiB of values in lane order, 256 B of indices
         //   block j of B: row 16 j + t, 16-byte chunks g and 4 + g of the row's 128 bytes
-        const uint32_t rdA = wm * 8192u + lane * 16u, rdM = OFF_META + wm * 2048u + lane * 4u;
+        const uint32_t rdA = wm * 8192u + lane * 16u, rdM = OFF_META + (wm * 2048u + lane * 4u) / ES;
         const uint32_t rB  = wn * 128u + t, swB = (t >> 1) & 7u;
         const uint32_t rdB0 = OFF_B + rB * 128u + ((g ^ swB) * 16u), rdB1 = OFF_B + rB * 128u + (((4u + g) ^ swB) * 16u);
 
@@ -228,7 +253,21 @@ namespace
         auto readA = [&](AGroup& grp, uint32_t at, uint32_t half, uint32_t r) {
             const uint32_t i = 4u * half + (r >> 1);
             if(r & 1u)
-                grp.idx[r >> 1] = *reinterpret_cast<const int*>(lds + at + rdM + i * 256u);
+            {
+                if constexpr(ES == 1u)
+                    grp.idx[r >> 1] = *reinterpret_cast<const int*>(lds + at + rdM + i * 256u);
+                else
+                {
+                    // Only the low 16 bits are index bits (ABID 0); the high half stays undefined on purpose: widening
+                    // the 16-bit value would put a VALU instruction between the LDS read and the matrix instruction,
+                    // and the inline-assembly matrix instructions are invisible to the compiler's hazard handling
+                    // (a VALU write directly followed by a matrix instruction that reads it delivers the old value).
+                    using s16x2 = short __attribute__((ext_vector_type(2)));
+                    s16x2 v;
+                    v[0]            = *reinterpret_cast<const short*>(lds + at + rdM + i * 128u);
+                    grp.idx[r >> 1] = __builtin_bit_cast(int, v);
+                }
+            }
             else
                 grp.v[r >> 1] = *reinterpret_cast<const i32x4*>(lds + at + rdA + i * 1024u);
         };
@@ -264,7 +303,7 @@ namespace
 #pragma unroll
             for(uint32_t n = 0; n < 16; ++n)
             {
-                smfmac16<FP8>(acc[n % 4u][n / 4u], aLo.v[n % 4u], bLo[n / 4u], aLo.idx[n % 4u]);
+                smfmac16<E>(acc[n % 4u][n / 4u], aLo.v[n % 4u], bLo[n / 4u], aLo.idx[n % 4u]);
                 readSlotB(bHi, cur, 1, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -272,7 +311,7 @@ namespace
 #pragma unroll
             for(uint32_t n = 0; n < 16; ++n)
             {
-                smfmac16<FP8>(acc[n % 4u][4u + n / 4u], aLo.v[n % 4u], bHi[n / 4u], aLo.idx[n % 4u]);
+                smfmac16<E>(acc[n % 4u][4u + n / 4u], aLo.v[n % 4u], bHi[n / 4u], aLo.idx[n % 4u]);
                 readSlotA(aHi, cur, 1, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -282,7 +321,7 @@ namespace
 #pragma unroll
             for(uint32_t n = 0; n < 16; ++n)
             {
-                smfmac16<FP8>(acc[4u + n / 4u][4u + n % 4u], aHi.v[n / 4u], bHi[n % 4u], aHi.idx[n / 4u]);
+                smfmac16<E>(acc[4u + n / 4u][4u + n % 4u], aHi.v[n / 4u], bHi[n % 4u], aHi.idx[n / 4u]);
                 readSlotA(aLo, nxt, 0, n);
                 if(n % 3u == 1u && n / 3u < 5u)
                     issueLoad(kt + 3u, cur, n / 3u);
@@ -292,7 +331,7 @@ namespace
 #pragma unroll
             for(uint32_t n = 0; n < 16; ++n)
             {
-                smfmac16<FP8>(acc[4u + n % 4u][n / 4u], aHi.v[n % 4u], bLo[n / 4u], aHi.idx[n % 4u]);
+                smfmac16<E>(acc[4u + n % 4u][n / 4u], aHi.v[n % 4u], bLo[n / 4u], aHi.idx[n % 4u]);
                 readSlotB(bHi, nxt, 0, n);
                 if(n & 1u)
                     issueLoad(kt + 3u, cur, 5u + (n >> 1));
@@ -364,6 +403,8 @@ namespace
                 for(uint32_t j = 0; j < 8; ++j)
                 {
                     const uint32_t row = m0 + 16u * i + 4u * g, col = n0 + 16u * j + t;
+                    if(row >= p.m || col >= p.n) // (m is a multiple of 16: a lane's four rows are inside or outside together)
+                        continue;
                     V4             out;
 #pragma unroll
                     for(uint32_t e = 0; e < 4; ++e)
@@ -404,6 +445,8 @@ namespace
                 const uint32_t L = it * 64u + lane, row = L >> 5, c = L & 31u;
                 V4             v = *reinterpret_cast<const V4*>(wl + row * 512u + ((c ^ (row & 31u)) * 16u));
                 const uint64_t off = (uint64_t)(m0 + 64u * pass + row);
+                if(off >= p.m || n0 + 4u * c >= p.n) // (n is a multiple of 16: a 16-byte chunk is inside or outside D as a whole)
+                    continue;
                 if(beta != static_cast<AccE>(0))
                 {
                     const V4 cv = *reinterpret_cast<const V4*>(p.c + (off * p.ldc + n0) * 4u + c * 16u);
@@ -417,11 +460,14 @@ namespace
         }
     }
 
+    // The macro tile runs any m, n (multiples of 16) and k (whole stages); under AUTO it is taken from half a tile in
+    // each direction on (below that most of its matrix instructions would multiply padding).
     bool tiledOk(const r355_gemm_args& g)
     {
-        return g.kernel != R355_KERNEL_SIMPLE && (g.in_type == R355_I8 || g.in_type == R355_E4M3) && g.m % T_M == 0 && g.n % T_N == 0 && g.k % T_K == 0
-               && g.layout_c == g.layout_d && (g.ldd % 4) == 0 && r355::aligned(g.d, 16)
-               && (g.beta == 0.0 || ((g.ldc % 4) == 0 && r355::aligned(g.c, 16))) && r355::aligned(g.a_meta, 16);
+        const uint32_t es = (g.in_type == R355_F16 || g.in_type == R355_BF16) ? 2u : 1u;
+        const bool     shape = g.kernel == R355_KERNEL_TILED || (g.m >= T_M / 2 && g.n >= T_N / 2);
+        return g.kernel != R355_KERNEL_SIMPLE && shape && g.layout_c == g.layout_d && r355::aligned(g.a_meta, 16)
+               && (uint64_t)g.ldb * es <= (1u << 23);
     }
 
     uint32_t simpleBlock(const r355_gemm_args& g)
@@ -453,17 +499,15 @@ namespace r355
             return fail(R355_ERR_MISALIGNED, "sparse gemm: values, B, C and D need 16-byte alignment (pointers and leading dimensions), metadata 4-byte");
         if(g.kernel == R355_KERNEL_TILED_128)
             return fail(R355_ERR_UNSUPPORTED, "sparse gemm: there is no 128 x 128 sparse macro tile (R355_KERNEL_TILED is 256 x 256)");
-        if(w && g.kernel == R355_KERNEL_TILED)
-            return fail(R355_ERR_UNSUPPORTED, "sparse gemm (macro tile): 1-byte elements only");
         if(g.kernel == R355_KERNEL_TILED && !tiledOk(g))
-            return fail(R355_ERR_BAD_SIZE, "sparse gemm (macro tile): m=%u n=%u must be multiples of 256, k=%u of 128, C/D same orientation and 16-byte aligned", g.m, g.n, g.k);
+            return fail(R355_ERR_UNSUPPORTED, "sparse gemm (macro tile): C and D must share an orientation, metadata 16-byte aligned, ldb below 8 MiB");
         if(plan && tiledOk(g))
         {
             plan->kernel       = R355_KERNEL_TILED;
             plan->macro_tile_m = T_M;
             plan->macro_tile_n = T_N;
-            plan->macro_tile_k = T_K;
-            plan->grid_x       = (((g.m / T_M) * (g.n / T_N) + 7u) / 8u) * 8u;
+            plan->macro_tile_k = T_K / es;
+            plan->grid_x       = ((((g.m + T_M - 1) / T_M) * ((g.n + T_N - 1) / T_N) + 7u) / 8u) * 8u;
             plan->grid_y       = 1;
             plan->block_x      = T_THREADS;
             plan->block_y      = 1;
@@ -516,13 +560,16 @@ namespace r355
             p.c = static_cast<const char*>(g.c), p.d = static_cast<char*>(g.d);
             p.ldb = g.ldb, p.ldc = g.ldc, p.ldd = g.ldd;
             p.alpha = g.alpha, p.beta = g.beta;
-            p.tilesM = g.m / T_M, p.tilesN = g.n / T_N;
+            p.tilesM = (g.m + T_M - 1) / T_M, p.tilesN = (g.n + T_N - 1) / T_N;
             p.dRow = g.layout_d == R355_ROW_MAJOR;
-            const uint32_t grid = ((p.tilesM * p.tilesN + 7u) / 8u) * 8u;
-            if(g.in_type == R355_E4M3)
-                hipLaunchKernelGGL(sparseTiledKernel<true>, dim3(grid), dim3(T_THREADS), 0, stream, p);
-            else
-                hipLaunchKernelGGL(sparseTiledKernel<false>, dim3(grid), dim3(T_THREADS), 0, stream, p);
+            const dim3 grid(((p.tilesM * p.tilesN + 7u) / 8u) * 8u), block(T_THREADS);
+            switch(g.in_type)
+            {
+            case R355_E4M3: hipLaunchKernelGGL(sparseTiledKernel<SpElem::E4M3>, grid, block, 0, stream, p); break;
+            case R355_F16: hipLaunchKernelGGL(sparseTiledKernel<SpElem::F16>, grid, block, 0, stream, p); break;
+            case R355_BF16: hipLaunchKernelGGL(sparseTiledKernel<SpElem::BF16>, grid, block, 0, stream, p); break;
+            default: hipLaunchKernelGGL(sparseTiledKernel<SpElem::I8>, grid, block, 0, stream, p); break;
+            }
             return checkLaunch("sparse gemm (macro tile)");
         }
         switch(g.in_type)

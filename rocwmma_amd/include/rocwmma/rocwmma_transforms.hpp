@@ -6,8 +6,7 @@
 // memory orientation and A / B layouts mirror each other (internal/layout.hpp), so both
 // transforms only relabel the fragment type: the registers are returned unchanged.
 //   transpose : fragment<matrix_a, M, N, K, T, L>  <->  fragment<matrix_b, N, M, K, T, orthogonal(L)>
-//               accumulators swap BlockM / BlockN only when square (their registers then
-//               name the transposed element, which is what an orthogonal layout stores).
+//               (matrix_a and matrix_b only, as in the reference)
 #ifndef ROCWMMA_TRANSFORMS_API_HPP
 #define ROCWMMA_TRANSFORMS_API_HPP
 

@@ -25,7 +25,7 @@ def _sparse_inputs(in_t, m, n, k, seed):
 
 @pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32)])
 @pytest.mark.parametrize("m,n,k", [(32, 32, 128), (16, 48, 128), (96, 64, 256), (256, 128, 1024), (256, 256, 128), (256, 256, 640),
-                                   (512, 768, 384), (256, 512, 896)])
+                                   (512, 768, 384), (256, 512, 896), (272, 400, 256), (144, 368, 384), (528, 128, 128)])
 @pytest.mark.parametrize("ldl", [O.ROW, O.COL])
 def test_sparse_gemm_vs_dense_oracle(in_t, out_t, m, n, k, ldl):
     dense, b = _sparse_inputs(in_t, m, n, k, 40)
@@ -39,9 +39,9 @@ def test_sparse_gemm_vs_dense_oracle(in_t, out_t, m, n, k, ldl):
     R.gemm(in_t, out_t, m, n, k, dv, db, dc, dd, 1.0, 1.0, O.ROW, O.COL, ldl, ldl, a_meta=dm)
     got = to_host(dd, O.NP_STORAGE[out_t])
     plan = R.gemm_query(R.gemm_args(in_t, out_t, m, n, k, dv, db, dc, dd, 1.0, 1.0, O.ROW, O.COL, ldl, ldl, a_meta=dm))
-    # the macro tile takes every K that fills whole 128-wide stages (1, 3, 5 and 7 stages above: every remainder of
-    # the six-stage loop trip)
-    assert plan.kernel == (R.KERNEL_TILED if (m % 256 == 0 and n % 256 == 0) else R.KERNEL_SIMPLE)
+    # the macro tile takes every K that fills whole 128-wide stages (1 .. 8 stages above: every remainder of the
+    # six-stage loop trip) and, from half a tile in each direction on, any m and n (edge tiles)
+    assert plan.kernel == (R.KERNEL_TILED if (m >= 128 and n >= 128) else R.KERNEL_SIMPLE)
     if in_t == O.I8:
         assert np.array_equal(got, want)
     else:
@@ -79,11 +79,12 @@ def test_sparse_config4_sampled_rows(in_t, out_t):
 
 
 @pytest.mark.parametrize("in_t", [O.F16, O.BF16])
-@pytest.mark.parametrize("m,n,k", [(32, 32, 64), (16, 48, 64), (96, 64, 192), (256, 128, 1024), (64, 32, 4096)])
+@pytest.mark.parametrize("m,n,k", [(32, 32, 64), (16, 48, 64), (96, 64, 192), (256, 128, 1024), (64, 32, 4096), (256, 256, 448),
+                                   (272, 144, 320), (512, 256, 64)])
 @pytest.mark.parametrize("ldl", [O.ROW, O.COL])
 def test_sparse_gemm_16bit_vs_dense_oracle(in_t, m, n, k, ldl):
     """f16 / bf16 operands on v_smfmac_f32_32x32x32 / 16x16x64_{f16,bf16} (block-per-wave kernel on the sparse fragment
-    API), f32 out.  Same products as the
+    API, and the macro-tile kernel from 128 x 128 on), f32 out.  Same products as the
     oracle's dense GEMM on the decompressed A, summed in another order: the 16-bit bar of 1e-3 on the relative metric."""
     mask = O.sparse24_mask(70, m, k)
     a = O.f32_to_storage(O.uniform_pm1(71, m * k), in_t).reshape(m, k)
@@ -98,7 +99,7 @@ def test_sparse_gemm_16bit_vs_dense_oracle(in_t, m, n, k, ldl):
     R.gemm(in_t, O.F32, m, n, k, dv, db, dc, dd, 2.0, 2.0, O.ROW, O.COL, ldl, ldl, a_meta=dm)
     got = to_host(dd, np.float32)
     plan = R.gemm_query(R.gemm_args(in_t, O.F32, m, n, k, dv, db, dc, dd, 2.0, 2.0, O.ROW, O.COL, ldl, ldl, a_meta=dm))
-    assert plan.kernel == R.KERNEL_SIMPLE and plan.macro_tile_k == 64
+    assert plan.kernel == (R.KERNEL_TILED if (m >= 128 and n >= 128) else R.KERNEL_SIMPLE) and plan.macro_tile_k == 64
     g, w = got.astype(np.float64), want.astype(np.float64)
     assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= 1e-3
 
@@ -128,8 +129,42 @@ def test_sparse_size_and_selector_errors():
                                                                   R.ROW_MAJOR, R.COL_MAJOR, R.ROW_MAJOR, R.ROW_MAJOR, a_meta=0x4000,
                                                                   kernel=kernel, lda=lda)
     for args, code in ((g(256, 256, 192), -3), (g(24, 256, 128), -3), (g(256, 256, 256, R.KERNEL_TILED_128), -2),
-                       (g(128, 256, 256, R.KERNEL_TILED), -3), (g(256, 256, 256, lda=136), -1)):
+                       (g(256, 256, 256, lda=136), -1)):
         with pytest.raises(R.R355Error) as e:
             R.gemm_query(args)
         assert e.value.code == code
     assert R.gemm_query(g(256, 256, 128, R.KERNEL_TILED)).macro_tile_k == 128  # k % 128, as the header says
+    assert R.gemm_query(g(48, 64, 128, R.KERNEL_TILED)).kernel == R.KERNEL_TILED  # forced: any m, n multiple of 16
+    assert R.gemm_query(g(48, 64, 128)).kernel == R.KERNEL_SIMPLE
+
+
+@pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.F16, O.F32)])
+def test_sparse_macro_tile_forced_on_small_and_ragged_shapes(in_t, out_t):
+    """R355_KERNEL_TILED on shapes far below a tile and off the tile grid: rows of A and B beyond the matrix load as zeros
+    and nothing outside D is written (the output sits between two guard regions)."""
+    for m, n, k in ((16, 16, 256), (48, 272, 128), (304, 80, 384)):
+        es = 1 if in_t == O.I8 else 2
+        k = k // es
+        mask = O.sparse24_mask(80, m, k)
+        if in_t == O.I8:
+            a, b = O.uniform_int8(81, m * k).reshape(m, k), O.uniform_int8(82, k * n)
+            dense = np.where(mask, a, np.int8(0)).astype(np.int8)
+        else:
+            a = O.f32_to_storage(O.uniform_pm1(81, m * k), in_t).reshape(m, k)
+            b = O.f32_to_storage(O.uniform_pm1(82, k * n), in_t)
+            dense = np.where(mask, a, np.uint16(0)).astype(np.uint16)
+        vals, meta = R.compress_24(dense)
+        want = O.gemm(in_t, out_t, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, dense.ravel(), b, None, 1.0, 0.0)
+        dv, dm, db = to_device(vals), to_device(meta), to_device(b)
+        guard = 4096
+        dd = device_filled(m * n + 2 * guard, O.NP_STORAGE[out_t], 0xEE)
+        # (device_filled hands back a byte tensor: the slice offset is in bytes)
+        R.gemm(in_t, out_t, m, n, k, dv, db, None, dd[guard * 4:], 1.0, 0.0, O.ROW, O.COL, O.ROW, O.ROW, a_meta=dm, kernel=R.KERNEL_TILED)
+        full = to_host(dd, O.NP_STORAGE[out_t])
+        assert np.all(full[:guard].view(np.uint32) == np.uint32(0xEEEEEEEE)) and np.all(full[guard + m * n:].view(np.uint32) == np.uint32(0xEEEEEEEE))
+        got = full[guard:guard + m * n]
+        if in_t == O.I8:
+            assert np.array_equal(got, want), (m, n, k)
+        else:
+            g, w = got.astype(np.float64), want.astype(np.float64)
+            assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= 1e-3, (m, n, k)
