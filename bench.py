@@ -185,8 +185,6 @@ def main():
     }
     print(json.dumps(line))
     sys.stdout.flush()
-    # leave nothing behind: the OpenMP pool of the oracle and torch's helper threads end with the process
-    os._exit(0)
 
 
 def settle(torch, fn, seconds=0.1):

@@ -10,6 +10,8 @@
 //   host_bench dlrm  [--type f16|bf16|f32] [--bwd 1] [--batch B --m M --k K] [--warmup W --iters I]
 //   host_bench gemv  [--m M --k K --layout n|t]
 //   host_bench copy  [--bytes N]      plain device copy of known size (counter calibration)
+//   host_bench lds   [--iters I]      LDS read instructions from fixed conflict-free addresses with 4, 2 and 1 waves per CU:
+//                                     shader clocks per wave-level read and bytes per clock per CU
 //   host_bench mfma  [--iters I]      register-resident MFMA loops, one wave per SIMD, 16 independent
 //                                     accumulators: the rate the matrix cores sustain under the board's
 //                                     power limit with all-zero and with random operands
@@ -217,6 +219,91 @@ namespace
         }
     }
 
+    // LDS read rate with nothing else in the loop: 16 reads per trip from fixed addresses (consecutive lanes,
+    // consecutive pieces: conflict-free), 8 always in flight.  MODE: 0 ds_read_b128, 1 ds_read_b64, 2 ds_read_b64_tr_b16,
+    // 3 ds_read_b32, 4 ds_read_b64_tr_b8.
+#define R355_RD8(OP, R0, OFFB)                                                                                          \
+    asm volatile(OP " %0, %8 offset:" #OFFB "+0\n\t" OP " %1, %8 offset:" #OFFB "+2048\n\t" OP " %2, %8 offset:" #OFFB      \
+                    "+4096\n\t" OP " %3, %8 offset:" #OFFB "+6144\n\t" OP " %4, %8 offset:" #OFFB "+8192\n\t" OP          \
+                    " %5, %8 offset:" #OFFB "+10240\n\t" OP " %6, %8 offset:" #OFFB "+12288\n\t" OP " %7, %8 offset:" #OFFB \
+                    "+14336\n\t"                                                                                        \
+                 : "=v"(R0[0]), "=v"(R0[1]), "=v"(R0[2]), "=v"(R0[3]), "=v"(R0[4]), "=v"(R0[5]), "=v"(R0[6]), "=v"(R0[7])  \
+                 : "v"(addr))
+    using i32x2 = int __attribute__((ext_vector_type(2)));
+    template <int MODE>
+    __global__ void __launch_bounds__(256) ldsReadLoop(int* out, int iters, unsigned long long* cyc)
+    {
+        __shared__ __attribute__((aligned(16))) char lds[65536];
+        const int t = threadIdx.x;
+        for(int i = t; i < 65536 / 4; i += blockDim.x)
+            reinterpret_cast<int*>(lds)[i] = i;
+        __syncthreads();
+        const uint32_t           addr = (MODE == 0 ? t * 16 : (MODE == 3 ? t * 4 : t * 8)) & 2047;
+        const unsigned long long c0   = __builtin_readcyclecounter();
+        int                      s    = 0;
+        if constexpr(MODE == 0)
+        {
+            i32x4 x[8], y[8];
+            for(int it = 0; it < iters; ++it)
+            {
+                R355_RD8("ds_read_b128", x, 0);
+                asm volatile("s_waitcnt lgkmcnt(8)");
+                R355_RD8("ds_read_b128", y, 16384);
+                asm volatile("s_waitcnt lgkmcnt(8)");
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)");
+            for(int i = 0; i < 8; ++i)
+                s ^= x[i][0] ^ y[i][3];
+        }
+        else if constexpr(MODE == 3)
+        {
+            int x[8], y[8];
+            for(int it = 0; it < iters; ++it)
+            {
+                R355_RD8("ds_read_b32", x, 0);
+                asm volatile("s_waitcnt lgkmcnt(8)");
+                R355_RD8("ds_read_b32", y, 16384);
+                asm volatile("s_waitcnt lgkmcnt(8)");
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)");
+            for(int i = 0; i < 8; ++i)
+                s ^= x[i] ^ y[i];
+        }
+        else
+        {
+            i32x2 x[8], y[8];
+            for(int it = 0; it < iters; ++it)
+            {
+                if constexpr(MODE == 1)
+                {
+                    R355_RD8("ds_read_b64", x, 0);
+                    asm volatile("s_waitcnt lgkmcnt(8)");
+                    R355_RD8("ds_read_b64", y, 16384);
+                }
+                else if constexpr(MODE == 2)
+                {
+                    R355_RD8("ds_read_b64_tr_b16", x, 0);
+                    asm volatile("s_waitcnt lgkmcnt(8)");
+                    R355_RD8("ds_read_b64_tr_b16", y, 16384);
+                }
+                else
+                {
+                    R355_RD8("ds_read_b64_tr_b8", x, 0);
+                    asm volatile("s_waitcnt lgkmcnt(8)");
+                    R355_RD8("ds_read_b64_tr_b8", y, 16384);
+                }
+                asm volatile("s_waitcnt lgkmcnt(8)");
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)");
+            for(int i = 0; i < 8; ++i)
+                s ^= x[i][0] ^ y[i][1];
+        }
+        const unsigned long long c1 = __builtin_readcyclecounter();
+        out[blockIdx.x * 256 + t]   = s;
+        if(t == 0 && blockIdx.x == 0)
+            cyc[0] = c1 - c0;
+    }
+
     __global__ void copyKernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n)
     {
         for(size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
@@ -228,7 +315,7 @@ int main(int argc, char** argv)
 {
     if(argc < 2)
     {
-        fprintf(stderr, "usage: host_bench gemm|dlrm|gemv|copy|mfma [options]\n");
+        fprintf(stderr, "usage: host_bench gemm|dlrm|gemv|copy|mfma|lds [options]\n");
         return 2;
     }
     const std::string op = argv[1];
@@ -465,6 +552,42 @@ int main(int argc, char** argv)
                 printf("%s\n {\"op\": \"mfma\", \"instr\": \"%s\", \"operands\": \"%s\", \"ms\": %.3f, \"tflops\": %.1f, "
                        "\"frac_vendor_peak\": %.4f}",
                        (random || kind) ? "," : "", names[kind], random ? "random" : "zero", ms, tf, tf / vendorPeak[kind]);
+            }
+        printf("\n]\n");
+    }
+    else if(op == "lds")
+    {
+        // wave-level read instructions per shader clock and bytes per clock per CU, with 4, 2 and 1 waves per CU reading
+        int*                out;
+        unsigned long long* cyc;
+        HIP_OK(hipMalloc(&out, (size_t)dev.compute_units * 256 * sizeof(int)));
+        HIP_OK(hipMalloc(&cyc, 64));
+        const int          loops   = itersSet ? iters : 4000;
+        static const char* names[] = {"ds_read_b128", "ds_read_b64", "ds_read_b64_tr_b16", "ds_read_b32", "ds_read_b64_tr_b8"};
+        static const int   width[] = {16, 8, 8, 4, 8};
+        printf("[");
+        for(int waves = 4; waves >= 1; waves /= 2)
+            for(int mode = 0; mode < 5; ++mode)
+            {
+                for(int rep = 0; rep < 2; ++rep)
+                {
+                    const dim3 g(dev.compute_units), b(64 * waves);
+                    switch(mode)
+                    {
+                    case 0: hipLaunchKernelGGL(ldsReadLoop<0>, g, b, 0, 0, out, loops, cyc); break;
+                    case 1: hipLaunchKernelGGL(ldsReadLoop<1>, g, b, 0, 0, out, loops, cyc); break;
+                    case 2: hipLaunchKernelGGL(ldsReadLoop<2>, g, b, 0, 0, out, loops, cyc); break;
+                    case 3: hipLaunchKernelGGL(ldsReadLoop<3>, g, b, 0, 0, out, loops, cyc); break;
+                    default: hipLaunchKernelGGL(ldsReadLoop<4>, g, b, 0, 0, out, loops, cyc); break;
+                    }
+                    HIP_OK(hipDeviceSynchronize());
+                }
+                unsigned long long clocks = 0;
+                HIP_OK(hipMemcpy(&clocks, cyc, 8, hipMemcpyDeviceToHost));
+                const double reads = 16.0 * loops * waves; // wave-level instructions per CU
+                printf("%s\n {\"op\": \"lds\", \"instr\": \"%s\", \"waves_per_cu\": %d, \"clocks_per_wave_read\": %.2f, "
+                       "\"bytes_per_clock_per_cu\": %.1f}",
+                       (waves == 4 && mode == 0) ? "" : ",", names[mode], waves, clocks / reads, reads * 64 * width[mode] / clocks);
             }
         printf("\n]\n");
     }
