@@ -235,20 +235,28 @@ def run_extras(R, O, np, torch, args, counters):
         t = (torch.rand(nel, device="cuda") * 2 - 1)
         return t.to(torch.bfloat16 if bf else torch.float16)
 
-    def gemm_case(name, in_t, out_t, la, lb, a, b, peak, unit, sparse_meta=None, mm=s, nn=s, kk=s, peak_scale=1.0):
+    def gemm_case(name, in_t, out_t, la, lb, a, b, peak, unit, sparse_meta=None, mm=s, nn=s, kk=s, peak_scale=1.0, workspace=None):
         d = torch.empty(mm * nn * R.DTYPE_BYTES[out_t], dtype=torch.uint8, device="cuda")
         g = R.gemm_args(in_t, out_t, mm, nn, kk, a, b, None, d, 1.0, 0.0, la, lb, R.ROW_MAJOR, R.ROW_MAJOR,
-                        a_meta=sparse_meta)
+                        a_meta=sparse_meta, workspace=workspace)
         settle(torch, lambda: R.lib().r355_gemm(ctypes.byref(g), None))
         ms = R.gemm_timed(g, args.warmup, args.steps)
         tf = 2.0 * mm * nn * kk / ms / 1e9
         out[name] = with_counters(name, {"ms": round(ms, 4), "value": round(tf, 2), "unit": unit, "peak": peak * peak_scale,
                                          "frac": round(tf / (peak * peak_scale), 4),
                                          "validated": sampled_ok(in_t, out_t, la, lb, mm, nn, kk, a, b, d, sparse_meta)})
+        if workspace is not None:  # split-K: the same problem with one workgroup per tile beside it
+            out[name]["split_k"] = R.gemm_query(g).split_k
+            g1 = R.gemm_args(in_t, out_t, mm, nn, kk, a, b, None, d, 1.0, 0.0, la, lb, R.ROW_MAJOR, R.ROW_MAJOR)
+            out[name]["ms_without_workspace"] = round(R.gemm_timed(g1, args.warmup, args.steps), 4)
 
     if s == 8192:  # a problem with too few 256 x 256 tiles for the 256 CUs: the 128 x 128 macro tile
         gemm_case("gemm_f16_nt_2048x2048x8192", R.F16, R.F16, R.COL_MAJOR, R.ROW_MAJOR, rnd16(2048 * s, False),
                   rnd16(s * 2048, False), PEAK_TFLOPS["f16"], "TFLOP/s", mm=2048, nn=2048, kk=s)
+    if s == 8192:  # few tiles and a long K: split-K over a caller-provided workspace (16 tiles of 128 x 128 x 16 shares of K)
+        gemm_case("gemm_f16_nt_splitk_512x512x32768", R.F16, R.F16, R.COL_MAJOR, R.ROW_MAJOR, rnd16(512 * 32768, False),
+                  rnd16(32768 * 512, False), PEAK_TFLOPS["f16"], "TFLOP/s", mm=512, nn=512, kk=32768,
+                  workspace=torch.empty(32 * 512 * 512 * 4, dtype=torch.uint8, device="cuda"))
     if s == 8192:  # the reference perf sample's default size (samples/perf_hgemm.cpp:945): 784 tiles of 256 x 256 = 3 rounds
         # on 256 CUs + 16 tiles, which run on 128 x 128 tiles in a second launch (mixed tiling)
         # (f32 output: a kernel instantiation of its own, so that a kernel trace of this run keeps the headline's rows apart)

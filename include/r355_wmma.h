@@ -61,8 +61,11 @@ typedef enum
     R355_KERNEL_TILED  = 2, /* LDS-staged 256 x 256 macro tile (m, n multiples of 16; k of 8 for 16-bit, 16 for 8-bit operands)
                                (samples/perf_hgemm.cpp:515-711,
                                 test/gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp:52-283) */
-    R355_KERNEL_TILED_128 = 3 /* the same kernels with a 128 x 128 macro tile (the only one for f64): what AUTO
+    R355_KERNEL_TILED_128 = 3, /* the same kernels with a 128 x 128 macro tile (the only one for f64): what AUTO
                                picks when the 256 x 256 tiles of a problem would leave most CUs idle */
+    R355_KERNEL_TILED_128_SPLITK = 4 /* 128 x 128 tiles with K split over several workgroups per tile and a reduction
+                               (needs `workspace`; what AUTO picks for few tiles and a long K when a workspace is given).
+                               No counterpart in the reference. */
 } r355_gemm_kernel;
 
 /*
@@ -99,6 +102,14 @@ typedef struct
     int32_t     sparse24;
     const void* a_meta;
     int32_t     kernel; /* r355_gemm_kernel */
+    /* Optional device scratch for split-K (dense GEMM only): problems whose 128 x 128 tiles would occupy at most half of
+     * the CUs while k spans at least 16 stages of 128 bytes run `split_k` workgroups per tile, each over its own range of
+     * K, into workspace[split][m][n] (accumulator type: 4 bytes, f64: 8), followed by a reduction kernel that adds the
+     * partial results in split order and applies alpha, beta and C.  r355_gemm_query reports split_k and the bytes it
+     * needs for the workspace_bytes offered (offer UINT64_MAX to learn the size).  NULL / too small: no split.
+     * The library never allocates; calls that share a workspace must not overlap. */
+    void*       workspace;
+    uint64_t    workspace_bytes;
 } r355_gemm_args;
 
 /* Replaces: hipExtLaunchKernelGGL(gemm_rocwmma_d, ...) in samples/perf_hgemm.cpp:820-842 and
@@ -116,6 +127,8 @@ typedef struct
     uint32_t macro_tile_m, macro_tile_n, macro_tile_k;
     uint32_t grid_x, grid_y, block_x, block_y;
     uint32_t lds_bytes;
+    uint32_t split_k;         /* workgroups per tile along K (1: no split) */
+    uint64_t workspace_bytes; /* bytes of `workspace` the plan uses (0 without split-K) */
 } r355_gemm_plan;
 int r355_gemm_query(const r355_gemm_args* args, r355_gemm_plan* plan);
 

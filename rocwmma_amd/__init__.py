@@ -19,7 +19,7 @@ F16, BF16, E4M3, I8, F32, I32, F64, E5M2 = range(8)
 # r355_layout
 ROW_MAJOR, COL_MAJOR = 0, 1
 # r355_gemm_kernel
-KERNEL_AUTO, KERNEL_SIMPLE, KERNEL_TILED, KERNEL_TILED_128 = 0, 1, 2, 3
+KERNEL_AUTO, KERNEL_SIMPLE, KERNEL_TILED, KERNEL_TILED_128, KERNEL_TILED_128_SPLITK = 0, 1, 2, 3, 4
 
 DTYPE_BYTES = {F16: 2, BF16: 2, E4M3: 1, I8: 1, F32: 4, I32: 4, F64: 8, E5M2: 1}
 
@@ -47,6 +47,7 @@ class GemmArgs(ctypes.Structure):
         ("alpha", ctypes.c_double), ("beta", ctypes.c_double),
         ("sparse24", ctypes.c_int32), ("a_meta", ctypes.c_void_p),
         ("kernel", ctypes.c_int32),
+        ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_uint64),
     ]
 
 
@@ -57,6 +58,7 @@ class GemmPlan(ctypes.Structure):
         ("grid_x", ctypes.c_uint32), ("grid_y", ctypes.c_uint32),
         ("block_x", ctypes.c_uint32), ("block_y", ctypes.c_uint32),
         ("lds_bytes", ctypes.c_uint32),
+        ("split_k", ctypes.c_uint32), ("workspace_bytes", ctypes.c_uint64),
     ]
 
 
@@ -132,7 +134,7 @@ def default_ld(rows, cols, layout):
 
 
 def gemm_args(in_type, out_type, m, n, k, a, b, c, d, alpha, beta, layout_a, layout_b, layout_c, layout_d,
-              lda=None, ldb=None, ldc=None, ldd=None, kernel=KERNEL_AUTO, a_meta=None):
+              lda=None, ldb=None, ldc=None, ldd=None, kernel=KERNEL_AUTO, a_meta=None, workspace=None, workspace_bytes=None):
     sparse = a_meta is not None
     g = GemmArgs()
     g.in_type, g.out_type = in_type, out_type
@@ -146,15 +148,19 @@ def gemm_args(in_type, out_type, m, n, k, a, b, c, d, alpha, beta, layout_a, lay
     g.alpha, g.beta = alpha, beta
     g.sparse24, g.a_meta = int(sparse), _ptr(a_meta)
     g.kernel = kernel
+    g.workspace = _ptr(workspace)
+    if workspace_bytes is None:
+        workspace_bytes = workspace.numel() * workspace.element_size() if hasattr(workspace, "numel") else 0
+    g.workspace_bytes = workspace_bytes
     return g
 
 
 def gemm(in_type, out_type, m, n, k, a, b, c, d, alpha=1.0, beta=0.0, layout_a=ROW_MAJOR, layout_b=COL_MAJOR,
          layout_c=ROW_MAJOR, layout_d=ROW_MAJOR, lda=None, ldb=None, ldc=None, ldd=None, kernel=KERNEL_AUTO,
-         a_meta=None, stream=None):
+         a_meta=None, stream=None, workspace=None):
     """D = alpha * A * B + beta * C on device buffers; asynchronous on `stream`."""
     g = gemm_args(in_type, out_type, m, n, k, a, b, c, d, alpha, beta, layout_a, layout_b, layout_c, layout_d,
-                  lda, ldb, ldc, ldd, kernel, a_meta)
+                  lda, ldb, ldc, ldd, kernel, a_meta, workspace)
     _check(lib().r355_gemm(ctypes.byref(g), _stream_handle(stream)))
 
 

@@ -70,7 +70,13 @@ namespace r355
         // the launch covers tile indices [tileFirst, tileFirst + tileCount) of the tilesM x tilesN walk; with
         // tileQuad the walk is over tiles of twice the kernel's edge, four workgroups each (tile_map.hpp)
         uint32_t tileFirst, tileCount, tileQuad;
+        // split-K (128 x 128 tile kernels): workgroup row blockIdx.y multiplies K stages [y * splitStages, (y + 1) * splitStages)
+        // and writes its partial D (in the accumulator type) at d + y * splitStrideD bytes; 0 = the whole K in one workgroup
+        uint32_t splitStages;
+        uint64_t splitStrideD;
     };
+    // sum of `splits` partial results (accumulator type: f32, i32 or f64) + the alpha / beta epilogue into the output type
+    int splitKReduce(const r355_gemm_args& g, const GemmTileParams& p, uint32_t splits, hipStream_t stream);
     // launch of one kernel family; aK / bK: operand is K-contiguous; tile: 256 or 128
     int gemmTiledPart0(const r355_gemm_args& g, bool aK, bool bK, uint32_t tile, const GemmTileParams& p, hipStream_t s);
     int gemmTiledPart1(const r355_gemm_args& g, bool aK, bool bK, uint32_t tile, const GemmTileParams& p, hipStream_t s);
@@ -146,6 +152,25 @@ namespace
     };
 
     using Params = r355::GemmTileParams;
+
+    // The share of a split-K workgroup row: operands advanced to its first K stage, k cut to its stages, D pointed at its
+    // partial result.  kStage: bytes between K stages of A / B (128 for a K-contiguous operand, 128 rows of ld otherwise).
+    template <uint32_t ES>
+    __device__ __forceinline__ Params splitShare(const Params& in, uint64_t kStageA, uint64_t kStageB)
+    {
+        Params p = in;
+        if(in.splitStages != 0u)
+        {
+            const uint32_t y = blockIdx.y, first = y * in.splitStages; // first K stage of this share
+            p.a += first * kStageA;
+            p.b += first * kStageB;
+            const uint32_t kFirst = first * (STAGE_KB / ES); // elements
+            const uint32_t kShare = in.splitStages * (STAGE_KB / ES);
+            p.k = in.k - kFirst < kShare ? in.k - kFirst : kShare;
+            p.d += y * in.splitStrideD;
+        }
+        return p;
+    }
 
     // ------------------------------------------------------------------------------------------
     // f16 / bf16 on v_mfma_f32_16x16x32_{f16,bf16}.
@@ -846,12 +871,15 @@ namespace
     }
 
     template <Elem E, typename OutT, bool A_KCONTIG, bool B_KCONTIG, uint32_t WB>
-    __device__ __forceinline__ void gemmTiled5(const Params& p)
+    __device__ __forceinline__ void gemmTiled5(const Params& whole)
     {
         static_assert(WB == 8 || WB == 4, "wave tile of 8 x 8 or 4 x 4 blocks");
         static_assert(E != Elem::F64 || WB == 4, "f64 accumulators of an 8 x 8 wave tile would need 512 registers");
         static_assert(E != Elem::E4M3 && E != Elem::E5M2, "fp8 has its own stage structure");
         constexpr uint32_t ES = ElemTraits<E>::Bytes;
+        // split-K: this workgroup row's share of K (the whole problem when splitStages is 0)
+        const Params p = splitShare<ES>(whole, A_KCONTIG ? (uint64_t)STAGE_KB : (uint64_t)STAGE_KB * whole.lda,
+                                        B_KCONTIG ? (uint64_t)STAGE_KB : (uint64_t)STAGE_KB * whole.ldb);
         using AccV            = std::conditional_t<E == Elem::I8, i32x4v, std::conditional_t<E == Elem::F64, f64x4, f32x4>>;
         constexpr uint32_t TILE = 32u * WB, WT = 16u * WB; // macro tile and wave tile edge
         constexpr uint32_t OPER = TILE * STAGE_KB; // bytes of one operand per stage: 32 or 16 KiB
@@ -1102,9 +1130,11 @@ namespace
     }
 
     template <bool E5M2, bool A_KCONTIG, bool B_KCONTIG, uint32_t WB>
-    __device__ __forceinline__ void gemmTiledF8(const Params& p)
+    __device__ __forceinline__ void gemmTiledF8(const Params& whole)
     {
         static_assert(WB == 8 || WB == 4, "wave tile of 8 x 8 or 4 x 4 blocks");
+        const Params p = splitShare<1u>(whole, A_KCONTIG ? (uint64_t)STAGE_KB : (uint64_t)STAGE_KB * whole.lda,
+                                        B_KCONTIG ? (uint64_t)STAGE_KB : (uint64_t)STAGE_KB * whole.ldb);
         constexpr uint32_t TILE = 32u * WB, WT = 16u * WB; // macro tile and wave tile edge
         constexpr uint32_t OPER = TILE * STAGE_KB; // bytes of one operand per stage: 32 or 16 KiB
         constexpr uint32_t H = WB / 2u, NQ = H * H; // blocks per operand group, matrix instructions per quadrant
@@ -1313,7 +1343,8 @@ namespace
     int launchLayouts(bool aK, bool bK, uint32_t tile, const Params& p, hipStream_t stream)
     {
         // every XCD gets ceil(count / 8) tile indices (four workgroups each in a quad launch)
-        const dim3 grid(((p.tileCount + 7u) / 8u) * 8u * (p.tileQuad ? 4u : 1u)), block(THREADS);
+        const uint32_t splits = p.splitStages ? ((p.k * ElemTraits<E>::Bytes + STAGE_KB - 1u) / STAGE_KB + p.splitStages - 1u) / p.splitStages : 1u;
+        const dim3     grid(((p.tileCount + 7u) / 8u) * 8u * (p.tileQuad ? 4u : 1u), splits), block(THREADS);
         auto launch = [&](auto aKc, auto bKc) {
             constexpr bool AK = decltype(aKc)::value, BK = decltype(bKc)::value;
             if constexpr(E == Elem::I8)
@@ -1381,7 +1412,7 @@ namespace
     {
         if(g.kernel == R355_KERNEL_TILED)
             return 256u; // (f64 is then refused by the check)
-        if(g.kernel == R355_KERNEL_TILED_128 || g.in_type == R355_F64)
+        if(g.kernel == R355_KERNEL_TILED_128 || g.kernel == R355_KERNEL_TILED_128_SPLITK || g.in_type == R355_F64)
             return 128u; // f64 accumulators only fit the small wave tile
         if(g.in_type == R355_F32)
             return 128u; // bound by the matrix-instruction rate either way (146 TFLOP/s at 4096^2 x 2048 with both
@@ -1389,6 +1420,86 @@ namespace
         const uint64_t cus    = computeUnits();
         auto           rounds = [&](uint32_t t) { return ((uint64_t)((g.m + t - 1) / t) * ((g.n + t - 1) / t) + cus - 1) / cus; };
         return rounds(128u) * 5u < rounds(256u) * 11u ? 128u : 256u;
+    }
+
+    // ------------------------------------------------------------------------------------------
+    // Split-K.  A problem with few output tiles and a long K (m <= 64 against n, k in the thousands; 512 x 512 x 32768)
+    // leaves most CUs idle with one workgroup per tile.  With a caller-provided workspace the 128 x 128 tile kernels run
+    // `splits` workgroup rows, each over its own range of K stages, writing partial results in the accumulator type
+    // to workspace[split][m][n]; splitKReduceKernel then adds the partial results in split order (deterministic) and applies
+    // alpha, beta and C once, exactly as the single-pass epilogue does.
+    uint32_t accBytes(int32_t inType)
+    {
+        return inType == R355_F64 ? 8u : 4u;
+    }
+    // number of K splits for a problem, 1 = no split; kernel selectors other than AUTO and TILED_128_SPLITK never split
+    uint32_t splitCount(const r355_gemm_args& g)
+    {
+        if(g.kernel != R355_KERNEL_AUTO && g.kernel != R355_KERNEL_TILED_128_SPLITK)
+            return 1u;
+        if(!g.workspace || !r355::aligned(g.workspace, 16))
+            return 1u;
+        const uint32_t cus = computeUnits();
+        const uint64_t tiles = (uint64_t)((g.m + 127u) / 128u) * ((g.n + 127u) / 128u);
+        const uint32_t stages = (g.k * r355::dtypeBytes(g.in_type) + STAGE_KB - 1u) / STAGE_KB;
+        if(tiles * 2u > cus || stages < 16u)
+            return 1u;
+        // one workgroup per CU (two per CU, which the 80 KiB of LDS allow, measured 5 - 20 % slower), at least 8 stages per share
+        uint32_t splits = static_cast<uint32_t>(cus / tiles);
+        splits = splits < stages / 8u ? splits : stages / 8u;
+        splits = splits < 32u ? splits : 32u;
+        if(splits < 2u)
+            return 1u;
+        // shares are whole stages; recompute the count from the share so that no share is empty
+        const uint32_t share = (stages + splits - 1u) / splits;
+        splits               = (stages + share - 1u) / share;
+        if(splits < 2u || (uint64_t)splits * g.m * g.n * accBytes(g.in_type) > g.workspace_bytes)
+            return 1u;
+        return splits;
+    }
+    uint32_t splitStagesOf(const r355_gemm_args& g, uint32_t splits)
+    {
+        const uint32_t stages = (g.k * r355::dtypeBytes(g.in_type) + STAGE_KB - 1u) / STAGE_KB;
+        return (stages + splits - 1u) / splits;
+    }
+
+    // One thread per 4 consecutive columns of a row of D (n is a multiple of 16).  AccT: f32, i32 or f64.
+    template <typename AccT, typename OutT>
+    __global__ void __launch_bounds__(256) splitKReduceKernel(const AccT* __restrict__ ws, uint32_t splits, uint64_t sliceElems, uint32_t m,
+                                                              uint32_t n, const OutT* c, uint32_t ldc, OutT* d, uint32_t ldd, double alphaD,
+                                                              double betaD)
+    {
+        const uint64_t idx = (uint64_t)blockIdx.x * 256u + threadIdx.x; // 4-column group
+        const uint32_t groupsPerRow = n / 4u;
+        if(idx >= (uint64_t)m * groupsPerRow)
+            return;
+        const uint32_t row = static_cast<uint32_t>(idx / groupsPerRow), col = static_cast<uint32_t>(idx % groupsPerRow) * 4u;
+        using AccV = AccT __attribute__((ext_vector_type(4)));
+        using OutV = OutT __attribute__((ext_vector_type(4)));
+        AccV sum = *reinterpret_cast<const AccV*>(ws + (uint64_t)row * n + col);
+        for(uint32_t s = 1; s < splits; ++s)
+        {
+            const AccV v = *reinterpret_cast<const AccV*>(ws + s * sliceElems + (uint64_t)row * n + col);
+#pragma unroll
+            for(uint32_t e = 0; e < 4; ++e)
+                sum[e] += v[e];
+        }
+        const AccT alpha = static_cast<AccT>(alphaD), beta = static_cast<AccT>(betaD);
+        OutV       out;
+        if(beta != static_cast<AccT>(0))
+        {
+            const OutV cv = *reinterpret_cast<const OutV*>(c + (uint64_t)row * ldc + col);
+#pragma unroll
+            for(uint32_t e = 0; e < 4; ++e)
+                out[e] = static_cast<OutT>(alpha * sum[e] + beta * static_cast<AccT>(cv[e]));
+        }
+        else
+        {
+#pragma unroll
+            for(uint32_t e = 0; e < 4; ++e)
+                out[e] = static_cast<OutT>(alpha * sum[e]);
+        }
+        *reinterpret_cast<OutV*>(d + (uint64_t)row * ldd + col) = out;
     }
 
     // Mixed tiling (R355_KERNEL_AUTO only).  A problem of a few rounds whose last round of 256 x 256 tiles would
@@ -1411,6 +1522,30 @@ namespace
 namespace r355
 {
 #if R355_TILED_HAS(0)
+    int splitKReduce(const r355_gemm_args& g, const GemmTileParams& p, uint32_t splits, hipStream_t stream)
+    {
+        // p is the kernel's view of the problem (D row-major m x n; a col-major D runs as its transpose)
+        const uint64_t groups = (uint64_t)p.m * (p.n / 4u);
+        const dim3     grid(static_cast<uint32_t>((groups + 255u) / 256u)), block(256);
+        const uint64_t slice = (uint64_t)p.m * p.n;
+        auto go = [&](auto acc, auto out) {
+            using AccT = decltype(acc);
+            using OutT = decltype(out);
+            hipLaunchKernelGGL((splitKReduceKernel<AccT, OutT>), grid, block, 0, stream, static_cast<const AccT*>(g.workspace), splits, slice,
+                               p.m, p.n, reinterpret_cast<const OutT*>(p.c), p.ldc, reinterpret_cast<OutT*>(p.d), p.ldd, p.alpha, p.beta);
+        };
+        switch(g.out_type)
+        {
+        case R355_F16: go(0.0f, _Float16{}); break;
+        case R355_BF16: go(0.0f, __bf16{}); break;
+        case R355_F32: go(0.0f, 0.0f); break;
+        case R355_F64: go(0.0, 0.0); break;
+        case R355_I32: go(int{}, int{}); break;
+        default: go(int{}, static_cast<signed char>(0)); break; // int8 result: the low byte, as the single-pass epilogue narrows it
+        }
+        return checkLaunch("gemm (split-K reduction)");
+    }
+
     int gemmTiledCheck(const r355_gemm_args& g, r355_gemm_plan* plan)
     {
         const bool pairOk = (g.in_type == R355_F16 && (g.out_type == R355_F16 || g.out_type == R355_F32))
@@ -1451,7 +1586,15 @@ namespace r355
             plan->block_x      = THREADS;
             plan->block_y      = 1;
             plan->lds_bytes    = (fiveBuffers || tile == 128u ? 5u * OPER_BYTES : NUM_STAGES * STAGE_BYTES) * tile / 256u;
+            const uint32_t splits = tile == 128u ? splitCount(g) : 1u;
+            plan->split_k         = splits;
+            plan->grid_y          = splits;
+            plan->workspace_bytes = splits > 1u ? (uint64_t)splits * g.m * g.n * accBytes(g.in_type) : 0u;
         }
+        if(g.kernel == R355_KERNEL_TILED_128_SPLITK && splitCount(g) < 2u)
+            return fail(R355_ERR_BAD_SIZE,
+                        "tiled gemm (split-K): needs a workspace of splits x m x n accumulator elements (r355_gemm_query with a large "
+                        "workspace_bytes reports the size), at most half as many 128 x 128 tiles as CUs and k of at least 16 stages of 128 bytes");
         return R355_OK;
     }
 
@@ -1497,6 +1640,34 @@ namespace r355
             default: return fail(R355_ERR_UNSUPPORTED, "tiled gemm: unknown in_type %d", g.in_type);
             }
         };
+        p.splitStages = 0u, p.splitStrideD = 0u;
+        const uint32_t splits = tile == 128u ? splitCount(g) : 1u;
+        if(splits > 1u)
+        {
+            // partial results in the accumulator type, row-major with leading dimension n, alpha = 1 and beta = 0; the
+            // reduction applies the caller's scalars and C
+            Params q        = p;
+            q.splitStages   = splitStagesOf(g, splits);
+            q.splitStrideD  = (uint64_t)p.m * p.n * accBytes(g.in_type);
+            q.d             = static_cast<char*>(g.workspace);
+            q.ldd           = p.n;
+            q.c             = nullptr;
+            q.alpha = 1.0, q.beta = 0.0;
+            r355_gemm_args ga = g; // the kernels of the accumulator-typed output
+            ga.out_type       = g.in_type == R355_F64 ? R355_F64 : (g.in_type == R355_I8 ? R355_I32 : R355_F32);
+            const int rc      = [&] {
+                switch(g.in_type)
+                {
+                case R355_F16: return gemmTiledPart0(ga, aK, bK, 128u, q, stream);
+                case R355_BF16: return gemmTiledPart1(ga, aK, bK, 128u, q, stream);
+                case R355_E4M3:
+                case R355_E5M2:
+                case R355_I8: return gemmTiledPart2(ga, aK, bK, 128u, q, stream);
+                default: return gemmTiledPart3(ga, aK, bK, 128u, q, stream);
+                }
+            }();
+            return rc != R355_OK ? rc : splitKReduce(g, p, splits, stream);
+        }
         const uint32_t rest = mixedRemainder(g);
         if(rest == 0u)
             return part(tile, p);

@@ -6,6 +6,7 @@
 //   host_bench gemm  [--type f16|bf16|i8|e4m3|f32|f64] [--out f16|bf16|f32|i32|f64] [--layout nt|tn|nn|tt]
 //                    [--m M --n N --k K] [--kernel auto|simple|tiled|tiled128] [--warmup W --iters I]
 //                    [--sparse 1]   A is 2:4 structured sparse (compressed values + index nibbles)
+//                    [--workspace MiB]  device workspace offered for split-K (few tiles, long K); 0 = none
 //                    [--ldpad E]    lda and ldb grow by E elements (power-of-two strides cost L2 efficiency)
 //   host_bench dlrm  [--type f16|bf16|f32] [--bwd 1] [--batch B --m M --k K] [--warmup W --iters I]
 //   host_bench gemv  [--m M --k K --layout n|t]
@@ -324,7 +325,7 @@ int main(int argc, char** argv)
     uint32_t          m = 8192, n = 8192, k = 8192, batch = 65536, ldpad = 0;
     bool              mSet = false, kSet = false;
     int               warmup = 2, iters = 10;
-    size_t            bytes = 1ull << 30;
+    size_t            bytes = 1ull << 30, workspaceMiB = 0;
     for(int i = 2; i + 1 < argc; i += 2)
     {
         const std::string a = argv[i], v = argv[i + 1];
@@ -341,6 +342,7 @@ int main(int argc, char** argv)
         else if(a == "--iters") iters = atoi(v.c_str()), itersSet = true;
         else if(a == "--sparse") sparse = atoi(v.c_str()) != 0;
         else if(a == "--bwd") bwd = atoi(v.c_str()) != 0;
+        else if(a == "--workspace") workspaceMiB = strtoull(v.c_str(), nullptr, 10);
         else if(a == "--bytes") bytes = strtoull(v.c_str(), nullptr, 10);
         else
         {
@@ -401,6 +403,11 @@ int main(int argc, char** argv)
         HIP_OK(hipMemcpy(db, hb.data(), hb.size(), hipMemcpyHostToDevice));
         HIP_OK(hipMemset(dd, 0xFF, (size_t)m * n * bytesOf(outT))); // NaN-prefill as the reference does
         g.a = da, g.b = db, g.d = dd;
+        if(workspaceMiB)
+        {
+            HIP_OK(hipMalloc(&g.workspace, workspaceMiB << 20));
+            g.workspace_bytes = workspaceMiB << 20;
+        }
         r355_gemm_plan plan;
         if(r355_gemm_query(&g, &plan) != R355_OK || r355_gemm_timed(&g, nullptr, warmup, iters, &ms) != R355_OK)
         {
@@ -417,10 +424,10 @@ int main(int argc, char** argv)
         const double perClk = inT == R355_F64 ? 128.0 : inT == R355_F32 ? 256.0 : (inT == R355_I8 || inT == R355_E4M3) ? 8192.0 : 4096.0; // flop / CU / clk
         const double model  = perClk * dev.compute_units * dev.clock_mhz * 1e-6; // TFLOP/s at the reported clock
         printf("{\"op\": \"%s\", \"type\": \"%s\", \"out\": \"%s\", \"layout\": \"%s\", \"m\": %u, \"n\": %u, \"k\": %u, "
-               "\"kernel\": %d, \"macro_tile\": [%u, %u, %u], \"lds_bytes\": %u, \"ms\": %.4f, \"tflops\": %.1f, "
+               "\"kernel\": %d, \"macro_tile\": [%u, %u, %u], \"split_k\": %u, \"lds_bytes\": %u, \"ms\": %.4f, \"tflops\": %.1f, "
                "\"frac_vendor_peak\": %.4f, \"frac_clock_model_peak\": %.4f, \"cus\": %d, \"clock_mhz\": %d}\n",
                sparse ? "gemm_sparse24" : "gemm", type.c_str(), out.c_str(), layout.c_str(), m, n, k, plan.kernel, plan.macro_tile_m, plan.macro_tile_n,
-               plan.macro_tile_k, plan.lds_bytes, ms, tflops, tflops / vendor, tflops / model, dev.compute_units,
+               plan.macro_tile_k, plan.split_k, plan.lds_bytes, ms, tflops, tflops / vendor, tflops / model, dev.compute_units,
                dev.clock_mhz);
     }
     else if(op == "dlrm")

@@ -497,7 +497,7 @@ namespace r355
         if(!aligned(g.a, 16) || !aligned(g.b, 16) || (g.ldb * es) % 16 || !aligned(g.a_meta, 4) || !aligned(g.d, 16) || (g.ldd % 4)
            || (g.beta != 0.0 && (!aligned(g.c, 16) || (g.ldc % 4))))
             return fail(R355_ERR_MISALIGNED, "sparse gemm: values, B, C and D need 16-byte alignment (pointers and leading dimensions), metadata 4-byte");
-        if(g.kernel == R355_KERNEL_TILED_128)
+        if(g.kernel == R355_KERNEL_TILED_128 || g.kernel == R355_KERNEL_TILED_128_SPLITK)
             return fail(R355_ERR_UNSUPPORTED, "sparse gemm: there is no 128 x 128 sparse macro tile (R355_KERNEL_TILED is 256 x 256)");
         if(g.kernel == R355_KERNEL_TILED && !tiledOk(g))
             return fail(R355_ERR_UNSUPPORTED, "sparse gemm (macro tile): C and D must share an orientation, metadata 16-byte aligned, ldb below 8 MiB");

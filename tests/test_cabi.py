@@ -83,7 +83,8 @@ def test_query_selects_kernel_family_and_reports_launch_shape():
     (dict(kernel=R.KERNEL_TILED, m=120), -3),
     (dict(kernel=R.KERNEL_TILED, k=100), -3),
     (dict(kernel=R.KERNEL_TILED_128, m=120), -3),
-    (dict(kernel=4), -1),
+    (dict(kernel=5), -1),
+    (dict(kernel=R.KERNEL_TILED_128_SPLITK), -3),  # no workspace
     (dict(kernel=R.KERNEL_TILED, in_type=R.I8, out_type=R.I32, layout_a=R.ROW_MAJOR, layout_b=R.COL_MAJOR, k=(1 << 23) + 16), -2),
     (dict(kernel=R.KERNEL_TILED, in_type=R.F64, out_type=R.F64), -2),
     (dict(a=0x1002, layout_a=R.ROW_MAJOR), -4),
