@@ -132,6 +132,16 @@ typedef struct
 } r355_gemm_plan;
 int r355_gemm_query(const r355_gemm_args* args, r355_gemm_plan* plan);
 
+/* r355_gemm for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc) and have no workspace to pass.  No counterpart in the reference.
+ * Identical to r355_gemm, except that args->workspace / workspace_bytes are ignored and split-K keeps its partial
+ * results in a 16 MiB buffer that is part of the library's device image (one per GPU, held until the process ends);
+ * the call allocates and frees nothing.  A problem whose split-K plan needs more than 16 MiB (r355_gemm_query with
+ * workspace_bytes = UINT64_MAX reports the need) is refused with R355_ERR_BAD_SIZE; with 4-byte accumulators no plan
+ * on 256 CUs needs more.  Nothing in the buffer has to start at zero (every partial result is written before it is
+ * read), but all calls on one GPU share it: calls that overlap in time on one GPU (two streams, two threads) race. */
+int r355_gemm_noalloc(const r355_gemm_args* args, void* stream);
+
 /* Timing helper in the reference's protocol (test/gemm/gemm_kernel_base_impl.hpp:647-676):
  * `warmup` untimed launches, then `iters` launches between two hipEvents on `stream`;
  * *avg_ms = elapsed / iters.  Synchronises the stream. */

@@ -24,7 +24,7 @@ KERNEL_AUTO, KERNEL_SIMPLE, KERNEL_TILED, KERNEL_TILED_128, KERNEL_TILED_128_SPL
 DTYPE_BYTES = {F16: 2, BF16: 2, E4M3: 1, I8: 1, F32: 4, I32: 4, F64: 8, E5M2: 1}
 
 EXPORTS = [
-    "r355_gemm", "r355_gemm_query", "r355_gemm_timed", "r355_dlrm_fwd", "r355_dlrm_fwd_timed",
+    "r355_gemm", "r355_gemm_noalloc", "r355_gemm_query", "r355_gemm_timed", "r355_dlrm_fwd", "r355_dlrm_fwd_timed",
     "r355_dlrm_bwd", "r355_gemv", "r355_gemv_timed", "r355_dgemv", "r355_compress_24", "r355_decompress_24", "r355_compress_24_16", "r355_decompress_24_16",
     "r355_get_device_info", "r355_last_error", "r355_version",
 ]
@@ -162,6 +162,11 @@ def gemm(in_type, out_type, m, n, k, a, b, c, d, alpha=1.0, beta=0.0, layout_a=R
     g = gemm_args(in_type, out_type, m, n, k, a, b, c, d, alpha, beta, layout_a, layout_b, layout_c, layout_d,
                   lda, ldb, ldc, ldd, kernel, a_meta, workspace)
     _check(lib().r355_gemm(ctypes.byref(g), _stream_handle(stream)))
+
+
+def gemm_noalloc(g, stream=None):
+    """r355_gemm_noalloc on prepared GemmArgs: split-K partial results go to the library's static device buffer."""
+    _check(lib().r355_gemm_noalloc(ctypes.byref(g), _stream_handle(stream)))
 
 
 def gemm_query(g):

@@ -2,12 +2,46 @@
 // validation, kernel-family selection, timing helpers, error text.
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 #include "common.hpp"
 
 namespace
 {
     thread_local char g_lastError[512] = "";
+
+    // Device memory of r355_gemm_noalloc: the split-K partial results of one call.  Every device the library runs on
+    // holds its own copy, at its own address, until the process ends.  The name below is only a host-side handle for
+    // hipGetSymbolAddress; kernels and copies take the address that call returns.
+    constexpr size_t SCRATCH_BYTES = size_t{16} << 20;
+    static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
+
+    constexpr int MAX_DEVICES = 64;
+    std::mutex    g_scratchLock;
+    void*         g_scratchAt[MAX_DEVICES] = {};
+
+    // address of `scratch` on the current device (looked up once per device)
+    int scratchOfCurrentDevice(void** ptr)
+    {
+        int dev = 0;
+        if(hipGetDevice(&dev) != hipSuccess)
+            return r355::fail(R355_ERR_LAUNCH, "gemm_noalloc: no HIP device");
+        if(dev < 0 || dev >= MAX_DEVICES)
+            return r355::fail(R355_ERR_UNSUPPORTED, "gemm_noalloc: device ordinal %d beyond the %d the library keeps scratch for", dev,
+                              MAX_DEVICES);
+        std::lock_guard<std::mutex> hold(g_scratchLock);
+        if(!g_scratchAt[dev])
+        {
+            void*            at = nullptr;
+            const hipError_t e  = hipGetSymbolAddress(&at, HIP_SYMBOL(scratch));
+            if(e != hipSuccess || !at)
+                return r355::fail(R355_ERR_LAUNCH, "gemm_noalloc: hipGetSymbolAddress(scratch) failed on device %d: %s", dev,
+                                  hipGetErrorString(e));
+            g_scratchAt[dev] = at;
+        }
+        *ptr = g_scratchAt[dev];
+        return R355_OK;
+    }
 
     int validateCommon(const r355_gemm_args* g)
     {
@@ -136,6 +170,33 @@ int r355_gemm(const r355_gemm_args* args, void* stream)
     if(rc != R355_OK)
         return rc;
     return launch(args, family, static_cast<hipStream_t>(stream));
+}
+
+int r355_gemm_noalloc(const r355_gemm_args* args, void* stream)
+{
+    if(!args)
+        return r355::fail(R355_ERR_BAD_ARG, "gemm_noalloc: args is null");
+    void* at = nullptr;
+    int   rc = scratchOfCurrentDevice(&at);
+    if(rc != R355_OK)
+        return rc;
+    // plan as if the workspace were unbounded to learn what split-K of this problem needs, then hold it against the array
+    r355_gemm_args g  = *args;
+    g.workspace       = at;
+    g.workspace_bytes = UINT64_MAX;
+    r355_gemm_plan need;
+    int32_t        family = 0;
+    rc                    = plan(&g, &need, &family);
+    if(rc != R355_OK)
+        return rc;
+    if(need.workspace_bytes > SCRATCH_BYTES)
+        return r355::fail(R355_ERR_BAD_SIZE,
+                          "gemm_noalloc: split-K of this problem (%u shares of %u x %u) needs %llu bytes of scratch, the library's "
+                          "static buffer holds %llu; call r355_gemm with a workspace of that size, or without one",
+                          need.split_k, g.m, g.n, static_cast<unsigned long long>(need.workspace_bytes),
+                          static_cast<unsigned long long>(SCRATCH_BYTES));
+    g.workspace_bytes = SCRATCH_BYTES;
+    return launch(&g, family, static_cast<hipStream_t>(stream));
 }
 
 int r355_gemm_query(const r355_gemm_args* args, r355_gemm_plan* out)
