@@ -13,6 +13,8 @@
 //   host_bench copy  [--bytes N]      plain device copy of known size (counter calibration)
 //   host_bench lds   [--iters I]      LDS read instructions from fixed conflict-free addresses with 4, 2 and 1 waves per CU:
 //                                     shader clocks per wave-level read and bytes per clock per CU
+//   host_bench fill                   direct global -> LDS loads alone, in the access stream of the 8192^3 1-byte GEMM
+//                                     (1024 tiles x 64 stages x 64 KiB), 1 - 3 stages in flight: aggregate TB/s
 //   host_bench mfma  [--iters I]      register-resident MFMA loops, one wave per SIMD, 16 independent
 //                                     accumulators: the rate the matrix cores sustain under the board's
 //                                     power limit with all-zero and with random operands
@@ -26,6 +28,8 @@
 #include <hip/hip_runtime.h>
 
 #include "../../include/r355_wmma.h"
+#include "lds_dma.hpp"
+#include "tile_map.hpp"
 
 #define HIP_OK(expr)                                                                       \
     do                                                                                     \
@@ -231,6 +235,55 @@ namespace
                  : "=v"(R0[0]), "=v"(R0[1]), "=v"(R0[2]), "=v"(R0[3]), "=v"(R0[4]), "=v"(R0[5]), "=v"(R0[6]), "=v"(R0[7])  \
                  : "v"(addr))
     using i32x2 = int __attribute__((ext_vector_type(2)));
+    // Direct global -> LDS loads and nothing else: every workgroup walks the K stages of a 256 x 256 tile of the 8192^3
+    // 1-byte GEMM (64 KiB per stage: 8 + 8 loads of 1 KiB per wave), the tiles in the library's own order, DEPTH stages in
+    // flight.  PATTERN 0: K-contiguous operands with `pitch` bytes per row (a load touches 8 rows x 128 bytes);
+    // 1: K-blocked operands (a tile's share of a stage is 32 KiB of consecutive bytes); 2: pattern 0 with every workgroup on
+    // tile (0, 0) (no L2 misses).
+    template <int DEPTH, int PATTERN>
+    __global__ void __launch_bounds__(256) fillLoop(const char* a, const char* b, uint32_t pitch, uint32_t stages, uint32_t tiles)
+    {
+        __shared__ __attribute__((aligned(1024))) char lds[65536];
+        uint32_t tm = 0, tn = 0;
+        if(!r355::tileCoordRange(blockIdx.x, tiles, tiles, 0u, tiles * tiles, false, tm, tn))
+            return;
+        if(PATTERN == 2)
+            tm = tn = 0;
+        const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const uint32_t ldsBase = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds));
+        uint32_t       off[8];
+        uint32_t       stageStride;
+        uint64_t       panel;
+        if(PATTERN == 1)
+        {
+            for(uint32_t j = 0; j < 8; ++j)
+                off[j] = j * 4096u + tid * 16u;
+            stageStride = 32768u;
+            panel       = (uint64_t)stages * 32768u; // a tile row's K stages, one after the other
+        }
+        else
+        {
+            for(uint32_t j = 0; j < 8; ++j)
+                off[j] = ((tid >> 3) + 32u * j) * pitch + (tid & 7u) * 16u;
+            stageStride = 128u;
+            panel       = 256ull * pitch;
+        }
+        const r355::dma_i32x4 ra = r355::rawBuffer(r355::uniformAddress(a + tm * panel));
+        const r355::dma_i32x4 rb = r355::rawBuffer(r355::uniformAddress(b + tn * panel));
+        for(uint32_t st = 0; st < stages; ++st)
+        {
+#pragma unroll
+            for(uint32_t j = 0; j < 8; ++j)
+                r355::loadToLds(ra, off[j], st * stageStride, ldsBase + wave * 1024u + j * 4096u);
+#pragma unroll
+            for(uint32_t j = 0; j < 8; ++j)
+                r355::loadToLds(rb, off[j], st * stageStride, ldsBase + 32768u + wave * 1024u + j * 4096u);
+            r355::waitVmcnt<16 * (DEPTH - 1)>();
+        }
+        r355::waitVmcnt<0>();
+    }
+
+
     template <int MODE>
     __global__ void __launch_bounds__(256) ldsReadLoop(int* out, int iters, unsigned long long* cyc)
     {
@@ -316,7 +369,7 @@ int main(int argc, char** argv)
 {
     if(argc < 2)
     {
-        fprintf(stderr, "usage: host_bench gemm|dlrm|gemv|copy|mfma|lds [options]\n");
+        fprintf(stderr, "usage: host_bench gemm|dlrm|gemv|copy|mfma|lds|fill [options]\n");
         return 2;
     }
     const std::string op = argv[1];
@@ -595,6 +648,54 @@ int main(int argc, char** argv)
                 printf("%s\n {\"op\": \"lds\", \"instr\": \"%s\", \"waves_per_cu\": %d, \"clocks_per_wave_read\": %.2f, "
                        "\"bytes_per_clock_per_cu\": %.1f}",
                        (waves == 4 && mode == 0) ? "" : ",", names[mode], waves, clocks / reads, reads * 64 * width[mode] / clocks);
+            }
+        printf("\n]\n");
+    }
+    else if(op == "fill")
+    {
+        // aggregate rate of direct global -> LDS loads in the access stream of the 8192^3 1-byte GEMM (no matrix instructions,
+        // no LDS reads, no stores): 1024 tiles x 64 stages x 64 KiB
+        const uint32_t tiles = 32, stages = 64;
+        const size_t   pitchMax = 8192 + 128;
+        void *         pa, *pb;
+        HIP_OK(hipMalloc(&pa, 8192 * pitchMax));
+        HIP_OK(hipMalloc(&pb, 8192 * pitchMax));
+        HIP_OK(hipMemset(pa, 1, 8192 * pitchMax));
+        HIP_OK(hipMemset(pb, 2, 8192 * pitchMax));
+        hipEvent_t e0, e1;
+        HIP_OK(hipEventCreate(&e0));
+        HIP_OK(hipEventCreate(&e1));
+        const char* names[4] = {"K-contiguous rows, pitch 8192", "K-contiguous rows, pitch 8320", "K-blocked (32 KiB runs)",
+                                "every workgroup on tile (0, 0)"};
+        printf("[");
+        for(int pat = 0; pat < 4; ++pat)
+            for(int depth = 1; depth <= 3; ++depth)
+            {
+                const uint32_t pitch = pat == 1 ? 8320u : 8192u;
+                auto           go    = [&] {
+                    const dim3 g(tiles * tiles), blk(256);
+                    const char *a = static_cast<const char*>(pa), *b = static_cast<const char*>(pb);
+#define R355_FILL(D, P) hipLaunchKernelGGL((fillLoop<D, P>), g, blk, 0, 0, a, b, pitch, stages, tiles)
+                    const int p = pat == 0 || pat == 1 ? 0 : pat - 1;
+                    if(depth == 1) { if(p == 0) R355_FILL(1, 0); else if(p == 1) R355_FILL(1, 1); else R355_FILL(1, 2); }
+                    else if(depth == 2) { if(p == 0) R355_FILL(2, 0); else if(p == 1) R355_FILL(2, 1); else R355_FILL(2, 2); }
+                    else { if(p == 0) R355_FILL(3, 0); else if(p == 1) R355_FILL(3, 1); else R355_FILL(3, 2); }
+#undef R355_FILL
+                };
+                for(int i = 0; i < 20; ++i)
+                    go();
+                HIP_OK(hipEventRecord(e0));
+                for(int i = 0; i < 20; ++i)
+                    go();
+                HIP_OK(hipEventRecord(e1));
+                HIP_OK(hipEventSynchronize(e1));
+                HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+                ms /= 20;
+                const double bytes = (double)tiles * tiles * stages * 65536.0;
+                const double rounds = (double)tiles * tiles / dev.compute_units;
+                printf("%s\n {\"op\": \"fill\", \"pattern\": \"%s\", \"stages_in_flight\": %d, \"ms\": %.4f, \"tb_per_s\": %.2f, "
+                       "\"us_per_64KiB_stage_per_cu\": %.3f}",
+                       (pat == 0 && depth == 1) ? "" : ",", names[pat], depth, ms, bytes / ms / 1e9, ms * 1e3 / (rounds * stages));
             }
         printf("\n]\n");
     }
