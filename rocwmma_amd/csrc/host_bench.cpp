@@ -15,6 +15,7 @@
 //                                     shader clocks per wave-level read and bytes per clock per CU
 //   host_bench fill                   direct global -> LDS loads alone, in the access stream of the 8192^3 1-byte GEMM
 //                                     (1024 tiles x 64 stages x 64 KiB), 1 - 3 stages in flight: aggregate TB/s
+//   host_bench store                  global stores alone in the shape of the macro-tile epilogue (256 KiB per workgroup)
 //   host_bench mfma  [--iters I]      register-resident MFMA loops, one wave per SIMD, 16 independent
 //                                     accumulators: the rate the matrix cores sustain under the board's
 //                                     power limit with all-zero and with random operands
@@ -284,6 +285,41 @@ namespace
     }
 
 
+    // Global stores alone, in the shape of the macro-tile epilogue: every workgroup of 4 waves writes a 256 x 256 tile of
+    // 4-byte elements (256 KiB) of a row-major matrix with `pitch` bytes per row, 16 bytes per lane; a wave owns a
+    // 128 x 128 quarter and one store instruction covers SEG consecutive bytes of 1024 / SEG rows.  NT: nontemporal.
+    template <uint32_t SEG, bool NT>
+    __global__ void __launch_bounds__(256) storeLoop(char* d, uint32_t pitch, uint32_t tiles, unsigned long long* cyc)
+    {
+        uint32_t tm = 0, tn = 0;
+        if(!r355::tileCoordRange(blockIdx.x, tiles, tiles, 0u, tiles * tiles, false, tm, tn))
+            return;
+        using v4            = int __attribute__((ext_vector_type(4)));
+        const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+        const uint32_t wm = wave >> 1, wn = wave & 1u;
+        constexpr uint32_t LPR = SEG / 16u, ROWS = 64u / LPR; // lanes per row, rows per instruction
+        char* base = d + ((uint64_t)tm * 256u + wm * 128u) * pitch + (tn * 256u + wn * 128u) * 4u;
+        const v4 v = {(int)lane, (int)wave, (int)tm, (int)tn};
+        const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();
+#pragma unroll 8
+        for(uint32_t it = 0; it < 65536u / 1024u; ++it)
+        {
+            // 512 bytes per row of the wave tile: SEG-byte segment s of row r
+            const uint32_t unit = it * ROWS + lane / LPR; // (row, segment) pairs in row-major order
+            const uint32_t row = unit / (512u / SEG), seg = unit % (512u / SEG);
+            v4* at = reinterpret_cast<v4*>(base + (uint64_t)row * pitch + seg * SEG + (lane % LPR) * 16u);
+            if(NT)
+                __builtin_nontemporal_store(v, at);
+            else
+                *at = v;
+        }
+        __builtin_amdgcn_s_waitcnt(0);
+        const unsigned long long t1 = __builtin_amdgcn_s_memrealtime();
+        if(threadIdx.x == 0)
+            atomicMax(cyc, t1 - t0);
+    }
+
+
     template <int MODE>
     __global__ void __launch_bounds__(256) ldsReadLoop(int* out, int iters, unsigned long long* cyc)
     {
@@ -369,7 +405,7 @@ int main(int argc, char** argv)
 {
     if(argc < 2)
     {
-        fprintf(stderr, "usage: host_bench gemm|dlrm|gemv|copy|mfma|lds|fill [options]\n");
+        fprintf(stderr, "usage: host_bench gemm|dlrm|gemv|copy|mfma|lds|fill|store [options]\n");
         return 2;
     }
     const std::string op = argv[1];
@@ -696,6 +732,56 @@ int main(int argc, char** argv)
                 printf("%s\n {\"op\": \"fill\", \"pattern\": \"%s\", \"stages_in_flight\": %d, \"ms\": %.4f, \"tb_per_s\": %.2f, "
                        "\"us_per_64KiB_stage_per_cu\": %.3f}",
                        (pat == 0 && depth == 1) ? "" : ",", names[pat], depth, ms, bytes / ms / 1e9, ms * 1e3 / (rounds * stages));
+            }
+        printf("\n]\n");
+    }
+    else if(op == "store")
+    {
+        // epilogue-shaped global stores alone: 1, 64, 256 or 1024 tiles of 256 KiB
+        void* pd;
+        const size_t pitch = 8192 * 4;
+        HIP_OK(hipMalloc(&pd, 8192 * pitch));
+        unsigned long long* cyc;
+        HIP_OK(hipMalloc(&cyc, 8));
+        hipEvent_t e0, e1;
+        HIP_OK(hipEventCreate(&e0));
+        HIP_OK(hipEventCreate(&e1));
+        printf("[");
+        bool first = true;
+        for(uint32_t tiles : {1u, 8u, 16u, 32u})
+            for(int var = 0; var < 6; ++var)
+            {
+                auto go = [&] {
+                    const dim3 g(((tiles * tiles + 7u) / 8u) * 8u), blk(256);
+                    char*      d = static_cast<char*>(pd);
+                    switch(var)
+                    {
+                    case 0: hipLaunchKernelGGL((storeLoop<512, true>), g, blk, 0, 0, d, (uint32_t)pitch, tiles, cyc); break;
+                    case 1: hipLaunchKernelGGL((storeLoop<512, false>), g, blk, 0, 0, d, (uint32_t)pitch, tiles, cyc); break;
+                    case 2: hipLaunchKernelGGL((storeLoop<256, true>), g, blk, 0, 0, d, (uint32_t)pitch, tiles, cyc); break;
+                    case 3: hipLaunchKernelGGL((storeLoop<128, true>), g, blk, 0, 0, d, (uint32_t)pitch, tiles, cyc); break;
+                    case 4: hipLaunchKernelGGL((storeLoop<64, true>), g, blk, 0, 0, d, (uint32_t)pitch, tiles, cyc); break;
+                    default: hipLaunchKernelGGL((storeLoop<64, false>), g, blk, 0, 0, d, (uint32_t)pitch, tiles, cyc); break;
+                    }
+                };
+                const char* names[6] = {"512 B x 2 rows, nontemporal", "512 B x 2 rows, plain", "256 B x 4 rows, nontemporal",
+                                        "128 B x 8 rows, nontemporal", "64 B x 16 rows, nontemporal", "64 B x 16 rows, plain"};
+                for(int i = 0; i < 10; ++i)
+                    go();
+                HIP_OK(hipMemset(cyc, 0, 8));
+                HIP_OK(hipEventRecord(e0));
+                for(int i = 0; i < 20; ++i)
+                    go();
+                HIP_OK(hipEventRecord(e1));
+                HIP_OK(hipEventSynchronize(e1));
+                HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+                ms /= 20;
+                unsigned long long worst = 0;
+                HIP_OK(hipMemcpy(&worst, cyc, 8, hipMemcpyDeviceToHost));
+                printf("%s\n {\"op\": \"store\", \"tiles\": %u, \"instruction\": \"%s\", \"ms_per_launch\": %.4f, "
+                       "\"slowest_workgroup_us\": %.2f, \"tb_per_s\": %.2f}",
+                       first ? "" : ",", tiles * tiles, names[var], ms, worst / 100.0, tiles * tiles * 262144.0 / ms / 1e9);
+                first = false;
             }
         printf("\n]\n");
     }
