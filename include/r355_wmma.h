@@ -106,7 +106,8 @@ typedef struct
      * the CUs while k spans at least 16 stages of 128 bytes run `split_k` workgroups per tile, each over its own range of
      * K, into workspace[split][m][n] (accumulator type: 4 bytes, f64: 8), followed by a reduction kernel that adds the
      * partial results in split order and applies alpha, beta and C.  r355_gemm_query reports split_k and the bytes it
-     * needs for the workspace_bytes offered (offer UINT64_MAX to learn the size).  NULL / too small: no split.
+     * needs for the workspace_bytes offered (to learn the size, offer UINT64_MAX; the query accepts workspace = NULL with
+     * it).  A launch with workspace = NULL, one that is not 16-byte aligned or one that is too small does not split.
      * The library never allocates; calls that share a workspace must not overlap. */
     void*       workspace;
     uint64_t    workspace_bytes;

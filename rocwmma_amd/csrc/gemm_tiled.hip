@@ -1432,12 +1432,13 @@ namespace
     {
         return inType == R355_F64 ? 8u : 4u;
     }
-    // number of K splits for a problem, 1 = no split; kernel selectors other than AUTO and TILED_128_SPLITK never split
-    uint32_t splitCount(const r355_gemm_args& g)
+    // number of K splits for a problem, 1 = no split; kernel selectors other than AUTO and TILED_128_SPLITK never split.
+    // sizing: a query may offer workspace_bytes without a workspace to learn what a launch would use
+    uint32_t splitCount(const r355_gemm_args& g, bool sizing = false)
     {
         if(g.kernel != R355_KERNEL_AUTO && g.kernel != R355_KERNEL_TILED_128_SPLITK)
             return 1u;
-        if(!g.workspace || !r355::aligned(g.workspace, 16))
+        if(g.workspace ? !r355::aligned(g.workspace, 16) : !sizing)
             return 1u;
         const uint32_t cus = computeUnits();
         const uint64_t tiles = (uint64_t)((g.m + 127u) / 128u) * ((g.n + 127u) / 128u);
@@ -1586,12 +1587,12 @@ namespace r355
             plan->block_x      = THREADS;
             plan->block_y      = 1;
             plan->lds_bytes    = (fiveBuffers || tile == 128u ? 5u * OPER_BYTES : NUM_STAGES * STAGE_BYTES) * tile / 256u;
-            const uint32_t splits = tile == 128u ? splitCount(g) : 1u;
+            const uint32_t splits = tile == 128u ? splitCount(g, true) : 1u;
             plan->split_k         = splits;
             plan->grid_y          = splits;
             plan->workspace_bytes = splits > 1u ? (uint64_t)splits * g.m * g.n * accBytes(g.in_type) : 0u;
         }
-        if(g.kernel == R355_KERNEL_TILED_128_SPLITK && splitCount(g) < 2u)
+        if(g.kernel == R355_KERNEL_TILED_128_SPLITK && splitCount(g, plan != nullptr) < 2u)
             return fail(R355_ERR_BAD_SIZE,
                         "tiled gemm (split-K): needs a workspace of splits x m x n accumulator elements (r355_gemm_query with a large "
                         "workspace_bytes reports the size), at most half as many 128 x 128 tiles as CUs and k of at least 16 stages of 128 bytes");

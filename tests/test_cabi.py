@@ -73,6 +73,24 @@ def test_query_selects_kernel_family_and_reports_launch_shape():
     assert plan.kernel == R.KERNEL_SIMPLE and plan.lds_bytes == 0 and plan.macro_tile_m == 32
 
 
+def test_query_sizes_a_split_k_workspace_without_a_pointer():
+    # (no device needed: 256 CUs are assumed when none answers)
+    skinny = dict(m=64, n=1024, k=8192)
+    plan = R.gemm_query(_args(**skinny))
+    assert plan.split_k == 1 and plan.workspace_bytes == 0 and plan.grid_y == 1
+    plan = R.gemm_query(_args(workspace=None, workspace_bytes=2 ** 64 - 1, **skinny))
+    assert plan.split_k == 16 and plan.grid_y == 16 and plan.workspace_bytes == 16 * 64 * 1024 * 4
+    assert (plan.macro_tile_m, plan.grid_x) == (128, 8)
+    assert R.gemm_query(_args(workspace=None, workspace_bytes=plan.workspace_bytes - 1, **skinny)).split_k == 1
+    f64 = dict(in_type=R.F64, out_type=R.F64, m=128, n=128, k=1024, layout_a=R.ROW_MAJOR, layout_b=R.COL_MAJOR)
+    plan = R.gemm_query(_args(workspace=None, workspace_bytes=2 ** 64 - 1, **f64))
+    assert plan.split_k == 8 and plan.workspace_bytes == 8 * 128 * 128 * 8  # 64 stages, at least 8 per share; f64 partial sums
+    # problems that fill the chip, short K, other selectors: no split
+    assert R.gemm_query(_args(m=8192, n=8192, k=8192, workspace_bytes=2 ** 64 - 1)).split_k == 1
+    assert R.gemm_query(_args(m=64, n=1024, k=512, workspace_bytes=2 ** 64 - 1)).split_k == 1
+    assert R.gemm_query(_args(kernel=R.KERNEL_TILED_128, workspace_bytes=2 ** 64 - 1, **skinny)).split_k == 1
+
+
 @pytest.mark.parametrize("kw,code", [
     (dict(a=None), -1),
     (dict(beta=1.0, c=None), -1),

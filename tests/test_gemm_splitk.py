@@ -19,7 +19,7 @@ ACC_BYTES = {O.F64: 8}
 
 def _plan(in_t, out_t, m, n, k, la, lb, ldl, workspace_bytes, kernel, beta=0.0):
     g = R.gemm_args(in_t, out_t, m, n, k, 0x1000, 0x2000, 0x3000 if beta else None, 0x4000, 1.0, beta, la, lb, ldl, ldl,
-                    kernel=kernel, workspace=0x5000 if workspace_bytes else None, workspace_bytes=workspace_bytes)
+                    kernel=kernel, workspace=None, workspace_bytes=workspace_bytes)  # sizing needs no pointer
     return R.gemm_query(g)
 
 
@@ -191,6 +191,13 @@ def test_auto_splits_only_with_a_workspace_and_only_skinny_problems():
     assert e.value.code == -3
     with pytest.raises(R.R355Error):
         _plan(*skinny, 0, R.KERNEL_TILED_128_SPLITK)
+    # a launch needs the pointer: without it the forced selector is an error and AUTO does not split (the same D either way)
+    in_t, out_t, m, n, k, la, lb, ldl = skinny
+    g = R.gemm_args(in_t, out_t, m, n, k, 0x1000, 0x2000, None, 0x4000, 1.0, 0.0, la, lb, ldl, ldl, kernel=R.KERNEL_TILED_128_SPLITK,
+                    workspace=None, workspace_bytes=2 ** 62)
+    assert R.lib().r355_gemm(R.ctypes.byref(g), None) == -3
+    g.workspace = 0x5008  # not 16-byte aligned
+    assert R.lib().r355_gemm(R.ctypes.byref(g), None) == -3
     # problems that fill the chip or have a short K do not split
     assert _plan(O.F16, O.F16, 8192, 8192, 8192, O.COL, O.ROW, O.ROW, 2 ** 62, R.KERNEL_AUTO).split_k == 1
     assert _plan(O.F16, O.F16, 2048, 2048, 8192, O.COL, O.ROW, O.ROW, 2 ** 62, R.KERNEL_AUTO).split_k == 1
