@@ -67,6 +67,45 @@ namespace rocwmma
                 return Map1d::fromMatrixCoord(Layout::matrixCoord(d, k), ldm);
             }
 
+            // Elements of 8 or 16 bits that arrived one by one sit in a 32-bit register each for as long as the compiler
+            // sees them as separate values: the 64 halves of four 32 x 32 accumulator blocks loaded ahead of an epilogue
+            // then hold 64 registers.  Passing every 32-bit word of the chunk through an opaque statement makes the packed
+            // word the value that stays live (one v_perm / v_lshl_or per word; unpacking at the use is an operand select).
+            ROCWMMA_DEVICE static inline void keepPacked(DataT* chunk)
+            {
+#if ROCWMMA_DEVICE_COMPILE
+                if constexpr(Layout::IsAcc && sizeof(DataT) < 4u && ChunkBytes % 4u == 0u)
+                {
+#pragma unroll
+                    for(uint32_t w = 0; w < ChunkBytes / 4u; ++w)
+                    {
+                        uint32_t word;
+                        __builtin_memcpy(&word, reinterpret_cast<char*>(chunk) + 4u * w, 4);
+                        asm volatile("" : "+v"(word));
+                        __builtin_memcpy(reinterpret_cast<char*>(chunk) + 4u * w, &word, 4);
+                    }
+                }
+#else
+                (void)chunk;
+#endif
+            }
+
+            // An offset (or leading dimension) the compiler cannot use before this point of the program, for the
+            // element accesses of accumulator fragments: the addresses of a block's 16 or 64 accesses, and the offsets
+            // they share with the next block's, are otherwise all formed ahead and held in registers, and that
+            // footprint sets the occupancy of a kernel whose epilogue uses these accesses (the reference's perf_hgemm
+            // sample through these headers: 132 -> 101 registers, 2 -> 3 waves per SIMD, 274 -> 364 TFLOP/s).  Matrix
+            // fragments keep free scheduling: their element loads sit in K loops, where ordering them costs more
+            // than the registers.
+            ROCWMMA_DEVICE static inline uint32_t justInTime(uint32_t off)
+            {
+#if ROCWMMA_DEVICE_COMPILE
+                if constexpr(Layout::IsAcc)
+                    asm volatile("" : "+v"(off) : : "memory");
+#endif
+                return off;
+            }
+
             // Chunks [FirstChunk, FirstChunk + Count) of memory <-> registers [RegChunk...)
             template <uint32_t Count>
             ROCWMMA_DEVICE static inline void
@@ -133,11 +172,19 @@ namespace rocwmma
                     }
                     else
                     {
-                        const uint32_t base = offset(d, k, ldm);
+                        const uint32_t ld   = justInTime(ldm);
+                        const uint32_t base = offset(d, k, ld);
 #pragma unroll
                         for(uint32_t e = 0; e < KW; ++e)
-                            regs[c * KW + e] = data[base + e * ldm];
+                            regs[c * KW + e] = data[justInTime(base + e * ld)];
                     }
+                }
+                // (after the last access has been issued: the statement waits for the data it is given)
+                if constexpr(!Contiguous)
+                {
+#pragma unroll
+                    for(uint32_t c = 0; c < Count; ++c)
+                        keepPacked(regs + c * KW);
                 }
             }
 
@@ -159,10 +206,11 @@ namespace rocwmma
                     }
                     else
                     {
-                        const uint32_t base = offset(d, k, ldm);
+                        const uint32_t ld   = justInTime(ldm);
+                        const uint32_t base = offset(d, k, ld);
 #pragma unroll
                         for(uint32_t e = 0; e < KW; ++e)
-                            data[base + e * ldm] = regs[c * KW + e];
+                            data[justInTime(base + e * ld)] = regs[c * KW + e];
                     }
                 }
             }
