@@ -1477,13 +1477,25 @@ namespace
         const uint32_t row = static_cast<uint32_t>(idx / groupsPerRow), col = static_cast<uint32_t>(idx % groupsPerRow) * 4u;
         using AccV = AccT __attribute__((ext_vector_type(4)));
         using OutV = OutT __attribute__((ext_vector_type(4)));
-        AccV sum = *reinterpret_cast<const AccV*>(ws + (uint64_t)row * n + col);
-        for(uint32_t s = 1; s < splits; ++s)
+        const AccT* mine = ws + (uint64_t)row * n + col;
+        AccV        sum  = *reinterpret_cast<const AccV*>(mine);
+        // up to eight partial results requested at a time, added in split order (the order never depends on timing)
+        for(uint32_t s = 1; s < splits; s += 8u)
         {
-            const AccV v = *reinterpret_cast<const AccV*>(ws + s * sliceElems + (uint64_t)row * n + col);
+            const uint32_t count = splits - s < 8u ? splits - s : 8u; // uniform
+            AccV           v[8];
 #pragma unroll
-            for(uint32_t e = 0; e < 4; ++e)
-                sum[e] += v[e];
+            for(uint32_t u = 0; u < 8; ++u)
+                if(u < count)
+                    v[u] = *reinterpret_cast<const AccV*>(mine + (s + u) * sliceElems);
+#pragma unroll
+            for(uint32_t u = 0; u < 8; ++u)
+                if(u < count)
+                {
+#pragma unroll
+                    for(uint32_t e = 0; e < 4; ++e)
+                        sum[e] += v[u][e];
+                }
         }
         const AccT alpha = static_cast<AccT>(alphaD), beta = static_cast<AccT>(betaD);
         OutV       out;
