@@ -91,6 +91,36 @@ def test_query_sizes_a_split_k_workspace_without_a_pointer():
     assert R.gemm_query(_args(kernel=R.KERNEL_TILED_128, workspace_bytes=2 ** 64 - 1, **skinny)).split_k == 1
 
 
+def test_query_plans_cover_every_tile_and_every_k_stage():
+    # seeded sweep over shapes and types: the launch shape the plan reports covers the problem, and a split-K plan gives
+    # every share at least one whole stage, needs exactly split_k * m * n accumulator elements and never exceeds 32 shares
+    import random
+    rng = random.Random(7)
+    types = [(R.F16, R.F16, 2), (R.BF16, R.F32, 2), (R.I8, R.I32, 1), (R.E4M3, R.F32, 1), (R.F32, R.F32, 4), (R.F64, R.F64, 8)]
+    for _ in range(400):
+        in_t, out_t, es = rng.choice(types)
+        m, n = 16 * rng.randint(1, 300), 16 * rng.randint(1, 300)
+        k = (16 // es) * rng.randint(1, 4000)
+        la, lb = rng.choice([R.ROW_MAJOR, R.COL_MAJOR]), rng.choice([R.ROW_MAJOR, R.COL_MAJOR])
+        plan = R.gemm_query(_args(in_type=in_t, out_type=out_t, m=m, n=n, k=k, layout_a=la, layout_b=lb, workspace_bytes=2 ** 64 - 1))
+        assert plan.kernel == R.KERNEL_TILED
+        tm, tn = plan.macro_tile_m, plan.macro_tile_n
+        assert (tm, tn) in ((128, 128), (256, 256)) and plan.macro_tile_k * es == 128
+        tiles = -(-m // tm) * -(-n // tn)
+        stages = -(-k * es // 128)
+        if plan.split_k > 1:
+            assert tm == 128 and 2 * tiles <= 256 and stages >= 16 and plan.split_k <= 32 and plan.grid_y == plan.split_k
+            share = -(-stages // plan.split_k)
+            assert share >= 8 or plan.split_k * 8 > stages - 8  # at least 8 stages per share where K allows
+            assert (plan.split_k - 1) * share < stages  # the last share is not empty
+            assert plan.workspace_bytes == plan.split_k * m * n * (8 if in_t == R.F64 else 4)
+            assert plan.grid_x >= tiles
+        else:
+            assert plan.workspace_bytes == 0 and plan.grid_y == 1
+            # one launch covers every tile, or the rest (at most half a round of 256 x 256 tiles) runs in the second launch
+            assert plan.grid_x >= tiles or (tm == 256 and tiles > 256 and 0 < tiles % 256 <= 128 and plan.grid_x >= tiles - tiles % 256)
+
+
 @pytest.mark.parametrize("kw,code", [
     (dict(a=None), -1),
     (dict(beta=1.0, c=None), -1),
