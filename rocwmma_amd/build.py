@@ -1,6 +1,6 @@
 """Builds the gfx950 shared library (csrc/*.hip, csrc/api.cpp -> lib/librocwmma_amd.so) with hipcc.
 
-Usage: python -m rocwmma_amd.build [--force]
+Usage: python -m rocwmma_amd.build [--force] [--timeline]
 Objects are rebuilt when their source (or any header) is newer; translation units compile in parallel.
 """
 import os
@@ -69,6 +69,25 @@ def build(force=False, verbose=True):
     return LIB
 
 
+TIMELINE_LIB = os.path.join(LIBDIR, "librocwmma_amd_timeline.so")
+
+
+def build_timeline(verbose=True):
+    """The profiling twin of the library (lib/librocwmma_amd_timeline.so, read by rocwmma_amd.timeline): the macro-tile
+    kernels compiled with -DR355_TIMELINE, everything else from the ordinary objects.  Never loaded by the package itself."""
+    build(verbose=False)
+    tiled = [s for s in SOURCES if s[0] == "gemm_tiled.hip"]
+    with ThreadPoolExecutor(max_workers=min(4, os.cpu_count() or 1)) as ex:
+        tl = list(ex.map(lambda s: _compile((s[0], "tl_" + s[1], s[2] + ["-DR355_TIMELINE"]), False), tiled))
+    objs = [os.path.join(OBJDIR, stem + ".o") for src, stem, _ in SOURCES if src != "gemm_tiled.hip"] + [o for o, _ in tl]
+    r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", TIMELINE_LIB] + objs, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n" + r.stderr)
+    if verbose:
+        print("built", TIMELINE_LIB)
+    return TIMELINE_LIB
+
+
 def build_host_bench(verbose=True):
     """C++ host bench (csrc/host_bench.cpp -> lib/host_bench), linked against the C-ABI library."""
     exe = os.path.join(LIBDIR, "host_bench")
@@ -85,3 +104,5 @@ def build_host_bench(verbose=True):
 if __name__ == "__main__":
     build(force="--force" in sys.argv)
     build_host_bench()
+    if "--timeline" in sys.argv:
+        build_timeline()

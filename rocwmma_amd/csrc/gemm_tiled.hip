@@ -55,6 +55,45 @@
 #endif
 #define R355_TILED_HAS(part) (R355_TILED_PART < 0 || R355_TILED_PART == (part))
 
+// Profiling build (-DR355_TIMELINE, `python -m rocwmma_amd.build --timeline`; never the shipped library): thread 0 of every
+// workgroup of the 256 x 256 tile kernels records the 100 MHz counter at entry (0), when the first stage is in LDS (1),
+// after the K loop (2) and after the last store has been issued and acknowledged (3), and its hardware id (4, 5).
+// `python -m rocwmma_amd.timeline` reads the records through r355_timeline_read_p<part>.
+#ifdef R355_TIMELINE
+#define R355_TL_PASTE2(a, b) a##b
+#define R355_TL_PASTE(a, b) R355_TL_PASTE2(a, b)
+static __device__ unsigned long long r355_timeline[8192 * 8];
+extern "C" int R355_TL_PASTE(r355_timeline_read_p, R355_TILED_PART)(void* host, size_t bytes)
+{
+    return static_cast<int>(hipMemcpyFromSymbol(host, HIP_SYMBOL(r355_timeline), bytes));
+}
+#define R355_STAMP(slot)                                                                            \
+    do                                                                                              \
+    {                                                                                               \
+        if(WB == 8 && threadIdx.x == 0 && blockIdx.x < 8192u)                                       \
+            r355_timeline[blockIdx.x * 8u + (slot)] = __builtin_amdgcn_s_memrealtime();             \
+    } while(0)
+#define R355_STAMP_ID()                                                                             \
+    do                                                                                              \
+    {                                                                                               \
+        if(WB == 8 && threadIdx.x == 0 && blockIdx.x < 8192u)                                       \
+        {                                                                                           \
+            r355_timeline[blockIdx.x * 8u + 4u] = __builtin_amdgcn_s_getreg(63492); /* HW_ID */     \
+            r355_timeline[blockIdx.x * 8u + 5u] = __builtin_amdgcn_s_getreg(63508); /* XCC_ID */    \
+        }                                                                                           \
+    } while(0)
+#define R355_STAMP_END()                                                                            \
+    do                                                                                              \
+    {                                                                                               \
+        __builtin_amdgcn_s_waitcnt(0);                                                              \
+        R355_STAMP(3);                                                                              \
+    } while(0)
+#else
+#define R355_STAMP(slot)
+#define R355_STAMP_ID()
+#define R355_STAMP_END()
+#endif
+
 namespace r355
 {
     struct GemmTileParams
@@ -356,6 +395,8 @@ namespace
         constexpr uint32_t TK = STAGE_KB / ES; // 64 K elements per stage = two K steps of 32
         static_assert(ES == 2, "16-bit element types only");
         static_assert(WB == 8 || WB == 4, "wave tile of 8 x 8 or 4 x 4 blocks");
+        R355_STAMP(0);
+        R355_STAMP_ID();
         constexpr uint32_t TILE  = 32u * WB; // macro tile edge
         constexpr uint32_t WT    = 16u * WB; // wave tile edge
         constexpr uint32_t OPER  = TILE * STAGE_KB; // bytes of one operand per stage
@@ -623,6 +664,7 @@ namespace
         issueGlobal(1, stage1);
         __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
         __syncthreads();
+        R355_STAMP(1);
         readStep(stage0, 0);
         refillA = uniform64(gA + (numStages > 2u ? 2u : numStages - 1u) * gStageA);
         refillB = uniform64(gB + (numStages > 2u ? 2u : numStages - 1u) * gStageB);
@@ -633,6 +675,7 @@ namespace
             stageBody(kt + 1, stage1, stage0);
         }
 
+        R355_STAMP(2);
         // the refills past the end (zeros) are still landing in the buffers the epilogue reuses
         __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
         __syncthreads();
@@ -640,6 +683,7 @@ namespace
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
         storeTile16<f32x4, OutT, WB>(acc, p, tm * TILE + wm * WT, tn * TILE + wn * WT, lane,
                                      ((wave < 2u) ? stage0 : stage1) + (wave & 1u) * (WB * 4096u));
+        R355_STAMP_END();
     }
 
     // (a waves-per-EU attribute that depends on a template parameter makes the compiler drop the host-side
@@ -876,6 +920,8 @@ namespace
         static_assert(WB == 8 || WB == 4, "wave tile of 8 x 8 or 4 x 4 blocks");
         static_assert(E != Elem::F64 || WB == 4, "f64 accumulators of an 8 x 8 wave tile would need 512 registers");
         static_assert(E != Elem::E4M3 && E != Elem::E5M2, "fp8 has its own stage structure");
+        R355_STAMP(0);
+        R355_STAMP_ID();
         constexpr uint32_t ES = ElemTraits<E>::Bytes;
         // split-K: this workgroup row's share of K (the whole problem when splitStages is 0)
         const Params p = splitShare<ES>(whole, A_KCONTIG ? (uint64_t)STAGE_KB : (uint64_t)STAGE_KB * whole.lda,
@@ -1026,6 +1072,7 @@ namespace
         refillA = stageAddr(gA, gStageA, 2u), refillB = stageAddr(gB, gStageB, 3u);
         waitVmcnt<3u * WB>();
         ldsBarrier();
+        R355_STAMP(1);
 #pragma unroll
         for(uint32_t x = 0; x < XS; ++x)
         {
@@ -1064,12 +1111,14 @@ namespace
             }
         }
 
+        R355_STAMP(2);
         // the loads past the last stage (zeros) are still landing in buffers the epilogue reuses, and the
         // last matrix instructions are still in the pipeline (the compiler does not know either)
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
         waitVmcnt<0>();
         ldsBarrier();
         storeTile16<AccV, OutT, WB>(acc, p, tm * TILE + wm * WT, tn * TILE + wn * WT, lane, lds + wave * (WB * 4096u));
+        R355_STAMP_END();
     }
 
     template <typename OutT, bool A_KCONTIG, bool B_KCONTIG>
@@ -1133,6 +1182,8 @@ namespace
     __device__ __forceinline__ void gemmTiledF8(const Params& whole)
     {
         static_assert(WB == 8 || WB == 4, "wave tile of 8 x 8 or 4 x 4 blocks");
+        R355_STAMP(0);
+        R355_STAMP_ID();
         const Params p = splitShare<1u>(whole, A_KCONTIG ? (uint64_t)STAGE_KB : (uint64_t)STAGE_KB * whole.lda,
                                         B_KCONTIG ? (uint64_t)STAGE_KB : (uint64_t)STAGE_KB * whole.ldb);
         constexpr uint32_t TILE = 32u * WB, WT = 16u * WB; // macro tile and wave tile edge
@@ -1284,6 +1335,7 @@ namespace
         refillA = stageAddr(gA, gStageA, 2u), refillB = stageAddr(gB, gStageB, 3u);
         waitVmcnt<3u * WB>();
         ldsBarrier();
+        R355_STAMP(1);
 #pragma unroll
         for(uint32_t n = 0; n < NQ; ++n)
         {
@@ -1322,10 +1374,12 @@ namespace
             }
         }
 
+        R355_STAMP(2);
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); // the last matrix instructions are still in the pipeline
         waitVmcnt<0>();
         ldsBarrier();
         storeTile16<f32x4, float, WB>(acc, p, tm * TILE + wm * WT, tn * TILE + wn * WT, lane, lds + wave * (WB * 4096u));
+        R355_STAMP_END();
     }
 
     template <bool E5M2, bool A_KCONTIG, bool B_KCONTIG>
