@@ -7,6 +7,7 @@
 //                    [--m M --n N --k K] [--kernel auto|simple|tiled|tiled128] [--warmup W --iters I]
 //                    [--sparse 1]   A is 2:4 structured sparse (compressed values + index nibbles)
 //                    [--workspace MiB]  device workspace offered for split-K (few tiles, long K); 0 = none
+//                    [--zero 1]     all-zero operands (no switching power: the engine clock stays at its maximum)
 //                    [--ldpad E]    lda and ldb grow by E elements (power-of-two strides cost L2 efficiency)
 //   host_bench dlrm  [--type f16|bf16|f32] [--bwd 1] [--batch B --m M --k K] [--warmup W --iters I]
 //   host_bench gemv  [--m M --k K --layout n|t]
@@ -410,7 +411,7 @@ int main(int argc, char** argv)
     }
     const std::string op = argv[1];
     std::string       type = "f16", out = "", layout = "nt", kernel = "auto";
-    bool              sparse = false, itersSet = false, bwd = false;
+    bool              sparse = false, itersSet = false, bwd = false, zeroFill = false;
     uint32_t          m = 8192, n = 8192, k = 8192, batch = 65536, ldpad = 0;
     bool              mSet = false, kSet = false;
     int               warmup = 2, iters = 10;
@@ -431,6 +432,7 @@ int main(int argc, char** argv)
         else if(a == "--iters") iters = atoi(v.c_str()), itersSet = true;
         else if(a == "--sparse") sparse = atoi(v.c_str()) != 0;
         else if(a == "--bwd") bwd = atoi(v.c_str()) != 0;
+        else if(a == "--zero") zeroFill = atoi(v.c_str()) != 0;
         else if(a == "--workspace") workspaceMiB = strtoull(v.c_str(), nullptr, 10);
         else if(a == "--bytes") bytes = strtoull(v.c_str(), nullptr, 10);
         else
@@ -471,8 +473,11 @@ int main(int argc, char** argv)
         const size_t rowsA = g.layout_a == R355_ROW_MAJOR ? m : k, rowsB = g.layout_b == R355_ROW_MAJOR ? k : n;
         std::vector<uint8_t> ha(sparse ? (size_t)m * k * bytesOf(inT) / 2 : rowsA * g.lda * bytesOf(inT)),
             hb(rowsB * g.ldb * bytesOf(inT));
-        fillBytes(ha, inT, 1);
-        fillBytes(hb, inT, 2);
+        if(!zeroFill)
+        {
+            fillBytes(ha, inT, 1);
+            fillBytes(hb, inT, 2);
+        }
         void *da, *db, *dd, *dmeta = nullptr;
         if(sparse)
         {
