@@ -616,6 +616,46 @@ def test_full_size_8192_sampled_rows(in_t, out_t, la, lb):
     torch.cuda.empty_cache()
 
 
+@pytest.mark.parametrize("in_t,out_t,la,lb,ldl,kernel", [(O.F16, O.F16, O.COL, O.ROW, O.ROW, "tiled"), (O.I8, O.I32, O.ROW, O.COL, O.ROW, "tiled"),
+                                                          (O.F16, O.F16, O.ROW, O.COL, O.COL, "tiled"), (O.F16, O.F32, O.ROW, O.COL, O.ROW, "simple")])
+def test_output_beyond_2_to_the_32_elements(in_t, out_t, la, lb, ldl, kernel):
+    # D has 65792 x 65536 = 2^32 + 2^24 elements (8.6 to 17 GB): element offsets into D do not fit 32 bits.  Complete rows
+    # (columns of a col-major D) on both sides of the 2^32 boundary against the oracle's rows.
+    import torch
+
+    m, n, k = 65536 + 256, 65536, 64
+    if ldl == O.COL:
+        m, n = n, m  # the long dimension is the one D's lines run along
+    if in_t == O.I8:
+        a, b = O.uniform_int8(5, m * k), O.uniform_int8(6, k * n)
+    else:
+        a, b = O.f32_to_storage(O.uniform_pm1(5, m * k), in_t), O.f32_to_storage(O.uniform_pm1(6, k * n), in_t)
+    da, db = to_device(a), to_device(b)
+    dd = device_filled(m * n, O.NP_STORAGE[out_t], 0xFF)
+    sel = {"tiled": R.KERNEL_TILED, "simple": R.KERNEL_SIMPLE}[kernel]
+    R.gemm(in_t, out_t, m, n, k, da, db, None, dd, 1.0, 0.0, la, lb, ldl, ldl, kernel=sel)
+    torch.cuda.synchronize()
+    es = np.dtype(O.NP_STORAGE[out_t]).itemsize
+    if ldl == O.ROW:
+        lines = np.array([0, 1, 32767, 65535, 65536, 65537, m - 1], dtype=np.uint32)  # rows of D; 65536 starts at element 2^32
+        want = O.gemm_rows(in_t, out_t, la, lb, m, n, k, a, b, lines)
+        length = n
+    else:
+        # columns of a col-major D are rows of D^T = B^T A^T: the oracle's rows with the operands exchanged
+        lines = np.array([0, 1, 32767, 65535, 65536, 65537, n - 1], dtype=np.uint32)
+        other = {O.ROW: O.COL, O.COL: O.ROW}
+        want = O.gemm_rows(in_t, out_t, other[lb], other[la], n, m, k, b, a, lines)
+        length = m
+    for i, line in enumerate(lines):
+        got = dd[int(line) * length * es:(int(line) + 1) * length * es].cpu().numpy().view(O.NP_STORAGE[out_t])
+        if in_t == O.I8:
+            assert np.array_equal(got, want[i]), line
+        else:
+            _check(in_t, out_t, got, want[i].ravel())
+    del da, db, dd
+    torch.cuda.empty_cache()
+
+
 def _embed(flat, rows, cols, layout, ld, fill):
     """Packed rows x cols matrix (layout) -> storage with leading dimension ld, padding = fill."""
     major, minor = (rows, cols) if layout == O.ROW else (cols, rows)
