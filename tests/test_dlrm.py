@@ -129,6 +129,35 @@ def test_fwd_full_batch_65536_properties():
     assert np.max(np.abs(tri - ident)) < 0.5  # 351 f16 roundings of values up to ~40
 
 
+def test_fwd_and_bwd_batch_beyond_4_gib_of_input():
+    # 700 000 samples of 27 x 128 f16 are 4.8 GB: byte offsets of samples from 621 379 on do not fit 32 bits.  Samples on
+    # both sides of that boundary against the oracle (every sample is independent of the others).
+    import torch
+
+    m, k, batch = 27, 128, 700000
+    tri = m * (m - 1) // 2
+    g = torch.Generator(device="cuda").manual_seed(11)
+    x = torch.randn(batch * m * k, device="cuda", generator=g).to(torch.float16)
+    up = torch.randn(batch * (k + tri), device="cuda", generator=g).to(torch.float16)
+    out = device_filled(batch * (k + tri), np.uint16)
+    R.dlrm_fwd(R.F16, x, out, m, k, batch)
+    mlp, grad = device_filled(batch * k, np.uint16), device_filled(batch * m * k, np.uint16)
+    R.dlrm_bwd(R.F16, x, up, mlp, grad, m, k, batch)
+    torch.cuda.synchronize()
+    sel = [0, 1, 310000, 621377, 621378, 621379, 621380, batch - 1]
+    take = lambda t, width: np.stack([t.view(torch.int16)[i * width:(i + 1) * width].cpu().numpy().view(np.uint16) for i in sel])
+    xs, ups = take(x, m * k), take(up, k + tri)
+    want = O.dlrm_fwd(O.F16, xs.ravel(), m, k, len(sel))
+    ok, mx = O.compare(O.F16, take(out, k + tri), want, 10.0)
+    assert ok, mx
+    wmlp, wgrad = O.dlrm_bwd(O.F16, xs.ravel(), ups.ravel(), m, k, len(sel))
+    assert np.array_equal(take(mlp, k), wmlp)
+    ok, mx = O.compare(O.F16, take(grad, m * k).ravel(), wgrad.ravel(), 10.0)
+    assert ok, mx
+    del x, up, out, mlp, grad
+    torch.cuda.empty_cache()
+
+
 @pytest.mark.parametrize("suffix", ["fp16"])
 def test_bwd_reference_fixture(suffix):
     x = np.fromfile(os.path.join(GOLD, "input_fp16"), dtype=np.uint16)
