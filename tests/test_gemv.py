@@ -49,3 +49,26 @@ def test_dgemv_vs_oracle(layout, m, k):
     want = O.gemm(O.F64, O.F64, layout, O.COL, O.COL, O.COL, m, 1, k, ai, xi, None, 1.0, 0.0)
     R.dgemv(layout, m, k, to_device(ai), to_device(xi), None, dout, 1.0, 0.0)
     assert np.array_equal(to_host(dout, np.float64), want)
+
+
+@pytest.mark.parametrize("layout", [O.ROW, O.COL])
+def test_gemv_matrix_beyond_4_gib(layout):
+    # A is 36864 x 32768 f32 = 4.8 GB: byte (and, for a 2^32-element matrix, element) offsets past 32 bits.  Sampled
+    # elements of y on both sides of the boundary against a float64 dot product of the same row of A.
+    import torch
+
+    m, k = 36864, 32768
+    g = torch.Generator(device="cuda").manual_seed(3)
+    a = torch.rand(m * k, device="cuda", generator=g) * 2 - 1
+    x = torch.rand(k, device="cuda", generator=g) * 2 - 1
+    y = torch.empty(m, device="cuda")
+    R.gemv(layout, m, k, a, x, None, y, 1.0, 0.0)
+    torch.cuda.synchronize()
+    A = a.view(m, k) if layout == O.ROW else a.view(k, m).t()
+    rows = torch.tensor([0, 1, 16383, 32767, 32768, 32769, m - 1], device="cuda")  # row 32768 starts at byte 2^32 (row-major)
+    exact = (A[rows].double() @ x.double()).cpu().numpy()
+    bound = (A[rows].abs().double() @ x.abs().double()).cpu().numpy() * k * 6e-8
+    got = y[rows].double().cpu().numpy()
+    assert np.all(np.abs(got - exact) <= bound), np.max(np.abs(got - exact) / bound)
+    # the bound sees a wrong row
+    assert not np.all(np.abs(np.roll(got, 1) - exact) <= bound)
