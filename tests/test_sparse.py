@@ -168,3 +168,32 @@ def test_sparse_macro_tile_forced_on_small_and_ragged_shapes(in_t, out_t):
         else:
             g, w = got.astype(np.float64), want.astype(np.float64)
             assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= 1e-3, (m, n, k)
+
+
+@pytest.mark.parametrize("ldl", [O.ROW, O.COL])
+def test_sparse_output_beyond_2_to_the_32_elements(ldl):
+    # D (int32, 17 GB) has 65792 x 65536 elements: offsets into it pass 32 bits.  Lines of D on both sides of the boundary
+    # against the dense oracle on the decompressed A.
+    import torch
+
+    m, n, k = (65536 + 256, 65536, 128) if ldl == O.ROW else (65536, 65536 + 256, 128)
+    dense, b = _sparse_inputs(O.I8, m, n, k, 70)
+    vals, meta = R.compress_24(dense)
+    dv, dm, db = to_device(vals), to_device(meta), to_device(b)
+    dd = device_filled(m * n, np.int32, 0xFF)
+    R.gemm(O.I8, O.I32, m, n, k, dv, db, None, dd, 1.0, 0.0, O.ROW, O.COL, ldl, ldl, a_meta=dm, kernel=R.KERNEL_TILED)
+    torch.cuda.synchronize()
+    if ldl == O.ROW:
+        lines = np.array([0, 1, 65535, 65536, 65537, m - 1], dtype=np.uint32)
+        want = O.gemm_rows(O.I8, O.I32, O.ROW, O.COL, m, n, k, dense.ravel(), b, lines)
+        length = n
+    else:
+        # columns of a col-major D are rows of D^T = B^T A^T (B col-major k x n is B^T row-major n x k)
+        lines = np.array([0, 1, 65535, 65536, 65537, n - 1], dtype=np.uint32)
+        want = O.gemm_rows(O.I8, O.I32, O.ROW, O.COL, n, m, k, b, dense.ravel(), lines)
+        length = m
+    for i, line in enumerate(lines):
+        got = dd[int(line) * length * 4:(int(line) + 1) * length * 4].cpu().numpy().view(np.int32)
+        assert np.array_equal(got, want[i]), line
+    del dv, dm, db, dd
+    torch.cuda.empty_cache()
