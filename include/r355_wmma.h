@@ -77,8 +77,8 @@ typedef enum
  * reference's static_cast narrows it), f32 -> f32 (f32), f64 -> f64 (f64).
  * beta == 0 means C is never read and may be NULL.
  *
- * sparse24 != 0: A is 2:4 structured-sparse along k (i8 -> i32, e4m3 -> f32 with a 256 x 256 macro-tile kernel for
- * m, n % 256 == 0 and a block-per-wave kernel otherwise; f16 | bf16 -> f32 with the block-per-wave kernel), B col-major:
+ * sparse24 != 0: A is 2:4 structured-sparse along k (i8 -> i32, e4m3 | f16 | bf16 -> f32; a 256 x 256 macro-tile kernel
+ * from m, n >= 128 on when B is col-major, a block-per-wave kernel otherwise, which takes B in either orientation):
  * `a` holds the m * k/2 kept values and `a_meta` the m * k/8 index bytes in the K-blocked storage that
  * r355_compress_24 / r355_compress_24_16 write (layout_a = R355_ROW_MAJOR, lda = k / 2: the storage has no padding);
  * m, n multiples of 16, k of 128 bytes' worth of elements (128 for 1-byte, 64 for 2-byte elements).

@@ -11,7 +11,8 @@
 // so that all a 256-row macro tile needs of one stage is 16 + 4 KiB of consecutive bytes (whole cache lines;
 // with row-major compressed rows a stage touched 64 + 16 bytes of every row's lines and the direct-to-LDS
 // loads ran at two thirds of the rate), and a fragment's 16 bytes per lane are consecutive across lanes.
-// B is dense, col-major (k contiguous); D row- or col-major.  m % 16 == 0, k % (128 / ES) == 0.
+// B is dense, col-major (k contiguous) for the macro tile, either orientation for the block-per-wave kernel; D row- or
+// col-major.  m % 16 == 0, k % (128 / ES) == 0.
 //
 // Two kernels:
 //   sparseTiledKernel    256 x 256 macro tile, one K step of 128 bytes per stage, a ring of three LDS slots filled
@@ -58,6 +59,7 @@ namespace
                                                                                uint32_t       ldb,
                                                                                uint32_t       ldc,
                                                                                uint32_t       ldd,
+                                                                               layout_t       layoutB,
                                                                                layout_t       layoutC,
                                                                                layout_t       layoutD,
                                                                                AccE           alpha,
@@ -67,7 +69,7 @@ namespace
         constexpr uint32_t BK   = S::StageK; // one stage per trip
         using FragA             = fragment<sparse_matrix_a, Blk, Blk, BK, InT, row_major>;
         using FragMeta          = fragment<sparse_metadata, Blk, Blk, BK, InT>;
-        using FragB             = fragment<matrix_b, Blk, Blk, BK, InT, col_major>;
+        using FragB             = fragment<matrix_b, Blk, Blk, BK, InT>; // orientation given at run time
         using FragAcc           = fragment<accumulator, Blk, Blk, BK, AccE>;
         const uint32_t row = (blockIdx.x * WAVES_X + threadIdx.x / 64u) * Blk;
         const uint32_t col = (blockIdx.y * WAVES_Y + threadIdx.y) * Blk;
@@ -75,7 +77,9 @@ namespace
             return;
         const InT*     pa = aVals + S::valueOffset(row, 0u, m);
         const uint8_t* pm = aMeta + S::metaOffset(row, 0u, m);
-        const InT*     pb = b + (uint64_t)col * ldb;
+        const bool     bCol = layoutB == mem_col_major;
+        const InT*     pb   = bCol ? b + (uint64_t)col * ldb : b + col;
+        const uint64_t stepB = bCol ? (uint64_t)BK : (uint64_t)BK * ldb; // one stage further along k
         const uint32_t strideV = S::valueStageStride(m), strideM = S::metaStageStride(m);
 
         FragA    fragA;
@@ -87,9 +91,9 @@ namespace
         {
             load_matrix_sync(fragA, pa, strideV);
             load_matrix_sync(fragMeta, pm, strideM);
-            load_matrix_sync(fragB, pb, ldb);
+            load_matrix_sync(fragB, pb, ldb, layoutB);
             mma_sync(fragAcc, fragA, fragMeta, fragB, fragAcc);
-            pa += strideV, pm += strideM, pb += BK;
+            pa += strideV, pm += strideM, pb += stepB;
         }
         const uint64_t offC = layoutC == mem_row_major ? (uint64_t)row * ldc + col : (uint64_t)col * ldc + row;
         const uint64_t offD = layoutD == mem_row_major ? (uint64_t)row * ldd + col : (uint64_t)col * ldd + row;
@@ -466,7 +470,7 @@ namespace
     {
         const uint32_t es = (g.in_type == R355_F16 || g.in_type == R355_BF16) ? 2u : 1u;
         const bool     shape = g.kernel == R355_KERNEL_TILED || (g.m >= T_M / 2 && g.n >= T_N / 2);
-        return g.kernel != R355_KERNEL_SIMPLE && shape && g.layout_c == g.layout_d && r355::aligned(g.a_meta, 16)
+        return g.kernel != R355_KERNEL_SIMPLE && shape && g.layout_b == R355_COL_MAJOR && g.layout_c == g.layout_d && r355::aligned(g.a_meta, 16)
                && (uint64_t)g.ldb * es <= (1u << 23);
     }
 
@@ -485,8 +489,8 @@ namespace r355
         const bool w  = (g.in_type == R355_F16 || g.in_type == R355_BF16) && g.out_type == R355_F32;
         if(!i8 && !f8 && !w)
             return fail(R355_ERR_UNSUPPORTED, "sparse gemm: supported types are i8 -> i32 and e4m3 | f16 | bf16 -> f32");
-        if(g.layout_a != R355_ROW_MAJOR || g.layout_b != R355_COL_MAJOR)
-            return fail(R355_ERR_UNSUPPORTED, "sparse gemm: compressed A is K-blocked row storage (R355_ROW_MAJOR) and B must be col-major");
+        if(g.layout_a != R355_ROW_MAJOR)
+            return fail(R355_ERR_UNSUPPORTED, "sparse gemm: compressed A is K-blocked row storage (R355_ROW_MAJOR)");
         if(!g.a_meta)
             return fail(R355_ERR_BAD_ARG, "sparse gemm: a_meta is null");
         const uint32_t es = w ? 2u : 1u, kStage = 128u / es; // element bytes, dense k per stage of the storage format
@@ -500,7 +504,8 @@ namespace r355
         if(g.kernel == R355_KERNEL_TILED_128 || g.kernel == R355_KERNEL_TILED_128_SPLITK)
             return fail(R355_ERR_UNSUPPORTED, "sparse gemm: there is no 128 x 128 sparse macro tile (R355_KERNEL_TILED is 256 x 256)");
         if(g.kernel == R355_KERNEL_TILED && !tiledOk(g))
-            return fail(R355_ERR_UNSUPPORTED, "sparse gemm (macro tile): C and D must share an orientation, metadata 16-byte aligned, ldb below 8 MiB");
+            return fail(R355_ERR_UNSUPPORTED,
+                        "sparse gemm (macro tile): B must be col-major, C and D must share an orientation, metadata 16-byte aligned, ldb below 8 MiB");
         if(plan && tiledOk(g))
         {
             plan->kernel       = R355_KERNEL_TILED;
@@ -535,12 +540,13 @@ namespace r355
         const uint32_t blk = simpleBlock(g);
         dim3           block(WAVES_X * 64, WAVES_Y);
         dim3           grid((g.m + blk * WAVES_X - 1) / (blk * WAVES_X), (g.n + blk * WAVES_Y - 1) / (blk * WAVES_Y));
+        const layout_t lb = g.layout_b == R355_ROW_MAJOR ? mem_row_major : mem_col_major;
         const layout_t lc = g.layout_c == R355_ROW_MAJOR ? mem_row_major : mem_col_major;
         const layout_t ld = g.layout_d == R355_ROW_MAJOR ? mem_row_major : mem_col_major;
         auto           go = [&](auto kernel) {
             hipLaunchKernelGGL(kernel, grid, block, 0, stream, g.m, g.n, g.k, static_cast<const InT*>(g.a),
                                static_cast<const uint8_t*>(g.a_meta), static_cast<const InT*>(g.b), static_cast<const AccE*>(g.c),
-                               static_cast<AccE*>(g.d), g.ldb, g.ldc, g.ldd, lc, ld, static_cast<AccE>(g.alpha), static_cast<AccE>(g.beta));
+                               static_cast<AccE*>(g.d), g.ldb, g.ldc, g.ldd, lb, lc, ld, static_cast<AccE>(g.alpha), static_cast<AccE>(g.beta));
         };
         if(blk == 32u)
             go(sparseBlockPerWave<InT, AccE, 32>);

@@ -104,6 +104,44 @@ def test_sparse_gemm_16bit_vs_dense_oracle(in_t, m, n, k, ldl):
     assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= 1e-3
 
 
+@pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32), (O.F16, O.F32), (O.BF16, O.F32)])
+@pytest.mark.parametrize("m,n,k", [(32, 32, 128), (16, 48, 256), (272, 144, 384)])
+@pytest.mark.parametrize("ldl", [O.ROW, O.COL])
+def test_sparse_gemm_row_major_b(in_t, out_t, m, n, k, ldl):
+    """B (k x n) with n contiguous: the block-per-wave kernel takes either orientation of B (the macro tile wants
+    K-contiguous columns and is not chosen), against the oracle's dense GEMM with the same orientation."""
+    mask = O.sparse24_mask(80, m, k)
+    if in_t == O.I8:
+        dense = np.where(mask, O.uniform_int8(81, m * k).reshape(m, k), np.int8(0)).astype(np.int8)
+        b = O.uniform_int8(82, k * n)
+        storage = dense
+    elif in_t == O.E4M3:
+        dense = np.where(mask, O.f32_to_storage(O.normal(81, m * k), O.E4M3).view(np.int8).reshape(m, k), np.int8(0)).astype(np.int8)
+        b = O.f32_to_storage(O.normal(82, k * n), O.E4M3)
+        storage = dense.view(np.uint8)
+    else:
+        dense = np.where(mask, O.f32_to_storage(O.uniform_pm1(81, m * k), in_t).reshape(m, k), np.uint16(0)).astype(np.uint16)
+        b = O.f32_to_storage(O.uniform_pm1(82, k * n), in_t)
+        storage = dense
+    vals, meta = R.compress_24(dense)
+    c = (O.uniform_int8(83, m * n).astype(np.int32) * 7) if in_t == O.I8 else O.uniform_pm1(83, m * n)
+    want = O.gemm(in_t, out_t, O.ROW, O.ROW, ldl, ldl, m, n, k, storage.ravel(), b, c, 1.0, 1.0)
+    dv, dm, db, dc = to_device(vals), to_device(meta), to_device(b), to_device(c)
+    dd = device_filled(m * n, O.NP_STORAGE[out_t], 0xFF)
+    args = R.gemm_args(in_t, out_t, m, n, k, dv, db, dc, dd, 1.0, 1.0, O.ROW, O.ROW, ldl, ldl, a_meta=dm)
+    assert R.gemm_query(args).kernel == R.KERNEL_SIMPLE
+    R.gemm(in_t, out_t, m, n, k, dv, db, dc, dd, 1.0, 1.0, O.ROW, O.ROW, ldl, ldl, a_meta=dm)
+    got = to_host(dd, O.NP_STORAGE[out_t])
+    if in_t == O.I8:
+        assert np.array_equal(got, want)
+    else:
+        g, w = got.astype(np.float64), want.astype(np.float64)
+        assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= (1e-2 if in_t == O.E4M3 else 1e-3)
+    with pytest.raises(R.R355Error) as e:  # the macro tile cannot be forced onto a row-major B
+        R.gemm_query(R.gemm_args(in_t, out_t, m, n, k, dv, db, dc, dd, 1.0, 1.0, O.ROW, O.ROW, ldl, ldl, a_meta=dm, kernel=R.KERNEL_TILED))
+    assert e.value.code == -2
+
+
 def test_sparse_16bit_one_hot_positions():
     """Every (row, kept position) of A in turn is the only non-zero: D must be that row of B scaled - exact, and it
     fails for any wrong pairing of lane groups or index bits."""
