@@ -56,6 +56,21 @@ namespace
             return __builtin_bit_cast(uint16_t, static_cast<_Float16>(v));
     }
 
+    // A run of `bytes` bytes at base + offset (wave-uniform) as a raw buffer: a lane whose offset lies beyond it loads zeros
+    // (stores nothing) without touching memory.  Loads and stores through it need no branches, so every vector-memory
+    // instruction is issued on every path and the compiler can count them: the wait for one sample's loads then leaves
+    // the next sample's loads and the previous sample's stores in flight.  (With a branch around each guarded access the
+    // number of younger operations is unknown and every wait becomes "until nothing is outstanding".)
+    __device__ inline __amdgpu_buffer_rsrc_t runBuffer(const void* base, uint64_t offset, uint32_t bytes)
+    {
+        const uint64_t addr = reinterpret_cast<uint64_t>(base) + offset;
+        const uint32_t lo   = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(addr));
+        const uint32_t hi   = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(addr >> 32));
+        return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>((static_cast<uint64_t>(hi) << 32) | lo), 0,
+                                                 static_cast<int>(__builtin_amdgcn_readfirstlane(bytes)), 0x00020000);
+    }
+    constexpr int NONTEMPORAL = 2; // cache-policy bits of the raw buffer builtins: nt
+
     // K is a template parameter (32, 64, 128, 256): rows of X are K * 2 bytes = K / 8 chunks.
     // ROWS (28 or 32) bounds m: the LDS image of a sample holds ROWS rows, which at m <= 28 and
     // K = 128 lets four workgroups share a CU instead of three.
@@ -72,34 +87,29 @@ namespace
 
         const uint32_t tid       = threadIdx.x;
         const uint32_t lane      = tid & 63u;
-        const uint32_t wave      = tid >> 6;
+        const uint32_t wave      = __builtin_amdgcn_readfirstlane(tid >> 6);
         const uint32_t outStride = K + m * (m - 1) / 2; // elements per sample
         const uint32_t b0        = blockIdx.x * SAMPLES_PER_WG;
-        const uint32_t inChunks  = m * ROW_CHUNKS; // 16-byte chunks of one sample
+        const uint32_t inBytes   = m * K * 2u; // of one sample
 
         char* xw = xLds[wave];
         // rows m..31 of the 32 x 32 product are padding: their lanes feed zeros (see below)
 
         // Both samples of this wave are requested from HBM before either is consumed: the kernel is
-        // bandwidth-bound, and bytes in flight per CU are what keeps HBM busy.
+        // bandwidth-bound, and bytes in flight per CU are what keeps HBM busy.  The loads go through a raw buffer of
+        // exactly the sample's bytes (runBuffer; none for a sample beyond the batch), so the first sample is consumed
+        // while the second is still arriving.
         constexpr uint32_t PER_WAVE   = SAMPLES_PER_WG / WAVES; // 2
         constexpr uint32_t MAX_CHUNKS = (ROWS * ROW_CHUNKS + 63u) / 64u; // loads per lane per sample
         i32x4              stash[PER_WAVE][MAX_CHUNKS];
 #pragma unroll
         for(uint32_t q = 0; q < PER_WAVE; ++q)
         {
-            const uint32_t b = b0 + wave + q * WAVES;
-            if(b < batch)
-            {
-                const char* src = reinterpret_cast<const char*>(in) + (uint64_t)b * m * K * 2u;
+            const uint32_t b   = b0 + wave + q * WAVES;
+            const auto     src = runBuffer(in, (uint64_t)(b < batch ? b : 0u) * inBytes, b < batch ? inBytes : 0u);
 #pragma unroll
-                for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
-                {
-                    const uint32_t c = j * 64u + lane;
-                    if(c < inChunks)
-                        stash[q][j] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(src + c * 16u)); // read once
-                }
-            }
+            for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
+                stash[q][j] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (j * 64u + lane) * 16u, 0, NONTEMPORAL)); // read once
         }
 
 #pragma unroll
@@ -110,11 +120,12 @@ namespace
             if(b >= batch)
                 break;
             // ---- X -> LDS: chunk c of the sample goes to row c / ROW_CHUNKS, slot (c % ROW_CHUNKS) ^ (row % 16)
+            // (chunks of rows m .. ROWS - 1 arrived as zeros and are written like the others: those rows are never used)
 #pragma unroll
             for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
             {
                 const uint32_t c = j * 64u + lane;
-                if(c < inChunks)
+                if(c < ROWS * ROW_CHUNKS)
                 {
                     const uint32_t row  = c / ROW_CHUNKS, col = c % ROW_CHUNKS;
                     const uint32_t slot = col ^ (row & (ROW_CHUNKS - 1u) & 15u);
@@ -168,61 +179,70 @@ namespace
     }
 
     // f32 variant.  An f32 sample is 13.8 KB, so only a few fit in LDS per CU and the matrix core
-    // (v_mfma_f32_16x16x4_f32, 96 instructions per sample) is busy a good third of the time: the loads
-    // of a wave's next sample are therefore issued before the current sample is computed, and every
-    // wave walks F32_PER_WAVE consecutive samples, writing each result row from its own LDS image
-    // with coalesced 4-byte stores (a sample's output row is only 4-byte aligned).
-    constexpr uint32_t F32_PER_WAVE = 8;
+    // (v_mfma_f32_16x16x4_f32, 96 instructions per sample) is busy a good third of the time.  A wave walks the samples
+    // first, first + stride, ... (stride = the launch's waves); a sample's loads are requested as soon as the sample two
+    // steps before has been unloaded from its register stash into LDS, and each result row leaves from the wave's own
+    // LDS image with coalesced 4-byte stores (a sample's output row is only 4-byte aligned) that are still in flight when
+    // the next sample is taken up.  The launch gives every wave F32_STEPS samples: two workgroups share a CU and the
+    // older one is served first, so with long walks (one launch-wide round of workgroups) the first half of the
+    // workgroups finished after 135 us of 198 and the others ran the rest of the time alone, one wave per SIMD with
+    // nothing to overlap its phases; short walks let the dispatcher refill a CU as soon as a workgroup ends
+    // (0.196 ms with 32 samples per wave, 0.183 with 4, 0.178 with 2 at a batch of 65536).
+    constexpr uint32_t F32_STEPS = 2;
 
     template <uint32_t K, uint32_t ROWS>
-    __global__ void __launch_bounds__(THREADS)
+    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2)))
         dlrmFwdF32Kernel(const float* __restrict__ in, float* __restrict__ out, uint32_t m, uint32_t batch)
     {
         constexpr uint32_t ROW_CHUNKS = K / 4; // 16-byte chunks per row
         constexpr uint32_t MAX_OUT    = K + ROWS * (ROWS - 1) / 2;
+        constexpr uint32_t OUT_STEPS  = (MAX_OUT + 63u) / 64u; // 4-byte stores per lane and sample
         constexpr uint32_t MAX_CHUNKS = (ROWS * ROW_CHUNKS + 63u) / 64u;
-        constexpr uint32_t SWZ        = 31u & (ROW_CHUNKS - 1u);
+        // Rows of the LDS image are one chunk longer than the data: (K + 4) / 4 is odd, so the 16 rows x 4 k values that
+        // one operand read touches fall into 64 different banks, and a row's chunks keep their order (every read and
+        // write of the image is one lane address plus a constant).
+        constexpr uint32_t ROWP       = K * 4u + 16u;
         using f32x4                   = float __attribute__((ext_vector_type(4)));
 
-        __shared__ __attribute__((aligned(16))) float xLds[WAVES][ROWS * K];
-        __shared__ __attribute__((aligned(16))) float outLds[WAVES][MAX_OUT];
+        __shared__ __attribute__((aligned(16))) char  xLds[WAVES][ROWS * ROWP];
+        __shared__ __attribute__((aligned(16))) float outLds[WAVES][OUT_STEPS * 64u];
 
-        const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+        const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const uint32_t outStride = K + m * (m - 1) / 2;
-        const uint32_t inChunks  = m * ROW_CHUNKS;
-        const uint32_t first     = (blockIdx.x * WAVES + wave) * F32_PER_WAVE; // this wave's first sample
-        char*          xw        = reinterpret_cast<char*>(xLds[wave]);
+        const uint32_t inBytes   = m * K * 4u;
+        // a wave walks the samples first, first + stride, ...: what the four waves of a workgroup request at one time is
+        // one run of consecutive bytes
+        const uint32_t first = blockIdx.x * WAVES + wave, stride = gridDim.x * WAVES;
+        char*          xw        = xLds[wave];
         float*         o         = outLds[wave];
 
-        f32x4 stash[2][MAX_CHUNKS];
-        auto  request = [&](uint32_t b, f32x4 (&dst)[MAX_CHUNKS]) {
-            if(b < batch)
-            {
-                const char* src = reinterpret_cast<const char*>(in) + (uint64_t)b * m * K * 4u;
+        // Two register stashes, used in turn: the loads of the next two samples are in flight while one is computed
+        // (a wave holds 2 x 13.8 KB in flight, a CU's eight waves 220 KB).
+        // (a sample beyond the batch is a buffer of no bytes: the loads are issued and move nothing)
+        f32x4 stashA[MAX_CHUNKS], stashB[MAX_CHUNKS];
+        auto  request = [&](f32x4 (&stash)[MAX_CHUNKS], uint64_t b) {
+            const bool valid = b < batch;
+            const auto src   = runBuffer(in, (uint64_t)(valid ? b : 0u) * inBytes, valid ? inBytes : 0u);
 #pragma unroll
-                for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
-                {
-                    const uint32_t c = j * 64u + lane;
-                    if(c < inChunks)
-                        dst[j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src + c * 16u));
-                }
-            }
+            for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
+                stash[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (j * 64u + lane) * 16u, 0, NONTEMPORAL));
         };
-        auto process = [&](uint32_t b, const f32x4 (&src)[MAX_CHUNKS]) {
-            if(b >= batch)
-                return;
+        // sample b from its stash, which then takes the sample two steps further on
+        auto process = [&](f32x4 (&stash)[MAX_CHUNKS], uint64_t b) {
+            // chunks of rows m .. ROWS - 1 arrive as zeros and are written like the others: those rows are never used
 #pragma unroll
             for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
             {
                 const uint32_t c = j * 64u + lane;
-                if(c < inChunks)
+                if(c < ROWS * ROW_CHUNKS)
                 {
                     const uint32_t row = c / ROW_CHUNKS, col = c % ROW_CHUNKS;
-                    *reinterpret_cast<f32x4*>(xw + (row * ROW_CHUNKS + (col ^ (row & SWZ))) * 16u) = src[j];
+                    *reinterpret_cast<f32x4*>(xw + row * ROWP + col * 16u) = stash[j];
                 }
             }
             __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_wave_barrier();
+            request(stash, b + 2u * stride); // the stash is free again
 
             // v_mfma_f32_16x16x4_f32 on the three 16 x 16 blocks of the Gram matrix that hold its lower
             // triangle (rows < 16 x rows < 16, rows >= 16 x rows < 16, rows >= 16 x rows >= 16): a quarter
@@ -233,22 +253,40 @@ namespace
             const uint32_t r16 = lane & 15u, kq = lane >> 4;
             const bool     validLo = r16 < m, validHi = 16u + r16 < m;
             const uint32_t rowLo = validLo ? r16 : 0u, rowHi = validHi ? 16u + r16 : 0u;
-#pragma unroll 8
-            for(uint32_t s = 0; s < K / 4; ++s)
+            // eight steps of k (24 matrix instructions, 768 matrix-core clocks) per group; a group's 16 operand reads are
+            // issued before the previous group's matrix instructions, so what the reads wait for in the LDS queue (the
+            // other waves' 16-byte writes take 13 clocks each) is not what the matrix core waits for
+            constexpr uint32_t GROUP = (ROWS > 28u && K > 64u) ? 4u : 8u, GROUPS = K / 4 / GROUP; // (registers: two waves per SIMD)
+            float              xl[2][GROUP], xh[2][GROUP];
+            auto fetch = [&](uint32_t grp, float (&lo)[GROUP], float (&hi)[GROUP]) {
+#pragma unroll
+                for(uint32_t u = 0; u < GROUP; ++u)
+                {
+                    const uint32_t s = grp * GROUP + u;
+                    lo[u] = *reinterpret_cast<const float*>(xw + rowLo * ROWP + kq * 4u + s * 16u);
+                    hi[u] = *reinterpret_cast<const float*>(xw + rowHi * ROWP + kq * 4u + s * 16u);
+                }
+            };
+            fetch(0, xl[0], xh[0]);
+#pragma unroll
+            for(uint32_t grp = 0; grp < GROUPS; ++grp)
             {
-                float xl = *reinterpret_cast<const float*>(xw + (rowLo * ROW_CHUNKS + (s ^ (rowLo & SWZ))) * 16u + kq * 4u);
-                float xh = *reinterpret_cast<const float*>(xw + (rowHi * ROW_CHUNKS + (s ^ (rowHi & SWZ))) * 16u + kq * 4u);
-                if(!validLo)
-                    xl = 0.0f;
-                if(!validHi)
-                    xh = 0.0f;
-                accLL = __builtin_amdgcn_mfma_f32_16x16x4f32(xl, xl, accLL, 0, 0, 0);
-                accHL = __builtin_amdgcn_mfma_f32_16x16x4f32(xh, xl, accHL, 0, 0, 0);
-                accHH = __builtin_amdgcn_mfma_f32_16x16x4f32(xh, xh, accHH, 0, 0, 0);
+                if(grp + 1u < GROUPS)
+                    fetch(grp + 1u, xl[(grp + 1u) & 1u], xh[(grp + 1u) & 1u]);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for(uint32_t u = 0; u < GROUP; ++u)
+                {
+                    const float lo = validLo ? xl[grp & 1u][u] : 0.0f, hi = validHi ? xh[grp & 1u][u] : 0.0f;
+                    accLL          = __builtin_amdgcn_mfma_f32_16x16x4f32(lo, lo, accLL, 0, 0, 0);
+                    accHL          = __builtin_amdgcn_mfma_f32_16x16x4f32(hi, lo, accHL, 0, 0, 0);
+                    accHH          = __builtin_amdgcn_mfma_f32_16x16x4f32(hi, hi, accHH, 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
 
             for(uint32_t e = lane; e < K; e += 64)
-                o[e] = reinterpret_cast<const float*>(xw)[e]; // row 0 is stored unswizzled
+                o[e] = reinterpret_cast<const float*>(xw)[e]; // row 0
             // a 16 x 16 result block: lane holds rows 4 (lane / 16) + e, column lane % 16
 #pragma unroll
             for(uint32_t e = 0; e < 4; ++e)
@@ -266,22 +304,28 @@ namespace
             }
             __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_wave_barrier();
-            float* dst = out + (uint64_t)b * outStride;
-            for(uint32_t e = lane; e < outStride; e += 64)
-                __builtin_nontemporal_store(o[e], dst + e);
+            const auto dst = runBuffer(out, (uint64_t)(b < batch ? b : 0u) * outStride * 4u, b < batch ? outStride * 4u : 0u);
+#pragma unroll
+            for(uint32_t e = 0; e < OUT_STEPS; ++e)
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, o[e * 64u + lane]), dst, (e * 64u + lane) * 4u, 0, NONTEMPORAL);
             __builtin_amdgcn_s_waitcnt(0xC07F); // the image is rewritten by the next sample
             __builtin_amdgcn_wave_barrier();
         };
 
-        request(first, stash[0]);
+        // The first two samples stand outside the loop so that the loop is entered with the same operations in flight
+        // as its own trips leave behind (loads, stores, loads, stores): the waits inside are then exact on both paths.
+        // (A sample index is 64-bit here: the walk looks two steps beyond the batch.)
+        if(first >= batch)
+            return;
+        request(stashA, first);
+        request(stashB, (uint64_t)first + stride);
+        process(stashA, first);
+        process(stashB, (uint64_t)first + stride);
 #pragma unroll 1
-        for(uint32_t it = 0; it < F32_PER_WAVE; it += 2)
+        for(uint64_t b = (uint64_t)first + 2u * stride; b < batch; b += 2u * stride)
         {
-            request(first + it + 1u, stash[1]);
-            process(first + it, stash[0]);
-            if(it + 2u < F32_PER_WAVE)
-                request(first + it + 2u, stash[0]);
-            process(first + it + 1u, stash[1]);
+            process(stashA, b);
+            process(stashB, b + stride);
         }
     }
 
@@ -482,8 +526,8 @@ namespace
     // f32 backward.  grad (m x k) = S X with S = T + T^T from the upstream triangle, on
     // v_mfma_f32_16x16x4_f32: A operand = a 16 x 4 piece of S (lane l: row l % 16, column l / 16), B
     // operand = a 4 x 16 piece of X (lane l: row l / 16, column l % 16), 2 x (k / 16) result blocks, 8
-    // steps over the 32 (zero-padded) rows of X.  Every wave walks F32_PER_WAVE consecutive samples with
-    // the loads of the next one in flight.  Per sample: X goes to an LDS image whose 64-byte column
+    // steps over the 32 (zero-padded) rows of X.  Every wave walks F32_STEPS samples (first, first + stride, ...) with the
+    // loads of the next sample in flight.  Per sample: X goes to an LDS image whose 64-byte column
     // groups are XOR-swizzled with the row (four consecutive rows of one column group land in
     // different banks), the upstream row to a second image from which each lane gathers its 16 values
     // of S; the gradient is written over X and leaves with 128-bit nontemporal stores; the first k
@@ -503,22 +547,19 @@ namespace
         using f32x4                   = float __attribute__((ext_vector_type(4)));
 
         __shared__ __attribute__((aligned(16))) char  xLds[WAVES][MAX_M * ROWB];
-        __shared__ __attribute__((aligned(16))) float upLds[WAVES][MAX_UP];
+        __shared__ __attribute__((aligned(16))) float upLds[WAVES][UP_WORDS * 64u];
 
-        const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+        const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const uint32_t upStride = K + m * (m - 1) / 2;
-        const uint32_t inChunks = m * ROW_CHUNKS;
-        const uint32_t first    = (blockIdx.x * WAVES + wave) * F32_PER_WAVE;
+        const uint32_t inBytes  = m * ROWB;
+        // a wave walks the samples first, first + stride, ...
+        const uint32_t first = blockIdx.x * WAVES + wave, stride = gridDim.x * WAVES;
         char*          xw       = xLds[wave];
         float*         uw       = upLds[wave];
         const uint32_t r16 = lane & 15u, q4 = lane >> 4;
 
         // byte address of 16-byte chunk c (0 .. ROW_CHUNKS) of row `row` in the swizzled image
         auto chunkAt = [&](uint32_t row, uint32_t c) { return row * ROWB + ((((c >> 2) ^ (row & SWZ)) << 2) + (c & 3u)) * 16u; };
-
-        // rows >= m of the image stay zero for every sample
-        for(uint32_t c = inChunks + lane; c < MAX_M * ROW_CHUNKS; c += 64u)
-            *reinterpret_cast<f32x4*>(xw + chunkAt(c / ROW_CHUNKS, c % ROW_CHUNKS)) = f32x4{0, 0, 0, 0};
 
         // where lane l finds S(i, j) in the upstream image: the strict lower triangle is stored row by
         // row behind the first k values; the diagonal is zero (recomputed per sample: registers are
@@ -529,52 +570,43 @@ namespace
         };
 
         // one register stash: a sample's loads are requested while the previous sample is computed and
-        // unloaded into LDS before the next request reuses the registers
+        // unloaded into LDS before the next request reuses the registers.  All loads and stores go through raw
+        // buffers of exactly the sample's bytes (runBuffer): no branches, every wait exact.  (A sample beyond the batch
+        // is a buffer of no bytes.)  Chunks of rows >= m arrive as zeros, which is what the
+        // product needs there.
         f32x4 xs[X_CHUNKS];
         float us[UP_WORDS];
-        auto  request = [&](uint32_t b) {
-            if(b < batch)
-            {
-                const char*  src = reinterpret_cast<const char*>(in) + (uint64_t)b * m * ROWB;
-                const float* up  = upstream + (uint64_t)b * upStride;
+        auto  request = [&](uint64_t b) {
+            const bool valid = b < batch;
+            const auto src   = runBuffer(in, (uint64_t)(valid ? b : 0u) * inBytes, valid ? inBytes : 0u);
+            const auto up    = runBuffer(upstream, (uint64_t)(valid ? b : 0u) * upStride * 4u, valid ? upStride * 4u : 0u);
 #pragma unroll
-                for(uint32_t j = 0; j < X_CHUNKS; ++j)
-                    if(j * 64u + lane < inChunks)
-                        xs[j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(src + (j * 64u + lane) * 16u));
+            for(uint32_t j = 0; j < X_CHUNKS; ++j)
+                xs[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (j * 64u + lane) * 16u, 0, NONTEMPORAL));
 #pragma unroll
-                for(uint32_t j = 0; j < UP_WORDS; ++j)
-                    if(j * 64u + lane < upStride)
-                        us[j] = __builtin_nontemporal_load(up + j * 64u + lane);
-            }
+            for(uint32_t j = 0; j < UP_WORDS; ++j)
+                us[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(up, (j * 64u + lane) * 4u, 0, NONTEMPORAL));
         };
 
-        request(first);
-#pragma unroll 1
-        for(uint32_t it = 0; it < F32_PER_WAVE; ++it)
-        {
-            const uint32_t b = first + it;
-            if(b >= batch)
-                break;
+        auto process = [&](uint64_t b) {
 #pragma unroll
             for(uint32_t j = 0; j < X_CHUNKS; ++j)
             {
-                const uint32_t c = j * 64u + lane;
-                if(c < inChunks)
-                    *reinterpret_cast<f32x4*>(xw + chunkAt(c / ROW_CHUNKS, c % ROW_CHUNKS)) = xs[j];
+                const uint32_t c = j * 64u + lane; // (X_CHUNKS * 64 chunks are exactly the 32 rows of the image)
+                *reinterpret_cast<f32x4*>(xw + chunkAt(c / ROW_CHUNKS, c % ROW_CHUNKS)) = xs[j];
             }
 #pragma unroll
             for(uint32_t j = 0; j < UP_WORDS; ++j)
-                if(j * 64u + lane < upStride)
-                    uw[j * 64u + lane] = us[j];
+                uw[j * 64u + lane] = us[j];
             __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_wave_barrier();
-            if(it + 1u < F32_PER_WAVE)
-                request(b + 1u);
+            request(b + stride);
 
             // bottom-MLP gradient: the first k upstream values
-            float* mg = mlpGrad + (uint64_t)b * K;
-            for(uint32_t e = lane; e < K; e += 64u)
-                __builtin_nontemporal_store(uw[e], mg + e);
+            const auto mg = runBuffer(mlpGrad, (uint64_t)b * K * 4u, K * 4u);
+#pragma unroll
+            for(uint32_t e = 0; e < (K + 63u) / 64u; ++e)
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, uw[e * 64u + lane]), mg, (e * 64u + lane) * 4u, 0, NONTEMPORAL);
 
             float sv[2][8];
 #pragma unroll
@@ -619,18 +651,28 @@ namespace
                     }
             __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_wave_barrier();
-            char* dst = reinterpret_cast<char*>(inGrad) + (uint64_t)b * m * ROWB;
+            const auto dst = runBuffer(inGrad, (uint64_t)b * inBytes, inBytes);
 #pragma unroll
             for(uint32_t j = 0; j < X_CHUNKS; ++j)
             {
                 const uint32_t c = j * 64u + lane;
-                if(c < inChunks)
-                    __builtin_nontemporal_store(*reinterpret_cast<const f32x4*>(xw + chunkAt(c / ROW_CHUNKS, c % ROW_CHUNKS)),
-                                                reinterpret_cast<f32x4*>(dst + c * 16u));
+                using u32x4      = uint32_t __attribute__((ext_vector_type(4)));
+                __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(xw + chunkAt(c / ROW_CHUNKS, c % ROW_CHUNKS)), dst,
+                                                       c * 16u, 0, NONTEMPORAL);
             }
             __builtin_amdgcn_s_waitcnt(0xC07F); // the images are rewritten by the next sample
             __builtin_amdgcn_wave_barrier();
-        }
+        };
+
+        // The first sample stands outside the loop so that the loop is entered with the same operations in flight as
+        // its own trips leave behind: the waits inside are then exact on both paths.
+        if(first >= batch)
+            return;
+        request(first);
+        process(first);
+#pragma unroll 1
+        for(uint64_t b = (uint64_t)first + stride; b < batch; b += stride)
+            process(b);
     }
 
     int checkArgs(const char* what, int32_t dtype, const void* in, const void* out, uint32_t m, uint32_t k, uint32_t batch,
@@ -662,8 +704,8 @@ extern "C" int r355_dlrm_fwd(int32_t dtype, const void* in, void* out, uint32_t 
     hipStream_t s = static_cast<hipStream_t>(stream);
     if(dtype == R355_F32)
     {
-        const uint32_t perWg = WAVES * F32_PER_WAVE;
-        const dim3     grid32((batch + perWg - 1) / perWg), block32(THREADS);
+        const uint32_t steps = (batch + WAVES - 1) / WAVES; // of one sample per wave
+        const dim3     grid32((steps + F32_STEPS - 1) / F32_STEPS), block32(THREADS);
         auto*      fi = static_cast<const float*>(in);
         auto*      fo = static_cast<float*>(out);
 #define R355_FWD32(KK)                                                                                \
@@ -727,8 +769,8 @@ extern "C" int r355_dlrm_bwd(int32_t dtype, const void* in, const void* upstream
     {
         if(!r355::aligned(upstream, 4) || !r355::aligned(mlp_grad, 4))
             return r355::fail(R355_ERR_MISALIGNED, "dlrm_bwd: upstream and mlp_grad must be 4-byte aligned");
-        const uint32_t perWg = WAVES * F32_PER_WAVE;
-        const dim3     grid32((batch + perWg - 1) / perWg), block32(THREADS);
+        const uint32_t steps = (batch + WAVES - 1) / WAVES; // of one sample per wave
+        const dim3     grid32((steps + F32_STEPS - 1) / F32_STEPS), block32(THREADS);
         hipStream_t    s32 = static_cast<hipStream_t>(stream);
         auto*          fi  = static_cast<const float*>(in);
         auto*          fu  = static_cast<const float*>(upstream);

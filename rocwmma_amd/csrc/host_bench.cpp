@@ -12,7 +12,7 @@
 //   host_bench dlrm  [--type f16|bf16|f32] [--bwd 1] [--batch B --m M --k K] [--warmup W --iters I]
 //   host_bench gemv  [--m M --k K --layout n|t]
 //   host_bench copy  [--bytes N]      plain device copy of known size (counter calibration)
-//   host_bench lds   [--iters I]      LDS read instructions from fixed conflict-free addresses with 4, 2 and 1 waves per CU:
+//   host_bench lds   [--iters I]      LDS read and write instructions from fixed conflict-free addresses with 4, 2 and 1 waves per CU:
 //                                     shader clocks per wave-level read and bytes per clock per CU
 //   host_bench fill                   direct global -> LDS loads alone, in the access stream of the 8192^3 1-byte GEMM
 //                                     (1024 tiles x 64 stages x 64 KiB), 1 - 3 stages in flight: aggregate TB/s
@@ -236,6 +236,14 @@ namespace
                     "+14336\n\t"                                                                                        \
                  : "=v"(R0[0]), "=v"(R0[1]), "=v"(R0[2]), "=v"(R0[3]), "=v"(R0[4]), "=v"(R0[5]), "=v"(R0[6]), "=v"(R0[7])  \
                  : "v"(addr))
+#define R355_WR8(OP, R0, OFFB)                                                                                          \
+    asm volatile(OP " %8, %0 offset:" #OFFB "+0\n\t" OP " %8, %1 offset:" #OFFB "+2048\n\t" OP " %8, %2 offset:" #OFFB      \
+                    "+4096\n\t" OP " %8, %3 offset:" #OFFB "+6144\n\t" OP " %8, %4 offset:" #OFFB "+8192\n\t" OP          \
+                    " %8, %5 offset:" #OFFB "+10240\n\t" OP " %8, %6 offset:" #OFFB "+12288\n\t" OP " %8, %7 offset:" #OFFB \
+                    "+14336\n\t"                                                                                        \
+                 :                                                                                                      \
+                 : "v"(R0[0]), "v"(R0[1]), "v"(R0[2]), "v"(R0[3]), "v"(R0[4]), "v"(R0[5]), "v"(R0[6]), "v"(R0[7]), "v"(addr) \
+                 : "memory")
     using i32x2 = int __attribute__((ext_vector_type(2)));
     // Direct global -> LDS loads and nothing else: every workgroup walks the K stages of a 256 x 256 tile of the 8192^3
     // 1-byte GEMM (64 KiB per stage: 8 + 8 loads of 1 KiB per wave), the tiles in the library's own order, DEPTH stages in
@@ -329,7 +337,7 @@ namespace
         for(int i = t; i < 65536 / 4; i += blockDim.x)
             reinterpret_cast<int*>(lds)[i] = i;
         __syncthreads();
-        const uint32_t           addr = (MODE == 0 ? t * 16 : (MODE == 3 ? t * 4 : t * 8)) & 2047;
+        const uint32_t           addr = ((MODE == 0 || MODE == 5) ? t * 16 : ((MODE == 3 || MODE == 7) ? t * 4 : t * 8)) & 2047;
         const unsigned long long c0   = __builtin_readcyclecounter();
         int                      s    = 0;
         if constexpr(MODE == 0)
@@ -345,6 +353,39 @@ namespace
             asm volatile("s_waitcnt lgkmcnt(0)");
             for(int i = 0; i < 8; ++i)
                 s ^= x[i][0] ^ y[i][3];
+        }
+        else if constexpr(MODE >= 5)
+        {
+            // writes: the same addresses and pacing, data from registers that never change
+            using W = std::conditional_t<MODE == 5, i32x4, std::conditional_t<MODE == 6, i32x2, int>>;
+            W x[8];
+            for(int i = 0; i < 8; ++i)
+                x[i] = W{} + (t + i);
+            for(int it = 0; it < iters; ++it)
+            {
+                if constexpr(MODE == 5)
+                {
+                    R355_WR8("ds_write_b128", x, 0);
+                    asm volatile("s_waitcnt lgkmcnt(8)");
+                    R355_WR8("ds_write_b128", x, 16384);
+                }
+                else if constexpr(MODE == 6)
+                {
+                    R355_WR8("ds_write_b64", x, 0);
+                    asm volatile("s_waitcnt lgkmcnt(8)");
+                    R355_WR8("ds_write_b64", x, 16384);
+                }
+                else
+                {
+                    R355_WR8("ds_write_b32", x, 0);
+                    asm volatile("s_waitcnt lgkmcnt(8)");
+                    R355_WR8("ds_write_b32", x, 16384);
+                }
+                asm volatile("s_waitcnt lgkmcnt(8)");
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)");
+            __syncthreads();
+            s = reinterpret_cast<const int*>(lds)[t];
         }
         else if constexpr(MODE == 3)
         {
@@ -664,11 +705,12 @@ int main(int argc, char** argv)
         HIP_OK(hipMalloc(&out, (size_t)dev.compute_units * 256 * sizeof(int)));
         HIP_OK(hipMalloc(&cyc, 64));
         const int          loops   = itersSet ? iters : 4000;
-        static const char* names[] = {"ds_read_b128", "ds_read_b64", "ds_read_b64_tr_b16", "ds_read_b32", "ds_read_b64_tr_b8"};
-        static const int   width[] = {16, 8, 8, 4, 8};
+        static const char* names[] = {"ds_read_b128", "ds_read_b64", "ds_read_b64_tr_b16", "ds_read_b32", "ds_read_b64_tr_b8",
+                                      "ds_write_b128", "ds_write_b64", "ds_write_b32"};
+        static const int   width[] = {16, 8, 8, 4, 8, 16, 8, 4};
         printf("[");
         for(int waves = 4; waves >= 1; waves /= 2)
-            for(int mode = 0; mode < 5; ++mode)
+            for(int mode = 0; mode < 8; ++mode)
             {
                 for(int rep = 0; rep < 2; ++rep)
                 {
@@ -679,7 +721,10 @@ int main(int argc, char** argv)
                     case 1: hipLaunchKernelGGL(ldsReadLoop<1>, g, b, 0, 0, out, loops, cyc); break;
                     case 2: hipLaunchKernelGGL(ldsReadLoop<2>, g, b, 0, 0, out, loops, cyc); break;
                     case 3: hipLaunchKernelGGL(ldsReadLoop<3>, g, b, 0, 0, out, loops, cyc); break;
-                    default: hipLaunchKernelGGL(ldsReadLoop<4>, g, b, 0, 0, out, loops, cyc); break;
+                    case 4: hipLaunchKernelGGL(ldsReadLoop<4>, g, b, 0, 0, out, loops, cyc); break;
+                    case 5: hipLaunchKernelGGL(ldsReadLoop<5>, g, b, 0, 0, out, loops, cyc); break;
+                    case 6: hipLaunchKernelGGL(ldsReadLoop<6>, g, b, 0, 0, out, loops, cyc); break;
+                    default: hipLaunchKernelGGL(ldsReadLoop<7>, g, b, 0, 0, out, loops, cyc); break;
                     }
                     HIP_OK(hipDeviceSynchronize());
                 }
