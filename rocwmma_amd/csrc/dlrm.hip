@@ -217,7 +217,9 @@ namespace
         float*         o         = outLds[wave];
 
         // Two register stashes, used in turn: the loads of the next two samples are in flight while one is computed
-        // (a wave holds 2 x 13.8 KB in flight, a CU's eight waves 220 KB).
+        // (a wave holds 2 x 13.8 KB in flight, a CU's eight waves 220 KB).  One stash where two would not fit the 256
+        // registers that two waves per SIMD leave each wave (32 rows of 128).
+        constexpr bool TWO = MAX_CHUNKS < 16u;
         // (a sample beyond the batch is a buffer of no bytes: the loads are issued and move nothing)
         f32x4 stashA[MAX_CHUNKS], stashB[MAX_CHUNKS];
         auto  request = [&](f32x4 (&stash)[MAX_CHUNKS], uint64_t b) {
@@ -242,7 +244,7 @@ namespace
             }
             __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_wave_barrier();
-            request(stash, b + 2u * stride); // the stash is free again
+            request(stash, b + (TWO ? 2u : 1u) * stride); // the stash is free again
 
             // v_mfma_f32_16x16x4_f32 on the three 16 x 16 blocks of the Gram matrix that hold its lower
             // triangle (rows < 16 x rows < 16, rows >= 16 x rows < 16, rows >= 16 x rows >= 16): a quarter
@@ -318,14 +320,24 @@ namespace
         if(first >= batch)
             return;
         request(stashA, first);
-        request(stashB, (uint64_t)first + stride);
-        process(stashA, first);
-        process(stashB, (uint64_t)first + stride);
-#pragma unroll 1
-        for(uint64_t b = (uint64_t)first + 2u * stride; b < batch; b += 2u * stride)
+        if constexpr(TWO)
         {
-            process(stashA, b);
-            process(stashB, b + stride);
+            request(stashB, (uint64_t)first + stride);
+            process(stashA, first);
+            process(stashB, (uint64_t)first + stride);
+#pragma unroll 1
+            for(uint64_t b = (uint64_t)first + 2u * stride; b < batch; b += 2u * stride)
+            {
+                process(stashA, b);
+                process(stashB, b + stride);
+            }
+        }
+        else
+        {
+            process(stashA, first);
+#pragma unroll 1
+            for(uint64_t b = (uint64_t)first + stride; b < batch; b += stride)
+                process(stashA, b);
         }
     }
 
