@@ -370,45 +370,51 @@ namespace
         constexpr uint32_t SWZ_IN     = 12u & (ROW_CHUNKS - 1u); // (j & 3) << 2: four j rows -> four 64-byte groups
         constexpr uint32_t SWZ_OUT    = 15u & (ROW_CHUNKS - 1u);
 
+        constexpr uint32_t UP_VECS = (SAMPLES_PER_WG * MAX_UP + 7u) / 8u; // 16-byte pieces of the workgroup's upstream run
+        constexpr uint32_t UP_LOADS = (UP_VECS + THREADS - 1u) / THREADS; // per thread
+
         __shared__ __attribute__((aligned(16))) char     xLds[WAVES][X_BYTES];
-        __shared__ __attribute__((aligned(16))) uint16_t upLds[SAMPLES_PER_WG * MAX_UP + 8];
+        __shared__ __attribute__((aligned(16))) uint16_t upLds[UP_LOADS * THREADS * 8u];
 
         const uint32_t tid      = threadIdx.x;
         const uint32_t lane     = tid & 63u;
-        const uint32_t wave     = tid >> 6;
+        const uint32_t wave     = __builtin_amdgcn_readfirstlane(tid >> 6);
         const uint32_t upStride = K + m * (m - 1) / 2;
         const uint32_t b0       = blockIdx.x * SAMPLES_PER_WG;
         const uint32_t inChunks = m * ROW_CHUNKS;
+        const uint32_t inBytes  = inChunks * 16u;
         char*          xw       = xLds[wave];
 
+        // Everything the workgroup reads is requested at once, through raw buffers of exactly the bytes that exist (runBuffer):
+        // X of the wave's two samples, then the workgroup's run of upstream rows.  (With a loop of guarded loads each trip
+        // waited for its own load - one memory latency per trip.)
         i32x4 stash[PER_WAVE][MAX_CHUNKS];
 #pragma unroll
         for(uint32_t q = 0; q < PER_WAVE; ++q)
         {
-            const uint32_t b = b0 + wave + q * WAVES;
-            if(b < batch)
-            {
-                const char* src = reinterpret_cast<const char*>(in) + (uint64_t)b * m * K * 2u;
+            const uint32_t b   = b0 + wave + q * WAVES;
+            const auto     src = runBuffer(in, (uint64_t)(b < batch ? b : 0u) * inBytes, b < batch ? inBytes : 0u);
 #pragma unroll
-                for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
-                {
-                    const uint32_t c = j * 64u + lane;
-                    if(c < inChunks)
-                        stash[q][j] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(src + c * 16u));
-                }
-            }
+            for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
+                stash[q][j] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (j * 64u + lane) * 16u, 0, NONTEMPORAL));
         }
 
         // ---- upstream rows of the workgroup's samples -> LDS; zero rows m..31 of the X image
         const uint32_t nSamples = (batch - b0) < SAMPLES_PER_WG ? (batch - b0) : SAMPLES_PER_WG;
         {
-            const uint32_t  total = nSamples * upStride;
-            const uint16_t* src   = upstream + (uint64_t)b0 * upStride;
-            const uint32_t  vecs  = total / 8u;
-            for(uint32_t v = tid; v < vecs; v += THREADS)
-                reinterpret_cast<i32x4*>(upLds)[v] = __builtin_nontemporal_load(reinterpret_cast<const i32x4*>(src) + v);
-            for(uint32_t e = vecs * 8u + tid; e < total; e += THREADS)
-                upLds[e] = src[e];
+            // the run is a whole number of 16-byte pieces unless the batch ends inside this workgroup; whole 4-byte words go
+            // through the buffer (its range check works on words), a last odd element on its own
+            const uint32_t total = nSamples * upStride; // elements
+            const auto     src   = runBuffer(upstream, (uint64_t)b0 * upStride * 2u, (total & ~1u) * 2u);
+            i32x4          upv[UP_LOADS];
+#pragma unroll
+            for(uint32_t j = 0; j < UP_LOADS; ++j)
+                upv[j] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (j * THREADS + tid) * 16u, 0, NONTEMPORAL));
+#pragma unroll
+            for(uint32_t j = 0; j < UP_LOADS; ++j)
+                reinterpret_cast<i32x4*>(upLds)[j * THREADS + tid] = upv[j];
+            if((total & 1u) && tid == 0)
+                upLds[total - 1u] = upstream[(uint64_t)b0 * upStride + total - 1u];
             for(uint32_t c = inChunks + lane; c < MAX_M * ROW_CHUNKS; c += 64u)
                 *reinterpret_cast<i32x4*>(xw + c * 16u) = i32x4{0, 0, 0, 0};
         }
