@@ -142,6 +142,53 @@ def test_sparse_gemm_row_major_b(in_t, out_t, m, n, k, ldl):
     assert e.value.code == -2
 
 
+@pytest.mark.parametrize("case", range(40))
+def test_sparse_random_sweep(case):
+    """Seeded random draw of element type, sizes (both kernels, edge tiles, every stage-count remainder), orientation of B
+    and of C / D, scalars and kernel selector, against the oracle's dense GEMM on the decompressed A."""
+    rng = np.random.default_rng(5000 + case)
+    in_t, out_t = [(O.I8, O.I32), (O.E4M3, O.F32), (O.F16, O.F32), (O.BF16, O.F32)][case % 4]
+    es = 2 if in_t in (O.F16, O.BF16) else 1
+    big = bool(rng.integers(0, 2))
+    m = 16 * int(rng.integers(8, 40) if big else rng.integers(1, 12))
+    n = 16 * int(rng.integers(8, 40) if big else rng.integers(1, 12))
+    k = (128 // es) * int(rng.integers(1, 14))
+    lb = [O.COL, O.COL, O.ROW][int(rng.integers(0, 3))]
+    ldl = [O.ROW, O.COL][int(rng.integers(0, 2))]
+    alpha, beta = (float(rng.integers(-2, 3)), float(rng.integers(-1, 2))) if in_t == O.I8 else (float(rng.choice([1.0, 2.0, -0.5])), float(rng.choice([0.0, 1.0])))
+    mask = O.sparse24_mask(case + 1, m, k)
+    if in_t == O.I8:
+        dense = np.where(mask, O.uniform_int8(case + 2, m * k).reshape(m, k), np.int8(0)).astype(np.int8)
+        b, storage = O.uniform_int8(case + 3, k * n), dense
+        c = O.uniform_int8(case + 4, m * n).astype(np.int32) * 5
+    elif in_t == O.E4M3:
+        dense = np.where(mask, O.f32_to_storage(O.normal(case + 2, m * k), O.E4M3).view(np.int8).reshape(m, k), np.int8(0)).astype(np.int8)
+        b, storage = O.f32_to_storage(O.normal(case + 3, k * n), O.E4M3), dense.view(np.uint8)
+        c = O.uniform_pm1(case + 4, m * n)
+    else:
+        dense = np.where(mask, O.f32_to_storage(O.uniform_pm1(case + 2, m * k), in_t).reshape(m, k), np.uint16(0)).astype(np.uint16)
+        b, storage = O.f32_to_storage(O.uniform_pm1(case + 3, k * n), in_t), dense
+        c = O.uniform_pm1(case + 4, m * n)
+    vals, meta = R.compress_24(dense)
+    assert np.array_equal(R.decompress_24(vals, meta), dense)
+    want = O.gemm(in_t, out_t, O.ROW, lb, ldl, ldl, m, n, k, storage.ravel(), b, c, alpha, beta)
+    dv, dm, db, dc = to_device(vals), to_device(meta), to_device(b), to_device(c)
+    dd = device_filled(m * n + 4, O.NP_STORAGE[out_t], 0xEE)
+    kernel = [R.KERNEL_AUTO, R.KERNEL_TILED, R.KERNEL_SIMPLE][int(rng.integers(0, 3))]
+    if lb == O.ROW and kernel == R.KERNEL_TILED:
+        kernel = R.KERNEL_AUTO  # the macro tile wants K-contiguous columns of B
+    R.gemm(in_t, out_t, m, n, k, dv, db, dc if beta != 0.0 else None, dd, alpha, beta, O.ROW, lb, ldl, ldl, a_meta=dm, kernel=kernel)
+    full = to_host(dd, O.NP_STORAGE[out_t])
+    assert np.all(full[m * n:].view(np.uint8) == 0xEE)
+    got = full[:m * n]
+    if in_t == O.I8:
+        assert np.array_equal(got, want), (m, n, k, lb, ldl, kernel)
+    else:
+        g, w = got.astype(np.float64), want.astype(np.float64)
+        assert np.all(np.isfinite(g))
+        assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= (1e-2 if in_t == O.E4M3 else 1e-3), (m, n, k, lb, ldl, kernel)
+
+
 def test_sparse_16bit_one_hot_positions():
     """Every (row, kept position) of A in turn is the only non-zero: D must be that row of B scaled - exact, and it
     fails for any wrong pairing of lane groups or index bits."""
