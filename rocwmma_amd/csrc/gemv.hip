@@ -1,14 +1,16 @@
 // GEMV y = alpha * A x + beta * y for f32 and f64, HBM-bound: A is read exactly once with
-// coalesced 128-bit loads, x is staged through LDS, and f32 FMAs accumulate in the
-// order k = 0..K-1 per output row within a lane.
+// coalesced 128-bit loads, several per lane requested before the first is used; the order of the
+// sums is fixed by the shape alone (never by scheduling).
 //
 // Takes the place of samples/simple_sgemv.cpp:103-150 (f64: samples/simple_dgemv.cpp:103), which feeds 16x16x16 f32 fragments
 // (the B fragment being x broadcast 16 times) to the matrix core.  At 0.5 flop per byte
 // the matrix core contributes nothing; the kernel is organised for memory bandwidth.
-//   col-major A (the sample's layout): a workgroup owns 64 (or 256) rows; its 16 waves split
+//   col-major A (the sample's layout): a workgroup of sixteen waves owns 32 or 64 rows (f64: 16 or 32); its lanes split
 //     the columns and combine their partial sums through LDS in a fixed order.
-//   row-major A: one wave per row, lanes stride k in float4, then a wave reduction.
+//   row-major A: one wave per row, lanes stride k in 16-byte pieces, then a wave reduction.
 #include <hip/hip_runtime.h>
+
+#include <type_traits>
 
 #include "common.hpp"
 
@@ -16,12 +18,14 @@ namespace
 {
     constexpr uint32_t THREADS = 256;
 
-    // col-major A (m contiguous): a wave reads V * 64 consecutive rows of one column per load;
-    // the 16 waves of a workgroup split the columns and their partial sums meet in LDS in a fixed
-    // order, so the result does not depend on scheduling.
-    constexpr uint32_t COL_WAVES = 16;
-
-    template <typename T, uint32_t V>
+    // col-major A (m contiguous).  A lane loads 16 bytes = V consecutive rows of one column; RL lanes side by side make a
+    // run of RL * 16 bytes of that column and the wave's other lanes take the next 64 / RL - 1 columns, so a workgroup of
+    // COL_WAVES waves owns RL * V rows and walks the columns COL_WAVES * 64 / RL at a time, DEPTH steps requested before the
+    // first is used.  RL = 8 (128-byte runs, 32 rows of f32 per workgroup) gives 8192 rows a workgroup per CU; RL = 16
+    // (256-byte runs) is taken when the rows suffice for that.  Every lane sums its columns in increasing order; the
+    // COL_WAVES * 64 / RL partial sums of a row meet in LDS and are added in a fixed order, so the result does not depend
+    // on scheduling.  STREAM as in the row-major kernel.
+    template <typename T, uint32_t RL, uint32_t COL_WAVES, bool STREAM>
     __global__ void __launch_bounds__(COL_WAVES * 64) gemvColMajor(uint32_t m,
                                                                   uint32_t k,
                                                                   const T* a,
@@ -32,31 +36,46 @@ namespace
                                                                   T        alpha,
                                                                   T        beta)
     {
+        constexpr uint32_t V = 16u / sizeof(T), ROWS = RL * V, CL = 64u / RL, COLS = COL_WAVES * CL, DEPTH = 8;
         using VecT = T __attribute__((ext_vector_type(V)));
-        __shared__ T   partial[COL_WAVES][64 * V];
+        __shared__ T   partial[COLS][ROWS];
         const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-        const uint32_t r0   = (blockIdx.x * 64u + lane) * V;
+        const uint32_t r = lane % RL, c = lane / RL;
+        const uint32_t row0 = blockIdx.x * ROWS + r * V; // (m is a multiple of V: a lane's rows are inside or outside together)
         T              acc[V];
 #pragma unroll
         for(uint32_t e = 0; e < V; ++e)
             acc[e] = T(0);
-        if(r0 < m)
+        if(row0 < m)
         {
-            const T* p = a + r0;
-#pragma unroll 8
-            for(uint32_t kk = wave; kk < k; kk += COL_WAVES)
-            {
-                T v[V];
-                if constexpr(V == 1)
-                    v[0] = p[(uint64_t)kk * lda];
+            const T* p     = a + row0;
+            auto     fetch = [](const T* at) {
+                if constexpr(STREAM)
+                    return __builtin_nontemporal_load(reinterpret_cast<const VecT*>(at));
                 else
-                {
-                    const VecT vv = *reinterpret_cast<const VecT*>(p + (uint64_t)kk * lda);
+                    return *reinterpret_cast<const VecT*>(at);
+            };
+            uint32_t kk = wave * CL + c;
+            for(; kk + (DEPTH - 1u) * COLS < k; kk += DEPTH * COLS)
+            {
+                VecT v[DEPTH];
+                T    xv[DEPTH];
+#pragma unroll
+                for(uint32_t u = 0; u < DEPTH; ++u)
+                    v[u] = fetch(p + (uint64_t)(kk + u * COLS) * lda);
+#pragma unroll
+                for(uint32_t u = 0; u < DEPTH; ++u)
+                    xv[u] = x[kk + u * COLS];
+#pragma unroll
+                for(uint32_t u = 0; u < DEPTH; ++u)
 #pragma unroll
                     for(uint32_t e = 0; e < V; ++e)
-                        v[e] = vv[e];
-                }
-                const T xv = x[kk];
+                        acc[e] += v[u][e] * xv[u];
+            }
+            for(; kk < k; kk += COLS)
+            {
+                const VecT v  = fetch(p + (uint64_t)kk * lda);
+                const T    xv = x[kk];
 #pragma unroll
                 for(uint32_t e = 0; e < V; ++e)
                     acc[e] += v[e] * xv;
@@ -64,24 +83,27 @@ namespace
         }
 #pragma unroll
         for(uint32_t e = 0; e < V; ++e)
-            partial[wave][lane * V + e] = acc[e];
+            partial[wave * CL + c][r * V + e] = acc[e];
         __syncthreads();
-        // 64 * V rows, summed over the waves in wave order
-        for(uint32_t r = threadIdx.x; r < 64u * V; r += COL_WAVES * 64u)
+        if(threadIdx.x < ROWS)
         {
-            const uint32_t row = blockIdx.x * 64u * V + r;
+            const uint32_t row = blockIdx.x * ROWS + threadIdx.x;
             if(row < m)
             {
                 T sum = T(0);
 #pragma unroll
-                for(uint32_t w = 0; w < COL_WAVES; ++w)
-                    sum += partial[w][r];
+                for(uint32_t w = 0; w < COLS; ++w)
+                    sum += partial[w][threadIdx.x];
                 yOut[row] = beta != T(0) ? alpha * sum + beta * yIn[row] : alpha * sum;
             }
         }
     }
 
-    template <typename T>
+    // STREAM: A does not fit the 256 MiB memory-side cache, so nothing of it can be there from an earlier call or be wanted
+    // by a later one: nontemporal loads (measured: 16384^2 f32 0.174 -> 0.164 ms, 65536 x 2048 0.086 -> 0.073).  Otherwise
+    // ordinary loads (8192^2 f32, exactly 256 MiB, called again and again: 0.0389 -> 0.0370 ms; 0.0409 with nontemporal
+    // loads) and rows that start at different groups of k.
+    template <typename T, bool STREAM>
     __global__ void __launch_bounds__(THREADS) gemvRowMajor(uint32_t m,
                                                            uint32_t k,
                                                            const T* a,
@@ -100,9 +122,38 @@ namespace
             return;
         const T* p   = a + (uint64_t)row * lda;
         T        acc = T(0);
-        for(uint32_t kk = lane * V; kk < k; kk += 64u * V)
+        // DEPTH loads of A per lane are requested before the first is used (bytes in flight are what keeps HBM busy; one load
+        // per trip, waited for at once, left that to the number of resident waves alone).  Unless A streams, rows start at
+        // different groups of k and wrap around: with a power-of-two leading dimension all rows are aligned alike, and waves
+        // that walk their rows in step are all on the same few memory channels at any one time.
+        constexpr uint32_t DEPTH = 4, STEP = 64u * V, GROUP = DEPTH * STEP;
+        const uint32_t     groups = k / GROUP, g0 = (!STREAM && groups) ? (row * 5u) % groups : 0u;
+        auto               fetch  = [](const T* at) {
+            if constexpr(STREAM)
+                return __builtin_nontemporal_load(reinterpret_cast<const VecT*>(at));
+            else
+                return *reinterpret_cast<const VecT*>(at);
+        };
+        for(uint32_t t = 0; t < groups; ++t)
         {
-            const VecT v  = *reinterpret_cast<const VecT*>(p + kk);
+            const uint32_t g  = g0 + t < groups ? g0 + t : g0 + t - groups;
+            const uint32_t kk = g * GROUP + lane * V;
+            VecT           v[DEPTH], xv[DEPTH];
+#pragma unroll
+            for(uint32_t u = 0; u < DEPTH; ++u)
+                v[u] = fetch(p + kk + u * STEP);
+#pragma unroll
+            for(uint32_t u = 0; u < DEPTH; ++u)
+                xv[u] = *reinterpret_cast<const VecT*>(x + kk + u * STEP);
+#pragma unroll
+            for(uint32_t u = 0; u < DEPTH; ++u)
+#pragma unroll
+                for(uint32_t e = 0; e < V; ++e)
+                    acc += v[u][e] * xv[u][e];
+        }
+        for(uint32_t kk = groups * GROUP + lane * V; kk < k; kk += STEP)
+        {
+            const VecT v  = fetch(p + kk);
             const VecT xv = *reinterpret_cast<const VecT*>(x + kk);
 #pragma unroll
             for(uint32_t e = 0; e < V; ++e)
@@ -133,20 +184,32 @@ namespace
         {
             if(lda < m)
                 return r355::fail(R355_ERR_BAD_ARG, "gemv: lda < m");
-            // narrow loads while they are what it takes to give every CU a workgroup
-            if(m >= 64u * V * 256u)
-                hipLaunchKernelGGL((gemvColMajor<T, V>), dim3((m + 64u * V - 1u) / (64u * V)), dim3(COL_WAVES * 64), 0, s, m, k, a,
-                                   lda, x, y_in, y_out, alpha, beta);
+            const bool stream = (uint64_t)k * lda * sizeof(T) > (256ull << 20);
+            auto       go     = [&](auto rl, auto waves) {
+                constexpr uint32_t RL = decltype(rl)::value, ROWS = RL * V, WAVES = decltype(waves)::value;
+                const dim3         grid((m + ROWS - 1u) / ROWS), block(WAVES * 64);
+                if(stream)
+                    hipLaunchKernelGGL((gemvColMajor<T, RL, WAVES, true>), grid, block, 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
+                else
+                    hipLaunchKernelGGL((gemvColMajor<T, RL, WAVES, false>), grid, block, 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
+            };
+            // 256-byte runs once the rows give every CU a workgroup with them (8192^2 f32: 0.0415 ms against 0.0374 with
+            // 128-byte runs and twice the workgroups; 16384^2: 0.151 against 0.161); sixteen waves per workgroup either way
+            // (four: 0.0399 and 0.163)
+            if(m >= 16u * V * 256u)
+                go(std::integral_constant<uint32_t, 16>{}, std::integral_constant<uint32_t, 16>{});
             else
-                hipLaunchKernelGGL((gemvColMajor<T, 1>), dim3((m + 63u) / 64u), dim3(COL_WAVES * 64), 0, s, m, k, a, lda, x,
-                                   y_in, y_out, alpha, beta);
+                go(std::integral_constant<uint32_t, 8>{}, std::integral_constant<uint32_t, 16>{});
         }
         else if(layout_a == R355_ROW_MAJOR)
         {
             if(lda < k)
                 return r355::fail(R355_ERR_BAD_ARG, "gemv: lda < k");
-            hipLaunchKernelGGL((gemvRowMajor<T>), dim3((m + THREADS / 64 - 1) / (THREADS / 64)), dim3(THREADS), 0, s, m, k, a,
-                               lda, x, y_in, y_out, alpha, beta);
+            const dim3 grid((m + THREADS / 64 - 1) / (THREADS / 64));
+            if((uint64_t)m * lda * sizeof(T) > (256ull << 20))
+                hipLaunchKernelGGL((gemvRowMajor<T, true>), grid, dim3(THREADS), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
+            else
+                hipLaunchKernelGGL((gemvRowMajor<T, false>), grid, dim3(THREADS), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
         }
         else
             return r355::fail(R355_ERR_BAD_ARG, "gemv: unknown layout");

@@ -11,7 +11,10 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("layout", [O.ROW, O.COL])
-@pytest.mark.parametrize("m,k", [(256, 256), (1024, 512), (8192, 8192), (4100, 260), (65536 + 256, 64)])
+@pytest.mark.parametrize("m,k", [(256, 256), (1024, 512), (8192, 8192), (4100, 260), (65536 + 256, 64),
+                                 # whole groups of loads plus a remainder, partial last workgroups, both run widths of the
+                                 # col-major kernel (128- and 256-byte runs: the wide one from 16384 rows on)
+                                 (96, 2500), (272, 1300), (16384 + 68, 1100), (20, 4096 + 4)])
 def test_gemv_vs_oracle(layout, m, k):
     a, x, y = O.uniform_pm1(1, m * k), O.uniform_pm1(2, k), O.uniform_pm1(3, m)
     want = O.gemm(O.F32, O.F32, layout, O.COL, O.COL, O.COL, m, 1, k, a, x, y, 2.0, 2.0)
@@ -30,7 +33,7 @@ def test_gemv_vs_oracle(layout, m, k):
 
 
 @pytest.mark.parametrize("layout", [O.ROW, O.COL])
-@pytest.mark.parametrize("m,k", [(256, 256), (4098, 262), (32768 + 128, 64)])
+@pytest.mark.parametrize("m,k", [(256, 256), (4098, 262), (32768 + 128, 64), (66, 2310), (8192 + 6, 1030)])
 def test_dgemv_vs_oracle(layout, m, k):
     """The f64 twin (samples/simple_dgemv.cpp): against the oracle's f64 GEMM with n = 1 and the exact integer case."""
     a = O.uniform_pm1(4, m * k).astype(np.float64) + O.uniform_pm1(5, m * k).astype(np.float64) * 2.0 ** -30
