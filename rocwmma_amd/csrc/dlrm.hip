@@ -95,6 +95,10 @@ namespace
         char* xw = xLds[wave];
         // rows m..31 of the 32 x 32 product are padding: their lanes feed zeros (see below)
 
+        // (Tried and dropped: two groups of 8 samples per workgroup with the next group's loads in flight during compute
+        // and copy-out - the compiler then keeps 137 instead of 85 registers at k = 128, three workgroups per CU instead
+        // of four, 0.0852 against 0.0823 ms at a batch of 65536; and the copy-out through a raw buffer - the same at
+        // k <= 128, 0.162 against 0.155 ms at k = 256.)
         // Both samples of this wave are requested from HBM before either is consumed: the kernel is
         // bandwidth-bound, and bytes in flight per CU are what keeps HBM busy.  The loads go through a raw buffer of
         // exactly the sample's bytes (runBuffer; none for a sample beyond the batch), so the first sample is consumed
