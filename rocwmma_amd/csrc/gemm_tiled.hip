@@ -1018,13 +1018,26 @@ namespace
                 readBlock8<A_KCONTIG, WB, ES>(lds + aAt, rdA, x >> 1, s, part, fa[s][x >> 1], 0u);
         };
 
-        uint64_t refillA, refillB; // stage kt + 2 of A, stage kt + 3 of B (clamped)
-        // One K stage: K step 0 is in registers; step 1 arrives under its matrix instructions; then the
-        // stage's buffers are refilled (A two stages ahead, B three) while step 0 of the next stage
-        // arrives under the matrix instructions of step 1.  Per four (small wave tile: two) matrix
-        // instructions: one operand block read (two reads when it is transposed on the way) and, in the
-        // second half, one direct load; nothing moves between the pieces.
-        auto stageBody = [&](uint32_t kt, uint32_t aCur, uint32_t aNxt, uint32_t bCur, uint32_t bNxt) {
+        // One K stage: K step 0 is in registers; step 1 arrives under its matrix instructions; then step 0 of
+        // the next stage arrives under the matrix instructions of step 1.  Per four (small wave tile: two) matrix
+        // instructions one operand block read (two reads when it is transposed on the way); nothing moves between
+        // the pieces.  The direct loads, one at a time between matrix instructions:
+        //   large wave tile (SPREAD)  dealt out over the whole stage - B of stage kt + 2 under step 0, into the third
+        //       B buffer (free since the barrier of stage kt - 1, not needed before the one of stage kt + 1), A of
+        //       stage kt + 2 under step 1, into the A buffer this stage's barrier has freed.  With all of a stage's
+        //       loads under step 1 the memory pipeline ran dry during the other half of every stage (int8 8192^3:
+        //       0.4145 -> 0.4115 ms; with all-zero operands 0.3230 -> 0.3170).
+        //   small wave tile  all under step 1: A of stage kt + 2, then B of stage kt + 3 into the B buffer the barrier
+        //       has freed.  Its stages are a quarter as long, and B requested only a stage and a half ahead arrives
+        //       late (f16 2048^2 x 8192: 0.0745 ms this way, 0.0770 the other).
+        constexpr bool     SPREAD = WB == 8;
+        constexpr uint32_t B_AHEAD = SPREAD ? 2u : 3u;
+        uint64_t           refillA, refillB; // stage kt + 2 of A, stage kt + B_AHEAD of B (clamped)
+        auto stageBody = [&](uint32_t kt, uint32_t aCur, uint32_t aNxt, uint32_t bCur, uint32_t bNxt, uint32_t bFree) {
+            const uint32_t vB    = validOf(kt + B_AHEAD);
+            const i32x4    rsrcB = stageRsrc8(B_KCONTIG, refillB, vB, p.ldb);
+            if(kt + B_AHEAD + 1u < numStages)
+                refillB += gStageB;
 #pragma unroll
             for(uint32_t x = 0; x < XS; ++x)
 #pragma unroll
@@ -1033,16 +1046,18 @@ namespace
                     mfmaAt(0, QS * x + q);
                     if(q < 2u)
                         readAt(aCur, bCur, 1, x, q);
+                    if constexpr(SPREAD)
+                        if(q == LOAD_Q && (x & 1u))
+                            loadToLds(rsrcB, tailOffset(B_KCONTIG, gOffB[x >> 1], kByteB, vB), (x >> 1) * gStepB,
+                                      dmaDst + bFree + (x >> 1) * THREADS * CHUNK);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             waitVmcnt<WB>(); // this wave's part of stage kt + 1 has landed (the youngest WB loads are B of kt + 2)
             ldsBarrier();
-            const uint32_t vA = validOf(kt + 2u), vB = validOf(kt + 3u);
-            const i32x4    rsrcA = stageRsrc8(A_KCONTIG, refillA, vA, p.lda), rsrcB = stageRsrc8(B_KCONTIG, refillB, vB, p.ldb);
+            const uint32_t vA    = validOf(kt + 2u);
+            const i32x4    rsrcA = stageRsrc8(A_KCONTIG, refillA, vA, p.lda);
             if(kt + 3u < numStages)
                 refillA += gStageA;
-            if(kt + 4u < numStages)
-                refillB += gStageB;
 #pragma unroll
             for(uint32_t x = 0; x < XS; ++x)
 #pragma unroll
@@ -1051,7 +1066,13 @@ namespace
                     mfmaAt(1, QS * x + q);
                     if(q < 2u)
                         readAt(aNxt, bNxt, 0, x, q);
-                    if(q == LOAD_Q)
+                    if constexpr(SPREAD)
+                    {
+                        if(q == LOAD_Q && (x & 1u))
+                            loadToLds(rsrcA, tailOffset(A_KCONTIG, gOffA[x >> 1], kByteA, vA), (x >> 1) * gStepA,
+                                      dmaDst + aCur + (x >> 1) * THREADS * CHUNK);
+                    }
+                    else if(q == LOAD_Q)
                     {
                         if(x < WB)
                             loadToLds(rsrcA, tailOffset(A_KCONTIG, gOffA[x], kByteA, vA), x * gStepA, dmaDst + aCur + x * THREADS * CHUNK);
@@ -1063,14 +1084,26 @@ namespace
                 }
         };
 
-        // prologue: stages 0 and 1 and the B half of stage 2 requested; stage 0 published
-        issueHalf(A_KCONTIG, stageAddr(gA, gStageA, 0u), gOffA, gStepA, kByteA, p.lda, validOf(0u), A_AT[0]);
-        issueHalf(B_KCONTIG, stageAddr(gB, gStageB, 0u), gOffB, gStepB, kByteB, p.ldb, validOf(0u), B_AT[0]);
-        issueHalf(A_KCONTIG, stageAddr(gA, gStageA, 1u), gOffA, gStepA, kByteA, p.lda, validOf(1u), A_AT[1]);
-        issueHalf(B_KCONTIG, stageAddr(gB, gStageB, 1u), gOffB, gStepB, kByteB, p.ldb, validOf(1u), B_AT[1]);
-        issueHalf(B_KCONTIG, stageAddr(gB, gStageB, 2u), gOffB, gStepB, kByteB, p.ldb, validOf(2u), B_AT[2]);
-        refillA = stageAddr(gA, gStageA, 2u), refillB = stageAddr(gB, gStageB, 3u);
-        waitVmcnt<3u * WB>();
+        // prologue: stages 0 and 1 (and, where B runs three stages ahead, B of stage 2) requested in the order the
+        // loop keeps; stage 0 published
+        if constexpr(SPREAD)
+        {
+            issueHalf(B_KCONTIG, stageAddr(gB, gStageB, 0u), gOffB, gStepB, kByteB, p.ldb, validOf(0u), B_AT[0]);
+            issueHalf(A_KCONTIG, stageAddr(gA, gStageA, 0u), gOffA, gStepA, kByteA, p.lda, validOf(0u), A_AT[0]);
+            issueHalf(B_KCONTIG, stageAddr(gB, gStageB, 1u), gOffB, gStepB, kByteB, p.ldb, validOf(1u), B_AT[1]);
+            issueHalf(A_KCONTIG, stageAddr(gA, gStageA, 1u), gOffA, gStepA, kByteA, p.lda, validOf(1u), A_AT[1]);
+            waitVmcnt<2u * WB>();
+        }
+        else
+        {
+            issueHalf(A_KCONTIG, stageAddr(gA, gStageA, 0u), gOffA, gStepA, kByteA, p.lda, validOf(0u), A_AT[0]);
+            issueHalf(B_KCONTIG, stageAddr(gB, gStageB, 0u), gOffB, gStepB, kByteB, p.ldb, validOf(0u), B_AT[0]);
+            issueHalf(A_KCONTIG, stageAddr(gA, gStageA, 1u), gOffA, gStepA, kByteA, p.lda, validOf(1u), A_AT[1]);
+            issueHalf(B_KCONTIG, stageAddr(gB, gStageB, 1u), gOffB, gStepB, kByteB, p.ldb, validOf(1u), B_AT[1]);
+            issueHalf(B_KCONTIG, stageAddr(gB, gStageB, 2u), gOffB, gStepB, kByteB, p.ldb, validOf(2u), B_AT[2]);
+            waitVmcnt<3u * WB>();
+        }
+        refillA = stageAddr(gA, gStageA, 2u), refillB = stageAddr(gB, gStageB, B_AHEAD);
         ldsBarrier();
         R355_STAMP(1);
 #pragma unroll
@@ -1084,28 +1117,28 @@ namespace
         uint32_t kt = 0;
         for(uint32_t trips = numStages / 6u; trips > 0; --trips, kt += 6u)
         {
-            stageBody(kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1]);
-            stageBody(kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2]);
-            stageBody(kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0]);
-            stageBody(kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1]);
-            stageBody(kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2]);
-            stageBody(kt + 5u, A_AT[1], A_AT[0], B_AT[2], B_AT[0]);
+            stageBody(kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1], B_AT[2]);
+            stageBody(kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2], B_AT[0]);
+            stageBody(kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0], B_AT[1]);
+            stageBody(kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1], B_AT[2]);
+            stageBody(kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2], B_AT[0]);
+            stageBody(kt + 5u, A_AT[1], A_AT[0], B_AT[2], B_AT[0], B_AT[1]);
         }
         const uint32_t rem = numStages - kt;
         if(rem > 0u)
         {
-            stageBody(kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1]);
+            stageBody(kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1], B_AT[2]);
             if(rem > 1u)
             {
-                stageBody(kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2]);
+                stageBody(kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2], B_AT[0]);
                 if(rem > 2u)
                 {
-                    stageBody(kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0]);
+                    stageBody(kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0], B_AT[1]);
                     if(rem > 3u)
                     {
-                        stageBody(kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1]);
+                        stageBody(kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1], B_AT[2]);
                         if(rem > 4u)
-                            stageBody(kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2]);
+                            stageBody(kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2], B_AT[0]);
                     }
                 }
             }
