@@ -261,126 +261,193 @@ namespace
 
     // D = alpha * acc + beta * C for one wave's tile of WB x WB accumulator blocks (16 x 16 each), row-major;
     // the wave tile starts at (m0, n0).  `scratch` is WB * 4 KiB of LDS owned by this wave.
+    //
+    // A lane holds four consecutive columns of one row of every block.  The tile is transposed through the wave's own LDS,
+    // 128 to 16 rows at a time, so that an access to C or D covers whole rows of the wave tile (128 to 512 bytes) with up
+    // to 128 bits per lane.  What is staged: alpha * acc in the output type when beta is zero; in the compute type
+    // otherwise, so that alpha * acc + beta * C is rounded once, as the reference's epilogue rounds it
+    // (test/reference_impl.hpp:71-77).  C and D are reached through raw buffers that end with the tile's last valid row,
+    // and a lane whose columns lie beyond n uses an offset no buffer contains: no branch around any access, so a pass's
+    // reads of C are all requested before its part of the tile goes through LDS, its stores all follow their LDS reads in
+    // batches, and no wait is for more than it needs.  (With a branch around every guarded access each store waited for
+    // everything before it: beta != 0 cost 12 % (f16) to 25 % (e4m3) of an 8192^3 launch instead of the 4 - 13 % that
+    // reading C takes.)  C may alias D: every element's C is read before its D is written, and passes, waves and
+    // workgroups own disjoint rows and columns.
+    template <typename StageT, bool WITH_C, typename AccV, typename OutT, uint32_t WB>
+    __device__ __forceinline__ void storeTileStaged(AccV (&acc)[WB][WB], const Params& p, uint32_t m0, uint32_t n0, uint32_t lane,
+                                                    char* scratch)
+    {
+        using AccE = std::remove_reference_t<decltype(acc[0][0][0])>;
+        const AccE     alpha = static_cast<AccE>(p.alpha), beta = static_cast<AccE>(p.beta);
+        const uint32_t r16 = lane & 15u, g = lane >> 4;
+        constexpr uint32_t SS = sizeof(StageT), OS = sizeof(OutT);
+        constexpr uint32_t ROW_BYTES  = 16u * WB * SS;
+        constexpr uint32_t ROW_CHUNKS = ROW_BYTES / CHUNK; // 8, 16 or 32
+        constexpr uint32_t SWZ        = ROW_CHUNKS < 16u ? ROW_CHUNKS - 1u : 15u;
+        constexpr uint32_t EPC        = CHUNK / SS; // elements of a staged 16-byte chunk
+        constexpr uint32_t OUT_WORDS  = EPC * OS / 4u; // 32-bit words of C and of D per lane and chunk: 4, 2 or 1
+        // rows per pass: what the scratch holds, halved where a pass's part of C would take 128 registers
+        constexpr uint32_t FIT        = WB * 4096u / ROW_BYTES / ((WITH_C && OUT_WORDS == 4u && WB == 8u) ? 2u : 1u);
+        constexpr uint32_t ROWS_PASS  = FIT < 16u * WB ? FIT : 16u * WB;
+        constexpr uint32_t BLOCKS_I   = ROWS_PASS / 16u; // row blocks per pass
+        constexpr uint32_t ITERS      = ROWS_PASS * ROW_CHUNKS / 64u; // chunks per lane and pass
+        constexpr uint32_t BATCH      = ITERS < 8u ? ITERS : 8u;
+        constexpr int      NT         = 2; // cache policy of the raw buffer accesses: nontemporal (C is read, D written, once)
+        static_assert(EPC * OS % 4u == 0u && ITERS % BATCH == 0u, "whole words per lane, whole batches per pass");
+
+        const uint32_t lddB = p.ldd * OS, ldcB = p.ldc * OS;
+        const uint32_t um0 = __builtin_amdgcn_readfirstlane(m0), un0 = __builtin_amdgcn_readfirstlane(n0); // (wave-uniform)
+        const uint32_t colsValid = un0 < p.n ? (p.n - un0 < 16u * WB ? p.n - un0 : 16u * WB) : 0u;
+        auto tileBuffer = [&](const char* base, uint32_t ldB, uint32_t rowFirst) {
+            // from the wave tile's first column in row rowFirst to the end of the tile's last valid row (nothing if there is none)
+            const uint32_t rowsLeft  = rowFirst < p.m ? p.m - rowFirst : 0u;
+            const uint32_t rowsValid = rowsLeft < ROWS_PASS ? rowsLeft : ROWS_PASS;
+            const uint32_t records   = (rowsValid && colsValid) ? (rowsValid - 1u) * ldB + colsValid * OS : 0u;
+            const uint64_t addr      = reinterpret_cast<uint64_t>(base) + ((uint64_t)rowFirst * ldB + (uint64_t)un0 * OS);
+            const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(addr));
+            const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(addr >> 32));
+            return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>((static_cast<uint64_t>(hi) << 32) | lo), 0,
+                                                     static_cast<int>(__builtin_amdgcn_readfirstlane(records)), 0x00020000);
+        };
+        // (lane offset + wave-uniform offset: the range check covers their sum)
+        auto loadWords = [](__amdgpu_buffer_rsrc_t rsrc, uint32_t off, uint32_t uni, uint32_t (&w)[OUT_WORDS]) {
+            if constexpr(OUT_WORDS == 4u)
+            {
+                const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, uni, NT);
+                w[0] = v[0], w[1] = v[1], w[2] = v[2], w[3] = v[3];
+            }
+            else if constexpr(OUT_WORDS == 2u)
+            {
+                const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, off, uni, NT);
+                w[0] = v[0], w[1] = v[1];
+            }
+            else
+                w[0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, off, uni, NT);
+        };
+        auto storeWords = [](__amdgpu_buffer_rsrc_t rsrc, uint32_t off, uint32_t uni, const uint32_t (&w)[OUT_WORDS]) {
+            using u32x4 = uint32_t __attribute__((ext_vector_type(4)));
+            using u32x2 = uint32_t __attribute__((ext_vector_type(2)));
+            if constexpr(OUT_WORDS == 4u)
+                __builtin_amdgcn_raw_buffer_store_b128(u32x4{w[0], w[1], w[2], w[3]}, rsrc, off, uni, NT);
+            else if constexpr(OUT_WORDS == 2u)
+                __builtin_amdgcn_raw_buffer_store_b64(u32x2{w[0], w[1]}, rsrc, off, uni, NT);
+            else
+                __builtin_amdgcn_raw_buffer_store_b32(w[0], rsrc, off, uni, NT);
+        };
+        // chunk `it` of a lane: row it * RPI + lane / ROW_CHUNKS of the pass, 16-byte chunk lane % ROW_CHUNKS of the staged row
+        constexpr uint32_t RPI = 64u / ROW_CHUNKS;
+        const uint32_t rowLane = lane / ROW_CHUNKS, cLane = lane % ROW_CHUNKS;
+        const bool     colOk   = cLane * EPC < colsValid;
+        const uint32_t dLane = colOk ? rowLane * lddB + cLane * (EPC * OS) : 0x80000000u;
+
+#pragma unroll
+        for(uint32_t pass = 0; pass < WB / BLOCKS_I; ++pass)
+        {
+            const auto dBuf = tileBuffer(p.d, lddB, um0 + pass * ROWS_PASS);
+            // C of this pass, requested before anything else (m and n are multiples of 16, so a chunk of up to 16 elements
+            // is inside the matrix or outside as a whole)
+            uint32_t cWords[WITH_C ? ITERS : 1u][OUT_WORDS];
+            if constexpr(WITH_C)
+            {
+                const auto     cBuf  = tileBuffer(p.c, ldcB, um0 + pass * ROWS_PASS);
+                const uint32_t cLaneOff = colOk ? rowLane * ldcB + cLane * (EPC * OS) : 0x80000000u;
+#pragma unroll
+                for(uint32_t it = 0; it < ITERS; ++it)
+                    loadWords(cBuf, cLaneOff, it * RPI * ldcB, cWords[it]);
+            }
+#pragma unroll
+            for(uint32_t ii = 0; ii < BLOCKS_I; ++ii)
+            {
+                const uint32_t i = pass * BLOCKS_I + ii, row = 16u * ii + r16;
+#pragma unroll
+                for(uint32_t j = 0; j < WB; ++j)
+                {
+                    if constexpr(sizeof(AccE) == 8)
+                    {
+                        // f64 accumulators: element e is column 4 e + lane / 16 of the block
+#pragma unroll
+                        for(uint32_t e = 0; e < 4; ++e)
+                        {
+                            const uint32_t byteInRow = (16u * j + 4u * e + g) * SS;
+                            const uint32_t c = byteInRow / CHUNK, within = byteInRow % CHUNK;
+                            *reinterpret_cast<StageT*>(scratch + row * ROW_BYTES + ((c ^ (row & SWZ)) * CHUNK) + within)
+                                = static_cast<StageT>(alpha * acc[i][j][e]);
+                        }
+                    }
+                    else
+                    {
+                        using StageV = StageT __attribute__((ext_vector_type(4)));
+                        StageV out;
+#pragma unroll
+                        for(uint32_t e = 0; e < 4; ++e)
+                            out[e] = static_cast<StageT>(alpha * acc[i][j][e]);
+                        // 16 consecutive rows take 16 (8) different chunk slots
+                        const uint32_t byteInRow = (16u * j + 4u * g) * SS;
+                        const uint32_t c = byteInRow / CHUNK, within = byteInRow % CHUNK;
+                        *reinterpret_cast<StageV*>(scratch + row * ROW_BYTES + ((c ^ (row & SWZ)) * CHUNK) + within) = out;
+                    }
+                }
+            }
+            __builtin_amdgcn_wave_barrier(); // the same wave reads back what it wrote (LDS is in order per wave)
+#pragma unroll
+            for(uint32_t b0 = 0; b0 < ITERS; b0 += BATCH)
+            {
+                union
+                {
+                    i32x4  v;
+                    StageT s[EPC];
+                } staged[BATCH];
+#pragma unroll
+                for(uint32_t u = 0; u < BATCH; ++u)
+                {
+                    const uint32_t row = (b0 + u) * RPI + rowLane;
+                    staged[u].v = *reinterpret_cast<const i32x4*>(scratch + row * ROW_BYTES + ((cLane ^ (row & SWZ)) * CHUNK));
+                }
+#pragma unroll
+                for(uint32_t u = 0; u < BATCH; ++u)
+                {
+                    union
+                    {
+                        uint32_t w[OUT_WORDS];
+                        OutT     o[EPC];
+                    } res;
+                    if constexpr(WITH_C)
+                    {
+                        union
+                        {
+                            uint32_t w[OUT_WORDS];
+                            OutT     o[EPC];
+                        } cin;
+#pragma unroll
+                        for(uint32_t w = 0; w < OUT_WORDS; ++w)
+                            cin.w[w] = cWords[b0 + u][w];
+#pragma unroll
+                        for(uint32_t e = 0; e < EPC; ++e)
+                            res.o[e] = static_cast<OutT>(static_cast<AccE>(staged[u].s[e]) + beta * static_cast<AccE>(cin.o[e]));
+                    }
+                    else
+                    {
+                        static_assert(WITH_C || sizeof(StageT) == sizeof(OutT), "staged in the output type when beta is zero");
+#pragma unroll
+                        for(uint32_t w = 0; w < OUT_WORDS; ++w)
+                            res.w[w] = static_cast<uint32_t>(staged[u].v[w]);
+                    }
+                    storeWords(dBuf, dLane, (b0 + u) * RPI * lddB, res.w);
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
+
     template <typename AccV, typename OutT, uint32_t WB>
     __device__ __forceinline__ void storeTile16(AccV (&acc)[WB][WB], const Params& p, uint32_t m0, uint32_t n0, uint32_t lane,
                                                 char* scratch)
     {
         using AccE = std::remove_reference_t<decltype(acc[0][0][0])>;
-        using OutV = OutT __attribute__((ext_vector_type(4)));
-        const AccE     alpha = static_cast<AccE>(p.alpha), beta = static_cast<AccE>(p.beta);
-        const uint32_t r16 = lane & 15u, g = lane >> 4;
-
-        if(beta == static_cast<AccE>(0))
-        {
-            // Transpose through the wave's own LDS so that a store instruction covers whole rows of
-            // the wave tile (128 to 512 bytes) with 128 bits per lane.  (The epilogue of a 256 x 256 int32 tile
-            // takes 7-9 us whatever else the chip is doing and however few instructions it is made of -- skipping
-            // the alpha multiplication and the per-store address arithmetic changed nothing: 256 KiB leave a CU at
-            // about 16 bytes per clock.)
-            constexpr uint32_t OS         = sizeof(OutT);
-            constexpr uint32_t ROW_BYTES  = 16u * WB * OS;
-            constexpr uint32_t ROW_CHUNKS = ROW_BYTES / CHUNK; // 8, 16 or 32
-            constexpr uint32_t SWZ        = ROW_CHUNKS < 16u ? ROW_CHUNKS - 1u : 15u;
-            constexpr uint32_t FIT        = WB * 4096u / ROW_BYTES; // rows the scratch holds
-            constexpr uint32_t ROWS_PASS  = FIT < 16u * WB ? FIT : 16u * WB;
-            constexpr uint32_t BLOCKS_I   = ROWS_PASS / 16u; // row blocks per pass
-#pragma unroll
-            for(uint32_t pass = 0; pass < WB / BLOCKS_I; ++pass)
-            {
-#pragma unroll
-                for(uint32_t ii = 0; ii < BLOCKS_I; ++ii)
-                {
-                    const uint32_t i = pass * BLOCKS_I + ii, row = 16u * ii + r16;
-#pragma unroll
-                    for(uint32_t j = 0; j < WB; ++j)
-                    {
-                        if constexpr(sizeof(AccE) == 8)
-                        {
-                            // f64 accumulators: element e is column 4 e + lane / 16 of the block
-#pragma unroll
-                            for(uint32_t e = 0; e < 4; ++e)
-                            {
-                                const uint32_t byteInRow = (16u * j + 4u * e + g) * OS;
-                                const uint32_t c = byteInRow / CHUNK, within = byteInRow % CHUNK;
-                                *reinterpret_cast<OutT*>(scratch + row * ROW_BYTES + ((c ^ (row & SWZ)) * CHUNK) + within)
-                                    = static_cast<OutT>(alpha * acc[i][j][e]);
-                            }
-                        }
-                        else
-                        {
-                            OutV out;
-#pragma unroll
-                            for(uint32_t e = 0; e < 4; ++e)
-                                out[e] = static_cast<OutT>(alpha * acc[i][j][e]);
-                            // 16 consecutive rows take 16 (8) different chunk slots
-                            const uint32_t byteInRow = (16u * j + 4u * g) * OS;
-                            const uint32_t c = byteInRow / CHUNK, within = byteInRow % CHUNK;
-                            *reinterpret_cast<OutV*>(scratch + row * ROW_BYTES + ((c ^ (row & SWZ)) * CHUNK) + within) = out;
-                        }
-                    }
-                }
-                __builtin_amdgcn_wave_barrier(); // the same wave reads back what it wrote (LDS is in order per wave)
-#pragma unroll
-                for(uint32_t it = 0; it < ROWS_PASS * ROW_CHUNKS / 64u; ++it)
-                {
-                    const uint32_t L = it * 64u + lane, row = L / ROW_CHUNKS, c = L % ROW_CHUNKS;
-                    const i32x4    v = *reinterpret_cast<const i32x4*>(scratch + row * ROW_BYTES + ((c ^ (row & SWZ)) * CHUNK));
-                    const uint32_t gRow = m0 + pass * ROWS_PASS + row, gCol = n0 + c * (CHUNK / OS);
-                    const uint64_t offD = (uint64_t)gRow * p.ldd + n0;
-                    // D is written once and not read again: stream it past the caches.  Edge tiles:
-                    // m and n are multiples of 16, so a 16-byte chunk is inside D or outside as a whole.
-                    if(gRow < p.m && gCol < p.n)
-                        __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(p.d + offD * OS + c * CHUNK));
-                }
-                __builtin_amdgcn_wave_barrier();
-            }
-            return;
-        }
-        // C may alias D, so loads cannot move above earlier stores: fetch a block row of C at a time
-        if constexpr(sizeof(AccE) == 8)
-        {
-            // f64 accumulators: element e is column 4 e + lane / 16 of the block
-#pragma unroll
-            for(uint32_t i = 0; i < WB; ++i)
-            {
-                const uint32_t row = m0 + 16u * i + r16;
-                OutT           cv[WB][4];
-#pragma unroll
-                for(uint32_t j = 0; j < WB; ++j)
-#pragma unroll
-                    for(uint32_t e = 0; e < 4; ++e)
-                        if(row < p.m && n0 + 16u * j < p.n)
-                            cv[j][e] = *reinterpret_cast<const OutT*>(p.c + ((uint64_t)row * p.ldc + n0 + 16u * j + 4u * e + g) * sizeof(OutT));
-#pragma unroll
-                for(uint32_t j = 0; j < WB; ++j)
-#pragma unroll
-                    for(uint32_t e = 0; e < 4; ++e)
-                        if(row < p.m && n0 + 16u * j < p.n)
-                            *reinterpret_cast<OutT*>(p.d + ((uint64_t)row * p.ldd + n0 + 16u * j + 4u * e + g) * sizeof(OutT))
-                                = static_cast<OutT>(alpha * acc[i][j][e] + beta * static_cast<AccE>(cv[j][e]));
-            }
-            return;
-        }
-#pragma unroll
-        for(uint32_t i = 0; i < WB; ++i)
-        {
-            const uint32_t row = m0 + 16u * i + r16;
-            OutV           cv[WB];
-#pragma unroll
-            for(uint32_t j = 0; j < WB; ++j)
-                if(row < p.m && n0 + 16u * j < p.n)
-                    cv[j] = *reinterpret_cast<const OutV*>(p.c + ((uint64_t)row * p.ldc + n0 + 16u * j + 4u * g) * sizeof(OutT));
-#pragma unroll
-            for(uint32_t j = 0; j < WB; ++j)
-            {
-                OutV out;
-#pragma unroll
-                for(uint32_t e = 0; e < 4; ++e)
-                    out[e] = static_cast<OutT>(alpha * acc[i][j][e] + beta * static_cast<AccE>(cv[j][e]));
-                if(row < p.m && n0 + 16u * j < p.n)
-                    *reinterpret_cast<OutV*>(p.d + ((uint64_t)row * p.ldd + n0 + 16u * j + 4u * g) * sizeof(OutT)) = out;
-            }
-        }
+        if(static_cast<AccE>(p.beta) == static_cast<AccE>(0)) // (as the accumulator type sees it: an int8 problem's beta = 0.5 is 0)
+            storeTileStaged<OutT, false, AccV, OutT, WB>(acc, p, m0, n0, lane, scratch);
+        else
+            storeTileStaged<AccE, true, AccV, OutT, WB>(acc, p, m0, n0, lane, scratch);
     }
 
     //
@@ -1668,8 +1735,10 @@ namespace r355
         const uint32_t kGranule    = CHUNK / es;
         if(g.m % 16 || g.n % 16 || g.m == 0 || g.n == 0 || g.k % kGranule || g.k == 0)
             return fail(R355_ERR_BAD_SIZE, "tiled gemm: m=%u n=%u must be multiples of 16 and k=%u of %u", g.m, g.n, g.k, kGranule);
-        // lane offsets are 32-bit (255 rows of ld elements) and a K stage of an M/N-contiguous operand is one buffer
-        if((uint64_t)g.lda * es > (1u << 23) || (uint64_t)g.ldb * es > (1u << 23))
+        // lane offsets are 32-bit (255 rows of ld elements; the epilogue's: 128 rows of C / D) and a K stage of an
+        // M/N-contiguous operand is one buffer
+        if((uint64_t)g.lda * es > (1u << 23) || (uint64_t)g.ldb * es > (1u << 23) || (uint64_t)g.ldd * os > (1u << 23)
+           || (g.beta != 0.0 && (uint64_t)g.ldc * os > (1u << 23)))
             return fail(R355_ERR_UNSUPPORTED, "tiled gemm: leading dimensions above 8 MiB per row / column");
         if(!aligned(g.a, 16) || !aligned(g.b, 16) || (g.lda * es) % 16 || (g.ldb * es) % 16 || !aligned(g.d, 16)
            || (g.ldd * os) % 16 || (g.beta != 0.0 && (!aligned(g.c, 16) || (g.ldc * os) % 16)))
