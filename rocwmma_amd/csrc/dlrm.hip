@@ -417,7 +417,9 @@ namespace
 #pragma unroll
             for(uint32_t j = 0; j < UP_LOADS; ++j)
                 reinterpret_cast<i32x4*>(upLds)[j * THREADS + tid] = upv[j];
-            if((total & 1u) && tid == 0)
+            // (by the thread whose own 16-byte piece covers it and has just put a zero there: LDS writes of one wave stay
+            // in order, those of different waves do not)
+            if((total & 1u) && tid == ((total - 1u) / 8u) % THREADS)
                 upLds[total - 1u] = upstream[(uint64_t)b0 * upStride + total - 1u];
             for(uint32_t c = inChunks + lane; c < MAX_M * ROW_CHUNKS; c += 64u)
                 *reinterpret_cast<i32x4*>(xw + c * 16u) = i32x4{0, 0, 0, 0};

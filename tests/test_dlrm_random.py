@@ -54,3 +54,24 @@ def test_random_dlrm_fwd_bwd_exact(case):
     gf = g if dtype == O.F32 else O.storage_to_f32(g, dtype)
     wf = w if dtype == O.F32 else O.storage_to_f32(w, dtype)
     assert np.array_equal(gf, wf), (dtype, m, k, batch)
+
+
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16])
+def test_bwd_odd_upstream_run_of_the_last_group_repeated(dtype):
+    """batch = 55, m = 31: the last workgroup's 7 upstream rows of 721 elements are an odd number of 16-bit elements, so
+    the run ends in the middle of a 32-bit word: that last element is fetched on its own and must land in LDS after the
+    16-byte piece around it, whichever wave writes that piece.  Forty launches, every one bit-exact."""
+    m, k, batch = 31, 256, 55
+    store = O.NP_STORAGE[dtype]
+    stride = k + m * (m - 1) // 2
+    assert ((batch % 8) * stride) % 2 == 1
+    x, up = _ints(11, batch * m * k, dtype), _ints(12, batch * stride, dtype)
+    up[-1] = O.f32_to_storage(np.array([3.0], np.float32), dtype)[0]  # the element in question is not zero
+    dx, dup = to_device(x), to_device(up)
+    want_mlp, want_grad = O.dlrm_bwd(dtype, x, up, m, k, batch)
+    wf = O.storage_to_f32(want_grad.ravel(), dtype)
+    for launch in range(40):
+        dmlp, dgrad = device_filled(batch * k, store, 0xEE), device_filled(batch * m * k, store, 0xEE)
+        R.dlrm_bwd(dtype, dx, dup, dmlp, dgrad, m, k, batch)
+        assert np.array_equal(to_host(dmlp, store).view(np.uint8), want_mlp.ravel().view(np.uint8)), launch
+        assert np.array_equal(O.storage_to_f32(to_host(dgrad, store), dtype), wf), launch

@@ -51,7 +51,9 @@ def _draw(case):
     return in_t, out_t, m, n, k, la, lb, ldl, pad_in, pad_out, alpha, beta, workspace, kernel
 
 
-@pytest.mark.parametrize("case", range(CASES))
+# 167, 477: e5m2 -> f32 on the 128 x 128 tile over some 4000 wave tiles.  A 128-bit store whose data registers the next
+# instruction rewrote put that new value into D a few times per thousand wave tiles; only launches this large showed it.
+@pytest.mark.parametrize("case", list(range(CASES)) + [167, 477])
 def test_random_gemm_vs_oracle(case):
     in_t, out_t, m, n, k, la, lb, ldl, pad_in, pad_out, alpha, beta, workspace, kernel = _draw(case)
     layouts = [O.ROW, O.COL]
