@@ -75,7 +75,8 @@ typedef enum
  * Supported (in -> out, accumulate): f16 -> f32|f16 (f32), bf16 -> f32|bf16 (f32),
  * e4m3 -> f32 (f32), e5m2 -> f32 (f32), i8 -> i32|i8 (i32, alpha/beta truncated to int32; an i8 result is the low 8 bits, as the
  * reference's static_cast narrows it), f32 -> f32 (f32), f64 -> f64 (f64).
- * beta == 0 means C is never read and may be NULL.
+ * beta == 0 means C is never read and may be NULL.  C may be D itself (same pointer, leading dimension and orientation:
+ * D = alpha * A * B + beta * D in place); any other overlap of D with A, B or C is undefined.
  *
  * sparse24 != 0: A is 2:4 structured-sparse along k (i8 -> i32, e4m3 | f16 | bf16 -> f32; a 256 x 256 macro-tile kernel
  * from m, n >= 128 on when B is col-major, a block-per-wave kernel otherwise, which takes B in either orientation):

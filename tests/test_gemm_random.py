@@ -112,3 +112,45 @@ def test_random_gemm_vs_oracle(case):
         assert np.all(np.abs(G - exact) <= bound)
     else:
         _check(in_t, out_t, got, want, w32)
+
+
+@pytest.mark.parametrize("kernel", ["auto_large", "tiled_128", "simple", "split_k"])
+@pytest.mark.parametrize("in_t,out_t", [(O.F16, O.F16), (O.F16, O.F32), (O.BF16, O.BF16), (O.I8, O.I32), (O.I8, O.I8), (O.E4M3, O.F32),
+                                        (O.F32, O.F32), (O.F64, O.F64)])
+@pytest.mark.parametrize("ldl", [O.ROW, O.COL])
+def test_c_may_alias_d(kernel, in_t, out_t, ldl):
+    """D = alpha A B + beta D in place (C and D the same pointer, leading dimension and orientation): every kernel reads
+    an element's C before it writes that element's D, and tiles, waves and passes own disjoint elements."""
+    if kernel == "auto_large":
+        m, n, k = 16 * 70, 16 * 66, 16 * 10  # several 256 x 256 tiles plus partial ones
+    elif kernel == "split_k":
+        m, n, k = 64, 192, 16 * 300
+        if in_t in (O.F32, O.F64):
+            pytest.skip("split-K is offered for the 16-bit and 8-bit kernels")
+    else:
+        m, n, k = 16 * 13, 16 * 11, 16 * 8
+    if in_t in (O.F32, O.F64):
+        a = O.uniform_pm1(31, m * k).astype(O.NP_STORAGE[in_t])
+        b = O.uniform_pm1(32, k * n).astype(O.NP_STORAGE[in_t])
+        c = O.uniform_pm1(33, m * n).astype(O.NP_STORAGE[out_t])
+    else:
+        a, b, c = _inputs(in_t, out_t, m, n, k, seed=31)
+    if in_t == O.I8 and out_t == O.I8:
+        c = O.uniform_int8(33, m * n)
+    alpha, beta = (2.0, -1.0) if in_t == O.I8 else (1.0, 1.0) if in_t == O.E4M3 else (0.5, 2.0)
+    want = O.gemm(in_t, out_t, O.ROW, O.COL, ldl, ldl, m, n, k, a, b, c, alpha, beta)
+    da, db, dcd = to_device(a), to_device(b), to_device(c)
+    sel = {"auto_large": R.KERNEL_AUTO, "tiled_128": R.KERNEL_TILED_128, "simple": R.KERNEL_SIMPLE, "split_k": R.KERNEL_AUTO}[kernel]
+    ws = device_filled(8 << 20, np.uint8, 0xA5) if kernel == "split_k" else None
+    if kernel == "split_k":
+        q = R.gemm_query(R.gemm_args(in_t, out_t, m, n, k, da, db, dcd, dcd, alpha, beta, O.ROW, O.COL, ldl, ldl, workspace=ws))
+        assert q.split_k > 1
+    R.gemm(in_t, out_t, m, n, k, da, db, dcd, dcd, alpha, beta, O.ROW, O.COL, ldl, ldl, kernel=sel, workspace=ws)
+    got = to_host(dcd, O.NP_STORAGE[out_t])
+    w32 = None
+    if out_t in (O.F16, O.BF16):
+        w32 = O.gemm(in_t, O.F32, O.ROW, O.COL, ldl, ldl, m, n, k, a, b, O.storage_to_f32(c, out_t), alpha, beta)
+    if in_t == O.F32:
+        assert np.max(np.abs(got.astype(np.float64) - want.astype(np.float64))) <= 1e-4
+    else:
+        _check(in_t, out_t, got, want, w32)
