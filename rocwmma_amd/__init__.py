@@ -85,6 +85,7 @@ def lib():
         vp, u32, i32, f32 = ctypes.c_void_p, ctypes.c_uint32, ctypes.c_int32, ctypes.c_float
         fp = ctypes.POINTER(ctypes.c_float)
         L.r355_gemm.argtypes = [ctypes.POINTER(GemmArgs), vp]
+        L.r355_gemm_noalloc.argtypes = [ctypes.POINTER(GemmArgs), vp]
         L.r355_gemm_query.argtypes = [ctypes.POINTER(GemmArgs), ctypes.POINTER(GemmPlan)]
         L.r355_gemm_timed.argtypes = [ctypes.POINTER(GemmArgs), vp, ctypes.c_int, ctypes.c_int, fp]
         L.r355_dlrm_fwd.argtypes = [i32, vp, vp, u32, u32, u32, vp]
@@ -98,6 +99,8 @@ def lib():
         L.r355_compress_24_16.argtypes = [vp, u32, u32, vp, vp]
         L.r355_decompress_24_16.argtypes = [vp, vp, u32, u32, vp]
         L.r355_get_device_info.argtypes = [ctypes.POINTER(DeviceInfo)]
+        L.r355_last_error.argtypes = []
+        L.r355_version.argtypes = []
         L.r355_last_error.restype = ctypes.c_char_p
         L.r355_version.restype = ctypes.c_char_p
         for name in EXPORTS:

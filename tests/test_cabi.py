@@ -27,6 +27,18 @@ def test_library_exports_every_declared_symbol():
     assert sorted(R.EXPORTS) == names
 
 
+def test_every_export_has_a_ctypes_prototype():
+    """Without argtypes ctypes passes a Python int as a C int: a 64-bit stream handle or pointer would lose its upper half
+    (a call with stream = None hides it).  Every parameter of every declaration must be covered."""
+    text = open(os.path.join(ROOT, "include", "r355_wmma.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    L = R.lib()
+    for name, params in re.findall(r"\b(r355_[a-z0-9_]+)\s*\(([^)]*)\)", text):
+        want = 0 if params.strip() in ("", "void") else params.count(",") + 1
+        fn = getattr(L, name)
+        assert fn.argtypes is not None and len(fn.argtypes) == want, (name, want, fn.argtypes)
+
+
 def test_version_and_error_channel():
     assert "gfx950" in R.version()
     g = R.gemm_args(R.F16, R.F16, 0, 256, 256, 1, 1, None, 1, 1.0, 0.0, R.ROW_MAJOR, R.COL_MAJOR, R.ROW_MAJOR, R.ROW_MAJOR)

@@ -1,0 +1,85 @@
+"""The entry points only launch kernels on the caller's stream (no allocation, no synchronisation, no memset), so a caller
+may record them into a HIP graph.  One graph holding a mixed-tiling GEMM with beta != 0, a split-K GEMM with a workspace,
+the no-allocation split-K GEMM, a 2:4 sparse GEMM, DLRM forward and backward and a GEMV is replayed three times, with eager
+work and synchronisations between the replays; the outputs are reset to a canary before every replay and must equal the
+eager results bit for bit each time (the same kernels in the same order)."""
+import numpy as np
+import pytest
+
+import oraclelib as O
+import rocwmma_amd as R
+from gpuutil import device_filled, to_device, to_host
+from test_gemm import _inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def test_entry_points_replay_from_a_graph():
+    import torch
+
+    ops, outs = [], []
+
+    def add(name, np_dtype, elems, launch):
+        out = device_filled(elems, np_dtype, 0xEE)
+        ops.append((name, launch, out))
+        outs.append((name, np_dtype, out))
+
+    # dense GEMM, several 256 x 256 tiles plus a remainder on the small tile, C read
+    m, n, k = 16 * 70, 16 * 66, 160
+    a, b, c = _inputs(O.F16, O.F16, m, n, k, seed=41)
+    da, db, dc = to_device(a), to_device(b), to_device(c)
+    add("gemm", np.uint16, m * n, lambda out, s: R.gemm(O.F16, O.F16, m, n, k, da, db, dc, out, 2.0, -1.0, O.COL, O.ROW, O.ROW, O.ROW, stream=s))
+    # split-K with a caller's workspace, and through the library's static buffer
+    ms, ns, ks = 64, 192, 4800
+    a2, b2, c2 = _inputs(O.I8, O.I32, ms, ns, ks, seed=42)
+    da2, db2, dc2 = to_device(a2), to_device(b2), to_device(c2)
+    ws = device_filled(8 << 20, np.uint8, 0xA5)
+    add("split_k", np.int32, ms * ns,
+        lambda out, s: R.gemm(O.I8, O.I32, ms, ns, ks, da2, db2, dc2, out, 1.0, 1.0, O.ROW, O.COL, O.ROW, O.ROW, stream=s, workspace=ws))
+    add("noalloc", np.int32, ms * ns,
+        lambda out, s: R.gemm_noalloc(R.gemm_args(O.I8, O.I32, ms, ns, ks, da2, db2, dc2, out, 1.0, 1.0, O.ROW, O.COL, O.ROW, O.ROW), stream=s))
+    # 2:4 sparse
+    mp, np_, kp = 256, 384, 512
+    dense = np.where(O.sparse24_mask(43, mp, kp), O.uniform_int8(44, mp * kp).reshape(mp, kp), np.int8(0)).astype(np.int8)
+    vals, meta = R.compress_24(dense)
+    dv, dm, dbs = to_device(vals), to_device(meta), to_device(O.uniform_int8(45, kp * np_))
+    add("sparse", np.int32, mp * np_,
+        lambda out, s: R.gemm(O.I8, O.I32, mp, np_, kp, dv, dbs, None, out, 1.0, 0.0, O.ROW, O.COL, O.ROW, O.ROW, a_meta=dm, stream=s))
+    # DLRM forward / backward, GEMV
+    f, kd, batch = 27, 128, 203
+    stride = kd + f * (f - 1) // 2
+    x = O.f32_to_storage(O.uniform_pm1(46, batch * f * kd), O.F16)
+    up = O.f32_to_storage(O.uniform_pm1(47, batch * stride), O.F16)
+    dx, dup = to_device(x), to_device(up)
+    add("dlrm_fwd", np.uint16, batch * stride, lambda out, s: R.dlrm_fwd(O.F16, dx, out, f, kd, batch, stream=s))
+    mlp = device_filled(batch * kd, np.uint16, 0xEE)
+    add("dlrm_bwd", np.uint16, batch * f * kd, lambda out, s: R.dlrm_bwd(O.F16, dx, dup, mlp, out, f, kd, batch, stream=s))
+    mv, kv = 4100, 260
+    dav, dxv, dyv = to_device(O.uniform_pm1(48, mv * kv)), to_device(O.uniform_pm1(49, kv)), to_device(O.uniform_pm1(50, mv))
+    add("gemv", np.float32, mv, lambda out, s: R.gemv(O.COL, mv, kv, dav, dxv, dyv, out, 2.0, 2.0, stream=s))
+
+    # eager results (this is also the first call of the no-allocation entry point on this device: its set-up is done here)
+    for _, launch, out in ops:
+        launch(out, None)
+    eager = {name: to_host(out, dt).copy() for name, dt, out in outs}
+    eager_mlp = to_host(mlp, np.uint16).copy()
+    assert not np.all(eager["gemm"].view(np.uint8) == 0xEE)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        for _, launch, out in ops:
+            launch(out, torch.cuda.current_stream())
+    for replay in range(3):
+        for _, _, out in outs:
+            out.fill_(0xEE)
+        mlp.fill_(0xEE)
+        scratch = torch.randn(1 << 20, device="cuda").sum().item()  # the program's own eager work between replays
+        assert np.isfinite(scratch)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, dt, out in outs:
+            assert np.array_equal(to_host(out, dt).view(np.uint8), eager[name].view(np.uint8)), (replay, name)
+        assert np.array_equal(to_host(mlp, np.uint16), eager_mlp), replay
