@@ -698,3 +698,70 @@ def test_padded_leading_dimensions(kernel, in_t, out_t, la, lb, ldl):
     if out_t in (O.F16, O.BF16):
         w32 = O.gemm(in_t, O.F32, la, lb, ldl, ldl, m, n, k, a, b, O.storage_to_f32(c, out_t), alpha, beta)
     _check(in_t, out_t, got, want, w32)
+
+
+@pytest.mark.parametrize("kernel", ["tiled", "auto", "simple"])
+@pytest.mark.parametrize("la", [O.ROW, O.COL])
+def test_operand_beyond_4_gib(la, kernel):
+    """A is 4.6 GB of int8, so byte offsets into it pass 2^32: rows past row 65536 of a row-major A (lda = k = 65536), K rows
+    past 32704 of a col-major one (lda = m = 131328).  Complete rows of D from both sides of the boundary, and rows whose
+    dot product runs across it, against the oracle on the same rows of A; the checksum of checksums covers the rest."""
+    import torch
+
+    if la == O.ROW:
+        m, n, k = 70000, 64, 65536
+        rows = [0, 1, 65535, 65536, 65537, 69999]
+    else:
+        m, n, k = 131072 + 256, 64, 34816
+        rows = [0, 255, 256, 70001, 131071, 131327]
+    g = torch.Generator(device="cuda").manual_seed(21)
+    da = torch.randint(-128, 128, (m * k,), dtype=torch.int8, device="cuda", generator=g)
+    db = torch.randint(-128, 128, (k * n,), dtype=torch.int8, device="cuda", generator=g)  # col-major: n columns of k
+    dd = device_filled(m * n, np.int32, 0xEE)
+    sel = {"tiled": R.KERNEL_TILED, "auto": R.KERNEL_AUTO, "simple": R.KERNEL_SIMPLE}[kernel]
+    R.gemm(O.I8, O.I32, m, n, k, da, db, None, dd, 1.0, 0.0, la, O.COL, O.ROW, O.ROW, kernel=sel)
+    torch.cuda.synchronize()
+    A = da.view(m, k) if la == O.ROW else da.view(k, m).t()
+    a_rows = A[torch.tensor(rows, device="cuda")].contiguous().cpu().numpy()  # (len(rows), k), row-major
+    b = db.cpu().numpy()
+    want = O.gemm(O.I8, O.I32, O.ROW, O.COL, O.ROW, O.ROW, len(rows), n, k, a_rows.ravel(), b, None, 1.0, 0.0)
+    got = dd.view(torch.int32).view(m, n)
+    assert np.array_equal(got[torch.tensor(rows, device="cuda")].cpu().numpy(), want.reshape(len(rows), n))
+    # sum(D) = (1^T A)(B 1), exact in int64
+    col_sums = A.to(torch.int64).sum(dim=0) if la == O.COL else da.view(m, k).to(torch.int32).sum(dim=0, dtype=torch.int64)
+    row_sums = db.view(n, k).to(torch.int64).sum(dim=0)
+    assert int(got.to(torch.int64).sum().item()) == int((col_sums * row_sums).sum().item())
+    del da, db, dd, A, got
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("kernel", ["tiled", "auto", "simple"])
+@pytest.mark.parametrize("lb", [O.COL, O.ROW])
+def test_b_operand_beyond_4_gib(lb, kernel):
+    """The same for B: 4.6 GB of int8, columns past 65536 of a col-major B (ldb = k = 65536) or K rows past 32704 of a
+    row-major one (ldb = n = 131328); complete columns of D against the oracle on the same columns of B."""
+    import torch
+
+    if lb == O.COL:
+        m, n, k = 64, 70000, 65536
+        cols = [0, 1, 65535, 65536, 65537, 69999]
+    else:
+        m, n, k = 64, 131072 + 256, 34816
+        cols = [0, 255, 256, 70001, 131071, 131327]
+    g = torch.Generator(device="cuda").manual_seed(22)
+    da = torch.randint(-128, 128, (m * k,), dtype=torch.int8, device="cuda", generator=g)  # row-major: m rows of k
+    db = torch.randint(-128, 128, (k * n,), dtype=torch.int8, device="cuda", generator=g)
+    dd = device_filled(m * n, np.int32, 0xEE)
+    sel = {"tiled": R.KERNEL_TILED, "auto": R.KERNEL_AUTO, "simple": R.KERNEL_SIMPLE}[kernel]
+    R.gemm(O.I8, O.I32, m, n, k, da, db, None, dd, 1.0, 0.0, O.ROW, lb, O.ROW, O.ROW, kernel=sel)
+    torch.cuda.synchronize()
+    Bt = db.view(n, k) if lb == O.COL else db.view(k, n).t()  # (n, k): row j is column j of B
+    b_cols = Bt[torch.tensor(cols, device="cuda")].contiguous().cpu().numpy()  # as a col-major k x len(cols) matrix
+    want = O.gemm(O.I8, O.I32, O.ROW, O.COL, O.ROW, O.ROW, m, len(cols), k, da.cpu().numpy(), b_cols.ravel(), None, 1.0, 0.0)
+    got = dd.view(torch.int32).view(m, n)
+    assert np.array_equal(got[:, torch.tensor(cols, device="cuda")].cpu().numpy(), want.reshape(m, len(cols)))
+    col_sums = da.view(m, k).to(torch.int64).sum(dim=0)
+    row_sums = Bt.to(torch.int32).sum(dim=0, dtype=torch.int64) if lb == O.COL else db.view(k, n).to(torch.int32).sum(dim=1, dtype=torch.int64)
+    assert int(got.to(torch.int64).sum().item()) == int((col_sums * row_sums).sum().item())
+    del da, db, dd, Bt, got
+    torch.cuda.empty_cache()
