@@ -702,35 +702,50 @@ def test_padded_leading_dimensions(kernel, in_t, out_t, la, lb, ldl):
 
 @pytest.mark.parametrize("kernel", ["tiled", "auto", "simple"])
 @pytest.mark.parametrize("la", [O.ROW, O.COL])
-def test_operand_beyond_4_gib(la, kernel):
-    """A is 4.6 GB of int8, so byte offsets into it pass 2^32: rows past row 65536 of a row-major A (lda = k = 65536), K rows
-    past 32704 of a col-major one (lda = m = 131328).  Complete rows of D from both sides of the boundary, and rows whose
-    dot product runs across it, against the oracle on the same rows of A; the checksum of checksums covers the rest."""
+@pytest.mark.parametrize("in_t", [O.I8, O.F16])
+def test_operand_beyond_4_gib(in_t, la, kernel):
+    """A is 4.6 GB, so byte offsets into it pass 2^32: for int8, rows past row 65536 of a row-major A (lda = k = 65536) or
+    K rows past 32704 of a col-major one (lda = m = 131328); for f16 (values -3 .. 3, every sum exact in f32) half as many
+    columns.  Complete rows of D from both sides of the boundary, and rows whose dot product runs across it, against the
+    oracle on the same rows of A; the checksum of checksums covers the rest."""
     import torch
 
+    es = 1 if in_t == O.I8 else 2
     if la == O.ROW:
-        m, n, k = 70000, 64, 65536
+        m, n, k = 70000, 64, 65536 // es
         rows = [0, 1, 65535, 65536, 65537, 69999]
     else:
-        m, n, k = 131072 + 256, 64, 34816
+        m, n, k = 131072 + 256, 64, 34816 // es
         rows = [0, 255, 256, 70001, 131071, 131327]
     g = torch.Generator(device="cuda").manual_seed(21)
-    da = torch.randint(-128, 128, (m * k,), dtype=torch.int8, device="cuda", generator=g)
-    db = torch.randint(-128, 128, (k * n,), dtype=torch.int8, device="cuda", generator=g)  # col-major: n columns of k
+    if in_t == O.I8:
+        out_t, tdt = O.I32, torch.int32
+        da = torch.randint(-128, 128, (m * k,), dtype=torch.int8, device="cuda", generator=g)
+        db = torch.randint(-128, 128, (k * n,), dtype=torch.int8, device="cuda", generator=g)  # col-major: n columns of k
+    else:
+        out_t, tdt = O.F32, torch.float32
+        da = torch.randint(-3, 4, (m * k,), dtype=torch.int8, device="cuda", generator=g).to(torch.float16)
+        db = torch.randint(-3, 4, (k * n,), dtype=torch.int8, device="cuda", generator=g).to(torch.float16)
     dd = device_filled(m * n, np.int32, 0xEE)
     sel = {"tiled": R.KERNEL_TILED, "auto": R.KERNEL_AUTO, "simple": R.KERNEL_SIMPLE}[kernel]
-    R.gemm(O.I8, O.I32, m, n, k, da, db, None, dd, 1.0, 0.0, la, O.COL, O.ROW, O.ROW, kernel=sel)
+    R.gemm(in_t, out_t, m, n, k, da, db, None, dd, 1.0, 0.0, la, O.COL, O.ROW, O.ROW, kernel=sel)
     torch.cuda.synchronize()
     A = da.view(m, k) if la == O.ROW else da.view(k, m).t()
-    a_rows = A[torch.tensor(rows, device="cuda")].contiguous().cpu().numpy()  # (len(rows), k), row-major
-    b = db.cpu().numpy()
-    want = O.gemm(O.I8, O.I32, O.ROW, O.COL, O.ROW, O.ROW, len(rows), n, k, a_rows.ravel(), b, None, 1.0, 0.0)
-    got = dd.view(torch.int32).view(m, n)
+    host = (lambda t: t.cpu().numpy()) if in_t == O.I8 else (lambda t: t.view(torch.int16).cpu().numpy().view(np.uint16))
+    a_rows = host(A[torch.tensor(rows, device="cuda")].contiguous())  # (len(rows), k), row-major
+    want = O.gemm(in_t, out_t, O.ROW, O.COL, O.ROW, O.ROW, len(rows), n, k, a_rows.ravel(), host(db), None, 1.0, 0.0)
+    got = dd.view(tdt).view(m, n)
     assert np.array_equal(got[torch.tensor(rows, device="cuda")].cpu().numpy(), want.reshape(len(rows), n))
     # sum(D) = (1^T A)(B 1), exact in int64
-    col_sums = A.to(torch.int64).sum(dim=0) if la == O.COL else da.view(m, k).to(torch.int32).sum(dim=0, dtype=torch.int64)
-    row_sums = db.view(n, k).to(torch.int64).sum(dim=0)
-    assert int(got.to(torch.int64).sum().item()) == int((col_sums * row_sums).sum().item())
+    col_sums = torch.zeros(k, dtype=torch.int64, device="cuda")
+    step = 8192 if la == O.ROW else k
+    for r0 in range(0, m if la == O.ROW else k, step):  # in slices: a widened copy of all of A would not fit beside it
+        if la == O.ROW:
+            col_sums += da.view(m, k)[r0:r0 + step].to(torch.int32).sum(dim=0, dtype=torch.int64)
+        else:
+            col_sums = da.view(k, m).to(torch.float32).sum(dim=1).to(torch.int64) if in_t == O.F16 else da.view(k, m).sum(dim=1, dtype=torch.int64)
+    row_sums = db.view(n, k).to(torch.float32).sum(dim=0).to(torch.int64)
+    assert int(got.to(torch.float64).sum().item()) == int((col_sums * row_sums).sum().item())
     del da, db, dd, A, got
     torch.cuda.empty_cache()
 
