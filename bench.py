@@ -262,6 +262,9 @@ def run_extras(R, O, np, torch, args, counters):
         # (f32 output: a kernel instantiation of its own, so that a kernel trace of this run keeps the headline's rows apart)
         gemm_case("gemm_f16_nt_f32out_7168", R.F16, R.F32, R.COL_MAJOR, R.ROW_MAJOR, rnd16(7168 * 7168, False),
                   rnd16(7168 * 7168, False), PEAK_TFLOPS["f16"], "TFLOP/s", mm=7168, nn=7168, kk=7168)
+    if s == 8192:  # operands beyond the 256 MiB memory-side cache (2 x 256 MiB): the 16-bit 256 x 256 tile on its five-buffer K loop
+        gemm_case("gemm_f16_tn_8192x8192x16384", R.F16, R.F16, R.ROW_MAJOR, R.COL_MAJOR, rnd16(s * 16384, False),
+                  rnd16(16384 * s, False), PEAK_TFLOPS["f16"], "TFLOP/s", mm=s, nn=s, kk=16384)
     # f32 and f64 (the reference's perf_sgemm / perf_dgemm samples), TN
     for nm, it, dt, key in (("gemm_f32_tn_%d" % s, R.F32, torch.float32, "f32"), ("gemm_f64_tn_%d" % s, R.F64, torch.float64, "f64")):
         gemm_case(nm, it, it, R.ROW_MAJOR, R.COL_MAJOR, torch.rand(s * s, device="cuda", dtype=dt) * 2 - 1,

@@ -63,9 +63,13 @@ typedef enum
                                 test/gemm/gemm_PGR1_LB2_MP0_MB_CP/device/kernel_device_func.hpp:52-283) */
     R355_KERNEL_TILED_128 = 3, /* the same kernels with a 128 x 128 macro tile (the only one for f64): what AUTO
                                picks when the 256 x 256 tiles of a problem would leave most CUs idle */
-    R355_KERNEL_TILED_128_SPLITK = 4 /* 128 x 128 tiles with K split over several workgroups per tile and a reduction
+    R355_KERNEL_TILED_128_SPLITK = 4, /* 128 x 128 tiles with K split over several workgroups per tile and a reduction
                                (needs `workspace`; what AUTO picks for few tiles and a long K when a workspace is given).
                                No counterpart in the reference. */
+    R355_KERNEL_TILED_DEEP = 5 /* the 256 x 256 macro tile with its K loop on five LDS buffers filled two to three stages ahead.
+                               8-bit and f32 operands always run that way (the selector then equals R355_KERNEL_TILED); for
+                               f16 / bf16 it is what AUTO and R355_KERNEL_TILED take once A and B together exceed the 256 MiB
+                               memory-side cache, where the default two-buffer loop no longer hides the HBM latency. */
 } r355_gemm_kernel;
 
 /*

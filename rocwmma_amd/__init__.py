@@ -19,7 +19,7 @@ F16, BF16, E4M3, I8, F32, I32, F64, E5M2 = range(8)
 # r355_layout
 ROW_MAJOR, COL_MAJOR = 0, 1
 # r355_gemm_kernel
-KERNEL_AUTO, KERNEL_SIMPLE, KERNEL_TILED, KERNEL_TILED_128, KERNEL_TILED_128_SPLITK = 0, 1, 2, 3, 4
+KERNEL_AUTO, KERNEL_SIMPLE, KERNEL_TILED, KERNEL_TILED_128, KERNEL_TILED_128_SPLITK, KERNEL_TILED_DEEP = 0, 1, 2, 3, 4, 5
 
 DTYPE_BYTES = {F16: 2, BF16: 2, E4M3: 1, I8: 1, F32: 4, I32: 4, F64: 8, E5M2: 1}
 

@@ -66,7 +66,7 @@ namespace
         if(g->lda < minLda || g->ldb < minLdb || g->ldd < minLdd || (g->beta != 0.0 && g->ldc < minLdc))
             return r355::fail(R355_ERR_BAD_ARG, "gemm: leading dimension smaller than the contiguous extent");
         if(g->kernel != R355_KERNEL_AUTO && g->kernel != R355_KERNEL_SIMPLE && g->kernel != R355_KERNEL_TILED
-           && g->kernel != R355_KERNEL_TILED_128 && g->kernel != R355_KERNEL_TILED_128_SPLITK)
+           && g->kernel != R355_KERNEL_TILED_128 && g->kernel != R355_KERNEL_TILED_128_SPLITK && g->kernel != R355_KERNEL_TILED_DEEP)
             return r355::fail(R355_ERR_BAD_ARG, "gemm: unknown kernel selector %d", g->kernel);
         return R355_OK;
     }
@@ -89,7 +89,7 @@ namespace
         // clamped edge loads is faster than one block per wave without LDS); the block-per-wave kernel
         // covers the rest: f32 / f64, strides or pointers off 16-byte alignment, k off a 16-byte chunk.
         const bool forced = g->kernel == R355_KERNEL_TILED || g->kernel == R355_KERNEL_TILED_128
-                            || g->kernel == R355_KERNEL_TILED_128_SPLITK;
+                            || g->kernel == R355_KERNEL_TILED_128_SPLITK || g->kernel == R355_KERNEL_TILED_DEEP;
         if(forced || g->kernel == R355_KERNEL_AUTO)
         {
             rc = r355::gemmTiledCheck(*g, out);

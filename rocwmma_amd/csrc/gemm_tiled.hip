@@ -113,6 +113,8 @@ namespace r355
         // and writes its partial D (in the accumulator type) at d + y * splitStrideD bytes; 0 = the whole K in one workgroup
         uint32_t splitStages;
         uint64_t splitStrideD;
+        // host side only: 16-bit operands on the 256 x 256 tile take the five-buffer K loop instead of the two-buffer one
+        uint32_t deepPipeline;
     };
     // sum of `splits` partial results (accumulator type: f32, i32 or f64) + the alpha / beta epilogue into the output type
     int splitKReduce(const r355_gemm_args& g, const GemmTileParams& p, uint32_t splits, hipStream_t stream);
@@ -1259,6 +1261,16 @@ namespace
     {
         gemmTiled5<E, OutT, A_KCONTIG, B_KCONTIG, 4>(p);
     }
+    // The 256 x 256 tile of f16 / bf16 on the five-buffer body: loads two to three stages ahead instead of one.  While the
+    // operands stay in the 256 MiB memory-side cache the two-buffer kernel is 1 - 2.6 % ahead; once A and B together
+    // exceed it, panels are re-fetched from HBM and one stage of lookahead no longer covers the latency
+    // (8192^2 x 16384 TN: 1268 against 1435 TFLOP/s here; 8192 x 12288 x 8192 NN: 1317 against 1474; this body within
+    // 1430 - 1490 over every size and orientation tried).
+    template <Elem E, typename OutT, bool A_KCONTIG, bool B_KCONTIG>
+    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) gemmTiledKernel16Deep(Params p)
+    {
+        gemmTiled5<E, OutT, A_KCONTIG, B_KCONTIG, 8>(p);
+    }
 
     // ------------------------------------------------------------------------------------------
     // fp8 e4m3 on v_mfma_f32_16x16x128_f8f6f4.  One instruction spans the whole 128-byte K stage
@@ -1531,6 +1543,8 @@ namespace
             }
             else if(tile == 128u)
                 hipLaunchKernelGGL((gemmTiledKernel16Small<E, OutT, AK, BK>), grid, block, 0, stream, p);
+            else if(p.deepPipeline)
+                hipLaunchKernelGGL((gemmTiledKernel16Deep<E, OutT, AK, BK>), grid, block, 0, stream, p);
             else
                 hipLaunchKernelGGL((gemmTiledKernel16<E, OutT, AK, BK>), grid, block, 0, stream, p);
         };
@@ -1569,7 +1583,7 @@ namespace
     // the large tiles would leave most CUs idle.
     uint32_t macroTile(const r355_gemm_args& g)
     {
-        if(g.kernel == R355_KERNEL_TILED)
+        if(g.kernel == R355_KERNEL_TILED || g.kernel == R355_KERNEL_TILED_DEEP)
             return 256u; // (f64 is then refused by the check)
         if(g.kernel == R355_KERNEL_TILED_128 || g.kernel == R355_KERNEL_TILED_128_SPLITK || g.in_type == R355_F64)
             return 128u; // f64 accumulators only fit the small wave tile
@@ -1579,6 +1593,20 @@ namespace
         const uint64_t cus    = computeUnits();
         auto           rounds = [&](uint32_t t) { return ((uint64_t)((g.m + t - 1) / t) * ((g.n + t - 1) / t) + cus - 1) / cus; };
         return rounds(128u) * 5u < rounds(256u) * 11u ? 128u : 256u;
+    }
+
+    // 16-bit operands on the 256 x 256 tile: the five-buffer K loop when asked for, or when A and B (as they lie in memory,
+    // leading dimensions included) do not fit the memory-side cache together (gemmTiledKernel16Deep).
+    constexpr uint64_t MEMORY_SIDE_CACHE_BYTES = uint64_t{256} << 20;
+    bool deepPipeline(const r355_gemm_args& g)
+    {
+        if(r355::dtypeBytes(g.in_type) != 2u || macroTile(g) != 256u)
+            return false;
+        if(g.kernel == R355_KERNEL_TILED_DEEP)
+            return true;
+        const uint64_t bytesA = (uint64_t)(g.layout_a == R355_ROW_MAJOR ? g.m : g.k) * g.lda * 2u;
+        const uint64_t bytesB = (uint64_t)(g.layout_b == R355_ROW_MAJOR ? g.k : g.n) * g.ldb * 2u;
+        return bytesA + bytesB > MEMORY_SIDE_CACHE_BYTES;
     }
 
     // ------------------------------------------------------------------------------------------
@@ -1736,7 +1764,7 @@ namespace r355
             return fail(R355_ERR_UNSUPPORTED, "tiled gemm: C and D must share an orientation");
         const uint32_t tk = STAGE_KB / es;
         // K moves in 16-byte chunks; a last K stage that is not full is completed with zeros by the loads
-        const bool     fiveBuffers = es != 2;
+        const bool     fiveBuffers = es != 2 || deepPipeline(g);
         const uint32_t kGranule    = CHUNK / es;
         if(g.m % 16 || g.n % 16 || g.m == 0 || g.n == 0 || g.k % kGranule || g.k == 0)
             return fail(R355_ERR_BAD_SIZE, "tiled gemm: m=%u n=%u must be multiples of 16 and k=%u of %u", g.m, g.n, g.k, kGranule);
@@ -1815,6 +1843,7 @@ namespace r355
             }
         };
         p.splitStages = 0u, p.splitStrideD = 0u;
+        p.deepPipeline = deepPipeline(g) ? 1u : 0u;
         const uint32_t splits = tile == 128u ? splitCount(g) : 1u;
         if(splits > 1u)
         {

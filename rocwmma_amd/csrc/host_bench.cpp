@@ -4,7 +4,7 @@
 // reference does (2 m n k flop, test/performance.hpp:424-442), plus the fraction of MI355X's
 // published peak.  Usage:
 //   host_bench gemm  [--type f16|bf16|i8|e4m3|f32|f64] [--out f16|bf16|f32|i32|f64] [--layout nt|tn|nn|tt]
-//                    [--m M --n N --k K] [--kernel auto|simple|tiled|tiled128] [--warmup W --iters I]
+//                    [--m M --n N --k K] [--kernel auto|simple|tiled|tiled128|deep] [--warmup W --iters I]
 //                    [--sparse 1]   A is 2:4 structured sparse (compressed values + index nibbles)
 //                    [--workspace MiB]  device workspace offered for split-K (few tiles, long K); 0 = none
 //                    [--zero 1]     all-zero operands (no switching power: the engine clock stays at its maximum)
@@ -510,6 +510,7 @@ int main(int argc, char** argv)
         g.kernel = kernel == "simple"     ? R355_KERNEL_SIMPLE
                    : kernel == "tiled"    ? R355_KERNEL_TILED
                    : kernel == "tiled128" ? R355_KERNEL_TILED_128
+                   : kernel == "deep"     ? R355_KERNEL_TILED_DEEP
                                           : R355_KERNEL_AUTO;
         const size_t rowsA = g.layout_a == R355_ROW_MAJOR ? m : k, rowsB = g.layout_b == R355_ROW_MAJOR ? k : n;
         std::vector<uint8_t> ha(sparse ? (size_t)m * k * bytesOf(inT) / 2 : rowsA * g.lda * bytesOf(inT)),

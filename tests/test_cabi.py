@@ -143,7 +143,8 @@ def test_query_plans_cover_every_tile_and_every_k_stage():
     (dict(kernel=R.KERNEL_TILED, m=120), -3),
     (dict(kernel=R.KERNEL_TILED, k=100), -3),
     (dict(kernel=R.KERNEL_TILED_128, m=120), -3),
-    (dict(kernel=5), -1),
+    (dict(kernel=6), -1),
+    (dict(kernel=R.KERNEL_TILED_DEEP, in_type=R.F64, out_type=R.F64), -2),
     (dict(kernel=R.KERNEL_TILED_128_SPLITK), -3),  # no workspace
     (dict(kernel=R.KERNEL_TILED, in_type=R.I8, out_type=R.I32, layout_a=R.ROW_MAJOR, layout_b=R.COL_MAJOR, k=(1 << 23) + 16), -2),
     (dict(kernel=R.KERNEL_TILED, in_type=R.F64, out_type=R.F64), -2),
@@ -228,3 +229,16 @@ def test_compress_24_16bit_elements_same_format():
     with pytest.raises(R.R355Error) as e:
         R.compress_24(bad)
     assert e.value.code == -6
+
+
+def test_deep_pipeline_is_chosen_by_operand_footprint():
+    # A and B of 8192^3 f16 are 256 MiB together - the two-buffer kernel (128 KiB of LDS); a little more k, or a padded
+    # leading dimension, and they no longer fit the memory-side cache: the five-buffer K loop (160 KiB)
+    def q(k, pad, kern=R.KERNEL_AUTO, t=R.F16):
+        return R.gemm_query(_args(in_type=t, out_type=t if t != R.I8 else R.I32, m=8192, n=8192, k=k, layout_a=R.ROW_MAJOR,
+                                  layout_b=R.COL_MAJOR, lda=k + pad, ldb=k + pad, kernel=kern))
+    assert q(8192, 0).lds_bytes == 131072 and q(8192, 0, R.KERNEL_TILED).lds_bytes == 131072
+    assert q(8192, 64).lds_bytes == 163840 and q(8192 + 256, 0).lds_bytes == 163840
+    assert q(16384, 0, R.KERNEL_TILED).lds_bytes == 163840 and q(8192, 0, R.KERNEL_TILED_DEEP).lds_bytes == 163840
+    assert q(8192, 0, R.KERNEL_TILED_DEEP, R.I8).lds_bytes == q(8192, 0, R.KERNEL_TILED, R.I8).lds_bytes == 163840
+    assert q(8192, 0, R.KERNEL_TILED_DEEP).kernel == R.KERNEL_TILED and q(8192, 0, R.KERNEL_TILED_DEEP).macro_tile_m == 256

@@ -780,3 +780,26 @@ def test_b_operand_beyond_4_gib(lb, kernel):
     assert int(got.to(torch.int64).sum().item()) == int((col_sums * row_sums).sum().item())
     del da, db, dd, Bt, got
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("la,lb", [(O.COL, O.ROW), (O.ROW, O.COL), (O.ROW, O.ROW), (O.COL, O.COL)])
+@pytest.mark.parametrize("in_t,out_t", [(O.F16, O.F16), (O.F16, O.F32), (O.BF16, O.BF16), (O.BF16, O.F32)])
+def test_deep_pipeline_16_bit(in_t, out_t, la, lb):
+    """R355_KERNEL_TILED_DEEP: the 256 x 256 tile of the 16-bit types on the five-buffer K loop (what AUTO takes for operands
+    beyond the memory-side cache, forced here at a size the oracle finishes quickly): partial edge tiles in both
+    directions, a K tail, six stages and a remainder, padded leading dimensions, C read."""
+    m, n, k = 16 * 37, 16 * 41, 64 * 7 + 24
+    a, b, c = _inputs(in_t, out_t, m, n, k, seed=71)
+    want = O.gemm(in_t, out_t, la, lb, O.ROW, O.ROW, m, n, k, a, b, c, 2.0, -1.0)
+    lda, ldb = (k if la == O.ROW else m) + 8, (n if lb == O.ROW else k) + 16
+    da, db, dc = to_device(_embed(a, m, k, la, lda, 1)), to_device(_embed(b, k, n, lb, ldb, 1)), to_device(c)
+    dd = device_filled(m * n, O.NP_STORAGE[out_t], 0xEE)
+    args = R.gemm_args(in_t, out_t, m, n, k, da, db, dc, dd, 2.0, -1.0, la, lb, O.ROW, O.ROW, lda=lda, ldb=ldb, kernel=R.KERNEL_TILED_DEEP)
+    plan = R.gemm_query(args)
+    assert plan.kernel == R.KERNEL_TILED and plan.macro_tile_m == 256 and plan.lds_bytes == 5 * 32768
+    R.gemm(in_t, out_t, m, n, k, da, db, dc, dd, 2.0, -1.0, la, lb, O.ROW, O.ROW, lda=lda, ldb=ldb, kernel=R.KERNEL_TILED_DEEP)
+    got = to_host(dd, O.NP_STORAGE[out_t])
+    w32 = None
+    if out_t in (O.F16, O.BF16):
+        w32 = O.gemm(in_t, O.F32, la, lb, O.ROW, O.ROW, m, n, k, a, b, O.storage_to_f32(c, out_t), 2.0, -1.0)
+    _check(in_t, out_t, got, want, w32)

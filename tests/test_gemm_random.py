@@ -48,6 +48,8 @@ def _draw(case):
     kernel = [R.KERNEL_AUTO, R.KERNEL_AUTO, R.KERNEL_TILED, R.KERNEL_TILED_128, R.KERNEL_SIMPLE][int(rng.integers(0, 5))]
     if shape == 4 and kernel == R.KERNEL_SIMPLE:
         kernel = R.KERNEL_AUTO
+    if kernel == R.KERNEL_TILED and case % 2:
+        kernel = R.KERNEL_TILED_DEEP  # the five-buffer K loop also for 16-bit operands (for the others it is the same kernel)
     return in_t, out_t, m, n, k, la, lb, ldl, pad_in, pad_out, alpha, beta, workspace, kernel
 
 
