@@ -69,7 +69,8 @@ typedef enum
     R355_KERNEL_TILED_DEEP = 5 /* the 256 x 256 macro tile with its K loop on five LDS buffers filled two to three stages ahead.
                                8-bit and f32 operands always run that way (the selector then equals R355_KERNEL_TILED); for
                                f16 / bf16 it is what AUTO and R355_KERNEL_TILED take once A and B together exceed the 256 MiB
-                               memory-side cache, where the default two-buffer loop no longer hides the HBM latency. */
+                               memory-side cache, where the default two-buffer loop no longer hides the HBM latency, and for
+                               k <= 1536. */
 } r355_gemm_kernel;
 
 /*

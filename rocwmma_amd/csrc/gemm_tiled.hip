@@ -1578,9 +1578,27 @@ namespace
         return cus;
     }
 
-    // Macro tile edge for a problem.  The 128 x 128 tile (16-bit types) is a quarter of the work of the
-    // 256 x 256 one at about 0.55 of its efficiency (measured with one workgroup per CU): it pays when
-    // the large tiles would leave most CUs idle.
+    // Macro tile edge for a problem.
+    // Long K: the 128 x 128 tile is a quarter of the work of the 256 x 256 one at about 0.55 of its efficiency with one
+    // workgroup per CU, so it pays when the large tiles would leave most CUs idle: 5 rounds128 < 11 rounds256.
+    // Short K (up to 8 stages of 128 bytes): the large tile's prologue, epilogue and the gap between workgroups, which
+    // nothing overlaps with one workgroup per CU, weigh as much as its K loop, while the two small workgroups of a CU hide
+    // each other's.  There the choice follows a timing model - a launch is a number of rounds over the CUs, a round costs a
+    // fixed part plus a part per stage; microseconds fitted to launches of 4096^2 ... 8192^2 with k from 256 to 4096:
+    //                              per round     per stage
+    //   256 x 256, one per CU      9.5 / 13.9      1.30          (16-bit / 8-bit operands: D is 128 / 256 KiB per tile)
+    //   128 x 128, two per CU      3.5 /  5.0    0.84 / 0.88     (a round = both workgroups of a CU; half a round = one)
+    // (8-bit operands at 8192^2: the small tile up to k = 1024, +4 % there, +29 % at 512, +50 % at 256; 16-bit: at k = 256
+    // only, +7 ... +30 %.)  The large tiling's last round runs on small tiles when it would fill at most half of the CUs
+    // (mixedRemainder), and the model prices it that way.
+    struct TileCosts
+    {
+        double round256, stage256, round128, stage128;
+    };
+    TileCosts tileCosts(int32_t inType)
+    {
+        return r355::dtypeBytes(inType) == 1u ? TileCosts{13.9, 1.30, 5.0, 0.88} : TileCosts{9.5, 1.30, 3.5, 0.84};
+    }
     uint32_t macroTile(const r355_gemm_args& g)
     {
         if(g.kernel == R355_KERNEL_TILED || g.kernel == R355_KERNEL_TILED_DEEP)
@@ -1590,19 +1608,34 @@ namespace
         if(g.in_type == R355_F32)
             return 128u; // bound by the matrix-instruction rate either way (146 TFLOP/s at 4096^2 x 2048 with both
                          // tiles), and four times finer rounds: 6144^2 x 2048 runs at 148 TFLOP/s against 111
-        const uint64_t cus    = computeUnits();
-        auto           rounds = [&](uint32_t t) { return ((uint64_t)((g.m + t - 1) / t) * ((g.n + t - 1) / t) + cus - 1) / cus; };
-        return rounds(128u) * 5u < rounds(256u) * 11u ? 128u : 256u;
+        const uint64_t cus  = computeUnits();
+        const uint64_t t256 = (uint64_t)((g.m + 255u) / 256u) * ((g.n + 255u) / 256u);
+        const uint64_t t128 = (uint64_t)((g.m + 127u) / 128u) * ((g.n + 127u) / 128u);
+        if(((t128 + cus - 1u) / cus) * 5u < ((t256 + cus - 1u) / cus) * 11u)
+            return 128u;
+        const uint64_t stages = ((uint64_t)g.k * r355::dtypeBytes(g.in_type) + STAGE_KB - 1u) / STAGE_KB;
+        if(stages > 8u)
+            return 256u; // (at 16 stages the model still picks the small tile now and then where the large one is 3 - 9 % faster)
+        const TileCosts c       = tileCosts(g.in_type);
+        const double    tile256 = c.round256 + c.stage256 * static_cast<double>(stages);
+        const double    pair128 = c.round128 + c.stage128 * static_cast<double>(stages);
+        auto            rounds128 = [&](uint64_t tiles) { return 0.5 * static_cast<double>((tiles + cus - 1u) / cus); };
+        const uint64_t  full = t256 / cus, rest = t256 % cus;
+        double          cost256 = static_cast<double>(full) * tile256;
+        if(rest != 0u)
+            cost256 += (g.kernel == R355_KERNEL_AUTO && full > 0u && rest <= cus / 2u) ? rounds128(4u * rest) * pair128 : tile256;
+        return rounds128(t128) * pair128 < cost256 ? 128u : 256u;
     }
 
-    // 16-bit operands on the 256 x 256 tile: the five-buffer K loop when asked for, or when A and B (as they lie in memory,
-    // leading dimensions included) do not fit the memory-side cache together (gemmTiledKernel16Deep).
+    // 16-bit operands on the 256 x 256 tile: the five-buffer K loop when asked for, when A and B (as they lie in memory,
+    // leading dimensions included) do not fit the memory-side cache together, or when K is short (its prologue has two
+    // stages in flight instead of one: +4 % at k = 512 ... 768, +1 % at 1536, nothing from 2048 on) - gemmTiledKernel16Deep.
     constexpr uint64_t MEMORY_SIDE_CACHE_BYTES = uint64_t{256} << 20;
     bool deepPipeline(const r355_gemm_args& g)
     {
         if(r355::dtypeBytes(g.in_type) != 2u || macroTile(g) != 256u)
             return false;
-        if(g.kernel == R355_KERNEL_TILED_DEEP)
+        if(g.kernel == R355_KERNEL_TILED_DEEP || (uint64_t)g.k * 2u <= 24u * STAGE_KB)
             return true;
         const uint64_t bytesA = (uint64_t)(g.layout_a == R355_ROW_MAJOR ? g.m : g.k) * g.lda * 2u;
         const uint64_t bytesB = (uint64_t)(g.layout_b == R355_ROW_MAJOR ? g.k : g.n) * g.ldb * 2u;

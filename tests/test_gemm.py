@@ -219,25 +219,38 @@ def test_auto_takes_the_small_tile_for_few_tile_problems():
 
 
 @pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.F16, O.F16), (O.E4M3, O.F32), (O.BF16, O.F32)])
-@pytest.mark.parametrize("m,n,k,la,lb,ldl", [(4352, 4352, 128, O.COL, O.ROW, O.ROW),   # 289 tiles: 256 + 33
-                                             (4368, 4112, 80, O.ROW, O.COL, O.ROW),    # partial edge tiles: 18 x 17
-                                             (768, 22016, 64, O.ROW, O.ROW, O.COL),    # 3 x 86 = 258: 2 left over
-                                             (5120, 4880, 48, O.COL, O.COL, O.COL)])   # 20 x 20 = 400: 144 left, one launch
-def test_auto_mixed_tiling_covers_every_tile_once(in_t, out_t, m, n, k, la, lb, ldl):
+@pytest.mark.parametrize("m,n,kbytes,la,lb,ldl", [(4352, 4352, 1280, O.COL, O.ROW, O.ROW),   # 289 tiles: 256 + 33
+                                                  (4368, 4112, 1168, O.ROW, O.COL, O.ROW),   # partial edge tiles: 18 x 17
+                                                  (768, 22016, 1216, O.ROW, O.ROW, O.COL),   # 3 x 86 = 258: 2 left over
+                                                  (5120, 4880, 1200, O.COL, O.COL, O.COL)])  # 20 x 20 = 400: 144 left, one launch
+def test_auto_mixed_tiling_covers_every_tile_once(in_t, out_t, m, n, kbytes, la, lb, ldl):
     """AUTO on a problem whose last round of 256 x 256 tiles would fill at most half of the CUs: whole rounds on the
-    large tile, the rest on 128 x 128 tiles in a second launch.  D starts as 0xFF bytes and C is added, so a tile
-    written twice or not at all shows against the oracle."""
+    large tile, the rest on 128 x 128 tiles in a second launch.  (K is more than 8 stages of 128 bytes: below that AUTO
+    weighs the two tilings by their fixed costs and may take the small tile throughout.)  D starts as 0xFF bytes; four
+    complete rows of every row of tiles are held against the oracle, and a tile nobody wrote shows as NaN, or in the
+    checksum of checksums for int8."""
+    k = kbytes // O.NP_STORAGE[in_t]().itemsize
     cus = R.device_info().compute_units
     total = -(-m // 256) * -(-n // 256)
     rest = total % cus
     mixed = total > cus and 0 < rest <= cus // 2
-    a, b, c = _inputs(in_t, out_t, m, n, k, seed=88)
-    g = R.gemm_args(in_t, out_t, m, n, k, 0x1000, 0x2000, 0x3000, 0x4000, 1.0, 1.0, la, lb, ldl, ldl)
+    a, b, _ = _inputs(in_t, out_t, m, n, k, seed=88)
+    g = R.gemm_args(in_t, out_t, m, n, k, 0x1000, 0x2000, None, 0x4000, 1.0, 0.0, la, lb, ldl, ldl)
     plan = R.gemm_query(g)
     assert plan.macro_tile_m == 256 and plan.grid_x == (total - (rest if mixed else 0) + 7) // 8 * 8
-    want = O.gemm(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, c, 1.0, 1.0)
-    got = _run(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, c, 1.0, 1.0, R.KERNEL_AUTO)
-    _check(in_t, out_t, got, want)
+    got = _run(in_t, out_t, la, lb, ldl, ldl, m, n, k, a, b, None, 1.0, 0.0, R.KERNEL_AUTO)
+    got = got.reshape(m, n) if ldl == O.ROW else got.reshape(n, m).T
+    rows = sorted({min(m - 1, 256 * t + o) for t in range(-(-m // 256)) for o in (0, 127, 128, 255)})
+    want = O.gemm_rows(in_t, out_t, la, lb, m, n, k, a, b, rows)
+    if in_t == O.I8:
+        assert np.array_equal(got[rows], want)
+        A, B = O.as_matrix(a, m, k, la).astype(np.int64), O.as_matrix(b, k, n, lb).astype(np.int64)
+        assert int(got.astype(np.int64).sum()) == int(A.sum(axis=0) @ B.sum(axis=1))
+    else:
+        w32 = O.gemm_rows(in_t, O.F32, la, lb, m, n, k, a, b, rows) if out_t != O.F32 else None
+        _check(in_t, out_t, np.ascontiguousarray(got[rows]).ravel(), want.ravel(), None if w32 is None else w32.ravel())
+        full = got if out_t == O.F32 else O.storage_to_f32(np.ascontiguousarray(got).ravel(), out_t)
+        assert np.all(np.isfinite(full))
 
 
 @pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32)])
