@@ -1591,6 +1591,7 @@ namespace
     // (8-bit operands at 8192^2: the small tile up to k = 1024, +4 % there, +29 % at 512, +50 % at 256; 16-bit: at k = 256
     // only, +7 ... +30 %.)  The large tiling's last round runs on small tiles when it would fill at most half of the CUs
     // (mixedRemainder), and the model prices it that way.
+    constexpr double SECOND_LAUNCH = 4.0; // microseconds between the two launches of a mixed tiling
     struct TileCosts
     {
         double round256, stage256, round128, stage128;
@@ -1623,7 +1624,8 @@ namespace
         const uint64_t  full = t256 / cus, rest = t256 % cus;
         double          cost256 = static_cast<double>(full) * tile256;
         if(rest != 0u)
-            cost256 += (g.kernel == R355_KERNEL_AUTO && full > 0u && rest <= cus / 2u) ? rounds128(4u * rest) * pair128 : tile256;
+            cost256 += (g.kernel == R355_KERNEL_AUTO && full > 0u && rest <= cus / 2u) ? rounds128(4u * rest) * pair128 + SECOND_LAUNCH
+                                                                                      : tile256;
         return rounds128(t128) * pair128 < cost256 ? 128u : 256u;
     }
 
