@@ -157,9 +157,10 @@ int r355_gemm_timed(const r355_gemm_args* args, void* stream, int warmup, int it
 /*
  * DLRM dot-interaction forward.  in: [batch][m][k], out: [batch][k + m(m-1)/2]:
  * out[b][0:k] = in[b][0][:], then the strict lower triangle of X X^T in row-major (i, j<i)
- * order, f32 accumulation, rounded to dtype (R355_F16, R355_BF16 or R355_F32).  2 <= m <= 32,
- * k in {32, 64, 128, 256} (R355_F32: up to 128).  No scratch buffer (the reference's `acc`
- * argument is gone).
+ * order, f32 accumulation, rounded to dtype (R355_F16, R355_BF16 or R355_F32).  Bandwidth-bound kernels for
+ * 2 <= m <= 32 with k in {32, 64, 128, 256} (R355_F32: up to 128); any other m and k that are multiples of 16 - the
+ * reference's own constraint, test/dlrm/dlrm_kernel_base_impl.hpp:146-151; its tests run m = 128, k = 128 and m = k = 1024 -
+ * run block-per-wave kernels (batch <= 65535 there).  No scratch buffer either way (the reference's `acc` argument is gone).
  * Replaces: dlrmDotFwd launch, test/dlrm/dlrm_kernel_base_impl.hpp:78-96,
  * test/dlrm/device/dlrm_dot_fwd.hpp:35-138, samples/simple_dlrm.cpp:184-284.
  */
@@ -170,7 +171,8 @@ int r355_dlrm_fwd_timed(int32_t dtype, const void* in, void* out, uint32_t m, ui
 /*
  * DLRM dot-interaction backward.  upstream: [batch][k + m(m-1)/2]; mlp_grad: [batch][k];
  * in_grad: [batch][m][k].  dtype R355_F16, R355_BF16 (all four pointers 16-byte aligned) or R355_F32
- * (k <= 128; in / in_grad 16-byte, upstream / mlp_grad 4-byte aligned).  Replaces: dlrmDotBwd +
+ * (in / in_grad 16-byte, upstream / mlp_grad 4-byte aligned).  Shapes as for the forward call; the general kernels form S = T + T^T
+ * block by block from the packed triangle instead of reconstructing it in memory.  Replaces: dlrmDotBwd +
  * trilReconstruct launches, test/dlrm/device/dlrm_dot_bwd.hpp:35-176.
  */
 int r355_dlrm_bwd(int32_t dtype, const void* in, const void* upstream, void* mlp_grad, void* in_grad,

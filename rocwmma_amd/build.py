@@ -21,7 +21,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 SOURCES = [("api.cpp", "api", []), ("gemm_simple.hip", "gemm_simple", []),
            ("gemm_tiled.hip", "gemm_tiled_p0", ["-DR355_TILED_PART=0"]), ("gemm_tiled.hip", "gemm_tiled_p1", ["-DR355_TILED_PART=1"]),
            ("gemm_tiled.hip", "gemm_tiled_p2", ["-DR355_TILED_PART=2"]), ("gemm_tiled.hip", "gemm_tiled_p3", ["-DR355_TILED_PART=3"]),
-           ("dlrm.hip", "dlrm", []), ("sparse.hip", "sparse", []), ("gemv.hip", "gemv", [])]
+           ("dlrm.hip", "dlrm", []), ("dlrm_general.hip", "dlrm_general", []), ("sparse.hip", "sparse", []), ("gemv.hip", "gemv", [])]
 
 # packed-fp32 instructions are disabled on purpose (device pass only; the host pass warns that it
 # does not know the feature, which is harmless)

@@ -51,6 +51,10 @@ namespace r355
     int gemmTiledLaunch(const r355_gemm_args& g, hipStream_t stream);
     int gemmSparseCheck(const r355_gemm_args& g, r355_gemm_plan* plan);
     int gemmSparseLaunch(const r355_gemm_args& g, hipStream_t stream);
+    // DLRM shapes beyond the specialised kernels (dlrm_general.hip): m, k multiples of 16
+    int dlrmGeneralFwd(int32_t dtype, const void* in, void* out, uint32_t m, uint32_t k, uint32_t batch, hipStream_t stream);
+    int dlrmGeneralBwd(int32_t dtype, const void* in, const void* upstream, void* mlpGrad, void* inGrad, uint32_t m, uint32_t k,
+                       uint32_t batch, hipStream_t stream);
 } // namespace r355
 
 #endif // R355_COMMON_HPP

@@ -706,17 +706,19 @@ namespace
             return r355::fail(R355_ERR_BAD_ARG, "%s: null pointer", what);
         if(dtype != R355_F16 && dtype != R355_BF16 && !(allowF32 && dtype == R355_F32))
             return r355::fail(R355_ERR_UNSUPPORTED, "%s: dtype must be R355_F16, R355_BF16%s", what, allowF32 ? " or R355_F32" : "");
-        if(dtype == R355_F32 && k > 128)
-            return r355::fail(R355_ERR_BAD_SIZE, "%s: k=%u must be at most 128 for R355_F32", what, k);
-        if(m < 2 || m > MAX_M)
-            return r355::fail(R355_ERR_BAD_SIZE, "%s: m=%u must be in [2, %u]", what, m, MAX_M);
-        if(k != 32 && k != 64 && k != 128 && k != 256)
-            return r355::fail(R355_ERR_BAD_SIZE, "%s: k=%u must be 32, 64, 128 or 256", what, k);
+        if(m < 2)
+            return r355::fail(R355_ERR_BAD_SIZE, "%s: m=%u must be at least 2", what, m);
         if(batch == 0)
             return r355::fail(R355_ERR_BAD_ARG, "%s: batch is zero", what);
         if(!r355::aligned(in, 16) || !r355::aligned(out, 16))
             return r355::fail(R355_ERR_MISALIGNED, "%s: in / out must be 16-byte aligned", what);
         return R355_OK;
+    }
+    // the kernels of this file: up to 32 features and an embedding width they are instantiated for; everything else goes
+    // to the block-per-wave kernels of dlrm_general.hip
+    bool specialised(int32_t dtype, uint32_t m, uint32_t k)
+    {
+        return m <= MAX_M && (k == 32 || k == 64 || k == 128 || (k == 256 && dtype != R355_F32));
     }
 } // namespace
 
@@ -726,6 +728,8 @@ extern "C" int r355_dlrm_fwd(int32_t dtype, const void* in, void* out, uint32_t 
     if(rc != R355_OK)
         return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if(!specialised(dtype, m, k))
+        return r355::dlrmGeneralFwd(dtype, in, out, m, k, batch, s);
     if(dtype == R355_F32)
     {
         const uint32_t steps = (batch + WAVES - 1) / WAVES; // of one sample per wave
@@ -789,6 +793,8 @@ extern "C" int r355_dlrm_bwd(int32_t dtype, const void* in, const void* upstream
         return rc;
     if(!upstream || !mlp_grad)
         return r355::fail(R355_ERR_BAD_ARG, "dlrm_bwd: null pointer");
+    if(!specialised(dtype, m, k))
+        return r355::dlrmGeneralBwd(dtype, in, upstream, mlp_grad, in_grad, m, k, batch, static_cast<hipStream_t>(stream));
     if(dtype == R355_F32)
     {
         if(!r355::aligned(upstream, 4) || !r355::aligned(mlp_grad, 4))

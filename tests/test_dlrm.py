@@ -277,3 +277,53 @@ def test_bwd_integer_inputs_exact():
     R.dlrm_bwd(R.F16, dx, dup, dmlp, dgrad, m, k, batch)
     assert np.array_equal(to_host(dmlp, np.uint16), want_mlp.ravel())
     assert np.array_equal(to_host(dgrad, np.uint16), want.ravel())
+
+
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16, O.F32])
+@pytest.mark.parametrize("m,k,batch", [(128, 128, 64),   # the reference's own test sizes: test/dlrm/test/dlrm_test_params.hpp:57
+                                       (1024, 1024, 2),  # (its fourth size with a smaller batch: the oracle's time)
+                                       (48, 80, 9),      # 3 x 5 blocks of 16: neither a power of two
+                                       (32, 512, 5),     # few features, an embedding width the specialised kernels have no instance for
+                                       (16, 256, 7)])    # (f32: k = 256 is beyond the specialised f32 kernels)
+def test_general_shapes_fwd_and_bwd(dtype, m, k, batch):
+    """More than 32 features, or an embedding width other than 32 / 64 / 128 / 256: the block-per-wave kernels on the fragment
+    API.  Forward and backward against the oracle on the reference's metric (10 eps of the type); integer-valued inputs
+    must come out exactly."""
+    if dtype != O.F32 and (m, k) == (16, 256):
+        pytest.skip("the specialised 16-bit kernels take this shape")
+    store = O.NP_STORAGE[dtype]
+    stride = k + m * (m - 1) // 2
+    scale = 1.0 / np.sqrt(k)  # keeps the dot products of k terms near 1
+    xf, uf = O.normal(91, batch * m * k) * scale, O.normal(92, batch * stride)
+    x = xf.astype(np.float32) if dtype == O.F32 else O.f32_to_storage(xf.astype(np.float32), dtype)
+    up = uf.astype(np.float32) if dtype == O.F32 else O.f32_to_storage(uf.astype(np.float32), dtype)
+    dx, dup = to_device(x), to_device(up)
+    dout = device_filled(batch * stride + 8, store, 0xEE)
+    R.dlrm_fwd(dtype, dx, dout, m, k, batch)
+    out = to_host(dout, store)
+    assert np.all(out[batch * stride:].view(np.uint8) == 0xEE)
+    want = O.dlrm_fwd(dtype, x, m, k, batch)
+    tol = 40.0 if dtype == O.F32 else 10.0  # (f32: the bar of the specialised f32 kernels, a different summation order than the oracle's)
+    ok, mx = O.compare(dtype, out[:batch * stride], want.ravel(), tol)
+    assert ok, mx
+    dmlp, dgrad = device_filled(batch * k + 8, store, 0xEE), device_filled(batch * m * k + 8, store, 0xEE)
+    R.dlrm_bwd(dtype, dx, dup, dmlp, dgrad, m, k, batch)
+    mlp, grad = to_host(dmlp, store), to_host(dgrad, store)
+    assert np.all(mlp[batch * k:].view(np.uint8) == 0xEE) and np.all(grad[batch * m * k:].view(np.uint8) == 0xEE)
+    wmlp, wgrad = O.dlrm_bwd(dtype, x, up, m, k, batch)
+    assert np.array_equal(mlp[:batch * k].view(np.uint8), wmlp.ravel().view(np.uint8))
+    ok, mx = O.compare(dtype, grad[:batch * m * k], wgrad.ravel(), tol)
+    assert ok, mx
+    # small integers: exact in any order
+    xi = np.round(O.uniform_pm1(93, batch * m * k) * 2.0).astype(np.float32)
+    ui = np.round(O.uniform_pm1(94, batch * stride) * 2.0).astype(np.float32)
+    if m * 4 * 2 > 2048 and dtype != O.F32:
+        return  # sums of m products of up to 4 leave the integers a 16-bit gradient holds exactly
+    xi_s, ui_s = (xi, ui) if dtype == O.F32 else (O.f32_to_storage(xi, dtype), O.f32_to_storage(ui, dtype))
+    R.dlrm_fwd(dtype, to_device(xi_s), dout, m, k, batch)
+    assert np.array_equal(to_host(dout, store)[:batch * stride].view(np.uint8), O.dlrm_fwd(dtype, xi_s, m, k, batch).ravel().view(np.uint8))
+    R.dlrm_bwd(dtype, to_device(xi_s), to_device(ui_s), dmlp, dgrad, m, k, batch)
+    g = to_host(dgrad, store)[:batch * m * k]
+    w = O.dlrm_bwd(dtype, xi_s, ui_s, m, k, batch)[1].ravel()
+    gf, wf = (g, w) if dtype == O.F32 else (O.storage_to_f32(g, dtype), O.storage_to_f32(w, dtype))
+    assert np.array_equal(gf, wf)
