@@ -81,6 +81,7 @@ def lib():
             raise ImportError(
                 "rocwmma_amd: %s is missing -- build it with `python -m rocwmma_amd.build`; "
                 "there is no CPU fallback" % LIB_PATH)
+        _share_torch_hip_runtime()
         L = ctypes.CDLL(LIB_PATH)
         vp, u32, i32, f32 = ctypes.c_void_p, ctypes.c_uint32, ctypes.c_int32, ctypes.c_float
         fp = ctypes.POINTER(ctypes.c_float)
@@ -108,6 +109,31 @@ def lib():
                 getattr(L, name).restype = ctypes.c_int
         _lib = L
     return _lib
+
+
+def _share_torch_hip_runtime():
+    """One HIP runtime per process.  A PyTorch wheel ships its own libamdhip64 and loads it by path; this library asks the
+    loader for the system's.  With torch imported first the loader hands this library torch's copy (same SONAME) and all
+    is well; the other way round the process ends up with two runtimes, torch's owns the device and every launch of this
+    library fails with "no ROCm-capable device is detected".  So when a torch installation is present its runtime is
+    loaded first - without importing torch."""
+    import importlib.util
+    import sys
+
+    if "torch" in sys.modules:
+        return
+    try:
+        spec = importlib.util.find_spec("torch")
+    except (ImportError, ValueError):
+        return
+    if spec is None or not spec.submodule_search_locations:
+        return
+    path = os.path.join(list(spec.submodule_search_locations)[0], "lib", "libamdhip64.so")
+    if os.path.exists(path):
+        try:
+            ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
+        except OSError:
+            pass  # (the system's runtime then; only a later `import torch` in this process would be a problem)
 
 
 def _check(rc):

@@ -6,6 +6,7 @@ import pytest
 
 import oraclelib as O
 import rocwmma_amd as R
+from test_gemm import _embed
 from gpuutil import device_filled, to_device, to_host
 
 pytestmark = pytest.mark.gpu
@@ -177,10 +178,22 @@ def test_sparse_random_sweep(case):
     kernel = [R.KERNEL_AUTO, R.KERNEL_TILED, R.KERNEL_SIMPLE][int(rng.integers(0, 3))]
     if lb == O.ROW and kernel == R.KERNEL_TILED:
         kernel = R.KERNEL_AUTO  # the macro tile wants K-contiguous columns of B
-    R.gemm(in_t, out_t, m, n, k, dv, db, dc if beta != 0.0 else None, dd, alpha, beta, O.ROW, lb, ldl, ldl, a_meta=dm, kernel=kernel)
+    # padded leading dimensions of B, C and D (drawn last, so the cases above keep their other draws)
+    pad_b = (16 // es) * int(rng.integers(0, 3))
+    pad_c, pad_d = 4 * int(rng.integers(0, 3)), 4 * int(rng.integers(0, 3))
+    ldb = (n if lb == O.ROW else k) + pad_b
+    ldc, ldd = (n if ldl == O.ROW else m) + pad_c, (n if ldl == O.ROW else m) + pad_d
+    major, minor = (m, n) if ldl == O.ROW else (n, m)
+    canary = np.array([0xEE] * 4, dtype=np.uint8).view(c.dtype)[0]
+    db, dc = to_device(_embed(b, k, n, lb, ldb, 1)), to_device(_embed(c, m, n, ldl, ldc, canary))
+    dd = device_filled(major * ldd + 4, O.NP_STORAGE[out_t], 0xEE)
+    R.gemm(in_t, out_t, m, n, k, dv, db, dc if beta != 0.0 else None, dd, alpha, beta, O.ROW, lb, ldl, ldl, a_meta=dm, kernel=kernel,
+           ldb=ldb, ldc=ldc, ldd=ldd)
     full = to_host(dd, O.NP_STORAGE[out_t])
-    assert np.all(full[m * n:].view(np.uint8) == 0xEE)
-    got = full[:m * n]
+    assert np.all(full[major * ldd:].view(np.uint8) == 0xEE)
+    rows = full[:major * ldd].reshape(major, ldd)
+    assert np.all(rows[:, minor:].view(np.uint8) == 0xEE), "bytes outside D were written"
+    got = np.ascontiguousarray(rows[:, :minor]).ravel()
     if in_t == O.I8:
         assert np.array_equal(got, want), (m, n, k, lb, ldl, kernel)
     else:
