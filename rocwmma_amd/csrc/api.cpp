@@ -165,6 +165,7 @@ extern "C" {
 
 int r355_gemm(const r355_gemm_args* args, void* stream)
 {
+    r355::beginCall();
     int32_t family = 0;
     int     rc     = plan(args, nullptr, &family);
     if(rc != R355_OK)
@@ -176,6 +177,7 @@ int r355_gemm_noalloc(const r355_gemm_args* args, void* stream)
 {
     if(!args)
         return r355::fail(R355_ERR_BAD_ARG, "gemm_noalloc: args is null");
+    r355::beginCall();
     void* at = nullptr;
     int   rc = scratchOfCurrentDevice(&at);
     if(rc != R355_OK)
@@ -214,6 +216,7 @@ int r355_gemm_timed(const r355_gemm_args* args, void* stream, int warmup, int it
     if(rc != R355_OK)
         return rc;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    r355::beginCall();
     return timed(s, warmup, iters, avg_ms, [&] { return launch(args, family, s); });
 }
 

@@ -36,6 +36,13 @@ namespace r355
         return (reinterpret_cast<uintptr_t>(p) % bytes) == 0;
     }
 
+    // At the start of an entry point: the thread's last HIP error is whatever an earlier call of anybody left there (a
+    // probing call that failed harmlessly in another library, say); checkLaunch below must report this call's own.
+    inline void beginCall()
+    {
+        (void)hipGetLastError();
+    }
+
     inline int checkLaunch(const char* what)
     {
         hipError_t e = hipGetLastError();

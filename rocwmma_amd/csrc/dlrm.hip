@@ -727,6 +727,7 @@ extern "C" int r355_dlrm_fwd(int32_t dtype, const void* in, void* out, uint32_t 
     int rc = checkArgs("dlrm_fwd", dtype, in, out, m, k, batch, true);
     if(rc != R355_OK)
         return rc;
+    r355::beginCall();
     hipStream_t s = static_cast<hipStream_t>(stream);
     if(!specialised(dtype, m, k))
         return r355::dlrmGeneralFwd(dtype, in, out, m, k, batch, s);
@@ -793,6 +794,7 @@ extern "C" int r355_dlrm_bwd(int32_t dtype, const void* in, const void* upstream
         return rc;
     if(!upstream || !mlp_grad)
         return r355::fail(R355_ERR_BAD_ARG, "dlrm_bwd: null pointer");
+    r355::beginCall();
     if(!specialised(dtype, m, k))
         return r355::dlrmGeneralBwd(dtype, in, upstream, mlp_grad, in_grad, m, k, batch, static_cast<hipStream_t>(stream));
     if(dtype == R355_F32)

@@ -180,6 +180,7 @@ namespace
         if(!r355::aligned(a, 16) || lda % V || !r355::aligned(x, 16) || !r355::aligned(y_out, 16))
             return r355::fail(R355_ERR_MISALIGNED, "gemv: a, x, y need 16-byte alignment and lda %% %u == 0", V);
         hipStream_t s = static_cast<hipStream_t>(stream);
+        r355::beginCall();
         if(layout_a == R355_COL_MAJOR)
         {
             if(lda < m)
