@@ -200,7 +200,7 @@ def settle(torch, fn, seconds=0.1):
 
 def run_extras(R, O, np, torch, args, counters):
     """The remaining benchmark configurations, each timed with HIP events over args.steps launches; every result is
-    checked for finite values and, for the GEMMs, on sampled elements against a float64 / int64 dot product on the device
+    checked for finite values and on sampled elements (GEMM), samples (DLRM) or rows (GEMV) against a float64 / int64 evaluation on the device
     (the oracle-based parity of the same configurations is in tests/)."""
     out = {}
     s = args.size
@@ -210,6 +210,22 @@ def run_extras(R, O, np, torch, args, counters):
         if c:
             rec["counters"] = {k: v for k, v in c.items() if v is not None}
         return rec
+
+    def dlrm_ok(x, o, up, gmlp, gin, bsz, mm, kk, tol):
+        """32 evenly spaced samples of the batch against a float64 evaluation on the device: the forward's row copy and
+        interaction triangle when `o` is given, the backward's two gradients when `up` is."""
+        pick = torch.arange(0, bsz, bsz // 32, device="cuda")
+        ii, jj = torch.tril_indices(mm, mm, -1, device="cuda")
+        xs = x.view(bsz, mm, kk)[pick].double()
+        close = lambda got, want: bool(((got.double() - want).abs() <= tol * (want.abs() + 1.0)).all())
+        if o is not None:
+            os_ = o.view(bsz, -1)[pick]
+            return close(os_[:, :kk], xs[:, 0]) and close(os_[:, kk:], (xs @ xs.transpose(1, 2))[:, ii, jj])
+        us = up.view(bsz, -1)[pick].double()
+        sm = torch.zeros(len(pick), mm, mm, dtype=torch.float64, device="cuda")
+        sm[:, ii, jj] = us[:, kk:]
+        sm = sm + sm.transpose(1, 2)
+        return close(gmlp.view(bsz, kk)[pick], us[:, :kk]) and close(gin.view(bsz, mm, kk)[pick], sm @ xs)
 
     def sampled_ok(in_t, out_t, la, lb, mm, nn, kk, a, b, d, sparse_meta):
         """64 sampled elements of D against a float64 dot product of the operands as stored (dense cases)."""
@@ -309,7 +325,8 @@ def run_extras(R, O, np, torch, args, counters):
     out["dlrm_fwd_b65536_f27_d128"] = with_counters("dlrm_fwd_b65536_f27_d128", {
         "ms": round(ms, 4), "value": round(byts / ms / 1e6, 1), "unit": "GB/s", "peak": HBM_PEAK_GBPS,
         "frac": round(byts / ms / 1e6 / HBM_PEAK_GBPS, 4), "algorithmic_bytes": byts,
-        "gflops_ref_convention": round(2.0 * mm * mm * kk * bsz / ms / 1e6, 1), "validated": bool(torch.isfinite(o.float()).all())})
+        "gflops_ref_convention": round(2.0 * mm * mm * kk * bsz / ms / 1e6, 1),
+        "validated": bool(torch.isfinite(o.float()).all()) and dlrm_ok(x, o, None, None, None, bsz, mm, kk, 2e-3)})
     # DLRM backward on the same shape: reads X and the upstream gradient, writes both gradients
     up = torch.randn(bsz * (kk + mm * (mm - 1) // 2), device="cuda").to(torch.float16)
     gmlp = torch.empty(bsz * kk, dtype=torch.float16, device="cuda")
@@ -327,7 +344,52 @@ def run_extras(R, O, np, torch, args, counters):
     out["dlrm_bwd_b65536_f27_d128"] = with_counters("dlrm_bwd_b65536_f27_d128", {
         "ms": round(ms, 4), "value": round(byts / ms / 1e6, 1), "unit": "GB/s", "peak": HBM_PEAK_GBPS,
         "frac": round(byts / ms / 1e6 / HBM_PEAK_GBPS, 4), "algorithmic_bytes": byts,
-        "validated": bool(torch.isfinite(gin.float()).all() and torch.isfinite(gmlp.float()).all())})
+        "validated": bool(torch.isfinite(gin.float()).all() and torch.isfinite(gmlp.float()).all())
+        and dlrm_ok(x, None, up, gmlp, gin, bsz, mm, kk, 4e-3)})
+    del up, gmlp, gin, x, o
+    # the same DLRM configuration in f32 (the reference's second DLRM type: test/dlrm/test/dlrm_test_params.hpp:50-53)
+    x32 = torch.randn(bsz * mm * kk, device="cuda")
+    o32 = torch.empty(bsz * (kk + mm * (mm - 1) // 2), device="cuda")
+    up32 = torch.randn(bsz * (kk + mm * (mm - 1) // 2), device="cuda")
+    gmlp32, gin32 = torch.empty(bsz * kk, device="cuda"), torch.empty(bsz * mm * kk, device="cuda")
+
+    def event_ms(fn):
+        settle(torch, fn)
+        a0, a1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for it in range(args.warmup + args.steps):
+            if it == args.warmup:
+                a0.record()
+            fn()
+        a1.record()
+        torch.cuda.synchronize()
+        return a0.elapsed_time(a1) / args.steps
+
+    def hbm_case(name, ms, byts, ok):
+        out[name] = {"ms": round(ms, 4), "value": round(byts / ms / 1e6, 1), "unit": "GB/s", "peak": HBM_PEAK_GBPS,
+                     "frac": round(byts / ms / 1e6 / HBM_PEAK_GBPS, 4), "algorithmic_bytes": byts, "validated": ok}
+
+    ms = event_ms(lambda: R.dlrm_fwd(R.F32, x32, o32, mm, kk, bsz))
+    hbm_case("dlrm_fwd_f32_b65536_f27_d128", ms, bsz * (mm * kk + kk + mm * (mm - 1) // 2) * 4,
+             bool(torch.isfinite(o32).all()) and dlrm_ok(x32, o32, None, None, None, bsz, mm, kk, 1e-5))
+    ms = event_ms(lambda: R.dlrm_bwd(R.F32, x32, up32, gmlp32, gin32, mm, kk, bsz))
+    hbm_case("dlrm_bwd_f32_b65536_f27_d128", ms, (2 * bsz * mm * kk + bsz * (kk + mm * (mm - 1) // 2) + bsz * kk) * 4,
+             bool(torch.isfinite(gin32).all() and torch.isfinite(gmlp32).all()) and dlrm_ok(x32, None, up32, gmlp32, gin32, bsz, mm, kk, 1e-5))
+    del x32, o32, up32, gmlp32, gin32
+    # GEMV y = A x (the reference's simple_sgemv / simple_dgemv samples), A read once: bytes of A, x and y over the HBM peak;
+    # checked against a float64 product on sampled rows
+    for name, dt, fn, gm, gk in (("gemv_f32_col_8192", torch.float32, R.gemv, 8192, 8192), ("gemv_f32_row_16384", torch.float32, R.gemv, 16384, 16384),
+                                 ("gemv_f64_col_8192", torch.float64, R.dgemv, 8192, 8192)):
+        lay = R.COL_MAJOR if "_col_" in name else R.ROW_MAJOR
+        av = torch.rand(gm * gk, device="cuda", dtype=dt) * 2 - 1
+        xv = torch.rand(gk, device="cuda", dtype=dt) * 2 - 1
+        yv = torch.empty(gm, device="cuda", dtype=dt)
+        ms = event_ms(lambda: fn(lay, gm, gk, av, xv, None, yv, 1.0, 0.0))
+        rows = torch.arange(0, gm, gm // 64, device="cuda")
+        amat = av.view(gm, gk) if lay == R.ROW_MAJOR else av.view(gk, gm).t()
+        want = amat[rows].double() @ xv.double()
+        ok = bool(((yv[rows].double() - want).abs() <= 1e-4 * (want.abs() + 1.0)).all())
+        hbm_case(name, ms, (gm * gk + gm + gk) * av.element_size(), ok)
+        del av, xv, yv
     return out
 
 
