@@ -17,6 +17,7 @@
 namespace
 {
     constexpr uint32_t THREADS = 256;
+    constexpr uint32_t SHARED_ROWS = 4; // rows per workgroup of gemvRowMajorShared
 
     // col-major A (m contiguous).  A lane loads 16 bytes = V consecutive rows of one column; RL lanes side by side make a
     // run of RL * 16 bytes of that column and the wave's other lanes take the next 64 / RL - 1 columns, so a workgroup of
@@ -166,6 +167,92 @@ namespace
             yOut[row] = beta != T(0) ? alpha * acc + beta * yIn[row] : alpha * acc;
     }
 
+    // Long rows of a matrix too large for the memory-side cache.  One row per wave (above) has every resident wave on a
+    // row of its own, thousands of 4 KiB pieces a row length apart at any moment, and its rate falls with the row length
+    // (f32, 1 GiB of A: 0.92 of the HBM peak at k = 2048, 0.86 at 8192, 0.82 at 16384, 0.79 at 32768), while the
+    // column-major kernel, whose workgroups together sweep memory linearly, holds 0.89.  Here the WAVES waves of a workgroup
+    // share each row: one load instruction per wave covers WAVES KiB of it together, the workgroup goes through its RB rows one
+    // after the other with that piece of x held in registers, and only then moves on along k.  Each wave waits for its
+    // load before it asks for the next row: variants with two or four loads per row under way, or with the next row's
+    // requested ahead, were slower the more they had in flight (16384^2 f32: 0.77, 0.67, 0.64 of the peak against 0.86),
+    // and so were 8 and 16 rows per workgroup.  Eight waves are ahead for rows below 128 KiB, sixteen from there on
+    // (16384^2: 0.887 / 0.844; 8192 x 32768: 0.818 / 0.882; 32768^2: 0.842 / 0.895; one row per wave: 0.82, 0.79, 0.82).
+    template <typename T, uint32_t WAVES>
+    __global__ void __launch_bounds__(WAVES * 64u) gemvRowMajorShared(uint32_t m,
+                                                                      uint32_t k,
+                                                                      const T* a,
+                                                                      uint32_t lda,
+                                                                      const T* x,
+                                                                      const T* yIn,
+                                                                      T*       yOut,
+                                                                      T        alpha,
+                                                                      T        beta)
+    {
+        constexpr uint32_t V = 16u / sizeof(T), RB = SHARED_ROWS;
+        constexpr uint32_t SLICE = WAVES * 64u * 16u; // bytes one load instruction of the whole workgroup covers
+        constexpr int      NT    = 2; // cache policy: nontemporal (A is read once)
+        using VecT               = T __attribute__((ext_vector_type(V)));
+        __shared__ T   partial[WAVES][RB];
+        const uint32_t lane = threadIdx.x & 63u, w = threadIdx.x / 64u;
+        const uint32_t row0 = blockIdx.x * RB, kBytes = k * (uint32_t)sizeof(T);
+        // One buffer per row and one for x, each k elements long: what a load asks for beyond that comes back as zero, so
+        // a row that does not fill its last slice needs no separate tail, and a row past m (a buffer of no bytes) adds
+        // nothing.  The rows are wave-uniform: their descriptors stay in scalar registers.
+        auto buffer = [](const T* base, uint32_t bytes) {
+            const uint64_t addr = reinterpret_cast<uint64_t>(base);
+            const uint32_t lo   = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(addr));
+            const uint32_t hi   = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(addr >> 32));
+            return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>((static_cast<uint64_t>(hi) << 32) | lo), 0,
+                                                     static_cast<int>(__builtin_amdgcn_readfirstlane(bytes)), 0x00020000);
+        };
+        const __amdgpu_buffer_rsrc_t xr = buffer(x, kBytes);
+        __amdgpu_buffer_rsrc_t       rows[RB];
+        T                            acc[RB];
+#pragma unroll
+        for(uint32_t r = 0; r < RB; ++r)
+        {
+            rows[r] = buffer(a + (uint64_t)(row0 + r < m ? row0 + r : 0u) * lda, row0 + r < m ? kBytes : 0u);
+            acc[r]  = T(0);
+        }
+        const uint32_t mine = (w * 64u + lane) * 16u;
+        for(uint32_t kc = 0; kc < kBytes; kc += SLICE)
+        {
+            const VecT xv = __builtin_bit_cast(VecT, __builtin_amdgcn_raw_buffer_load_b128(xr, mine, kc, 0));
+            VecT       v  = __builtin_bit_cast(VecT, __builtin_amdgcn_raw_buffer_load_b128(rows[0], mine, kc, NT));
+#pragma unroll
+            for(uint32_t r = 0; r < RB; ++r)
+            {
+                __builtin_amdgcn_sched_barrier(0); // (keeps the next row's load behind this row's arithmetic)
+#pragma unroll
+                for(uint32_t e = 0; e < V; ++e)
+                    acc[r] += v[e] * xv[e];
+                __builtin_amdgcn_sched_barrier(0);
+                if(r + 1u < RB)
+                    v = __builtin_bit_cast(VecT, __builtin_amdgcn_raw_buffer_load_b128(rows[r + 1u], mine, kc, NT));
+            }
+        }
+#pragma unroll
+        for(uint32_t r = 0; r < RB; ++r)
+        {
+            T sum = acc[r];
+#pragma unroll
+            for(uint32_t off = 32; off > 0; off >>= 1)
+                sum += __shfl_xor(sum, off, 64);
+            if(lane == 0)
+                partial[w][r] = sum;
+        }
+        __syncthreads();
+        if(threadIdx.x < RB && row0 + threadIdx.x < m)
+        {
+            T sum = T(0);
+#pragma unroll
+            for(uint32_t i = 0; i < WAVES; ++i)
+                sum += partial[i][threadIdx.x];
+            const uint32_t row = row0 + threadIdx.x;
+            yOut[row]          = beta != T(0) ? alpha * sum + beta * yIn[row] : alpha * sum;
+        }
+    }
+
     template <typename T>
     int gemvLaunch(int32_t layout_a, uint32_t m, uint32_t k, const T* a, uint32_t lda, const T* x, const T* y_in, T* y_out,
                    T alpha, T beta, void* stream)
@@ -207,7 +294,19 @@ namespace
             if(lda < k)
                 return r355::fail(R355_ERR_BAD_ARG, "gemv: lda < k");
             const dim3 grid((m + THREADS / 64 - 1) / (THREADS / 64));
-            if((uint64_t)m * lda * sizeof(T) > (256ull << 20))
+            const bool     stream   = (uint64_t)m * lda * sizeof(T) > (256ull << 20);
+            const uint64_t rowBytes = (uint64_t)k * sizeof(T);
+            // rows of 48 KiB and more (measured down to there: 12288 f32; 32 KiB rows are better off with a wave each),
+            // short enough for a 32-bit buffer offset, and enough of them for two workgroups per CU
+            if(stream && rowBytes >= (48u << 10) && rowBytes < (1ull << 31) && m >= SHARED_ROWS * 512u)
+            {
+                const dim3 blocks((m + SHARED_ROWS - 1u) / SHARED_ROWS);
+                if(rowBytes < (128u << 10))
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 8>), blocks, dim3(8 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
+                else
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16>), blocks, dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
+            }
+            else if(stream)
                 hipLaunchKernelGGL((gemvRowMajor<T, true>), grid, dim3(THREADS), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
             else
                 hipLaunchKernelGGL((gemvRowMajor<T, false>), grid, dim3(THREADS), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);

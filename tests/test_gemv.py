@@ -75,3 +75,43 @@ def test_gemv_matrix_beyond_4_gib(layout):
     assert np.all(np.abs(got - exact) <= bound), np.max(np.abs(got - exact) / bound)
     # the bound sees a wrong row
     assert not np.all(np.abs(np.roll(got, 1) - exact) <= bound)
+
+
+@pytest.mark.parametrize("dtype,m,k,pad", [("f32", 4100, 16392, 8),   # rows of 64 KiB and a bit: eight waves per row
+                                           ("f32", 2052, 32772, 0),   # rows beyond 128 KiB: sixteen waves per row
+                                           ("f64", 4098, 8200, 2),    # f64, eight waves; the last workgroup holds two rows
+                                           ("f64", 2050, 16386, 0)])  # f64, sixteen waves
+def test_row_major_rows_shared_by_a_workgroup(dtype, m, k, pad):
+    """Row-major A beyond 256 MiB with rows of 48 KiB and more takes the kernel whose workgroups share each row; the
+    shapes leave a partly filled last slice of k, a partly filled last group of rows and a padded leading dimension.
+    Every row against a float64 (f64: exact integer) evaluation on the device."""
+    import torch
+
+    tdt = torch.float32 if dtype == "f32" else torch.float64
+    fn = R.gemv if dtype == "f32" else R.dgemv
+    lda = k + pad
+    assert m * lda * (4 if dtype == "f32" else 8) > (256 << 20)
+    g = torch.Generator(device="cuda").manual_seed(11)
+    a = (torch.rand(m * lda, device="cuda", generator=g, dtype=tdt) * 2 - 1)
+    x = (torch.rand(k, device="cuda", generator=g, dtype=tdt) * 2 - 1)
+    yin = (torch.rand(m, device="cuda", generator=g, dtype=tdt) * 2 - 1)
+    A = a.view(m, lda)
+    A[:, k:] = float("nan")  # the padding is never read
+    y = torch.full((m,), float("nan"), device="cuda", dtype=tdt)
+    fn(O.ROW, m, k, a, x, yin, y, 2.0, 2.0, lda=lda)
+    torch.cuda.synchronize()
+    Ad, xd = A[:, :k].double(), x.double()
+    exact = 2.0 * (Ad @ xd) + 2.0 * yin.double()
+    eps = 6e-8 if dtype == "f32" else 1.2e-16
+    bound = (Ad.abs() @ xd.abs()) * 2.0 * k * eps + 4.0 * eps
+    err = (y.double() - exact).abs()
+    assert bool((err <= bound).all()), float((err / bound).max())
+    # the bound sees a wrong row
+    assert not bool(((torch.roll(y, 1).double() - exact).abs() <= bound).all())
+    if dtype == "f64":
+        # integer-valued operands: exact in any summation order
+        ai, xi = torch.round(a * 8.0), torch.round(x * 8.0)
+        ai.view(m, lda)[:, k:] = float("nan")
+        fn(O.ROW, m, k, ai, xi, None, y, 1.0, 0.0, lda=lda)
+        torch.cuda.synchronize()
+        assert torch.equal(y, ai.view(m, lda)[:, :k] @ xi)
