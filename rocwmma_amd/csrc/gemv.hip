@@ -296,9 +296,10 @@ namespace
             const dim3 grid((m + THREADS / 64 - 1) / (THREADS / 64));
             const bool     stream   = (uint64_t)m * lda * sizeof(T) > (256ull << 20);
             const uint64_t rowBytes = (uint64_t)k * sizeof(T);
-            // rows of 48 KiB and more (measured down to there: 12288 f32; 32 KiB rows are better off with a wave each),
-            // short enough for a 32-bit buffer offset, and enough of them for two workgroups per CU
-            if(stream && rowBytes >= (48u << 10) && rowBytes < (1ull << 31) && m >= SHARED_ROWS * 512u)
+            // rows of 16 KiB and more (f32, 1 GiB of A, against a wave per row: +1..2 % at 16 KiB, +4 % at 24 KiB, none at
+            // 32 KiB, +5 % at 40 KiB, +7..11 % from 64 KiB on; 8 KiB rows lose 6 %), short enough for a 32-bit buffer
+            // offset, and enough of them for two workgroups per CU
+            if(stream && rowBytes >= (16u << 10) && rowBytes < (1ull << 31) && m >= SHARED_ROWS * 512u)
             {
                 const dim3 blocks((m + SHARED_ROWS - 1u) / SHARED_ROWS);
                 if(rowBytes < (128u << 10))

@@ -77,12 +77,13 @@ def test_gemv_matrix_beyond_4_gib(layout):
     assert not np.all(np.abs(np.roll(got, 1) - exact) <= bound)
 
 
-@pytest.mark.parametrize("dtype,m,k,pad", [("f32", 4100, 16392, 8),   # rows of 64 KiB and a bit: eight waves per row
+@pytest.mark.parametrize("dtype,m,k,pad", [("f32", 10920, 6148, 4),   # rows of 24 KiB: three slices and a bit
+                                           ("f32", 4100, 16392, 8),   # rows of 64 KiB and a bit: eight waves per row
                                            ("f32", 2052, 32772, 0),   # rows beyond 128 KiB: sixteen waves per row
                                            ("f64", 4098, 8200, 2),    # f64, eight waves; the last workgroup holds two rows
                                            ("f64", 2050, 16386, 0)])  # f64, sixteen waves
 def test_row_major_rows_shared_by_a_workgroup(dtype, m, k, pad):
-    """Row-major A beyond 256 MiB with rows of 48 KiB and more takes the kernel whose workgroups share each row; the
+    """Row-major A beyond 256 MiB with rows of 16 KiB and more takes the kernel whose workgroups share each row; the
     shapes leave a partly filled last slice of k, a partly filled last group of rows and a padded leading dimension.
     Every row against a float64 (f64: exact integer) evaluation on the device."""
     import torch
