@@ -83,6 +83,25 @@ def test_gemv_matrix_beyond_4_gib(layout):
                                            ("f64", 4098, 8200, 2),    # f64, eight waves; the last workgroup holds two rows
                                            ("f64", 2050, 16386, 0)])  # f64, sixteen waves
 def test_row_major_rows_shared_by_a_workgroup(dtype, m, k, pad):
+    _shared_rows_case(dtype, m, k, pad)
+
+
+def _random_shared_rows_case(seed):
+    rng = np.random.default_rng(1000 + seed)
+    dtype = "f32" if seed % 2 == 0 else "f64"
+    size, v = (4, 4) if dtype == "f32" else (8, 2)
+    k = int(rng.integers((16 << 10) // size, (300 << 10) // size)) // v * v
+    pad = int(rng.integers(0, 17)) * v
+    m = ((256 << 20) // ((k + pad) * size) + 1 + int(rng.integers(1, 60)) + v - 1) // v * v
+    return dtype, max(m, 2048 + v), k, pad
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_row_major_shared_rows_random_shapes(seed):
+    _shared_rows_case(*_random_shared_rows_case(seed))
+
+
+def _shared_rows_case(dtype, m, k, pad):
     """Row-major A beyond 256 MiB with rows of 16 KiB and more takes the kernel whose workgroups share each row; the
     shapes leave a partly filled last slice of k, a partly filled last group of rows and a padded leading dimension.
     Every row against a float64 (f64: exact integer) evaluation on the device."""
