@@ -12,6 +12,8 @@
 //   host_bench dlrm  [--type f16|bf16|f32] [--bwd 1] [--batch B --m M --k K] [--warmup W --iters I]
 //   host_bench gemv  [--m M --k K --layout n|t]
 //   host_bench copy  [--bytes N]      plain device copy of known size (counter calibration)
+//   host_bench mix                    a bare kernel at the DLRM forward's read / write mix (7 KiB read, 1 KiB written per
+//                                     unit and wave, 65536 units): what plain streaming code reaches at that mix
 //   host_bench lds   [--iters I]      LDS read and write instructions from fixed conflict-free addresses with 4, 2 and 1 waves per CU:
 //                                     shader clocks per wave-level read and bytes per clock per CU
 //   host_bench fill                   direct global -> LDS loads alone, in the access stream of the 8192^3 1-byte GEMM
@@ -436,6 +438,40 @@ namespace
             cyc[0] = c1 - c0;
     }
 
+    // A wave reads seven 1 KiB pieces of a unit with nontemporal loads, adds them up and writes 1 KiB; UNITS consecutive units
+    // per wave, the next one requested before (AHEAD) or after the current one is written.
+    template <int UNITS, bool AHEAD>
+    __global__ void __launch_bounds__(256) mixKernel(const f32x4* __restrict__ in, f32x4* __restrict__ out, uint32_t units)
+    {
+        const uint32_t lane = threadIdx.x & 63u, first = (blockIdx.x * 4u + (threadIdx.x >> 6)) * UNITS;
+        f32x4          cur[7], nxt[7];
+        auto           load = [&](f32x4(&d)[7], uint32_t u) {
+#pragma unroll
+            for(int i = 0; i < 7; ++i)
+                d[i] = __builtin_nontemporal_load(in + (size_t)u * 448u + i * 64u + lane);
+        };
+        if(first >= units)
+            return;
+        load(cur, first);
+        for(int i = 0; i < UNITS && first + i < units; ++i)
+        {
+            const uint32_t u    = first + i;
+            const bool     more = i + 1 < UNITS && u + 1u < units;
+            if(AHEAD && more)
+                load(nxt, u + 1u);
+            f32x4 acc = cur[0];
+#pragma unroll
+            for(int j = 1; j < 7; ++j)
+                acc += cur[j];
+            __builtin_nontemporal_store(acc, out + (size_t)u * 64u + lane);
+            if(!AHEAD && more)
+                load(nxt, u + 1u);
+#pragma unroll
+            for(int j = 0; j < 7; ++j)
+                cur[j] = nxt[j];
+        }
+    }
+
     __global__ void copyKernel(const uint4* __restrict__ src, uint4* __restrict__ dst, size_t n)
     {
         for(size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
@@ -447,7 +483,7 @@ int main(int argc, char** argv)
 {
     if(argc < 2)
     {
-        fprintf(stderr, "usage: host_bench gemm|dlrm|gemv|copy|mfma|lds|fill|store [options]\n");
+        fprintf(stderr, "usage: host_bench gemm|dlrm|gemv|copy|mix|mfma|lds|fill|store [options]\n");
         return 2;
     }
     const std::string op = argv[1];
@@ -856,6 +892,40 @@ int main(int argc, char** argv)
         ms /= iters;
         printf("{\"op\": \"copy\", \"bytes_read\": %zu, \"bytes_written\": %zu, \"ms\": %.4f, \"gbps\": %.1f}\n", bytes,
                bytes, ms, 2.0 * bytes / ms / 1e6);
+    }
+    else if(op == "mix")
+    {
+        const uint32_t units = 65536;
+        void *         src, *dst;
+        HIP_OK(hipMalloc(&src, (size_t)units * 7168));
+        HIP_OK(hipMalloc(&dst, (size_t)units * 1024));
+        HIP_OK(hipMemset(src, 1, (size_t)units * 7168));
+        hipEvent_t e0, e1;
+        HIP_OK(hipEventCreate(&e0));
+        HIP_OK(hipEventCreate(&e1));
+        auto run = [&](auto unitsPerWave, auto ahead) {
+            constexpr int  U = decltype(unitsPerWave)::value;
+            constexpr bool A = decltype(ahead)::value;
+            const dim3     grid((units + 4 * U - 1) / (4 * U));
+            for(int i = 0; i < warmup; ++i)
+                hipLaunchKernelGGL((mixKernel<U, A>), grid, dim3(256), 0, 0, (const f32x4*)src, (f32x4*)dst, units);
+            HIP_OK(hipEventRecord(e0));
+            for(int i = 0; i < iters; ++i)
+                hipLaunchKernelGGL((mixKernel<U, A>), grid, dim3(256), 0, 0, (const f32x4*)src, (f32x4*)dst, units);
+            HIP_OK(hipEventRecord(e1));
+            HIP_OK(hipEventSynchronize(e1));
+            HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+            ms /= iters;
+            printf("{\"op\": \"mix\", \"units_per_wave\": %d, \"next_requested_first\": %d, \"ms\": %.4f, \"gbps\": %.1f, "
+                   "\"frac_hbm_peak\": %.4f}\n",
+                   U, (int)A, ms, units * 8192.0 / ms / 1e6, units * 8192.0 / ms / 1e6 / 8000.0);
+            return 0;
+        };
+        run(std::integral_constant<int, 1>{}, std::false_type{});
+        run(std::integral_constant<int, 2>{}, std::true_type{});
+        run(std::integral_constant<int, 2>{}, std::false_type{});
+        run(std::integral_constant<int, 8>{}, std::true_type{});
+        run(std::integral_constant<int, 8>{}, std::false_type{});
     }
     else
     {
