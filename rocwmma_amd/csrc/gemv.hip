@@ -177,7 +177,7 @@ namespace
     // requested ahead, were slower the more they had in flight (16384^2 f32: 0.77, 0.67, 0.64 of the peak against 0.86),
     // and so were 8 and 16 rows per workgroup.  Eight waves are ahead for rows below 128 KiB, sixteen from there on
     // (16384^2: 0.887 / 0.844; 8192 x 32768: 0.818 / 0.882; 32768^2: 0.842 / 0.895; one row per wave: 0.82, 0.79, 0.82).
-    template <typename T, uint32_t WAVES>
+    template <typename T, uint32_t WAVES, uint32_t RB = SHARED_ROWS>
     __global__ void __launch_bounds__(WAVES * 64u) gemvRowMajorShared(uint32_t m,
                                                                       uint32_t k,
                                                                       const T* a,
@@ -188,7 +188,7 @@ namespace
                                                                       T        alpha,
                                                                       T        beta)
     {
-        constexpr uint32_t V = 16u / sizeof(T), RB = SHARED_ROWS;
+        constexpr uint32_t V = 16u / sizeof(T);
         constexpr uint32_t SLICE = WAVES * 64u * 16u; // bytes one load instruction of the whole workgroup covers
         constexpr int      NT    = 2; // cache policy: nontemporal (A is read once)
         using VecT               = T __attribute__((ext_vector_type(V)));
@@ -299,7 +299,12 @@ namespace
             // rows of 16 KiB and more (f32, 1 GiB of A, against a wave per row: +1..2 % at 16 KiB, +4 % at 24 KiB, none at
             // 32 KiB, +5 % at 40 KiB, +7..11 % from 64 KiB on; 8 KiB rows lose 6 %), short enough for a 32-bit buffer
             // offset, and enough of them for two workgroups per CU
-            if(stream && rowBytes >= (16u << 10) && rowBytes < (1ull << 31) && m >= SHARED_ROWS * 512u)
+            // Few and very long rows leave a wave per row with a handful of waves on the whole chip: a workgroup of sixteen
+            // waves per row instead (f32, 512 MiB of A: 512 rows 0.42 -> 0.64 of the HBM peak, 256 rows 0.23 -> 0.77, 128 rows
+            // 0.12 -> 0.43; from 1024 rows on a wave per row is ahead again)
+            if(m <= 512u && rowBytes >= (128u << 10) && rowBytes < (1ull << 31))
+                hipLaunchKernelGGL((gemvRowMajorShared<T, 16, 1>), dim3(m), dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
+            else if(stream && rowBytes >= (16u << 10) && rowBytes < (1ull << 31) && m >= SHARED_ROWS * 512u)
             {
                 const dim3 blocks((m + SHARED_ROWS - 1u) / SHARED_ROWS);
                 if(rowBytes < (128u << 10))

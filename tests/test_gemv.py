@@ -101,7 +101,14 @@ def test_row_major_shared_rows_random_shapes(seed):
     _shared_rows_case(*_random_shared_rows_case(seed))
 
 
-def _shared_rows_case(dtype, m, k, pad):
+@pytest.mark.parametrize("dtype,m,k,pad", [("f32", 300, 32772, 4), ("f32", 512, 40000, 0), ("f32", 4, 65536, 0),
+                                           ("f64", 66, 16386, 2), ("f64", 2, 20000, 0)])
+def test_row_major_few_long_rows(dtype, m, k, pad):
+    """Up to 512 rows of 128 KiB and more: a workgroup per row, whatever the size of the matrix."""
+    _shared_rows_case(dtype, m, k, pad, streamed=False)
+
+
+def _shared_rows_case(dtype, m, k, pad, streamed=True):
     """Row-major A beyond 256 MiB with rows of 16 KiB and more takes the kernel whose workgroups share each row; the
     shapes leave a partly filled last slice of k, a partly filled last group of rows and a padded leading dimension.
     Every row against a float64 (f64: exact integer) evaluation on the device."""
@@ -110,7 +117,7 @@ def _shared_rows_case(dtype, m, k, pad):
     tdt = torch.float32 if dtype == "f32" else torch.float64
     fn = R.gemv if dtype == "f32" else R.dgemv
     lda = k + pad
-    assert m * lda * (4 if dtype == "f32" else 8) > (256 << 20)
+    assert not streamed or m * lda * (4 if dtype == "f32" else 8) > (256 << 20)
     g = torch.Generator(device="cuda").manual_seed(11)
     a = (torch.rand(m * lda, device="cuda", generator=g, dtype=tdt) * 2 - 1)
     x = (torch.rand(k, device="cuda", generator=g, dtype=tdt) * 2 - 1)
