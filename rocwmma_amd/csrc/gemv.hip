@@ -301,8 +301,9 @@ namespace
             // offset, and enough of them for two workgroups per CU
             // Few and very long rows leave a wave per row with a handful of waves on the whole chip: a workgroup of sixteen
             // waves per row instead (f32, 512 MiB of A: 512 rows 0.42 -> 0.64 of the HBM peak, 256 rows 0.23 -> 0.77, 128 rows
-            // 0.12 -> 0.43; from 1024 rows on a wave per row is ahead again)
-            if(m <= 512u && rowBytes >= (128u << 10) && rowBytes < (1ull << 31))
+            // 0.12 -> 0.43; rows of 512 KiB: 640 rows 0.52 -> 0.67, 768 rows 0.61 -> 0.76, 896 rows even; a wave per row is
+            // ahead again from there on, and from 768 rows of 128 or 256 KiB)
+            if((m <= 512u || (m <= 768u && rowBytes >= (512u << 10))) && rowBytes >= (128u << 10) && rowBytes < (1ull << 31))
                 hipLaunchKernelGGL((gemvRowMajorShared<T, 16, 1>), dim3(m), dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
             else if(stream && rowBytes >= (16u << 10) && rowBytes < (1ull << 31) && m >= SHARED_ROWS * 512u)
             {

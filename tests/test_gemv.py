@@ -102,9 +102,9 @@ def test_row_major_shared_rows_random_shapes(seed):
 
 
 @pytest.mark.parametrize("dtype,m,k,pad", [("f32", 300, 32772, 4), ("f32", 512, 40000, 0), ("f32", 4, 65536, 0),
-                                           ("f64", 66, 16386, 2), ("f64", 2, 20000, 0)])
+                                           ("f32", 700, 131076, 0), ("f64", 66, 16386, 2), ("f64", 2, 20000, 0)])
 def test_row_major_few_long_rows(dtype, m, k, pad):
-    """Up to 512 rows of 128 KiB and more: a workgroup per row, whatever the size of the matrix."""
+    """Up to 512 rows of 128 KiB and more (768 of 512 KiB and more): a workgroup per row, whatever the size of the matrix."""
     _shared_rows_case(dtype, m, k, pad, streamed=False)
 
 
