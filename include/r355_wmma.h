@@ -146,7 +146,11 @@ int r355_gemm_query(const r355_gemm_args* args, r355_gemm_plan* plan);
  * the call allocates and frees nothing.  A problem whose split-K plan needs more than 16 MiB (r355_gemm_query with
  * workspace_bytes = UINT64_MAX reports the need) is refused with R355_ERR_BAD_SIZE; with 4-byte accumulators no plan
  * on 256 CUs needs more.  Nothing in the buffer has to start at zero (every partial result is written before it is
- * read), but all calls on one GPU share it: calls that overlap in time on one GPU (two streams, two threads) race. */
+ * read), but all calls on one GPU share it: calls that overlap in time on one GPU (two streams, two threads) race.
+ * The first call on a device looks up the buffer's address (hipGetSymbolAddress, which may load the library's device
+ * image): it must be made outside stream capture - r355_get_device_info() on that device performs the same look-up and
+ * serves as the set-up call.  A first call that arrives while its stream is capturing is refused with
+ * R355_ERR_UNSUPPORTED and records nothing. */
 int r355_gemm_noalloc(const r355_gemm_args* args, void* stream);
 
 /* Timing helper in the reference's protocol (test/gemm/gemm_kernel_base_impl.hpp:647-676):

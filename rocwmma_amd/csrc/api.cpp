@@ -20,8 +20,11 @@ namespace
     std::mutex    g_scratchLock;
     void*         g_scratchAt[MAX_DEVICES] = {};
 
-    // address of `scratch` on the current device (looked up once per device)
-    int scratchOfCurrentDevice(void** ptr)
+    // address of `scratch` on the current device (looked up once per device).  The lookup may make the runtime load the
+    // library's device image and back the array, which is not something to do while a stream is recording a graph: a
+    // first call on a device that arrives under capture is refused (`capturing` names the stream to test, or nullptr
+    // for "do the lookup": r355_get_device_info is the eager call that prepares a device).
+    int scratchOfCurrentDevice(void** ptr, const hipStream_t* capturing)
     {
         int dev = 0;
         if(hipGetDevice(&dev) != hipSuccess)
@@ -32,6 +35,16 @@ namespace
         std::lock_guard<std::mutex> hold(g_scratchLock);
         if(!g_scratchAt[dev])
         {
+            if(capturing)
+            {
+                hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+                if(hipStreamIsCapturing(*capturing, &status) != hipSuccess || status != hipStreamCaptureStatusNone)
+                    return r355::fail(R355_ERR_UNSUPPORTED,
+                                      "gemm_noalloc: the first call on device %d looks up the library's scratch buffer, which cannot happen "
+                                      "while a stream is capturing; call r355_get_device_info (or r355_gemm_noalloc once) on this device "
+                                      "before the capture begins",
+                                      dev);
+            }
             void*            at = nullptr;
             const hipError_t e  = hipGetSymbolAddress(&at, HIP_SYMBOL(scratch));
             if(e != hipSuccess || !at)
@@ -178,8 +191,9 @@ int r355_gemm_noalloc(const r355_gemm_args* args, void* stream)
     if(!args)
         return r355::fail(R355_ERR_BAD_ARG, "gemm_noalloc: args is null");
     r355::beginCall();
-    void* at = nullptr;
-    int   rc = scratchOfCurrentDevice(&at);
+    void*             at = nullptr;
+    const hipStream_t s  = static_cast<hipStream_t>(stream);
+    int               rc = scratchOfCurrentDevice(&at, &s);
     if(rc != R355_OK)
         return rc;
     // plan as if the workspace were unbounded to learn what split-K of this problem needs, then hold it against the array
@@ -254,7 +268,9 @@ int r355_get_device_info(r355_device_info* info)
     info->memory_clock_mhz    = props.memoryClockRate / 1000;
     info->lds_bytes_per_block = static_cast<int32_t>(props.sharedMemPerBlock);
     info->hbm_bytes           = props.totalGlobalMem;
-    return R355_OK;
+    // the library's per-device set-up: from here on r355_gemm_noalloc on this device calls nothing but kernel launches
+    void* at = nullptr;
+    return scratchOfCurrentDevice(&at, nullptr);
 }
 
 const char* r355_last_error(void)

@@ -36,18 +36,30 @@ namespace r355
         return (reinterpret_cast<uintptr_t>(p) % bytes) == 0;
     }
 
-    // At the start of an entry point: the thread's last HIP error is whatever an earlier call of anybody left there (a
-    // probing call that failed harmlessly in another library, say); checkLaunch below must report this call's own.
+    // The thread's pending HIP error belongs to whoever caused it: an error the caller has not fetched yet (its own
+    // failed call, a probing call of another library) must still be there after a call into this library, as it is
+    // after the reference's plain kernel launch.  So an entry point only looks at it (beginCall), and checkLaunch
+    // reports - and then fetches, since the status code carries it - an error that was not pending at entry.  (A launch
+    // failure with the very code that was already pending cannot be told apart and goes unreported.)
+    inline hipError_t& pendingAtEntry()
+    {
+        thread_local hipError_t pending = hipSuccess;
+        return pending;
+    }
+
     inline void beginCall()
     {
-        (void)hipGetLastError();
+        pendingAtEntry() = hipPeekAtLastError();
     }
 
     inline int checkLaunch(const char* what)
     {
-        hipError_t e = hipGetLastError();
-        if(e != hipSuccess)
+        const hipError_t e = hipPeekAtLastError();
+        if(e != hipSuccess && e != pendingAtEntry())
+        {
+            (void)hipGetLastError();
             return fail(R355_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+        }
         return R355_OK;
     }
 

@@ -15,6 +15,7 @@ using namespace rocwmma;
 namespace
 {
     constexpr uint32_t BLK = 16, WAVES = 4, THREADS = WAVES * 64;
+    constexpr uint32_t GRID_BATCH = 65535; // samples per launch (the batch is grid dimension y or z)
 
     template <typename T>
     constexpr uint32_t blockK()
@@ -141,15 +142,27 @@ namespace
     int fwd(const void* in, void* out, uint32_t m, uint32_t k, uint32_t batch, hipStream_t s)
     {
         const uint32_t tiles = m / BLK, pairs = tiles * (tiles + 1u) / 2u;
-        hipLaunchKernelGGL((dlrmFwdGeneral<T>), dim3((pairs + WAVES - 1u) / WAVES, batch), dim3(THREADS), 0, s, static_cast<const T*>(in),
-                           static_cast<T*>(out), m, k, pairs);
+        const uint64_t stride = (uint64_t)k + (uint64_t)m * (m - 1u) / 2u;
+        // the batch is a grid dimension of at most 65535: a larger one goes out in several launches on the same stream
+        for(uint32_t first = 0; first < batch; first += GRID_BATCH)
+        {
+            const uint32_t count = batch - first < GRID_BATCH ? batch - first : GRID_BATCH;
+            hipLaunchKernelGGL((dlrmFwdGeneral<T>), dim3((pairs + WAVES - 1u) / WAVES, count), dim3(THREADS), 0, s,
+                               static_cast<const T*>(in) + (uint64_t)first * m * k, static_cast<T*>(out) + (uint64_t)first * stride, m, k, pairs);
+        }
         return r355::checkLaunch("dlrm_fwd (general)");
     }
     template <typename T>
     int bwd(const void* in, const void* up, void* mlp, void* grad, uint32_t m, uint32_t k, uint32_t batch, hipStream_t s)
     {
-        hipLaunchKernelGGL((dlrmBwdGeneral<T>), dim3((k / BLK + WAVES - 1u) / WAVES, m / BLK, batch), dim3(THREADS), 0, s,
-                           static_cast<const T*>(in), static_cast<const T*>(up), static_cast<T*>(mlp), static_cast<T*>(grad), m, k);
+        const uint64_t stride = (uint64_t)k + (uint64_t)m * (m - 1u) / 2u;
+        for(uint32_t first = 0; first < batch; first += GRID_BATCH)
+        {
+            const uint32_t count = batch - first < GRID_BATCH ? batch - first : GRID_BATCH;
+            hipLaunchKernelGGL((dlrmBwdGeneral<T>), dim3((k / BLK + WAVES - 1u) / WAVES, m / BLK, count), dim3(THREADS), 0, s,
+                               static_cast<const T*>(in) + (uint64_t)first * m * k, static_cast<const T*>(up) + (uint64_t)first * stride,
+                               static_cast<T*>(mlp) + (uint64_t)first * k, static_cast<T*>(grad) + (uint64_t)first * m * k, m, k);
+        }
         return r355::checkLaunch("dlrm_bwd (general)");
     }
 
@@ -159,8 +172,7 @@ namespace
             return r355::fail(R355_ERR_BAD_SIZE,
                               "%s: m=%u, k=%u - beyond m <= 32 with k of 32, 64, 128 or 256 (f32: up to 128) both must be multiples of %u", what,
                               m, k, BLK);
-        if(batch > 65535u)
-            return r355::fail(R355_ERR_BAD_SIZE, "%s: the general kernels take a batch of at most 65535 (m=%u, k=%u)", what, m, k);
+        (void)batch; // any batch: beyond 65535 samples the launch is repeated (fwd / bwd above)
         return R355_OK;
     }
 } // namespace

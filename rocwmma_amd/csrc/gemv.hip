@@ -177,7 +177,10 @@ namespace
     // requested ahead, were slower the more they had in flight (16384^2 f32: 0.77, 0.67, 0.64 of the peak against 0.86),
     // and so were 8 and 16 rows per workgroup.  Eight waves are ahead for rows below 128 KiB, sixteen from there on
     // (16384^2: 0.887 / 0.844; 8192 x 32768: 0.818 / 0.882; 32768^2: 0.842 / 0.895; one row per wave: 0.82, 0.79, 0.82).
-    template <typename T, uint32_t WAVES, uint32_t RB = SHARED_ROWS>
+    // STREAM: A lies beyond the memory-side cache and is read with nontemporal loads; a smaller one (few very long rows
+    // of a matrix that is multiplied again and again) keeps ordinary loads so that the next call finds it there, as in
+    // gemvRowMajor / gemvColMajor.
+    template <typename T, uint32_t WAVES, uint32_t RB = SHARED_ROWS, bool STREAM = true>
     __global__ void __launch_bounds__(WAVES * 64u) gemvRowMajorShared(uint32_t m,
                                                                       uint32_t k,
                                                                       const T* a,
@@ -190,7 +193,7 @@ namespace
     {
         constexpr uint32_t V = 16u / sizeof(T);
         constexpr uint32_t SLICE = WAVES * 64u * 16u; // bytes one load instruction of the whole workgroup covers
-        constexpr int      NT    = 2; // cache policy: nontemporal (A is read once)
+        constexpr int      NT    = STREAM ? 2 : 0; // cache policy of the loads of A: nontemporal when it is read once
         using VecT               = T __attribute__((ext_vector_type(V)));
         __shared__ T   partial[WAVES][RB];
         const uint32_t lane = threadIdx.x & 63u, w = threadIdx.x / 64u;
@@ -304,7 +307,12 @@ namespace
             // 0.12 -> 0.43; rows of 512 KiB: 640 rows 0.52 -> 0.67, 768 rows 0.61 -> 0.76, 896 rows even; a wave per row is
             // ahead again from there on, and from 768 rows of 128 or 256 KiB)
             if((m <= 512u || (m <= 768u && rowBytes >= (512u << 10))) && rowBytes >= (128u << 10) && rowBytes < (1ull << 31))
-                hipLaunchKernelGGL((gemvRowMajorShared<T, 16, 1>), dim3(m), dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
+            {
+                if(stream)
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16, 1, true>), dim3(m), dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
+                else
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16, 1, false>), dim3(m), dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
+            }
             else if(stream && rowBytes >= (16u << 10) && rowBytes < (1ull << 31) && m >= SHARED_ROWS * 512u)
             {
                 const dim3 blocks((m + SHARED_ROWS - 1u) / SHARED_ROWS);

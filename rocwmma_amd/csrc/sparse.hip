@@ -481,7 +481,8 @@ namespace
         const uint32_t es = (g.in_type == R355_F16 || g.in_type == R355_BF16) ? 2u : 1u;
         const bool     forced = g.kernel == R355_KERNEL_TILED || g.kernel == R355_KERNEL_TILED_DEEP; // (one and the same here)
         const bool     shape  = forced || (g.m >= T_M / 2 && g.n >= T_N / 2);
-        return g.kernel != R355_KERNEL_SIMPLE && shape && g.layout_b == R355_COL_MAJOR && g.layout_c == g.layout_d && r355::aligned(g.a_meta, 16)
+        return g.kernel != R355_KERNEL_SIMPLE && shape && g.layout_b == R355_COL_MAJOR && (g.beta == 0.0 || g.layout_c == g.layout_d)
+               && r355::aligned(g.a_meta, 16)
                && (uint64_t)g.ldb * es <= (1u << 23);
     }
 
@@ -516,7 +517,7 @@ namespace r355
             return fail(R355_ERR_UNSUPPORTED, "sparse gemm: there is no 128 x 128 sparse macro tile (R355_KERNEL_TILED is 256 x 256)");
         if((g.kernel == R355_KERNEL_TILED || g.kernel == R355_KERNEL_TILED_DEEP) && !tiledOk(g))
             return fail(R355_ERR_UNSUPPORTED,
-                        "sparse gemm (macro tile): B must be col-major, C and D must share an orientation, metadata 16-byte aligned, ldb below 8 MiB");
+                        "sparse gemm (macro tile): B must be col-major, C (when beta != 0) and D must share an orientation, metadata 16-byte aligned, ldb below 8 MiB");
         if(plan && tiledOk(g))
         {
             plan->kernel       = R355_KERNEL_TILED;

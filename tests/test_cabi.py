@@ -158,6 +158,19 @@ def test_argument_validation(kw, code):
     assert str(e.value)
 
 
+def test_sparse_macro_tile_ignores_the_orientation_of_an_unread_c():
+    # beta == 0: C is never read, so layout_c means nothing and must not push the call off the 256 x 256 sparse macro tile
+    sp = dict(in_type=R.I8, out_type=R.I32, m=512, n=512, k=1024, lda=512, layout_a=R.ROW_MAJOR, layout_b=R.COL_MAJOR,
+              a_meta=0x4000)
+    assert R.gemm_query(_args(layout_c=R.COL_MAJOR, layout_d=R.ROW_MAJOR, **sp)).kernel == R.KERNEL_TILED
+    assert R.gemm_query(_args(layout_c=R.COL_MAJOR, layout_d=R.ROW_MAJOR, kernel=R.KERNEL_TILED, **sp)).kernel == R.KERNEL_TILED
+    # beta != 0 with differing orientations: the block-per-wave kernel, and the forced macro tile is refused
+    assert R.gemm_query(_args(layout_c=R.COL_MAJOR, layout_d=R.ROW_MAJOR, beta=1.0, c=0x5000, **sp)).kernel == R.KERNEL_SIMPLE
+    with pytest.raises(R.R355Error) as e:
+        R.gemm_query(_args(layout_c=R.COL_MAJOR, layout_d=R.ROW_MAJOR, beta=1.0, c=0x5000, kernel=R.KERNEL_TILED, **sp))
+    assert e.value.code == -2
+
+
 def test_dlrm_and_gemv_validation_without_gpu():
     with pytest.raises(R.R355Error) as e:
         R.dlrm_fwd(R.F16, 0x1000, 0x2000, 40, 128, 8)

@@ -327,3 +327,25 @@ def test_general_shapes_fwd_and_bwd(dtype, m, k, batch):
     w = O.dlrm_bwd(dtype, xi_s, ui_s, m, k, batch)[1].ravel()
     gf, wf = (g, w) if dtype == O.F32 else (O.storage_to_f32(g, dtype), O.storage_to_f32(w, dtype))
     assert np.array_equal(gf, wf)
+
+
+def test_general_shapes_take_a_batch_beyond_one_grid_dimension():
+    """The general kernels put the batch into a grid dimension (at most 65535); a larger batch goes out in several
+    launches, as the specialised kernels take any batch.  Samples either side of the launch boundary against the oracle."""
+    m, k, batch = 48, 16, 65536 + 40
+    stride = k + m * (m - 1) // 2
+    x = O.f32_to_storage(np.round(O.uniform_pm1(95, batch * m * k) * 2.0), O.F16)
+    up = O.f32_to_storage(np.round(O.uniform_pm1(96, batch * stride) * 2.0), O.F16)
+    dx, dup = to_device(x), to_device(up)
+    dout = device_filled(batch * stride + 8, np.uint16, 0xEE)
+    dmlp, dgrad = device_filled(batch * k + 8, np.uint16, 0xEE), device_filled(batch * m * k + 8, np.uint16, 0xEE)
+    R.dlrm_fwd(R.F16, dx, dout, m, k, batch)
+    R.dlrm_bwd(R.F16, dx, dup, dmlp, dgrad, m, k, batch)
+    out, mlp, grad = to_host(dout, np.uint16), to_host(dmlp, np.uint16), to_host(dgrad, np.uint16)
+    assert np.all(out[batch * stride:] == 0xEEEE) and np.all(mlp[batch * k:] == 0xEEEE) and np.all(grad[batch * m * k:] == 0xEEEE)
+    for first, count in ((0, 8), (65535 - 20, 40), (batch - 8, 8)):
+        xs, us = x[first * m * k:(first + count) * m * k], up[first * stride:(first + count) * stride]
+        assert np.array_equal(out[first * stride:(first + count) * stride], O.dlrm_fwd(O.F16, xs, m, k, count).ravel())
+        wmlp, wgrad = O.dlrm_bwd(O.F16, xs, us, m, k, count)
+        assert np.array_equal(mlp[first * k:(first + count) * k], wmlp.ravel())
+        assert np.array_equal(grad[first * m * k:(first + count) * m * k], wgrad.ravel())

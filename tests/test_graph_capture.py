@@ -83,3 +83,56 @@ def test_entry_points_replay_from_a_graph():
         for name, dt, out in outs:
             assert np.array_equal(to_host(out, dt).view(np.uint8), eager[name].view(np.uint8)), (replay, name)
         assert np.array_equal(to_host(mlp, np.uint16), eager_mlp), replay
+
+
+_FIRST_CALL_UNDER_CAPTURE = r"""
+import sys
+sys.path.insert(0, %(root)r); sys.path.insert(0, %(tests)r)
+import numpy as np, torch
+import oraclelib as O, rocwmma_amd as R
+from gpuutil import device_filled, to_device, to_host
+from test_gemm import _inputs
+m, n, k = 64, 192, 4800
+a, b, c = _inputs(O.I8, O.I32, m, n, k, seed=42)
+da, db, dc = to_device(a), to_device(b), to_device(c)
+out = device_filled(m * n, np.int32, 0xEE)
+args = R.gemm_args(O.I8, O.I32, m, n, k, da, db, dc, out, 1.0, 1.0, O.ROW, O.COL, O.ROW, O.ROW)
+side = torch.cuda.Stream()
+side.wait_stream(torch.cuda.current_stream())
+graph = torch.cuda.CUDAGraph()
+refused = None
+with torch.cuda.graph(graph, stream=side):
+    try:  # the very first call of the entry point in this process, while the stream records
+        R.gemm_noalloc(args, stream=torch.cuda.current_stream())
+    except R.R355Error as e:
+        refused = (e.code, str(e))
+assert refused is not None and refused[0] == -2 and "r355_get_device_info" in refused[1], refused
+torch.cuda.synchronize()
+R.device_info()  # the set-up call: looks the scratch buffer up
+graph = torch.cuda.CUDAGraph()
+with torch.cuda.graph(graph, stream=side):
+    R.gemm_noalloc(args, stream=torch.cuda.current_stream())
+assert np.all(to_host(out, np.int32).view(np.uint8) == 0xEE)  # recorded, not run
+for _ in range(2):
+    out.fill_(0xEE)
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    want = O.gemm(O.I8, O.I32, O.ROW, O.COL, O.ROW, O.ROW, m, n, k, a, b, c, 1.0, 1.0)
+    assert np.array_equal(to_host(out, np.int32), want)
+print("ok")
+"""
+
+
+def test_first_noalloc_call_under_capture_is_refused_until_the_device_is_set_up():
+    """In a fresh process: the first r355_gemm_noalloc on a device would look up the library's scratch buffer, which must
+    not happen while a stream records - it is refused with a message that names the set-up call; after
+    r355_get_device_info the same call records and replays bit-exact against the oracle."""
+    import os
+    import subprocess
+    import sys
+
+    tests = os.path.dirname(os.path.abspath(__file__))
+    code = _FIRST_CALL_UNDER_CAPTURE % {"root": os.path.dirname(tests), "tests": tests}
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and r.stdout.strip().endswith("ok"), r.stdout[-2000:] + r.stderr[-4000:]
