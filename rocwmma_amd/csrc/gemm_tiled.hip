@@ -628,18 +628,21 @@ namespace
         auto rsrcAt = [](uint64_t addr, uint32_t records) { // raw buffer, 32-bit data format, no swizzle
             return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>(addr), 0, static_cast<int>(records), 0x00020000);
         };
-        // load x of a stage with vA / vB valid bytes of K: x = 2 j loads piece j of A, x = 2 j + 1 piece j of B
-        auto issueLoad = [&](__amdgpu_buffer_rsrc_t srcA, __amdgpu_buffer_rsrc_t srcB, uint32_t vA, uint32_t vB, char* stage,
-                             uint32_t x) {
+        // load x of a stage with vA / vB valid bytes of K: x = 2 j loads piece j of A, x = 2 j + 1 piece j of B.  `full`
+        // (a compile-time tag): the stage is known to be a whole one, so no lane has a chunk beyond K and the lane offsets
+        // are used as they are - the K loop's main part carries no select per load.
+        auto issueLoad = [&](auto full, __amdgpu_buffer_rsrc_t srcA, __amdgpu_buffer_rsrc_t srcB, uint32_t vA, uint32_t vB,
+                             char* stage, uint32_t x) {
             using lp         = __attribute__((address_space(3))) void*;
+            constexpr bool FULL = decltype(full)::value;
             const uint32_t j = x >> 1;
             char*          dst = stage + (j * THREADS + wave * 64u) * CHUNK;
             if(x & 1u)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(srcB, (lp)(dst + OPER), 16, tailOffset(B_KCONTIG, gOffB[j], kByteB, vB),
-                                                         j * gStepB, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(srcB, (lp)(dst + OPER), 16,
+                                                         FULL ? gOffB[j] : tailOffset(B_KCONTIG, gOffB[j], kByteB, vB), j * gStepB, 0, 0);
             else
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(srcA, (lp)dst, 16, tailOffset(A_KCONTIG, gOffA[j], kByteA, vA), j * gStepA, 0,
-                                                         0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(srcA, (lp)dst, 16,
+                                                         FULL ? gOffA[j] : tailOffset(A_KCONTIG, gOffA[j], kByteA, vA), j * gStepA, 0, 0);
         };
         auto issueGlobal = [&](uint32_t kt, char* stage) {
             const uint32_t               v    = validOf(kt);
@@ -647,7 +650,7 @@ namespace
                                          srcB = rsrcAt(uniform64(gB + kt * gStageB), stageRecords(B_KCONTIG, v, p.ldb));
 #pragma unroll
             for(uint32_t x = 0; x < 2u * LOADS; ++x)
-                issueLoad(srcA, srcB, v, v, stage, x);
+                issueLoad(std::false_type{}, srcA, srcB, v, v, stage, x);
         };
 
         f32x4          acc[WB][WB];
@@ -696,8 +699,11 @@ namespace
         // between pieces (groups of two with the small wave tile: read, read + direct load).  Every stage
         // runs the same code: past the end the refill has nothing in range (it writes zeros) and the operands read
         // ahead are never used.
+        // `full` (compile-time tag): the stage this one refills (kt + 2) and the one after it are whole stages inside K - the
+        // main part of the K loop, whose loads then carry no tail select and whose refill pointers always advance.
         constexpr uint32_t LOAD_Q = QS > 2u ? 2u : QS - 1u;
-        auto stageBody = [&](uint32_t kt, char* cur, char* nxt) {
+        auto stageBody = [&](auto full, uint32_t kt, char* cur, char* nxt) {
+            constexpr bool FULL = decltype(full)::value;
 #pragma unroll
             for(uint32_t x = 0; x < XS; ++x)
             {
@@ -712,10 +718,10 @@ namespace
             }
             __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): stage kt + 1 has landed
             __syncthreads();
-            const uint32_t               v    = validOf(kt + 2u);
+            const uint32_t               v    = FULL ? STAGE_KB : validOf(kt + 2u);
             const __amdgpu_buffer_rsrc_t srcA = rsrcAt(refillA, stageRecords(A_KCONTIG, v, p.lda)),
                                          srcB = rsrcAt(refillB, stageRecords(B_KCONTIG, v, p.ldb));
-            if(kt + 3u < numStages) // the refill of the next stage is one stage further, or the last again
+            if(FULL || kt + 3u < numStages) // the refill of the next stage is one stage further, or the last again
                 refillA += gStageA, refillB += gStageB;
 #pragma unroll
             for(uint32_t x = 0; x < XS; ++x)
@@ -727,7 +733,7 @@ namespace
                     if(q < 2u)
                         readAt(nxt, 0, x, q);
                     if(q == LOAD_Q)
-                        issueLoad(srcA, srcB, v, v, cur, x);
+                        issueLoad(full, srcA, srcB, v, v, cur, x);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -743,10 +749,19 @@ namespace
         refillA = uniform64(gA + (numStages > 2u ? 2u : numStages - 1u) * gStageA);
         refillB = uniform64(gB + (numStages > 2u ? 2u : numStages - 1u) * gStageB);
 
-        for(uint32_t kt = 0; kt < numStages; kt += 2)
+        // main part: every stage a pair refills (up to kt + 3) is a whole stage of K; then the pairs around the end of K
+        // (only a K-contiguous operand has a select to lose: with none, the main part is empty and compiles away)
+        const uint32_t wholeStages = (A_KCONTIG || B_KCONTIG) ? kBytes / STAGE_KB : 0u;
+        uint32_t       kt          = 0;
+        for(; kt + 3u < wholeStages; kt += 2)
         {
-            stageBody(kt, stage0, stage1);
-            stageBody(kt + 1, stage1, stage0);
+            stageBody(std::true_type{}, kt, stage0, stage1);
+            stageBody(std::true_type{}, kt + 1, stage1, stage0);
+        }
+        for(; kt < numStages; kt += 2)
+        {
+            stageBody(std::false_type{}, kt, stage0, stage1);
+            stageBody(std::false_type{}, kt + 1, stage1, stage0);
         }
 
         R355_STAMP(2);
@@ -1107,11 +1122,16 @@ namespace
         constexpr bool     SPREAD = WB == 8;
         constexpr uint32_t B_AHEAD = SPREAD ? 2u : 3u;
         uint64_t           refillA, refillB; // stage kt + 2 of A, stage kt + B_AHEAD of B (clamped)
-        auto stageBody = [&](uint32_t kt, uint32_t aCur, uint32_t aNxt, uint32_t bCur, uint32_t bNxt, uint32_t bFree) {
-            const uint32_t vB    = validOf(kt + B_AHEAD);
+        // `full` (compile-time tag): every stage this one requests is a whole stage inside K - the main part of the K
+        // loop, whose loads carry no tail select and whose refill pointers always advance
+        auto stageBody = [&](auto full, uint32_t kt, uint32_t aCur, uint32_t aNxt, uint32_t bCur, uint32_t bNxt, uint32_t bFree) {
+            constexpr bool FULL  = decltype(full)::value;
+            const uint32_t vB    = FULL ? STAGE_KB : validOf(kt + B_AHEAD);
             const i32x4    rsrcB = stageRsrc8(B_KCONTIG, refillB, vB, p.ldb);
-            if(kt + B_AHEAD + 1u < numStages)
+            if(FULL || kt + B_AHEAD + 1u < numStages)
                 refillB += gStageB;
+            auto offA = [&](uint32_t j, uint32_t valid) { return FULL ? gOffA[j] : tailOffset(A_KCONTIG, gOffA[j], kByteA, valid); };
+            auto offB = [&](uint32_t j, uint32_t valid) { return FULL ? gOffB[j] : tailOffset(B_KCONTIG, gOffB[j], kByteB, valid); };
 #pragma unroll
             for(uint32_t x = 0; x < XS; ++x)
 #pragma unroll
@@ -1122,15 +1142,14 @@ namespace
                         readAt(aCur, bCur, 1, x, q);
                     if constexpr(SPREAD)
                         if(q == LOAD_Q && (x & 1u))
-                            loadToLds(rsrcB, tailOffset(B_KCONTIG, gOffB[x >> 1], kByteB, vB), (x >> 1) * gStepB,
-                                      dmaDst + bFree + (x >> 1) * THREADS * CHUNK);
+                            loadToLds(rsrcB, offB(x >> 1, vB), (x >> 1) * gStepB, dmaDst + bFree + (x >> 1) * THREADS * CHUNK);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             waitVmcnt<WB>(); // this wave's part of stage kt + 1 has landed (the youngest WB loads are B of kt + 2)
             ldsBarrier();
-            const uint32_t vA    = validOf(kt + 2u);
+            const uint32_t vA    = FULL ? STAGE_KB : validOf(kt + 2u);
             const i32x4    rsrcA = stageRsrc8(A_KCONTIG, refillA, vA, p.lda);
-            if(kt + 3u < numStages)
+            if(FULL || kt + 3u < numStages)
                 refillA += gStageA;
 #pragma unroll
             for(uint32_t x = 0; x < XS; ++x)
@@ -1143,16 +1162,14 @@ namespace
                     if constexpr(SPREAD)
                     {
                         if(q == LOAD_Q && (x & 1u))
-                            loadToLds(rsrcA, tailOffset(A_KCONTIG, gOffA[x >> 1], kByteA, vA), (x >> 1) * gStepA,
-                                      dmaDst + aCur + (x >> 1) * THREADS * CHUNK);
+                            loadToLds(rsrcA, offA(x >> 1, vA), (x >> 1) * gStepA, dmaDst + aCur + (x >> 1) * THREADS * CHUNK);
                     }
                     else if(q == LOAD_Q)
                     {
                         if(x < WB)
-                            loadToLds(rsrcA, tailOffset(A_KCONTIG, gOffA[x], kByteA, vA), x * gStepA, dmaDst + aCur + x * THREADS * CHUNK);
+                            loadToLds(rsrcA, offA(x, vA), x * gStepA, dmaDst + aCur + x * THREADS * CHUNK);
                         else
-                            loadToLds(rsrcB, tailOffset(B_KCONTIG, gOffB[x - WB], kByteB, vB), (x - WB) * gStepB,
-                                      dmaDst + bCur + (x - WB) * THREADS * CHUNK);
+                            loadToLds(rsrcB, offB(x - WB, vB), (x - WB) * gStepB, dmaDst + bCur + (x - WB) * THREADS * CHUNK);
                     }
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -1187,32 +1204,49 @@ namespace
             readAt(A_AT[0], B_AT[0], 0, x, 1);
         }
 
-        // six stages per trip bring every buffer back to its role; single-exit loop, then the remainder
+        // six stages per trip bring every buffer back to its role; single-exit loops, then the remainder.  The main part
+        // runs the trips whose requests (up to stage kt + 5 + B_AHEAD) all are whole stages inside K without the tail
+        // handling; the trips around the end of K and the remainder carry it.
+        // (Only a K-contiguous operand has a select to lose: with none, the main part is empty and compiles away.)
+        const uint32_t     wholeStages = (A_KCONTIG || B_KCONTIG) ? kBytes / STAGE_KB : 0u;
+        constexpr uint32_t REACH       = 5u + B_AHEAD;
+        const uint32_t     mainTrips   = wholeStages > REACH ? (wholeStages - REACH + 5u) / 6u : 0u;
+        using Main = std::true_type;
+        using Tail = std::false_type;
         uint32_t kt = 0;
-        for(uint32_t trips = numStages / 6u; trips > 0; --trips, kt += 6u)
+        for(uint32_t trips = mainTrips; trips > 0; --trips, kt += 6u)
         {
-            stageBody(kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1], B_AT[2]);
-            stageBody(kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2], B_AT[0]);
-            stageBody(kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0], B_AT[1]);
-            stageBody(kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1], B_AT[2]);
-            stageBody(kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2], B_AT[0]);
-            stageBody(kt + 5u, A_AT[1], A_AT[0], B_AT[2], B_AT[0], B_AT[1]);
+            stageBody(Main{}, kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1], B_AT[2]);
+            stageBody(Main{}, kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2], B_AT[0]);
+            stageBody(Main{}, kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0], B_AT[1]);
+            stageBody(Main{}, kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1], B_AT[2]);
+            stageBody(Main{}, kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2], B_AT[0]);
+            stageBody(Main{}, kt + 5u, A_AT[1], A_AT[0], B_AT[2], B_AT[0], B_AT[1]);
+        }
+        for(uint32_t trips = numStages / 6u - mainTrips; trips > 0; --trips, kt += 6u)
+        {
+            stageBody(Tail{}, kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1], B_AT[2]);
+            stageBody(Tail{}, kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2], B_AT[0]);
+            stageBody(Tail{}, kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0], B_AT[1]);
+            stageBody(Tail{}, kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1], B_AT[2]);
+            stageBody(Tail{}, kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2], B_AT[0]);
+            stageBody(Tail{}, kt + 5u, A_AT[1], A_AT[0], B_AT[2], B_AT[0], B_AT[1]);
         }
         const uint32_t rem = numStages - kt;
         if(rem > 0u)
         {
-            stageBody(kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1], B_AT[2]);
+            stageBody(Tail{}, kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1], B_AT[2]);
             if(rem > 1u)
             {
-                stageBody(kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2], B_AT[0]);
+                stageBody(Tail{}, kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2], B_AT[0]);
                 if(rem > 2u)
                 {
-                    stageBody(kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0], B_AT[1]);
+                    stageBody(Tail{}, kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0], B_AT[1]);
                     if(rem > 3u)
                     {
-                        stageBody(kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1], B_AT[2]);
+                        stageBody(Tail{}, kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1], B_AT[2]);
                         if(rem > 4u)
-                            stageBody(kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2], B_AT[0]);
+                            stageBody(Tail{}, kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2], B_AT[0]);
                     }
                 }
             }
@@ -1380,11 +1414,13 @@ namespace
             }
         };
         // direct load j of an operand goes out in slot n when [n WB / NQ, (n + 1) WB / NQ) contains j
-        auto loadSlot = [&](bool kContig, const i32x4& rsrc, const uint32_t (&gOff)[WB], uint32_t step, uint32_t kByte,
+        // (`full`, a compile-time tag: the stage is a whole one inside K, no lane has a chunk beyond K)
+        auto loadSlot = [&](auto full, bool kContig, const i32x4& rsrc, const uint32_t (&gOff)[WB], uint32_t step, uint32_t kByte,
                             uint32_t valid, uint32_t at, uint32_t n) {
 #pragma unroll
             for(uint32_t j = n * WB / NQ; j < (n + 1u) * WB / NQ; ++j)
-                loadToLds(rsrc, tailOffset(kContig, gOff[j], kByte, valid), j * step, dmaDst + at + j * THREADS * CHUNK);
+                loadToLds(rsrc, decltype(full)::value ? gOff[j] : tailOffset(kContig, gOff[j], kByte, valid), j * step,
+                          dmaDst + at + j * THREADS * CHUNK);
         };
 
         f32x4 acc[WB][WB];
@@ -1397,8 +1433,11 @@ namespace
         i32x8 aLo[H], aHi[H], bX[H], bY[H]; // bX / bY alternate as the low / high half of B's blocks
 
         uint64_t refillA, refillB; // stage kt + 2 of A, stage kt + 3 of B (clamped)
-        auto stageBody = [&](uint32_t kt, uint32_t aCur, uint32_t aNxt, uint32_t bCur, uint32_t bNxt, i32x8 (&bLo)[H],
+        // `full` (compile-time tag): the stages this one requests (kt + 2 of A, kt + 3 of B) are whole stages inside K -
+        // the main part of the K loop, without tail selects and with refill pointers that always advance
+        auto stageBody = [&](auto full, uint32_t kt, uint32_t aCur, uint32_t aNxt, uint32_t bCur, uint32_t bNxt, i32x8 (&bLo)[H],
                              i32x8 (&bHi)[H]) {
+            constexpr bool FULL = decltype(full)::value;
             // Q1: A low x B low; B high arrives
 #pragma unroll
             for(uint32_t n = 0; n < NQ; ++n)
@@ -1417,11 +1456,11 @@ namespace
             }
             waitVmcnt<WB>(); // this wave's part of stage kt + 1 has landed (the youngest WB loads are B of kt + 2)
             ldsBarrier();
-            const uint32_t vA = validOf(kt + 2u), vB = validOf(kt + 3u);
+            const uint32_t vA = FULL ? STAGE_KB : validOf(kt + 2u), vB = FULL ? STAGE_KB : validOf(kt + 3u);
             const i32x4    rsrcA = stageRsrc8(A_KCONTIG, refillA, vA, p.lda), rsrcB = stageRsrc8(B_KCONTIG, refillB, vB, p.ldb);
-            if(kt + 3u < numStages)
+            if(FULL || kt + 3u < numStages)
                 refillA += gStageA;
-            if(kt + 4u < numStages)
+            if(FULL || kt + 4u < numStages)
                 refillB += gStageB;
             // Q3: A high x B high (row by row, in the order A arrived); next A low arrives; A refill
 #pragma unroll
@@ -1429,7 +1468,7 @@ namespace
             {
                 mfma16f8<E5M2>(acc[H + n / H][H + n % H], bHi[n % H], aHi[n / H]);
                 readSlotA(aLo, aNxt, 0, n);
-                loadSlot(A_KCONTIG, rsrcA, gOffA, gStepA, kByteA, vA, aCur, n);
+                loadSlot(full, A_KCONTIG, rsrcA, gOffA, gStepA, kByteA, vA, aCur, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
             // Q4: A high x B low; next B low arrives in the registers B high has left; B refill
@@ -1438,7 +1477,7 @@ namespace
             {
                 mfma16f8<E5M2>(acc[H + n % H][n / H], bLo[n / H], aHi[n % H]);
                 readSlotB(bHi, bNxt, 0, n);
-                loadSlot(B_KCONTIG, rsrcB, gOffB, gStepB, kByteB, vB, bCur, n);
+                loadSlot(full, B_KCONTIG, rsrcB, gOffB, gStepB, kByteB, vB, bCur, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
@@ -1461,31 +1500,47 @@ namespace
         }
 
         // six stages per trip bring every buffer and both B register groups back to their roles
+        // (main part: the trips whose requests, up to stage kt + 8, all are whole stages inside K)
+        // (kept to K-contiguous B: with the transposing reads of an N-contiguous B the second copy of the loop costs more
+        // than a hundred spilled registers, and without a K-contiguous operand there is no select to lose)
+        const uint32_t wholeStages = B_KCONTIG ? p.k / STAGE_KB : 0u;
+        const uint32_t mainTrips   = wholeStages > 8u ? (wholeStages - 8u + 5u) / 6u : 0u;
+        using Main = std::true_type;
+        using Tail = std::false_type;
         uint32_t kt = 0;
-        for(uint32_t trips = numStages / 6u; trips > 0; --trips, kt += 6u)
+        for(uint32_t trips = mainTrips; trips > 0; --trips, kt += 6u)
         {
-            stageBody(kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1], bX, bY);
-            stageBody(kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2], bY, bX);
-            stageBody(kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0], bX, bY);
-            stageBody(kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1], bY, bX);
-            stageBody(kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2], bX, bY);
-            stageBody(kt + 5u, A_AT[1], A_AT[0], B_AT[2], B_AT[0], bY, bX);
+            stageBody(Main{}, kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1], bX, bY);
+            stageBody(Main{}, kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2], bY, bX);
+            stageBody(Main{}, kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0], bX, bY);
+            stageBody(Main{}, kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1], bY, bX);
+            stageBody(Main{}, kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2], bX, bY);
+            stageBody(Main{}, kt + 5u, A_AT[1], A_AT[0], B_AT[2], B_AT[0], bY, bX);
+        }
+        for(uint32_t trips = numStages / 6u - mainTrips; trips > 0; --trips, kt += 6u)
+        {
+            stageBody(Tail{}, kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1], bX, bY);
+            stageBody(Tail{}, kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2], bY, bX);
+            stageBody(Tail{}, kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0], bX, bY);
+            stageBody(Tail{}, kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1], bY, bX);
+            stageBody(Tail{}, kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2], bX, bY);
+            stageBody(Tail{}, kt + 5u, A_AT[1], A_AT[0], B_AT[2], B_AT[0], bY, bX);
         }
         const uint32_t rem = numStages - kt;
         if(rem > 0u)
         {
-            stageBody(kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1], bX, bY);
+            stageBody(Tail{}, kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1], bX, bY);
             if(rem > 1u)
             {
-                stageBody(kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2], bY, bX);
+                stageBody(Tail{}, kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2], bY, bX);
                 if(rem > 2u)
                 {
-                    stageBody(kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0], bX, bY);
+                    stageBody(Tail{}, kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0], bX, bY);
                     if(rem > 3u)
                     {
-                        stageBody(kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1], bY, bX);
+                        stageBody(Tail{}, kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1], bY, bX);
                         if(rem > 4u)
-                            stageBody(kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2], bX, bY);
+                            stageBody(Tail{}, kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2], bX, bY);
                     }
                 }
             }
