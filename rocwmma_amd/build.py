@@ -1,6 +1,6 @@
 """Builds the gfx950 shared library (csrc/*.hip, csrc/api.cpp -> lib/librocwmma_amd.so) with hipcc.
 
-Usage: python -m rocwmma_amd.build [--force] [--timeline]
+Usage: python -m rocwmma_amd.build [--force] [--timeline] [--variant <name> -D<macro> ...]
 Objects are rebuilt when their source (or any header) is newer; translation units compile in parallel.
 """
 import os
@@ -72,20 +72,34 @@ def build(force=False, verbose=True):
 TIMELINE_LIB = os.path.join(LIBDIR, "librocwmma_amd_timeline.so")
 
 
-def build_timeline(verbose=True):
-    """The profiling twin of the library (lib/librocwmma_amd_timeline.so, read by rocwmma_amd.timeline): the macro-tile
-    kernels compiled with -DR355_TIMELINE, everything else from the ordinary objects.  Never loaded by the package itself."""
+def _build_twin(prefix, defines, sources, out, verbose):
+    """A second library beside the shipped one: the objects of `sources` (names of csrc files) recompiled with `defines`,
+    everything else from the ordinary objects.  Never loaded by the package itself."""
     build(verbose=False)
-    tiled = [s for s in SOURCES if s[0] == "gemm_tiled.hip"]
+    again = [s for s in SOURCES if s[0] in sources]
     with ThreadPoolExecutor(max_workers=min(4, os.cpu_count() or 1)) as ex:
-        tl = list(ex.map(lambda s: _compile((s[0], "tl_" + s[1], s[2] + ["-DR355_TIMELINE"]), False), tiled))
-    objs = [os.path.join(OBJDIR, stem + ".o") for src, stem, _ in SOURCES if src != "gemm_tiled.hip"] + [o for o, _ in tl]
-    r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", TIMELINE_LIB] + objs, capture_output=True, text=True)
+        twin = list(ex.map(lambda s: _compile((s[0], prefix + s[1], s[2] + defines), False), again))
+    objs = [os.path.join(OBJDIR, stem + ".o") for src, stem, _ in SOURCES if src not in sources] + [o for o, _ in twin]
+    os.makedirs(os.path.dirname(out), exist_ok=True)
+    r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + objs, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stderr)
     if verbose:
-        print("built", TIMELINE_LIB)
-    return TIMELINE_LIB
+        print("built", out)
+    return out
+
+
+def build_timeline(verbose=True):
+    """The profiling twin of the library (lib/librocwmma_amd_timeline.so, read by rocwmma_amd.timeline): the macro-tile
+    kernels compiled with -DR355_TIMELINE."""
+    return _build_twin("tl_", ["-DR355_TIMELINE"], ["gemm_tiled.hip"], TIMELINE_LIB, verbose)
+
+
+def build_variant(name, defines, verbose=True):
+    """A measurement build (lib/variant_<name>/librocwmma_amd.so): the kernel sources that know measurement macros
+    recompiled with `defines` (e.g. ["-DR355_ABLATE_MFMA"]).  `LD_LIBRARY_PATH=rocwmma_amd/lib/variant_<name>
+    rocwmma_amd/lib/host_bench ...` then runs host_bench on it."""
+    return _build_twin("var_%s_" % name, list(defines), ["sparse.hip"], os.path.join(LIBDIR, "variant_" + name, "librocwmma_amd.so"), verbose)
 
 
 def build_host_bench(verbose=True):
@@ -106,3 +120,5 @@ if __name__ == "__main__":
     build_host_bench()
     if "--timeline" in sys.argv:
         build_timeline()
+    if "--variant" in sys.argv:  # --variant <name> -D<macro> [-D<macro> ...]
+        build_variant(sys.argv[sys.argv.index("--variant") + 1], [a for a in sys.argv if a.startswith("-D")])

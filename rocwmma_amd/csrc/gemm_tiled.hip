@@ -41,6 +41,7 @@
 // columns of a row of D; a col-major D is computed as the row-major D^T = B^T A^T.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
 #include <type_traits>
 
 #include "common.hpp"
@@ -115,6 +116,10 @@ namespace r355
         uint64_t splitStrideD;
         // host side only: 16-bit operands on the 256 x 256 tile take the five-buffer K loop instead of the two-buffer one
         uint32_t deepPipeline;
+        // experiment (R355_STAGGER_TICKS in the environment, 10 ns units; 0 = off): the first staggerBlocks workgroups - the
+        // first round over the CUs - start 0, 1, 2 or 3 x stagger ticks late, by groups of CUs within each XCD, so that
+        // the rounds' epilogues do not all store at once
+        uint32_t stagger, staggerBlocks;
     };
     // sum of `splits` partial results (accumulator type: f32, i32 or f64) + the alpha / beta epilogue into the output type
     int splitKReduce(const r355_gemm_args& g, const GemmTileParams& p, uint32_t splits, hipStream_t stream);
@@ -193,6 +198,17 @@ namespace
     };
 
     using Params = r355::GemmTileParams;
+
+    __device__ __forceinline__ void staggeredStart(const Params& p)
+    {
+        if(p.stagger != 0u && blockIdx.x < p.staggerBlocks)
+        {
+            const uint32_t group = (blockIdx.x >> 3) & 3u; // workgroup ids go round the 8 XCDs: four groups of CUs in each
+            const uint64_t until = __builtin_amdgcn_s_memrealtime() + (uint64_t)group * p.stagger; // 100 MHz counter
+            while(__builtin_amdgcn_s_memrealtime() < until)
+                __builtin_amdgcn_s_sleep(8);
+        }
+    }
 
     // The share of a split-K workgroup row: operands advanced to its first K stage, k cut to its stages, D pointed at its
     // partial result.  kStage: bytes between K stages of A / B (128 for a K-contiguous operand, 128 rows of ld otherwise).
@@ -275,22 +291,24 @@ namespace
     // everything before it: beta != 0 cost 12 % (f16) to 25 % (e4m3) of an 8192^3 launch instead of the 4 - 13 % that
     // reading C takes.)  C may alias D: every element's C is read before its D is written, and passes, waves and
     // workgroups own disjoint rows and columns.
-    template <typename StageT, bool WITH_C, typename AccV, typename OutT, uint32_t WB>
-    __device__ __forceinline__ void storeTileStaged(AccV (&acc)[WB][WB], const Params& p, uint32_t m0, uint32_t n0, uint32_t lane,
+    // The wave tile is WBM x WBN blocks (rows x columns of 16 x 16) and `scratch` SCRATCH bytes of LDS owned by this wave.
+    template <typename StageT, bool WITH_C, typename AccV, typename OutT, uint32_t WBM, uint32_t WBN, uint32_t SCRATCH>
+    __device__ __forceinline__ void storeTileStaged(AccV (&acc)[WBM][WBN], const Params& p, uint32_t m0, uint32_t n0, uint32_t lane,
                                                     char* scratch)
     {
         using AccE = std::remove_reference_t<decltype(acc[0][0][0])>;
         const AccE     alpha = static_cast<AccE>(p.alpha), beta = static_cast<AccE>(p.beta);
         const uint32_t r16 = lane & 15u, g = lane >> 4;
         constexpr uint32_t SS = sizeof(StageT), OS = sizeof(OutT);
-        constexpr uint32_t ROW_BYTES  = 16u * WB * SS;
+        constexpr uint32_t ROW_BYTES  = 16u * WBN * SS;
         constexpr uint32_t ROW_CHUNKS = ROW_BYTES / CHUNK; // 8, 16 or 32
         constexpr uint32_t SWZ        = ROW_CHUNKS < 16u ? ROW_CHUNKS - 1u : 15u;
         constexpr uint32_t EPC        = CHUNK / SS; // elements of a staged 16-byte chunk
         constexpr uint32_t OUT_WORDS  = EPC * OS / 4u; // 32-bit words of C and of D per lane and chunk: 4, 2 or 1
         // rows per pass: what the scratch holds, halved where a pass's part of C would take 128 registers
-        constexpr uint32_t FIT        = WB * 4096u / ROW_BYTES / ((WITH_C && OUT_WORDS == 4u && WB == 8u) ? 2u : 1u);
-        constexpr uint32_t ROWS_PASS  = FIT < 16u * WB ? FIT : 16u * WB;
+        constexpr uint32_t FIT_ALL    = SCRATCH / ROW_BYTES;
+        constexpr uint32_t FIT        = FIT_ALL / ((WITH_C && FIT_ALL * ROW_CHUNKS / 64u * OUT_WORDS >= 128u) ? 2u : 1u);
+        constexpr uint32_t ROWS_PASS  = FIT < 16u * WBM ? FIT : 16u * WBM;
         constexpr uint32_t BLOCKS_I   = ROWS_PASS / 16u; // row blocks per pass
         constexpr uint32_t ITERS      = ROWS_PASS * ROW_CHUNKS / 64u; // chunks per lane and pass
         constexpr uint32_t BATCH      = ITERS < 8u ? ITERS : 8u;
@@ -299,7 +317,7 @@ namespace
 
         const uint32_t lddB = p.ldd * OS, ldcB = p.ldc * OS;
         const uint32_t um0 = __builtin_amdgcn_readfirstlane(m0), un0 = __builtin_amdgcn_readfirstlane(n0); // (wave-uniform)
-        const uint32_t colsValid = un0 < p.n ? (p.n - un0 < 16u * WB ? p.n - un0 : 16u * WB) : 0u;
+        const uint32_t colsValid = un0 < p.n ? (p.n - un0 < 16u * WBN ? p.n - un0 : 16u * WBN) : 0u;
         auto tileBuffer = [&](const char* base, uint32_t ldB, uint32_t rowFirst) {
             // from the wave tile's first column in row rowFirst to the end of the tile's last valid row (nothing if there is none)
             const uint32_t rowsLeft  = rowFirst < p.m ? p.m - rowFirst : 0u;
@@ -348,7 +366,7 @@ namespace
         const uint32_t dLane = colOk ? rowLane * lddB + cLane * (EPC * OS) : 0x80000000u;
 
 #pragma unroll
-        for(uint32_t pass = 0; pass < WB / BLOCKS_I; ++pass)
+        for(uint32_t pass = 0; pass < WBM / BLOCKS_I; ++pass)
         {
             const auto dBuf = tileBuffer(p.d, lddB, um0 + pass * ROWS_PASS);
             // C of this pass, requested before anything else (m and n are multiples of 16, so a chunk of up to 16 elements
@@ -367,7 +385,7 @@ namespace
             {
                 const uint32_t i = pass * BLOCKS_I + ii, row = 16u * ii + r16;
 #pragma unroll
-                for(uint32_t j = 0; j < WB; ++j)
+                for(uint32_t j = 0; j < WBN; ++j)
                 {
                     if constexpr(sizeof(AccE) == 8)
                     {
@@ -446,15 +464,16 @@ namespace
         }
     }
 
-    template <typename AccV, typename OutT, uint32_t WB>
-    __device__ __forceinline__ void storeTile16(AccV (&acc)[WB][WB], const Params& p, uint32_t m0, uint32_t n0, uint32_t lane,
+    // (`scratch`: WB x 4 KiB of the wave's own; the eight-wave kernel has 16 KiB for its 8 x 4 blocks)
+    template <typename AccV, typename OutT, uint32_t WBM, uint32_t WBN, uint32_t SCRATCH = WBM * 4096u>
+    __device__ __forceinline__ void storeTile16(AccV (&acc)[WBM][WBN], const Params& p, uint32_t m0, uint32_t n0, uint32_t lane,
                                                 char* scratch)
     {
         using AccE = std::remove_reference_t<decltype(acc[0][0][0])>;
         if(static_cast<AccE>(p.beta) == static_cast<AccE>(0)) // (as the accumulator type sees it: an int8 problem's beta = 0.5 is 0)
-            storeTileStaged<OutT, false, AccV, OutT, WB>(acc, p, m0, n0, lane, scratch);
+            storeTileStaged<OutT, false, AccV, OutT, WBM, WBN, SCRATCH>(acc, p, m0, n0, lane, scratch);
         else
-            storeTileStaged<AccE, true, AccV, OutT, WB>(acc, p, m0, n0, lane, scratch);
+            storeTileStaged<AccE, true, AccV, OutT, WBM, WBN, SCRATCH>(acc, p, m0, n0, lane, scratch);
     }
 
     //
@@ -489,6 +508,7 @@ namespace
             return;
         if(p.tileQuad && (tm * TILE >= p.m || tn * TILE >= p.n))
             return; // a quarter of a partial edge tile that lies outside the matrix
+        staggeredStart(p);
 
         const uint32_t tid  = threadIdx.x;
         const uint32_t lane = tid & 63u;
@@ -770,7 +790,7 @@ namespace
         __syncthreads();
         // the last matrix instructions are still in the pipeline and the compiler does not know it
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-        storeTile16<f32x4, OutT, WB>(acc, p, tm * TILE + wm * WT, tn * TILE + wn * WT, lane,
+        storeTile16<f32x4, OutT, WB, WB>(acc, p, tm * TILE + wm * WT, tn * TILE + wn * WT, lane,
                                      ((wave < 2u) ? stage0 : stage1) + (wave & 1u) * (WB * 4096u));
         R355_STAMP_END();
     }
@@ -1030,6 +1050,7 @@ namespace
             return;
         if(p.tileQuad && (tm * TILE >= p.m || tn * TILE >= p.n))
             return; // a quarter of a partial edge tile that lies outside the matrix
+        staggeredStart(p);
 
         const uint32_t tid  = threadIdx.x;
         const uint32_t lane = tid & 63u;
@@ -1258,8 +1279,271 @@ namespace
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
         waitVmcnt<0>();
         ldsBarrier();
-        storeTile16<AccV, OutT, WB>(acc, p, tm * TILE + wm * WT, tn * TILE + wn * WT, lane, lds + wave * (WB * 4096u));
+        storeTile16<AccV, OutT, WB, WB>(acc, p, tm * TILE + wm * WT, tn * TILE + wn * WT, lane, lds + wave * (WB * 4096u));
         R355_STAMP_END();
+    }
+
+    // ------------------------------------------------------------------------------------------
+    // int8, the 256 x 256 macro tile on EIGHT waves: two waves per SIMD, 2 x 4 waves with wave tiles of 128 x 64 (8 x 4
+    // accumulator blocks = 128 registers, so two waves fit a SIMD's register file).  With one wave per SIMD every LDS read
+    // or direct load that its unit cannot take at once holds up the matrix instruction behind it (a wave issues in
+    // order); here the SIMD's other wave can issue meanwhile.  The price: every wave reads 12 operand blocks per 32 matrix
+    // instructions instead of 16 per 64 (1.5 x the LDS read volume).  Same five LDS buffers, same K-step structure and
+    // the same storage swizzles as gemmTiled5; 512 threads move a 32 KiB operand tile in 4 loads each.
+    constexpr uint32_t THREADS_WIDE = 512;
+
+    template <bool KCONTIG>
+    __device__ __forceinline__ void laneOffsetsWide(uint32_t tid, uint32_t ld, uint32_t valid, uint32_t (&off)[4], uint32_t& step,
+                                                    uint64_t& stage, uint32_t& kByte)
+    {
+        kByte = 0u;
+        if constexpr(KCONTIG)
+        {
+            const uint32_t r = tid >> 3, slot = tid & 7u; // chunk j * 512 + tid: row 64 j + r (the swizzle does not change with j)
+            kByte            = (slot ^ swzK8(r)) * CHUNK;
+#pragma unroll
+            for(uint32_t j = 0; j < 4; ++j)
+            {
+                const uint32_t row = r + 64u * j < valid ? r + 64u * j : valid - 1u;
+                off[j]             = row * ld + kByte;
+            }
+            step = 0u, stage = STAGE_KB;
+        }
+        else
+        {
+            const uint32_t r = tid >> 4, slot = tid & 15u; // k-row 32 j + r: bits 0 .. 2 and 4 of it, which the swizzle uses, are r's
+#pragma unroll
+            for(uint32_t j = 0; j < 4; ++j)
+            {
+                const uint32_t c = slot ^ swzMN8<8>(32u * j + r);
+                off[j]           = r * ld + (c * CHUNK < valid ? c : 0u) * CHUNK;
+            }
+            step = 32u * ld, stage = (uint64_t)STAGE_KB * ld;
+        }
+    }
+
+    template <typename OutT, bool A_KCONTIG, bool B_KCONTIG>
+    __device__ __forceinline__ void gemmTiledI8Wide(const Params& p)
+    {
+        constexpr uint32_t WBM = 8, WBN = 4, TILE = 256, OPER = TILE * STAGE_KB; // wave tile 128 x 64; 32 KiB per operand and stage
+        constexpr uint32_t NL = OPER / CHUNK / THREADS_WIDE; // 4 direct loads per operand, stage and thread
+        constexpr uint32_t NM = WBM * WBN; // 32 matrix instructions per K step
+        constexpr uint32_t A_AT[2] = {0u, OPER};
+        constexpr uint32_t B_AT[3] = {2u * OPER, 3u * OPER, 4u * OPER};
+        __shared__ __attribute__((aligned(1024))) char lds[5u * OPER];
+
+        uint32_t tm, tn;
+        if(!r355::tileCoordRange(blockIdx.x, p.tilesM, p.tilesN, p.tileFirst, p.tileCount, false, tm, tn))
+            return;
+        staggeredStart(p);
+        const uint32_t tid  = threadIdx.x;
+        const uint32_t lane = tid & 63u;
+        const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const uint32_t wm = wave >> 2, wn = wave & 3u;
+        const uint32_t t = lane & 15u, g = lane >> 4;
+        const uint32_t ldsBase
+            = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds));
+
+        uint32_t       gOffA[NL], gOffB[NL], gStepA, gStepB, kByteA, kByteB;
+        uint64_t       gStageA, gStageB;
+        const uint32_t validM = p.m - tm * TILE < TILE ? p.m - tm * TILE : TILE;
+        const uint32_t validN = p.n - tn * TILE < TILE ? p.n - tn * TILE : TILE;
+        laneOffsetsWide<A_KCONTIG>(tid, p.lda, validM, gOffA, gStepA, gStageA, kByteA);
+        laneOffsetsWide<B_KCONTIG>(tid, p.ldb, validN, gOffB, gStepB, gStageB, kByteB);
+        const uint32_t numStages = (p.k + STAGE_KB - 1u) / STAGE_KB;
+        const uint32_t lastBytes = p.k - (numStages - 1u) * STAGE_KB;
+        auto validOf = [&](uint32_t stage) { return stage + 1u < numStages ? STAGE_KB : (stage + 1u == numStages ? lastBytes : 0u); };
+        const uint32_t dmaDst = ldsBase + wave * 64u * CHUNK; // + buffer + j * 8 KiB
+        const uint64_t gA = r355::uniformAddress(p.a + (A_KCONTIG ? (uint64_t)tm * TILE * p.lda : (uint64_t)tm * TILE));
+        const uint64_t gB = r355::uniformAddress(p.b + (B_KCONTIG ? (uint64_t)tn * TILE * p.ldb : (uint64_t)tn * TILE));
+        auto stageAddr = [&](uint64_t panel, uint64_t perStage, uint32_t stage) { // clamped to the last stage
+            return panel + (uint64_t)(stage < numStages ? stage : numStages - 1u) * perStage;
+        };
+        auto issueHalf = [&](bool kContig, uint64_t addr, const uint32_t (&gOff)[NL], uint32_t step, uint32_t kByte, uint32_t ld,
+                             uint32_t valid, uint32_t at) {
+            const i32x4 rsrc = stageRsrc8(kContig, addr, valid, ld);
+#pragma unroll
+            for(uint32_t j = 0; j < NL; ++j)
+                loadToLds(rsrc, tailOffset(kContig, gOff[j], kByte, valid), j * step, dmaDst + at + j * THREADS_WIDE * CHUNK);
+        };
+
+        // LDS -> registers: K-contiguous rd[q] is 64-byte K step q of block 0 (block i 16 rows further); M/N-contiguous rd[i]
+        // is block i (16-byte chunk first + i of the 256-byte k-rows), the first 8 k-rows of the lane's 16 of K step 0
+        uint32_t rdA[8], rdB[8];
+        auto readOffsets = [&](bool kContig, uint32_t firstBlock, uint32_t blocks, uint32_t (&rd)[8]) {
+#pragma unroll
+            for(uint32_t i = 0; i < 8; ++i)
+                rd[i] = 0u;
+            if(kContig)
+            {
+                const uint32_t r = firstBlock * 16u + t;
+                rd[0]            = r * STAGE_KB + ((g ^ swzK8(r)) * CHUNK);
+                rd[1]            = r * STAGE_KB + (((4u + g) ^ swzK8(r)) * CHUNK);
+            }
+            else
+            {
+                const uint32_t kr = 16u * g + (t >> 1);
+#pragma unroll
+                for(uint32_t i = 0; i < 8; ++i)
+                    if(i < blocks)
+                        rd[i] = kr * 256u + (((firstBlock + i) ^ swzMN8<8>(kr)) * CHUNK) + (t & 1u) * 8u;
+            }
+        };
+        readOffsets(A_KCONTIG, wm * WBM, WBM, rdA);
+        readOffsets(B_KCONTIG, wn * WBN, WBN, rdB);
+
+        i32x4v acc[WBM][WBN];
+#pragma unroll
+        for(uint32_t i = 0; i < WBM; ++i)
+#pragma unroll
+            for(uint32_t j = 0; j < WBN; ++j)
+                acc[i][j] = i32x4v{0, 0, 0, 0};
+
+        i32x4 fa[2][WBM], fb[2][WBN];
+        // Matrix instruction n (0 .. 31) of a K step: the 4 x 4 corner in L-shaped shells, then block rows 4 .. 7; the
+        // operand blocks are read in the order they are first needed: A0 B0 A1 B1 A2 B2 A3 B3 A4 A5 A6 A7.
+        auto mfmaAt = [&](uint32_t s, uint32_t n) {
+            uint32_t i, j;
+            if(n < WBN * WBN)
+            {
+                uint32_t d = 0;
+                while((d + 1u) * (d + 1u) <= n)
+                    ++d;
+                const uint32_t r = n - d * d;
+                i = r <= d ? d : r - d - 1u, j = r <= d ? r : d;
+            }
+            else
+                i = n / WBN, j = n % WBN;
+            mfma16i8(acc[i][j], fb[s][j], fa[s][i]);
+        };
+        // read piece r of a K step: the blocks in the order above, one piece each when K-contiguous, two (the halves
+        // of a transposing read pair) otherwise; pieces are dealt out evenly over the 32 slots of the previous K step
+        constexpr uint32_t PA = A_KCONTIG ? 1u : 2u, PB = B_KCONTIG ? 1u : 2u;
+        constexpr uint32_t NR = WBM * PA + WBN * PB;
+        auto readPiece = [&](uint32_t aAt, uint32_t bAt, uint32_t s, uint32_t r) {
+            // pieces of blocks 0 .. 3 alternate A, B; then A's blocks 4 .. 7
+            uint32_t left = r;
+#pragma unroll
+            for(uint32_t x = 0; x < WBM + WBN; ++x)
+            {
+                const bool     isB = x < 2u * WBN && (x & 1u);
+                const uint32_t blk = x < 2u * WBN ? x >> 1 : x - WBN, parts = isB ? PB : PA;
+                if(left < parts)
+                {
+                    if(isB)
+                        readBlock8<B_KCONTIG, 8>(lds + bAt, rdB, blk, s, left, fb[s][blk], 0u);
+                    else
+                        readBlock8<A_KCONTIG, 8>(lds + aAt, rdA, blk, s, left, fa[s][blk], 0u);
+                    return;
+                }
+                left -= parts;
+            }
+        };
+        auto readSlot = [&](uint32_t aAt, uint32_t bAt, uint32_t s, uint32_t n) {
+#pragma unroll
+            for(uint32_t r = (n * NR + NM - 1u) / NM; r < ((n + 1u) * NR + NM - 1u) / NM; ++r)
+                readPiece(aAt, bAt, s, r);
+        };
+
+        uint64_t refillA, refillB; // stage kt + 2 of A and of B (clamped)
+        auto stageBody = [&](auto full, uint32_t kt, uint32_t aCur, uint32_t aNxt, uint32_t bCur, uint32_t bNxt, uint32_t bFree) {
+            constexpr bool FULL  = decltype(full)::value;
+            const uint32_t vB    = FULL ? STAGE_KB : validOf(kt + 2u);
+            const i32x4    rsrcB = stageRsrc8(B_KCONTIG, refillB, vB, p.ldb);
+            if(FULL || kt + 3u < numStages)
+                refillB += gStageB;
+#pragma unroll
+            for(uint32_t n = 0; n < NM; ++n)
+            {
+                mfmaAt(0, n);
+                readSlot(aCur, bCur, 1, n);
+                if(n % 8u == 3u) // B of stage kt + 2 into the third B buffer
+                    loadToLds(rsrcB, FULL ? gOffB[n / 8u] : tailOffset(B_KCONTIG, gOffB[n / 8u], kByteB, vB), (n / 8u) * gStepB,
+                              dmaDst + bFree + (n / 8u) * THREADS_WIDE * CHUNK);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            waitVmcnt<NL>(); // this wave's part of stage kt + 1 has landed (the youngest NL loads are B of kt + 2)
+            ldsBarrier();
+            const uint32_t vA    = FULL ? STAGE_KB : validOf(kt + 2u);
+            const i32x4    rsrcA = stageRsrc8(A_KCONTIG, refillA, vA, p.lda);
+            if(FULL || kt + 3u < numStages)
+                refillA += gStageA;
+#pragma unroll
+            for(uint32_t n = 0; n < NM; ++n)
+            {
+                mfmaAt(1, n);
+                readSlot(aNxt, bNxt, 0, n);
+                if(n % 8u == 3u) // A of stage kt + 2 into the A buffer this stage's barrier has freed
+                    loadToLds(rsrcA, FULL ? gOffA[n / 8u] : tailOffset(A_KCONTIG, gOffA[n / 8u], kByteA, vA), (n / 8u) * gStepA,
+                              dmaDst + aCur + (n / 8u) * THREADS_WIDE * CHUNK);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+
+        issueHalf(B_KCONTIG, stageAddr(gB, gStageB, 0u), gOffB, gStepB, kByteB, p.ldb, validOf(0u), B_AT[0]);
+        issueHalf(A_KCONTIG, stageAddr(gA, gStageA, 0u), gOffA, gStepA, kByteA, p.lda, validOf(0u), A_AT[0]);
+        issueHalf(B_KCONTIG, stageAddr(gB, gStageB, 1u), gOffB, gStepB, kByteB, p.ldb, validOf(1u), B_AT[1]);
+        issueHalf(A_KCONTIG, stageAddr(gA, gStageA, 1u), gOffA, gStepA, kByteA, p.lda, validOf(1u), A_AT[1]);
+        waitVmcnt<2u * NL>();
+        refillA = stageAddr(gA, gStageA, 2u), refillB = stageAddr(gB, gStageB, 2u);
+        ldsBarrier();
+#pragma unroll
+        for(uint32_t r = 0; r < NR; ++r)
+            readPiece(A_AT[0], B_AT[0], 0, r);
+
+        const uint32_t wholeStages = (A_KCONTIG || B_KCONTIG) ? p.k / STAGE_KB : 0u;
+        const uint32_t mainTrips   = wholeStages > 7u ? (wholeStages - 7u + 5u) / 6u : 0u;
+        using Main = std::true_type;
+        using Tail = std::false_type;
+        uint32_t kt = 0;
+        for(uint32_t trips = mainTrips; trips > 0; --trips, kt += 6u)
+        {
+            stageBody(Main{}, kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1], B_AT[2]);
+            stageBody(Main{}, kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2], B_AT[0]);
+            stageBody(Main{}, kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0], B_AT[1]);
+            stageBody(Main{}, kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1], B_AT[2]);
+            stageBody(Main{}, kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2], B_AT[0]);
+            stageBody(Main{}, kt + 5u, A_AT[1], A_AT[0], B_AT[2], B_AT[0], B_AT[1]);
+        }
+        for(uint32_t trips = numStages / 6u - mainTrips; trips > 0; --trips, kt += 6u)
+        {
+            stageBody(Tail{}, kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1], B_AT[2]);
+            stageBody(Tail{}, kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2], B_AT[0]);
+            stageBody(Tail{}, kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0], B_AT[1]);
+            stageBody(Tail{}, kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1], B_AT[2]);
+            stageBody(Tail{}, kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2], B_AT[0]);
+            stageBody(Tail{}, kt + 5u, A_AT[1], A_AT[0], B_AT[2], B_AT[0], B_AT[1]);
+        }
+        const uint32_t rem = numStages - kt;
+        if(rem > 0u)
+        {
+            stageBody(Tail{}, kt, A_AT[0], A_AT[1], B_AT[0], B_AT[1], B_AT[2]);
+            if(rem > 1u)
+            {
+                stageBody(Tail{}, kt + 1u, A_AT[1], A_AT[0], B_AT[1], B_AT[2], B_AT[0]);
+                if(rem > 2u)
+                {
+                    stageBody(Tail{}, kt + 2u, A_AT[0], A_AT[1], B_AT[2], B_AT[0], B_AT[1]);
+                    if(rem > 3u)
+                    {
+                        stageBody(Tail{}, kt + 3u, A_AT[1], A_AT[0], B_AT[0], B_AT[1], B_AT[2]);
+                        if(rem > 4u)
+                            stageBody(Tail{}, kt + 4u, A_AT[0], A_AT[1], B_AT[1], B_AT[2], B_AT[0]);
+                    }
+                }
+            }
+        }
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+        waitVmcnt<0>();
+        ldsBarrier();
+        storeTile16<i32x4v, OutT, WBM, WBN, 16384u>(acc, p, tm * TILE + wm * (16u * WBM), tn * TILE + wn * (16u * WBN), lane,
+                                                    lds + wave * 16384u);
+    }
+
+    template <typename OutT, bool A_KCONTIG, bool B_KCONTIG>
+    __global__ void __launch_bounds__(THREADS_WIDE) __attribute__((amdgpu_waves_per_eu(2, 2))) gemmTiledKernelI8Wide(Params p)
+    {
+        gemmTiledI8Wide<OutT, A_KCONTIG, B_KCONTIG>(p);
     }
 
     template <typename OutT, bool A_KCONTIG, bool B_KCONTIG>
@@ -1349,6 +1633,7 @@ namespace
             return;
         if(p.tileQuad && (tm * TILE >= p.m || tn * TILE >= p.n))
             return; // a quarter of a partial edge tile that lies outside the matrix
+        staggeredStart(p);
 
         const uint32_t tid  = threadIdx.x;
         const uint32_t lane = tid & 63u;
@@ -1550,7 +1835,7 @@ namespace
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); // the last matrix instructions are still in the pipeline
         waitVmcnt<0>();
         ldsBarrier();
-        storeTile16<f32x4, float, WB>(acc, p, tm * TILE + wm * WT, tn * TILE + wn * WT, lane, lds + wave * (WB * 4096u));
+        storeTile16<f32x4, float, WB, WB>(acc, p, tm * TILE + wm * WT, tn * TILE + wn * WT, lane, lds + wave * (WB * 4096u));
         R355_STAMP_END();
     }
 
@@ -1565,6 +1850,16 @@ namespace
         gemmTiledF8<E5M2, A_KCONTIG, B_KCONTIG, 4>(p);
     }
 
+    // experiment switch: R355_I8_WIDE=1 in the environment runs the int8 256 x 256 tile on the eight-wave kernel
+    inline bool wideI8()
+    {
+        static const bool on = [] {
+            const char* v = getenv("R355_I8_WIDE");
+            return v && v[0] == '1';
+        }();
+        return on;
+    }
+
     template <Elem E, typename OutT>
     int launchLayouts(bool aK, bool bK, uint32_t tile, const Params& p, hipStream_t stream)
     {
@@ -1577,6 +1872,8 @@ namespace
             {
                 if(tile == 128u)
                     hipLaunchKernelGGL((gemmTiledKernelI8Small<OutT, AK, BK>), grid, block, 0, stream, p);
+                else if(wideI8())
+                    hipLaunchKernelGGL((gemmTiledKernelI8Wide<OutT, AK, BK>), grid, dim3(THREADS_WIDE), 0, stream, p);
                 else
                     hipLaunchKernelGGL((gemmTiledKernelI8<OutT, AK, BK>), grid, block, 0, stream, p);
             }
@@ -1934,6 +2231,11 @@ namespace r355
         };
         p.splitStages = 0u, p.splitStrideD = 0u;
         p.deepPipeline = deepPipeline(g) ? 1u : 0u;
+        static const uint32_t staggerTicks = [] {
+            const char* v = getenv("R355_STAGGER_TICKS");
+            return v ? static_cast<uint32_t>(atoi(v)) : 0u;
+        }();
+        p.stagger = staggerTicks, p.staggerBlocks = computeUnits();
         const uint32_t splits = tile == 128u ? splitCount(g) : 1u;
         if(splits > 1u)
         {

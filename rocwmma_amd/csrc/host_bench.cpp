@@ -252,10 +252,11 @@ namespace
     // flight.  PATTERN 0: K-contiguous operands with `pitch` bytes per row (a load touches 8 rows x 128 bytes);
     // 1: K-blocked operands (a tile's share of a stage is 32 KiB of consecutive bytes); 2: pattern 0 with every workgroup on
     // tile (0, 0) (no L2 misses).
-    template <int DEPTH, int PATTERN>
+    // SOLO: 96 KiB of LDS per workgroup, so that a CU holds one workgroup and DEPTH x 64 KiB is all it has in flight.
+    template <int DEPTH, int PATTERN, bool SOLO = false>
     __global__ void __launch_bounds__(256) fillLoop(const char* a, const char* b, uint32_t pitch, uint32_t stages, uint32_t tiles)
     {
-        __shared__ __attribute__((aligned(1024))) char lds[65536];
+        __shared__ __attribute__((aligned(1024))) char lds[SOLO ? 98304 : 65536];
         uint32_t tm = 0, tn = 0;
         if(!r355::tileCoordRange(blockIdx.x, tiles, tiles, 0u, tiles * tiles, false, tm, tn))
             return;
@@ -788,10 +789,10 @@ int main(int argc, char** argv)
         hipEvent_t e0, e1;
         HIP_OK(hipEventCreate(&e0));
         HIP_OK(hipEventCreate(&e1));
-        const char* names[4] = {"K-contiguous rows, pitch 8192", "K-contiguous rows, pitch 8320", "K-blocked (32 KiB runs)",
-                                "every workgroup on tile (0, 0)"};
+        const char* names[5] = {"K-contiguous rows, pitch 8192", "K-contiguous rows, pitch 8320", "K-blocked (32 KiB runs)",
+                                "every workgroup on tile (0, 0)", "K-contiguous rows, pitch 8192, one workgroup per CU"};
         printf("[");
-        for(int pat = 0; pat < 4; ++pat)
+        for(int pat = 0; pat < 5; ++pat)
             for(int depth = 1; depth <= 3; ++depth)
             {
                 const uint32_t pitch = pat == 1 ? 8320u : 8192u;
@@ -800,7 +801,16 @@ int main(int argc, char** argv)
                     const char *a = static_cast<const char*>(pa), *b = static_cast<const char*>(pb);
 #define R355_FILL(D, P) hipLaunchKernelGGL((fillLoop<D, P>), g, blk, 0, 0, a, b, pitch, stages, tiles)
                     const int p = pat == 0 || pat == 1 ? 0 : pat - 1;
-                    if(depth == 1) { if(p == 0) R355_FILL(1, 0); else if(p == 1) R355_FILL(1, 1); else R355_FILL(1, 2); }
+                    if(pat == 4)
+                    {
+                        if(depth == 1)
+                            hipLaunchKernelGGL((fillLoop<1, 0, true>), g, blk, 0, 0, a, b, pitch, stages, tiles);
+                        else if(depth == 2)
+                            hipLaunchKernelGGL((fillLoop<2, 0, true>), g, blk, 0, 0, a, b, pitch, stages, tiles);
+                        else
+                            hipLaunchKernelGGL((fillLoop<3, 0, true>), g, blk, 0, 0, a, b, pitch, stages, tiles);
+                    }
+                    else if(depth == 1) { if(p == 0) R355_FILL(1, 0); else if(p == 1) R355_FILL(1, 1); else R355_FILL(1, 2); }
                     else if(depth == 2) { if(p == 0) R355_FILL(2, 0); else if(p == 1) R355_FILL(2, 1); else R355_FILL(2, 2); }
                     else { if(p == 0) R355_FILL(3, 0); else if(p == 1) R355_FILL(3, 1); else R355_FILL(3, 2); }
 #undef R355_FILL

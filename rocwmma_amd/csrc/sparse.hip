@@ -27,6 +27,16 @@
 //   sparseBlockPerWave   one 16 x 16 or 32 x 32 block of D per wave through the sparse fragment API
 //                        (rocwmma_sparse.hpp) straight from global memory; fallback for shapes that do not fill a
 //                        macro tile.
+//
+// Measurement builds of the macro-tile kernel (`python -m rocwmma_amd.build --variant <name> -D<macro> ...` puts a
+// second library under lib/variant_<name>/; never the shipped one - the first three compute wrong results on purpose):
+//   R355_ABLATE_MFMA    no matrix instructions (data movement alone)
+//   R355_ABLATE_READS   no LDS reads of the operands
+//   R355_ABLATE_LOADS   no direct loads after the prologue's
+//   R355_SPARSE_A_DIRECT  every wave takes the kept values and indices of its own 128 rows straight from global memory
+//                       into registers, one stage ahead, and only B goes through LDS (results correct).  Measured
+//                       12 - 26 % slower: the two waves that share a block row both fetch it, so 72 instead of 52 KiB
+//                       per stage pass the CU's vector-memory path, which is what bounds this kernel.
 #include <hip/hip_runtime.h>
 
 #include <cstring>
@@ -176,6 +186,10 @@ namespace
     {
         // the accumulator is the instruction's destination and addend at once: updated in place, in an AGPR
         // (2-byte elements: the index bits are the low half of the register, which is what ABID 0 names)
+#ifdef R355_ABLATE_MFMA
+        asm volatile("" : "+a"(acc) : "v"(a), "v"(b), "v"(idx));
+        return;
+#endif
         if constexpr(E == SpElem::E4M3)
             asm volatile("v_smfmac_f32_16x16x128_fp8_fp8 %0, %1, %2, %3" : "+a"(acc) : "v"(a), "v"(b), "v"(idx));
         else if constexpr(E == SpElem::I8)
@@ -237,6 +251,14 @@ namespace
         };
         // load x (0..12) of stage `stage` into the slot at byte `at`: 0..3 kept values, 4 indices, 5..12 dense B
         auto issueLoad = [&](uint32_t stage, uint32_t at, uint32_t x) {
+#ifdef R355_ABLATE_LOADS
+            if(stage >= RING)
+                return;
+#endif
+#ifdef R355_SPARSE_A_DIRECT
+            if(x < 5u)
+                return; // A does not pass through LDS
+#endif
             const bool     valid = stage < numStages;
             const uint32_t st    = valid ? stage : 0u;
             if(x < 4u)
@@ -286,12 +308,16 @@ namespace
         };
         // the pieces / loads dealt to slot n (0..15) of a quadrant
         auto readSlotA = [&](AGroup& grp, uint32_t at, uint32_t half, uint32_t n) {
+#if !defined(R355_ABLATE_READS) && !defined(R355_SPARSE_A_DIRECT)
             if((n & 1u) == 0u)
                 readA(grp, at, half, n >> 1);
+#endif
         };
         auto readSlotB = [&](i32x8 (&grp)[4], uint32_t at, uint32_t half, uint32_t n) {
+#ifndef R355_ABLATE_READS
             if((n & 1u) == 0u)
                 readB(grp, at, half, n >> 1);
+#endif
         };
 
         AccV acc[8][8];
@@ -303,18 +329,60 @@ namespace
 
         AGroup aLo, aHi;
         i32x8  bX[4], bY[4]; // alternate as the low / high half of B's blocks
+#ifdef R355_SPARSE_A_DIRECT
+        AGroup         aOwn[2][2]; // [stage parity][low / high four blocks]: this wave's A, requested one stage ahead
+        const uint32_t aLaneV = wm * 8192u + lane * 16u, aLaneM = (wm * 2048u + lane * 4u) / ES;
+        // piece n of a stage's A: 0 .. 7 the values of block n, 8 .. 15 the indices of block n - 8 (buffers that end with
+        // the tile's last valid row; a stage past the end is a buffer of nothing)
+        auto loadOwnA = [&](uint32_t stage, uint32_t par, uint32_t n) {
+            const bool     valid = stage < numStages;
+            const uint32_t st    = valid ? stage : 0u;
+            if(n < 8u)
+            {
+                const auto rsrc = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>(gA + st * strideV), 0,
+                                                                    static_cast<int>(valid ? validM * 64u : 0u), 0x00020000);
+                aOwn[par][n / 4u].v[n % 4u] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, aLaneV, n * 1024u, 0));
+            }
+            else
+            {
+                const uint32_t i    = n - 8u;
+                const auto     rsrc = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>(gM + st * strideM), 0,
+                                                                        static_cast<int>(valid ? validM * (16u / ES) : 0u), 0x00020000);
+                if constexpr(ES == 1u)
+                    aOwn[par][i / 4u].idx[i % 4u] = static_cast<int>(__builtin_amdgcn_raw_buffer_load_b32(rsrc, aLaneM, i * 256u, 0));
+                else
+                {
+                    // (low 16 bits only, the high half left undefined: see readA)
+                    using s16x2 = short __attribute__((ext_vector_type(2)));
+                    s16x2 v;
+                    v[0]                          = __builtin_amdgcn_raw_buffer_load_b16(rsrc, aLaneM, i * 128u, 0);
+                    aOwn[par][i / 4u].idx[i % 4u] = __builtin_bit_cast(int, v);
+                }
+            }
+        };
+#endif
 
         // The 13 loads of a stage are dealt out over a whole stage's time, three or four per quadrant: 0 .. 6 under Q3 and Q4
         // of the stage that frees the slot, 7 .. 12 under Q1 and Q2 of the one after it (the memory pipeline then always has
         // requests to work on; issued under Q3 and Q4 only, it ran dry during the other half of every stage).
         constexpr uint32_t FIRST_HALF = 7;
-        auto stageBody = [&](uint32_t kt, uint32_t cur, uint32_t nxt, uint32_t prv, i32x8 (&bLo)[4], i32x8 (&bHi)[4]) {
+        // (par: parity of the stage, which names the register set of the measurement build that keeps A out of LDS)
+        auto stageBody = [&](uint32_t kt, uint32_t cur, uint32_t nxt, uint32_t prv, i32x8 (&bLo)[4], i32x8 (&bHi)[4], uint32_t par) {
+#ifdef R355_SPARSE_A_DIRECT
+            AGroup& aLo = aOwn[par][0];
+            AGroup& aHi = aOwn[par][1];
+#else
+            (void)par;
+#endif
             // Q1: A low x B low; B high arrives; loads 7 .. 9 of stage kt + 2 (into the slot stage kt - 1 has left)
 #pragma unroll
             for(uint32_t n = 0; n < 16; ++n)
             {
                 smfmac16<E>(acc[n % 4u][n / 4u], aLo.v[n % 4u], bLo[n / 4u], aLo.idx[n % 4u]);
                 readSlotB(bHi, cur, 1, n);
+#ifdef R355_SPARSE_A_DIRECT
+                loadOwnA(kt + 1u, par ^ 1u, n);
+#endif
                 if(n % 5u == 1u)
                     issueLoad(kt + 2u, prv, FIRST_HALF + n / 5u);
                 __builtin_amdgcn_sched_barrier(0);
@@ -329,7 +397,13 @@ namespace
                     issueLoad(kt + 2u, prv, FIRST_HALF + 3u + n / 5u);
                 __builtin_amdgcn_sched_barrier(0);
             }
+#if defined(R355_SPARSE_A_DIRECT)
+            r355::waitVmcnt<8 + 16>(); // the youngest: 8 B loads of stage kt + 2 and the 16 A loads of stage kt + 1 issued under Q1
+#elif defined(R355_ABLATE_LOADS)
+            r355::waitVmcnt<0>();
+#else
             r355::waitVmcnt<LOADS_PER_STAGE>(); // stage kt + 1 has landed; the youngest 13 loads are stage kt + 2
+#endif
             r355::ldsBarrier();
             // Q3: A high x B high (row by row, in the order A arrived); next A low arrives; loads 0 .. 3 of stage kt + 3
 #pragma unroll
@@ -364,35 +438,42 @@ namespace
 #pragma unroll
         for(uint32_t r = 0; r < 8; ++r)
         {
+#ifndef R355_SPARSE_A_DIRECT
             readA(aLo, SLOT[0], 0, r);
+#endif
             readB(bX, SLOT[0], 0, r);
         }
+#ifdef R355_SPARSE_A_DIRECT
+#pragma unroll
+        for(uint32_t n = 0; n < 16; ++n)
+            loadOwnA(0u, 0u, n);
+#endif
 
         uint32_t kt = 0;
         for(uint32_t trips = numStages / 6u; trips > 0; --trips, kt += 6u)
         {
-            stageBody(kt, SLOT[0], SLOT[1], SLOT[2], bX, bY);
-            stageBody(kt + 1u, SLOT[1], SLOT[2], SLOT[0], bY, bX);
-            stageBody(kt + 2u, SLOT[2], SLOT[0], SLOT[1], bX, bY);
-            stageBody(kt + 3u, SLOT[0], SLOT[1], SLOT[2], bY, bX);
-            stageBody(kt + 4u, SLOT[1], SLOT[2], SLOT[0], bX, bY);
-            stageBody(kt + 5u, SLOT[2], SLOT[0], SLOT[1], bY, bX);
+            stageBody(kt, SLOT[0], SLOT[1], SLOT[2], bX, bY, 0u);
+            stageBody(kt + 1u, SLOT[1], SLOT[2], SLOT[0], bY, bX, 1u);
+            stageBody(kt + 2u, SLOT[2], SLOT[0], SLOT[1], bX, bY, 0u);
+            stageBody(kt + 3u, SLOT[0], SLOT[1], SLOT[2], bY, bX, 1u);
+            stageBody(kt + 4u, SLOT[1], SLOT[2], SLOT[0], bX, bY, 0u);
+            stageBody(kt + 5u, SLOT[2], SLOT[0], SLOT[1], bY, bX, 1u);
         }
         const uint32_t rem = numStages - kt;
         if(rem > 0u)
         {
-            stageBody(kt, SLOT[0], SLOT[1], SLOT[2], bX, bY);
+            stageBody(kt, SLOT[0], SLOT[1], SLOT[2], bX, bY, 0u);
             if(rem > 1u)
             {
-                stageBody(kt + 1u, SLOT[1], SLOT[2], SLOT[0], bY, bX);
+                stageBody(kt + 1u, SLOT[1], SLOT[2], SLOT[0], bY, bX, 1u);
                 if(rem > 2u)
                 {
-                    stageBody(kt + 2u, SLOT[2], SLOT[0], SLOT[1], bX, bY);
+                    stageBody(kt + 2u, SLOT[2], SLOT[0], SLOT[1], bX, bY, 0u);
                     if(rem > 3u)
                     {
-                        stageBody(kt + 3u, SLOT[0], SLOT[1], SLOT[2], bY, bX);
+                        stageBody(kt + 3u, SLOT[0], SLOT[1], SLOT[2], bY, bX, 1u);
                         if(rem > 4u)
-                            stageBody(kt + 4u, SLOT[1], SLOT[2], SLOT[0], bX, bY);
+                            stageBody(kt + 4u, SLOT[1], SLOT[2], SLOT[0], bX, bY, 0u);
                     }
                 }
             }

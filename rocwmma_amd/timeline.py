@@ -78,6 +78,11 @@ def main():
     if gaps:
         gaps = np.array(gaps)
         print("| gap to the CU's next workgroup | %.2f | %.2f | %.2f | %.2f |" % (gaps.mean(), gaps.min(), np.median(gaps), gaps.max()))
+    # the XCDs (each with a clock of its own under the board's power management): mean K loop and when the last epilogue ends
+    xcd = (t[:, 5] & 0xF).astype(np.int64)
+    kloop = us[:, 2] - us[:, 1]
+    print("per XCD (mean K loop us / last epilogue ends at us): " + ", ".join(
+        "%d: %.1f / %.1f" % (x, kloop[xcd == x].mean(), us[xcd == x, 3].max()) for x in sorted(set(xcd.tolist()))))
     order = np.argsort(us[:, 2])
     per = len(cus)
     for r in range(-(-tiles // per)):
