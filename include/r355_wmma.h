@@ -84,7 +84,7 @@ typedef enum
  * D = alpha * A * B + beta * D in place); any other overlap of D with A, B or C is undefined.
  *
  * sparse24 != 0: A is 2:4 structured-sparse along k (i8 -> i32, e4m3 | f16 | bf16 -> f32; a 256 x 256 macro-tile kernel
- * from m, n >= 128 on when B is col-major, a block-per-wave kernel otherwise, which takes B in either orientation):
+ * from m, n >= 128 on, a block-per-wave kernel below that; B in either orientation):
  * `a` holds the m * k/2 kept values and `a_meta` the m * k/8 index bytes in the K-blocked storage that
  * r355_compress_24 / r355_compress_24_16 write (layout_a = R355_ROW_MAJOR, lda = k / 2: the storage has no padding);
  * m, n multiples of 16, k of 128 bytes' worth of elements (128 for 1-byte, 64 for 2-byte elements).

@@ -11,7 +11,7 @@
 // so that all a 256-row macro tile needs of one stage is 16 + 4 KiB of consecutive bytes (whole cache lines;
 // with row-major compressed rows a stage touched 64 + 16 bytes of every row's lines and the direct-to-LDS
 // loads ran at two thirds of the rate), and a fragment's 16 bytes per lane are consecutive across lanes.
-// B is dense, col-major (k contiguous) for the macro tile, either orientation for the block-per-wave kernel; D row- or
+// B is dense, in either orientation (the macro tile stages a col-major B as rows and a row-major B as k-rows); D row- or
 // col-major.  m % 16 == 0, k % (128 / ES) == 0.
 //
 // Two kernels:
@@ -45,6 +45,7 @@
 
 #include "common.hpp"
 #include "lds_dma.hpp"
+#include "operand_tile.hpp"
 #include "tile_map.hpp"
 
 namespace
@@ -200,7 +201,10 @@ namespace
             asm volatile("v_smfmac_f32_16x16x64_bf16 %0, %1, %2, %3" : "+a"(acc) : "v"(a), "v"(b), "v"(idx));
     }
 
-    template <SpElem E>
+    // B_KCONTIG: B is col-major (K contiguous: rows of the tile in LDS, one ds_read_b128 per 16-byte piece); otherwise
+    // row-major (N contiguous: k-rows in LDS, swizzled and read back with transposing reads as the dense kernels' M/N-
+    // contiguous operands are, operand_tile.hpp: two reads per piece).
+    template <SpElem E, bool B_KCONTIG>
     __global__ void __launch_bounds__(T_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
         sparseTiledKernel(TiledParams p)
     {
@@ -233,7 +237,7 @@ namespace
         const uint32_t gOffA = tid * 16u;
         const uint32_t rowB = tid >> 3, slotB = tid & 7u;
         const uint32_t ldbBytes = p.ldb * ES;
-        const uint32_t gOffB = rowB * ldbBytes + ((slotB ^ ((rowB >> 1) & 7u)) * 16u), gStepB = 32u * ldbBytes;
+        const uint32_t gOffB = rowB * ldbBytes + ((slotB ^ ((rowB >> 1) & 7u)) * 16u), gStepB = 32u * ldbBytes; // (col-major B)
         const uint32_t numStages = p.k * ES / T_K;
         const uint64_t strideV = (uint64_t)p.m * 64u, strideM = (uint64_t)p.m * (16u / ES); // bytes between stages
         // (wave-uniform; the readfirstlane calls only tell the compiler so, which keeps the buffer descriptors in scalar registers)
@@ -241,8 +245,14 @@ namespace
         const uint32_t validN = __builtin_amdgcn_readfirstlane(p.n - tn * T_N < T_N ? p.n - tn * T_N : T_N);
         const uint64_t gA = r355::uniformAddress(p.aVals + (uint64_t)tm * A_BYTES);
         const uint64_t gM = r355::uniformAddress(p.aMeta + (uint64_t)tm * (META_BYTES / ES));
-        const uint64_t gB = r355::uniformAddress(p.b + (uint64_t)tn * T_N * ldbBytes);
+        const uint64_t gB = r355::uniformAddress(p.b + (B_KCONTIG ? (uint64_t)tn * T_N * ldbBytes : (uint64_t)tn * T_N * ES));
         const uint32_t dmaDst = ldsBase + wave * 1024u; // lane l lands at dmaDst + slot + piece + 16 l
+        // row-major B: a stage is 128 / ES k-rows of the tile's 256 columns; a lane whose 16-byte chunk lies beyond n takes
+        // the tile's first chunk instead (what it brings only feeds columns of D that are never stored)
+        uint32_t gOffBn[8] = {}, gStepBn = 0u, kByteBn = 0u;
+        uint64_t gStageBn = 0u;
+        if constexpr(!B_KCONTIG)
+            r355::tile::laneOffsets8<false, 8, ES>(tid, p.ldb, validN, gOffBn, gStepBn, gStageBn, kByteBn);
 
         // a buffer of `bytes` bytes at addr, or over nothing for a stage past the end
         auto rsrcOf = [](uint64_t addr, uint32_t bytes, bool valid) {
@@ -265,8 +275,11 @@ namespace
                 loadToLds(rsrcOf(gA + st * strideV, validM * 64u, valid), gOffA, x * 4096u, dmaDst + at + x * 4096u);
             else if(x == 4u)
                 loadToLds(rsrcOf(gM + st * strideM, validM * (16u / ES), valid), gOffA, 0u, dmaDst + at + OFF_META);
-            else // 32 rows of B per load; the buffer ends with the tile's last valid row
+            else if constexpr(B_KCONTIG) // 32 rows of B per load; the buffer ends with the tile's last valid row
                 loadToLds(rsrcOf(gB + (uint64_t)st * T_K, validN * ldbBytes - st * T_K, valid), gOffB, (x - 5u) * gStepB,
+                          dmaDst + at + OFF_B + (x - 5u) * 4096u);
+            else // 16 / ES k-rows of B per load; the buffer is the stage's k-rows (K is whole stages: no tail)
+                loadToLds(rsrcOf(gB + st * gStageBn, (T_K / ES) * ldbBytes, valid), gOffBn[x - 5u], (x - 5u) * gStepBn,
                           dmaDst + at + OFF_B + (x - 5u) * 4096u);
         };
 
@@ -276,6 +289,9 @@ namespace
         const uint32_t rdA = wm * 8192u + lane * 16u, rdM = OFF_META + (wm * 2048u + lane * 4u) / ES;
         const uint32_t rB  = wn * 128u + t, swB = (t >> 1) & 7u;
         const uint32_t rdB0 = OFF_B + rB * 128u + ((g ^ swB) * 16u), rdB1 = OFF_B + rB * 128u + (((4u + g) ^ swB) * 16u);
+        uint32_t       rdBn[8] = {}; // row-major B: block j of the wave's eight, first half of the lane's k-rows of K half 0
+        if constexpr(!B_KCONTIG)
+            r355::tile::readOffsets8<false, 8, ES>(wn, lane, rdBn);
 
         // piece r (0..7) of an A group: block r / 2 of the half, values (r even) or indices (r odd)
         auto readA = [&](AGroup& grp, uint32_t at, uint32_t half, uint32_t r) {
@@ -299,12 +315,17 @@ namespace
             else
                 grp.v[r >> 1] = *reinterpret_cast<const i32x4*>(lds + at + rdA + i * 1024u);
         };
-        // piece r (0..7) of a B group: block r / 2 of the half, 64-byte K half r % 2
-        auto readB = [&](i32x8 (&grp)[4], uint32_t at, uint32_t half, uint32_t r) {
+        // piece r (0..7) of a B group: block r / 2 of the half, 64-byte K half r % 2 (row-major B: in two transposed parts)
+        auto readB = [&](i32x8 (&grp)[4], uint32_t at, uint32_t half, uint32_t r, uint32_t part = 0u) {
             const uint32_t j = 4u * half + (r >> 1);
-            const i32x4    v = *reinterpret_cast<const i32x4*>(lds + at + ((r & 1u) ? rdB1 : rdB0) + j * 2048u);
-            const uint32_t o = 4u * (r & 1u);
-            grp[r >> 1][o] = v[0], grp[r >> 1][o + 1u] = v[1], grp[r >> 1][o + 2u] = v[2], grp[r >> 1][o + 3u] = v[3];
+            if constexpr(B_KCONTIG)
+            {
+                const i32x4    v = *reinterpret_cast<const i32x4*>(lds + at + ((r & 1u) ? rdB1 : rdB0) + j * 2048u);
+                const uint32_t o = 4u * (r & 1u);
+                grp[r >> 1][o] = v[0], grp[r >> 1][o + 1u] = v[1], grp[r >> 1][o + 2u] = v[2], grp[r >> 1][o + 3u] = v[3];
+            }
+            else
+                r355::tile::readBlock8<false, 8, ES>(lds + at + OFF_B, rdBn, j, r & 1u, part, grp[r >> 1], 4u * (r & 1u));
         };
         // the pieces / loads dealt to slot n (0..15) of a quadrant
         auto readSlotA = [&](AGroup& grp, uint32_t at, uint32_t half, uint32_t n) {
@@ -315,7 +336,9 @@ namespace
         };
         auto readSlotB = [&](i32x8 (&grp)[4], uint32_t at, uint32_t half, uint32_t n) {
 #ifndef R355_ABLATE_READS
-            if((n & 1u) == 0u)
+            if constexpr(!B_KCONTIG)
+                readB(grp, at, half, n >> 1, n & 1u);
+            else if((n & 1u) == 0u)
                 readB(grp, at, half, n >> 1);
 #endif
         };
@@ -442,6 +465,8 @@ namespace
             readA(aLo, SLOT[0], 0, r);
 #endif
             readB(bX, SLOT[0], 0, r);
+            if constexpr(!B_KCONTIG)
+                readB(bX, SLOT[0], 0, r, 1u);
         }
 #ifdef R355_SPARSE_A_DIRECT
 #pragma unroll
@@ -562,8 +587,7 @@ namespace
         const uint32_t es = (g.in_type == R355_F16 || g.in_type == R355_BF16) ? 2u : 1u;
         const bool     forced = g.kernel == R355_KERNEL_TILED || g.kernel == R355_KERNEL_TILED_DEEP; // (one and the same here)
         const bool     shape  = forced || (g.m >= T_M / 2 && g.n >= T_N / 2);
-        return g.kernel != R355_KERNEL_SIMPLE && shape && g.layout_b == R355_COL_MAJOR && (g.beta == 0.0 || g.layout_c == g.layout_d)
-               && r355::aligned(g.a_meta, 16)
+        return g.kernel != R355_KERNEL_SIMPLE && shape && (g.beta == 0.0 || g.layout_c == g.layout_d) && r355::aligned(g.a_meta, 16)
                && (uint64_t)g.ldb * es <= (1u << 23);
     }
 
@@ -598,7 +622,7 @@ namespace r355
             return fail(R355_ERR_UNSUPPORTED, "sparse gemm: there is no 128 x 128 sparse macro tile (R355_KERNEL_TILED is 256 x 256)");
         if((g.kernel == R355_KERNEL_TILED || g.kernel == R355_KERNEL_TILED_DEEP) && !tiledOk(g))
             return fail(R355_ERR_UNSUPPORTED,
-                        "sparse gemm (macro tile): B must be col-major, C (when beta != 0) and D must share an orientation, metadata 16-byte aligned, ldb below 8 MiB");
+                        "sparse gemm (macro tile): C (when beta != 0) and D must share an orientation, metadata 16-byte aligned, ldb below 8 MiB");
         if(plan && tiledOk(g))
         {
             plan->kernel       = R355_KERNEL_TILED;
@@ -662,13 +686,20 @@ namespace r355
             p.tilesM = (g.m + T_M - 1) / T_M, p.tilesN = (g.n + T_N - 1) / T_N;
             p.dRow = g.layout_d == R355_ROW_MAJOR;
             const dim3 grid(((p.tilesM * p.tilesN + 7u) / 8u) * 8u), block(T_THREADS);
-            switch(g.in_type)
-            {
-            case R355_E4M3: hipLaunchKernelGGL(sparseTiledKernel<SpElem::E4M3>, grid, block, 0, stream, p); break;
-            case R355_F16: hipLaunchKernelGGL(sparseTiledKernel<SpElem::F16>, grid, block, 0, stream, p); break;
-            case R355_BF16: hipLaunchKernelGGL(sparseTiledKernel<SpElem::BF16>, grid, block, 0, stream, p); break;
-            default: hipLaunchKernelGGL(sparseTiledKernel<SpElem::I8>, grid, block, 0, stream, p); break;
-            }
+            auto go = [&](auto bk) {
+                constexpr bool BK = decltype(bk)::value;
+                switch(g.in_type)
+                {
+                case R355_E4M3: hipLaunchKernelGGL((sparseTiledKernel<SpElem::E4M3, BK>), grid, block, 0, stream, p); break;
+                case R355_F16: hipLaunchKernelGGL((sparseTiledKernel<SpElem::F16, BK>), grid, block, 0, stream, p); break;
+                case R355_BF16: hipLaunchKernelGGL((sparseTiledKernel<SpElem::BF16, BK>), grid, block, 0, stream, p); break;
+                default: hipLaunchKernelGGL((sparseTiledKernel<SpElem::I8, BK>), grid, block, 0, stream, p); break;
+                }
+            };
+            if(g.layout_b == R355_COL_MAJOR)
+                go(std::true_type{});
+            else
+                go(std::false_type{});
             return checkLaunch("sparse gemm (macro tile)");
         }
         switch(g.in_type)

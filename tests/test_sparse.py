@@ -60,6 +60,11 @@ def test_sparse_config4_sampled_rows(in_t, out_t):
     dd = device_filled(m * n, O.NP_STORAGE[out_t], 0xFF)
     R.gemm(in_t, out_t, m, n, k, dv, db, None, dd, 1.0, 0.0, O.ROW, O.COL, O.ROW, O.ROW, a_meta=dm)
     got = to_host(dd, O.NP_STORAGE[out_t]).reshape(m, n)
+    # the same problem with B stored row-major (k x n, n contiguous): the same products in the same order
+    dbt = to_device(np.ascontiguousarray(b.reshape(n, k).T))
+    ddt = device_filled(m * n, O.NP_STORAGE[out_t], 0xFF)
+    R.gemm(in_t, out_t, m, n, k, dv, dbt, None, ddt, 1.0, 0.0, O.ROW, O.ROW, O.ROW, O.ROW, a_meta=dm)
+    assert np.array_equal(to_host(ddt, O.NP_STORAGE[out_t]).reshape(m, n).view(np.uint8), got.view(np.uint8))
     rows = np.array([0, 31, 32, 2047, 4095, 1234], dtype=np.uint32)
     storage = dense.view(np.uint8) if in_t == O.E4M3 else dense
     want = O.gemm_rows(in_t, out_t, O.ROW, O.COL, m, n, k, storage.ravel(), b, rows)
@@ -106,11 +111,12 @@ def test_sparse_gemm_16bit_vs_dense_oracle(in_t, m, n, k, ldl):
 
 
 @pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32), (O.F16, O.F32), (O.BF16, O.F32)])
-@pytest.mark.parametrize("m,n,k", [(32, 32, 128), (16, 48, 256), (272, 144, 384)])
+@pytest.mark.parametrize("m,n,k", [(32, 32, 128), (16, 48, 256), (272, 144, 384), (256, 256, 128), (512, 384, 896), (144, 400, 640)])
 @pytest.mark.parametrize("ldl", [O.ROW, O.COL])
 def test_sparse_gemm_row_major_b(in_t, out_t, m, n, k, ldl):
-    """B (k x n) with n contiguous: the block-per-wave kernel takes either orientation of B (the macro tile wants
-    K-contiguous columns and is not chosen), against the oracle's dense GEMM with the same orientation."""
+    """B (k x n) with n contiguous: both kernels take either orientation of B (the macro tile stages k-rows of B and
+    reads them back with transposing LDS reads), against the oracle's dense GEMM with the same orientation.  Sizes: below a
+    tile, edge tiles in m and n, one to seven stages (every remainder of the six-stage loop trip)."""
     mask = O.sparse24_mask(80, m, k)
     if in_t == O.I8:
         dense = np.where(mask, O.uniform_int8(81, m * k).reshape(m, k), np.int8(0)).astype(np.int8)
@@ -130,7 +136,7 @@ def test_sparse_gemm_row_major_b(in_t, out_t, m, n, k, ldl):
     dv, dm, db, dc = to_device(vals), to_device(meta), to_device(b), to_device(c)
     dd = device_filled(m * n, O.NP_STORAGE[out_t], 0xFF)
     args = R.gemm_args(in_t, out_t, m, n, k, dv, db, dc, dd, 1.0, 1.0, O.ROW, O.ROW, ldl, ldl, a_meta=dm)
-    assert R.gemm_query(args).kernel == R.KERNEL_SIMPLE
+    assert R.gemm_query(args).kernel == (R.KERNEL_TILED if (m >= 128 and n >= 128) else R.KERNEL_SIMPLE)
     R.gemm(in_t, out_t, m, n, k, dv, db, dc, dd, 1.0, 1.0, O.ROW, O.ROW, ldl, ldl, a_meta=dm)
     got = to_host(dd, O.NP_STORAGE[out_t])
     if in_t == O.I8:
@@ -138,9 +144,15 @@ def test_sparse_gemm_row_major_b(in_t, out_t, m, n, k, ldl):
     else:
         g, w = got.astype(np.float64), want.astype(np.float64)
         assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= (1e-2 if in_t == O.E4M3 else 1e-3)
-    with pytest.raises(R.R355Error) as e:  # the macro tile cannot be forced onto a row-major B
-        R.gemm_query(R.gemm_args(in_t, out_t, m, n, k, dv, db, dc, dd, 1.0, 1.0, O.ROW, O.ROW, ldl, ldl, a_meta=dm, kernel=R.KERNEL_TILED))
-    assert e.value.code == -2
+    # the macro tile forced (any m, n: rows and columns beyond the matrix are clamped or load as zeros)
+    dd2 = device_filled(m * n, O.NP_STORAGE[out_t], 0xFF)
+    R.gemm(in_t, out_t, m, n, k, dv, db, dc, dd2, 1.0, 1.0, O.ROW, O.ROW, ldl, ldl, a_meta=dm, kernel=R.KERNEL_TILED)
+    got2 = to_host(dd2, O.NP_STORAGE[out_t])
+    if in_t == O.I8:
+        assert np.array_equal(got2, want)
+    else:
+        g, w = got2.astype(np.float64), want.astype(np.float64)
+        assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= (1e-2 if in_t == O.E4M3 else 1e-3)
 
 
 @pytest.mark.parametrize("case", range(40))
@@ -176,8 +188,6 @@ def test_sparse_random_sweep(case):
     dv, dm, db, dc = to_device(vals), to_device(meta), to_device(b), to_device(c)
     dd = device_filled(m * n + 4, O.NP_STORAGE[out_t], 0xEE)
     kernel = [R.KERNEL_AUTO, R.KERNEL_TILED, R.KERNEL_SIMPLE][int(rng.integers(0, 3))]
-    if lb == O.ROW and kernel == R.KERNEL_TILED:
-        kernel = R.KERNEL_AUTO  # the macro tile wants K-contiguous columns of B
     # padded leading dimensions of B, C and D (drawn last, so the cases above keep their other draws)
     pad_b = (16 // es) * int(rng.integers(0, 3))
     pad_c, pad_d = 4 * int(rng.integers(0, 3)), 4 * int(rng.integers(0, 3))
