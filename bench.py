@@ -30,7 +30,8 @@ HBM_PEAK_GBPS = 8000.0
 # was measured on; a row whose digest differs from the sources of this tree is reported as null, so a counter
 # can never outlive the kernel it belongs to.
 COUNTERS_FILE = os.path.join(ROOT, "profiles", "bench_counters.md")
-KERNEL_SOURCES = {"gemm": ["gemm_tiled.hip", "tile_map.hpp", "lds_dma.hpp"], "sparse": ["sparse.hip", "tile_map.hpp", "lds_dma.hpp"],
+KERNEL_SOURCES = {"gemm": ["gemm_tiled.hip", "tile_map.hpp", "lds_dma.hpp", "operand_tile.hpp"],
+                  "sparse": ["sparse.hip", "tile_map.hpp", "lds_dma.hpp", "operand_tile.hpp"],
                   "dlrm": ["dlrm.hip"]}
 
 

@@ -38,9 +38,11 @@ def test_library_loaded_before_torch():
     assert r.returncode == 0 and "one runtime, result exact" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
 
 
-def test_stale_hip_error_of_another_caller_is_not_reported():
+def test_stale_hip_error_of_another_caller_is_neither_reported_nor_consumed():
     """hipGetLastError is per thread and sticky: an earlier call of anybody that failed harmlessly (here a hipFree of a
-    pointer nobody allocated, refused on the host) must not come back as this library's launch failure."""
+    pointer nobody allocated, refused on the host) must not come back as this library's launch failure - and it must
+    still be there for its owner afterwards: the entry points only peek at the pending error, as a plain kernel launch of
+    the reference leaves it alone."""
     import ctypes
 
     import torch
@@ -49,14 +51,22 @@ def test_stale_hip_error_of_another_caller_is_not_reported():
 
     a = torch.randint(-5, 5, (64 * 64,), dtype=torch.int8, device="cuda")
     d = torch.empty(64 * 64, dtype=torch.int32, device="cuda")
+    y, ones_a, ones_x = torch.empty(64, device="cuda"), torch.ones(64 * 64, device="cuda"), torch.ones(64, device="cuda")
     loaded = sorted({l.split()[-1] for l in open("/proc/self/maps") if "libamdhip64" in l})
     assert len(loaded) == 1, loaded
     hip = ctypes.CDLL(loaded[0])  # the file is already mapped: this is a handle to the runtime in use, not another copy
     hip.hipFree.argtypes, hip.hipFree.restype = [ctypes.c_void_p], ctypes.c_int
-    assert hip.hipFree(ctypes.c_void_p(0x10)) != 0
-    R.gemm(R.I8, R.I32, 64, 64, 64, a, a, None, d, 1.0, 0.0, R.ROW_MAJOR, R.COL_MAJOR, R.ROW_MAJOR, R.ROW_MAJOR)
-    y, ones_a, ones_x = torch.empty(64, device="cuda"), torch.ones(64 * 64, device="cuda"), torch.ones(64, device="cuda")
-    assert hip.hipFree(ctypes.c_void_p(0x10)) != 0  # (torch itself raises on its next kernel after such an error: none follows)
+    hip.hipGetLastError.argtypes, hip.hipGetLastError.restype = [], ctypes.c_int
+    torch.cuda.synchronize()
+    assert hip.hipGetLastError() == 0
+    refused = hip.hipFree(ctypes.c_void_p(0x10))
+    assert refused != 0
+    R.gemm(R.I8, R.I32, 64, 64, 64, a, a, None, d, 1.0, 0.0, R.ROW_MAJOR, R.COL_MAJOR, R.ROW_MAJOR, R.ROW_MAJOR)  # no R355Error
+    assert hip.hipGetLastError() == refused  # still pending for whoever caused it (fetched here, before torch trips over it)
+    assert hip.hipGetLastError() == 0
+    assert hip.hipFree(ctypes.c_void_p(0x10)) == refused
     R.gemv(R.ROW_MAJOR, 64, 64, ones_a, ones_x, None, y)
+    assert hip.hipGetLastError() == refused and hip.hipGetLastError() == 0
     torch.cuda.synchronize()
     assert torch.equal(y, torch.full((64,), 64.0, device="cuda"))
+    assert torch.equal(d.view(64, 64).double(), a.view(64, 64).double() @ a.view(64, 64).double().t())
