@@ -83,8 +83,9 @@ typedef enum
  * beta == 0 means C is never read and may be NULL.  C may be D itself (same pointer, leading dimension and orientation:
  * D = alpha * A * B + beta * D in place); any other overlap of D with A, B or C is undefined.
  *
- * sparse24 != 0: A is 2:4 structured-sparse along k (i8 -> i32, e4m3 | f16 | bf16 -> f32; a 256 x 256 macro-tile kernel
- * from m, n >= 128 on, a block-per-wave kernel below that; B in either orientation):
+ * sparse24 != 0: A is 2:4 structured-sparse along k (i8 -> i32, e4m3 | f16 | bf16 -> f32; from m, n >= 128 on a macro-tile
+ * kernel of 256 x 256 or 128 x 128 - R355_KERNEL_TILED / R355_KERNEL_TILED_128 force one, AUTO takes the faster by a timing
+ * model - and a block-per-wave kernel below that; B in either orientation; no split along K):
  * `a` holds the m * k/2 kept values and `a_meta` the m * k/8 index bytes in the K-blocked storage that
  * r355_compress_24 / r355_compress_24_16 write (layout_a = R355_ROW_MAJOR, lda = k / 2: the storage has no padding);
  * m, n multiples of 16, k of 128 bytes' worth of elements (128 for 1-byte, 64 for 2-byte elements).

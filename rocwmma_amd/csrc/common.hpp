@@ -63,6 +63,22 @@ namespace r355
         return R355_OK;
     }
 
+    // CUs of the current device; where the query fails (no device: plan queries on a build host) MI355X's 256
+    inline uint32_t computeUnits()
+    {
+        static const uint32_t cus = [] {
+            int dev = 0, n = 0;
+            if(hipGetDevice(&dev) != hipSuccess
+               || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            {
+                (void)hipGetLastError();
+                return 256u;
+            }
+            return static_cast<uint32_t>(n);
+        }();
+        return cus;
+    }
+
     // Kernel families (defined in their own translation units)
     int gemmSimpleCheck(const r355_gemm_args& g, r355_gemm_plan* plan);
     int gemmSimpleLaunch(const r355_gemm_args& g, hipStream_t stream);

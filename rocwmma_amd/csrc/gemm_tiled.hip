@@ -1769,21 +1769,7 @@ namespace
     }
 
 #if R355_TILED_HAS(0)
-    // CUs of the current device; where the query fails (no device: plan queries on a build host) MI355X's 256
-    uint32_t computeUnits()
-    {
-        static const uint32_t cus = [] {
-            int dev = 0, n = 0;
-            if(hipGetDevice(&dev) != hipSuccess
-               || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-            {
-                (void)hipGetLastError();
-                return 256u;
-            }
-            return static_cast<uint32_t>(n);
-        }();
-        return cus;
-    }
+    using r355::computeUnits;
 
     // Macro tile edge for a problem.
     // Long K: the 128 x 128 tile is a quarter of the work of the 256 x 256 one at about 0.55 of its efficiency with one

@@ -125,15 +125,30 @@ namespace
         store_matrix_sync(d + offD, fragAcc, ldd, layoutD);
     }
 
-    // ------------------------------------------------------------------ macro-tile kernel
-    constexpr uint32_t T_M = 256, T_N = 256, T_K = 128; // dense bytes of K per stage
-    constexpr uint32_t T_THREADS   = 256;
-    constexpr uint32_t A_BYTES     = T_M * (T_K / 2); // 16 KiB kept values
-    constexpr uint32_t META_BYTES  = T_M * (T_K / 8); // 4 KiB indices (2 KiB of them used by 2-byte elements)
-    constexpr uint32_t B_BYTES     = T_N * T_K; // 32 KiB dense
-    constexpr uint32_t OFF_META    = A_BYTES;
-    constexpr uint32_t OFF_B       = A_BYTES + META_BYTES;
-    constexpr uint32_t STAGE_BYTES = A_BYTES + META_BYTES + B_BYTES; // 52 KiB
+    // ------------------------------------------------------------------ macro-tile kernels
+    // WB = accumulator blocks per wave-tile edge: 8 - macro tile 256 x 256, one workgroup per CU; 4 - macro tile 128 x 128,
+    // two workgroups per CU, for problems whose large tiles would leave most CUs idle.
+    constexpr uint32_t T_K = 128; // dense bytes of K per stage
+    constexpr uint32_t T_THREADS = 256;
+    template <uint32_t WB>
+    struct SpTile
+    {
+        static constexpr uint32_t M = 32u * WB, N = 32u * WB;
+        static constexpr uint32_t A_BYTES     = M * (T_K / 2); // kept values: 16 / 8 KiB
+        static constexpr uint32_t META_BYTES  = M * (T_K / 8); // indices: 4 / 2 KiB (half of them used by 2-byte elements)
+        static constexpr uint32_t B_BYTES     = N * T_K; // dense B: 32 / 16 KiB
+        static constexpr uint32_t OFF_META    = A_BYTES;
+        static constexpr uint32_t OFF_B       = A_BYTES + META_BYTES;
+        static constexpr uint32_t STAGE_BYTES = A_BYTES + META_BYTES + B_BYTES; // 52 / 26 KiB
+        // direct loads of 4 KiB (256 lanes x 16 bytes) per stage: NA of kept values, one of indices - issued by the first
+        // META_WAVES waves only, 1 KiB each, so that nothing lands beyond the index region - and NB of B
+        static constexpr uint32_t NA = A_BYTES / 4096u, NB = B_BYTES / 4096u, LOADS = NA + 1u + NB; // 13 / 7
+        static constexpr uint32_t META_WAVES = META_BYTES / 1024u; // 4 / 2
+        // how a stage's loads are dealt out over the four quadrants after the barrier that frees their slot (Q3, Q4 of that
+        // stage, Q1, Q2 of the next): load i of a quadrant goes out in its slot i * STEP + 1
+        //   large tile: 4 + 3 | 3 + 3 loads, every 4th / 5th slot of a quadrant's 16; small tile: 2 + 2 | 2 + 1, every 2nd of 4
+        static constexpr uint32_t FIRST_HALF = WB == 8 ? 7u : 4u;
+    };
 
     struct TiledParams
     {
@@ -149,29 +164,29 @@ namespace
         uint32_t       dRow; // D (and C) row-major
     };
 
-    // Three 52 KiB stage slots (156 of 160 KiB): the slot of stage kt is refilled with stage kt + 3 once every
-    // wave has its operands in registers, so one and a half to two stages of loads (78 - 104 KiB per CU) are in flight at
-    // any time.  The direct loads are explicit (lds_dma.hpp) and the only vmcnt wait is "all but the youngest 13" before
-    // each barrier; loads past the last stage are issued with nothing in range (zero fill, no memory traffic), so
-    // every stage issues the same 13.
+    // Three stage slots (3 x 52 = 156 of 160 KiB; small tile: 3 x 26 = 78 KiB): the slot of stage kt is refilled with stage
+    // kt + 3 once every wave has its operands in registers, so one and a half to two stages of loads are in flight at
+    // any time.  The direct loads are explicit (lds_dma.hpp) and the only vmcnt wait is "all but the youngest stage's
+    // loads" before each barrier; loads past the last stage are issued with nothing in range (zero fill, no memory
+    // traffic), so every stage issues the same loads.
     //
-    // A stage is one 128-wide K step: 64 matrix instructions per wave.  As in the dense fp8 kernel it is split
-    // into quadrants of the wave tile, consecutive quadrants sharing one operand group of four blocks:
-    //     Q1 = A[0..3] x B[0..3]   Q2 = A[0..3] x B[4..7]   Q3 = A[4..7] x B[4..7]   Q4 = A[4..7] x B[0..3]
-    //     under Q1: B[4..7] of this stage arrives      under Q3: A[0..3] of the next stage
-    //     under Q2: A[4..7] of this stage              under Q4: B[0..3] of the next stage
-    // After Q2 the stage's slot is no longer read: barrier, then its refill - loads 0 .. 6 of stage kt + 3 under Q3 and Q4,
-    // loads 7 .. 12 under Q1 and Q2 of the next stage, three or four per quadrant, so that the memory pipeline has
-    // requests to work on during the whole stage (all 13 under Q3 and Q4: 0.0722 ms for 4096 x 4096 x 8192 int8 against
-    // 0.0710).  One LDS read per two matrix instructions, pinned by scheduling barriers.  The two B register groups
-    // swap roles every stage and the ring has three slots: six stages per loop trip, single exit, then up to five
+    // A stage is one 128-byte K step: WB x WB matrix instructions per wave.  As in the dense fp8 kernel it is split
+    // into quadrants of the wave tile, consecutive quadrants sharing one operand group of H = WB / 2 blocks:
+    //     Q1 = A[lo] x B[lo]   Q2 = A[lo] x B[hi]   Q3 = A[hi] x B[hi]   Q4 = A[hi] x B[lo]
+    //     under Q1: B[hi] of this stage arrives      under Q3: A[lo] of the next stage
+    //     under Q2: A[hi] of this stage              under Q4: B[lo] of the next stage
+    // After Q2 the stage's slot is no longer read: barrier, then its refill - the first half of stage kt + 3's loads under
+    // Q3 and Q4, the rest under Q1 and Q2 of the next stage, so that the memory pipeline has requests to work on during the
+    // whole stage (all of them under Q3 and Q4: 0.0722 ms for 4096 x 4096 x 8192 int8 against 0.0710).  The two B register
+    // groups swap roles every stage and the ring has three slots: six stages per loop trip, single exit, then up to five
     // stages of straight-line code.
-    constexpr uint32_t RING = 3, LOADS_PER_STAGE = 13;
+    constexpr uint32_t RING = 3;
 
+    template <uint32_t H>
     struct AGroup
     {
-        i32x4 v[4]; // 16 kept bytes per lane and block
-        int   idx[4];
+        i32x4 v[H]; // 16 kept bytes per lane and block
+        int   idx[H];
     };
 
     enum class SpElem
@@ -204,15 +219,21 @@ namespace
     // B_KCONTIG: B is col-major (K contiguous: rows of the tile in LDS, one ds_read_b128 per 16-byte piece); otherwise
     // row-major (N contiguous: k-rows in LDS, swizzled and read back with transposing reads as the dense kernels' M/N-
     // contiguous operands are, operand_tile.hpp: two reads per piece).
-    template <SpElem E, bool B_KCONTIG>
-    __global__ void __launch_bounds__(T_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
-        sparseTiledKernel(TiledParams p)
+    template <SpElem E, bool B_KCONTIG, uint32_t WB>
+    __device__ __forceinline__ void sparseTiled(const TiledParams& p)
     {
+        using T = SpTile<WB>;
         constexpr bool     INT = E == SpElem::I8;
         constexpr uint32_t ES  = (E == SpElem::F16 || E == SpElem::BF16) ? 2u : 1u; // element bytes
+        constexpr uint32_t H = WB / 2u, NQ = H * H; // blocks per operand group, matrix instructions per quadrant
+        constexpr uint32_t OFF_META = T::OFF_META, OFF_B = T::OFF_B, STAGE_BYTES = T::STAGE_BYTES;
         using AccE = std::conditional_t<INT, int, float>;
         using AccV = std::conditional_t<INT, i32x4, f32x4>;
+        using AG   = AGroup<H>;
         using r355::loadToLds;
+#ifdef R355_SPARSE_A_DIRECT
+        static_assert(WB == 8, "the measurement build that keeps A out of LDS has the large tile only");
+#endif
 
         __shared__ __attribute__((aligned(1024))) char lds[RING * STAGE_BYTES];
 
@@ -229,7 +250,7 @@ namespace
             = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) char*)lds));
 
         // ---- global -> LDS (per thread, fixed).  LDS chunk L = j * 256 + tid of each operand tile.
-        //   kept values / indices: the tile's share of a stage is 16 / 4 KiB of consecutive bytes, copied as they are
+        //   kept values / indices: the tile's share of a stage is consecutive bytes, copied as they are
         //   dense B: 8 chunks per row, chunk c of row r in slot c ^ ((r >> 1) & 7)
         //   Edge tiles: the tile's rows of A are the first validM / 16 KiB (values) of its share of a stage and the rows
         //   of B the first validN * ldb bytes from the tile's first row: each load's buffer ends exactly there, and what
@@ -241,61 +262,74 @@ namespace
         const uint32_t numStages = p.k * ES / T_K;
         const uint64_t strideV = (uint64_t)p.m * 64u, strideM = (uint64_t)p.m * (16u / ES); // bytes between stages
         // (wave-uniform; the readfirstlane calls only tell the compiler so, which keeps the buffer descriptors in scalar registers)
-        const uint32_t validM = __builtin_amdgcn_readfirstlane(p.m - tm * T_M < T_M ? p.m - tm * T_M : T_M);
-        const uint32_t validN = __builtin_amdgcn_readfirstlane(p.n - tn * T_N < T_N ? p.n - tn * T_N : T_N);
-        const uint64_t gA = r355::uniformAddress(p.aVals + (uint64_t)tm * A_BYTES);
-        const uint64_t gM = r355::uniformAddress(p.aMeta + (uint64_t)tm * (META_BYTES / ES));
-        const uint64_t gB = r355::uniformAddress(p.b + (B_KCONTIG ? (uint64_t)tn * T_N * ldbBytes : (uint64_t)tn * T_N * ES));
+        const uint32_t validM = __builtin_amdgcn_readfirstlane(p.m - tm * T::M < T::M ? p.m - tm * T::M : T::M);
+        const uint32_t validN = __builtin_amdgcn_readfirstlane(p.n - tn * T::N < T::N ? p.n - tn * T::N : T::N);
+        const uint64_t gA = r355::uniformAddress(p.aVals + (uint64_t)tm * T::A_BYTES);
+        const uint64_t gM = r355::uniformAddress(p.aMeta + (uint64_t)tm * (T::META_BYTES / ES));
+        const uint64_t gB = r355::uniformAddress(p.b + (B_KCONTIG ? (uint64_t)tn * T::N * ldbBytes : (uint64_t)tn * T::N * ES));
         const uint32_t dmaDst = ldsBase + wave * 1024u; // lane l lands at dmaDst + slot + piece + 16 l
-        // row-major B: a stage is 128 / ES k-rows of the tile's 256 columns; a lane whose 16-byte chunk lies beyond n takes
+        // row-major B: a stage is 128 / ES k-rows of the tile's columns; a lane whose 16-byte chunk lies beyond n takes
         // the tile's first chunk instead (what it brings only feeds columns of D that are never stored)
-        uint32_t gOffBn[8] = {}, gStepBn = 0u, kByteBn = 0u;
+        uint32_t gOffBn[WB] = {}, gStepBn = 0u, kByteBn = 0u;
         uint64_t gStageBn = 0u;
         if constexpr(!B_KCONTIG)
-            r355::tile::laneOffsets8<false, 8, ES>(tid, p.ldb, validN, gOffBn, gStepBn, gStageBn, kByteBn);
+            r355::tile::laneOffsets8<false, WB, ES>(tid, p.ldb, validN, gOffBn, gStepBn, gStageBn, kByteBn);
+        const bool metaWave = wave < T::META_WAVES; // (wave-uniform) this wave brings 1 KiB of the stage's indices
 
         // a buffer of `bytes` bytes at addr, or over nothing for a stage past the end
         auto rsrcOf = [](uint64_t addr, uint32_t bytes, bool valid) {
             return i32x4{static_cast<int>(static_cast<uint32_t>(addr)), static_cast<int>(static_cast<uint32_t>(addr >> 32) & 0xFFFFu),
                          static_cast<int>(valid ? bytes : 0u), 0x00020000};
         };
-        // load x (0..12) of stage `stage` into the slot at byte `at`: 0..3 kept values, 4 indices, 5..12 dense B
+        // load x of stage `stage` into the slot at byte `at`: NA of kept values, then the indices, then NB of dense B
         auto issueLoad = [&](uint32_t stage, uint32_t at, uint32_t x) {
 #ifdef R355_ABLATE_LOADS
             if(stage >= RING)
                 return;
 #endif
 #ifdef R355_SPARSE_A_DIRECT
-            if(x < 5u)
+            if(x <= T::NA)
                 return; // A does not pass through LDS
 #endif
             const bool     valid = stage < numStages;
             const uint32_t st    = valid ? stage : 0u;
-            if(x < 4u)
+            if(x < T::NA)
                 loadToLds(rsrcOf(gA + st * strideV, validM * 64u, valid), gOffA, x * 4096u, dmaDst + at + x * 4096u);
-            else if(x == 4u)
-                loadToLds(rsrcOf(gM + st * strideM, validM * (16u / ES), valid), gOffA, 0u, dmaDst + at + OFF_META);
+            else if(x == T::NA)
+            {
+                if(T::META_WAVES == 4u || metaWave)
+                    loadToLds(rsrcOf(gM + st * strideM, validM * (16u / ES), valid), gOffA, 0u, dmaDst + at + OFF_META);
+            }
             else if constexpr(B_KCONTIG) // 32 rows of B per load; the buffer ends with the tile's last valid row
-                loadToLds(rsrcOf(gB + (uint64_t)st * T_K, validN * ldbBytes - st * T_K, valid), gOffB, (x - 5u) * gStepB,
-                          dmaDst + at + OFF_B + (x - 5u) * 4096u);
+                loadToLds(rsrcOf(gB + (uint64_t)st * T_K, validN * ldbBytes - st * T_K, valid), gOffB, (x - T::NA - 1u) * gStepB,
+                          dmaDst + at + OFF_B + (x - T::NA - 1u) * 4096u);
             else // 16 / ES k-rows of B per load; the buffer is the stage's k-rows (K is whole stages: no tail)
-                loadToLds(rsrcOf(gB + st * gStageBn, (T_K / ES) * ldbBytes, valid), gOffBn[x - 5u], (x - 5u) * gStepBn,
-                          dmaDst + at + OFF_B + (x - 5u) * 4096u);
+                loadToLds(rsrcOf(gB + st * gStageBn, (T_K / ES) * ldbBytes, valid), gOffBn[x - T::NA - 1u], (x - T::NA - 1u) * gStepBn,
+                          dmaDst + at + OFF_B + (x - T::NA - 1u) * 4096u);
+        };
+        // wait until only the youngest COUNT loads of this wave are outstanding, METAS of which are index loads (which
+        // only the first META_WAVES waves issue)
+        auto waitYoungest = [&](auto count, auto metas) {
+            constexpr uint32_t COUNT = decltype(count)::value, METAS = decltype(metas)::value;
+            if(T::META_WAVES == 4u || metaWave)
+                r355::waitVmcnt<COUNT>();
+            else
+                r355::waitVmcnt<COUNT - METAS>();
         };
 
         // ---- LDS -> registers (per lane, fixed)
-        //   block i of A (rows 16 i .. + 15 of the wave's 128): 1 KiB of values in lane order, 256 B of indices
+        //   block i of A (rows 16 i .. + 15 of the wave's 16 WB): 1 KiB of values in lane order, 256 B of indices
         //   block j of B: row 16 j + t, 16-byte chunks g and 4 + g of the row's 128 bytes
-        const uint32_t rdA = wm * 8192u + lane * 16u, rdM = OFF_META + (wm * 2048u + lane * 4u) / ES;
-        const uint32_t rB  = wn * 128u + t, swB = (t >> 1) & 7u;
+        const uint32_t rdA = wm * (WB * 1024u) + lane * 16u, rdM = OFF_META + (wm * (WB * 256u) + lane * 4u) / ES;
+        const uint32_t rB  = wn * (16u * WB) + t, swB = (t >> 1) & 7u;
         const uint32_t rdB0 = OFF_B + rB * 128u + ((g ^ swB) * 16u), rdB1 = OFF_B + rB * 128u + (((4u + g) ^ swB) * 16u);
-        uint32_t       rdBn[8] = {}; // row-major B: block j of the wave's eight, first half of the lane's k-rows of K half 0
+        uint32_t       rdBn[8] = {}; // row-major B: block j of the wave's own, first half of the lane's k-rows of K half 0
         if constexpr(!B_KCONTIG)
-            r355::tile::readOffsets8<false, 8, ES>(wn, lane, rdBn);
+            r355::tile::readOffsets8<false, WB, ES>(wn, lane, rdBn);
 
-        // piece r (0..7) of an A group: block r / 2 of the half, values (r even) or indices (r odd)
-        auto readA = [&](AGroup& grp, uint32_t at, uint32_t half, uint32_t r) {
-            const uint32_t i = 4u * half + (r >> 1);
+        // piece r (0 .. 2 H - 1) of an A group: block r / 2 of the half, values (r even) or indices (r odd)
+        auto readA = [&](AG& grp, uint32_t at, uint32_t half, uint32_t r) {
+            const uint32_t i = H * half + (r >> 1);
             if(r & 1u)
             {
                 if constexpr(ES == 1u)
@@ -315,9 +349,9 @@ namespace
             else
                 grp.v[r >> 1] = *reinterpret_cast<const i32x4*>(lds + at + rdA + i * 1024u);
         };
-        // piece r (0..7) of a B group: block r / 2 of the half, 64-byte K half r % 2 (row-major B: in two transposed parts)
-        auto readB = [&](i32x8 (&grp)[4], uint32_t at, uint32_t half, uint32_t r, uint32_t part = 0u) {
-            const uint32_t j = 4u * half + (r >> 1);
+        // piece r (0 .. 2 H - 1) of a B group: block r / 2 of the half, 64-byte K half r % 2 (row-major B: in two transposed parts)
+        auto readB = [&](i32x8 (&grp)[H], uint32_t at, uint32_t half, uint32_t r, uint32_t part = 0u) {
+            const uint32_t j = H * half + (r >> 1);
             if constexpr(B_KCONTIG)
             {
                 const i32x4    v = *reinterpret_cast<const i32x4*>(lds + at + ((r & 1u) ? rdB1 : rdB0) + j * 2048u);
@@ -325,35 +359,43 @@ namespace
                 grp[r >> 1][o] = v[0], grp[r >> 1][o + 1u] = v[1], grp[r >> 1][o + 2u] = v[2], grp[r >> 1][o + 3u] = v[3];
             }
             else
-                r355::tile::readBlock8<false, 8, ES>(lds + at + OFF_B, rdBn, j, r & 1u, part, grp[r >> 1], 4u * (r & 1u));
+                r355::tile::readBlock8<false, WB, ES>(lds + at + OFF_B, rdBn, j, r & 1u, part, grp[r >> 1], 4u * (r & 1u));
         };
-        // the pieces / loads dealt to slot n (0..15) of a quadrant
-        auto readSlotA = [&](AGroup& grp, uint32_t at, uint32_t half, uint32_t n) {
+        // the pieces dealt to slot n (0 .. NQ - 1) of a quadrant: a group's 2 H pieces (4 H transposed half pieces of a
+        // row-major B) evenly over the NQ slots - large tile: one read per two (one) matrix instructions, small tile: one (two)
+        auto readSlotA = [&](AG& grp, uint32_t at, uint32_t half, uint32_t n) {
 #if !defined(R355_ABLATE_READS) && !defined(R355_SPARSE_A_DIRECT)
-            if((n & 1u) == 0u)
-                readA(grp, at, half, n >> 1);
+            constexpr uint32_t P = 2u * H;
+#pragma unroll
+            for(uint32_t r = (n * P + NQ - 1u) / NQ; r < ((n + 1u) * P + NQ - 1u) / NQ; ++r)
+                readA(grp, at, half, r);
 #endif
         };
-        auto readSlotB = [&](i32x8 (&grp)[4], uint32_t at, uint32_t half, uint32_t n) {
+        auto readSlotB = [&](i32x8 (&grp)[H], uint32_t at, uint32_t half, uint32_t n) {
 #ifndef R355_ABLATE_READS
-            if constexpr(!B_KCONTIG)
-                readB(grp, at, half, n >> 1, n & 1u);
-            else if((n & 1u) == 0u)
-                readB(grp, at, half, n >> 1);
+            constexpr uint32_t P = B_KCONTIG ? 2u * H : 4u * H;
+#pragma unroll
+            for(uint32_t r = (n * P + NQ - 1u) / NQ; r < ((n + 1u) * P + NQ - 1u) / NQ; ++r)
+            {
+                if constexpr(B_KCONTIG)
+                    readB(grp, at, half, r);
+                else
+                    readB(grp, at, half, r >> 1, r & 1u);
+            }
 #endif
         };
 
-        AccV acc[8][8];
+        AccV acc[WB][WB];
 #pragma unroll
-        for(uint32_t i = 0; i < 8; ++i)
+        for(uint32_t i = 0; i < WB; ++i)
 #pragma unroll
-            for(uint32_t j = 0; j < 8; ++j)
+            for(uint32_t j = 0; j < WB; ++j)
                 acc[i][j] = AccV{0, 0, 0, 0};
 
-        AGroup aLo, aHi;
-        i32x8  bX[4], bY[4]; // alternate as the low / high half of B's blocks
+        AG    aLo, aHi;
+        i32x8 bX[H], bY[H]; // alternate as the low / high half of B's blocks
 #ifdef R355_SPARSE_A_DIRECT
-        AGroup         aOwn[2][2]; // [stage parity][low / high four blocks]: this wave's A, requested one stage ahead
+        AG             aOwn[2][2]; // [stage parity][low / high four blocks]: this wave's A, requested one stage ahead
         const uint32_t aLaneV = wm * 8192u + lane * 16u, aLaneM = (wm * 2048u + lane * 4u) / ES;
         // piece n of a stage's A: 0 .. 7 the values of block n, 8 .. 15 the indices of block n - 8 (buffers that end with
         // the tile's last valid row; a stage past the end is a buffer of nothing)
@@ -385,39 +427,46 @@ namespace
         };
 #endif
 
-        // The 13 loads of a stage are dealt out over a whole stage's time, three or four per quadrant: 0 .. 6 under Q3 and Q4
-        // of the stage that frees the slot, 7 .. 12 under Q1 and Q2 of the one after it (the memory pipeline then always has
-        // requests to work on; issued under Q3 and Q4 only, it ran dry during the other half of every stage).
-        constexpr uint32_t FIRST_HALF = 7;
+        // load slot n of quadrant q (0: Q3, 1: Q4 of the stage that frees the slot `at`; 2: Q1, 3: Q2 of the next stage)
+        auto loadSlot = [&](uint32_t q, uint32_t stage, uint32_t at, uint32_t n) {
+            constexpr uint32_t COUNT[4] = {WB == 8 ? 4u : 2u, WB == 8 ? 3u : 2u, WB == 8 ? 3u : 2u, WB == 8 ? 3u : 1u};
+            constexpr uint32_t STEP[4]  = {WB == 8 ? 4u : 2u, WB == 8 ? 5u : 2u, WB == 8 ? 5u : 2u, WB == 8 ? 5u : 2u};
+            static_assert(COUNT[0] + COUNT[1] == T::FIRST_HALF && COUNT[0] + COUNT[1] + COUNT[2] + COUNT[3] == T::LOADS, "every load has a slot");
+            uint32_t first = 0;
+#pragma unroll
+            for(uint32_t u = 0; u < 4; ++u)
+                if(u < q)
+                    first += COUNT[u];
+            if(n % STEP[q] == 1u && n / STEP[q] < COUNT[q])
+                issueLoad(stage, at, first + n / STEP[q]);
+        };
         // (par: parity of the stage, which names the register set of the measurement build that keeps A out of LDS)
-        auto stageBody = [&](uint32_t kt, uint32_t cur, uint32_t nxt, uint32_t prv, i32x8 (&bLo)[4], i32x8 (&bHi)[4], uint32_t par) {
+        auto stageBody = [&](uint32_t kt, uint32_t cur, uint32_t nxt, uint32_t prv, i32x8 (&bLo)[H], i32x8 (&bHi)[H], uint32_t par) {
 #ifdef R355_SPARSE_A_DIRECT
-            AGroup& aLo = aOwn[par][0];
-            AGroup& aHi = aOwn[par][1];
+            AG& aLo = aOwn[par][0];
+            AG& aHi = aOwn[par][1];
 #else
             (void)par;
 #endif
-            // Q1: A low x B low; B high arrives; loads 7 .. 9 of stage kt + 2 (into the slot stage kt - 1 has left)
+            // Q1: A low x B low; B high arrives; the third quarter of stage kt + 2's loads (into the slot stage kt - 1 has left)
 #pragma unroll
-            for(uint32_t n = 0; n < 16; ++n)
+            for(uint32_t n = 0; n < NQ; ++n)
             {
-                smfmac16<E>(acc[n % 4u][n / 4u], aLo.v[n % 4u], bLo[n / 4u], aLo.idx[n % 4u]);
+                smfmac16<E>(acc[n % H][n / H], aLo.v[n % H], bLo[n / H], aLo.idx[n % H]);
                 readSlotB(bHi, cur, 1, n);
 #ifdef R355_SPARSE_A_DIRECT
                 loadOwnA(kt + 1u, par ^ 1u, n);
 #endif
-                if(n % 5u == 1u)
-                    issueLoad(kt + 2u, prv, FIRST_HALF + n / 5u);
+                loadSlot(2u, kt + 2u, prv, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            // Q2: A low x B high (column by column, in the order B arrived); A high arrives; loads 10 .. 12 of stage kt + 2
+            // Q2: A low x B high (column by column, in the order B arrived); A high arrives; the last of stage kt + 2's loads
 #pragma unroll
-            for(uint32_t n = 0; n < 16; ++n)
+            for(uint32_t n = 0; n < NQ; ++n)
             {
-                smfmac16<E>(acc[n % 4u][4u + n / 4u], aLo.v[n % 4u], bHi[n / 4u], aLo.idx[n % 4u]);
+                smfmac16<E>(acc[n % H][H + n / H], aLo.v[n % H], bHi[n / H], aLo.idx[n % H]);
                 readSlotA(aHi, cur, 1, n);
-                if(n % 5u == 1u)
-                    issueLoad(kt + 2u, prv, FIRST_HALF + 3u + n / 5u);
+                loadSlot(3u, kt + 2u, prv, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
 #if defined(R355_SPARSE_A_DIRECT)
@@ -425,27 +474,26 @@ namespace
 #elif defined(R355_ABLATE_LOADS)
             r355::waitVmcnt<0>();
 #else
-            r355::waitVmcnt<LOADS_PER_STAGE>(); // stage kt + 1 has landed; the youngest 13 loads are stage kt + 2
+            // stage kt + 1 has landed; the youngest loads are stage kt + 2's
+            waitYoungest(std::integral_constant<uint32_t, T::LOADS>{}, std::integral_constant<uint32_t, 1>{});
 #endif
             r355::ldsBarrier();
-            // Q3: A high x B high (row by row, in the order A arrived); next A low arrives; loads 0 .. 3 of stage kt + 3
+            // Q3: A high x B high (row by row, in the order A arrived); next A low arrives; the first of stage kt + 3's loads
 #pragma unroll
-            for(uint32_t n = 0; n < 16; ++n)
+            for(uint32_t n = 0; n < NQ; ++n)
             {
-                smfmac16<E>(acc[4u + n / 4u][4u + n % 4u], aHi.v[n / 4u], bHi[n % 4u], aHi.idx[n / 4u]);
+                smfmac16<E>(acc[H + n / H][H + n % H], aHi.v[n / H], bHi[n % H], aHi.idx[n / H]);
                 readSlotA(aLo, nxt, 0, n);
-                if(n % 4u == 1u)
-                    issueLoad(kt + 3u, cur, n / 4u);
+                loadSlot(0u, kt + 3u, cur, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            // Q4: A high x B low; next B low arrives in the registers B high has left; loads 4 .. 6 of stage kt + 3
+            // Q4: A high x B low; next B low arrives in the registers B high has left; the second quarter of stage kt + 3's loads
 #pragma unroll
-            for(uint32_t n = 0; n < 16; ++n)
+            for(uint32_t n = 0; n < NQ; ++n)
             {
-                smfmac16<E>(acc[4u + n % 4u][n / 4u], aHi.v[n % 4u], bLo[n / 4u], aHi.idx[n % 4u]);
+                smfmac16<E>(acc[H + n % H][n / H], aHi.v[n % H], bLo[n / H], aHi.idx[n % H]);
                 readSlotB(bHi, nxt, 0, n);
-                if(n % 5u == 1u)
-                    issueLoad(kt + 3u, cur, 4u + n / 5u);
+                loadSlot(1u, kt + 3u, cur, n);
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
@@ -454,12 +502,13 @@ namespace
 #pragma unroll
         for(uint32_t st = 0; st < RING; ++st)
 #pragma unroll
-            for(uint32_t x = 0; x < (st + 1u < RING ? LOADS_PER_STAGE : FIRST_HALF); ++x)
+            for(uint32_t x = 0; x < (st + 1u < RING ? T::LOADS : T::FIRST_HALF); ++x)
                 issueLoad(st, SLOT[st], x); // (the rest of stage 2 follows under Q1 and Q2 of stage 0)
-        r355::waitVmcnt<LOADS_PER_STAGE + FIRST_HALF>();
+        // stage 0 has landed: stage 1 and the first half of stage 2 (an index load in each) may still be under way
+        waitYoungest(std::integral_constant<uint32_t, T::LOADS + T::FIRST_HALF>{}, std::integral_constant<uint32_t, 2>{});
         r355::ldsBarrier();
 #pragma unroll
-        for(uint32_t r = 0; r < 8; ++r)
+        for(uint32_t r = 0; r < 2u * H; ++r)
         {
 #ifndef R355_SPARSE_A_DIRECT
             readA(aLo, SLOT[0], 0, r);
@@ -511,18 +560,23 @@ namespace
 
         // ---- epilogue.  A lane holds D(16 i + 4 g + e, 16 j + t), e = 0..3, of each block: four consecutive
         // rows of one column.
+        // (the lane number is taken afresh - ordered after the K loop's matrix instructions - so that nothing derived from
+        // it for the epilogue occupies a register, or a spill slot, during the K loop)
+        uint32_t laneE;
+        asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(laneE));
+        const uint32_t tE = laneE & 15u, gE = laneE >> 4;
         const AccE     alpha = static_cast<AccE>(p.alpha), beta = static_cast<AccE>(p.beta);
-        const uint32_t m0 = tm * T_M + wm * 128u, n0 = tn * T_N + wn * 128u;
+        const uint32_t m0 = tm * T::M + wm * (16u * WB), n0 = tn * T::N + wn * (16u * WB);
         using V4 = AccE __attribute__((ext_vector_type(4)));
         if(!p.dRow)
         {
             // col-major: a lane's four rows are contiguous
 #pragma unroll
-            for(uint32_t i = 0; i < 8; ++i)
+            for(uint32_t i = 0; i < WB; ++i)
 #pragma unroll
-                for(uint32_t j = 0; j < 8; ++j)
+                for(uint32_t j = 0; j < WB; ++j)
                 {
-                    const uint32_t row = m0 + 16u * i + 4u * g, col = n0 + 16u * j + t;
+                    const uint32_t row = m0 + 16u * i + 4u * gE, col = n0 + 16u * j + tE;
                     if(row >= p.m || col >= p.n) // (m is a multiple of 16: a lane's four rows are inside or outside together)
                         continue;
                     V4             out;
@@ -540,30 +594,32 @@ namespace
                 }
             return;
         }
-        // row-major: transpose through this wave's 39 KiB of the idle stage slots, 64 rows (four block rows) at a
-        // time: rows of 128 x 4 bytes = 32 chunks, chunk c of row r in slot c ^ (r & 31) -- the 64 lanes of a write
-        // (rows 4 g + e, columns 16 j + t) and of a read (two whole rows) each cover all 64 banks once.
-        char* wl = lds + wave * 39936u;
+        // row-major: transpose through this wave's quarter of the idle stage slots, 64 rows (four block rows) at a time:
+        // rows of 16 WB x 4 bytes = CH chunks of 16 bytes, chunk c of row r in slot c ^ (r % CH) -- the 64 lanes of a write
+        // (rows 4 g + e, columns 16 j + t) and of a read (64 / CH whole rows) each cover all 64 banks once.
+        constexpr uint32_t CH = 4u * WB, ROW_BYTES = 64u * WB, PASSES = WB / 4u;
+        char*              wl = lds + wave * (RING * STAGE_BYTES / 4u);
+        static_assert(RING * STAGE_BYTES / 4u >= 64u * ROW_BYTES, "a wave's share of LDS holds 64 rows of its tile");
 #pragma unroll
-        for(uint32_t pass = 0; pass < 2; ++pass)
+        for(uint32_t pass = 0; pass < PASSES; ++pass)
         {
 #pragma unroll
             for(uint32_t ii = 0; ii < 4; ++ii)
 #pragma unroll
-                for(uint32_t j = 0; j < 8; ++j)
+                for(uint32_t j = 0; j < WB; ++j)
 #pragma unroll
                     for(uint32_t e = 0; e < 4; ++e)
                     {
-                        const uint32_t row = 16u * ii + 4u * g + e, col = 16u * j + t;
-                        *reinterpret_cast<AccE*>(wl + row * 512u + (((col >> 2) ^ (row & 31u)) * 16u) + (col & 3u) * 4u)
+                        const uint32_t row = 16u * ii + 4u * gE + e, col = 16u * j + tE;
+                        *reinterpret_cast<AccE*>(wl + row * ROW_BYTES + (((col >> 2) ^ (row & (CH - 1u))) * 16u) + (col & 3u) * 4u)
                             = alpha * acc[4u * pass + ii][j][e];
                     }
             __builtin_amdgcn_wave_barrier();
 #pragma unroll
-            for(uint32_t it = 0; it < 32; ++it)
+            for(uint32_t it = 0; it < CH; ++it)
             {
-                const uint32_t L = it * 64u + lane, row = L >> 5, c = L & 31u;
-                V4             v = *reinterpret_cast<const V4*>(wl + row * 512u + ((c ^ (row & 31u)) * 16u));
+                const uint32_t L = it * 64u + laneE, row = L / CH, c = L % CH;
+                V4             v = *reinterpret_cast<const V4*>(wl + row * ROW_BYTES + ((c ^ (row & (CH - 1u))) * 16u));
                 const uint64_t off = (uint64_t)(m0 + 64u * pass + row);
                 if(off >= p.m || n0 + 4u * c >= p.n) // (n is a multiple of 16: a 16-byte chunk is inside or outside D as a whole)
                     continue;
@@ -580,15 +636,73 @@ namespace
         }
     }
 
-    // The macro tile runs any m, n (multiples of 16) and k (whole stages); under AUTO it is taken from half a tile in
-    // each direction on (below that most of its matrix instructions would multiply padding).
+    // (a waves-per-EU attribute that depends on a template parameter makes the compiler drop the host-side launch stub:
+    // one __global__ wrapper per tile size)
+    template <SpElem E, bool B_KCONTIG>
+    __global__ void __launch_bounds__(T_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) sparseTiledKernel(TiledParams p)
+    {
+        sparseTiled<E, B_KCONTIG, 8>(p);
+    }
+#ifndef R355_SPARSE_A_DIRECT
+    template <SpElem E, bool B_KCONTIG>
+    __global__ void __launch_bounds__(T_THREADS) sparseTiledKernelSmall(TiledParams p)
+    {
+        sparseTiled<E, B_KCONTIG, 4>(p);
+    }
+#endif
+
+    // The macro tiles run any m, n (multiples of 16) and k (whole stages); under AUTO they are taken from 128 x 128 on
+    // (below that most of a tile's matrix instructions would multiply padding).
     bool tiledOk(const r355_gemm_args& g)
     {
         const uint32_t es = (g.in_type == R355_F16 || g.in_type == R355_BF16) ? 2u : 1u;
-        const bool     forced = g.kernel == R355_KERNEL_TILED || g.kernel == R355_KERNEL_TILED_DEEP; // (one and the same here)
-        const bool     shape  = forced || (g.m >= T_M / 2 && g.n >= T_N / 2);
+        const bool     forced = g.kernel == R355_KERNEL_TILED || g.kernel == R355_KERNEL_TILED_DEEP || g.kernel == R355_KERNEL_TILED_128;
+        const bool     shape  = forced || (g.m >= 128u && g.n >= 128u);
         return g.kernel != R355_KERNEL_SIMPLE && shape && (g.beta == 0.0 || g.layout_c == g.layout_d) && r355::aligned(g.a_meta, 16)
                && (uint64_t)g.ldb * es <= (1u << 23);
+    }
+
+    // Macro tile edge, from a timing model of a launch: rounds over the CUs - one large tile or two small ones per CU and
+    // round - each costing a fixed part plus a part per 128-byte stage of K.  Microseconds, fitted to 8-bit launches of
+    // 1024^2 ... 8192^2 with k from 512 to 8192 (the 16-bit kernels move the same bytes per stage):
+    //                                        fixed   per stage
+    //   256 x 256, every CU busy           15 / 18    0.79      (first / later rounds) the K loop is bound by what the L2 delivers
+    //   256 x 256, at most half the CUs    15 / 18    0.48      to all CUs at once; with half of them idle, by its matrix instructions
+    //   128 x 128, two on every CU            5.4     0.635     (half the work of a large round)
+    //   128 x 128, one on every CU            3.5     0.365
+    //   128 x 128, one on a few CUs           3.5     0.28
+    // and linear in the number of tiles of the last round in between.  So the small tile wins where the large tiles would
+    // leave CUs idle (2048^2 x 8192: 26 us against 48) and, with all CUs busy, up to about 12 stages, where the large
+    // tile's prologue and epilogue - which nothing overlaps with one workgroup per CU - weigh as much as its K loop
+    // (8192^2 x 1024: 81 us against 97); the large tile is 1.35 times faster on long K with the chip full.
+    uint32_t macroTile(const r355_gemm_args& g)
+    {
+#ifdef R355_SPARSE_A_DIRECT
+        return 256u;
+#endif
+        if(g.kernel == R355_KERNEL_TILED || g.kernel == R355_KERNEL_TILED_DEEP)
+            return 256u; // (DEEP: one and the same here)
+        if(g.kernel == R355_KERNEL_TILED_128)
+            return 128u;
+        const uint32_t es     = (g.in_type == R355_F16 || g.in_type == R355_BF16) ? 2u : 1u;
+        const double   stages = static_cast<double>((uint64_t)g.k * es / T_K);
+        const uint64_t cus    = r355::computeUnits();
+        const uint64_t t256   = (uint64_t)((g.m + 255u) / 256u) * ((g.n + 255u) / 256u);
+        const uint64_t t128   = (uint64_t)((g.m + 127u) / 128u) * ((g.n + 127u) / 128u);
+        const double   perCu  = 1.0 / static_cast<double>(cus);
+        double         cost256 = static_cast<double>(t256 / cus) * (18.0 + 0.79 * stages) - 3.0;
+        if(const uint64_t rest = t256 % cus)
+        {
+            const double over = 2.0 * static_cast<double>(rest) * perCu - 1.0; // 0 at half of the CUs, 1 at all of them
+            cost256 += 18.0 + stages * (0.48 + 0.31 * (over > 0.0 ? over : 0.0));
+        }
+        double cost128 = static_cast<double>(t128 / (2u * cus)) * (5.4 + 0.635 * stages);
+        if(const uint64_t rest = t128 % (2u * cus))
+        {
+            const double f = static_cast<double>(rest) * perCu; // tiles per CU: 0 .. 2
+            cost128 += f <= 1.0 ? 3.5 + stages * (0.28 + 0.085 * f) : 3.5 + 1.9 * (f - 1.0) + stages * (0.365 + 0.27 * (f - 1.0));
+        }
+        return cost128 * 1.02 < cost256 ? 128u : 256u; // (over 156 measured shapes the slower tile 6 times, by 2.6 % at most)
     }
 
     uint32_t simpleBlock(const r355_gemm_args& g)
@@ -618,22 +732,23 @@ namespace r355
         if(!aligned(g.a, 16) || !aligned(g.b, 16) || (g.ldb * es) % 16 || !aligned(g.a_meta, 4) || !aligned(g.d, 16) || (g.ldd % 4)
            || (g.beta != 0.0 && (!aligned(g.c, 16) || (g.ldc % 4))))
             return fail(R355_ERR_MISALIGNED, "sparse gemm: values, B, C and D need 16-byte alignment (pointers and leading dimensions), metadata 4-byte");
-        if(g.kernel == R355_KERNEL_TILED_128 || g.kernel == R355_KERNEL_TILED_128_SPLITK)
-            return fail(R355_ERR_UNSUPPORTED, "sparse gemm: there is no 128 x 128 sparse macro tile (R355_KERNEL_TILED is 256 x 256)");
-        if((g.kernel == R355_KERNEL_TILED || g.kernel == R355_KERNEL_TILED_DEEP) && !tiledOk(g))
+        if(g.kernel == R355_KERNEL_TILED_128_SPLITK)
+            return fail(R355_ERR_UNSUPPORTED, "sparse gemm: no split along K (R355_KERNEL_TILED_128 is the 128 x 128 macro tile)");
+        if((g.kernel == R355_KERNEL_TILED || g.kernel == R355_KERNEL_TILED_DEEP || g.kernel == R355_KERNEL_TILED_128) && !tiledOk(g))
             return fail(R355_ERR_UNSUPPORTED,
                         "sparse gemm (macro tile): C (when beta != 0) and D must share an orientation, metadata 16-byte aligned, ldb below 8 MiB");
         if(plan && tiledOk(g))
         {
-            plan->kernel       = R355_KERNEL_TILED;
-            plan->macro_tile_m = T_M;
-            plan->macro_tile_n = T_N;
+            const uint32_t tile = macroTile(g);
+            plan->kernel       = tile == 256u ? R355_KERNEL_TILED : R355_KERNEL_TILED_128;
+            plan->macro_tile_m = tile;
+            plan->macro_tile_n = tile;
             plan->macro_tile_k = T_K / es;
-            plan->grid_x       = ((((g.m + T_M - 1) / T_M) * ((g.n + T_N - 1) / T_N) + 7u) / 8u) * 8u;
+            plan->grid_x       = ((((g.m + tile - 1) / tile) * ((g.n + tile - 1) / tile) + 7u) / 8u) * 8u;
             plan->grid_y       = 1;
             plan->block_x      = T_THREADS;
             plan->block_y      = 1;
-            plan->lds_bytes    = RING * STAGE_BYTES;
+            plan->lds_bytes    = RING * (tile == 256u ? SpTile<8>::STAGE_BYTES : SpTile<4>::STAGE_BYTES);
         }
         else if(plan)
         {
@@ -683,23 +798,34 @@ namespace r355
             p.c = static_cast<const char*>(g.c), p.d = static_cast<char*>(g.d);
             p.ldb = g.ldb, p.ldc = g.ldc, p.ldd = g.ldd;
             p.alpha = g.alpha, p.beta = g.beta;
-            p.tilesM = (g.m + T_M - 1) / T_M, p.tilesN = (g.n + T_N - 1) / T_N;
+            const uint32_t tile = macroTile(g);
+            p.tilesM = (g.m + tile - 1) / tile, p.tilesN = (g.n + tile - 1) / tile;
             p.dRow = g.layout_d == R355_ROW_MAJOR;
             const dim3 grid(((p.tilesM * p.tilesN + 7u) / 8u) * 8u), block(T_THREADS);
-            auto go = [&](auto bk) {
+            auto go = [&](auto bk, auto large) {
                 constexpr bool BK = decltype(bk)::value;
+                auto           launch = [&](auto elem) {
+                    constexpr SpElem E = decltype(elem)::value;
+#ifndef R355_SPARSE_A_DIRECT
+                    if constexpr(!decltype(large)::value)
+                        hipLaunchKernelGGL((sparseTiledKernelSmall<E, BK>), grid, block, 0, stream, p);
+                    else
+#endif
+                        hipLaunchKernelGGL((sparseTiledKernel<E, BK>), grid, block, 0, stream, p);
+                };
                 switch(g.in_type)
                 {
-                case R355_E4M3: hipLaunchKernelGGL((sparseTiledKernel<SpElem::E4M3, BK>), grid, block, 0, stream, p); break;
-                case R355_F16: hipLaunchKernelGGL((sparseTiledKernel<SpElem::F16, BK>), grid, block, 0, stream, p); break;
-                case R355_BF16: hipLaunchKernelGGL((sparseTiledKernel<SpElem::BF16, BK>), grid, block, 0, stream, p); break;
-                default: hipLaunchKernelGGL((sparseTiledKernel<SpElem::I8, BK>), grid, block, 0, stream, p); break;
+                case R355_E4M3: launch(std::integral_constant<SpElem, SpElem::E4M3>{}); break;
+                case R355_F16: launch(std::integral_constant<SpElem, SpElem::F16>{}); break;
+                case R355_BF16: launch(std::integral_constant<SpElem, SpElem::BF16>{}); break;
+                default: launch(std::integral_constant<SpElem, SpElem::I8>{}); break;
                 }
             };
-            if(g.layout_b == R355_COL_MAJOR)
-                go(std::true_type{});
+            const bool colB = g.layout_b == R355_COL_MAJOR;
+            if(tile == 256u)
+                colB ? go(std::true_type{}, std::true_type{}) : go(std::false_type{}, std::true_type{});
             else
-                go(std::false_type{});
+                colB ? go(std::true_type{}, std::false_type{}) : go(std::false_type{}, std::false_type{});
             return checkLaunch("sparse gemm (macro tile)");
         }
         switch(g.in_type)

@@ -159,11 +159,12 @@ def test_argument_validation(kw, code):
 
 
 def test_sparse_macro_tile_ignores_the_orientation_of_an_unread_c():
-    # beta == 0: C is never read, so layout_c means nothing and must not push the call off the 256 x 256 sparse macro tile
+    # beta == 0: C is never read, so layout_c means nothing and must not push the call off the sparse macro tiles
     sp = dict(in_type=R.I8, out_type=R.I32, m=512, n=512, k=1024, lda=512, layout_a=R.ROW_MAJOR, layout_b=R.COL_MAJOR,
               a_meta=0x4000)
-    assert R.gemm_query(_args(layout_c=R.COL_MAJOR, layout_d=R.ROW_MAJOR, **sp)).kernel == R.KERNEL_TILED
-    assert R.gemm_query(_args(layout_c=R.COL_MAJOR, layout_d=R.ROW_MAJOR, kernel=R.KERNEL_TILED, **sp)).kernel == R.KERNEL_TILED
+    assert R.gemm_query(_args(layout_c=R.COL_MAJOR, layout_d=R.ROW_MAJOR, **sp)).kernel in (R.KERNEL_TILED, R.KERNEL_TILED_128)
+    for tile in (R.KERNEL_TILED, R.KERNEL_TILED_128):
+        assert R.gemm_query(_args(layout_c=R.COL_MAJOR, layout_d=R.ROW_MAJOR, kernel=tile, **sp)).kernel == tile
     # beta != 0 with differing orientations: the block-per-wave kernel, and the forced macro tile is refused
     assert R.gemm_query(_args(layout_c=R.COL_MAJOR, layout_d=R.ROW_MAJOR, beta=1.0, c=0x5000, **sp)).kernel == R.KERNEL_SIMPLE
     with pytest.raises(R.R355Error) as e:

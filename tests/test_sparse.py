@@ -11,6 +11,22 @@ from gpuutil import device_filled, to_device, to_host
 
 pytestmark = pytest.mark.gpu
 
+MACRO_TILES = (R.KERNEL_TILED, R.KERNEL_TILED_128)  # 256 x 256 and 128 x 128
+
+
+def _close(got, want, in_t):
+    """The bar of the element type: bit-exact for int8, 1e-2 (e4m3) / 1e-3 (16-bit) on the relative metric."""
+    if in_t == O.I8:
+        return np.array_equal(got, want)
+    g, w = got.astype(np.float64), want.astype(np.float64)
+    return bool(np.all(np.isfinite(g))) and np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= (1e-2 if in_t == O.E4M3 else 1e-3)
+
+
+def _auto_kernels(m, n):
+    """What AUTO may pick: a macro tile (which of the two depends on how many CUs the large tiles would fill) from
+    128 x 128 on, the block-per-wave kernel below that."""
+    return MACRO_TILES if (m >= 128 and n >= 128) else (R.KERNEL_SIMPLE,)
+
 
 def _sparse_inputs(in_t, m, n, k, seed):
     mask = O.sparse24_mask(seed, m, k)
@@ -40,14 +56,14 @@ def test_sparse_gemm_vs_dense_oracle(in_t, out_t, m, n, k, ldl):
     R.gemm(in_t, out_t, m, n, k, dv, db, dc, dd, 1.0, 1.0, O.ROW, O.COL, ldl, ldl, a_meta=dm)
     got = to_host(dd, O.NP_STORAGE[out_t])
     plan = R.gemm_query(R.gemm_args(in_t, out_t, m, n, k, dv, db, dc, dd, 1.0, 1.0, O.ROW, O.COL, ldl, ldl, a_meta=dm))
-    # the macro tile takes every K that fills whole 128-wide stages (1 .. 8 stages above: every remainder of the
-    # six-stage loop trip) and, from half a tile in each direction on, any m and n (edge tiles)
-    assert plan.kernel == (R.KERNEL_TILED if (m >= 128 and n >= 128) else R.KERNEL_SIMPLE)
-    if in_t == O.I8:
-        assert np.array_equal(got, want)
-    else:
-        g, w = got.astype(np.float64), want.astype(np.float64)
-        assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= 1e-2
+    # the macro tiles take every K that fills whole 128-wide stages (1 .. 8 stages above: every remainder of the
+    # six-stage loop trip) and, from 128 x 128 on, any m and n (edge tiles)
+    assert plan.kernel in _auto_kernels(m, n)
+    assert _close(got, want, in_t)
+    for tile in MACRO_TILES:  # each tile size forced (any m, n)
+        dd = device_filled(m * n, O.NP_STORAGE[out_t], 0xFF)
+        R.gemm(in_t, out_t, m, n, k, dv, db, dc, dd, 1.0, 1.0, O.ROW, O.COL, ldl, ldl, a_meta=dm, kernel=tile)
+        assert _close(to_host(dd, O.NP_STORAGE[out_t]), want, in_t), tile
 
 
 @pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32)])
@@ -65,6 +81,11 @@ def test_sparse_config4_sampled_rows(in_t, out_t):
     ddt = device_filled(m * n, O.NP_STORAGE[out_t], 0xFF)
     R.gemm(in_t, out_t, m, n, k, dv, dbt, None, ddt, 1.0, 0.0, O.ROW, O.ROW, O.ROW, O.ROW, a_meta=dm)
     assert np.array_equal(to_host(ddt, O.NP_STORAGE[out_t]).reshape(m, n).view(np.uint8), got.view(np.uint8))
+    # ... and on the other macro tile (AUTO takes the 256 x 256 one here): every element of D sums the same stages in order
+    assert R.gemm_query(R.gemm_args(in_t, out_t, m, n, k, dv, db, None, dd, 1.0, 0.0, O.ROW, O.COL, O.ROW, O.ROW, a_meta=dm)).kernel == R.KERNEL_TILED
+    for bb, lb in ((db, O.COL), (dbt, O.ROW)):
+        R.gemm(in_t, out_t, m, n, k, dv, bb, None, ddt, 1.0, 0.0, O.ROW, lb, O.ROW, O.ROW, a_meta=dm, kernel=R.KERNEL_TILED_128)
+        assert np.array_equal(to_host(ddt, O.NP_STORAGE[out_t]).reshape(m, n).view(np.uint8), got.view(np.uint8))
     rows = np.array([0, 31, 32, 2047, 4095, 1234], dtype=np.uint32)
     storage = dense.view(np.uint8) if in_t == O.E4M3 else dense
     want = O.gemm_rows(in_t, out_t, O.ROW, O.COL, m, n, k, storage.ravel(), b, rows)
@@ -105,9 +126,12 @@ def test_sparse_gemm_16bit_vs_dense_oracle(in_t, m, n, k, ldl):
     R.gemm(in_t, O.F32, m, n, k, dv, db, dc, dd, 2.0, 2.0, O.ROW, O.COL, ldl, ldl, a_meta=dm)
     got = to_host(dd, np.float32)
     plan = R.gemm_query(R.gemm_args(in_t, O.F32, m, n, k, dv, db, dc, dd, 2.0, 2.0, O.ROW, O.COL, ldl, ldl, a_meta=dm))
-    assert plan.kernel == (R.KERNEL_TILED if (m >= 128 and n >= 128) else R.KERNEL_SIMPLE) and plan.macro_tile_k == 64
-    g, w = got.astype(np.float64), want.astype(np.float64)
-    assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= 1e-3
+    assert plan.kernel in _auto_kernels(m, n) and plan.macro_tile_k == 64
+    assert _close(got, want, in_t)
+    for tile in MACRO_TILES:
+        dd = device_filled(m * n, np.float32, 0xFF)
+        R.gemm(in_t, O.F32, m, n, k, dv, db, dc, dd, 2.0, 2.0, O.ROW, O.COL, ldl, ldl, a_meta=dm, kernel=tile)
+        assert _close(to_host(dd, np.float32), want, in_t), tile
 
 
 @pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.E4M3, O.F32), (O.F16, O.F32), (O.BF16, O.F32)])
@@ -136,23 +160,14 @@ def test_sparse_gemm_row_major_b(in_t, out_t, m, n, k, ldl):
     dv, dm, db, dc = to_device(vals), to_device(meta), to_device(b), to_device(c)
     dd = device_filled(m * n, O.NP_STORAGE[out_t], 0xFF)
     args = R.gemm_args(in_t, out_t, m, n, k, dv, db, dc, dd, 1.0, 1.0, O.ROW, O.ROW, ldl, ldl, a_meta=dm)
-    assert R.gemm_query(args).kernel == (R.KERNEL_TILED if (m >= 128 and n >= 128) else R.KERNEL_SIMPLE)
+    assert R.gemm_query(args).kernel in _auto_kernels(m, n)
     R.gemm(in_t, out_t, m, n, k, dv, db, dc, dd, 1.0, 1.0, O.ROW, O.ROW, ldl, ldl, a_meta=dm)
-    got = to_host(dd, O.NP_STORAGE[out_t])
-    if in_t == O.I8:
-        assert np.array_equal(got, want)
-    else:
-        g, w = got.astype(np.float64), want.astype(np.float64)
-        assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= (1e-2 if in_t == O.E4M3 else 1e-3)
-    # the macro tile forced (any m, n: rows and columns beyond the matrix are clamped or load as zeros)
-    dd2 = device_filled(m * n, O.NP_STORAGE[out_t], 0xFF)
-    R.gemm(in_t, out_t, m, n, k, dv, db, dc, dd2, 1.0, 1.0, O.ROW, O.ROW, ldl, ldl, a_meta=dm, kernel=R.KERNEL_TILED)
-    got2 = to_host(dd2, O.NP_STORAGE[out_t])
-    if in_t == O.I8:
-        assert np.array_equal(got2, want)
-    else:
-        g, w = got2.astype(np.float64), want.astype(np.float64)
-        assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= (1e-2 if in_t == O.E4M3 else 1e-3)
+    assert _close(to_host(dd, O.NP_STORAGE[out_t]), want, in_t)
+    # the macro tiles forced (any m, n: rows and columns beyond the matrix are clamped or load as zeros)
+    for tile in MACRO_TILES:
+        dd2 = device_filled(m * n, O.NP_STORAGE[out_t], 0xFF)
+        R.gemm(in_t, out_t, m, n, k, dv, db, dc, dd2, 1.0, 1.0, O.ROW, O.ROW, ldl, ldl, a_meta=dm, kernel=tile)
+        assert _close(to_host(dd2, O.NP_STORAGE[out_t]), want, in_t), tile
 
 
 @pytest.mark.parametrize("case", range(40))
@@ -187,7 +202,7 @@ def test_sparse_random_sweep(case):
     want = O.gemm(in_t, out_t, O.ROW, lb, ldl, ldl, m, n, k, storage.ravel(), b, c, alpha, beta)
     dv, dm, db, dc = to_device(vals), to_device(meta), to_device(b), to_device(c)
     dd = device_filled(m * n + 4, O.NP_STORAGE[out_t], 0xEE)
-    kernel = [R.KERNEL_AUTO, R.KERNEL_TILED, R.KERNEL_SIMPLE][int(rng.integers(0, 3))]
+    kernel = [R.KERNEL_AUTO, R.KERNEL_TILED, R.KERNEL_SIMPLE, R.KERNEL_TILED_128][int(rng.integers(0, 4))]
     # padded leading dimensions of B, C and D (drawn last, so the cases above keep their other draws)
     pad_b = (16 // es) * int(rng.integers(0, 3))
     pad_c, pad_d = 4 * int(rng.integers(0, 3)), 4 * int(rng.integers(0, 3))
@@ -204,12 +219,7 @@ def test_sparse_random_sweep(case):
     rows = full[:major * ldd].reshape(major, ldd)
     assert np.all(rows[:, minor:].view(np.uint8) == 0xEE), "bytes outside D were written"
     got = np.ascontiguousarray(rows[:, :minor]).ravel()
-    if in_t == O.I8:
-        assert np.array_equal(got, want), (m, n, k, lb, ldl, kernel)
-    else:
-        g, w = got.astype(np.float64), want.astype(np.float64)
-        assert np.all(np.isfinite(g))
-        assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= (1e-2 if in_t == O.E4M3 else 1e-3), (m, n, k, lb, ldl, kernel)
+    assert _close(got, want, in_t), (m, n, k, lb, ldl, kernel)
 
 
 def test_sparse_16bit_one_hot_positions():
@@ -236,7 +246,7 @@ def test_sparse_size_and_selector_errors():
     g = lambda m, n, k, kernel=R.KERNEL_AUTO, lda=None: R.gemm_args(R.I8, R.I32, m, n, k, 0x1000, 0x2000, None, 0x3000, 1.0, 0.0,
                                                                   R.ROW_MAJOR, R.COL_MAJOR, R.ROW_MAJOR, R.ROW_MAJOR, a_meta=0x4000,
                                                                   kernel=kernel, lda=lda)
-    for args, code in ((g(256, 256, 192), -3), (g(24, 256, 128), -3), (g(256, 256, 256, R.KERNEL_TILED_128), -2),
+    for args, code in ((g(256, 256, 192), -3), (g(24, 256, 128), -3), (g(256, 256, 256, R.KERNEL_TILED_128_SPLITK), -2),
                        (g(256, 256, 256, lda=136), -1)):
         with pytest.raises(R.R355Error) as e:
             R.gemm_query(args)
@@ -244,13 +254,20 @@ def test_sparse_size_and_selector_errors():
     assert R.gemm_query(g(256, 256, 128, R.KERNEL_TILED)).macro_tile_k == 128  # k % 128, as the header says
     assert R.gemm_query(g(48, 64, 128, R.KERNEL_TILED)).kernel == R.KERNEL_TILED  # forced: any m, n multiple of 16
     assert R.gemm_query(g(48, 64, 128)).kernel == R.KERNEL_SIMPLE
+    small = R.gemm_query(g(48, 64, 128, R.KERNEL_TILED_128))
+    assert (small.kernel, small.macro_tile_m, small.macro_tile_n, small.lds_bytes) == (R.KERNEL_TILED_128, 128, 128, 3 * 26 * 1024)
+    large = R.gemm_query(g(48, 64, 128, R.KERNEL_TILED))
+    assert (large.macro_tile_m, large.macro_tile_n, large.lds_bytes) == (256, 256, 3 * 52 * 1024)
+    # AUTO: the small tile where the large tiles would leave most CUs idle, the large one where they fill the chip
+    assert R.gemm_query(g(1024, 1024, 8192)).kernel == R.KERNEL_TILED_128
+    assert R.gemm_query(g(4096, 4096, 8192)).kernel == R.KERNEL_TILED
 
 
 @pytest.mark.parametrize("in_t,out_t", [(O.I8, O.I32), (O.F16, O.F32)])
 def test_sparse_macro_tile_forced_on_small_and_ragged_shapes(in_t, out_t):
-    """R355_KERNEL_TILED on shapes far below a tile and off the tile grid: rows of A and B beyond the matrix load as zeros
+    """Both macro tiles on shapes far below a tile and off the tile grid: rows of A and B beyond the matrix load as zeros
     and nothing outside D is written (the output sits between two guard regions)."""
-    for m, n, k in ((16, 16, 256), (48, 272, 128), (304, 80, 384)):
+    for m, n, k, tile in [(m, n, k, t) for (m, n, k) in ((16, 16, 256), (48, 272, 128), (304, 80, 384), (144, 208, 896)) for t in MACRO_TILES]:
         es = 1 if in_t == O.I8 else 2
         k = k // es
         mask = O.sparse24_mask(80, m, k)
@@ -267,15 +284,10 @@ def test_sparse_macro_tile_forced_on_small_and_ragged_shapes(in_t, out_t):
         guard = 4096
         dd = device_filled(m * n + 2 * guard, O.NP_STORAGE[out_t], 0xEE)
         # (device_filled hands back a byte tensor: the slice offset is in bytes)
-        R.gemm(in_t, out_t, m, n, k, dv, db, None, dd[guard * 4:], 1.0, 0.0, O.ROW, O.COL, O.ROW, O.ROW, a_meta=dm, kernel=R.KERNEL_TILED)
+        R.gemm(in_t, out_t, m, n, k, dv, db, None, dd[guard * 4:], 1.0, 0.0, O.ROW, O.COL, O.ROW, O.ROW, a_meta=dm, kernel=tile)
         full = to_host(dd, O.NP_STORAGE[out_t])
         assert np.all(full[:guard].view(np.uint32) == np.uint32(0xEEEEEEEE)) and np.all(full[guard + m * n:].view(np.uint32) == np.uint32(0xEEEEEEEE))
-        got = full[guard:guard + m * n]
-        if in_t == O.I8:
-            assert np.array_equal(got, want), (m, n, k)
-        else:
-            g, w = got.astype(np.float64), want.astype(np.float64)
-            assert np.max(np.abs(g - w) / (np.abs(g) + np.abs(w) + 1.0)) <= 1e-3, (m, n, k)
+        assert _close(full[guard:guard + m * n], want, in_t), (m, n, k, tile)
 
 
 @pytest.mark.parametrize("ldl", [O.ROW, O.COL])
