@@ -446,11 +446,14 @@ def run_extras(R, O, np, torch, args, counters, clocks, cus):
     # ops against the sparse peak (2 x dense).  A is drawn dense on the host -- seeded values under a seeded mask that keeps 2 of
     # every group of 4 along k at random positions -- and compressed with the library's own r355_compress_24; sampled complete
     # rows of D are held against the oracle's dense GEMM on the uncompressed A (int8: bit for bit).
-    sm, sn, sk = 4096, 4096, 8192
-    mask = O.sparse24_mask(60, sm, sk)
-    srows = np.array([0, 31, 32, 1234, 2047, 2048, 4064, 4095], dtype=np.uint32)
-    for name, in_t, out_t, key, unit in (("gemm_i8_sparse24_4096x4096x8192", R.I8, R.I32, "i8", "TOP/s (dense-equivalent)"),
-                                         ("gemm_e4m3_sparse24_4096x4096x8192", R.E4M3, R.F32, "e4m3", "TFLOP/s (dense-equivalent)")):
+    # (third row: a quarter of the size, 64 tiles of 256 x 256 - the shape class the 128 x 128 sparse tile is for)
+    sk = 8192
+    for name, in_t, out_t, key, unit, sm in (("gemm_i8_sparse24_4096x4096x8192", R.I8, R.I32, "i8", "TOP/s (dense-equivalent)", 4096),
+                                             ("gemm_e4m3_sparse24_4096x4096x8192", R.E4M3, R.F32, "e4m3", "TFLOP/s (dense-equivalent)", 4096),
+                                             ("gemm_i8_sparse24_2048x2048x8192", R.I8, R.I32, "i8", "TOP/s (dense-equivalent)", 2048)):
+        sn = sm
+        mask = O.sparse24_mask(60, sm, sk)
+        srows = np.array([0, 31, 32, 1234, 2047, sm // 2, sm - 32, sm - 1], dtype=np.uint32)
         if in_t == R.I8:
             av, bh = O.uniform_int8(61, sm * sk).reshape(sm, sk), O.uniform_int8(62, sk * sn)
         else:
@@ -463,7 +466,7 @@ def run_extras(R, O, np, torch, args, counters, clocks, cus):
         gemm_case(name, in_t, out_t, R.ROW_MAJOR, R.COL_MAJOR, torch.from_numpy(vals.view(np.uint8)).cuda(),
                   torch.from_numpy(bh.view(np.uint8)).cuda(), PEAK_TFLOPS[key], unit,
                   sparse_meta=torch.from_numpy(meta).cuda(), mm=sm, nn=sn, kk=sk, peak_scale=2.0, sparse_rows=(srows, want))
-        del av, bh, dense, vals, meta, storage
+        del av, bh, dense, vals, meta, storage, mask
     # DLRM dot interaction forward, benchmark configuration 5
     bsz, mm, kk = 65536, 27, 128
     x = torch.randn(bsz * mm * kk, device="cuda").to(torch.float16)
@@ -546,6 +549,21 @@ def run_extras(R, O, np, torch, args, counters, clocks, cus):
         a_mib = gm * gk * av.element_size() >> 20
         hbm_case(name, ms, (gm * gk + gm + gk) * av.element_size(), ok, cache_note % a_mib if a_mib <= 512 else None)
         del av, xv, yv
+    # K split over several workgroups per block of rows (r355_gemv_ws): a col-major A with few rows, whose plain launch has
+    # eight workgroups, and a row count just above what fills the CUs (260 blocks of 64 rows)
+    for name, gm, gk in (("gemv_f32_col_splitk_256x1048576", 256, 1048576), ("gemv_f32_col_splitk_16640x16384", 16640, 16384)):
+        av = torch.rand(gm * gk, device="cuda") * 2 - 1
+        xv = torch.rand(gk, device="cuda") * 2 - 1
+        yv = torch.empty(gm, device="cuda")
+        need = R.gemv_workspace_bytes(R.COL_MAJOR, gm, gk, 4)
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
+        ms = event_ms(lambda: R.gemv(R.COL_MAJOR, gm, gk, av, xv, None, yv, 1.0, 0.0, workspace=ws))
+        rows = torch.arange(0, gm, gm // 64, device="cuda")
+        want = av.view(gk, gm).t()[rows].double() @ xv.double()
+        ok = need > 0 and bool(((yv[rows].double() - want).abs() <= 1e-4 * (want.abs() + 1.0)).all())
+        hbm_case(name, ms, (gm * gk + gm + gk) * 4, ok, "plain r355_gemv on this shape: %.4f ms" % event_ms(
+            lambda: R.gemv(R.COL_MAJOR, gm, gk, av, xv, None, yv, 1.0, 0.0)))
+        del av, xv, yv, ws
     return out
 
 

@@ -197,6 +197,24 @@ int r355_dgemv(int32_t layout_a, uint32_t m, uint32_t k, const double* a, uint32
                const double* y_in, double* y_out, double alpha, double beta, void* stream);
 
 /*
+ * The same products with K split over several workgroups per block of rows, for shapes that leave most CUs idle
+ * with one workgroup per block: a col-major A with few rows (256 x 262144) or a row count just above a multiple of
+ * what fills the CUs (8256 rows), a row-major A with few very long rows.  The splits' partial sums go to `workspace`
+ * (the caller's device memory, 16-byte aligned; its contents before the call do not matter) and a second kernel adds
+ * them in split order, so the result depends on the shape alone, never on scheduling.
+ * r355_gemv_workspace_bytes: what the split form wants for a shape (elem_bytes 4: f32, 8: f64); 0 where the plain
+ * kernels do as well.  With a null or smaller workspace r355_gemv_ws / r355_dgemv_ws run the plain kernels
+ * (the same as r355_gemv / r355_dgemv).  No counterpart in the reference (its sample has one kernel for all shapes).
+ */
+size_t r355_gemv_workspace_bytes(int32_t layout_a, uint32_t m, uint32_t k, uint32_t elem_bytes);
+int    r355_gemv_ws(int32_t layout_a, uint32_t m, uint32_t k, const float* a, uint32_t lda, const float* x,
+                    const float* y_in, float* y_out, float alpha, float beta, void* workspace, size_t workspace_bytes,
+                    void* stream);
+int    r355_dgemv_ws(int32_t layout_a, uint32_t m, uint32_t k, const double* a, uint32_t lda, const double* x,
+                     const double* y_in, double* y_out, double alpha, double beta, void* workspace,
+                     size_t workspace_bytes, void* stream);
+
+/*
  * Host-side 2:4 compressor for a row-major m x k matrix of 1-byte elements (host pointers); m % 16 == 0, k % 128 == 0.
  * Every aligned group of 4 along k keeps 2 elements (in position order) and a nibble idx0 | idx1 << 2 (idx0 < idx1).
  * The storage is K-blocked so that a kernel's share of one K stage is contiguous and in matrix-instruction order.

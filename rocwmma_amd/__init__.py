@@ -25,7 +25,7 @@ DTYPE_BYTES = {F16: 2, BF16: 2, E4M3: 1, I8: 1, F32: 4, I32: 4, F64: 8, E5M2: 1}
 
 EXPORTS = [
     "r355_gemm", "r355_gemm_noalloc", "r355_gemm_query", "r355_gemm_timed", "r355_dlrm_fwd", "r355_dlrm_fwd_timed",
-    "r355_dlrm_bwd", "r355_gemv", "r355_gemv_timed", "r355_dgemv", "r355_compress_24", "r355_decompress_24", "r355_compress_24_16", "r355_decompress_24_16",
+    "r355_dlrm_bwd", "r355_gemv", "r355_gemv_timed", "r355_dgemv", "r355_gemv_workspace_bytes", "r355_gemv_ws", "r355_dgemv_ws", "r355_compress_24", "r355_decompress_24", "r355_compress_24_16", "r355_decompress_24_16",
     "r355_get_device_info", "r355_last_error", "r355_version",
 ]
 
@@ -95,6 +95,9 @@ def lib():
         L.r355_gemv.argtypes = [i32, u32, u32, vp, u32, vp, vp, vp, f32, f32, vp]
         L.r355_gemv_timed.argtypes = [i32, u32, u32, vp, u32, vp, vp, vp, f32, f32, vp, ctypes.c_int, ctypes.c_int, fp]
         L.r355_dgemv.argtypes = [i32, u32, u32, vp, u32, vp, vp, vp, ctypes.c_double, ctypes.c_double, vp]
+        L.r355_gemv_workspace_bytes.argtypes, L.r355_gemv_workspace_bytes.restype = [i32, u32, u32, u32], ctypes.c_size_t
+        L.r355_gemv_ws.argtypes = [i32, u32, u32, vp, u32, vp, vp, vp, f32, f32, vp, ctypes.c_size_t, vp]
+        L.r355_dgemv_ws.argtypes = [i32, u32, u32, vp, u32, vp, vp, vp, ctypes.c_double, ctypes.c_double, vp, ctypes.c_size_t, vp]
         L.r355_compress_24.argtypes = [vp, u32, u32, vp, vp]
         L.r355_decompress_24.argtypes = [vp, vp, u32, u32, vp]
         L.r355_compress_24_16.argtypes = [vp, u32, u32, vp, vp]
@@ -227,17 +230,33 @@ def dlrm_bwd(dtype, x, upstream, mlp_grad, in_grad, m, k, batch, stream=None):
                                _stream_handle(stream)))
 
 
-def gemv(layout_a, m, k, a, x, y_in, y_out, alpha=1.0, beta=0.0, lda=None, stream=None):
-    lda = lda if lda is not None else default_ld(m, k, layout_a)
-    _check(lib().r355_gemv(layout_a, m, k, _ptr(a), lda, _ptr(x), _ptr(y_in), _ptr(y_out), alpha, beta,
-                           _stream_handle(stream)))
+def gemv_workspace_bytes(layout_a, m, k, elem_bytes=4):
+    """Bytes of workspace the split-K form of the GEMV wants for a shape (0: the plain kernels serve it)."""
+    return int(lib().r355_gemv_workspace_bytes(layout_a, m, k, elem_bytes))
 
 
-def dgemv(layout_a, m, k, a, x, y_in, y_out, alpha=1.0, beta=0.0, lda=None, stream=None):
-    """f64 GEMV (the reference's simple_dgemv sample)."""
+def gemv(layout_a, m, k, a, x, y_in, y_out, alpha=1.0, beta=0.0, lda=None, stream=None, workspace=None, workspace_bytes=None):
+    """workspace (device memory; workspace_bytes defaults to its size): r355_gemv_ws, which splits K where that pays."""
     lda = lda if lda is not None else default_ld(m, k, layout_a)
-    _check(lib().r355_dgemv(layout_a, m, k, _ptr(a), lda, _ptr(x), _ptr(y_in), _ptr(y_out), alpha, beta,
-                            _stream_handle(stream)))
+    if workspace is None:
+        _check(lib().r355_gemv(layout_a, m, k, _ptr(a), lda, _ptr(x), _ptr(y_in), _ptr(y_out), alpha, beta,
+                               _stream_handle(stream)))
+    else:
+        nbytes = workspace_bytes if workspace_bytes is not None else workspace.numel() * workspace.element_size()
+        _check(lib().r355_gemv_ws(layout_a, m, k, _ptr(a), lda, _ptr(x), _ptr(y_in), _ptr(y_out), alpha, beta,
+                                  _ptr(workspace), nbytes, _stream_handle(stream)))
+
+
+def dgemv(layout_a, m, k, a, x, y_in, y_out, alpha=1.0, beta=0.0, lda=None, stream=None, workspace=None, workspace_bytes=None):
+    """f64 GEMV (the reference's simple_dgemv sample); workspace as for gemv."""
+    lda = lda if lda is not None else default_ld(m, k, layout_a)
+    if workspace is None:
+        _check(lib().r355_dgemv(layout_a, m, k, _ptr(a), lda, _ptr(x), _ptr(y_in), _ptr(y_out), alpha, beta,
+                                _stream_handle(stream)))
+    else:
+        nbytes = workspace_bytes if workspace_bytes is not None else workspace.numel() * workspace.element_size()
+        _check(lib().r355_dgemv_ws(layout_a, m, k, _ptr(a), lda, _ptr(x), _ptr(y_in), _ptr(y_out), alpha, beta,
+                                   _ptr(workspace), nbytes, _stream_handle(stream)))
 
 
 def gemv_timed(layout_a, m, k, a, x, y_in, y_out, alpha, beta, warmup, iters, lda=None, stream=None):

@@ -26,7 +26,9 @@ namespace
     // (256-byte runs) is taken when the rows suffice for that.  Every lane sums its columns in increasing order; the
     // COL_WAVES * 64 / RL partial sums of a row meet in LDS and are added in a fixed order, so the result does not depend
     // on scheduling.  STREAM as in the row-major kernel.
-    template <typename T, uint32_t RL, uint32_t COL_WAVES, bool STREAM>
+    // SPLIT: workgroup (b, s) of a two-dimensional grid sums columns [s kPer, (s + 1) kPer) only and leaves its rows' sums,
+    // unscaled, in row s of a [splits][m] array (yOut) for gemvAddSplits.
+    template <typename T, uint32_t RL, uint32_t COL_WAVES, bool STREAM, bool SPLIT = false>
     __global__ void __launch_bounds__(COL_WAVES * 64) gemvColMajor(uint32_t m,
                                                                   uint32_t k,
                                                                   const T* a,
@@ -35,7 +37,8 @@ namespace
                                                                   const T* yIn,
                                                                   T*       yOut,
                                                                   T        alpha,
-                                                                  T        beta)
+                                                                  T        beta,
+                                                                  uint32_t kPer)
     {
         constexpr uint32_t V = 16u / sizeof(T), ROWS = RL * V, CL = 64u / RL, COLS = COL_WAVES * CL, DEPTH = 8;
         using VecT = T __attribute__((ext_vector_type(V)));
@@ -56,8 +59,9 @@ namespace
                 else
                     return *reinterpret_cast<const VecT*>(at);
             };
-            uint32_t kk = wave * CL + c;
-            for(; kk + (DEPTH - 1u) * COLS < k; kk += DEPTH * COLS)
+            const uint32_t kEnd = SPLIT ? (k - blockIdx.y * kPer < kPer ? k : (blockIdx.y + 1u) * kPer) : k;
+            uint32_t       kk   = (SPLIT ? blockIdx.y * kPer : 0u) + wave * CL + c;
+            for(; kk + (DEPTH - 1u) * COLS < kEnd; kk += DEPTH * COLS)
             {
                 VecT v[DEPTH];
                 T    xv[DEPTH];
@@ -73,7 +77,7 @@ namespace
                     for(uint32_t e = 0; e < V; ++e)
                         acc[e] += v[u][e] * xv[u];
             }
-            for(; kk < k; kk += COLS)
+            for(; kk < kEnd; kk += COLS)
             {
                 const VecT v  = fetch(p + (uint64_t)kk * lda);
                 const T    xv = x[kk];
@@ -95,9 +99,33 @@ namespace
 #pragma unroll
                 for(uint32_t w = 0; w < COLS; ++w)
                     sum += partial[w][threadIdx.x];
-                yOut[row] = beta != T(0) ? alpha * sum + beta * yIn[row] : alpha * sum;
+                if constexpr(SPLIT)
+                    yOut[(uint64_t)blockIdx.y * m + row] = sum;
+                else
+                    yOut[row] = beta != T(0) ? alpha * sum + beta * yIn[row] : alpha * sum;
             }
         }
+    }
+
+    // Second kernel of the split forms: y = alpha * (sum of the splits' partial sums, in split order) + beta * y.
+    template <typename T>
+    __global__ void __launch_bounds__(THREADS) gemvAddSplits(uint32_t m, uint32_t splits, const T* partial, const T* yIn, T* yOut, T alpha, T beta)
+    {
+        const uint32_t row = blockIdx.x * THREADS + threadIdx.x;
+        if(row >= m)
+            return;
+        T sum = T(0);
+        for(uint32_t s0 = 0; s0 < splits; s0 += 8u) // (eight requests under way per thread)
+        {
+            T v[8];
+#pragma unroll
+            for(uint32_t u = 0; u < 8u; ++u)
+                v[u] = s0 + u < splits ? partial[(uint64_t)(s0 + u) * m + row] : T(0);
+#pragma unroll
+            for(uint32_t u = 0; u < 8u; ++u)
+                sum += v[u];
+        }
+        yOut[row] = beta != T(0) ? alpha * sum + beta * yIn[row] : alpha * sum;
     }
 
     // STREAM: A does not fit the 256 MiB memory-side cache, so nothing of it can be there from an earlier call or be wanted
@@ -180,7 +208,9 @@ namespace
     // STREAM: A lies beyond the memory-side cache and is read with nontemporal loads; a smaller one (few very long rows
     // of a matrix that is multiplied again and again) keeps ordinary loads so that the next call finds it there, as in
     // gemvRowMajor / gemvColMajor.
-    template <typename T, uint32_t WAVES, uint32_t RB = SHARED_ROWS, bool STREAM = true>
+    // SPLIT: workgroup (b, s) takes elements [s kPer, (s + 1) kPer) of its rows only (kPer a multiple of the slice) and
+    // leaves the sums, unscaled, in row s of a [splits][m] array (yOut) for gemvAddSplits.
+    template <typename T, uint32_t WAVES, uint32_t RB = SHARED_ROWS, bool STREAM = true, bool SPLIT = false>
     __global__ void __launch_bounds__(WAVES * 64u) gemvRowMajorShared(uint32_t m,
                                                                       uint32_t k,
                                                                       const T* a,
@@ -189,7 +219,8 @@ namespace
                                                                       const T* yIn,
                                                                       T*       yOut,
                                                                       T        alpha,
-                                                                      T        beta)
+                                                                      T        beta,
+                                                                      uint32_t kPer)
     {
         constexpr uint32_t V = 16u / sizeof(T);
         constexpr uint32_t SLICE = WAVES * 64u * 16u; // bytes one load instruction of the whole workgroup covers
@@ -197,7 +228,9 @@ namespace
         using VecT               = T __attribute__((ext_vector_type(V)));
         __shared__ T   partial[WAVES][RB];
         const uint32_t lane = threadIdx.x & 63u, w = threadIdx.x / 64u;
-        const uint32_t row0 = blockIdx.x * RB, kBytes = k * (uint32_t)sizeof(T);
+        const uint32_t row0 = blockIdx.x * RB;
+        const uint32_t kBeg = SPLIT ? blockIdx.y * kPer : 0u; // (wave-uniform)
+        const uint32_t kBytes = (SPLIT ? (k - kBeg < kPer ? k - kBeg : kPer) : k) * (uint32_t)sizeof(T);
         // One buffer per row and one for x, each k elements long: what a load asks for beyond that comes back as zero, so
         // a row that does not fill its last slice needs no separate tail, and a row past m (a buffer of no bytes) adds
         // nothing.  The rows are wave-uniform: their descriptors stay in scalar registers.
@@ -208,17 +241,39 @@ namespace
             return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>((static_cast<uint64_t>(hi) << 32) | lo), 0,
                                                      static_cast<int>(__builtin_amdgcn_readfirstlane(bytes)), 0x00020000);
         };
-        const __amdgpu_buffer_rsrc_t xr = buffer(x, kBytes);
+        const __amdgpu_buffer_rsrc_t xr = buffer(x + kBeg, kBytes);
         __amdgpu_buffer_rsrc_t       rows[RB];
         T                            acc[RB];
 #pragma unroll
         for(uint32_t r = 0; r < RB; ++r)
         {
-            rows[r] = buffer(a + (uint64_t)(row0 + r < m ? row0 + r : 0u) * lda, row0 + r < m ? kBytes : 0u);
+            rows[r] = buffer(a + (uint64_t)(row0 + r < m ? row0 + r : 0u) * lda + kBeg, row0 + r < m ? kBytes : 0u);
             acc[r]  = T(0);
         }
         const uint32_t mine = (w * 64u + lane) * 16u;
-        for(uint32_t kc = 0; kc < kBytes; kc += SLICE)
+        uint32_t       kc   = 0;
+        if constexpr(RB == 1u)
+        {
+            // a single row per workgroup: nothing but this row's slices to overlap, so several of them are requested
+            // before the first is used
+            constexpr uint32_t AHEAD = 4;
+            for(; kc + (AHEAD - 1u) * SLICE < kBytes; kc += AHEAD * SLICE)
+            {
+                VecT v[AHEAD], xv[AHEAD];
+#pragma unroll
+                for(uint32_t u = 0; u < AHEAD; ++u)
+                    v[u] = __builtin_bit_cast(VecT, __builtin_amdgcn_raw_buffer_load_b128(rows[0], mine, kc + u * SLICE, NT));
+#pragma unroll
+                for(uint32_t u = 0; u < AHEAD; ++u)
+                    xv[u] = __builtin_bit_cast(VecT, __builtin_amdgcn_raw_buffer_load_b128(xr, mine, kc + u * SLICE, 0));
+#pragma unroll
+                for(uint32_t u = 0; u < AHEAD; ++u)
+#pragma unroll
+                    for(uint32_t e = 0; e < V; ++e)
+                        acc[0] += v[u][e] * xv[u][e];
+            }
+        }
+        for(; kc < kBytes; kc += SLICE)
         {
             const VecT xv = __builtin_bit_cast(VecT, __builtin_amdgcn_raw_buffer_load_b128(xr, mine, kc, 0));
             VecT       v  = __builtin_bit_cast(VecT, __builtin_amdgcn_raw_buffer_load_b128(rows[0], mine, kc, NT));
@@ -252,13 +307,79 @@ namespace
             for(uint32_t i = 0; i < WAVES; ++i)
                 sum += partial[i][threadIdx.x];
             const uint32_t row = row0 + threadIdx.x;
-            yOut[row]          = beta != T(0) ? alpha * sum + beta * yIn[row] : alpha * sum;
+            if constexpr(SPLIT)
+                yOut[(uint64_t)blockIdx.y * m + row] = sum;
+            else
+                yOut[row] = beta != T(0) ? alpha * sum + beta * yIn[row] : alpha * sum;
         }
+    }
+
+    // Lanes side by side on one column in the split form of the col-major kernel.  With K divided there are workgroups
+    // enough whatever the rows per workgroup, so the runs can be longer than the plain kernel's: 512 bytes from 256
+    // 16-byte pieces per column on (f32, 256 MiB of A: 1024 x 65536 0.79 of the HBM peak against 0.75 with 128-byte runs,
+    // 2048 x 32768 0.83 against 0.76, 16640 x 16384 0.83 against 0.65; 1 KiB runs: 0.72, 0.78, 0.78); shorter columns
+    // keep 128-byte runs (256 x 262144: 0.69 against 0.61 and 0.51).
+    template <typename T>
+    uint32_t splitRunLanes(uint32_t m)
+    {
+        constexpr uint32_t V = 16u / sizeof(T);
+        return m >= 256u * V ? 32u : 8u;
+    }
+
+    // Splits of K for a shape, 1 = the plain kernels serve it.
+    // Col-major A: a workgroup per block of 32 or 64 rows (f32) leaves CUs idle when the blocks are few, or just over a
+    // multiple of the CU count (8256 rows: 258 blocks, two of them in a round of their own).  The plain launch is priced
+    // as rounds over the CUs - a workgroup streams about 50 GB/s on its own, all CUs together 7.2 TB/s - and the split
+    // form as A at 7.0 TB/s plus 3 us for the second launch; measured (f32): 4096^2 12.8 us plain / 13.3 split,
+    // 4096 x 16384 42.4 / 40.2, 8256 x 8192 67.5 / 46.3, 12288 x 8192 77.0 / 60.0, 2048 x 32768 78.3 / 40.5,
+    // 256 x 262144 592 / 48.9, 64 x 1048576 2580 / 57.7, 16640 x 16384 261 / 164, 20000 x 16384 274 / 185.  K is divided into pieces of at least 1024 columns so that two
+    // (128-byte runs) or eight (512-byte runs) workgroups per CU result.
+    // Row-major A with at most half as many rows as CUs, each of 256 KiB or more: a workgroup per row leaves CUs without
+    // one (128 rows of 4 MiB: 0.46 of the HBM peak, split 0.73; 64 rows: 0.25 / 0.73; 32 rows: 0.13 / 0.71; the plain
+    // kernel is ahead with 200 rows of 1 MiB, 0.85 / 0.72, and from 256 rows on, 0.76 / 0.73); pieces of at least
+    // 128 KiB, about four workgroups per CU.
+    template <typename T>
+    uint32_t gemvSplits(int32_t layout_a, uint32_t m, uint32_t k, uint32_t& kPer)
+    {
+        constexpr uint32_t V = 16u / sizeof(T);
+        const uint32_t     cus = r355::computeUnits();
+        kPer = k;
+        uint32_t blocks, grain, perCu;
+        if(layout_a == R355_COL_MAJOR)
+        {
+            const uint32_t rows   = (m >= 16u * V * 256u ? 16u : 8u) * V; // per workgroup, as the plain launch chooses them
+            const uint32_t plain  = (m + rows - 1u) / rows, rounds = (plain + cus - 1u) / cus;
+            const double   bytes  = static_cast<double>(m) * k * sizeof(T), perGroup = static_cast<double>(rows) * k * sizeof(T);
+            const double   abreast = static_cast<double>(plain < cus ? plain : cus) * perGroup / 7.2e6; // us: all of a round's workgroups at the HBM's rate
+            const double   alone   = perGroup / 50.0e3; // us: a workgroup at its own
+            const double   tPlain  = static_cast<double>(rounds) * (abreast > alone ? abreast : alone);
+            const double   tSplit  = bytes / 7.0e6 + 3.0;
+            if(rounds > 3u || tSplit * 1.03 >= tPlain) // (many rounds even out by themselves as workgroups end at different times)
+                return 1u;
+            const uint32_t lanes = splitRunLanes<T>(m);
+            blocks = (m + lanes * V - 1u) / (lanes * V), grain = 1024u, perCu = lanes == 8u ? 2u : 8u;
+        }
+        else
+        {
+            const uint64_t rowBytes = (uint64_t)k * sizeof(T);
+            if(m > cus / 2u || rowBytes < (256u << 10) || rowBytes >= (1ull << 31))
+                return 1u;
+            blocks = m, grain = (128u << 10) / (uint32_t)sizeof(T), perCu = 4u;
+        }
+        uint32_t splits = (perCu * cus + blocks - 1u) / blocks;
+        if(splits > k / grain)
+            splits = k / grain;
+        if(splits > 256u)
+            splits = 256u;
+        if(splits < 2u)
+            return 1u;
+        kPer = ((k + splits - 1u) / splits + grain - 1u) / grain * grain; // whole grains: every split starts on a slice boundary
+        return (k + kPer - 1u) / kPer;
     }
 
     template <typename T>
     int gemvLaunch(int32_t layout_a, uint32_t m, uint32_t k, const T* a, uint32_t lda, const T* x, const T* y_in, T* y_out,
-                   T alpha, T beta, void* stream)
+                   T alpha, T beta, void* stream, void* workspace = nullptr, size_t workspaceBytes = 0)
     {
         constexpr uint32_t V = 16u / sizeof(T);
         if(!a || !x || !y_out || (beta != T(0) && !y_in))
@@ -269,8 +390,15 @@ namespace
             return r355::fail(R355_ERR_BAD_SIZE, "gemv: m=%u and k=%u must be multiples of %u", m, k, V);
         if(!r355::aligned(a, 16) || lda % V || !r355::aligned(x, 16) || !r355::aligned(y_out, 16))
             return r355::fail(R355_ERR_MISALIGNED, "gemv: a, x, y need 16-byte alignment and lda %% %u == 0", V);
+        if(workspace && !r355::aligned(workspace, 16))
+            return r355::fail(R355_ERR_MISALIGNED, "gemv: the workspace needs 16-byte alignment");
         hipStream_t s = static_cast<hipStream_t>(stream);
         r355::beginCall();
+        // K split over several workgroups per block of rows when the shape calls for it and the workspace holds the partial sums
+        uint32_t       kPer   = k;
+        const uint32_t splits = (layout_a == R355_COL_MAJOR || layout_a == R355_ROW_MAJOR) && workspace ? gemvSplits<T>(layout_a, m, k, kPer) : 1u;
+        const bool     split  = splits > 1u && (uint64_t)splits * m * sizeof(T) <= workspaceBytes;
+        T*             parts  = static_cast<T*>(workspace);
         if(layout_a == R355_COL_MAJOR)
         {
             if(lda < m)
@@ -278,16 +406,24 @@ namespace
             const bool stream = (uint64_t)k * lda * sizeof(T) > (256ull << 20);
             auto       go     = [&](auto rl, auto waves) {
                 constexpr uint32_t RL = decltype(rl)::value, ROWS = RL * V, WAVES = decltype(waves)::value;
-                const dim3         grid((m + ROWS - 1u) / ROWS), block(WAVES * 64);
-                if(stream)
-                    hipLaunchKernelGGL((gemvColMajor<T, RL, WAVES, true>), grid, block, 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
+                const dim3         grid((m + ROWS - 1u) / ROWS, split ? splits : 1u), block(WAVES * 64);
+                if(split && stream)
+                    hipLaunchKernelGGL((gemvColMajor<T, RL, WAVES, true, true>), grid, block, 0, s, m, k, a, lda, x, y_in, parts, alpha, beta, kPer);
+                else if(split)
+                    hipLaunchKernelGGL((gemvColMajor<T, RL, WAVES, false, true>), grid, block, 0, s, m, k, a, lda, x, y_in, parts, alpha, beta, kPer);
+                else if(stream)
+                    hipLaunchKernelGGL((gemvColMajor<T, RL, WAVES, true>), grid, block, 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k);
                 else
-                    hipLaunchKernelGGL((gemvColMajor<T, RL, WAVES, false>), grid, block, 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
+                    hipLaunchKernelGGL((gemvColMajor<T, RL, WAVES, false>), grid, block, 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k);
             };
             // 256-byte runs once the rows give every CU a workgroup with them (8192^2 f32: 0.0415 ms against 0.0374 with
             // 128-byte runs and twice the workgroups; 16384^2: 0.151 against 0.161); sixteen waves per workgroup either way
             // (four: 0.0399 and 0.163)
-            if(m >= 16u * V * 256u)
+            if(split && splitRunLanes<T>(m) == 32u)
+                go(std::integral_constant<uint32_t, 32>{}, std::integral_constant<uint32_t, 16>{});
+            else if(split)
+                go(std::integral_constant<uint32_t, 8>{}, std::integral_constant<uint32_t, 16>{});
+            else if(m >= 16u * V * 256u)
                 go(std::integral_constant<uint32_t, 16>{}, std::integral_constant<uint32_t, 16>{});
             else
                 go(std::integral_constant<uint32_t, 8>{}, std::integral_constant<uint32_t, 16>{});
@@ -306,20 +442,27 @@ namespace
             // waves per row instead (f32, 512 MiB of A: 512 rows 0.42 -> 0.64 of the HBM peak, 256 rows 0.23 -> 0.77, 128 rows
             // 0.12 -> 0.43; rows of 512 KiB: 640 rows 0.52 -> 0.67, 768 rows 0.61 -> 0.76, 896 rows even; a wave per row is
             // ahead again from there on, and from 768 rows of 128 or 256 KiB)
-            if((m <= 512u || (m <= 768u && rowBytes >= (512u << 10))) && rowBytes >= (128u << 10) && rowBytes < (1ull << 31))
+            if(split)
             {
                 if(stream)
-                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16, 1, true>), dim3(m), dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16, 1, true, true>), dim3(m, splits), dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, parts, alpha, beta, kPer);
                 else
-                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16, 1, false>), dim3(m), dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16, 1, false, true>), dim3(m, splits), dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, parts, alpha, beta, kPer);
+            }
+            else if((m <= 512u || (m <= 768u && rowBytes >= (512u << 10))) && rowBytes >= (128u << 10) && rowBytes < (1ull << 31))
+            {
+                if(stream)
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16, 1, true>), dim3(m), dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k);
+                else
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16, 1, false>), dim3(m), dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k);
             }
             else if(stream && rowBytes >= (16u << 10) && rowBytes < (1ull << 31) && m >= SHARED_ROWS * 512u)
             {
                 const dim3 blocks((m + SHARED_ROWS - 1u) / SHARED_ROWS);
                 if(rowBytes < (128u << 10))
-                    hipLaunchKernelGGL((gemvRowMajorShared<T, 8>), blocks, dim3(8 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 8>), blocks, dim3(8 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k);
                 else
-                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16>), blocks, dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16>), blocks, dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k);
             }
             else if(stream)
                 hipLaunchKernelGGL((gemvRowMajor<T, true>), grid, dim3(THREADS), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
@@ -328,9 +471,32 @@ namespace
         }
         else
             return r355::fail(R355_ERR_BAD_ARG, "gemv: unknown layout");
+        if(split)
+            hipLaunchKernelGGL(gemvAddSplits<T>, dim3((m + THREADS - 1u) / THREADS), dim3(THREADS), 0, s, m, splits, parts, y_in, y_out, alpha, beta);
         return r355::checkLaunch("gemv");
     }
 } // namespace
+
+extern "C" size_t r355_gemv_workspace_bytes(int32_t layout_a, uint32_t m, uint32_t k, uint32_t elem_bytes)
+{
+    if((layout_a != R355_COL_MAJOR && layout_a != R355_ROW_MAJOR) || m == 0 || k == 0)
+        return 0;
+    uint32_t       kPer   = k;
+    const uint32_t splits = elem_bytes == 8u ? gemvSplits<double>(layout_a, m, k, kPer) : gemvSplits<float>(layout_a, m, k, kPer);
+    return splits > 1u ? (size_t)splits * m * (elem_bytes == 8u ? 8u : 4u) : 0;
+}
+
+extern "C" int r355_gemv_ws(int32_t layout_a, uint32_t m, uint32_t k, const float* a, uint32_t lda, const float* x,
+                            const float* y_in, float* y_out, float alpha, float beta, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return gemvLaunch<float>(layout_a, m, k, a, lda, x, y_in, y_out, alpha, beta, stream, workspace, workspace_bytes);
+}
+
+extern "C" int r355_dgemv_ws(int32_t layout_a, uint32_t m, uint32_t k, const double* a, uint32_t lda, const double* x,
+                             const double* y_in, double* y_out, double alpha, double beta, void* workspace, size_t workspace_bytes, void* stream)
+{
+    return gemvLaunch<double>(layout_a, m, k, a, lda, x, y_in, y_out, alpha, beta, stream, workspace, workspace_bytes);
+}
 
 extern "C" int r355_gemv(int32_t layout_a, uint32_t m, uint32_t k, const float* a, uint32_t lda, const float* x,
                          const float* y_in, float* y_out, float alpha, float beta, void* stream)

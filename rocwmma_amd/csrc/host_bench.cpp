@@ -10,7 +10,7 @@
 //                    [--zero 1]     all-zero operands (no switching power: the engine clock stays at its maximum)
 //                    [--ldpad E]    lda and ldb grow by E elements (power-of-two strides cost L2 efficiency)
 //   host_bench dlrm  [--type f16|bf16|f32] [--bwd 1] [--batch B --m M --k K] [--warmup W --iters I]
-//   host_bench gemv  [--m M --k K --layout n|t]
+//   host_bench gemv  [--m M --k K --layout n|t] [--split 1]   (--split 1: r355_gemv_ws with the workspace its query asks for)
 //   host_bench copy  [--bytes N]      plain device copy of known size (counter calibration)
 //   host_bench mix                    a bare kernel at the DLRM forward's read / write mix (7 KiB read, 1 KiB written per
 //                                     unit and wave, 65536 units): what plain streaming code reaches at that mix
@@ -489,7 +489,7 @@ int main(int argc, char** argv)
     }
     const std::string op = argv[1];
     std::string       type = "f16", out = "", layout = "nt", kernel = "auto";
-    bool              sparse = false, itersSet = false, bwd = false, zeroFill = false;
+    bool              sparse = false, itersSet = false, bwd = false, zeroFill = false, split = false;
     uint32_t          m = 8192, n = 8192, k = 8192, batch = 65536, ldpad = 0;
     bool              mSet = false, kSet = false;
     int               warmup = 2, iters = 10;
@@ -509,6 +509,7 @@ int main(int argc, char** argv)
         else if(a == "--warmup") warmup = atoi(v.c_str());
         else if(a == "--iters") iters = atoi(v.c_str()), itersSet = true;
         else if(a == "--sparse") sparse = atoi(v.c_str()) != 0;
+        else if(a == "--split") split = atoi(v.c_str()) != 0;
         else if(a == "--bwd") bwd = atoi(v.c_str()) != 0;
         else if(a == "--zero") zeroFill = atoi(v.c_str()) != 0;
         else if(a == "--workspace") workspaceMiB = strtoull(v.c_str(), nullptr, 10);
@@ -673,17 +674,43 @@ int main(int argc, char** argv)
         HIP_OK(hipMalloc(&dy, (size_t)m * 4));
         HIP_OK(hipMemcpy(da, ha.data(), ha.size(), hipMemcpyHostToDevice));
         HIP_OK(hipMemcpy(dx, hx.data(), hx.size(), hipMemcpyHostToDevice));
-        const int lay = layout[0] == 't' ? R355_ROW_MAJOR : R355_COL_MAJOR;
-        if(r355_gemv_timed(lay, m, k, (const float*)da, lay == R355_ROW_MAJOR ? k : m, (const float*)dx, nullptr,
-                           (float*)dy, 1.0f, 0.0f, nullptr, warmup, iters, &ms)
-           != R355_OK)
+        const int    lay = layout[0] == 't' ? R355_ROW_MAJOR : R355_COL_MAJOR;
+        const size_t wsBytes = split ? r355_gemv_workspace_bytes(lay, m, k, 4) : 0;
+        if(wsBytes)
+        {
+            void* ws = nullptr;
+            HIP_OK(hipMalloc(&ws, wsBytes));
+            hipEvent_t e0, e1;
+            HIP_OK(hipEventCreate(&e0));
+            HIP_OK(hipEventCreate(&e1));
+            for(int it = 0; it < warmup + iters; ++it)
+            {
+                if(it == warmup)
+                    HIP_OK(hipEventRecord(e0));
+                if(r355_gemv_ws(lay, m, k, (const float*)da, lay == R355_ROW_MAJOR ? k : m, (const float*)dx, nullptr, (float*)dy, 1.0f,
+                                0.0f, ws, wsBytes, nullptr)
+                   != R355_OK)
+                {
+                    fprintf(stderr, "%s\n", r355_last_error());
+                    return 1;
+                }
+            }
+            HIP_OK(hipEventRecord(e1));
+            HIP_OK(hipEventSynchronize(e1));
+            HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+            ms /= (float)iters;
+        }
+        else if(r355_gemv_timed(lay, m, k, (const float*)da, lay == R355_ROW_MAJOR ? k : m, (const float*)dx, nullptr,
+                                (float*)dy, 1.0f, 0.0f, nullptr, warmup, iters, &ms)
+                != R355_OK)
         {
             fprintf(stderr, "%s\n", r355_last_error());
             return 1;
         }
         const double byts = (double)m * k * 4.0 + (double)(m + k) * 4.0;
-        printf("{\"op\": \"gemv\", \"m\": %u, \"k\": %u, \"ms\": %.4f, \"gbps\": %.1f, \"frac_hbm_peak\": %.4f}\n", m, k,
-               ms, byts / ms / 1e6, byts / ms / 1e6 / 8000.0);
+        printf("{\"op\": \"gemv\", \"m\": %u, \"k\": %u, \"layout\": \"%s\", \"workspace_bytes\": %zu, \"ms\": %.4f, \"gbps\": %.1f, "
+               "\"frac_hbm_peak\": %.4f}\n",
+               m, k, lay == R355_ROW_MAJOR ? "row" : "col", wsBytes, ms, byts / ms / 1e6, byts / ms / 1e6 / 8000.0);
     }
     else if(op == "mfma")
     {

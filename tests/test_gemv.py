@@ -142,3 +142,98 @@ def _shared_rows_case(dtype, m, k, pad, streamed=True):
         fn(O.ROW, m, k, ai, xi, None, y, 1.0, 0.0, lda=lda)
         torch.cuda.synchronize()
         assert torch.equal(y, ai.view(m, lda)[:, :k] @ xi)
+
+
+# ---- K split over several workgroups per block of rows (r355_gemv_ws / r355_dgemv_ws)
+
+SPLIT_SHAPES = [  # layout, m, k: each one a shape the query wants a workspace for
+    (O.COL, 256, 32768 + 260),   # few rows: 8 blocks of rows, 32 splits, the last one short and off the unrolled trip
+    (O.COL, 8256, 2048 + 8),     # 258 blocks: a row count just above what fills the CUs; 2 splits
+    (O.COL, 4, 16384),           # a single partial block of rows
+    (O.COL, 16384 + 576, 2052),  # the 256-byte-run kernel (64 rows per workgroup), 265 blocks
+    (O.ROW, 128, 65536 + 4100),  # few long rows: a workgroup per (row, split), the last split short
+    (O.ROW, 20, 262144),
+]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+@pytest.mark.parametrize("layout,m,k", SPLIT_SHAPES)
+def test_gemv_split_k_vs_oracle(dtype, layout, m, k):
+    """The split form against the oracle's GEMM with n = 1 (same bound as the plain kernels), with padded leading
+    dimension, alpha and beta, a workspace full of NaN bit patterns before the call and guard bytes behind it; twice
+    in a row: bit-identical (the partial sums are added in split order)."""
+    import torch
+
+    f64 = dtype == "f64"
+    if f64 and layout == O.ROW:
+        k = k // 2 + 2  # (rows of the same byte length)
+    nt, ot, es = (np.float64, O.F64, 8) if f64 else (np.float32, O.F32, 4)
+    need = R.gemv_workspace_bytes(layout, m, k, es)
+    assert need > 0 and need % (m * es) == 0
+    pad = 4
+    lda = (k if layout == O.ROW else m) + pad
+    a = O.uniform_pm1(21, m * k).astype(nt)
+    x, y = O.uniform_pm1(22, k).astype(nt), O.uniform_pm1(23, m).astype(nt)
+    want = O.gemm(ot, ot, layout, O.COL, O.COL, O.COL, m, 1, k, a, x, y, 2.0, -1.0)
+    A = O.as_matrix(a, m, k, layout)
+    padded = np.full((m, lda) if layout == O.ROW else (k, lda), 7.0, dtype=nt)
+    if layout == O.ROW:
+        padded[:, :k] = A
+    else:
+        padded[:, :m] = A.T
+    da, dx, dy = to_device(padded.ravel()), to_device(x), to_device(y)
+    guard = 4096
+    ws = device_filled((need + guard) // 4, np.float32, 0xFF)
+    call = R.dgemv if f64 else R.gemv
+    outs = []
+    for _ in range(2):
+        dout = device_filled(m, nt, 0xFF)
+        call(layout, m, k, da, dx, dy, dout, 2.0, -1.0, lda=lda, workspace=ws, workspace_bytes=need)
+        outs.append(to_host(dout, nt))
+    torch.cuda.synchronize()
+    assert np.all(to_host(ws, np.float32).view(np.uint8)[need:] == 0xFF), "bytes behind the workspace were written"
+    got = outs[0]
+    assert np.array_equal(outs[0].view(np.uint8), outs[1].view(np.uint8))
+    eps = 1.2e-16 if f64 else 6e-8
+    bound = (np.abs(A.astype(np.float64)) @ np.abs(x.astype(np.float64))) * 2.0 * k * eps + np.abs(y) * 4 * eps + (1e-15 if f64 else 1e-6)
+    assert np.all(np.abs(got.astype(np.float64) - want.astype(np.float64)) <= bound)
+    exact = 2.0 * (A.astype(np.float64) @ x.astype(np.float64)) - y.astype(np.float64)
+    g = got.astype(np.float64)
+    assert np.max(np.abs(g - exact) / (np.abs(g) + np.abs(exact) + 1.0)) <= (2e-16 if f64 else 1e-7) * k
+    # integer-valued operands: exact in any summation order, so the split form and the plain kernel agree bit for bit
+    ai, xi = np.round(padded * 8.0), np.round(x * 8.0)
+    dai, dxi = to_device(ai.ravel()), to_device(xi)
+    plain, split = device_filled(m, nt, 0xFF), device_filled(m, nt, 0xFF)
+    call(layout, m, k, dai, dxi, None, plain, 1.0, 0.0, lda=lda)
+    call(layout, m, k, dai, dxi, None, split, 1.0, 0.0, lda=lda, workspace=ws, workspace_bytes=need)
+    assert np.array_equal(to_host(plain, nt), to_host(split, nt))
+
+
+def test_gemv_split_k_workspace_rules():
+    """The query is 0 where the plain kernels serve the shape; a workspace that is null, too small or not wanted runs the
+    plain kernel (same bits as r355_gemv); a misaligned one is an error."""
+    assert R.gemv_workspace_bytes(O.COL, 8192, 8192, 4) == 0 and R.gemv_workspace_bytes(O.ROW, 8192, 8192, 4) == 0
+    assert R.gemv_workspace_bytes(O.COL, 64, 64, 4) == 0  # too short to split
+    m, k = 256, 16384
+    need = R.gemv_workspace_bytes(O.COL, m, k, 4)
+    assert need == 16 * m * 4  # 16 splits of 1024 columns
+    a, x = O.uniform_pm1(31, m * k), O.uniform_pm1(32, k)
+    da, dx = to_device(a), to_device(x)
+    ws = device_filled(need // 4, np.float32, 0xFF)
+    plain = device_filled(m, np.float32, 0xFF)
+    R.gemv(O.COL, m, k, da, dx, None, plain)
+    for nbytes in (0, need - 4):
+        out = device_filled(m, np.float32, 0xFF)
+        R.gemv(O.COL, m, k, da, dx, None, out, workspace=ws, workspace_bytes=nbytes)
+        assert np.array_equal(to_host(out, np.float32), to_host(plain, np.float32))
+        assert np.all(to_host(ws, np.float32).view(np.uint8) == 0xFF)  # untouched
+    with pytest.raises(R.R355Error) as e:
+        R.gemv(O.COL, m, k, da, dx, None, plain, workspace=ws[4:], workspace_bytes=need - 4)
+    assert e.value.code == -4
+    # a shape the plain kernels serve: the workspace is left alone
+    out, ref = device_filled(8192, np.float32, 0xFF), device_filled(8192, np.float32, 0xFF)
+    a2, x2 = to_device(O.uniform_pm1(33, 8192 * 256)), to_device(O.uniform_pm1(34, 256))
+    R.gemv(O.COL, 8192, 256, a2, x2, None, ref)
+    R.gemv(O.COL, 8192, 256, a2, x2, None, out, workspace=ws)
+    assert np.array_equal(to_host(out, np.float32), to_host(ref, np.float32))
+    assert np.all(to_host(ws, np.float32).view(np.uint8) == 0xFF)
