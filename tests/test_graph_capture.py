@@ -57,6 +57,13 @@ def test_entry_points_replay_from_a_graph():
     mv, kv = 4100, 260
     dav, dxv, dyv = to_device(O.uniform_pm1(48, mv * kv)), to_device(O.uniform_pm1(49, kv)), to_device(O.uniform_pm1(50, mv))
     add("gemv", np.float32, mv, lambda out, s: R.gemv(O.COL, mv, kv, dav, dxv, dyv, out, 2.0, 2.0, stream=s))
+    # ... and with K split over a workspace (two kernels, no memset)
+    ms2, ks2 = 260, 4100
+    dav2, dxv2 = to_device(O.uniform_pm1(51, ms2 * ks2)), to_device(O.uniform_pm1(52, ks2))
+    need = R.gemv_workspace_bytes(O.COL, ms2, ks2, 4)
+    assert need > 0
+    wsv = device_filled(need, np.uint8, 0xA5)
+    add("gemv_split_k", np.float32, ms2, lambda out, s: R.gemv(O.COL, ms2, ks2, dav2, dxv2, None, out, 1.0, 0.0, stream=s, workspace=wsv))
 
     # eager results (this is also the first call of the no-allocation entry point on this device: its set-up is done here)
     for _, launch, out in ops:
