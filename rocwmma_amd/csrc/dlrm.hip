@@ -69,7 +69,27 @@ namespace
         return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>((static_cast<uint64_t>(hi) << 32) | lo), 0,
                                                  static_cast<int>(__builtin_amdgcn_readfirstlane(bytes)), 0x00020000);
     }
-    constexpr int NONTEMPORAL = 2; // cache-policy bits of the raw buffer builtins: nt
+    // cache-policy bits of the raw buffer builtins (2 = nt): X, the upstream gradient and the results are touched once.
+    // Measurement builds (python -m rocwmma_amd.build --variant <name> -D...): R355_DLRM_PLAIN_LOADS / R355_DLRM_PLAIN_STORES
+    // take the default policy instead.
+#ifdef R355_DLRM_PLAIN_LOADS
+    constexpr int LOAD_POLICY = 0;
+#else
+    constexpr int LOAD_POLICY = 2;
+#endif
+#ifdef R355_DLRM_PLAIN_STORES
+    constexpr int STORE_POLICY = 0;
+#else
+    constexpr int STORE_POLICY = 2;
+#endif
+    template <typename V>
+    __device__ __forceinline__ void streamStore(const V& v, V* at)
+    {
+        if constexpr(STORE_POLICY != 0)
+            __builtin_nontemporal_store(v, at);
+        else
+            *at = v;
+    }
 
     // K is a template parameter (32, 64, 128, 256): rows of X are K * 2 bytes = K / 8 chunks.
     // ROWS (28 or 32) bounds m: the LDS image of a sample holds ROWS rows, which at m <= 28 and
@@ -113,7 +133,7 @@ namespace
             const auto     src = runBuffer(in, (uint64_t)(b < batch ? b : 0u) * inBytes, b < batch ? inBytes : 0u);
 #pragma unroll
             for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
-                stash[q][j] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (j * 64u + lane) * 16u, 0, NONTEMPORAL)); // read once
+                stash[q][j] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (j * 64u + lane) * 16u, 0, LOAD_POLICY)); // read once
         }
 
 #pragma unroll
@@ -177,7 +197,7 @@ namespace
         uint16_t*      dst      = out + (uint64_t)b0 * outStride;
         const uint32_t vecs     = total / 8u;
         for(uint32_t v = tid; v < vecs; v += THREADS)
-            __builtin_nontemporal_store(reinterpret_cast<const i32x4*>(outLds)[v], reinterpret_cast<i32x4*>(dst) + v);
+            streamStore(reinterpret_cast<const i32x4*>(outLds)[v], reinterpret_cast<i32x4*>(dst) + v);
         for(uint32_t e = vecs * 8u + tid; e < total; e += THREADS)
             dst[e] = outLds[e];
     }
@@ -231,7 +251,7 @@ namespace
             const auto src   = runBuffer(in, (uint64_t)(valid ? b : 0u) * inBytes, valid ? inBytes : 0u);
 #pragma unroll
             for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
-                stash[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (j * 64u + lane) * 16u, 0, NONTEMPORAL));
+                stash[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (j * 64u + lane) * 16u, 0, LOAD_POLICY));
         };
         // sample b from its stash, which then takes the sample two steps further on
         auto process = [&](f32x4 (&stash)[MAX_CHUNKS], uint64_t b) {
@@ -313,7 +333,7 @@ namespace
             const auto dst = runBuffer(out, (uint64_t)(b < batch ? b : 0u) * outStride * 4u, b < batch ? outStride * 4u : 0u);
 #pragma unroll
             for(uint32_t e = 0; e < OUT_STEPS; ++e)
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, o[e * 64u + lane]), dst, (e * 64u + lane) * 4u, 0, NONTEMPORAL);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, o[e * 64u + lane]), dst, (e * 64u + lane) * 4u, 0, STORE_POLICY);
             __builtin_amdgcn_s_waitcnt(0xC07F); // the image is rewritten by the next sample
             __builtin_amdgcn_wave_barrier();
         };
@@ -400,7 +420,7 @@ namespace
             const auto     src = runBuffer(in, (uint64_t)(b < batch ? b : 0u) * inBytes, b < batch ? inBytes : 0u);
 #pragma unroll
             for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
-                stash[q][j] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (j * 64u + lane) * 16u, 0, NONTEMPORAL));
+                stash[q][j] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (j * 64u + lane) * 16u, 0, LOAD_POLICY));
         }
 
         // ---- upstream rows of the workgroup's samples -> LDS; zero rows m..31 of the X image
@@ -413,7 +433,7 @@ namespace
             i32x4          upv[UP_LOADS];
 #pragma unroll
             for(uint32_t j = 0; j < UP_LOADS; ++j)
-                upv[j] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (j * THREADS + tid) * 16u, 0, NONTEMPORAL));
+                upv[j] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (j * THREADS + tid) * 16u, 0, LOAD_POLICY));
 #pragma unroll
             for(uint32_t j = 0; j < UP_LOADS; ++j)
                 reinterpret_cast<i32x4*>(upLds)[j * THREADS + tid] = upv[j];
@@ -438,7 +458,7 @@ namespace
 #pragma unroll
             for(uint32_t e = 0; e < 8; ++e)
                 o.h[e] = upLds[sIdx * upStride + cc * 8u + e];
-            __builtin_nontemporal_store(o.v, reinterpret_cast<i32x4*>(mlpGrad + ((uint64_t)(b0 + sIdx) * K + cc * 8u)));
+            streamStore(o.v, reinterpret_cast<i32x4*>(mlpGrad + ((uint64_t)(b0 + sIdx) * K + cc * 8u)));
         }
 
         const uint32_t i = lane & 31u, half = lane >> 5, t16 = lane & 15u;
@@ -539,7 +559,7 @@ namespace
                 {
                     const uint32_t row = c / ROW_CHUNKS, col = c % ROW_CHUNKS;
                     const i32x4    v   = *reinterpret_cast<const i32x4*>(xw + (row * ROW_CHUNKS + (col ^ (row & SWZ_OUT))) * 16u);
-                    __builtin_nontemporal_store(v, reinterpret_cast<i32x4*>(dst + c * 16u));
+                    streamStore(v, reinterpret_cast<i32x4*>(dst + c * 16u));
                 }
             }
             __builtin_amdgcn_s_waitcnt(0xC07F);
@@ -606,10 +626,10 @@ namespace
             const auto up    = runBuffer(upstream, (uint64_t)(valid ? b : 0u) * upStride * 4u, valid ? upStride * 4u : 0u);
 #pragma unroll
             for(uint32_t j = 0; j < X_CHUNKS; ++j)
-                xs[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (j * 64u + lane) * 16u, 0, NONTEMPORAL));
+                xs[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (j * 64u + lane) * 16u, 0, LOAD_POLICY));
 #pragma unroll
             for(uint32_t j = 0; j < UP_WORDS; ++j)
-                us[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(up, (j * 64u + lane) * 4u, 0, NONTEMPORAL));
+                us[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(up, (j * 64u + lane) * 4u, 0, LOAD_POLICY));
         };
 
         auto process = [&](uint64_t b) {
@@ -630,7 +650,7 @@ namespace
             const auto mg = runBuffer(mlpGrad, (uint64_t)b * K * 4u, K * 4u);
 #pragma unroll
             for(uint32_t e = 0; e < (K + 63u) / 64u; ++e)
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, uw[e * 64u + lane]), mg, (e * 64u + lane) * 4u, 0, NONTEMPORAL);
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, uw[e * 64u + lane]), mg, (e * 64u + lane) * 4u, 0, STORE_POLICY);
 
             float sv[2][8];
 #pragma unroll
@@ -682,7 +702,7 @@ namespace
                 const uint32_t c = j * 64u + lane;
                 using u32x4      = uint32_t __attribute__((ext_vector_type(4)));
                 __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(xw + chunkAt(c / ROW_CHUNKS, c % ROW_CHUNKS)), dst,
-                                                       c * 16u, 0, NONTEMPORAL);
+                                                       c * 16u, 0, STORE_POLICY);
             }
             __builtin_amdgcn_s_waitcnt(0xC07F); // the images are rewritten by the next sample
             __builtin_amdgcn_wave_barrier();
