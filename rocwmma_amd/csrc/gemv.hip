@@ -208,9 +208,19 @@ namespace
     // STREAM: A lies beyond the memory-side cache and is read with nontemporal loads; a smaller one (few very long rows
     // of a matrix that is multiplied again and again) keeps ordinary loads so that the next call finds it there, as in
     // gemvRowMajor / gemvColMajor.
-    // SPLIT: workgroup (b, s) takes elements [s kPer, (s + 1) kPer) of its rows only (kPer a multiple of the slice) and
-    // leaves the sums, unscaled, in row s of a [splits][m] array (yOut) for gemvAddSplits.
-    template <typename T, uint32_t WAVES, uint32_t RB = SHARED_ROWS, bool STREAM = true, bool SPLIT = false>
+    // SPLIT: workgroup (s, b) of a grid whose fast index is the split takes elements [s kPer, (s + 1) kPer) of its RB rows
+    // only (kPer a multiple of the slice) and leaves the sums, unscaled, in row s of a [splits][m] array (yOut) for
+    // gemvAddSplits.  With pieces of 128 KiB the workgroups that run at the same time read neighbouring pieces of the
+    // same rows, and the RB rows of a workgroup share every load of x: one row per workgroup reads as many bytes of x
+    // (from the caches) as of A, and no variant of it - 4 to 16 waves, 4 to 16 loads in flight, software-pipelined,
+    // either grid order - passed 0.80 of the HBM peak on 512 MiB ... 1 GiB of A, where four rows per workgroup of eight
+    // waves with two slices of each in flight reach 0.85 - 0.90 (256 x 524288: 0.78 -> 0.88, 1024 x 262144: 0.79 -> 0.90,
+    // 64 x 2097152: 0.78 -> 0.86; two rows: 0.89 / 0.89 / 0.86, eight: 0.84 / 0.86 / 0.84).
+    // BATCH (without SPLIT): the same loop - every load of a group requested before the first is used, x shared by the
+    // workgroup's rows - over whole rows, for a streamed matrix of 384 ... 2047 long rows, where it needs no workspace:
+    // two or four rows per workgroup, whichever leaves the CUs evenly loaded (f32, rows of 512 KiB - 1 MiB: 512 rows 0.77
+    // -> 0.86, 1024 rows 0.78 -> 0.88, 1536 rows 0.78 -> 0.87, 2000 rows 0.78 -> 0.88 of the HBM peak).
+    template <typename T, uint32_t WAVES, uint32_t RB = SHARED_ROWS, bool STREAM = true, bool SPLIT = false, bool BATCH = SPLIT>
     __global__ void __launch_bounds__(WAVES * 64u) gemvRowMajorShared(uint32_t m,
                                                                       uint32_t k,
                                                                       const T* a,
@@ -228,8 +238,8 @@ namespace
         using VecT               = T __attribute__((ext_vector_type(V)));
         __shared__ T   partial[WAVES][RB];
         const uint32_t lane = threadIdx.x & 63u, w = threadIdx.x / 64u;
-        const uint32_t row0 = blockIdx.x * RB;
-        const uint32_t kBeg = SPLIT ? blockIdx.y * kPer : 0u; // (wave-uniform)
+        const uint32_t row0 = (SPLIT ? blockIdx.y : blockIdx.x) * RB;
+        const uint32_t kBeg = SPLIT ? blockIdx.x * kPer : 0u; // (wave-uniform)
         const uint32_t kBytes = (SPLIT ? (k - kBeg < kPer ? k - kBeg : kPer) : k) * (uint32_t)sizeof(T);
         // One buffer per row and one for x, each k elements long: what a load asks for beyond that comes back as zero, so
         // a row that does not fill its last slice needs no separate tail, and a row past m (a buffer of no bytes) adds
@@ -252,7 +262,32 @@ namespace
         }
         const uint32_t mine = (w * 64u + lane) * 16u;
         uint32_t       kc   = 0;
-        if constexpr(RB == 1u)
+        if constexpr(BATCH)
+        {
+            // all of a group's loads - two (four rows) or four (two rows) slices of every row and of x - are requested
+            // before the first is used
+            constexpr uint32_t AHEAD = RB >= 4u ? 2u : 4u;
+            for(; kc < kBytes; kc += AHEAD * SLICE)
+            {
+                VecT v[RB][AHEAD], xv[AHEAD];
+#pragma unroll
+                for(uint32_t r = 0; r < RB; ++r)
+#pragma unroll
+                    for(uint32_t u = 0; u < AHEAD; ++u)
+                        v[r][u] = __builtin_bit_cast(VecT, __builtin_amdgcn_raw_buffer_load_b128(rows[r], mine, kc + u * SLICE, NT));
+#pragma unroll
+                for(uint32_t u = 0; u < AHEAD; ++u)
+                    xv[u] = __builtin_bit_cast(VecT, __builtin_amdgcn_raw_buffer_load_b128(xr, mine, kc + u * SLICE, 0));
+#pragma unroll
+                for(uint32_t r = 0; r < RB; ++r)
+#pragma unroll
+                    for(uint32_t u = 0; u < AHEAD; ++u)
+#pragma unroll
+                        for(uint32_t e = 0; e < V; ++e)
+                            acc[r] += v[r][u][e] * xv[u][e];
+            }
+        }
+        else if constexpr(RB == 1u)
         {
             // a single row per workgroup: nothing but this row's slices to overlap, so several of them are requested
             // before the first is used
@@ -308,7 +343,7 @@ namespace
                 sum += partial[i][threadIdx.x];
             const uint32_t row = row0 + threadIdx.x;
             if constexpr(SPLIT)
-                yOut[(uint64_t)blockIdx.y * m + row] = sum;
+                yOut[(uint64_t)blockIdx.x * m + row] = sum;
             else
                 yOut[row] = beta != T(0) ? alpha * sum + beta * yIn[row] : alpha * sum;
         }
@@ -334,10 +369,12 @@ namespace
     // 4096 x 16384 42.4 / 40.2, 8256 x 8192 67.5 / 46.3, 12288 x 8192 77.0 / 60.0, 2048 x 32768 78.3 / 40.5,
     // 256 x 262144 592 / 48.9, 64 x 1048576 2580 / 57.7, 16640 x 16384 261 / 164, 20000 x 16384 274 / 185.  K is divided into pieces of at least 1024 columns so that two
     // (128-byte runs) or eight (512-byte runs) workgroups per CU result.
-    // Row-major A with at most half as many rows as CUs, each of 256 KiB or more: a workgroup per row leaves CUs without
-    // one (128 rows of 4 MiB: 0.46 of the HBM peak, split 0.73; 64 rows: 0.25 / 0.73; 32 rows: 0.13 / 0.71; the plain
-    // kernel is ahead with 200 rows of 1 MiB, 0.85 / 0.72, and from 256 rows on, 0.76 / 0.73); pieces of at least
-    // 128 KiB, about four workgroups per CU.
+    // Row-major A with rows of 256 KiB or more, beyond the memory-side cache and fewer than 2048 of them, or at most half
+    // as many as CUs: the plain kernels have a workgroup per row (up to 512 rows; too few workgroups below 256 rows, and
+    // as many bytes of x as of A to read: 128 rows of 4 MiB 0.46 of the HBM peak, 256 rows of 2 MiB 0.75) or a wave per
+    // row (1024 x 262144: 0.76); split, four rows share a workgroup and K is cut into pieces of 128 KiB (32 rows: 0.75,
+    // 64 - 128: 0.82, 256: 0.86, 512: 0.87, 1024: 0.89).  From 2048 rows on the plain shared-row kernel does the same
+    // without a workspace (2000 x 131072: 0.885 plain, 0.877 split).
     template <typename T>
     uint32_t gemvSplits(int32_t layout_a, uint32_t m, uint32_t k, uint32_t& kPer)
     {
@@ -362,9 +399,12 @@ namespace
         else
         {
             const uint64_t rowBytes = (uint64_t)k * sizeof(T);
-            if(m > cus / 2u || rowBytes < (256u << 10) || rowBytes >= (1ull << 31))
+            const bool     beyondCache = rowBytes * m > (256ull << 20); // (within the memory-side cache the plain kernels are 1 - 9 % ahead)
+            if(rowBytes < (256u << 10) || rowBytes >= (1ull << 31) || !(m <= cus / 2u || (beyondCache && m < 2048u)))
                 return 1u;
-            blocks = m, grain = (128u << 10) / (uint32_t)sizeof(T), perCu = 4u;
+            const uint32_t piece = (128u << 10) / (uint32_t)sizeof(T); // pieces of 128 KiB, or the multiple of that which makes 256 of them
+            kPer = piece * ((k + 256u * piece - 1u) / (256u * piece));
+            return (k + kPer - 1u) / kPer;
         }
         uint32_t splits = (perCu * cus + blocks - 1u) / blocks;
         if(splits > k / grain)
@@ -375,6 +415,25 @@ namespace
             return 1u;
         kPer = ((k + splits - 1u) / splits + grain - 1u) / grain * grain; // whole grains: every split starts on a slice boundary
         return (k + kPer - 1u) / kPer;
+    }
+
+    // Rows per workgroup of the batched shared-row kernel for a streamed row-major A with long rows and fewer than 2048
+    // of them, 0 = another kernel serves it.  Four or two rows, the larger count whose workgroups load the CUs evenly:
+    // at least half of them in a single round, at least 80 % of the slots of several rounds (f32, rows of 512 KiB, four /
+    // two / one row per workgroup: 640 rows 0.71 / 0.63 / 0.68, 896 rows 0.86 / 0.81 / 0.71, 1152 rows 0.62 / 0.73 / 0.73,
+    // 1280 rows of 256 KiB 0.66 / 0.76 / 0.69, 1792 rows 0.83 / 0.80 / 0.71).
+    inline uint32_t batchedRows(uint32_t m, bool stream, uint64_t rowBytes)
+    {
+        if(!stream || m >= 2048u || rowBytes < (256u << 10) || rowBytes >= (1ull << 31))
+            return 0u;
+        const uint32_t cus = r355::computeUnits();
+        for(uint32_t rb = 4u; rb >= 2u; rb /= 2u)
+        {
+            const uint32_t groups = (m + rb - 1u) / rb, rounds = (groups + cus - 1u) / cus;
+            if(rounds == 1u ? groups * 2u >= cus : (uint64_t)groups * 10u >= (uint64_t)rounds * cus * 8u)
+                return rb;
+        }
+        return 0u;
     }
 
     template <typename T>
@@ -444,10 +503,19 @@ namespace
             // ahead again from there on, and from 768 rows of 128 or 256 KiB)
             if(split)
             {
+                const dim3 grid(splits, (m + SHARED_ROWS - 1u) / SHARED_ROWS);
                 if(stream)
-                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16, 1, true, true>), dim3(m, splits), dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, parts, alpha, beta, kPer);
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 8, SHARED_ROWS, true, true>), grid, dim3(8 * 64), 0, s, m, k, a, lda, x, y_in, parts, alpha, beta, kPer);
                 else
-                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16, 1, false, true>), dim3(m, splits), dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, parts, alpha, beta, kPer);
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 8, SHARED_ROWS, false, true>), grid, dim3(8 * 64), 0, s, m, k, a, lda, x, y_in, parts, alpha, beta, kPer);
+            }
+            else if(const uint32_t rb = batchedRows(m, stream, rowBytes); rb != 0u)
+            {
+                const dim3 blocks((m + rb - 1u) / rb);
+                if(rb == 4u)
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 8, 4, true, false, true>), blocks, dim3(8 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k);
+                else
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 8, 2, true, false, true>), blocks, dim3(8 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k);
             }
             else if((m <= 512u || (m <= 768u && rowBytes >= (512u << 10))) && rowBytes >= (128u << 10) && rowBytes < (1ull << 31))
             {

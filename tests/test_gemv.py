@@ -108,7 +108,19 @@ def test_row_major_few_long_rows(dtype, m, k, pad):
     _shared_rows_case(dtype, m, k, pad, streamed=False)
 
 
-def _shared_rows_case(dtype, m, k, pad, streamed=True):
+@pytest.mark.parametrize("dtype,m,k,pad", [("f32", 1028, 65540, 4),    # 257 groups of four rows... two rounds: two rows per workgroup
+                                           ("f32", 516, 131076, 0),    # 258 groups of two rows
+                                           ("f32", 772, 90000, 8),     # 193 groups of four rows
+                                           ("f64", 386, 131074, 2),    # f64, 193 groups of two rows
+                                           ("f64", 1030, 32770, 0)])   # f64, rows of 256 KiB and two elements
+@pytest.mark.parametrize("workspace", [False, True])
+def test_row_major_long_rows_of_a_streamed_matrix(dtype, m, k, pad, workspace):
+    """384 ... 2047 rows of 256 KiB and more, A beyond 256 MiB: without a workspace the batched shared-row kernel (two or four
+    rows per workgroup share the loads of x), with one the split form (four rows per workgroup, pieces of 128 KiB)."""
+    _shared_rows_case(dtype, m, k, pad, workspace=workspace)
+
+
+def _shared_rows_case(dtype, m, k, pad, streamed=True, workspace=False):
     """Row-major A beyond 256 MiB with rows of 16 KiB and more takes the kernel whose workgroups share each row; the
     shapes leave a partly filled last slice of k, a partly filled last group of rows and a padded leading dimension.
     Every row against a float64 (f64: exact integer) evaluation on the device."""
@@ -125,7 +137,12 @@ def _shared_rows_case(dtype, m, k, pad, streamed=True):
     A = a.view(m, lda)
     A[:, k:] = float("nan")  # the padding is never read
     y = torch.full((m,), float("nan"), device="cuda", dtype=tdt)
-    fn(O.ROW, m, k, a, x, yin, y, 2.0, 2.0, lda=lda)
+    ws = None
+    if workspace:
+        need = R.gemv_workspace_bytes(O.ROW, m, k, a.element_size())
+        assert need > 0
+        ws = torch.full((need,), 0xFF, dtype=torch.uint8, device="cuda")
+    fn(O.ROW, m, k, a, x, yin, y, 2.0, 2.0, lda=lda, workspace=ws)
     torch.cuda.synchronize()
     Ad, xd = A[:, :k].double(), x.double()
     exact = 2.0 * (Ad @ xd) + 2.0 * yin.double()
@@ -139,7 +156,7 @@ def _shared_rows_case(dtype, m, k, pad, streamed=True):
         # integer-valued operands: exact in any summation order
         ai, xi = torch.round(a * 8.0), torch.round(x * 8.0)
         ai.view(m, lda)[:, k:] = float("nan")
-        fn(O.ROW, m, k, ai, xi, None, y, 1.0, 0.0, lda=lda)
+        fn(O.ROW, m, k, ai, xi, None, y, 1.0, 0.0, lda=lda, workspace=ws)
         torch.cuda.synchronize()
         assert torch.equal(y, ai.view(m, lda)[:, :k] @ xi)
 
