@@ -27,7 +27,7 @@ namespace
     // COL_WAVES * 64 / RL partial sums of a row meet in LDS and are added in a fixed order, so the result does not depend
     // on scheduling.  STREAM as in the row-major kernel.
     // SPLIT: workgroup (b, s) of a two-dimensional grid sums columns [s kPer, (s + 1) kPer) only and leaves its rows' sums,
-    // unscaled, in row s of a [splits][m] array (yOut) for gemvAddSplits.
+    // unscaled, in an array of partial sums (yOut; element (row, s) at row * partRow + s * partSplit) for gemvAddSplits.
     template <typename T, uint32_t RL, uint32_t COL_WAVES, bool STREAM, bool SPLIT = false>
     __global__ void __launch_bounds__(COL_WAVES * 64) gemvColMajor(uint32_t m,
                                                                   uint32_t k,
@@ -38,7 +38,9 @@ namespace
                                                                   T*       yOut,
                                                                   T        alpha,
                                                                   T        beta,
-                                                                  uint32_t kPer)
+                                                                  uint32_t kPer,
+                                                                  uint32_t partRow,
+                                                                  uint32_t partSplit)
     {
         constexpr uint32_t V = 16u / sizeof(T), ROWS = RL * V, CL = 64u / RL, COLS = COL_WAVES * CL, DEPTH = 8;
         using VecT = T __attribute__((ext_vector_type(V)));
@@ -100,14 +102,35 @@ namespace
                 for(uint32_t w = 0; w < COLS; ++w)
                     sum += partial[w][threadIdx.x];
                 if constexpr(SPLIT)
-                    yOut[(uint64_t)blockIdx.y * m + row] = sum;
+                    yOut[(uint64_t)row * partRow + (uint64_t)blockIdx.y * partSplit] = sum;
                 else
                     yOut[row] = beta != T(0) ? alpha * sum + beta * yIn[row] : alpha * sum;
             }
         }
     }
 
-    // Second kernel of the split forms: y = alpha * (sum of the splits' partial sums, in split order) + beta * y.
+    // Second kernel of the split forms: y = alpha * (sum of a row's partial sums) + beta * y, in an order that the number
+    // of splits alone decides.
+    // Many splits (32 and more: few rows): the partial sums are stored [m][splits] and a wave takes a row - lane l adds
+    // those of splits l, l + 64, ... in that order and the 64 lane sums meet in a fixed tree; one memory latency, where a
+    // thread per row walking 64 splits took 4.7 us and 256 splits longer than the first kernel.
+    template <typename T>
+    __global__ void __launch_bounds__(THREADS) gemvAddSplitsByWave(uint32_t m, uint32_t splits, const T* partial, const T* yIn, T* yOut, T alpha, T beta)
+    {
+        const uint32_t lane = threadIdx.x & 63u, row = blockIdx.x * (THREADS / 64u) + threadIdx.x / 64u;
+        if(row >= m)
+            return;
+        const T* p   = partial + (uint64_t)row * splits;
+        T        sum = T(0);
+        for(uint32_t s0 = lane; s0 < splits; s0 += 64u)
+            sum += p[s0];
+#pragma unroll
+        for(uint32_t off = 32; off > 0; off >>= 1)
+            sum += __shfl_xor(sum, off, 64);
+        if(lane == 0)
+            yOut[row] = beta != T(0) ? alpha * sum + beta * yIn[row] : alpha * sum;
+    }
+    // Few splits (many rows): stored [splits][m], a thread per row adds them in split order, eight requests under way.
     template <typename T>
     __global__ void __launch_bounds__(THREADS) gemvAddSplits(uint32_t m, uint32_t splits, const T* partial, const T* yIn, T* yOut, T alpha, T beta)
     {
@@ -115,7 +138,7 @@ namespace
         if(row >= m)
             return;
         T sum = T(0);
-        for(uint32_t s0 = 0; s0 < splits; s0 += 8u) // (eight requests under way per thread)
+        for(uint32_t s0 = 0; s0 < splits; s0 += 8u)
         {
             T v[8];
 #pragma unroll
@@ -209,8 +232,8 @@ namespace
     // of a matrix that is multiplied again and again) keeps ordinary loads so that the next call finds it there, as in
     // gemvRowMajor / gemvColMajor.
     // SPLIT: workgroup (s, b) of a grid whose fast index is the split takes elements [s kPer, (s + 1) kPer) of its RB rows
-    // only (kPer a multiple of the slice) and leaves the sums, unscaled, in row s of a [splits][m] array (yOut) for
-    // gemvAddSplits.  With pieces of 128 KiB the workgroups that run at the same time read neighbouring pieces of the
+    // only (kPer a multiple of the slice) and leaves the sums, unscaled, in the array of partial sums (yOut, as in
+    // gemvColMajor) for gemvAddSplits.  With pieces of 128 KiB the workgroups that run at the same time read neighbouring pieces of the
     // same rows, and the RB rows of a workgroup share every load of x: one row per workgroup reads as many bytes of x
     // (from the caches) as of A, and no variant of it - 4 to 16 waves, 4 to 16 loads in flight, software-pipelined,
     // either grid order - passed 0.80 of the HBM peak on 512 MiB ... 1 GiB of A, where four rows per workgroup of eight
@@ -230,7 +253,9 @@ namespace
                                                                       T*       yOut,
                                                                       T        alpha,
                                                                       T        beta,
-                                                                      uint32_t kPer)
+                                                                      uint32_t kPer,
+                                                                      uint32_t partRow,
+                                                                      uint32_t partSplit)
     {
         constexpr uint32_t V = 16u / sizeof(T);
         constexpr uint32_t SLICE = WAVES * 64u * 16u; // bytes one load instruction of the whole workgroup covers
@@ -343,22 +368,29 @@ namespace
                 sum += partial[i][threadIdx.x];
             const uint32_t row = row0 + threadIdx.x;
             if constexpr(SPLIT)
-                yOut[(uint64_t)blockIdx.x * m + row] = sum;
+                yOut[(uint64_t)row * partRow + (uint64_t)blockIdx.x * partSplit] = sum;
             else
                 yOut[row] = beta != T(0) ? alpha * sum + beta * yIn[row] : alpha * sum;
         }
     }
 
     // Lanes side by side on one column in the split form of the col-major kernel.  With K divided there are workgroups
-    // enough whatever the rows per workgroup, so the runs can be longer than the plain kernel's: 512 bytes from 256
-    // 16-byte pieces per column on (f32, 256 MiB of A: 1024 x 65536 0.79 of the HBM peak against 0.75 with 128-byte runs,
-    // 2048 x 32768 0.83 against 0.76, 16640 x 16384 0.83 against 0.65; 1 KiB runs: 0.72, 0.78, 0.78); shorter columns
-    // keep 128-byte runs (256 x 262144: 0.69 against 0.61 and 0.51).
+    // enough whatever the rows per workgroup, so the runs can be longer than the plain kernel's.  Columns of 512 bytes and
+    // more, up to 256 16-byte pieces: a wave takes whole kilobytes of a column, eight waves per workgroup (f32 256 x 262144,
+    // 256 splits, first kernel alone: 0.89 of the HBM peak against 0.85 with 128-byte runs and sixteen waves; with sixteen
+    // waves 0.72; 128 x 524288: 0.87 - 0.89 against 0.76); shorter columns: 256-byte runs (64 x 1048576: 0.81 against 0.74
+    // and 0.58 - 0.67 with whole kilobytes); from 256 pieces per column on 512-byte runs and sixteen waves (1024 x 65536
+    // 0.79 against 0.75 with 128-byte runs, 2048 x 32768 0.83 against 0.76, 16640 x 16384 0.83 against 0.65; 1 KiB runs:
+    // 0.72, 0.78, 0.78).
     template <typename T>
-    uint32_t splitRunLanes(uint32_t m)
+    uint32_t splitRunLanes(uint32_t m, uint32_t k)
     {
         constexpr uint32_t V = 16u / sizeof(T);
-        return m >= 256u * V ? 32u : 8u;
+        if(m >= 256u * V)
+            return 32u;
+        if(k < 128u * 1024u)
+            return 8u; // too short for a workgroup per CU with one or two blocks of rows: many blocks of 32 rows (256 x 16384: 6 us against 13)
+        return m >= 32u * V ? 64u : 16u;
     }
 
     // Splits of K for a shape, 1 = the plain kernels serve it.
@@ -367,8 +399,8 @@ namespace
     // as rounds over the CUs - a workgroup streams about 50 GB/s on its own, all CUs together 7.2 TB/s - and the split
     // form as A at 7.0 TB/s plus 3 us for the second launch; measured (f32): 4096^2 12.8 us plain / 13.3 split,
     // 4096 x 16384 42.4 / 40.2, 8256 x 8192 67.5 / 46.3, 12288 x 8192 77.0 / 60.0, 2048 x 32768 78.3 / 40.5,
-    // 256 x 262144 592 / 48.9, 64 x 1048576 2580 / 57.7, 16640 x 16384 261 / 164, 20000 x 16384 274 / 185.  K is divided into pieces of at least 1024 columns so that two
-    // (128-byte runs) or eight (512-byte runs) workgroups per CU result.
+    // 16640 x 16384 261 / 164, 20000 x 16384 274 / 185.  K is divided into pieces of at least 1024 columns so that two
+    // (few rows) or eight (512-byte runs) workgroups per CU result, 256 pieces at most.
     // Row-major A with rows of 256 KiB or more, beyond the memory-side cache and fewer than 2048 of them, or at most half
     // as many as CUs: the plain kernels have a workgroup per row (up to 512 rows; too few workgroups below 256 rows, and
     // as many bytes of x as of A to read: 128 rows of 4 MiB 0.46 of the HBM peak, 256 rows of 2 MiB 0.75) or a wave per
@@ -393,8 +425,8 @@ namespace
             const double   tSplit  = bytes / 7.0e6 + 3.0;
             if(rounds > 3u || tSplit * 1.03 >= tPlain) // (many rounds even out by themselves as workgroups end at different times)
                 return 1u;
-            const uint32_t lanes = splitRunLanes<T>(m);
-            blocks = (m + lanes * V - 1u) / (lanes * V), grain = 1024u, perCu = lanes == 8u ? 2u : 8u;
+            const uint32_t lanes = splitRunLanes<T>(m, k);
+            blocks = (m + lanes * V - 1u) / (lanes * V), grain = 1024u, perCu = lanes == 32u ? 8u : 2u;
         }
         else
         {
@@ -419,9 +451,10 @@ namespace
 
     // Rows per workgroup of the batched shared-row kernel for a streamed row-major A with long rows and fewer than 2048
     // of them, 0 = another kernel serves it.  Four or two rows, the larger count whose workgroups load the CUs evenly:
-    // at least half of them in a single round, at least 80 % of the slots of several rounds (f32, rows of 512 KiB, four /
-    // two / one row per workgroup: 640 rows 0.71 / 0.63 / 0.68, 896 rows 0.86 / 0.81 / 0.71, 1152 rows 0.62 / 0.73 / 0.73,
-    // 1280 rows of 256 KiB 0.66 / 0.76 / 0.69, 1792 rows 0.83 / 0.80 / 0.71).
+    // at least five eighths of them in a single round, at least 80 % of the slots of several rounds (f32, rows of 512 KiB
+    // and more, four / two / one row per workgroup: 256 rows 0.35 / 0.56 / 0.75, 384 rows 0.49 / 0.77 / 0.63, 512 rows
+    // 0.61 / 0.86 / 0.77, 640 rows 0.71 / 0.63 / 0.68, 896 rows 0.86 / 0.81 / 0.71, 1152 rows 0.62 / 0.73 / 0.73, 1280
+    // rows of 256 KiB 0.66 / 0.76 / 0.69, 1792 rows 0.83 / 0.80 / 0.71).
     inline uint32_t batchedRows(uint32_t m, bool stream, uint64_t rowBytes)
     {
         if(!stream || m >= 2048u || rowBytes < (256u << 10) || rowBytes >= (1ull << 31))
@@ -430,7 +463,7 @@ namespace
         for(uint32_t rb = 4u; rb >= 2u; rb /= 2u)
         {
             const uint32_t groups = (m + rb - 1u) / rb, rounds = (groups + cus - 1u) / cus;
-            if(rounds == 1u ? groups * 2u >= cus : (uint64_t)groups * 10u >= (uint64_t)rounds * cus * 8u)
+            if(rounds == 1u ? groups * 8u >= cus * 5u : (uint64_t)groups * 10u >= (uint64_t)rounds * cus * 8u)
                 return rb;
         }
         return 0u;
@@ -458,6 +491,8 @@ namespace
         const uint32_t splits = (layout_a == R355_COL_MAJOR || layout_a == R355_ROW_MAJOR) && workspace ? gemvSplits<T>(layout_a, m, k, kPer) : 1u;
         const bool     split  = splits > 1u && (uint64_t)splits * m * sizeof(T) <= workspaceBytes;
         T*             parts  = static_cast<T*>(workspace);
+        const bool     byWave = splits >= 32u; // layout of the partial sums: [m][splits] for the wave-per-row reduction, else [splits][m]
+        const uint32_t partRow = byWave ? splits : 1u, partSplit = byWave ? 1u : m;
         if(layout_a == R355_COL_MAJOR)
         {
             if(lda < m)
@@ -467,19 +502,23 @@ namespace
                 constexpr uint32_t RL = decltype(rl)::value, ROWS = RL * V, WAVES = decltype(waves)::value;
                 const dim3         grid((m + ROWS - 1u) / ROWS, split ? splits : 1u), block(WAVES * 64);
                 if(split && stream)
-                    hipLaunchKernelGGL((gemvColMajor<T, RL, WAVES, true, true>), grid, block, 0, s, m, k, a, lda, x, y_in, parts, alpha, beta, kPer);
+                    hipLaunchKernelGGL((gemvColMajor<T, RL, WAVES, true, true>), grid, block, 0, s, m, k, a, lda, x, y_in, parts, alpha, beta, kPer, partRow, partSplit);
                 else if(split)
-                    hipLaunchKernelGGL((gemvColMajor<T, RL, WAVES, false, true>), grid, block, 0, s, m, k, a, lda, x, y_in, parts, alpha, beta, kPer);
+                    hipLaunchKernelGGL((gemvColMajor<T, RL, WAVES, false, true>), grid, block, 0, s, m, k, a, lda, x, y_in, parts, alpha, beta, kPer, partRow, partSplit);
                 else if(stream)
-                    hipLaunchKernelGGL((gemvColMajor<T, RL, WAVES, true>), grid, block, 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k);
+                    hipLaunchKernelGGL((gemvColMajor<T, RL, WAVES, true>), grid, block, 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k, 0u, 0u);
                 else
-                    hipLaunchKernelGGL((gemvColMajor<T, RL, WAVES, false>), grid, block, 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k);
+                    hipLaunchKernelGGL((gemvColMajor<T, RL, WAVES, false>), grid, block, 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k, 0u, 0u);
             };
             // 256-byte runs once the rows give every CU a workgroup with them (8192^2 f32: 0.0415 ms against 0.0374 with
             // 128-byte runs and twice the workgroups; 16384^2: 0.151 against 0.161); sixteen waves per workgroup either way
             // (four: 0.0399 and 0.163)
-            if(split && splitRunLanes<T>(m) == 32u)
+            if(split && splitRunLanes<T>(m, k) == 32u)
                 go(std::integral_constant<uint32_t, 32>{}, std::integral_constant<uint32_t, 16>{});
+            else if(split && splitRunLanes<T>(m, k) == 64u)
+                go(std::integral_constant<uint32_t, 64>{}, std::integral_constant<uint32_t, 8>{});
+            else if(split && splitRunLanes<T>(m, k) == 16u)
+                go(std::integral_constant<uint32_t, 16>{}, std::integral_constant<uint32_t, 8>{});
             else if(split)
                 go(std::integral_constant<uint32_t, 8>{}, std::integral_constant<uint32_t, 16>{});
             else if(m >= 16u * V * 256u)
@@ -505,32 +544,32 @@ namespace
             {
                 const dim3 grid(splits, (m + SHARED_ROWS - 1u) / SHARED_ROWS);
                 if(stream)
-                    hipLaunchKernelGGL((gemvRowMajorShared<T, 8, SHARED_ROWS, true, true>), grid, dim3(8 * 64), 0, s, m, k, a, lda, x, y_in, parts, alpha, beta, kPer);
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 8, SHARED_ROWS, true, true>), grid, dim3(8 * 64), 0, s, m, k, a, lda, x, y_in, parts, alpha, beta, kPer, partRow, partSplit);
                 else
-                    hipLaunchKernelGGL((gemvRowMajorShared<T, 8, SHARED_ROWS, false, true>), grid, dim3(8 * 64), 0, s, m, k, a, lda, x, y_in, parts, alpha, beta, kPer);
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 8, SHARED_ROWS, false, true>), grid, dim3(8 * 64), 0, s, m, k, a, lda, x, y_in, parts, alpha, beta, kPer, partRow, partSplit);
             }
             else if(const uint32_t rb = batchedRows(m, stream, rowBytes); rb != 0u)
             {
                 const dim3 blocks((m + rb - 1u) / rb);
                 if(rb == 4u)
-                    hipLaunchKernelGGL((gemvRowMajorShared<T, 8, 4, true, false, true>), blocks, dim3(8 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k);
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 8, 4, true, false, true>), blocks, dim3(8 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k, 0u, 0u);
                 else
-                    hipLaunchKernelGGL((gemvRowMajorShared<T, 8, 2, true, false, true>), blocks, dim3(8 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k);
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 8, 2, true, false, true>), blocks, dim3(8 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k, 0u, 0u);
             }
             else if((m <= 512u || (m <= 768u && rowBytes >= (512u << 10))) && rowBytes >= (128u << 10) && rowBytes < (1ull << 31))
             {
                 if(stream)
-                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16, 1, true>), dim3(m), dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k);
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16, 1, true>), dim3(m), dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k, 0u, 0u);
                 else
-                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16, 1, false>), dim3(m), dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k);
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16, 1, false>), dim3(m), dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k, 0u, 0u);
             }
             else if(stream && rowBytes >= (16u << 10) && rowBytes < (1ull << 31) && m >= SHARED_ROWS * 512u)
             {
                 const dim3 blocks((m + SHARED_ROWS - 1u) / SHARED_ROWS);
                 if(rowBytes < (128u << 10))
-                    hipLaunchKernelGGL((gemvRowMajorShared<T, 8>), blocks, dim3(8 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k);
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 8>), blocks, dim3(8 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k, 0u, 0u);
                 else
-                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16>), blocks, dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k);
+                    hipLaunchKernelGGL((gemvRowMajorShared<T, 16>), blocks, dim3(16 * 64), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta, k, 0u, 0u);
             }
             else if(stream)
                 hipLaunchKernelGGL((gemvRowMajor<T, true>), grid, dim3(THREADS), 0, s, m, k, a, lda, x, y_in, y_out, alpha, beta);
@@ -539,7 +578,9 @@ namespace
         }
         else
             return r355::fail(R355_ERR_BAD_ARG, "gemv: unknown layout");
-        if(split)
+        if(split && byWave)
+            hipLaunchKernelGGL(gemvAddSplitsByWave<T>, dim3((m + THREADS / 64u - 1u) / (THREADS / 64u)), dim3(THREADS), 0, s, m, splits, parts, y_in, y_out, alpha, beta);
+        else if(split)
             hipLaunchKernelGGL(gemvAddSplits<T>, dim3((m + THREADS - 1u) / THREADS), dim3(THREADS), 0, s, m, splits, parts, y_in, y_out, alpha, beta);
         return r355::checkLaunch("gemv");
     }
