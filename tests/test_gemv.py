@@ -108,11 +108,11 @@ def test_row_major_few_long_rows(dtype, m, k, pad):
     _shared_rows_case(dtype, m, k, pad, streamed=False)
 
 
-@pytest.mark.parametrize("dtype,m,k,pad", [("f32", 1028, 65540, 4),    # 257 groups of four rows... two rounds: two rows per workgroup
-                                           ("f32", 516, 131076, 0),    # 258 groups of two rows
+@pytest.mark.parametrize("dtype,m,k,pad", [("f32", 1028, 65540, 4),    # 257 groups of four rows or 514 of two: uneven rounds, so a wave per row (split: four rows)
+                                           ("f32", 512, 131076, 0),    # 256 groups of two rows
                                            ("f32", 772, 90000, 8),     # 193 groups of four rows
                                            ("f64", 386, 131074, 2),    # f64, 193 groups of two rows
-                                           ("f64", 1030, 32770, 0)])   # f64, rows of 256 KiB and two elements
+                                           ("f64", 768, 49154, 2)])    # f64, 192 groups of four rows
 @pytest.mark.parametrize("workspace", [False, True])
 def test_row_major_long_rows_of_a_streamed_matrix(dtype, m, k, pad, workspace):
     """384 ... 2047 rows of 256 KiB and more, A beyond 256 MiB: without a workspace the batched shared-row kernel (two or four
