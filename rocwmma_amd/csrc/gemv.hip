@@ -413,7 +413,7 @@ namespace
         constexpr uint32_t V = 16u / sizeof(T);
         const uint32_t     cus = r355::computeUnits();
         kPer = k;
-        uint32_t blocks, grain, perCu;
+        uint32_t blocks, grain, perCu, align, rowsPerBlock;
         if(layout_a == R355_COL_MAJOR)
         {
             const uint32_t rows   = (m >= 16u * V * 256u ? 16u : 8u) * V; // per workgroup, as the plain launch chooses them
@@ -427,6 +427,8 @@ namespace
                 return 1u;
             const uint32_t lanes = splitRunLanes<T>(m, k);
             blocks = (m + lanes * V - 1u) / (lanes * V), grain = 1024u, perCu = lanes == 32u ? 8u : 2u;
+            align  = lanes == 8u ? 1024u : 256u; // (a multiple of the columns one unrolled trip of the kernel covers)
+            rowsPerBlock = lanes * V;
         }
         else
         {
@@ -438,15 +440,39 @@ namespace
             kPer = piece * ((k + 256u * piece - 1u) / (256u * piece));
             return (k + kPer - 1u) / kPer;
         }
-        uint32_t splits = (perCu * cus + blocks - 1u) / blocks;
-        if(splits > k / grain)
-            splits = k / grain;
-        if(splits > 256u)
-            splits = 256u;
-        if(splits < 2u)
+        // About perCu workgroups per CU - and of the counts around that the cheapest by a small model of the launch: the
+        // workgroups are dealt out evenly over the CUs, all CUs together stream 7 TB/s, and the CUs that hold one workgroup
+        // more than the others finish it at what is left of that or at the 50 GB/s a CU streams on its own.  8256 rows are 65
+        // blocks, which eight splits turn into 520 workgroups - two per CU and a third on eight CUs - and seven into 455: 49.0
+        // -> 43.9 us (0.69 -> 0.77 of the HBM peak; the model says 48.8 and 42.7); 12288 rows, 96 blocks, stay with eight
+        // splits (768 workgroups: 60.1 us, model 57.5; five splits, 480 workgroups: 62.5, model 62.9); 16640 x 16384 takes
+        // eleven (162.9 us, model 160.5) over sixteen (164.9, 163.8).
+        uint32_t want = (perCu * cus + blocks - 1u) / blocks, most = k / grain < 256u ? k / grain : 256u;
+        if(want > most)
+            want = most;
+        if(want < 2u)
             return 1u;
-        kPer = ((k + splits - 1u) / splits + grain - 1u) / grain * grain; // whole grains: every split starts on a slice boundary
-        return (k + kPer - 1u) / kPer;
+        uint32_t best = 0, bestPer = k;
+        double   bestCost = 0.0;
+        for(uint32_t t = want / 2u > 2u ? want / 2u : 2u; t <= most && t <= 2u * want; ++t)
+        {
+            const uint32_t per = ((k + t - 1u) / t + align - 1u) / align * align; // every split but the last is whole unrolled trips
+            const uint32_t n = (k + per - 1u) / per, groups = blocks * n, each = groups / cus, over = groups % cus;
+            const double   bytes = static_cast<double>(per) * rowsPerBlock * sizeof(T); // of a workgroup
+            const double   left  = over ? 7.0e6 / over : 0.0; // bytes per us for each of the CUs with one more
+            const double   cost  = static_cast<double>(each) * bytes * cus / 7.0e6 + (over ? bytes / (left < 50.0e3 ? left : 50.0e3) : 0.0);
+            // (as cheap within 2 %: the larger count - smaller workgroups even out better than the model knows: 2048 x 32768,
+            // 16 workgroups of 128 rows, 0.75 with 16 splits and 0.85 with 32, one and two workgroups per CU)
+            if(n >= 2u && (best == 0u || cost < bestCost * 0.98 || (cost <= bestCost * 1.02 && n > best)))
+            {
+                bestCost = best == 0u || cost < bestCost ? cost : bestCost;
+                best = n, bestPer = per;
+            }
+        }
+        if(best < 2u)
+            return 1u;
+        kPer = bestPer;
+        return best;
     }
 
     // Rows per workgroup of the batched shared-row kernel for a streamed row-major A with long rows and fewer than 2048
