@@ -202,8 +202,8 @@ int r355_dgemv(int32_t layout_a, uint32_t m, uint32_t k, const double* a, uint32
  * what fills the CUs (8256 rows), a row-major A with few very long rows.  The splits' partial sums go to `workspace`
  * (the caller's device memory, 16-byte aligned; its contents before the call do not matter) and a second kernel adds
  * them in split order, so the result depends on the shape alone, never on scheduling.
- * r355_gemv_workspace_bytes: what the split form wants for a shape (elem_bytes 4: f32, 8: f64); 0 where the plain
- * kernels do as well.  With a null or smaller workspace r355_gemv_ws / r355_dgemv_ws run the plain kernels
+ * r355_gemv_workspace_bytes: what the split form wants for a shape (elem_bytes 4: f32, 8: f64; an unpadded A is
+ * assumed: lda = m col-major, k row-major); 0 where the plain kernels do as well.  With a null or smaller workspace r355_gemv_ws / r355_dgemv_ws run the plain kernels
  * (the same as r355_gemv / r355_dgemv).  No counterpart in the reference (its sample has one kernel for all shapes).
  */
 size_t r355_gemv_workspace_bytes(int32_t layout_a, uint32_t m, uint32_t k, uint32_t elem_bytes);

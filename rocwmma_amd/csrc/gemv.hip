@@ -408,7 +408,7 @@ namespace
     // 64 - 128: 0.82, 256: 0.86, 512: 0.87, 1024: 0.89).  From 2048 rows on the plain shared-row kernel does the same
     // without a workspace (2000 x 131072: 0.885 plain, 0.877 split).
     template <typename T>
-    uint32_t gemvSplits(int32_t layout_a, uint32_t m, uint32_t k, uint32_t& kPer)
+    uint32_t gemvSplits(int32_t layout_a, uint32_t m, uint32_t k, uint32_t lda, uint32_t& kPer)
     {
         constexpr uint32_t V = 16u / sizeof(T);
         const uint32_t     cus = r355::computeUnits();
@@ -421,8 +421,13 @@ namespace
             const double   bytes  = static_cast<double>(m) * k * sizeof(T), perGroup = static_cast<double>(rows) * k * sizeof(T);
             const double   abreast = static_cast<double>(plain < cus ? plain : cus) * perGroup / 7.2e6; // us: all of a round's workgroups at the HBM's rate
             const double   alone   = perGroup / 50.0e3; // us: a workgroup at its own
-            const double   tPlain  = static_cast<double>(rounds) * (abreast > alone ? abreast : alone);
-            const double   tSplit  = bytes / 7.0e6 + 3.0;
+            // Columns that do not start on a 128-byte boundary (lda not a multiple of 32 f32): the runs of neighbouring blocks
+            // of rows share cache lines, which then travel twice - the plain kernel's 128-byte runs take twice the time
+            // (5000 x 16384: 93 us where 4096 x 16384 takes 42), runs of 512 bytes a quarter more.
+            const bool     askew   = ((uint64_t)lda * sizeof(T)) % 128u != 0u;
+            const uint32_t wide    = splitRunLanes<T>(m, k);
+            const double   tPlain  = static_cast<double>(rounds) * (abreast > alone ? abreast : alone) * (askew ? 2.0 : 1.0);
+            const double   tSplit  = (bytes / 7.0e6) * (askew ? 1.0 + 8.0 / wide : 1.0) + 3.0;
             if(rounds > 3u || tSplit * 1.03 >= tPlain) // (many rounds even out by themselves as workgroups end at different times)
                 return 1u;
             const uint32_t lanes = splitRunLanes<T>(m, k);
@@ -514,7 +519,7 @@ namespace
         r355::beginCall();
         // K split over several workgroups per block of rows when the shape calls for it and the workspace holds the partial sums
         uint32_t       kPer   = k;
-        const uint32_t splits = (layout_a == R355_COL_MAJOR || layout_a == R355_ROW_MAJOR) && workspace ? gemvSplits<T>(layout_a, m, k, kPer) : 1u;
+        const uint32_t splits = (layout_a == R355_COL_MAJOR || layout_a == R355_ROW_MAJOR) && workspace ? gemvSplits<T>(layout_a, m, k, lda, kPer) : 1u;
         const bool     split  = splits > 1u && (uint64_t)splits * m * sizeof(T) <= workspaceBytes;
         T*             parts  = static_cast<T*>(workspace);
         const bool     byWave = splits >= 32u; // layout of the partial sums: [m][splits] for the wave-per-row reduction, else [splits][m]
@@ -617,7 +622,7 @@ extern "C" size_t r355_gemv_workspace_bytes(int32_t layout_a, uint32_t m, uint32
     if((layout_a != R355_COL_MAJOR && layout_a != R355_ROW_MAJOR) || m == 0 || k == 0)
         return 0;
     uint32_t       kPer   = k;
-    const uint32_t splits = elem_bytes == 8u ? gemvSplits<double>(layout_a, m, k, kPer) : gemvSplits<float>(layout_a, m, k, kPer);
+    const uint32_t splits = elem_bytes == 8u ? gemvSplits<double>(layout_a, m, k, layout_a == R355_COL_MAJOR ? m : k, kPer) : gemvSplits<float>(layout_a, m, k, layout_a == R355_COL_MAJOR ? m : k, kPer);
     return splits > 1u ? (size_t)splits * m * (elem_bytes == 8u ? 8u : 4u) : 0;
 }
 
