@@ -1,11 +1,13 @@
 // DLRM dot interaction for the shapes the specialised kernels of dlrm.hip do not take: more than 32 features, or an
 // embedding width other than 32 / 64 / 128 / 256 (the reference's own tests run m = 128, k = 128 and m = k = 1024 with a
-// batch of 64: test/dlrm/test/dlrm_test_params.hpp:55-58).  Written on the fragment API, one 16 x 16 block per wave as in
-// the reference's kernels (test/dlrm/device/dlrm_dot_fwd.hpp:37-135, dlrm_dot_bwd.hpp:35-176), m and k multiples of 16
-// as there (dlrm_kernel_base_impl.hpp:146-151) - but without their global scratch: the forward kernel takes the lower
-// triangle out of the accumulator block through 1 KiB of the wave's LDS instead of a [batch][m][m] f32 buffer, and the
-// backward kernel forms each 16 x 16 block of S = T + T^T in LDS from the packed upstream triangle instead of
-// reconstructing [batch][m][m] in memory first.  Correctness first: these run at the latency of block-per-wave code.
+// batch of 64: test/dlrm/test/dlrm_test_params.hpp:55-58).  Written on the fragment API as the reference's kernels are
+// (test/dlrm/device/dlrm_dot_fwd.hpp:37-135, dlrm_dot_bwd.hpp:35-176), m and k multiples of 16 as there
+// (dlrm_kernel_base_impl.hpp:146-151) - but without their global scratch: the forward kernels take the lower triangle
+// out of an accumulator block through 1 KiB of the wave's LDS instead of a [batch][m][m] f32 buffer, and the backward
+// kernels form each 16 x 16 block of S = T + T^T in LDS from the packed upstream triangle instead of reconstructing
+// [batch][m][m] in memory first.  Each direction has two forms: one 16 x 16 block per wave, as in the reference, for
+// small shapes, and a register-blocked one (several blocks per wave, so that a fragment feeds several matrix
+// instructions) for large ones.
 #include <rocwmma/rocwmma.hpp>
 
 #include "common.hpp"
@@ -75,6 +77,86 @@ namespace
         }
     }
 
+    // Forward from 64 features on: a wave owns NB x NB blocks at once - super-block (si, sj), sj <= si, of X X^T; p = si (si +
+    // 1) / 2 + sj - so that every fragment it loads feeds NB matrix instructions instead of one (a quarter of the bytes
+    // from the caches per flop at NB = 4: with a block per wave m = k = 1024 reads every row block of X 64 times over).
+    // BK: the K depth per step, 32 for 16-bit elements where k allows it (64-byte runs of a row per lane group instead of 32).
+    template <typename T, uint32_t NB, uint32_t BK>
+    __global__ void __launch_bounds__(THREADS) dlrmFwdGeneralBlocked(const T* __restrict__ in, T* __restrict__ out, uint32_t m, uint32_t k,
+                                                                    uint32_t pairs)
+    {
+        using FragA   = fragment<matrix_a, BLK, BLK, BK, T, row_major>;
+        using FragB   = fragment<matrix_b, BLK, BLK, BK, T, col_major>;
+        using FragAcc = fragment<accumulator, BLK, BLK, BK, float32_t>;
+        __shared__ float block[WAVES][BLK * BLK];
+
+        const uint32_t lane = threadIdx.x & 63u, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        const uint32_t p    = blockIdx.x * WAVES + wave;
+        if(p >= pairs)
+            return;
+        uint32_t si = 0;
+        while((si + 1u) * (si + 2u) / 2u <= p)
+            ++si;
+        const uint32_t sj     = p - si * (si + 1u) / 2u;
+        const uint32_t tiles  = m / BLK;
+        const uint64_t stride = (uint64_t)k + (uint64_t)m * (m - 1u) / 2u;
+        const T*       x      = in + (uint64_t)blockIdx.y * m * k;
+        T*             o      = out + (uint64_t)blockIdx.y * stride;
+
+        if(p == 0u) // the bottom-MLP row
+            for(uint32_t e = lane; e < k; e += 64u)
+                o[e] = x[e];
+
+        // block (i, j) of the super-block is block (ti, tj) = (si NB + i, sj NB + j) of X X^T; wanted when it exists and
+        // touches the strict lower triangle (tj <= ti)
+        auto wanted = [&](uint32_t i, uint32_t j) { return si * NB + i < tiles && sj * NB + j < tiles && sj * NB + j <= si * NB + i; };
+        FragAcc acc[NB][NB];
+#pragma unroll
+        for(uint32_t i = 0; i < NB; ++i)
+#pragma unroll
+            for(uint32_t j = 0; j < NB; ++j)
+                fill_fragment(acc[i][j], 0.0f);
+        for(uint32_t kk = 0; kk < k; kk += BK)
+        {
+            FragA a[NB];
+            FragB b[NB];
+#pragma unroll
+            for(uint32_t i = 0; i < NB; ++i)
+            {
+                // (a row block past the end reads the last one again: its products are not used)
+                const uint32_t ti = si * NB + i < tiles ? si * NB + i : tiles - 1u, tj = sj * NB + i < tiles ? sj * NB + i : tiles - 1u;
+                load_matrix_sync(a[i], x + (uint64_t)ti * BLK * k + kk, k);
+                load_matrix_sync(b[i], x + (uint64_t)tj * BLK * k + kk, k); // X^T as a col-major k x m matrix: column n is row n of X
+            }
+#pragma unroll
+            for(uint32_t i = 0; i < NB; ++i)
+#pragma unroll
+                for(uint32_t j = 0; j < NB; ++j)
+                    if(wanted(i, j))
+                        mma_sync(acc[i][j], a[i], b[j], acc[i][j]);
+        }
+        float* mine = block[wave];
+#pragma unroll
+        for(uint32_t i = 0; i < NB; ++i)
+#pragma unroll
+            for(uint32_t j = 0; j < NB; ++j)
+            {
+                if(!wanted(i, j))
+                    continue;
+                store_matrix_sync(mine, acc[i][j], BLK, mem_row_major);
+                __builtin_amdgcn_wave_barrier(); // (LDS is in order within a wave: the reads below see the block)
+#pragma unroll
+                for(uint32_t q = 0; q < BLK * BLK / 64u; ++q)
+                {
+                    const uint32_t e = q * 64u + lane, r = e / BLK, c = e % BLK;
+                    const uint64_t gi = (uint64_t)(si * NB + i) * BLK + r, gj = (uint64_t)(sj * NB + j) * BLK + c;
+                    if(gj < gi)
+                        o[k + gi * (gi - 1u) / 2u + gj] = static_cast<T>(mine[e]);
+                }
+                __builtin_amdgcn_wave_barrier(); // the block is rewritten by the next one
+            }
+    }
+
     // Backward.  Wave (ti, kc) of sample blockIdx.z owns block (ti, kc) of the gradient S X; S(i, j) is the upstream
     // triangle's element (max, min) of i, j and zero on the diagonal.
     template <typename T>
@@ -138,17 +220,154 @@ namespace
         }
     }
 
+    // Backward from 64 features on, or 64 embedding columns: a wave owns NBI x NBK blocks of the gradient - row blocks
+    // ti0 .. ti0 + NBI - 1, column blocks kc0 .. kc0 + NBK - 1 - so that every block of S it forms in LDS (256 gathers from
+    // the packed triangle with their index arithmetic) feeds NBK matrix instructions per K step instead of one, and every
+    // fragment of X NBI of them.
+    template <typename T, uint32_t NBI, uint32_t NBK>
+    __global__ void __launch_bounds__(THREADS) dlrmBwdGeneralBlocked(const T* __restrict__ in, const T* __restrict__ upstream,
+                                                                    T* __restrict__ mlpGrad, T* __restrict__ inGrad, uint32_t m, uint32_t k)
+    {
+        constexpr uint32_t BK = blockK<T>();
+        using FragA   = fragment<matrix_a, BLK, BLK, BK, T, row_major>;
+        using FragB   = fragment<matrix_b, BLK, BLK, BK, T, row_major>;
+        using FragAcc = fragment<accumulator, BLK, BLK, BK, float32_t>;
+        __shared__ T     sBlock[WAVES][NBI][BLK * BLK];
+        __shared__ float block[WAVES][BLK * BLK];
+
+        const uint32_t lane = threadIdx.x & 63u, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        const uint32_t kc0  = (blockIdx.x * WAVES + wave) * NBK, ti0 = blockIdx.y * NBI;
+        const uint32_t tilesK = k / BLK, tilesM = m / BLK;
+        if(kc0 >= tilesK)
+            return;
+        const uint64_t stride = (uint64_t)k + (uint64_t)m * (m - 1u) / 2u;
+        const T*       x      = in + (uint64_t)blockIdx.z * m * k;
+        const T*       up     = upstream + (uint64_t)blockIdx.z * stride;
+        const T*       tril   = up + k;
+
+        if(ti0 == 0u && lane < BLK) // bottom-MLP gradient: the first k values of the upstream row
+#pragma unroll
+            for(uint32_t c = 0; c < NBK; ++c)
+                if(kc0 + c < tilesK)
+                    mlpGrad[(uint64_t)blockIdx.z * k + (kc0 + c) * BLK + lane] = up[(kc0 + c) * BLK + lane];
+
+        FragAcc acc[NBI][NBK];
+#pragma unroll
+        for(uint32_t i = 0; i < NBI; ++i)
+#pragma unroll
+            for(uint32_t c = 0; c < NBK; ++c)
+                fill_fragment(acc[i][c], 0.0f);
+
+        // The step for column block tj of S works on values fetched one step before: the gathers from the packed triangle and
+        // the fragments of X for step tj + 1 are in flight while the matrix instructions of step tj run.  A lane gathers four
+        // elements of each block of S; below the diagonal a block's rows are contiguous in the triangle, above it its columns
+        // are, and the lanes are laid along whichever it is.
+        constexpr uint32_t PER_LANE = BLK * BLK / 64u, KSTEPS = BLK / BK;
+        T     sNext[NBI][PER_LANE];
+        FragB bNext[KSTEPS][NBK];
+        auto  place = [&](uint32_t i, uint32_t tj, uint32_t q, uint32_t& r, uint32_t& c) {
+            const uint32_t e = q * 64u + lane;
+            const bool upper = tj > ti0 + i;
+            r = upper ? e % BLK : e / BLK;
+            c = upper ? e / BLK : e % BLK;
+        };
+        auto fetch = [&](uint32_t tj) {
+#pragma unroll
+            for(uint32_t i = 0; i < NBI; ++i)
+#pragma unroll
+                for(uint32_t q = 0; q < PER_LANE; ++q)
+                {
+                    uint32_t r, c;
+                    place(i, tj, q, r, c);
+                    const uint64_t gi = (uint64_t)(ti0 + i < tilesM ? ti0 + i : ti0) * BLK + r, gj = (uint64_t)tj * BLK + c;
+                    const uint64_t hi = gi > gj ? gi : gj, lo = gi > gj ? gj : gi;
+                    sNext[i][q] = gi == gj ? static_cast<T>(0.0f) : tril[hi * (hi - 1u) / 2u + lo];
+                }
+#pragma unroll
+            for(uint32_t ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+                for(uint32_t c = 0; c < NBK; ++c) // (a column block past the end reads the last one again: its products are not used)
+                    load_matrix_sync(bNext[ks][c],
+                                     x + (uint64_t)tj * BLK * k + (uint64_t)(kc0 + c < tilesK ? kc0 + c : tilesK - 1u) * BLK + (uint64_t)ks * BK * k, k);
+        };
+        fetch(0u);
+        for(uint32_t tj = 0; tj < tilesM; ++tj)
+        {
+            FragB b[KSTEPS][NBK];
+#pragma unroll
+            for(uint32_t i = 0; i < NBI; ++i)
+#pragma unroll
+                for(uint32_t q = 0; q < PER_LANE; ++q)
+                {
+                    uint32_t r, c;
+                    place(i, tj, q, r, c);
+                    sBlock[wave][i][r * BLK + c] = sNext[i][q];
+                }
+#pragma unroll
+            for(uint32_t ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+                for(uint32_t c = 0; c < NBK; ++c)
+                    b[ks][c] = bNext[ks][c];
+            __builtin_amdgcn_wave_barrier();
+            if(tj + 1u < tilesM)
+                fetch(tj + 1u);
+#pragma unroll
+            for(uint32_t ks = 0; ks < KSTEPS; ++ks)
+            {
+                FragA a[NBI];
+#pragma unroll
+                for(uint32_t i = 0; i < NBI; ++i)
+                    load_matrix_sync(a[i], sBlock[wave][i] + ks * BK, BLK);
+#pragma unroll
+                for(uint32_t i = 0; i < NBI; ++i)
+#pragma unroll
+                    for(uint32_t c = 0; c < NBK; ++c)
+                        if(ti0 + i < tilesM && kc0 + c < tilesK)
+                            mma_sync(acc[i][c], a[i], b[ks][c], acc[i][c]);
+            }
+            __builtin_amdgcn_wave_barrier(); // the blocks of S are rewritten in the next trip
+        }
+        float* mine = block[wave];
+#pragma unroll
+        for(uint32_t i = 0; i < NBI; ++i)
+#pragma unroll
+            for(uint32_t c = 0; c < NBK; ++c)
+            {
+                if(ti0 + i >= tilesM || kc0 + c >= tilesK)
+                    continue;
+                store_matrix_sync(mine, acc[i][c], BLK, mem_row_major);
+                __builtin_amdgcn_wave_barrier();
+                T* g = inGrad + (uint64_t)blockIdx.z * m * k + (uint64_t)(ti0 + i) * BLK * k + (uint64_t)(kc0 + c) * BLK;
+#pragma unroll
+                for(uint32_t q = 0; q < BLK * BLK / 64u; ++q)
+                {
+                    const uint32_t e = q * 64u + lane, r = e / BLK, cc = e % BLK;
+                    g[(uint64_t)r * k + cc] = static_cast<T>(mine[e]);
+                }
+                __builtin_amdgcn_wave_barrier(); // the block is rewritten by the next one
+            }
+    }
+
     template <typename T>
     int fwd(const void* in, void* out, uint32_t m, uint32_t k, uint32_t batch, hipStream_t s)
     {
-        const uint32_t tiles = m / BLK, pairs = tiles * (tiles + 1u) / 2u;
+        constexpr uint32_t NB = 4;
+        const bool     blocked = m >= NB * BLK; // from 64 features on: NB x NB blocks per wave
+        const uint32_t tiles = blocked ? (m / BLK + NB - 1u) / NB : m / BLK, pairs = tiles * (tiles + 1u) / 2u;
         const uint64_t stride = (uint64_t)k + (uint64_t)m * (m - 1u) / 2u;
         // the batch is a grid dimension of at most 65535: a larger one goes out in several launches on the same stream
         for(uint32_t first = 0; first < batch; first += GRID_BATCH)
         {
             const uint32_t count = batch - first < GRID_BATCH ? batch - first : GRID_BATCH;
-            hipLaunchKernelGGL((dlrmFwdGeneral<T>), dim3((pairs + WAVES - 1u) / WAVES, count), dim3(THREADS), 0, s,
-                               static_cast<const T*>(in) + (uint64_t)first * m * k, static_cast<T*>(out) + (uint64_t)first * stride, m, k, pairs);
+            const dim3     grid((pairs + WAVES - 1u) / WAVES, count);
+            const T*       src = static_cast<const T*>(in) + (uint64_t)first * m * k;
+            T*             dst = static_cast<T*>(out) + (uint64_t)first * stride;
+            if(!blocked)
+                hipLaunchKernelGGL((dlrmFwdGeneral<T>), grid, dim3(THREADS), 0, s, src, dst, m, k, pairs);
+            else if(sizeof(T) == 2 && k % 32u == 0u)
+                hipLaunchKernelGGL((dlrmFwdGeneralBlocked<T, NB, sizeof(T) == 2 ? 32u : blockK<T>()>), grid, dim3(THREADS), 0, s, src, dst, m, k, pairs);
+            else
+                hipLaunchKernelGGL((dlrmFwdGeneralBlocked<T, NB, blockK<T>()>), grid, dim3(THREADS), 0, s, src, dst, m, k, pairs);
         }
         return r355::checkLaunch("dlrm_fwd (general)");
     }
@@ -159,9 +378,19 @@ namespace
         for(uint32_t first = 0; first < batch; first += GRID_BATCH)
         {
             const uint32_t count = batch - first < GRID_BATCH ? batch - first : GRID_BATCH;
-            hipLaunchKernelGGL((dlrmBwdGeneral<T>), dim3((k / BLK + WAVES - 1u) / WAVES, m / BLK, count), dim3(THREADS), 0, s,
-                               static_cast<const T*>(in) + (uint64_t)first * m * k, static_cast<const T*>(up) + (uint64_t)first * stride,
-                               static_cast<T*>(mlp) + (uint64_t)first * k, static_cast<T*>(grad) + (uint64_t)first * m * k, m, k);
+            constexpr uint32_t NBI = 2, NBK = 4;
+            const T*           src = static_cast<const T*>(in) + (uint64_t)first * m * k;
+            const T*           ups = static_cast<const T*>(up) + (uint64_t)first * stride;
+            T*                 dm  = static_cast<T*>(mlp) + (uint64_t)first * k;
+            T*                 dg  = static_cast<T*>(grad) + (uint64_t)first * m * k;
+            const uint64_t waves = (uint64_t)((k / BLK + NBK - 1u) / NBK) * ((m / BLK + NBI - 1u) / NBI) * count;
+            if(waves >= 8ull * r355::computeUnits()) // NBI x NBK blocks per wave, where that still leaves every SIMD two waves
+                hipLaunchKernelGGL((dlrmBwdGeneralBlocked<T, NBI, NBK>),
+                                   dim3(((k / BLK + NBK - 1u) / NBK + WAVES - 1u) / WAVES, (m / BLK + NBI - 1u) / NBI, count), dim3(THREADS), 0,
+                                   s, src, ups, dm, dg, m, k);
+            else
+                hipLaunchKernelGGL((dlrmBwdGeneral<T>), dim3((k / BLK + WAVES - 1u) / WAVES, m / BLK, count), dim3(THREADS), 0, s, src, ups, dm, dg,
+                                   m, k);
         }
         return r355::checkLaunch("dlrm_bwd (general)");
     }
