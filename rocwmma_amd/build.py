@@ -99,7 +99,7 @@ def build_variant(name, defines, verbose=True):
     """A measurement build (lib/variant_<name>/librocwmma_amd.so): the kernel sources that know measurement macros
     recompiled with `defines` (e.g. ["-DR355_ABLATE_MFMA"]).  `LD_LIBRARY_PATH=rocwmma_amd/lib/variant_<name>
     rocwmma_amd/lib/host_bench ...` then runs host_bench on it."""
-    return _build_twin("var_%s_" % name, list(defines), ["sparse.hip", "dlrm.hip"], os.path.join(LIBDIR, "variant_" + name, "librocwmma_amd.so"), verbose)
+    return _build_twin("var_%s_" % name, list(defines), ["sparse.hip", "dlrm.hip", "dlrm_general.hip"], os.path.join(LIBDIR, "variant_" + name, "librocwmma_amd.so"), verbose)
 
 
 def build_host_bench(verbose=True):

@@ -352,7 +352,14 @@ namespace
     int fwd(const void* in, void* out, uint32_t m, uint32_t k, uint32_t batch, hipStream_t s)
     {
         constexpr uint32_t NB = 4;
-        const bool     blocked = m >= NB * BLK; // from 64 features on: NB x NB blocks per wave
+#ifdef R355_DLRM_BLOCK_PER_WAVE // measurement build: the block-per-wave kernels for every shape
+        const bool blocked = false;
+#else
+        // NB x NB blocks per wave from 64 features on, where that still leaves every SIMD two waves or so (fewer, and the
+        // many short waves of the block-per-wave kernel hide latency better: 128 x 128 x 64 runs 8 us against 10)
+        const uint32_t supers  = (m / BLK + NB - 1u) / NB;
+        const bool     blocked = m >= NB * BLK && (uint64_t)supers * (supers + 1u) / 2u * batch >= 2ull * r355::computeUnits();
+#endif
         const uint32_t tiles = blocked ? (m / BLK + NB - 1u) / NB : m / BLK, pairs = tiles * (tiles + 1u) / 2u;
         const uint64_t stride = (uint64_t)k + (uint64_t)m * (m - 1u) / 2u;
         // the batch is a grid dimension of at most 65535: a larger one goes out in several launches on the same stream
@@ -384,7 +391,12 @@ namespace
             T*                 dm  = static_cast<T*>(mlp) + (uint64_t)first * k;
             T*                 dg  = static_cast<T*>(grad) + (uint64_t)first * m * k;
             const uint64_t waves = (uint64_t)((k / BLK + NBK - 1u) / NBK) * ((m / BLK + NBI - 1u) / NBI) * count;
-            if(waves >= 8ull * r355::computeUnits()) // NBI x NBK blocks per wave, where that still leaves every SIMD two waves
+#ifdef R355_DLRM_BLOCK_PER_WAVE
+            const bool blocked = false;
+#else
+            const bool blocked = waves >= 8ull * r355::computeUnits(); // where that still leaves every SIMD two waves
+#endif
+            if(blocked) // NBI x NBK blocks per wave
                 hipLaunchKernelGGL((dlrmBwdGeneralBlocked<T, NBI, NBK>),
                                    dim3(((k / BLK + NBK - 1u) / NBK + WAVES - 1u) / WAVES, (m / BLK + NBI - 1u) / NBI, count), dim3(THREADS), 0,
                                    s, src, ups, dm, dg, m, k);

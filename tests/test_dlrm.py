@@ -283,13 +283,14 @@ def test_bwd_integer_inputs_exact():
 @pytest.mark.parametrize("m,k,batch", [(128, 128, 64),   # the reference's own test sizes: test/dlrm/test/dlrm_test_params.hpp:57
                                        (1024, 1024, 2),  # (its fourth size with a smaller batch: the oracle's time)
                                        (48, 80, 9),      # 3 x 5 blocks of 16: neither a power of two
-                                       (80, 96, 5),      # 5 blocks: the forward kernel's 4 x 4 super-blocks, the second row of them partial
-                                       (112, 48, 3),     # 7 blocks; k not a multiple of 32 (16-bit: the 16-deep K step)
+                                       (256, 256, 64),   # the register-blocked kernels (they need a launch of 2 / 8 waves per CU), whole super-blocks
+                                       (80, 96, 700),    # 5 x 6 blocks: the forward kernel's 4 x 4 super-blocks and the backward kernel's 2 x 4 with partial edges
+                                       (112, 48, 600),   # 7 x 3 blocks; k not a multiple of 32 (16-bit: the 16-deep K step)
                                        (32, 512, 5),     # few features, an embedding width the specialised kernels have no instance for
                                        (16, 256, 7)])    # (f32: k = 256 is beyond the specialised f32 kernels)
 def test_general_shapes_fwd_and_bwd(dtype, m, k, batch):
-    """More than 32 features, or an embedding width other than 32 / 64 / 128 / 256: the block-per-wave kernels on the fragment
-    API.  Forward and backward against the oracle on the reference's metric (10 eps of the type); integer-valued inputs
+    """More than 32 features, or an embedding width other than 32 / 64 / 128 / 256: the block-per-wave and the register-blocked
+    kernels on the fragment API.  Forward and backward against the oracle on the reference's metric (10 eps of the type); integer-valued inputs
     must come out exactly."""
     if dtype != O.F32 and (m, k) == (16, 256):
         pytest.skip("the specialised 16-bit kernels take this shape")
