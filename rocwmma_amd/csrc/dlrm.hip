@@ -365,6 +365,91 @@ namespace
         }
     }
 
+    // f32 forward for up to 16 features, with the matrix instructions fed straight from the global loads: no LDS image of
+    // X.  Both operands of v_mfma_f32_16x16x4_f32 hold, in lane l, row l % 16 at k index l / 16 - and which four values
+    // of k one instruction sums is free as long as A and B agree.  Lane l therefore loads, for j = 0 .. K / 16 - 1, the 16
+    // bytes X[l % 16][16 j + 4 (l / 16) ...] (rows from m on lie beyond the sample's buffer and arrive as zeros), and
+    // instruction t of step j takes element t of those vectors as both operands: it sums k = 16 j + 4 q + t over q.  A
+    // sample is K / 16 vector registers per lane, the registers the loads arrive in are the operand file of the K / 4
+    // matrix instructions (on two accumulator chains), and the next sample is requested into them as soon as those have
+    // issued.  What stays in LDS is the image of the output row, so registers set the occupancy: four waves per SIMD.
+    // A load instruction covers 64 bytes of each of 16 rows, and the other half of every cache line comes with the next
+    // instruction: ordinary loads, which keep the line for it, not streaming ones (7 - 15 % faster here).
+    // The kernel above always computes the three blocks of 32 rows; with 16 rows or fewer this one does a third of the
+    // matrix work and holds four times the samples in flight per CU (batch 65536, k = 128: m = 16 0.166 -> 0.108 ms,
+    // m = 8 0.142 -> 0.054 ms).  From 17 features on - the second block of rows doubles the registers and the 64-byte
+    // pieces per sample - it is no faster than the LDS image (27 x 128: 0.214 against 0.216 ms, 32 x 128: 0.245 against
+    // 0.226), and that one stays.
+    constexpr uint32_t F32_DIRECT_STEPS = 2; // samples per wave
+    template <uint32_t K>
+    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4)))
+        dlrmFwdF32Direct(const float* __restrict__ in, float* __restrict__ out, uint32_t m, uint32_t batch)
+    {
+        constexpr uint32_t JS        = K / 16u; // 128-bit loads per lane and sample
+        constexpr uint32_t MAX_OUT   = K + 16u * 15u / 2u;
+        constexpr uint32_t OUT_STEPS = (MAX_OUT + 63u) / 64u; // 4-byte stores per lane and sample
+        using f32x4                  = float __attribute__((ext_vector_type(4)));
+
+        __shared__ __attribute__((aligned(16))) float outLds[WAVES][OUT_STEPS * 64u];
+
+        const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const uint32_t outStride = K + m * (m - 1u) / 2u;
+        const uint32_t inBytes   = m * K * 4u;
+        const uint32_t first = blockIdx.x * WAVES + wave, stride = gridDim.x * WAVES;
+        float*         o     = outLds[wave];
+        const uint32_t r16 = lane & 15u, kq = lane >> 4;
+        const uint32_t off = r16 * K * 4u + kq * 16u;
+
+        f32x4 x[JS];
+        // (a sample beyond the batch is a buffer of no bytes: the loads are issued and move nothing)
+        auto request = [&](uint64_t b) {
+            const bool valid = b < batch;
+            const auto src   = runBuffer(in, (uint64_t)(valid ? b : 0u) * inBytes, valid ? inBytes : 0u);
+#pragma unroll
+            for(uint32_t j = 0; j < JS; ++j)
+                x[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(src, off + j * 64u, 0, 0));
+        };
+        if(first >= batch)
+            return;
+        request(first);
+#pragma unroll 1
+        for(uint64_t b = first; b < batch; b += stride)
+        {
+            f32x4 acc0 = {0, 0, 0, 0}, acc1 = acc0;
+#pragma unroll
+            for(uint32_t j = 0; j < JS; ++j)
+            {
+                if(r16 == 0u) // the sample's first row is the head of its output row
+                    *reinterpret_cast<f32x4*>(o + j * 16u + kq * 4u) = x[j];
+                acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(x[j][0], x[j][0], acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(x[j][1], x[j][1], acc1, 0, 0, 0);
+                acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(x[j][2], x[j][2], acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(x[j][3], x[j][3], acc1, 0, 0, 0);
+            }
+            acc0 += acc1;
+            __builtin_amdgcn_sched_barrier(0);
+            request(b + stride); // the registers are free again
+            __builtin_amdgcn_sched_barrier(0);
+
+            // the 16 x 16 result block: a lane holds rows 4 (lane / 16) + e of column lane % 16
+#pragma unroll
+            for(uint32_t e = 0; e < 4; ++e)
+            {
+                const uint32_t i = 4u * kq + e, j = r16;
+                if(j < i && i < m)
+                    o[K + i * (i - 1u) / 2u + j] = acc0[e];
+            }
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_wave_barrier();
+            const auto dst = runBuffer(out, b * outStride * 4u, outStride * 4u);
+#pragma unroll
+            for(uint32_t e = 0; e < OUT_STEPS; ++e)
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, o[e * 64u + lane]), dst, (e * 64u + lane) * 4u, 0, STORE_POLICY);
+            __builtin_amdgcn_s_waitcnt(0xC07F); // the image is rewritten by the next sample
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
+
     // Backward: S = T + T^T (T = strict lower triangle from the upstream gradient, zero diagonal),
     // grad (m x k) = S X.  Same organisation as the forward kernel: a workgroup owns 8 consecutive
     // samples (their upstream rows form one 16-byte aligned run, staged in LDS with 128-bit loads),
@@ -754,9 +839,20 @@ extern "C" int r355_dlrm_fwd(int32_t dtype, const void* in, void* out, uint32_t 
     if(dtype == R355_F32)
     {
         const uint32_t steps = (batch + WAVES - 1) / WAVES; // of one sample per wave
-        const dim3     grid32((steps + F32_STEPS - 1) / F32_STEPS), block32(THREADS);
         auto*      fi = static_cast<const float*>(in);
         auto*      fo = static_cast<float*>(out);
+        if(m <= 16) // a single block of rows: matrix instructions straight from the loads
+        {
+            const dim3 grid((steps + F32_DIRECT_STEPS - 1) / F32_DIRECT_STEPS), block(THREADS);
+            switch(k)
+            {
+            case 32: hipLaunchKernelGGL((dlrmFwdF32Direct<32>), grid, block, 0, s, fi, fo, m, batch); break;
+            case 64: hipLaunchKernelGGL((dlrmFwdF32Direct<64>), grid, block, 0, s, fi, fo, m, batch); break;
+            default: hipLaunchKernelGGL((dlrmFwdF32Direct<128>), grid, block, 0, s, fi, fo, m, batch); break;
+            }
+            return r355::checkLaunch("dlrm_fwd");
+        }
+        const dim3     grid32((steps + F32_STEPS - 1) / F32_STEPS), block32(THREADS);
 #define R355_FWD32(KK)                                                                                \
     do                                                                                                \
     {                                                                                                 \
