@@ -365,28 +365,28 @@ namespace
         }
     }
 
-    // f32 forward for up to 16 features, with the matrix instructions fed straight from the global loads: no LDS image of
-    // X.  Both operands of v_mfma_f32_16x16x4_f32 hold, in lane l, row l % 16 at k index l / 16 - and which four values
-    // of k one instruction sums is free as long as A and B agree.  Lane l therefore loads, for j = 0 .. K / 16 - 1, the 16
-    // bytes X[l % 16][16 j + 4 (l / 16) ...] (rows from m on lie beyond the sample's buffer and arrive as zeros), and
-    // instruction t of step j takes element t of those vectors as both operands: it sums k = 16 j + 4 q + t over q.  A
-    // sample is K / 16 vector registers per lane, the registers the loads arrive in are the operand file of the K / 4
-    // matrix instructions (on two accumulator chains), and the next sample is requested into them as soon as those have
-    // issued.  What stays in LDS is the image of the output row, so registers set the occupancy: four waves per SIMD.
-    // A load instruction covers 64 bytes of each of 16 rows, and the other half of every cache line comes with the next
-    // instruction: ordinary loads, which keep the line for it, not streaming ones (7 - 15 % faster here).
-    // The kernel above always computes the three blocks of 32 rows; with 16 rows or fewer this one does a third of the
-    // matrix work and holds four times the samples in flight per CU (batch 65536, k = 128: m = 16 0.166 -> 0.108 ms,
-    // m = 8 0.142 -> 0.054 ms).  From 17 features on - the second block of rows doubles the registers and the 64-byte
-    // pieces per sample - it is no faster than the LDS image (27 x 128: 0.214 against 0.216 ms, 32 x 128: 0.245 against
-    // 0.226), and that one stays.
+    // f32 forward with the matrix instructions fed straight from the global loads: no LDS image of X.  Both operands of
+    // v_mfma_f32_16x16x4_f32 hold, in lane l, row l % 16 of a block of rows at k index l / 16 - and which four values of k
+    // one instruction sums is free as long as A and B agree.  Lane l therefore loads, for j = 0 .. K / 16 - 1, the 16
+    // bytes X[l % 16][16 j + 4 (l / 16) ...] (and, HIGH, the same of row 16 + l % 16; rows from m on lie beyond the
+    // sample's buffer and arrive as zeros), and instruction t of step j takes element t of those vectors: it sums
+    // k = 16 j + 4 q + t over q.  The registers the loads arrive in are the operand file of the matrix instructions, and
+    // the next sample is requested into them as soon as those have issued.  What stays in LDS is the image of the output
+    // row, so registers set the occupancy (eight waves per SIMD up to 16 features, four beyond).
+    // Every lane's 16 bytes are a memory access of their own here (neighbouring lanes are a row apart), and the other
+    // half of each cache line comes with the next instruction: ordinary loads, which keep the line for it, not streaming
+    // ones (7 - 15 % faster), and a rate that stops near 0.70 of the HBM peak for k = 64 and 128 whatever m is, where the
+    // LDS image's coalesced loads reach 0.72 - 0.80 once m is near 32.  Up to 16 features this kernel does a third of the
+    // matrix work of the one above, which always computes three blocks (batch 65536, k = 128: m = 16 0.144 -> 0.109 ms,
+    // m = 8 0.136 -> 0.048 ms); which of the two runs beyond 16 is decided by the launcher.
     constexpr uint32_t F32_DIRECT_STEPS = 2; // samples per wave
-    template <uint32_t K>
+    template <uint32_t K, bool HIGH = false>
     __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(4)))
         dlrmFwdF32Direct(const float* __restrict__ in, float* __restrict__ out, uint32_t m, uint32_t batch)
     {
         constexpr uint32_t JS        = K / 16u; // 128-bit loads per lane and sample
-        constexpr uint32_t MAX_OUT   = K + 16u * 15u / 2u;
+        constexpr uint32_t ROWS      = HIGH ? 32u : 16u;
+        constexpr uint32_t MAX_OUT   = K + ROWS * (ROWS - 1u) / 2u;
         constexpr uint32_t OUT_STEPS = (MAX_OUT + 63u) / 64u; // 4-byte stores per lane and sample
         using f32x4                  = float __attribute__((ext_vector_type(4)));
 
@@ -400,14 +400,18 @@ namespace
         const uint32_t r16 = lane & 15u, kq = lane >> 4;
         const uint32_t off = r16 * K * 4u + kq * 16u;
 
-        f32x4 x[JS];
+        f32x4 x[JS], hi[HIGH ? JS : 1u];
         // (a sample beyond the batch is a buffer of no bytes: the loads are issued and move nothing)
         auto request = [&](uint64_t b) {
             const bool valid = b < batch;
             const auto src   = runBuffer(in, (uint64_t)(valid ? b : 0u) * inBytes, valid ? inBytes : 0u);
 #pragma unroll
             for(uint32_t j = 0; j < JS; ++j)
+            {
                 x[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(src, off + j * 64u, 0, 0));
+                if constexpr(HIGH)
+                    hi[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(src, off + 16u * K * 4u + j * 64u, 0, 0));
+            }
         };
         if(first >= batch)
             return;
@@ -415,12 +419,23 @@ namespace
 #pragma unroll 1
         for(uint64_t b = first; b < batch; b += stride)
         {
-            f32x4 acc0 = {0, 0, 0, 0}, acc1 = acc0;
+            f32x4 acc0 = {0, 0, 0, 0}, acc1 = acc0, accHL = acc0, accHH = acc0;
 #pragma unroll
             for(uint32_t j = 0; j < JS; ++j)
             {
                 if(r16 == 0u) // the sample's first row is the head of its output row
                     *reinterpret_cast<f32x4*>(o + j * 16u + kq * 4u) = x[j];
+                if constexpr(HIGH)
+                {
+#pragma unroll
+                    for(uint32_t t = 0; t < 4u; ++t)
+                    {
+                        acc0  = __builtin_amdgcn_mfma_f32_16x16x4f32(x[j][t], x[j][t], acc0, 0, 0, 0);
+                        accHL = __builtin_amdgcn_mfma_f32_16x16x4f32(hi[j][t], x[j][t], accHL, 0, 0, 0);
+                        accHH = __builtin_amdgcn_mfma_f32_16x16x4f32(hi[j][t], hi[j][t], accHH, 0, 0, 0);
+                    }
+                    continue;
+                }
                 acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(x[j][0], x[j][0], acc0, 0, 0, 0);
                 acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(x[j][1], x[j][1], acc1, 0, 0, 0);
                 acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(x[j][2], x[j][2], acc0, 0, 0, 0);
@@ -438,6 +453,16 @@ namespace
                 const uint32_t i = 4u * kq + e, j = r16;
                 if(j < i && i < m)
                     o[K + i * (i - 1u) / 2u + j] = acc0[e];
+                if constexpr(HIGH)
+                {
+                    const uint32_t ih = 16u + i;
+                    if(ih < m)
+                    {
+                        o[K + ih * (ih - 1u) / 2u + j] = accHL[e];
+                        if(j < i)
+                            o[K + ih * (ih - 1u) / 2u + 16u + j] = accHH[e];
+                    }
+                }
             }
             __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_wave_barrier();
@@ -841,15 +866,35 @@ extern "C" int r355_dlrm_fwd(int32_t dtype, const void* in, void* out, uint32_t 
         const uint32_t steps = (batch + WAVES - 1) / WAVES; // of one sample per wave
         auto*      fi = static_cast<const float*>(in);
         auto*      fo = static_cast<float*>(out);
-        if(m <= 16) // a single block of rows: matrix instructions straight from the loads
+        // Matrix instructions straight from the loads (dlrmFwdF32Direct) or out of an LDS image of X (dlrmFwdF32Kernel): the
+        // first up to 16 features, where it runs one block of rows instead of three, and beyond that where the image's
+        // padding to 28 or 32 rows costs more than the direct kernel's scattered 16-byte pieces (measured over m = 17 .. 32
+        // at a batch of 65536: k = 32 always, k = 64 up to 21 features, k = 128 up to 24).  Measurement builds force either.
+#if defined(R355_DLRM_F32_LDS_IMAGE)
+        const bool direct = false;
+#elif defined(R355_DLRM_F32_DIRECT_ALL)
+        const bool direct = true;
+#else
+        const bool direct = m <= 16 || k == 32 || (k == 64 && m <= 21) || (k == 128 && m <= 24);
+#endif
+        if(direct)
         {
             const dim3 grid((steps + F32_DIRECT_STEPS - 1) / F32_DIRECT_STEPS), block(THREADS);
+#define R355_FWD32D(KK)                                                                              \
+    do                                                                                               \
+    {                                                                                                \
+        if(m <= 16)                                                                                  \
+            hipLaunchKernelGGL((dlrmFwdF32Direct<KK, false>), grid, block, 0, s, fi, fo, m, batch);  \
+        else                                                                                         \
+            hipLaunchKernelGGL((dlrmFwdF32Direct<KK, true>), grid, block, 0, s, fi, fo, m, batch);   \
+    } while(0)
             switch(k)
             {
-            case 32: hipLaunchKernelGGL((dlrmFwdF32Direct<32>), grid, block, 0, s, fi, fo, m, batch); break;
-            case 64: hipLaunchKernelGGL((dlrmFwdF32Direct<64>), grid, block, 0, s, fi, fo, m, batch); break;
-            default: hipLaunchKernelGGL((dlrmFwdF32Direct<128>), grid, block, 0, s, fi, fo, m, batch); break;
+            case 32: R355_FWD32D(32); break;
+            case 64: R355_FWD32D(64); break;
+            default: R355_FWD32D(128); break;
             }
+#undef R355_FWD32D
             return r355::checkLaunch("dlrm_fwd");
         }
         const dim3     grid32((steps + F32_STEPS - 1) / F32_STEPS), block32(THREADS);

@@ -42,6 +42,10 @@ def _rel(a, b):
 # and of the fixture in the reference's relative-error metric, and no further from the float64-exact
 # value than 1.5 x the sequential-f32 oracle's own distance from it.
 F32_TOL_EPS = 40.0
+# Unit-normal inputs (the shape tests below) put the terms of a dot product an order of magnitude above the reference's fixture
+# data: over 10^4 results the largest difference between two orders of summation reaches 41 - 46 eps in that metric for either
+# f32 kernel (16 x 128 x 64, 25 x 128 x 64).  Their bar against the oracle is 80 eps; the sharp one is the distance from the exact value.
+F32_NORMAL_TOL_EPS = 80.0
 
 
 def _check_f32(got, want_oracle, x, m, k, batch, tol_eps=F32_TOL_EPS):
@@ -68,7 +72,9 @@ def test_fwd_reference_fixture_fp32():
 
 
 @pytest.mark.parametrize("m,k,batch", [(32, 32, 64), (27, 128, 13), (2, 64, 5), (32, 128, 3), (17, 128, 70),
-                                       # up to 16 features: the kernel that feeds the matrix instructions from the loads
+                                       # the kernel that feeds the matrix instructions from the loads: every instance (k, one or two
+                                       # blocks of rows), the last shapes it takes (21 x 64, 24 x 128) and the first it leaves (22, 25)
+                                       (32, 32, 700), (17, 32, 33), (21, 64, 70), (22, 64, 70), (24, 128, 64), (25, 128, 64), (20, 128, 515),
                                        (16, 128, 64), (16, 128, 1000), (16, 32, 9), (8, 128, 517), (13, 64, 2049), (2, 32, 3), (5, 128, 1)])
 def test_fwd_f32_shapes_vs_oracle(m, k, batch):
     x = O.normal(3, batch * m * k)
@@ -80,9 +86,7 @@ def test_fwd_f32_shapes_vs_oracle(m, k, batch):
     assert np.all(out[want.size:].view(np.uint8) == 0xEE)
     got = out[:want.size].reshape(batch, -1)
     if batch <= 100:
-        # Up to 16 features the kernel adds k in two interleaved chains of steps that are themselves strided through k: further
-        # from the oracle's sequential order than the other f32 kernels' (16 x 128 x 64: 41 eps), no further from the exact value
-        _check_f32(got, want, x, m, k, batch, F32_TOL_EPS if m > 16 else 2.0 * F32_TOL_EPS)
+        _check_f32(got, want, x, m, k, batch, F32_NORMAL_TOL_EPS)
     else:
         # The largest of 10^5 differences between two orders of summation passes no fixed number of eps, and the largest distance
         # from the exact value is one element's luck (16 x 128 x 1000: 9.4e-6 against the oracle's 5.2e-6 in the reference's
