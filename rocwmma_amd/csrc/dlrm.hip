@@ -94,9 +94,13 @@ namespace
     // K is a template parameter (32, 64, 128, 256): rows of X are K * 2 bytes = K / 8 chunks.
     // ROWS (28 or 32) bounds m: the LDS image of a sample holds ROWS rows, which at m <= 28 and
     // K = 128 lets four workgroups share a CU instead of three.
+    // Few features: `pack` consecutive samples (pack * m <= ROWS rows, contiguous in memory) are taken as one block of
+    // rows.  The Gram matrix of the stacked rows holds each sample's own on its diagonal - the products across samples are
+    // computed and dropped - so loads, LDS image and matrix instructions are those of one large sample, and a workgroup's
+    // 8 * pack output rows are still one run of bytes.  (m = 8, k = 128 at a batch of 65536: four samples per block.)
     template <bool BF16, uint32_t K, uint32_t ROWS>
     __global__ void __launch_bounds__(THREADS)
-        dlrmFwdKernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out, uint32_t m, uint32_t batch)
+        dlrmFwdKernel(const uint16_t* __restrict__ in, uint16_t* __restrict__ out, uint32_t m, uint32_t batch, uint32_t pack)
     {
         constexpr uint32_t ROW_CHUNKS = K / 8; // 16-byte chunks per row
         constexpr uint32_t X_BYTES    = ROWS * K * 2; // LDS image of one sample
@@ -109,8 +113,10 @@ namespace
         const uint32_t lane      = tid & 63u;
         const uint32_t wave      = __builtin_amdgcn_readfirstlane(tid >> 6);
         const uint32_t outStride = K + m * (m - 1) / 2; // elements per sample
-        const uint32_t b0        = blockIdx.x * SAMPLES_PER_WG;
+        const uint32_t b0        = blockIdx.x * SAMPLES_PER_WG * pack;
         const uint32_t inBytes   = m * K * 2u; // of one sample
+        const uint32_t rows      = m * pack; // of one block
+        const uint32_t rcpM      = (65536u + m - 1u) / m; // i / m == (i * rcpM) >> 16 for i < 32
 
         char* xw = xLds[wave];
         // rows m..31 of the 32 x 32 product are padding: their lanes feed zeros (see below)
@@ -129,8 +135,9 @@ namespace
 #pragma unroll
         for(uint32_t q = 0; q < PER_WAVE; ++q)
         {
-            const uint32_t b   = b0 + wave + q * WAVES;
-            const auto     src = runBuffer(in, (uint64_t)(b < batch ? b : 0u) * inBytes, b < batch ? inBytes : 0u);
+            const uint32_t b   = b0 + (wave + q * WAVES) * pack; // the block's first sample
+            const uint32_t has = b < batch ? (batch - b < pack ? batch - b : pack) : 0u;
+            const auto     src = runBuffer(in, (uint64_t)(has ? b : 0u) * inBytes, has * inBytes);
 #pragma unroll
             for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
                 stash[q][j] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (j * 64u + lane) * 16u, 0, LOAD_POLICY)); // read once
@@ -140,7 +147,7 @@ namespace
         for(uint32_t q = 0; q < PER_WAVE; ++q)
         {
             const uint32_t sIdx = wave + q * WAVES;
-            const uint32_t b    = b0 + sIdx;
+            const uint32_t b    = b0 + sIdx * pack;
             if(b >= batch)
                 break;
             // ---- X -> LDS: chunk c of the sample goes to row c / ROW_CHUNKS, slot (c % ROW_CHUNKS) ^ (row % 16)
@@ -161,7 +168,7 @@ namespace
 
             // ---- Gram matrix: acc(i, j) = sum_k X(i, k) X(j, k)
             f32x16         acc   = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-            const bool     valid = (lane & 31u) < m;
+            const bool     valid = (lane & 31u) < rows;
             const uint32_t row   = valid ? (lane & 31u) : 0u; // padding lanes read row 0 and discard it
 #pragma unroll
             for(uint32_t s = 0; s < K / 16; ++s)
@@ -175,16 +182,21 @@ namespace
             }
 
             // ---- output image: first row, then strict lower triangle (i, j < i) row-major
-            uint16_t* o = outLds + sIdx * outStride;
-            for(uint32_t e = lane; e < K; e += 64)
-                o[e] = reinterpret_cast<const uint16_t*>(xw)[e]; // row 0 is stored unswizzled
-            const uint32_t j = lane & 31u;
+            uint16_t* o = outLds + sIdx * pack * outStride; // the block's samples one after the other
+            for(uint32_t e = lane; e < pack * K; e += 64)
+            {
+                const uint32_t s = e / K, c = e % K, row = s * m; // a sample's first row is the head of its output row
+                const uint32_t slot = (c / 8u) ^ (row & (ROW_CHUNKS - 1u) & 15u);
+                o[s * outStride + c] = reinterpret_cast<const uint16_t*>(xw)[(row * ROW_CHUNKS + slot) * 8u + c % 8u];
+            }
+            const uint32_t j = lane & 31u, sj = (j * rcpM) >> 16, lj = j - sj * m;
 #pragma unroll
             for(uint32_t r = 0; r < 16; ++r)
             {
                 const uint32_t i = 8u * (r >> 2) + 4u * (lane >> 5) + (r & 3u);
-                if(j < i && i < m)
-                    o[K + i * (i - 1u) / 2u + j] = roundOut<BF16>(acc[r]);
+                const uint32_t si = (i * rcpM) >> 16, li = i - si * m; // sample within the block, row within the sample
+                if(si == sj && lj < li && i < rows)
+                    o[si * outStride + K + li * (li - 1u) / 2u + lj] = roundOut<BF16>(acc[r]);
             }
             __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_wave_barrier();
@@ -192,7 +204,7 @@ namespace
         __syncthreads();
 
         // ---- coalesced copy-out of the workgroup's samples
-        const uint32_t nSamples = (batch - b0) < SAMPLES_PER_WG ? (batch - b0) : SAMPLES_PER_WG;
+        const uint32_t nSamples = (batch - b0) < SAMPLES_PER_WG * pack ? (batch - b0) : SAMPLES_PER_WG * pack;
         const uint32_t total    = nSamples * outStride; // elements
         uint16_t*      dst      = out + (uint64_t)b0 * outStride;
         const uint32_t vecs     = total / 8u;
@@ -492,8 +504,11 @@ namespace
                                                             uint16_t* __restrict__ mlpGrad,
                                                             uint16_t* __restrict__ inGrad,
                                                             uint32_t m,
-                                                            uint32_t batch)
+                                                            uint32_t batch,
+                                                            uint32_t pack)
     {
+        // (`pack` consecutive samples of few features as one block of rows, as in the forward kernel: S of the block is
+        // block-diagonal, X and the gradient are the samples' rows one after the other)
         constexpr uint32_t ROW_CHUNKS = K / 8; // 16-byte chunks per row
         constexpr uint32_t ROWB       = K * 2;
         constexpr uint32_t X_BYTES    = MAX_M * ROWB; // always 32 rows: rows >= m stay zero
@@ -514,9 +529,11 @@ namespace
         const uint32_t lane     = tid & 63u;
         const uint32_t wave     = __builtin_amdgcn_readfirstlane(tid >> 6);
         const uint32_t upStride = K + m * (m - 1) / 2;
-        const uint32_t b0       = blockIdx.x * SAMPLES_PER_WG;
-        const uint32_t inChunks = m * ROW_CHUNKS;
-        const uint32_t inBytes  = inChunks * 16u;
+        const uint32_t b0       = blockIdx.x * SAMPLES_PER_WG * pack;
+        const uint32_t rows     = m * pack; // of a block
+        const uint32_t inChunks = rows * ROW_CHUNKS;
+        const uint32_t inBytes  = m * ROW_CHUNKS * 16u; // of a sample
+        const uint32_t rcpM     = (65536u + m - 1u) / m; // i / m == (i * rcpM) >> 16 for i < 32
         char*          xw       = xLds[wave];
 
         // Everything the workgroup reads is requested at once, through raw buffers of exactly the bytes that exist (runBuffer):
@@ -526,15 +543,16 @@ namespace
 #pragma unroll
         for(uint32_t q = 0; q < PER_WAVE; ++q)
         {
-            const uint32_t b   = b0 + wave + q * WAVES;
-            const auto     src = runBuffer(in, (uint64_t)(b < batch ? b : 0u) * inBytes, b < batch ? inBytes : 0u);
+            const uint32_t b   = b0 + (wave + q * WAVES) * pack; // the block's first sample
+            const uint32_t has = b < batch ? (batch - b < pack ? batch - b : pack) : 0u;
+            const auto     src = runBuffer(in, (uint64_t)(has ? b : 0u) * inBytes, has * inBytes);
 #pragma unroll
             for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
                 stash[q][j] = __builtin_bit_cast(i32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (j * 64u + lane) * 16u, 0, LOAD_POLICY));
         }
 
         // ---- upstream rows of the workgroup's samples -> LDS; zero rows m..31 of the X image
-        const uint32_t nSamples = (batch - b0) < SAMPLES_PER_WG ? (batch - b0) : SAMPLES_PER_WG;
+        const uint32_t nSamples = (batch - b0) < SAMPLES_PER_WG * pack ? (batch - b0) : SAMPLES_PER_WG * pack;
         {
             // the run is a whole number of 16-byte pieces unless the batch ends inside this workgroup; whole 4-byte words go
             // through the buffer (its range check works on words), a last odd element on its own
@@ -576,10 +594,12 @@ namespace
         for(uint32_t q = 0; q < PER_WAVE; ++q)
         {
             const uint32_t sIdx = wave + q * WAVES;
-            const uint32_t b    = b0 + sIdx;
+            const uint32_t b    = b0 + sIdx * pack;
             if(b >= batch)
                 break;
+            const uint32_t has = batch - b < pack ? batch - b : pack; // samples of this block
             // ---- X -> LDS: chunk c goes to row j = c / ROW_CHUNKS, slot (c % ROW_CHUNKS) ^ ((j & 3) << 2)
+            // (the rows of samples beyond the batch arrived as zeros and are written like the others)
 #pragma unroll
             for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
             {
@@ -591,7 +611,8 @@ namespace
                 }
             }
             // ---- S operand: lane holds S(i, j) for its 8-wide runs of j (zero diagonal, zero padding)
-            const uint16_t* tril = upLds + sIdx * upStride + K;
+            const uint16_t* tril = upLds + sIdx * pack * upStride + K; // of the block's first sample
+            const uint32_t  si = (i * rcpM) >> 16, li = i - si * m; // the lane's row: sample within the block, row within it
             i32x4           sReg[2];
 #pragma unroll
             for(uint32_t s = 0; s < 2; ++s)
@@ -605,10 +626,11 @@ namespace
                 for(uint32_t e = 0; e < 8; ++e)
                 {
                     const uint32_t j  = 16u * s + 8u * half + e;
-                    const uint32_t hi = i > j ? i : j, lo = i > j ? j : i;
+                    const uint32_t sj = (j * rcpM) >> 16, lj = j - sj * m;
+                    const uint32_t hi = li > lj ? li : lj, lo = li > lj ? lj : li;
                     uint16_t       v  = 0;
-                    if(hi < m && hi != lo)
-                        v = tril[hi * (hi - 1u) / 2u + lo];
+                    if(si == sj && si < has && hi != lo)
+                        v = tril[si * upStride + hi * (hi - 1u) / 2u + lo];
                     so.h[e] = v;
                 }
                 sReg[s] = so.v;
@@ -637,8 +659,8 @@ namespace
             __builtin_amdgcn_s_waitcnt(0xC07F); // every read of X has returned before rows are overwritten
             __builtin_amdgcn_wave_barrier();
 
-            // ---- gradient image over rows < m: lane has c = 32 slab + 8 r + 4 half + (0..3) of row i
-            if(i < m)
+            // ---- gradient image over the block's rows: lane has c = 32 slab + 8 r + 4 half + (0..3) of row i
+            if(i < rows)
             {
 #pragma unroll
                 for(uint32_t slab = 0; slab < SLABS; ++slab)
@@ -665,7 +687,7 @@ namespace
             for(uint32_t j = 0; j < MAX_CHUNKS; ++j)
             {
                 const uint32_t c = j * 64u + lane;
-                if(c < inChunks)
+                if(c < has * m * ROW_CHUNKS)
                 {
                     const uint32_t row = c / ROW_CHUNKS, col = c % ROW_CHUNKS;
                     const i32x4    v   = *reinterpret_cast<const i32x4*>(xw + (row * ROW_CHUNKS + (col ^ (row & SWZ_OUT))) * 16u);
@@ -846,6 +868,32 @@ namespace
     }
     // the kernels of this file: up to 32 features and an embedding width they are instantiated for; everything else goes
     // to the block-per-wave kernels of dlrm_general.hip
+    // 16-bit kernels, up to 16 features: the samples that share a block of rows - as many as fit the rows of the LDS image
+    // (28 or 32: `small` says which instance) and, with their output / upstream rows, the space of that image's one
+    // full-size sample's row.  The 32-row instance where it takes more samples per block - except at k = 128, where the
+    // 28-row image lets four workgroups share a CU instead of three and fewer samples per block are still faster
+    // (forward, m = 16: 0.79 against 0.73 of the HBM peak, m = 8: 0.77 against 0.74).
+    uint32_t samplesPerBlock(uint32_t m, uint32_t k, bool& small)
+    {
+#ifdef R355_DLRM_NO_PACK // (measurement build: one sample per block whatever m is)
+        return 1u;
+#endif
+        if(m > 16)
+            return 1u;
+        auto fits = [&](uint32_t rows) {
+            const uint32_t byRows = rows / m, byRow = (k + rows * (rows - 1u) / 2u) / (k + m * (m - 1u) / 2u);
+            return byRows < byRow ? byRows : byRow;
+        };
+        const uint32_t p28 = fits(28), p32 = fits(32);
+#if defined(R355_DLRM_PACK_PREFER_28) // (measurement builds: always the 28-row image / always the one with more samples)
+        small = true;
+#elif defined(R355_DLRM_PACK_MORE_SAMPLES)
+        small = p28 == p32;
+#else
+        small = p28 == p32 || k == 128;
+#endif
+        return small ? p28 : p32;
+    }
     bool specialised(int32_t dtype, uint32_t m, uint32_t k)
     {
         return m <= MAX_M && (k == 32 || k == 64 || k == 128 || (k == 256 && dtype != R355_F32));
@@ -915,16 +963,18 @@ extern "C" int r355_dlrm_fwd(int32_t dtype, const void* in, void* out, uint32_t 
 #undef R355_FWD32
         return r355::checkLaunch("dlrm_fwd");
     }
-    const dim3 grid((batch + SAMPLES_PER_WG - 1) / SAMPLES_PER_WG), block(THREADS);
+    bool           small = m <= 28;
+    const uint32_t pack  = samplesPerBlock(m, k, small);
+    const dim3 grid((batch + SAMPLES_PER_WG * pack - 1) / (SAMPLES_PER_WG * pack)), block(THREADS);
     auto*       pi = static_cast<const uint16_t*>(in);
     auto*       po = static_cast<uint16_t*>(out);
-#define R355_FWD(BF, KK)                                                                         \
-    do                                                                                            \
-    {                                                                                             \
-        if(m <= 28)                                                                               \
-            hipLaunchKernelGGL((dlrmFwdKernel<BF, KK, 28>), grid, block, 0, s, pi, po, m, batch); \
-        else                                                                                      \
-            hipLaunchKernelGGL((dlrmFwdKernel<BF, KK, 32>), grid, block, 0, s, pi, po, m, batch); \
+#define R355_FWD(BF, KK)                                                                               \
+    do                                                                                                  \
+    {                                                                                                   \
+        if(small)                                                                                       \
+            hipLaunchKernelGGL((dlrmFwdKernel<BF, KK, 28>), grid, block, 0, s, pi, po, m, batch, pack); \
+        else                                                                                            \
+            hipLaunchKernelGGL((dlrmFwdKernel<BF, KK, 32>), grid, block, 0, s, pi, po, m, batch, pack); \
     } while(0)
 #define R355_FWD_K(BF)   \
     switch(k)            \
@@ -979,7 +1029,9 @@ extern "C" int r355_dlrm_bwd(int32_t dtype, const void* in, const void* upstream
     }
     if(!r355::aligned(upstream, 16) || !r355::aligned(mlp_grad, 16))
         return r355::fail(R355_ERR_MISALIGNED, "dlrm_bwd: upstream and mlp_grad must be 16-byte aligned");
-    const dim3  grid((batch + SAMPLES_PER_WG - 1) / SAMPLES_PER_WG), block(THREADS);
+    bool           small = m <= 28;
+    const uint32_t pack  = samplesPerBlock(m, k, small);
+    const dim3     grid((batch + SAMPLES_PER_WG * pack - 1) / (SAMPLES_PER_WG * pack)), block(THREADS);
     hipStream_t s  = static_cast<hipStream_t>(stream);
     auto*       pi = static_cast<const uint16_t*>(in);
     auto*       pu = static_cast<const uint16_t*>(upstream);
@@ -988,10 +1040,10 @@ extern "C" int r355_dlrm_bwd(int32_t dtype, const void* in, const void* upstream
 #define R355_BWD(BF, KK)                                                                                          \
     do                                                                                                            \
     {                                                                                                             \
-        if(m <= 28)                                                                                               \
-            hipLaunchKernelGGL((dlrmBwdKernel<BF, KK, 28>), grid, block, 0, s, pi, pu, pm, pg, m, batch);          \
+        if(small)                                                                                                 \
+            hipLaunchKernelGGL((dlrmBwdKernel<BF, KK, 28>), grid, block, 0, s, pi, pu, pm, pg, m, batch, pack);    \
         else                                                                                                      \
-            hipLaunchKernelGGL((dlrmBwdKernel<BF, KK, 32>), grid, block, 0, s, pi, pu, pm, pg, m, batch);          \
+            hipLaunchKernelGGL((dlrmBwdKernel<BF, KK, 32>), grid, block, 0, s, pi, pu, pm, pg, m, batch, pack);    \
     } while(0)
 #define R355_BWD_K(BF)   \
     switch(k)            \

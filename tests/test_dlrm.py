@@ -290,6 +290,48 @@ def test_bwd_shapes_vs_oracle(dtype, m, k, batch):
     assert ok, mx
 
 
+# Up to 16 features the 16-bit kernels take several consecutive samples as one block of rows (the products across samples
+# are computed and dropped): every number of samples per block the launcher's rule yields (2 ... 16, both LDS-image
+# instances), batches that end inside a block and inside a workgroup's 8 blocks, single samples
+FEW_FEATURE_SHAPES = [(8, 128, 1), (8, 128, 2), (8, 128, 3), (8, 128, 25), (8, 128, 193), (16, 128, 9), (16, 32, 33), (15, 64, 17),
+                      (5, 64, 77), (2, 256, 100), (2, 32, 131), (3, 32, 1000), (4, 64, 65), (9, 128, 50), (10, 128, 37), (12, 256, 19),
+                      (14, 128, 15), (7, 32, 57), (6, 64, 200)]
+
+
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16])
+@pytest.mark.parametrize("m,k,batch", FEW_FEATURE_SHAPES)
+def test_few_features_share_a_block_fwd_and_bwd(dtype, m, k, batch):
+    stride = k + m * (m - 1) // 2
+    rt = R.F16 if dtype == O.F16 else R.BF16
+    for exact in (False, True):
+        if exact:  # small integers: every product and partial sum is exact, so any summation order gives the oracle's bits
+            x = O.f32_to_storage(np.round(O.uniform_pm1(17, batch * m * k) * 2.0), dtype)
+            up = O.f32_to_storage(np.round(O.uniform_pm1(18, batch * stride) * 2.0), dtype)
+        else:
+            x = O.f32_to_storage(O.normal(15, batch * m * k) * 0.5, dtype)
+            up = O.f32_to_storage(O.normal(16, batch * stride) * 0.5, dtype)
+        dx, dup = to_device(x), to_device(up)
+        dout = device_filled(batch * stride + 8, np.uint16, 0xEE)
+        R.dlrm_fwd(rt, dx, dout, m, k, batch)
+        out = to_host(dout, np.uint16)
+        assert np.all(out[batch * stride:] == 0xEEEE)
+        want = O.dlrm_fwd(dtype, x, m, k, batch).ravel()
+        dmlp, dgrad = device_filled(batch * k + 8, np.uint16, 0xEE), device_filled(batch * m * k + 8, np.uint16, 0xEE)
+        R.dlrm_bwd(rt, dx, dup, dmlp, dgrad, m, k, batch)
+        mlp, grad = to_host(dmlp, np.uint16), to_host(dgrad, np.uint16)
+        assert np.all(mlp[batch * k:] == 0xEEEE) and np.all(grad[batch * m * k:] == 0xEEEE)
+        want_mlp, want_grad = O.dlrm_bwd(dtype, x, up, m, k, batch)
+        assert np.array_equal(mlp[:batch * k], want_mlp.ravel())
+        if exact:
+            assert np.array_equal(out[:batch * stride], want)
+            assert np.array_equal(grad[:batch * m * k], want_grad.ravel())
+        else:
+            ok, mx = O.compare(dtype, out[:batch * stride], want, 10.0)
+            assert ok, mx
+            ok, mx = O.compare(dtype, grad[:batch * m * k], want_grad.ravel(), 10.0)
+            assert ok, mx
+
+
 def test_bwd_integer_inputs_exact():
     """Small integers: every product and partial sum is exact, so any summation order gives the oracle's bits."""
     m, k, batch = 27, 128, 24
