@@ -708,11 +708,15 @@ namespace
     // different banks), the upstream row to a second image from which each lane gathers its 16 values
     // of S; the gradient is written over X and leaves with 128-bit nontemporal stores; the first k
     // upstream values are the bottom-MLP gradient (test/reference_impl.hpp:121-179).
-    template <uint32_t K>
+    template <uint32_t K, bool PACK>
     __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2))) dlrmBwdF32Kernel(const float* __restrict__ in, const float* __restrict__ upstream,
                                                                float* __restrict__ mlpGrad, float* __restrict__ inGrad,
-                                                               uint32_t m, uint32_t batch)
+                                                               uint32_t m, uint32_t batch, uint32_t packArg)
     {
+        // (PACK: `pack` consecutive samples of few features as one block of rows, as in the 16-bit kernels: S of the block
+        // is block-diagonal, X, the upstream rows and the gradient are the samples' one after the other.  An instance of its
+        // own: the index arithmetic of the block-diagonal S would cost the one-sample kernel registers it does not have.)
+        const uint32_t pack = PACK ? packArg : 1u;
         constexpr uint32_t ROW_CHUNKS = K / 4; // 16-byte chunks per row
         constexpr uint32_t ROWB       = K * 4;
         constexpr uint32_t MAX_UP     = K + MAX_M * (MAX_M - 1) / 2;
@@ -727,8 +731,11 @@ namespace
 
         const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const uint32_t upStride = K + m * (m - 1) / 2;
-        const uint32_t inBytes  = m * ROWB;
-        // a wave walks the samples first, first + stride, ...
+        const uint32_t inBytes  = m * ROWB; // of a sample
+        const uint32_t rows     = m * pack; // of a block
+        const uint32_t rcpM     = (65536u + m - 1u) / m; // i / m == (i * rcpM) >> 16 for i < 32
+        const uint32_t blocks   = (batch + pack - 1u) / pack;
+        // a wave walks the blocks first, first + stride, ...
         const uint32_t first = blockIdx.x * WAVES + wave, stride = gridDim.x * WAVES;
         char*          xw       = xLds[wave];
         float*         uw       = upLds[wave];
@@ -741,8 +748,17 @@ namespace
         // row behind the first k values; the diagonal is zero (recomputed per sample: registers are
         // scarcer than integer instructions here)
         auto sAt = [&](uint32_t i, uint32_t j) -> float {
-            const uint32_t hi = i > j ? i : j, lo = i > j ? j : i;
-            return (i != j && hi < m) ? uw[K + hi * (hi - 1u) / 2u + lo] : 0.0f;
+            if constexpr(PACK)
+            {
+                const uint32_t si = (i * rcpM) >> 16, sj = (j * rcpM) >> 16, li = i - si * m, lj = j - sj * m;
+                const uint32_t hi = li > lj ? li : lj, lo = li > lj ? lj : li;
+                return (si == sj && li != lj && si < pack) ? uw[si * upStride + K + hi * (hi - 1u) / 2u + lo] : 0.0f;
+            }
+            else
+            {
+                const uint32_t hi = i > j ? i : j, lo = i > j ? j : i;
+                return (i != j && hi < m) ? uw[K + hi * (hi - 1u) / 2u + lo] : 0.0f;
+            }
         };
 
         // one register stash: a sample's loads are requested while the previous sample is computed and
@@ -752,10 +768,12 @@ namespace
         // product needs there.
         f32x4 xs[X_CHUNKS];
         float us[UP_WORDS];
-        auto  request = [&](uint64_t b) {
-            const bool valid = b < batch;
-            const auto src   = runBuffer(in, (uint64_t)(valid ? b : 0u) * inBytes, valid ? inBytes : 0u);
-            const auto up    = runBuffer(upstream, (uint64_t)(valid ? b : 0u) * upStride * 4u, valid ? upStride * 4u : 0u);
+        // (block index -> its first sample and how many of its samples exist)
+        auto  request = [&](uint64_t blk) {
+            const uint64_t b   = blk * pack;
+            const uint32_t has = blk < blocks ? (batch - b < pack ? (uint32_t)(batch - b) : pack) : 0u;
+            const auto     src = runBuffer(in, (has ? b : 0u) * inBytes, has * inBytes);
+            const auto     up  = runBuffer(upstream, (has ? b : 0u) * upStride * 4u, has * upStride * 4u);
 #pragma unroll
             for(uint32_t j = 0; j < X_CHUNKS; ++j)
                 xs[j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (j * 64u + lane) * 16u, 0, LOAD_POLICY));
@@ -764,7 +782,9 @@ namespace
                 us[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(up, (j * 64u + lane) * 4u, 0, LOAD_POLICY));
         };
 
-        auto process = [&](uint64_t b) {
+        auto process = [&](uint64_t blk) {
+            const uint64_t b   = blk * pack;
+            const uint32_t has = batch - b < pack ? (uint32_t)(batch - b) : pack;
 #pragma unroll
             for(uint32_t j = 0; j < X_CHUNKS; ++j)
             {
@@ -776,13 +796,16 @@ namespace
                 uw[j * 64u + lane] = us[j];
             __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_wave_barrier();
-            request(b + stride);
+            request(blk + stride);
 
-            // bottom-MLP gradient: the first k upstream values
-            const auto mg = runBuffer(mlpGrad, (uint64_t)b * K * 4u, K * 4u);
+            // bottom-MLP gradient: the first k upstream values of every sample of the block
+            const auto mg = runBuffer(mlpGrad, b * K * 4u, has * K * 4u);
+            for(uint32_t s = 0; s < has; ++s)
 #pragma unroll
-            for(uint32_t e = 0; e < (K + 63u) / 64u; ++e)
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, uw[e * 64u + lane]), mg, (e * 64u + lane) * 4u, 0, STORE_POLICY);
+                for(uint32_t e = 0; e < (K + 63u) / 64u; ++e)
+                    if(K >= 64u || lane < K)
+                        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, uw[s * upStride + e * 64u + lane]), mg,
+                                                              (s * K + e * 64u + lane) * 4u, 0, STORE_POLICY);
 
             float sv[2][8];
 #pragma unroll
@@ -822,12 +845,12 @@ namespace
                     for(uint32_t e = 0; e < 4; ++e)
                     {
                         const uint32_t row = 16u * ib + 4u * q4 + e;
-                        if(row < m)
+                        if(row < rows)
                             *reinterpret_cast<float*>(xw + row * ROWB + ((cb ^ (row & SWZ)) << 6) + r16 * 4u) = acc[ib][cb][e];
                     }
             __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_wave_barrier();
-            const auto dst = runBuffer(inGrad, (uint64_t)b * inBytes, inBytes);
+            const auto dst = runBuffer(inGrad, b * inBytes, has * inBytes);
 #pragma unroll
             for(uint32_t j = 0; j < X_CHUNKS; ++j)
             {
@@ -842,13 +865,13 @@ namespace
 
         // The first sample stands outside the loop so that the loop is entered with the same operations in flight as
         // its own trips leave behind: the waits inside are then exact on both paths.
-        if(first >= batch)
+        if(first >= blocks)
             return;
         request(first);
         process(first);
 #pragma unroll 1
-        for(uint64_t b = (uint64_t)first + stride; b < batch; b += stride)
-            process(b);
+        for(uint64_t blk = (uint64_t)first + stride; blk < blocks; blk += stride)
+            process(blk);
     }
 
     int checkArgs(const char* what, int32_t dtype, const void* in, const void* out, uint32_t m, uint32_t k, uint32_t batch,
@@ -1012,19 +1035,39 @@ extern "C" int r355_dlrm_bwd(int32_t dtype, const void* in, const void* upstream
     {
         if(!r355::aligned(upstream, 4) || !r355::aligned(mlp_grad, 4))
             return r355::fail(R355_ERR_MISALIGNED, "dlrm_bwd: upstream and mlp_grad must be 4-byte aligned");
-        const uint32_t steps = (batch + WAVES - 1) / WAVES; // of one sample per wave
+        // up to 16 features several samples share a block of rows, as many as fit the 32 rows of the image and, with
+        // their upstream rows, the space of one 32-feature sample's
+        uint32_t pack = 1;
+#ifndef R355_DLRM_NO_PACK
+        if(m <= 16)
+        {
+            const uint32_t byRows = 32u / m, byRow = (k + 32u * 31u / 2u) / (k + m * (m - 1u) / 2u);
+            pack = byRows < byRow ? byRows : byRow;
+        }
+#endif
+        const uint32_t blocks = (batch + pack - 1) / pack;
+        const uint32_t steps  = (blocks + WAVES - 1) / WAVES; // of one block per wave
         const dim3     grid32((steps + F32_STEPS - 1) / F32_STEPS), block32(THREADS);
         hipStream_t    s32 = static_cast<hipStream_t>(stream);
         auto*          fi  = static_cast<const float*>(in);
         auto*          fu  = static_cast<const float*>(upstream);
         auto*          fm  = static_cast<float*>(mlp_grad);
         auto*          fg  = static_cast<float*>(in_grad);
+#define R355_BWD32(KK)                                                                                                   \
+    do                                                                                                                   \
+    {                                                                                                                    \
+        if(pack > 1)                                                                                                     \
+            hipLaunchKernelGGL((dlrmBwdF32Kernel<KK, true>), grid32, block32, 0, s32, fi, fu, fm, fg, m, batch, pack);   \
+        else                                                                                                             \
+            hipLaunchKernelGGL((dlrmBwdF32Kernel<KK, false>), grid32, block32, 0, s32, fi, fu, fm, fg, m, batch, pack);  \
+    } while(0)
         switch(k)
         {
-        case 32: hipLaunchKernelGGL(dlrmBwdF32Kernel<32>, grid32, block32, 0, s32, fi, fu, fm, fg, m, batch); break;
-        case 64: hipLaunchKernelGGL(dlrmBwdF32Kernel<64>, grid32, block32, 0, s32, fi, fu, fm, fg, m, batch); break;
-        default: hipLaunchKernelGGL(dlrmBwdF32Kernel<128>, grid32, block32, 0, s32, fi, fu, fm, fg, m, batch); break;
+        case 32: R355_BWD32(32); break;
+        case 64: R355_BWD32(64); break;
+        default: R355_BWD32(128); break;
         }
+#undef R355_BWD32
         return r355::checkLaunch("dlrm_bwd");
     }
     if(!r355::aligned(upstream, 16) || !r355::aligned(mlp_grad, 16))

@@ -298,37 +298,41 @@ FEW_FEATURE_SHAPES = [(8, 128, 1), (8, 128, 2), (8, 128, 3), (8, 128, 25), (8, 1
                       (14, 128, 15), (7, 32, 57), (6, 64, 200)]
 
 
-@pytest.mark.parametrize("dtype", [O.F16, O.BF16])
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16, O.F32])
 @pytest.mark.parametrize("m,k,batch", FEW_FEATURE_SHAPES)
 def test_few_features_share_a_block_fwd_and_bwd(dtype, m, k, batch):
+    """(f32: the backward kernel shares blocks the same way; the forward kernel for these shapes is the one fed from the loads.)"""
+    if dtype == O.F32 and k == 256:
+        pytest.skip("k = 256 in f32 goes to the general kernels")
     stride = k + m * (m - 1) // 2
-    rt = R.F16 if dtype == O.F16 else R.BF16
+    store = O.NP_STORAGE[dtype]
+    rt = {O.F16: R.F16, O.BF16: R.BF16, O.F32: R.F32}[dtype]
+    tol = F32_NORMAL_TOL_EPS if dtype == O.F32 else 10.0
+    pack = (lambda v: v.astype(np.float32)) if dtype == O.F32 else (lambda v: O.f32_to_storage(v.astype(np.float32), dtype))
     for exact in (False, True):
         if exact:  # small integers: every product and partial sum is exact, so any summation order gives the oracle's bits
-            x = O.f32_to_storage(np.round(O.uniform_pm1(17, batch * m * k) * 2.0), dtype)
-            up = O.f32_to_storage(np.round(O.uniform_pm1(18, batch * stride) * 2.0), dtype)
+            x, up = pack(np.round(O.uniform_pm1(17, batch * m * k) * 2.0)), pack(np.round(O.uniform_pm1(18, batch * stride) * 2.0))
         else:
-            x = O.f32_to_storage(O.normal(15, batch * m * k) * 0.5, dtype)
-            up = O.f32_to_storage(O.normal(16, batch * stride) * 0.5, dtype)
+            x, up = pack(O.normal(15, batch * m * k) * 0.5), pack(O.normal(16, batch * stride) * 0.5)
         dx, dup = to_device(x), to_device(up)
-        dout = device_filled(batch * stride + 8, np.uint16, 0xEE)
+        dout = device_filled(batch * stride + 8, store, 0xEE)
         R.dlrm_fwd(rt, dx, dout, m, k, batch)
-        out = to_host(dout, np.uint16)
-        assert np.all(out[batch * stride:] == 0xEEEE)
+        out = to_host(dout, store)
+        assert np.all(out[batch * stride:].view(np.uint8) == 0xEE)
         want = O.dlrm_fwd(dtype, x, m, k, batch).ravel()
-        dmlp, dgrad = device_filled(batch * k + 8, np.uint16, 0xEE), device_filled(batch * m * k + 8, np.uint16, 0xEE)
+        dmlp, dgrad = device_filled(batch * k + 8, store, 0xEE), device_filled(batch * m * k + 8, store, 0xEE)
         R.dlrm_bwd(rt, dx, dup, dmlp, dgrad, m, k, batch)
-        mlp, grad = to_host(dmlp, np.uint16), to_host(dgrad, np.uint16)
-        assert np.all(mlp[batch * k:] == 0xEEEE) and np.all(grad[batch * m * k:] == 0xEEEE)
+        mlp, grad = to_host(dmlp, store), to_host(dgrad, store)
+        assert np.all(mlp[batch * k:].view(np.uint8) == 0xEE) and np.all(grad[batch * m * k:].view(np.uint8) == 0xEE)
         want_mlp, want_grad = O.dlrm_bwd(dtype, x, up, m, k, batch)
-        assert np.array_equal(mlp[:batch * k], want_mlp.ravel())
+        assert np.array_equal(mlp[:batch * k].view(np.uint8), want_mlp.ravel().view(np.uint8))
         if exact:
-            assert np.array_equal(out[:batch * stride], want)
-            assert np.array_equal(grad[:batch * m * k], want_grad.ravel())
+            assert np.array_equal(out[:batch * stride].view(np.uint8), want.view(np.uint8))
+            assert np.array_equal(grad[:batch * m * k].view(np.uint8), want_grad.ravel().view(np.uint8))
         else:
-            ok, mx = O.compare(dtype, out[:batch * stride], want, 10.0)
+            ok, mx = O.compare(dtype, out[:batch * stride], want, tol)
             assert ok, mx
-            ok, mx = O.compare(dtype, grad[:batch * m * k], want_grad.ravel(), 10.0)
+            ok, mx = O.compare(dtype, grad[:batch * m * k], want_grad.ravel(), tol)
             assert ok, mx
 
 
