@@ -529,6 +529,22 @@ def run_extras(R, O, np, torch, args, counters, clocks, cus):
     hbm_case("dlrm_bwd_f32_b65536_f27_d128", ms, (2 * bsz * mm * kk + bsz * (kk + mm * (mm - 1) // 2) + bsz * kk) * 4,
              bool(torch.isfinite(gin32).all() and torch.isfinite(gmlp32).all()) and dlrm_ok(x32, None, up32, gmlp32, gin32, bsz, mm, kk, 1e-5))
     del x32, o32, up32, gmlp32, gin32
+    # few features (8 x 64, f16): the kernels take four consecutive samples as one block of rows
+    fm, fk = 8, 64
+    fstride = fk + fm * (fm - 1) // 2
+    x8 = torch.randn(bsz * fm * fk, device="cuda").to(torch.float16)
+    o8 = torch.empty(bsz * fstride, dtype=torch.float16, device="cuda")
+    up8 = torch.randn(bsz * fstride, device="cuda").to(torch.float16)
+    gmlp8 = torch.empty(bsz * fk, dtype=torch.float16, device="cuda")
+    gin8 = torch.empty(bsz * fm * fk, dtype=torch.float16, device="cuda")
+    ms = event_ms(lambda: R.dlrm_fwd(R.F16, x8, o8, fm, fk, bsz))
+    hbm_case("dlrm_fwd_b65536_f8_d64", ms, bsz * (fm * fk + fstride) * 2,
+             bool(torch.isfinite(o8.float()).all()) and dlrm_ok(x8, o8, None, None, None, bsz, fm, fk, 2e-3))
+    ms = event_ms(lambda: R.dlrm_bwd(R.F16, x8, up8, gmlp8, gin8, fm, fk, bsz))
+    hbm_case("dlrm_bwd_b65536_f8_d64", ms, (2 * bsz * fm * fk + bsz * fstride + bsz * fk) * 2,
+             bool(torch.isfinite(gin8.float()).all() and torch.isfinite(gmlp8.float()).all())
+             and dlrm_ok(x8, None, up8, gmlp8, gin8, bsz, fm, fk, 4e-3))
+    del x8, o8, up8, gmlp8, gin8
     # GEMV y = A x (the reference's simple_sgemv / simple_dgemv samples), A read once: bytes of A, x and y over the HBM peak;
     # checked against a float64 product on sampled rows
     # The HBM fraction of GEMV is the one of the 16384^2 cases (1 GiB of A, four times the 256 MiB memory-side cache, read with
