@@ -220,26 +220,29 @@ namespace
         }
     }
 
-    // Backward from 64 features on, or 64 embedding columns: a wave owns NBI x NBK blocks of the gradient - row blocks
-    // ti0 .. ti0 + NBI - 1, column blocks kc0 .. kc0 + NBK - 1 - so that every block of S it forms in LDS (256 gathers from
-    // the packed triangle with their index arithmetic) feeds NBK matrix instructions per K step instead of one, and every
-    // fragment of X NBI of them.
+    // Backward for large launches: a wave owns NBI x NBK blocks of the gradient - row blocks ti0 .. ti0 + NBI - 1, column
+    // blocks kc0 .. kc0 + NBK - 1 - and the four waves of a workgroup share ti0: the NBI blocks of S that a step needs
+    // (gathers from the packed triangle with their index arithmetic, the expensive part) are formed once per workgroup,
+    // one element per thread and block, in an LDS image that every wave reads, and each feeds NBK matrix instructions per
+    // wave and K step.  The image has two buffers, so a step costs one barrier; the gathers and the fragments of X for
+    // step tj + 1 are in flight while the matrix instructions of step tj run.  Below the diagonal a block's rows are
+    // contiguous in the triangle, above it its columns are, and the threads are laid along whichever it is.
     template <typename T, uint32_t NBI, uint32_t NBK>
     __global__ void __launch_bounds__(THREADS) dlrmBwdGeneralBlocked(const T* __restrict__ in, const T* __restrict__ upstream,
                                                                     T* __restrict__ mlpGrad, T* __restrict__ inGrad, uint32_t m, uint32_t k)
     {
-        constexpr uint32_t BK = blockK<T>();
+        constexpr uint32_t BK = blockK<T>(), KSTEPS = BLK / BK;
+        static_assert(THREADS == BLK * BLK, "one thread per element of a block of S");
         using FragA   = fragment<matrix_a, BLK, BLK, BK, T, row_major>;
         using FragB   = fragment<matrix_b, BLK, BLK, BK, T, row_major>;
         using FragAcc = fragment<accumulator, BLK, BLK, BK, float32_t>;
-        __shared__ T     sBlock[WAVES][NBI][BLK * BLK];
+        __shared__ T     sBlock[2][NBI][BLK * BLK];
         __shared__ float block[WAVES][BLK * BLK];
 
-        const uint32_t lane = threadIdx.x & 63u, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+        const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const uint32_t kc0  = (blockIdx.x * WAVES + wave) * NBK, ti0 = blockIdx.y * NBI;
         const uint32_t tilesK = k / BLK, tilesM = m / BLK;
-        if(kc0 >= tilesK)
-            return;
+        const bool     active = kc0 < tilesK; // (a wave without column blocks still gathers its share of S)
         const uint64_t stride = (uint64_t)k + (uint64_t)m * (m - 1u) / 2u;
         const T*       x      = in + (uint64_t)blockIdx.z * m * k;
         const T*       up     = upstream + (uint64_t)blockIdx.z * stride;
@@ -258,75 +261,71 @@ namespace
             for(uint32_t c = 0; c < NBK; ++c)
                 fill_fragment(acc[i][c], 0.0f);
 
-        // The step for column block tj of S works on values fetched one step before: the gathers from the packed triangle and
-        // the fragments of X for step tj + 1 are in flight while the matrix instructions of step tj run.  A lane gathers four
-        // elements of each block of S; below the diagonal a block's rows are contiguous in the triangle, above it its columns
-        // are, and the lanes are laid along whichever it is.
-        constexpr uint32_t PER_LANE = BLK * BLK / 64u, KSTEPS = BLK / BK;
-        T     sNext[NBI][PER_LANE];
+        T     sNext[NBI];
         FragB bNext[KSTEPS][NBK];
-        auto  place = [&](uint32_t i, uint32_t tj, uint32_t q, uint32_t& r, uint32_t& c) {
-            const uint32_t e = q * 64u + lane;
+        auto  place = [&](uint32_t i, uint32_t tj, uint32_t& r, uint32_t& c) {
             const bool upper = tj > ti0 + i;
-            r = upper ? e % BLK : e / BLK;
-            c = upper ? e / BLK : e % BLK;
+            r = upper ? tid % BLK : tid / BLK;
+            c = upper ? tid / BLK : tid % BLK;
         };
         auto fetch = [&](uint32_t tj) {
 #pragma unroll
             for(uint32_t i = 0; i < NBI; ++i)
+            {
+                uint32_t r, c;
+                place(i, tj, r, c);
+                const uint64_t gi = (uint64_t)(ti0 + i < tilesM ? ti0 + i : ti0) * BLK + r, gj = (uint64_t)tj * BLK + c;
+                const uint64_t hi = gi > gj ? gi : gj, lo = gi > gj ? gj : gi;
+                sNext[i] = gi == gj ? static_cast<T>(0.0f) : tril[hi * (hi - 1u) / 2u + lo];
+            }
+            if(active)
 #pragma unroll
-                for(uint32_t q = 0; q < PER_LANE; ++q)
-                {
-                    uint32_t r, c;
-                    place(i, tj, q, r, c);
-                    const uint64_t gi = (uint64_t)(ti0 + i < tilesM ? ti0 + i : ti0) * BLK + r, gj = (uint64_t)tj * BLK + c;
-                    const uint64_t hi = gi > gj ? gi : gj, lo = gi > gj ? gj : gi;
-                    sNext[i][q] = gi == gj ? static_cast<T>(0.0f) : tril[hi * (hi - 1u) / 2u + lo];
-                }
+                for(uint32_t ks = 0; ks < KSTEPS; ++ks)
 #pragma unroll
-            for(uint32_t ks = 0; ks < KSTEPS; ++ks)
-#pragma unroll
-                for(uint32_t c = 0; c < NBK; ++c) // (a column block past the end reads the last one again: its products are not used)
-                    load_matrix_sync(bNext[ks][c],
-                                     x + (uint64_t)tj * BLK * k + (uint64_t)(kc0 + c < tilesK ? kc0 + c : tilesK - 1u) * BLK + (uint64_t)ks * BK * k, k);
+                    for(uint32_t c = 0; c < NBK; ++c) // (a column block past the end reads the last one again: its products are not used)
+                        load_matrix_sync(bNext[ks][c],
+                                         x + (uint64_t)tj * BLK * k + (uint64_t)(kc0 + c < tilesK ? kc0 + c : tilesK - 1u) * BLK + (uint64_t)ks * BK * k, k);
         };
         fetch(0u);
         for(uint32_t tj = 0; tj < tilesM; ++tj)
         {
             FragB b[KSTEPS][NBK];
+            T(*s)[BLK * BLK] = sBlock[tj & 1u];
 #pragma unroll
             for(uint32_t i = 0; i < NBI; ++i)
-#pragma unroll
-                for(uint32_t q = 0; q < PER_LANE; ++q)
-                {
-                    uint32_t r, c;
-                    place(i, tj, q, r, c);
-                    sBlock[wave][i][r * BLK + c] = sNext[i][q];
-                }
+            {
+                uint32_t r, c;
+                place(i, tj, r, c);
+                s[i][r * BLK + c] = sNext[i];
+            }
 #pragma unroll
             for(uint32_t ks = 0; ks < KSTEPS; ++ks)
 #pragma unroll
                 for(uint32_t c = 0; c < NBK; ++c)
                     b[ks][c] = bNext[ks][c];
-            __builtin_amdgcn_wave_barrier();
+            // the one barrier of the step: this buffer is complete; the other one, which the next step writes, was last read
+            // in the step before this one, and every wave has finished that step to get here
+            __syncthreads();
             if(tj + 1u < tilesM)
                 fetch(tj + 1u);
+            if(active)
 #pragma unroll
-            for(uint32_t ks = 0; ks < KSTEPS; ++ks)
-            {
-                FragA a[NBI];
+                for(uint32_t ks = 0; ks < KSTEPS; ++ks)
+                {
+                    FragA a[NBI];
 #pragma unroll
-                for(uint32_t i = 0; i < NBI; ++i)
-                    load_matrix_sync(a[i], sBlock[wave][i] + ks * BK, BLK);
+                    for(uint32_t i = 0; i < NBI; ++i)
+                        load_matrix_sync(a[i], s[i] + ks * BK, BLK);
 #pragma unroll
-                for(uint32_t i = 0; i < NBI; ++i)
+                    for(uint32_t i = 0; i < NBI; ++i)
 #pragma unroll
-                    for(uint32_t c = 0; c < NBK; ++c)
-                        if(ti0 + i < tilesM && kc0 + c < tilesK)
-                            mma_sync(acc[i][c], a[i], b[ks][c], acc[i][c]);
-            }
-            __builtin_amdgcn_wave_barrier(); // the blocks of S are rewritten in the next trip
+                        for(uint32_t c = 0; c < NBK; ++c)
+                            if(ti0 + i < tilesM && kc0 + c < tilesK)
+                                mma_sync(acc[i][c], a[i], b[ks][c], acc[i][c]);
+                }
         }
+        if(!active)
+            return;
         float* mine = block[wave];
 #pragma unroll
         for(uint32_t i = 0; i < NBI; ++i)
