@@ -14,7 +14,12 @@
 //     matrix instructions, one 128-bit LDS read each; lanes of rows >= m feed zeros, which is
 //     the 27 -> 32 padding;
 //   * the strict lower triangle and the copied first row are assembled in an LDS image of
-//     the output and leave with coalesced 128-bit stores.  No global scratch.
+//     the output and leave with coalesced 128-bit stores.  No global scratch;
+//   * up to 16 features, "one sample" above is a block of several consecutive samples, whose
+//     rows are contiguous in memory: the products across samples are computed and dropped.
+//
+// f32 has kernels of its own on v_mfma_f32_16x16x4_f32 (an LDS image of X, or the matrix
+// instructions fed straight from the global loads: see dlrmFwdF32Kernel, dlrmFwdF32Direct).
 //
 // Backward takes the place of test/dlrm/device/dlrm_dot_bwd.hpp:35-176: the symmetric matrix
 // of the upstream triangle (trilReconstruct) is formed directly as a matrix-instruction operand
@@ -889,8 +894,6 @@ namespace
             return r355::fail(R355_ERR_MISALIGNED, "%s: in / out must be 16-byte aligned", what);
         return R355_OK;
     }
-    // the kernels of this file: up to 32 features and an embedding width they are instantiated for; everything else goes
-    // to the block-per-wave kernels of dlrm_general.hip
     // 16-bit kernels, up to 16 features: the samples that share a block of rows - as many as fit the rows of the LDS image
     // (28 or 32: `small` says which instance) and, with their output / upstream rows, the space of that image's one
     // full-size sample's row.  The 32-row instance where it takes more samples per block - except at k = 128, where the
@@ -917,6 +920,8 @@ namespace
 #endif
         return small ? p28 : p32;
     }
+    // the kernels of this file: up to 32 features and an embedding width they are instantiated for; everything else goes
+    // to the kernels of dlrm_general.hip
     bool specialised(int32_t dtype, uint32_t m, uint32_t k)
     {
         return m <= MAX_M && (k == 32 || k == 64 || k == 128 || (k == 256 && dtype != R355_F32));

@@ -224,9 +224,12 @@ namespace
     // blocks kc0 .. kc0 + NBK - 1 - and the four waves of a workgroup share ti0: the NBI blocks of S that a step needs
     // (gathers from the packed triangle with their index arithmetic, the expensive part) are formed once per workgroup,
     // one element per thread and block, in an LDS image that every wave reads, and each feeds NBK matrix instructions per
-    // wave and K step.  The image has two buffers, so a step costs one barrier; the gathers and the fragments of X for
-    // step tj + 1 are in flight while the matrix instructions of step tj run.  Below the diagonal a block's rows are
-    // contiguous in the triangle, above it its columns are, and the threads are laid along whichever it is.
+    // wave and K step.  The 16 rows of X that a step multiplies them with go the same way: the workgroup's 256 columns of
+    // them are fetched with 128-bit loads into an LDS image, from which every wave takes its matrix_b fragments (16-bit
+    // types: transposing reads) - a row-major matrix_b fragment straight from global memory is four 2-byte loads per lane.
+    // Both images have two buffers, so a step costs one barrier; the gathers and the rows of X for step tj + 1 are in
+    // flight while the matrix instructions of step tj run.  Below the diagonal a block's rows are contiguous in the
+    // triangle, above it its columns are, and the threads are laid along whichever it is.
     template <typename T, uint32_t NBI, uint32_t NBK>
     __global__ void __launch_bounds__(THREADS) dlrmBwdGeneralBlocked(const T* __restrict__ in, const T* __restrict__ upstream,
                                                                     T* __restrict__ mlpGrad, T* __restrict__ inGrad, uint32_t m, uint32_t k)
@@ -236,10 +239,19 @@ namespace
         using FragA   = fragment<matrix_a, BLK, BLK, BK, T, row_major>;
         using FragB   = fragment<matrix_b, BLK, BLK, BK, T, row_major>;
         using FragAcc = fragment<accumulator, BLK, BLK, BK, float32_t>;
+        // (16-bit types.  f32 fragments are four 4-byte loads per lane either way, and the image - 33 KiB - costs more in
+        // resident workgroups than it saves: 512 x 128 x 256 0.28 -> 0.32 ms with it; f32 takes its fragments from global memory)
+        constexpr bool     STAGE_X = sizeof(T) == 2;
+        constexpr uint32_t COLS = WAVES * NBK * BLK; // columns of X (and of the gradient) per workgroup
+        constexpr uint32_t XLD  = COLS + 16u / sizeof(T); // row pitch of the image of X: 16 bytes of padding
+        constexpr uint32_t CH   = 16u / sizeof(T), XLOADS = BLK * COLS / CH / THREADS; // elements per 128-bit load, loads per thread
+        using i32x4             = int __attribute__((ext_vector_type(4)));
         __shared__ T     sBlock[2][NBI][BLK * BLK];
+        __shared__ __attribute__((aligned(16))) T xBlock[STAGE_X ? 2 : 1][STAGE_X ? BLK * XLD : CH];
         __shared__ float block[WAVES][BLK * BLK];
 
         const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const uint32_t col0 = blockIdx.x * COLS; // first column of the workgroup
         const uint32_t kc0  = (blockIdx.x * WAVES + wave) * NBK, ti0 = blockIdx.y * NBI;
         const uint32_t tilesK = k / BLK, tilesM = m / BLK;
         const bool     active = kc0 < tilesK; // (a wave without column blocks still gathers its share of S)
@@ -262,7 +274,8 @@ namespace
                 fill_fragment(acc[i][c], 0.0f);
 
         T     sNext[NBI];
-        FragB bNext[KSTEPS][NBK];
+        i32x4 xNext[STAGE_X ? XLOADS : 1u];
+        FragB bNext[STAGE_X ? 1u : KSTEPS][NBK];
         auto  place = [&](uint32_t i, uint32_t tj, uint32_t& r, uint32_t& c) {
             const bool upper = tj > ti0 + i;
             r = upper ? tid % BLK : tid / BLK;
@@ -278,19 +291,32 @@ namespace
                 const uint64_t hi = gi > gj ? gi : gj, lo = gi > gj ? gj : gi;
                 sNext[i] = gi == gj ? static_cast<T>(0.0f) : tril[hi * (hi - 1u) / 2u + lo];
             }
-            if(active)
+            if constexpr(STAGE_X)
+            {
+#pragma unroll
+                for(uint32_t j = 0; j < XLOADS; ++j) // rows tj * 16 ... of X, the workgroup's columns (k is a multiple of 16: whole pieces)
+                {
+                    const uint32_t piece = j * THREADS + tid, r = piece / (COLS / CH), c = col0 + (piece % (COLS / CH)) * CH;
+                    if(c < k)
+                        xNext[j] = *reinterpret_cast<const i32x4*>(x + ((uint64_t)tj * BLK + r) * k + c);
+                }
+            }
+            else if(active)
+            {
 #pragma unroll
                 for(uint32_t ks = 0; ks < KSTEPS; ++ks)
 #pragma unroll
                     for(uint32_t c = 0; c < NBK; ++c) // (a column block past the end reads the last one again: its products are not used)
                         load_matrix_sync(bNext[ks][c],
                                          x + (uint64_t)tj * BLK * k + (uint64_t)(kc0 + c < tilesK ? kc0 + c : tilesK - 1u) * BLK + (uint64_t)ks * BK * k, k);
+            }
         };
         fetch(0u);
         for(uint32_t tj = 0; tj < tilesM; ++tj)
         {
-            FragB b[KSTEPS][NBK];
             T(*s)[BLK * BLK] = sBlock[tj & 1u];
+            T* xs            = xBlock[STAGE_X ? tj & 1u : 0u];
+            FragB bNow[STAGE_X ? 1u : KSTEPS][NBK];
 #pragma unroll
             for(uint32_t i = 0; i < NBI; ++i)
             {
@@ -298,12 +324,25 @@ namespace
                 place(i, tj, r, c);
                 s[i][r * BLK + c] = sNext[i];
             }
+            if constexpr(STAGE_X)
+            {
 #pragma unroll
-            for(uint32_t ks = 0; ks < KSTEPS; ++ks)
+                for(uint32_t j = 0; j < XLOADS; ++j)
+                {
+                    const uint32_t piece = j * THREADS + tid, r = piece / (COLS / CH), c = (piece % (COLS / CH)) * CH;
+                    if(col0 + c < k)
+                        *reinterpret_cast<i32x4*>(xs + r * XLD + c) = xNext[j];
+                }
+            }
+            else
+            {
 #pragma unroll
-                for(uint32_t c = 0; c < NBK; ++c)
-                    b[ks][c] = bNext[ks][c];
-            // the one barrier of the step: this buffer is complete; the other one, which the next step writes, was last read
+                for(uint32_t ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+                    for(uint32_t c = 0; c < NBK; ++c)
+                        bNow[ks][c] = bNext[ks][c];
+            }
+            // the one barrier of the step: these buffers are complete; the others, which the next step writes, were last read
             // in the step before this one, and every wave has finished that step to get here
             __syncthreads();
             if(tj + 1u < tilesM)
@@ -313,15 +352,22 @@ namespace
                 for(uint32_t ks = 0; ks < KSTEPS; ++ks)
                 {
                     FragA a[NBI];
+                    FragB b[NBK];
 #pragma unroll
                     for(uint32_t i = 0; i < NBI; ++i)
                         load_matrix_sync(a[i], s[i] + ks * BK, BLK);
+#pragma unroll
+                    for(uint32_t c = 0; c < NBK; ++c)
+                        if constexpr(STAGE_X)
+                            load_matrix_sync(b[c], xs + ks * BK * XLD + ((kc0 + c < tilesK ? kc0 + c : tilesK - 1u) * BLK - col0), XLD);
+                        else
+                            b[c] = bNow[ks][c];
 #pragma unroll
                     for(uint32_t i = 0; i < NBI; ++i)
 #pragma unroll
                         for(uint32_t c = 0; c < NBK; ++c)
                             if(ti0 + i < tilesM && kc0 + c < tilesK)
-                                mma_sync(acc[i][c], a[i], b[ks][c], acc[i][c]);
+                                mma_sync(acc[i][c], a[i], b[c], acc[i][c]);
                 }
         }
         if(!active)
