@@ -165,7 +165,8 @@ int r355_gemm_timed(const r355_gemm_args* args, void* stream, int warmup, int it
  * order, f32 accumulation, rounded to dtype (R355_F16, R355_BF16 or R355_F32).  Bandwidth-bound kernels for
  * 2 <= m <= 32 with k in {32, 64, 128, 256} (R355_F32: up to 128); any other m and k that are multiples of 16 - the
  * reference's own constraint, test/dlrm/dlrm_kernel_base_impl.hpp:146-151; its tests run m = 128, k = 128 and m = k = 1024 -
- * run block-per-wave kernels (batch <= 65535 there).  No scratch buffer either way (the reference's `acc` argument is gone).
+ * run kernels written on the fragment API (a 16 x 16 block per wave for small launches, several blocks per wave otherwise;
+ * any batch).  No scratch buffer either way (the reference's `acc` argument is gone).
  * Replaces: dlrmDotFwd launch, test/dlrm/dlrm_kernel_base_impl.hpp:78-96,
  * test/dlrm/device/dlrm_dot_fwd.hpp:35-138, samples/simple_dlrm.cpp:184-284.
  */
