@@ -154,6 +154,38 @@ def test_fwd_full_batch_65536_properties():
     assert np.max(np.abs(tri - ident)) < 0.5  # 351 f16 roundings of values up to ~40
 
 
+@pytest.mark.parametrize("dtype,m,k", [(O.F16, 8, 64), (O.BF16, 16, 128), (O.F32, 8, 128), (O.F16, 3, 32)])
+def test_few_features_full_batch(dtype, m, k):
+    """The benchmark's batch with few features (several samples per block of rows; f32 forward: the kernel fed from the loads),
+    ending inside a block: integer-valued inputs, samples from the first, a middle and the last blocks bit for bit against the oracle."""
+    batch = 65536 + 3
+    stride = k + m * (m - 1) // 2
+    store = O.NP_STORAGE[dtype]
+    rt = {O.F16: R.F16, O.BF16: R.BF16, O.F32: R.F32}[dtype]
+    pack = (lambda v: v.astype(np.float32)) if dtype == O.F32 else (lambda v: O.f32_to_storage(v.astype(np.float32), dtype))
+    x, up = pack(np.round(O.uniform_pm1(31, batch * m * k) * 2.0)), pack(np.round(O.uniform_pm1(32, batch * stride) * 2.0))
+    dx, dup = to_device(x), to_device(up)
+    dout = device_filled(batch * stride + 8, store, 0xEE)
+    dmlp, dgrad = device_filled(batch * k + 8, store, 0xEE), device_filled(batch * m * k + 8, store, 0xEE)
+    R.dlrm_fwd(rt, dx, dout, m, k, batch)
+    R.dlrm_bwd(rt, dx, dup, dmlp, dgrad, m, k, batch)
+    out, mlp, grad = to_host(dout, store), to_host(dmlp, store), to_host(dgrad, store)
+    assert np.all(out[batch * stride:].view(np.uint8) == 0xEE) and np.all(mlp[batch * k:].view(np.uint8) == 0xEE)
+    assert np.all(grad[batch * m * k:].view(np.uint8) == 0xEE)
+    sel = np.array(list(range(0, 40)) + list(range(32760, 32800)) + list(range(batch - 40, batch)))
+    xs, ups = x.reshape(batch, m * k)[sel].ravel(), up.reshape(batch, stride)[sel].ravel()
+    want = O.dlrm_fwd(dtype, xs, m, k, len(sel))
+    assert np.array_equal(out[:batch * stride].reshape(batch, stride)[sel].view(np.uint8), want.reshape(len(sel), stride).view(np.uint8))
+    wmlp, wgrad = O.dlrm_bwd(dtype, xs, ups, m, k, len(sel))
+    assert np.array_equal(mlp[:batch * k].reshape(batch, k)[sel].view(np.uint8), wmlp.reshape(len(sel), k).view(np.uint8))
+    g, w = grad[:batch * m * k].reshape(batch, m * k)[sel], wgrad.reshape(len(sel), m * k)
+    gf, wf = (g, w) if dtype == O.F32 else (O.storage_to_f32(g.ravel(), dtype), O.storage_to_f32(w.ravel(), dtype))
+    assert np.array_equal(gf, wf)  # (values: -0.0 and +0.0 are the same gradient)
+    # every sample's first output values are its first input row, and the bottom-MLP gradient the head of its upstream row
+    assert np.array_equal(out[:batch * stride].reshape(batch, stride)[:, :k].view(np.uint8), x.reshape(batch, m, k)[:, 0, :].view(np.uint8))
+    assert np.array_equal(mlp[:batch * k].reshape(batch, k).view(np.uint8), up.reshape(batch, stride)[:, :k].view(np.uint8))
+
+
 def test_fwd_and_bwd_batch_beyond_4_gib_of_input():
     # 700 000 samples of 27 x 128 f16 are 4.8 GB: byte offsets of samples from 621 379 on do not fit 32 bits.  Samples on
     # both sides of that boundary against the oracle (every sample is independent of the others).
