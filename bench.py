@@ -450,20 +450,25 @@ def run_extras(R, O, np, torch, args, counters, clocks, cus):
     sk = 8192
     for name, in_t, out_t, key, unit, sm in (("gemm_i8_sparse24_4096x4096x8192", R.I8, R.I32, "i8", "TOP/s (dense-equivalent)", 4096),
                                              ("gemm_e4m3_sparse24_4096x4096x8192", R.E4M3, R.F32, "e4m3", "TFLOP/s (dense-equivalent)", 4096),
-                                             ("gemm_i8_sparse24_2048x2048x8192", R.I8, R.I32, "i8", "TOP/s (dense-equivalent)", 2048)):
+                                             ("gemm_i8_sparse24_2048x2048x8192", R.I8, R.I32, "i8", "TOP/s (dense-equivalent)", 2048),
+                                             # (beyond the benchmark's configurations: the 16-bit sparse instruction, U[-1, 1] operands)
+                                             ("gemm_f16_sparse24_4096x4096x8192", R.F16, R.F32, "f16", "TFLOP/s (dense-equivalent)", 4096)):
         sn = sm
         mask = O.sparse24_mask(60, sm, sk)
         srows = np.array([0, 31, 32, 1234, 2047, sm // 2, sm - 32, sm - 1], dtype=np.uint32)
         if in_t == R.I8:
             av, bh = O.uniform_int8(61, sm * sk).reshape(sm, sk), O.uniform_int8(62, sk * sn)
+        elif in_t == R.F16:
+            av = O.f32_to_storage(O.uniform_pm1(61, sm * sk), O.F16).reshape(sm, sk)
+            bh = O.f32_to_storage(O.uniform_pm1(62, sk * sn), O.F16)
         else:
             av = O.f32_to_storage(O.normal(61, sm * sk), O.E4M3).view(np.int8).reshape(sm, sk)
             bh = O.f32_to_storage(O.normal(62, sk * sn), O.E4M3)
-        dense = np.where(mask, av, np.int8(0)).astype(np.int8)
+        dense = np.where(mask, av, av.dtype.type(0)).astype(av.dtype)
         vals, meta = R.compress_24(dense)
         storage = dense.view(np.uint8) if in_t == R.E4M3 else dense
         want = O.gemm_rows(in_t, out_t, O.ROW, O.COL, sm, sn, sk, storage.ravel(), bh, srows)
-        gemm_case(name, in_t, out_t, R.ROW_MAJOR, R.COL_MAJOR, torch.from_numpy(vals.view(np.uint8)).cuda(),
+        gemm_case(name, in_t, out_t, R.ROW_MAJOR, R.COL_MAJOR, torch.from_numpy(np.ascontiguousarray(vals).view(np.uint8)).cuda(),
                   torch.from_numpy(bh.view(np.uint8)).cuda(), PEAK_TFLOPS[key], unit,
                   sparse_meta=torch.from_numpy(meta).cuda(), mm=sm, nn=sn, kk=sk, peak_scale=2.0, sparse_rows=(srows, want))
         del av, bh, dense, vals, meta, storage, mask
