@@ -382,6 +382,143 @@ namespace
         }
     }
 
+    // f32 forward, k = 64 or 128: a workgroup owns 8 consecutive samples, as in the 16-bit kernel, and their output rows - one
+    // run of 8 (k + m (m - 1) / 2) floats, a whole number of 16-byte pieces that starts on one - leave together with
+    // 128-bit stores.  (A wave that stores its own sample's row writes 4-byte pieces of a row that starts anywhere: every
+    // store instruction and every sample ends inside a cache line that another instruction or wave completes later; taking
+    // the stores out of that kernel took a quarter of its time with them, for an eighth of its bytes.)
+    // A sample of 128 columns passes through the wave's LDS image in two halves of 64 that accumulate into the same three
+    // blocks, each half with a register stash of its own that is requested again (the same half of the wave's second
+    // sample) as soon as it has been unloaded: the image of half a sample leaves the LDS for the eight output rows.
+    // Rows from m on lie beyond the sample's buffer and cost no traffic, so the time follows m (the matrix work does not).
+    template <uint32_t K, uint32_t ROWS>
+    __global__ void __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(ROWS <= 28u ? 3 : 2)))
+        dlrmFwdF32Run(const float* __restrict__ in, float* __restrict__ out, uint32_t m, uint32_t batch)
+    {
+        constexpr uint32_t KH = 64u, HALVES = K / KH; // columns of a half, halves of a sample
+        static_assert(K == 64u || K == 128u, "one or two halves");
+        constexpr uint32_t ROW_CHUNKS = KH / 4u; // 16-byte chunks per row of a half
+        constexpr uint32_t MAX_OUT    = K + ROWS * (ROWS - 1) / 2;
+        constexpr uint32_t CHUNKS     = ROWS * ROW_CHUNKS / 64u; // loads per lane and half (ROWS * 16 is a multiple of 64)
+        constexpr uint32_t ROWP       = KH * 4u + 16u; // rows one chunk longer than the data: (KH + 4) / 4 is odd (see dlrmFwdF32Kernel)
+        constexpr uint32_t PER_WAVE   = SAMPLES_PER_WG / WAVES; // 2
+        using f32x4                   = float __attribute__((ext_vector_type(4)));
+        static_assert(ROWS * ROW_CHUNKS % 64u == 0u, "whole load instructions");
+
+        __shared__ __attribute__((aligned(16))) char  xLds[WAVES][ROWS * ROWP];
+        __shared__ __attribute__((aligned(16))) float outLds[SAMPLES_PER_WG * MAX_OUT + 4u];
+
+        const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const uint32_t outStride = K + m * (m - 1) / 2;
+        const uint32_t inBytes   = m * K * 4u;
+        const uint32_t b0        = blockIdx.x * SAMPLES_PER_WG;
+        char*          xw = xLds[wave];
+        const uint32_t r16 = lane & 15u, kq = lane >> 4;
+        const bool     validLo = r16 < m, validHi = 16u + r16 < m;
+        const uint32_t rowLo = validLo ? r16 : 0u, rowHi = validHi ? 16u + r16 : 0u;
+
+        f32x4 stash[HALVES][CHUNKS];
+        // (a sample beyond the batch is a buffer of no bytes: the loads are issued and move nothing)
+        auto request = [&](uint32_t h, uint32_t b) {
+            const bool valid = b < batch;
+            const auto src   = runBuffer(in, (uint64_t)(valid ? b : 0u) * inBytes, valid ? inBytes : 0u);
+#pragma unroll
+            for(uint32_t j = 0; j < CHUNKS; ++j)
+            {
+                const uint32_t c = j * 64u + lane;
+                stash[h][j]      = __builtin_bit_cast(
+                    f32x4, __builtin_amdgcn_raw_buffer_load_b128(src, (c / ROW_CHUNKS) * (K * 4u) + h * (KH * 4u) + (c % ROW_CHUNKS) * 16u, 0, LOAD_POLICY));
+            }
+        };
+#pragma unroll
+        for(uint32_t h = 0; h < HALVES; ++h)
+            request(h, b0 + wave);
+#pragma unroll
+        for(uint32_t q = 0; q < PER_WAVE; ++q)
+        {
+            const uint32_t sIdx = wave + q * WAVES, b = b0 + sIdx;
+            float*         o    = outLds + sIdx * outStride;
+            f32x4 accLL = {0, 0, 0, 0}, accHL = accLL, accHH = accLL;
+#pragma unroll
+            for(uint32_t h = 0; h < HALVES; ++h)
+            {
+                // chunks of rows m .. ROWS - 1 arrive as zeros and are written like the others: those rows are never used
+#pragma unroll
+                for(uint32_t j = 0; j < CHUNKS; ++j)
+                {
+                    const uint32_t c = j * 64u + lane;
+                    *reinterpret_cast<f32x4*>(xw + (c / ROW_CHUNKS) * ROWP + (c % ROW_CHUNKS) * 16u) = stash[h][j];
+                }
+                __builtin_amdgcn_s_waitcnt(0xC07F);
+                __builtin_amdgcn_wave_barrier();
+                if(q + 1u < PER_WAVE)
+                    request(h, b + WAVES); // this half's stash is free again: the wave's second sample
+
+                // lane l feeds row l % 16 (+ 16) at k = 4 s + l / 16; a group's operand reads are issued before the
+                // previous group's matrix instructions (see dlrmFwdF32Kernel)
+                constexpr uint32_t GROUP = 4u, GROUPS = KH / 4u / GROUP;
+                float              xl[2][GROUP], xh[2][GROUP];
+                auto fetch = [&](uint32_t grp, float (&lo)[GROUP], float (&hi)[GROUP]) {
+#pragma unroll
+                    for(uint32_t u = 0; u < GROUP; ++u)
+                    {
+                        const uint32_t st = grp * GROUP + u;
+                        lo[u] = *reinterpret_cast<const float*>(xw + rowLo * ROWP + kq * 4u + st * 16u);
+                        hi[u] = *reinterpret_cast<const float*>(xw + rowHi * ROWP + kq * 4u + st * 16u);
+                    }
+                };
+                fetch(0, xl[0], xh[0]);
+#pragma unroll
+                for(uint32_t grp = 0; grp < GROUPS; ++grp)
+                {
+                    if(grp + 1u < GROUPS)
+                        fetch(grp + 1u, xl[(grp + 1u) & 1u], xh[(grp + 1u) & 1u]);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for(uint32_t u = 0; u < GROUP; ++u)
+                    {
+                        const float lo = validLo ? xl[grp & 1u][u] : 0.0f, hi = validHi ? xh[grp & 1u][u] : 0.0f;
+                        accLL          = __builtin_amdgcn_mfma_f32_16x16x4f32(lo, lo, accLL, 0, 0, 0);
+                        accHL          = __builtin_amdgcn_mfma_f32_16x16x4f32(hi, lo, accHL, 0, 0, 0);
+                        accHH          = __builtin_amdgcn_mfma_f32_16x16x4f32(hi, hi, accHH, 0, 0, 0);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if(b < batch)
+                    o[h * KH + lane] = reinterpret_cast<const float*>(xw)[lane]; // row 0: 64 values of this half
+                __builtin_amdgcn_s_waitcnt(0xC07F);
+                __builtin_amdgcn_wave_barrier(); // every read of this half has returned: the image takes the next one
+            }
+            // a 16 x 16 result block: lane holds rows 4 (lane / 16) + e, column lane % 16
+            if(b < batch)
+#pragma unroll
+                for(uint32_t e = 0; e < 4; ++e)
+                {
+                    const uint32_t i = 4u * kq + e, j = r16;
+                    if(j < i && i < m)
+                        o[K + i * (i - 1u) / 2u + j] = accLL[e];
+                    const uint32_t ih = 16u + i;
+                    if(ih < m)
+                    {
+                        o[K + ih * (ih - 1u) / 2u + j] = accHL[e];
+                        if(j < i)
+                            o[K + ih * (ih - 1u) / 2u + 16u + j] = accHH[e];
+                    }
+                }
+        }
+        __syncthreads();
+
+        // ---- coalesced copy-out of the workgroup's samples
+        const uint32_t nSamples = (batch - b0) < SAMPLES_PER_WG ? (batch - b0) : SAMPLES_PER_WG;
+        const uint32_t total    = nSamples * outStride; // floats
+        float*         dst      = out + (uint64_t)b0 * outStride;
+        const uint32_t vecs     = total / 4u;
+        for(uint32_t v = tid; v < vecs; v += THREADS)
+            streamStore(reinterpret_cast<const f32x4*>(outLds)[v], reinterpret_cast<f32x4*>(dst) + v);
+        for(uint32_t e = vecs * 4u + tid; e < total; e += THREADS)
+            dst[e] = outLds[e];
+    }
+
     // f32 forward with the matrix instructions fed straight from the global loads: no LDS image of X.  Both operands of
     // v_mfma_f32_16x16x4_f32 hold, in lane l, row l % 16 of a block of rows at k index l / 16 - and which four values of k
     // one instruction sums is free as long as A and B agree.  Lane l therefore loads, for j = 0 .. K / 16 - 1, the 16
@@ -942,16 +1079,20 @@ extern "C" int r355_dlrm_fwd(int32_t dtype, const void* in, void* out, uint32_t 
         const uint32_t steps = (batch + WAVES - 1) / WAVES; // of one sample per wave
         auto*      fi = static_cast<const float*>(in);
         auto*      fo = static_cast<float*>(out);
-        // Matrix instructions straight from the loads (dlrmFwdF32Direct) or out of an LDS image of X (dlrmFwdF32Kernel): the
-        // first up to 16 features, where it runs one block of rows instead of three, and beyond that where the image's
-        // padding to 28 or 32 rows costs more than the direct kernel's scattered 16-byte pieces (measured over m = 17 .. 32
-        // at a batch of 65536: k = 32 always, k = 64 up to 21 features, k = 128 up to 24).  Measurement builds force either.
+        // Three kernels.  dlrmFwdF32Direct (matrix instructions straight from the loads): up to 16 features, where it runs one
+        // block of rows instead of three, and a few more while its scattered 16-byte pieces cost less than what the others
+        // pay per sample.  dlrmFwdF32Run (eight samples per workgroup, one run of output rows, the image in halves of k): its
+        // time follows m.  dlrmFwdF32Kernel (a wave per sample, the whole sample in the image): k = 64 near 32 features.
+        // Chosen per (m, k) from measurements at a batch of 65536 (m = 17 .. 32); measurement builds force one of them.
 #if defined(R355_DLRM_F32_LDS_IMAGE)
-        const bool direct = false;
+        const bool direct = false, run = false;
 #elif defined(R355_DLRM_F32_DIRECT_ALL)
-        const bool direct = true;
+        const bool direct = true, run = false;
+#elif defined(R355_DLRM_F32_RUN_ALL)
+        const bool direct = false, run = k >= 64;
 #else
-        const bool direct = m <= 16 || k == 32 || (k == 64 && m <= 21) || (k == 128 && m <= 24);
+        const bool direct = m <= 16 || k == 32 || (k == 64 && m <= 20) || (k == 128 && m <= 17);
+        const bool run    = !direct && (k == 128 || (k == 64 && m <= 26));
 #endif
         if(direct)
         {
@@ -974,6 +1115,19 @@ extern "C" int r355_dlrm_fwd(int32_t dtype, const void* in, void* out, uint32_t 
             return r355::checkLaunch("dlrm_fwd");
         }
         const dim3     grid32((steps + F32_STEPS - 1) / F32_STEPS), block32(THREADS);
+        if(run)
+        {
+            const dim3 gridRun((batch + SAMPLES_PER_WG - 1) / SAMPLES_PER_WG);
+            if(k == 64 && m <= 28)
+                hipLaunchKernelGGL((dlrmFwdF32Run<64, 28>), gridRun, block32, 0, s, fi, fo, m, batch);
+            else if(k == 64)
+                hipLaunchKernelGGL((dlrmFwdF32Run<64, 32>), gridRun, block32, 0, s, fi, fo, m, batch);
+            else if(m <= 28)
+                hipLaunchKernelGGL((dlrmFwdF32Run<128, 28>), gridRun, block32, 0, s, fi, fo, m, batch);
+            else
+                hipLaunchKernelGGL((dlrmFwdF32Run<128, 32>), gridRun, block32, 0, s, fi, fo, m, batch);
+            return r355::checkLaunch("dlrm_fwd");
+        }
 #define R355_FWD32(KK)                                                                                \
     do                                                                                                \
     {                                                                                                 \

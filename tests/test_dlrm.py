@@ -74,7 +74,11 @@ def test_fwd_reference_fixture_fp32():
 @pytest.mark.parametrize("m,k,batch", [(32, 32, 64), (27, 128, 13), (2, 64, 5), (32, 128, 3), (17, 128, 70),
                                        # the kernel that feeds the matrix instructions from the loads: every instance (k, one or two
                                        # blocks of rows), the last shapes it takes (21 x 64, 24 x 128) and the first it leaves (22, 25)
-                                       (32, 32, 700), (17, 32, 33), (21, 64, 70), (22, 64, 70), (24, 128, 64), (25, 128, 64), (20, 128, 515),
+                                       (32, 32, 700), (17, 32, 33), (20, 64, 70), (17, 128, 64), (17, 128, 515),
+                                       # eight samples per workgroup, one run of output rows: both k, both images, batches that end
+                                       # inside a workgroup, the shapes either side of the launcher's choices
+                                       (21, 64, 70), (26, 64, 9), (27, 64, 70), (18, 128, 64), (25, 128, 61), (32, 128, 70), (29, 128, 1), (28, 128, 515),
+                                       (22, 64, 1001),
                                        (16, 128, 64), (16, 128, 1000), (16, 32, 9), (8, 128, 517), (13, 64, 2049), (2, 32, 3), (5, 128, 1)])
 def test_fwd_f32_shapes_vs_oracle(m, k, batch):
     x = O.normal(3, batch * m * k)
