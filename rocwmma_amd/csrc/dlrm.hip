@@ -77,8 +77,10 @@ namespace
     // cache-policy bits of the raw buffer builtins (2 = nt): X, the upstream gradient and the results are touched once.
     // Measurement builds (python -m rocwmma_amd.build --variant <name> -D...): R355_DLRM_PLAIN_LOADS / R355_DLRM_PLAIN_STORES
     // take the default policy instead.
-#ifdef R355_DLRM_PLAIN_LOADS
+#if defined(R355_DLRM_PLAIN_LOADS)
     constexpr int LOAD_POLICY = 0;
+#elif defined(R355_DLRM_LOAD_POLICY)
+    constexpr int LOAD_POLICY = R355_DLRM_LOAD_POLICY;
 #else
     constexpr int LOAD_POLICY = 2;
 #endif
